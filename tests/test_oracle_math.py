@@ -1,0 +1,314 @@
+"""Pins the oracle's GEMV, activation, router select, FFN, combine and host grouping logic against
+library routines in fp64, brute force, invariants and the reference tests' exact expected arrays."""
+import numpy as np
+import pytest
+import torch
+
+
+def _rel(actual, ref):
+    # RelError.compute, Tests/Support/Validation/Tolerance/RelError.swift:7-16
+    return float(np.abs(actual - ref).max() / max(np.abs(ref).max(), 1e-6))
+
+
+def _deq64(oracle, W, S, B):
+    q = np.stack([W & 15, W >> 4], -1).reshape(W.shape[0], -1).astype(np.float64)
+    s = np.repeat(oracle.bf16_to_float(S).astype(np.float64), 64, axis=1)
+    b = np.repeat(oracle.bf16_to_float(B).astype(np.float64), 64, axis=1)
+    return q * s + b
+
+
+def test_gemv_special_inputs_and_fp64(oracle):
+    # shapes of DequantInt4SmallBatchTests.swift:66-73, same seed derivation
+    m, n = 300, 2112
+    rng = oracle.seed_tree_key(0xD8, f"int4-small-batch-m{m}-n{n}-r3-off0")
+    rows = rng.uniform(-0.5, 0.5, m * n).reshape(m, n)
+    W, S, B = oracle.quantize_int4(rows)
+    deq = oracle.dequantize_int4(W, S, B)
+    # quantisation error bound: half a step of the bf16-rounded scale (plus its rounding)
+    step = np.repeat(oracle.bf16_to_float(S), 64, axis=1)
+    assert np.all(np.abs(deq - rows) <= 0.5 * step * 1.02 + 1e-6)
+    # one-hot x picks a single dequantised weight exactly (pins row/column indexing)
+    for k in (0, 1, 63, 64, 65, 1055, n - 1):
+        x = np.zeros(n, np.float32)
+        x[k] = 1.0
+        assert np.array_equal(oracle.gemv_int4_ref(W, S, B, x), deq[:, k])
+    # general x against a float64 BLAS product
+    x = rng.uniform(-1.0, 1.0, n)
+    y = oracle.gemv_int4_ref(W, S, B, x)
+    y64 = _deq64(oracle, W, S, B) @ x.astype(np.float64)
+    assert _rel(y, y64.astype(np.float32)) < 1e-5
+    # linearity in x
+    x2 = rng.uniform(-1.0, 1.0, n)
+    y2 = oracle.gemv_int4_ref(W, S, B, x2)
+    y12 = oracle.gemv_int4_ref(W, S, B, (x + x2).astype(np.float32))
+    assert _rel(y12, y + y2) < 1e-5
+
+
+def test_int4_dot_matches_gemv_and_factored_form(oracle):
+    rng = np.random.default_rng(5)
+    pool = oracle.random_pool(rng, 2, 128, 64)
+    x = rng.normal(0, 1, 128).astype(np.float32)
+    for which, rows in (("gate", 64), ("up", 64)):
+        W, S, B = pool.sub(1, which)
+        y = oracle.gemv_int4_ref(W, S, B, x)
+        got = np.array([oracle.int4_dot(pool, 1, which, r, x) for r in range(rows)], np.float32)
+        assert np.array_equal(got, y)     # same arithmetic: (q*s+b)*x summed left to right
+        # factored form s*sum(q x) + b*sum(x) (moe.metal:323-378) agrees within fp32 noise
+        q = np.stack([W & 15, W >> 4], -1).reshape(rows, -1).astype(np.float64)
+        s = oracle.bf16_to_float(S).astype(np.float64)
+        b = oracle.bf16_to_float(B).astype(np.float64)
+        xs = x.astype(np.float64).reshape(-1, 64)
+        fact = (s * (q.reshape(rows, -1, 64) * xs).sum(-1) + b * xs.sum(-1)).sum(-1)
+        assert _rel(got, fact.astype(np.float32)) < 1e-5
+    xd = rng.normal(0, 1, 64).astype(np.float32)
+    W, S, B = pool.sub(0, "down")
+    got = np.array([oracle.int4_dot(pool, 0, "down", r, xd) for r in range(128)], np.float32)
+    assert np.array_equal(got, oracle.gemv_int4_ref(W, S, B, xd))
+
+
+def test_gelu_tanh_vs_torch(oracle):
+    x = np.concatenate([np.linspace(-12, 12, 4001), [0.0, -0.0, 1e-8, -30.0, 30.0]]).astype(np.float32)
+    ref = torch.nn.functional.gelu(torch.from_numpy(x).double(), approximate="tanh").numpy()
+    got = oracle.gelu_tanh(x)
+    assert np.abs(got - ref).max() < 2e-6
+    assert oracle.gelu_tanh([0.0])[0] == 0.0
+    assert oracle.gelu_tanh([30.0])[0] == 30.0 and oracle.gelu_tanh([-30.0])[0] == 0.0
+
+
+def test_topk_against_full_sort(oracle):
+    rng = np.random.default_rng(7)
+    for _ in range(200):
+        e = int(rng.choice([8, 16, 100, 128, 256]))
+        logits = rng.normal(0, 1, e).astype(np.float32)
+        if rng.random() < 0.5:                      # force exact ties
+            logits[rng.integers(0, e, 6)] = logits[rng.integers(0, e)]
+        idx, w = oracle.topk_softmax(logits, 8)
+        # RouterTopKTests.swift:55-63: sort by (score desc, index asc), take 8
+        order = sorted(range(e), key=lambda i: (-float(logits[i]), i))[:8]
+        assert list(idx) == order
+        s = logits[order].astype(np.float64)
+        ref = np.exp(s - s[0]) / np.exp(s - s[0]).sum()
+        assert np.abs(w - ref).max() < 1e-6
+        assert abs(w.sum() - 1.0) < 1e-6 and np.all(np.diff(w) <= 0)
+
+
+def test_topk_special_cases(oracle):
+    # all-equal scores -> indices 0..7, equal weights
+    idx, w = oracle.topk_softmax(np.zeros(128, np.float32), 8)
+    assert list(idx) == list(range(8)) and np.allclose(w, 0.125)
+    # fewer than 8 candidates: -inf and NaN are never taken; missing slots = (index 0, weight 0)
+    logits = np.full(128, -np.inf, np.float32)
+    logits[[5, 77, 9]] = [1.0, 3.0, 1.0]
+    logits[3] = np.nan
+    idx, w = oracle.topk_softmax(logits, 8)
+    assert list(idx) == [77, 5, 9, 0, 0, 0, 0, 0]
+    assert np.all(w[3:] == 0) and abs(w[:3].sum() - 1) < 1e-6
+    # per-expert scale multiplies the softmax weight of the chosen expert (moe.metal:235)
+    pes = oracle.bf16_bits(np.linspace(0.6, 1.4, 128).astype(np.float32))
+    logits = np.arange(128, dtype=np.float32) * 0.1
+    idx, w = oracle.topk_softmax(logits, 8, pes)
+    idx0, w0 = oracle.topk_softmax(logits, 8)
+    assert list(idx) == list(range(127, 119, -1))
+    assert np.allclose(w, w0 * oracle.bf16_to_float(pes)[idx], rtol=1e-6)
+    # generic top_k (prefill kernel, prefill.metal:499-541)
+    idx3, w3 = oracle.topk_softmax(logits, 3)
+    assert list(idx3) == [127, 126, 125] and abs(w3.sum() - 1) < 1e-6
+
+
+def test_router_reference_test_restated(oracle):
+    # RouterTopKTests.swift:17-44: 16 experts x 128, INT8-affine weights, ordering by full sort
+    g = oracle.SplitMix64(0xA5B6_1234)
+    weights = np.stack([g.uniform(-0.05, 0.05, 128) + np.float32(e) * np.float32(0.01) for e in range(16)])
+    hidden = g.uniform(-1.0, 1.0, 128)
+    inv = np.float32(1.0) / np.sqrt(np.float32(128))
+    es = g.uniform(0.5, 1.5, 128) * inv
+    pes = g.uniform(0.6, 1.4, 16)
+    P, S, B = oracle.quantize_int8(weights)
+    Wdeq = oracle.dequantize_int8(P, S, B)
+    # the kernel sees fp16 hidden and bf16 effective scale / per-expert scale
+    xb = oracle.bits16(hidden, oracle.FP16)
+    esb, pesb = oracle.bf16_bits(es), oracle.bf16_bits(pes)
+    logits = oracle.router_logits_pinned(Wdeq, xb, oracle.FP16, esb)
+    ref = Wdeq.astype(np.float64) @ (oracle.from_bits16(xb, oracle.FP16).astype(np.float64) * oracle.bf16_to_float(esb))
+    assert np.abs(logits - ref).max() < 1e-5
+    idx, w = oracle.topk_softmax(logits, 8, pesb)
+    # the Swift reference: fp32 inputs (no 16-bit rounding), sort, softmax, times expertScale
+    ref32 = Wdeq.astype(np.float64) @ (hidden.astype(np.float64) * es.astype(np.float64))
+    order = sorted(range(16), key=lambda i: (-ref32[i], i))[:8]
+    assert list(idx) == order
+    ex = np.exp(ref32[order] - ref32[order[0]])
+    assert np.abs(w - ex / ex.sum() * pes[order]).max() < 5e-3
+
+
+def test_router_pinned_order_definition(oracle):
+    # the pinned order equals an explicit numpy evaluation of the same tree, and a fp64 dot within noise
+    rng = np.random.default_rng(11)
+    e, d = 128, 2816
+    Wb = oracle.bf16_bits(rng.normal(0, 0.02, (e, d)).astype(np.float32))
+    xb = oracle.bf16_bits(rng.normal(0, 1, d).astype(np.float32))
+    got = oracle.router_logits_pinned(Wb, xb)
+    W = oracle.bf16_to_float(Wb).astype(np.float64)
+    x = oracle.bf16_to_float(xb).astype(np.float64)
+    assert np.abs(got - W @ x).max() < 2e-5
+    # lanes: fp32 fma chain over k = l + 64 i. bf16*bf16 products are exact in fp32, so fma == mul+add here.
+    Wf, xf = oracle.bf16_to_float(Wb), oracle.bf16_to_float(xb)
+    p = np.zeros((e, 64), np.float32)
+    for i in range(d // 64):
+        p = (Wf[:, 64 * i:64 * i + 64] * xf[64 * i:64 * i + 64] + p).astype(np.float32)
+    for m in (32, 16, 8, 4, 2, 1):
+        p = (p + p[:, np.arange(64) ^ m]).astype(np.float32)
+    assert np.array_equal(got, p[:, 0])
+
+
+def test_ffn_and_layer_vs_torch_fp64(oracle):
+    rng = np.random.default_rng(3)
+    d, f, e, t = 128, 64, 16, 5
+    pool = oracle.random_pool(rng, e, d, f)
+    router = oracle.bf16_bits(rng.normal(0, 0.02, (e, d)).astype(np.float32))
+    xb = oracle.bf16_bits(rng.normal(0, 1, (t, d)).astype(np.float32))
+    idx, w, y = oracle.moe_layer(pool, router, xb, 8)
+    x64 = torch.from_numpy(oracle.bf16_to_float(xb).astype(np.float64))
+    R = torch.from_numpy(oracle.bf16_to_float(router).astype(np.float64))
+    logits = x64 @ R.T
+    top = torch.topk(logits, 8, dim=1)
+    assert np.array_equal(idx, top.indices.numpy().astype(np.uint32))
+    wref = torch.softmax(top.values, dim=1).numpy()
+    assert np.abs(w - wref).max() < 2 ** -8          # weights are rounded to bf16
+    yref = np.zeros((t, d))
+    for tok in range(t):
+        for r in range(8):
+            ex = int(idx[tok, r])
+            G = torch.from_numpy(_deq64(oracle, *pool.sub(ex, "gate")))
+            U = torch.from_numpy(_deq64(oracle, *pool.sub(ex, "up")))
+            D = torch.from_numpy(_deq64(oracle, *pool.sub(ex, "down")))
+            act = torch.nn.functional.gelu(G @ x64[tok], approximate="tanh") * (U @ x64[tok])
+            yref[tok] += float(w[tok, r]) * (D @ act).numpy()
+    assert _rel(y, yref.astype(np.float32)) < 1e-4
+    # run_ffn alone and moe_experts agree with the layer composition
+    y2 = oracle.moe_experts(pool, xb, idx, w)
+    assert np.array_equal(y, y2)
+
+
+def test_streamed_routed_reference_test_restated(oracle):
+    # MoEFusedFFNTests.swift:17-46: D=128, F=64, K=8, SeedTree(0x2D3).key("production-routed-moe")
+    g = oracle.seed_tree_key(0x2D3, "production-routed-moe")
+    gates, ups, downs = [], [], []
+    for _ in range(8):
+        gates.append(g.uniform(-0.4, 0.4, 64 * 128).reshape(64, 128))
+        ups.append(g.uniform(-0.4, 0.4, 64 * 128).reshape(64, 128))
+        downs.append(g.uniform(-0.4, 0.4, 128 * 64).reshape(128, 64))
+    x = g.uniform(-0.5, 0.5, 128).astype(np.float16).astype(np.float32)
+    residual = g.uniform(-0.5, 0.5, 128).astype(np.float16).astype(np.float32)
+    rw = (np.float32(0.04) + np.arange(8, dtype=np.float32) * np.float32(0.015)).astype(np.float16).astype(np.float32)
+    pool = oracle.pool_from_float(gates, ups, downs)
+    # blob layout of makeBlob (MoEFusedFFNTests.swift:221-257): nine tightly packed sub-tensors
+    assert pool.offsets.as_tuple() == (0, 4096, 4352, 4608, 8704, 8960, 9216, 13312, 13568) and pool.stride == 13824
+    y = oracle.apply_streamed_routed(pool, list(range(8)), x, residual, rw)
+    ref = residual.astype(np.float64).copy()
+    for k in range(8):
+        G, U, D = (_deq64(oracle, *pool.sub(k, n)) for n in ("gate", "up", "down"))
+        act = torch.nn.functional.gelu(torch.from_numpy(G @ x.astype(np.float64)), approximate="tanh").numpy() * (U @ x.astype(np.float64))
+        ref += float(rw[k]) * (D @ act)
+    assert _rel(y, ref.astype(np.float32)) < 1e-5
+    # top_k = 5 ignores the other slots (MoEFusedFFNTests.swift:150-219)
+    y5 = oracle.apply_streamed_routed(pool, list(range(5)), x, residual, rw[:5])
+    ref5 = residual.astype(np.float64).copy()
+    for k in range(5):
+        ref5 += float(rw[k]) * oracle.run_ffn(pool, k, x).astype(np.float64)
+    assert _rel(y5, ref5.astype(np.float32)) < 1e-6
+
+
+def test_reduce_token_major(oracle):
+    # PrefillMoETests.swift:10-20,46-64
+    g = oracle.SplitMix64(0x4D0E_2026)
+    rows, k, d = 3, 8, 64
+    partials = g.uniform(-2.0, 2.0, rows * k * d).astype(np.float16)
+    weights = g.uniform(-1.0, 1.0, rows * k).astype(np.float16)
+    h2 = oracle.reduce_token_major(partials.view(np.uint16).reshape(rows, k, d), oracle.FP16,
+                                   weights.view(np.uint16), oracle.FP16)
+    ref = (weights.astype(np.float64).reshape(rows, k, 1) * partials.astype(np.float64).reshape(rows, k, d)).sum(1)
+    assert np.abs(h2.view(np.float16).astype(np.float64) - ref).max() <= 2e-3
+    # one-hot weights reproduce the selected partial bit for bit
+    onehot = np.zeros((rows, k), np.float16)
+    onehot[:, 5] = 1
+    h = oracle.reduce_token_major(partials.view(np.uint16).reshape(rows, k, d), oracle.FP16, onehot.view(np.uint16), oracle.FP16)
+    assert np.array_equal(h, partials.view(np.uint16).reshape(rows, k, d)[:, 5, :])
+    # bf16 data, fp32 partials
+    pf = g.uniform(-2.0, 2.0, rows * k * d).reshape(rows, k, d)
+    wb = oracle.bf16_bits(g.uniform(0.0, 1.0, rows * k))
+    hb = oracle.reduce_token_major(pf, oracle.F32, wb, oracle.BF16)
+    refb = (oracle.bf16_to_float(wb).astype(np.float64).reshape(rows, k, 1) * pf).sum(1)
+    assert np.abs(oracle.bf16_to_float(hb) - refb).max() <= np.abs(refb).max() * 2 ** -8
+
+
+def test_pairs_are_token_major(oracle):
+    # PrefillRouterTests.swift:12-22
+    w = np.array([0.1, 0.2, 0.3, 0.4, 0.5, 0.6], np.float16)
+    pairs = oracle.make_token_expert_pairs([3, 1, 2, 4, 0, 5], w.view(np.uint16), 2, 3)
+    assert list(pairs["token"]) == [0, 0, 0, 1, 1, 1]
+    assert list(pairs["rank"]) == [0, 1, 2, 0, 1, 2]
+    assert list(pairs["expert"]) == [3, 1, 2, 4, 0, 5]
+    assert np.array_equal(pairs["weight_bits"].astype(np.uint16).view(np.float16), w)
+
+
+def _pair(token, expert, rank, bits):
+    return (token, expert, rank, bits)
+
+
+def test_grouping_exact_arrays(oracle):
+    # PrefillMoEGroupingTests.swift:5-50
+    raw = [_pair(0, 3, 0, 10), _pair(0, 1, 1, 11), _pair(0, 4, 2, 12), _pair(1, 1, 0, 13), _pair(1, 3, 1, 14),
+           _pair(1, 2, 2, 15), _pair(2, 4, 0, 16), _pair(2, 3, 1, 17), _pair(2, 1, 2, 18), _pair(3, 5, 0, 19),
+           _pair(3, 1, 1, 20), _pair(3, 4, 2, 21)][::-1]
+    pairs = np.array(raw, oracle.PAIR_DTYPE)
+    sp, groups, tiles = oracle.group_token_expert_pairs(pairs, 6, 2)
+    assert list(sp["expert"]) == [1, 1, 1, 1, 2, 3, 3, 3, 4, 4, 4, 5]
+    assert [[int(p["token"]), int(p["rank"])] for p in sp] == [[0, 1], [1, 0], [2, 2], [3, 1], [1, 2], [0, 0], [1, 1],
+                                                               [2, 1], [0, 2], [2, 0], [3, 2], [3, 0]]
+    assert list(sp["weight_bits"]) == [11, 13, 18, 20, 15, 10, 14, 17, 12, 16, 21, 19]
+    assert groups == [(1, 0, 4), (2, 4, 1), (3, 5, 3), (4, 8, 3), (5, 11, 1)]
+    assert tiles == [(0, 2, 0, 5), (2, 2, 5, 6), (4, 1, 11, 1)]
+
+
+def test_grouping_sort_keys_and_errors(oracle):
+    # PrefillMoEGroupingTests.swift:52-96
+    raw = [_pair(0, 1, 0, 10), _pair(0, 2, 1, 20), _pair(1, 3, 0, 30), _pair(1, 1, 1, 11), _pair(2, 2, 0, 21),
+           _pair(2, 3, 1, 31)]
+    sp, groups, tiles = oracle.group_token_expert_pairs(np.array(raw, oracle.PAIR_DTYPE), 4, 2, [0, 30, 10, 20])
+    assert [g[0] for g in groups] == [2, 3, 1]
+    assert list(sp["expert"]) == [2, 2, 3, 3, 1, 1]
+    assert tiles == [(0, 2, 0, 4), (2, 1, 4, 2)]
+    with pytest.raises(ValueError, match="route expert 2 is out of range"):
+        oracle.group_token_expert_pairs(np.array([_pair(0, 2, 0, 1)], oracle.PAIR_DTYPE), 2, 1)
+    # PrefillGroupedRoutedMoETests+Binding.swift:21-40: tiles never exceed 16 experts
+    raw = [_pair(i // 8, min(i, 19), i % 8, 0) for i in range(24)]
+    sp, groups, tiles = oracle.group_token_expert_pairs(np.array(raw, oracle.PAIR_DTYPE), 128, 16)
+    assert [g[0] for g in groups[tiles[0][0]:tiles[0][0] + tiles[0][1]]] == list(range(16))
+    assert [g[0] for g in groups[tiles[1][0]:tiles[1][0] + tiles[1][1]]] == list(range(16, 20))
+
+
+def test_route_partials_reference_test_restated(oracle):
+    # PrefillGroupedRoutedMoETests+Execution.swift:9-97 with syntheticRows (…Tests.swift:100-109)
+    d = f = 64
+    rows, top_k = 3, 2
+
+    def synthetic(nrows, ncols, expert, role):
+        r = np.arange(nrows, dtype=np.float32)[:, None]
+        c = np.arange(ncols, dtype=np.float32)[None, :]
+        return (np.float32(expert + 1) * np.float32(0.001) + np.float32(role + 1) * np.float32(0.003)
+                + ((r % 7) - 3) * np.float32(0.0004) + ((c % 11) - 5) * np.float32(0.0002)).astype(np.float32)
+
+    pool = oracle.pool_from_float([synthetic(f, d, e, 0) for e in range(16)], [synthetic(f, d, e, 1) for e in range(16)],
+                                  [synthetic(d, f, e, 2) for e in range(16)])
+    raw = [(0, 2, 0), (0, 0, 1), (1, 1, 0), (1, 2, 1), (2, 0, 0), (2, 1, 1)]
+    pairs = np.array([(t, e, r, 0) for t, e, r in raw], oracle.PAIR_DTYPE)
+    sp, groups, tiles = oracle.group_token_expert_pairs(pairs, 16, 16)
+    hidden = (((np.arange(rows * d) % 17) - 8).astype(np.float32) * np.float32(0.01)).astype(np.float16)
+    out = oracle.route_partials(pool, sp, hidden.view(np.uint16), d, rows, top_k, oracle.FP16, fill=-99.0)
+    x64 = hidden.astype(np.float64).reshape(rows, d)
+    for t, e, r in raw:
+        G, U, D = (_deq64(oracle, *pool.sub(e, n)) for n in ("gate", "up", "down"))
+        act = torch.nn.functional.gelu(torch.from_numpy(G @ x64[t]), approximate="tanh").numpy() * (U @ x64[t])
+        ref = D @ act
+        got = out[t, r].view(np.float16).astype(np.float64)
+        assert np.abs(got - ref).max() <= 0.0015
