@@ -1,0 +1,326 @@
+// C ABI of libfieldfare_moe_hip.so (declared in include/fieldfare_moe.h): context, HBM expert arena,
+// argument validation and stream-ordered launches. No call here touches a CPU implementation of the
+// math: without a working HIP device every entry point fails with FFMOE_ERR_RUNTIME.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "kernels.hpp"
+
+using namespace ffmoe;
+
+struct ffmoe_layer {
+    bool experts_loaded = false;
+    void *router_w = nullptr;       // bf16 or float [E][D]
+    int router_is_f32 = 0;
+    uint16_t *effective_scale = nullptr;
+    uint16_t *per_expert_scale = nullptr;
+};
+
+struct ffmoe_ctx {
+    int device = 0;
+    ffmoe_shape shape{};
+    ArenaGeom geom{};
+    uint8_t *arena = nullptr;
+    size_t layer_bytes = 0;
+    std::vector<ffmoe_layer> layers;
+    // scratch (owned by the context, sized at creation; calls on one context must not overlap)
+    float *logits = nullptr;         // [max(max_tokens,16)][E]
+    VerifyPlan *plan = nullptr;
+    float *xsum = nullptr;           // [16][D/64]
+    uint16_t *acts = nullptr;        // [16*top_k][F]
+    float *partials = nullptr;       // [16*top_k][D]
+};
+
+namespace {
+
+int fail(char **err, int code, const char *fmt, ...) {
+    if (err) {
+        char buf[512];
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(buf, sizeof buf, fmt, ap);
+        va_end(ap);
+        *err = strdup(buf);
+    }
+    return code;
+}
+
+#define FF_HIP(call)                                                                                  \
+    do {                                                                                              \
+        hipError_t e_ = (call);                                                                       \
+        if (e_ != hipSuccess) return fail(err, FFMOE_ERR_RUNTIME, "%s: %s", #call, hipGetErrorString(e_)); \
+    } while (0)
+
+int check_ctx(ffmoe_ctx *ctx, char **err) {
+    if (!ctx) return fail(err, FFMOE_ERR_INVALID, "null context");
+    FF_HIP(hipSetDevice(ctx->device));
+    return FFMOE_OK;
+}
+
+int check_layer(ffmoe_ctx *ctx, uint32_t layer, bool need_experts, bool need_router, char **err) {
+    if (layer >= ctx->shape.n_layers)
+        return fail(err, FFMOE_ERR_INVALID, "layer %u out of range (n_layers = %u)", layer, ctx->shape.n_layers);
+    if (need_experts && !ctx->layers[layer].experts_loaded)
+        return fail(err, FFMOE_ERR_NO_LAYER, "experts of layer %u were not uploaded", layer);
+    if (need_router && !ctx->layers[layer].router_w)
+        return fail(err, FFMOE_ERR_NO_LAYER, "router of layer %u was not uploaded", layer);
+    return FFMOE_OK;
+}
+
+template <typename T>
+int upload_vec(T **dst, const T *src, size_t count, char **err) {
+    if (*dst) { (void)hipFree(*dst); *dst = nullptr; }
+    if (!src) return FFMOE_OK;
+    FF_HIP(hipMalloc(reinterpret_cast<void **>(dst), count * sizeof(T)));
+    FF_HIP(hipMemcpy(*dst, src, count * sizeof(T), hipMemcpyHostToDevice));
+    return FFMOE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *ffmoe_version(void) { return "fieldfare-moe-hip 0.1 (gfx950)"; }
+
+int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **err) {
+    if (!shape || !out) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    *out = nullptr;
+    if (shape->d == 0 || shape->d % FFMOE_GROUP || shape->f == 0 || shape->f % FFMOE_GROUP)
+        return fail(err, FFMOE_ERR_INVALID, "d = %u and f = %u must be positive multiples of %d", shape->d, shape->f,
+                    FFMOE_GROUP);
+    if (shape->n_experts == 0 || shape->n_experts > FFMOE_MAX_EXPERTS)
+        return fail(err, FFMOE_ERR_INVALID, "n_experts = %u outside 1...%d", shape->n_experts, FFMOE_MAX_EXPERTS);
+    if (shape->top_k == 0 || shape->top_k > 8 || shape->top_k > shape->n_experts)
+        return fail(err, FFMOE_ERR_INVALID, "top_k = %u outside 1...8", shape->top_k);
+    if (shape->n_layers == 0) return fail(err, FFMOE_ERR_INVALID, "n_layers must be positive");
+    int count = 0;
+    FF_HIP(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return fail(err, FFMOE_ERR_INVALID, "device %d not present (%d visible)", device, count);
+    FF_HIP(hipSetDevice(device));
+
+    ffmoe_ctx *ctx = new (std::nothrow) ffmoe_ctx();
+    if (!ctx) return fail(err, FFMOE_ERR_ALLOC, "out of host memory");
+    ctx->device = device;
+    ctx->shape = *shape;
+    ctx->geom = make_geom(shape->d, shape->f);
+    ctx->layer_bytes = (size_t)shape->n_experts * ctx->geom.expert_bytes;
+    ctx->layers.resize(shape->n_layers);
+    const uint32_t router_rows = shape->max_tokens > FFMOE_MAX_VERIFY_ROWS ? shape->max_tokens : FFMOE_MAX_VERIFY_ROWS;
+    const size_t routes = (size_t)FFMOE_MAX_VERIFY_ROWS * shape->top_k;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&ctx->arena), ctx->layer_bytes * shape->n_layers);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->logits), (size_t)router_rows * shape->n_experts * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->plan), sizeof(VerifyPlan));
+    if (e == hipSuccess) e = hipMemset(ctx->plan, 0, sizeof(VerifyPlan));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->xsum), (size_t)FFMOE_MAX_VERIFY_ROWS * ctx->geom.gd * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->acts), routes * shape->f * sizeof(uint16_t));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->partials), routes * shape->d * sizeof(float));
+    if (e != hipSuccess) {
+        ffmoe_destroy(ctx);
+        return fail(err, FFMOE_ERR_ALLOC, "failed to allocate the expert arena (%zu bytes) or scratch: %s",
+                    ctx->layer_bytes * shape->n_layers, hipGetErrorString(e));
+    }
+    *out = ctx;
+    return FFMOE_OK;
+}
+
+void ffmoe_destroy(ffmoe_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipDeviceSynchronize();
+    for (auto &l : ctx->layers) {
+        if (l.router_w) (void)hipFree(l.router_w);
+        if (l.effective_scale) (void)hipFree(l.effective_scale);
+        if (l.per_expert_scale) (void)hipFree(l.per_expert_scale);
+    }
+    if (ctx->arena) (void)hipFree(ctx->arena);
+    if (ctx->logits) (void)hipFree(ctx->logits);
+    if (ctx->plan) (void)hipFree(ctx->plan);
+    if (ctx->xsum) (void)hipFree(ctx->xsum);
+    if (ctx->acts) (void)hipFree(ctx->acts);
+    if (ctx->partials) (void)hipFree(ctx->partials);
+    delete ctx;
+}
+
+size_t ffmoe_layer_arena_bytes(const ffmoe_ctx *ctx) { return ctx ? ctx->layer_bytes : 0; }
+
+int ffmoe_upload_layer(ffmoe_ctx *ctx, uint32_t layer, const void *blobs, size_t stride,
+                       const ffmoe_offsets *offsets, int src_is_device, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, false, false, err)) return rc;
+    if (!blobs || !offsets) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    const ffmoe_shape &sh = ctx->shape;
+    // every sub-tensor must lie inside one blob (the reference trusts its layout.json; a bad offset
+    // here would send the re-tiling kernel out of bounds)
+    const size_t gu_w = (size_t)sh.f * sh.d / 2, gu_s = (size_t)sh.f * (sh.d / FFMOE_GROUP) * 2;
+    const size_t dn_w = (size_t)sh.d * sh.f / 2, dn_s = (size_t)sh.d * (sh.f / FFMOE_GROUP) * 2;
+    const struct { uint32_t off; size_t len; const char *name; } parts[9] = {
+        {offsets->gate_w, gu_w, "gate_w"}, {offsets->gate_s, gu_s, "gate_s"}, {offsets->gate_b, gu_s, "gate_b"},
+        {offsets->up_w, gu_w, "up_w"},     {offsets->up_s, gu_s, "up_s"},     {offsets->up_b, gu_s, "up_b"},
+        {offsets->down_w, dn_w, "down_w"}, {offsets->down_s, dn_s, "down_s"}, {offsets->down_b, dn_s, "down_b"}};
+    for (const auto &p : parts)
+        if ((size_t)p.off + p.len > stride)
+            return fail(err, FFMOE_ERR_INVALID, "sub-tensor %s (offset %u, %zu bytes) exceeds the blob stride %zu", p.name,
+                        p.off, p.len, stride);
+    const uint8_t *src = static_cast<const uint8_t *>(blobs);
+    uint8_t *staging = nullptr;
+    if (!src_is_device) {
+        const size_t bytes = stride * sh.n_experts;
+        FF_HIP(hipMalloc(reinterpret_cast<void **>(&staging), bytes));
+        hipError_t e = hipMemcpy(staging, blobs, bytes, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(staging);
+            return fail(err, FFMOE_ERR_RUNTIME, "copy of layer %u to the device failed: %s", layer, hipGetErrorString(e));
+        }
+        src = staging;
+    }
+    hipError_t e = launch_repack_layer(nullptr, src, stride, *offsets, sh.n_experts, ctx->geom,
+                                       ctx->arena + (size_t)layer * ctx->layer_bytes);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (staging) (void)hipFree(staging);
+    if (e != hipSuccess) return fail(err, FFMOE_ERR_RUNTIME, "re-tiling layer %u failed: %s", layer, hipGetErrorString(e));
+    ctx->layers[layer].experts_loaded = true;
+    return FFMOE_OK;
+}
+
+int ffmoe_upload_router_bf16(ffmoe_ctx *ctx, uint32_t layer, const uint16_t *w, const uint16_t *effective_scale,
+                             const uint16_t *per_expert_scale, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, false, false, err)) return rc;
+    if (!w) return fail(err, FFMOE_ERR_INVALID, "null router weights");
+    ffmoe_layer &l = ctx->layers[layer];
+    const size_t n = (size_t)ctx->shape.n_experts * ctx->shape.d;
+    uint16_t *dw = nullptr;
+    if (l.router_w) { (void)hipFree(l.router_w); l.router_w = nullptr; }
+    if (int rc = upload_vec(&dw, w, n, err)) return rc;
+    l.router_w = dw;
+    l.router_is_f32 = 0;
+    if (int rc = upload_vec(&l.effective_scale, effective_scale, ctx->shape.d, err)) return rc;
+    return upload_vec(&l.per_expert_scale, per_expert_scale, ctx->shape.n_experts, err);
+}
+
+int ffmoe_upload_router_int8(ffmoe_ctx *ctx, uint32_t layer, const uint8_t *w, const uint16_t *scales,
+                             const uint16_t *biases, const uint16_t *effective_scale,
+                             const uint16_t *per_expert_scale, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, false, false, err)) return rc;
+    if (!w || !scales || !biases) return fail(err, FFMOE_ERR_INVALID, "null router weights");
+    ffmoe_layer &l = ctx->layers[layer];
+    const uint32_t e_count = ctx->shape.n_experts, d = ctx->shape.d, groups = d / FFMOE_GROUP;
+    // fp32(q * s + b): q * s is exact (8-bit x 8-bit significands), one rounding in the add
+    std::vector<float> deq((size_t)e_count * d);
+    for (uint32_t e = 0; e < e_count; ++e)
+        for (uint32_t k = 0; k < d; ++k) {
+            uint32_t sb = (uint32_t)scales[(size_t)e * groups + k / FFMOE_GROUP] << 16;
+            uint32_t bb = (uint32_t)biases[(size_t)e * groups + k / FFMOE_GROUP] << 16;
+            float s, b;
+            memcpy(&s, &sb, 4);
+            memcpy(&b, &bb, 4);
+            const float prod = (float)w[(size_t)e * d + k] * s;
+            deq[(size_t)e * d + k] = prod + b;
+        }
+    float *dw = nullptr;
+    if (l.router_w) { (void)hipFree(l.router_w); l.router_w = nullptr; }
+    if (int rc = upload_vec(&dw, deq.data(), deq.size(), err)) return rc;
+    l.router_w = dw;
+    l.router_is_f32 = 1;
+    if (int rc = upload_vec(&l.effective_scale, effective_scale, d, err)) return rc;
+    return upload_vec(&l.per_expert_scale, per_expert_scale, e_count, err);
+}
+
+int ffmoe_dequant_expert(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint32_t expert, int which,
+                         uint16_t *out_bf16, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, true, false, err)) return rc;
+    if (expert >= ctx->shape.n_experts) return fail(err, FFMOE_ERR_INVALID, "expert %u out of range", expert);
+    if (which < FFMOE_GATE || which > FFMOE_DOWN || !out_bf16) return fail(err, FFMOE_ERR_INVALID, "bad sub-tensor or null output");
+    if (reinterpret_cast<uintptr_t>(out_bf16) % 16) return fail(err, FFMOE_ERR_INVALID, "output must be 16-byte aligned");
+    const uint8_t *base = ctx->arena + (size_t)layer * ctx->layer_bytes + (size_t)expert * ctx->geom.expert_bytes;
+    FF_HIP(launch_dequant_expert(static_cast<hipStream_t>(stream), base, ctx->geom, which, out_bf16));
+    return FFMOE_OK;
+}
+
+int ffmoe_router(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *router_x, uint32_t x_stride,
+                 uint32_t t, uint32_t *out_idx, uint16_t *out_w, float *out_logits, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, false, true, err)) return rc;
+    if (!router_x || !out_idx || !out_w) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (t == 0) return fail(err, FFMOE_ERR_INVALID, "queryCount must be positive");
+    if (x_stride < ctx->shape.d) return fail(err, FFMOE_ERR_INVALID, "hidden stride is too small");
+    const uint32_t cap = ctx->shape.max_tokens > FFMOE_MAX_VERIFY_ROWS ? ctx->shape.max_tokens : FFMOE_MAX_VERIFY_ROWS;
+    if (!out_logits && t > cap) return fail(err, FFMOE_ERR_INVALID, "t = %u exceeds max_tokens = %u", t, cap);
+    const ffmoe_layer &l = ctx->layers[layer];
+    RouterWeights rw{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale};
+    FF_HIP(launch_router(static_cast<hipStream_t>(stream), rw, router_x, x_stride, t, ctx->shape.n_experts,
+                         ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w));
+    return FFMOE_OK;
+}
+
+static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
+                         uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual, uint16_t *y,
+                         uint16_t *partials_bf16, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, true, false, err)) return rc;
+    if (!x || !idx || !w || (!y && !partials_bf16)) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (t == 0 || t > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%d", t, FFMOE_MAX_VERIFY_ROWS);
+    if (x_stride < ctx->shape.d || x_stride % 8 || reinterpret_cast<uintptr_t>(x) % 16)
+        return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
+    if ((y && reinterpret_cast<uintptr_t>(y) % 8) || (residual && reinterpret_cast<uintptr_t>(residual) % 8))
+        return fail(err, FFMOE_ERR_INVALID, "y and residual must be 8-byte aligned");
+    FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
+                         ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
+                         ctx->plan, ctx->xsum, ctx->acts, ctx->partials));
+    return FFMOE_OK;
+}
+
+int ffmoe_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride, uint32_t t,
+                 const uint32_t *idx, const uint16_t *w, const uint16_t *residual, uint16_t *y, char **err) {
+    if (!y) return fail(err, FFMOE_ERR_INVALID, "null output");
+    return verify_common(ctx, stream, layer, x, x_stride, t, idx, w, residual, y, nullptr, err);
+}
+
+int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
+                          uint32_t t, const uint32_t *idx, const uint16_t *w, uint16_t *partials, char **err) {
+    if (!partials) return fail(err, FFMOE_ERR_INVALID, "null output");
+    return verify_common(ctx, stream, layer, x, x_stride, t, idx, w, nullptr, nullptr, partials, err);
+}
+
+int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!n_live) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    FF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    FF_HIP(hipMemcpy(n_live, &ctx->plan->n_live, sizeof(uint32_t), hipMemcpyDeviceToHost));
+    return FFMOE_OK;
+}
+
+int ffmoe_reduce_token_major(ffmoe_ctx *ctx, void *stream, const uint16_t *partials, const uint16_t *weights,
+                             uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!partials || !weights || !h2) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (t == 0) return fail(err, FFMOE_ERR_INVALID, "queryCount must be positive");
+    if (top_k == 0) return fail(err, FFMOE_ERR_INVALID, "topK must be positive");
+    if (d == 0) return fail(err, FFMOE_ERR_INVALID, "D must be positive");
+    FF_HIP(launch_reduce_token_major(static_cast<hipStream_t>(stream), partials, weights, h2, t, top_k, d));
+    return FFMOE_OK;
+}
+
+int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                    const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows, uint32_t x_stride,
+                    uint32_t y_stride, int y_f32, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!w || !scales || !biases || !x || !y) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (n == 0 || n % FFMOE_GROUP) return fail(err, FFMOE_ERR_INVALID, "N must be a multiple of %d", FFMOE_GROUP);
+    if (reinterpret_cast<uintptr_t>(w) % 2) return fail(err, FFMOE_ERR_INVALID, "weights need a 2-aligned offset");
+    if (m == 0) return fail(err, FFMOE_ERR_INVALID, "M must be positive");
+    if (rows == 0 || rows > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows=%u outside 1...%d", rows, FFMOE_MAX_VERIFY_ROWS);
+    if (x_stride < n || y_stride < m) return fail(err, FFMOE_ERR_INVALID, "stride smaller than the row");
+    FF_HIP(launch_gemv_int4(static_cast<hipStream_t>(stream), w, scales, biases, x, y, m, n, rows, x_stride, y_stride, y_f32));
+    return FFMOE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,84 @@
+// Shared device helpers for the gfx950 kernels of libfieldfare_moe_hip.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ffmoe {
+
+constexpr int kGroup = 64;     // MLX-affine group size (Infrastructure/ModelIO/Quantization.swift:2)
+constexpr int kWave = 64;      // CDNA wavefront
+constexpr int kTileRows = 16;  // weight rows per arena tile = MFMA 16x16x32 column block
+constexpr int kTileBytes = 1024;   // one arena tile: 64 lanes x 16 B (two 16-row x 64-k nibble blocks)
+constexpr int kTileScaleBytes = 128;  // 16 rows x 4 bf16 (scale/bias of the two blocks)
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t pair) { return __uint_as_float(pair & 0xFFFF0000u); }
+
+// Round-to-nearest-even fp32 -> bf16 with no NaN special case: the exact integer recipe of
+// Quantization.bf16Bits (Infrastructure/ModelIO/Quantization.swift:9-15), so the bits match the
+// reference's encoder for every input.
+__device__ __forceinline__ uint16_t f32_to_bf16(float x) {
+    uint32_t bits = __float_as_uint(x);
+    uint32_t lsb = (bits >> 16) & 1u;
+    return (uint16_t)((bits + (0x7FFFu + lsb)) >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+// gelu_pytorch_tanh, Metal/MoE/moe.metal:40-47 (clamp kept: it guards tanh at large magnitudes).
+__device__ __forceinline__ float gelu_tanh(float x) {
+    const float x3 = x * x * x;
+    float inner = 0.7978845608028654f * (x + 0.044715f * x3);
+    inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+    return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+// Arena nibble order inside one dword: nibble position m (m = 0..3) holds element 2m of the lane's
+// eight k-slots and position m + 4 holds element 2m + 1, so that ((w >> 4m) & 0x000F000F) is the
+// 16-bit pair (element 2m, element 2m + 1) with no cross-lane or cross-register shuffling.
+//
+// unpack8_offset128: the eight nibbles as bf16 values 128 + q (0x4300 | q is exact: the bf16 ulp at
+// 128 is 1). The matrix unit then accumulates sum (128 + q) x; the caller removes 128 * sum x.
+__device__ __forceinline__ bf16x8 unpack8_offset128(uint32_t w) {
+    uint4 r;
+    r.x = (w & 0x000F000Fu) | 0x43004300u;
+    r.y = ((w >> 4) & 0x000F000Fu) | 0x43004300u;
+    r.z = ((w >> 8) & 0x000F000Fu) | 0x43004300u;
+    r.w = ((w >> 12) & 0x000F000Fu) | 0x43004300u;
+    return __builtin_bit_cast(bf16x8, r);
+}
+
+// dequant8_bf16: the eight nibbles as bf16(fma(q, scale, bias)) - the reference's 16-bit tile weight
+// (Metal/Prefill/prefill.metal:581-590 with half replaced by bfloat as Metal/TensorCore/tensorops.metal:267).
+// q * scale is exact in fp32 (4-bit x 8-bit significands), so fma and mul-then-add agree.
+__device__ __forceinline__ uint4 dequant8_bf16(uint32_t w, float scale, float bias) {
+    uint4 r;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        const float q0 = (float)((w >> (4 * m)) & 0xFu);
+        const float q1 = (float)((w >> (4 * m + 16)) & 0xFu);
+        const uint32_t p = pack_bf16x2(__builtin_fmaf(q0, scale, bias), __builtin_fmaf(q1, scale, bias));
+        if (m == 0) r.x = p; else if (m == 1) r.y = p; else if (m == 2) r.z = p; else r.w = p;
+    }
+    return r;
+}
+
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// xor-butterfly sum across the 64 lanes (masks 32,16,8,4,2,1): every lane ends with the same value.
+__device__ __forceinline__ float wave_butterfly_sum(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = v + __shfl_xor(v, m, 64);
+    return v;
+}
+
+}  // namespace ffmoe

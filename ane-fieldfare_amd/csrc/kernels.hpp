@@ -1,0 +1,77 @@
+// Internal launch interface between the C ABI (api.hip) and the kernel translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/fieldfare_moe.h"
+
+namespace ffmoe {
+
+// Geometry of one expert inside the HBM arena. Every expert occupies `expert_bytes`, split into four
+// contiguous regions:
+//   gu_tiles  [F/16][D/64] tiles of 1024 B: lane l (weight row 16*rb + l%16, k-quarter l/16) owns 16 B =
+//             {gate k-half 0, gate k-half 1, up k-half 0, up k-half 1}, each dword eight nibbles
+//   gu_scales [F/16][D/64][16] x {gate scale, gate bias, up scale, up bias} bf16
+//   dn_tiles  [D/32][F/64] tiles of 1024 B: lane owns {row a half 0, row a half 1, row b half 0, row b half 1}
+//             with a = 32*rbp + l%16 and b = a + 16
+//   dn_scales [D/32][F/64][16] x {scale a, bias a, scale b, bias b} bf16
+// A wave reads one tile with one 16-byte load per lane: 1 KiB contiguous.
+struct ArenaGeom {
+    uint32_t d, f;
+    uint32_t gd;          // d / 64: groups along a gate/up row
+    uint32_t gf;          // f / 64: groups along a down row
+    uint32_t gu_rb;       // f / 16: gate/up row blocks
+    uint32_t dn_rbp;      // d / 32: down row-block pairs
+    size_t gu_tiles_off, gu_scales_off, dn_tiles_off, dn_scales_off;
+    size_t expert_bytes;
+};
+
+ArenaGeom make_geom(uint32_t d, uint32_t f);
+
+// Per-call routing plan of a decode / verify block, built on the GPU (no host round trip).
+struct PlanSlot {
+    uint32_t expert;
+    uint32_t n;                               // routes of this expert, 1..16
+    uint32_t routes[FFMOE_MAX_VERIFY_ROWS];   // route = token * top_k + rank
+};
+struct VerifyPlan {
+    uint32_t n_live;
+    uint32_t pad[3];
+    PlanSlot slots[FFMOE_MAX_EXPERTS];
+    uint32_t route_valid[FFMOE_MAX_VERIFY_ROWS * 8];   // 1 when the route was planned (weight != 0, expert in range)
+};
+
+struct RouterWeights {
+    const void *w;          // bf16 [E][D] or float [E][D]
+    int w_is_f32;
+    const uint16_t *effective_scale;   // bf16 [D] or nullptr
+    const uint16_t *per_expert_scale;  // bf16 [E] or nullptr
+};
+
+// repack.hip
+hipError_t launch_repack_layer(hipStream_t s, const uint8_t *blobs, size_t stride, ffmoe_offsets off,
+                               uint32_t n_experts, ArenaGeom g, uint8_t *arena_layer);
+hipError_t launch_dequant_expert(hipStream_t s, const uint8_t *arena_expert, ArenaGeom g, int which,
+                                 uint16_t *out);
+
+// router.hip
+hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
+                         uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
+                         uint16_t *out_w);
+
+// skinny.hip
+hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
+                         uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
+                         const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
+                         VerifyPlan *plan, float *xsum, uint16_t *acts, float *partials_f32);
+hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,
+                                     uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d);
+
+// gemv.hip
+hipError_t launch_gemv_int4(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                            const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows,
+                            uint32_t x_stride, uint32_t y_stride, int y_f32);
+
+}  // namespace ffmoe

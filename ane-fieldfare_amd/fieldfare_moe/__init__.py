@@ -1,0 +1,262 @@
+"""ctypes binding of libfieldfare_moe_hip.so (the C ABI in include/fieldfare_moe.h).
+
+PyTorch is used for device memory and streams only: every method takes torch CUDA tensors, passes
+their raw device pointers through the C ABI, and enqueues on torch's current stream. There is no CPU
+or eager fallback: a missing library raises at import of the symbols, a missing GPU at Context().
+"""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+_PKG = Path(__file__).resolve().parent.parent
+LIB_PATH = _PKG / "libfieldfare_moe_hip.so"
+CSRC = _PKG / "csrc"
+
+OK = 0
+GATE, UP, DOWN = 0, 1, 2
+GROUP = 64
+MAX_VERIFY_ROWS = 16
+
+
+class FieldfareError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"ffmoe status {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+class Shape(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("d", "f", "n_experts", "top_k", "n_layers", "max_tokens")]
+
+
+class Offsets(C.Structure):
+    """MoEExpertOffsets (Kernels/MoE/MoE.swift:4-29)."""
+    _fields_ = [(n, C.c_uint32) for n in
+                ("gate_w", "gate_s", "gate_b", "up_w", "up_s", "up_b", "down_w", "down_s", "down_b")]
+
+
+EXPORTS = [
+    "ffmoe_version", "ffmoe_create", "ffmoe_destroy", "ffmoe_layer_arena_bytes", "ffmoe_upload_layer",
+    "ffmoe_upload_router_bf16", "ffmoe_upload_router_int8", "ffmoe_dequant_expert", "ffmoe_router",
+    "ffmoe_verify", "ffmoe_verify_partials", "ffmoe_last_live_experts", "ffmoe_reduce_token_major",
+    "ffmoe_gemv_int4",
+]
+
+
+def build() -> Path:
+    """Compile the library for gfx950 with the Makefile in csrc/ (hipcc cross-compiles without a GPU)."""
+    subprocess.run(["make", "-C", str(CSRC), "-B", "-j8"], check=True, stdout=subprocess.DEVNULL,
+                   stderr=subprocess.DEVNULL)
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise FileNotFoundError(f"{LIB_PATH} is not built; run __graft_entry__.build() (there is no fallback path)")
+    L = C.CDLL(str(LIB_PATH))
+    vp, u32, sz, i32 = C.c_void_p, C.c_uint32, C.c_size_t, C.c_int
+    errp = C.POINTER(C.c_char_p)
+    L.ffmoe_version.restype = C.c_char_p
+    L.ffmoe_create.argtypes = [i32, C.POINTER(Shape), C.POINTER(vp), errp]
+    L.ffmoe_destroy.argtypes = [vp]
+    L.ffmoe_destroy.restype = None
+    L.ffmoe_layer_arena_bytes.argtypes = [vp]
+    L.ffmoe_layer_arena_bytes.restype = sz
+    L.ffmoe_upload_layer.argtypes = [vp, u32, vp, sz, C.POINTER(Offsets), i32, errp]
+    L.ffmoe_upload_router_bf16.argtypes = [vp, u32, vp, vp, vp, errp]
+    L.ffmoe_upload_router_int8.argtypes = [vp, u32, vp, vp, vp, vp, vp, errp]
+    L.ffmoe_dequant_expert.argtypes = [vp, vp, u32, u32, i32, vp, errp]
+    L.ffmoe_router.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
+    L.ffmoe_verify.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, vp, errp]
+    L.ffmoe_verify_partials.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
+    L.ffmoe_last_live_experts.argtypes = [vp, vp, C.POINTER(u32), errp]
+    L.ffmoe_reduce_token_major.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, errp]
+    L.ffmoe_gemv_int4.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, i32, errp]
+    if hasattr(L, "ffmoe_prefill"):
+        L.ffmoe_prefill.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
+        L.ffmoe_prefill_pairs.argtypes = [vp, vp, u32, vp, u32, vp, u32, u32, vp, errp]
+        L.ffmoe_prefill_plan_stats.argtypes = [vp, vp, vp, errp]
+    _lib = L
+    return L
+
+
+def _check(code: int, err: C.c_char_p):
+    if code != OK:
+        msg = err.value.decode() if err.value else "(no message)"
+        raise FieldfareError(code, msg)
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _row_stride(t):
+    """Row stride in elements; a single-row tensor may report any stride for its size-1 dimension."""
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class Context:
+    """One ffmoe_ctx: the HBM expert arena of `n_layers` layers plus scratch, on one GPU."""
+
+    def __init__(self, d: int, f: int, n_experts: int, top_k: int = 8, n_layers: int = 1, max_tokens: int = 4096,
+                 device: int = 0):
+        import torch
+        if not torch.cuda.is_available():
+            raise RuntimeError("no HIP device visible: the fieldfare MoE kernels have no CPU fallback")
+        self.L = lib()
+        self.shape = Shape(d, f, n_experts, top_k, n_layers, max_tokens)
+        self.device = device
+        self._h = C.c_void_p()
+        err = C.c_char_p()
+        _check(self.L.ffmoe_create(device, C.byref(self.shape), C.byref(self._h), C.byref(err)), err)
+
+    def close(self):
+        if getattr(self, "_h", None) and self._h.value:
+            self.L.ffmoe_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def layer_arena_bytes(self) -> int:
+        return int(self.L.ffmoe_layer_arena_bytes(self._h))
+
+    # -- weights ---------------------------------------------------------------------------------
+    def upload_layer(self, layer: int, blobs, stride: int, offsets: Offsets):
+        """`blobs`: torch uint8 tensor (CPU or CUDA) or numpy uint8 array holding n_experts blobs."""
+        import numpy as np
+        import torch
+        err = C.c_char_p()
+        if isinstance(blobs, np.ndarray):
+            assert blobs.dtype == np.uint8 and blobs.flags["C_CONTIGUOUS"]
+            p, on_dev = C.c_void_p(blobs.ctypes.data), 0
+        else:
+            assert blobs.dtype == torch.uint8 and blobs.is_contiguous()
+            p, on_dev = C.c_void_p(blobs.data_ptr()), int(blobs.is_cuda)
+        _check(self.L.ffmoe_upload_layer(self._h, layer, p, stride, C.byref(offsets), on_dev, C.byref(err)), err)
+
+    def upload_router_bf16(self, layer: int, w_bits, effective_scale_bits=None, per_expert_scale_bits=None):
+        """numpy uint16 arrays (bf16 bit patterns), host side."""
+        import numpy as np
+        err = C.c_char_p()
+        keep = [np.ascontiguousarray(a, np.uint16) if a is not None else None
+                for a in (w_bits, effective_scale_bits, per_expert_scale_bits)]
+        ptrs = [C.c_void_p(a.ctypes.data) if a is not None else None for a in keep]
+        _check(self.L.ffmoe_upload_router_bf16(self._h, layer, *ptrs, C.byref(err)), err)
+
+    def upload_router_int8(self, layer: int, w_u8, scale_bits, bias_bits, effective_scale_bits=None,
+                           per_expert_scale_bits=None):
+        import numpy as np
+        err = C.c_char_p()
+        keep = [np.ascontiguousarray(w_u8, np.uint8)] + [
+            np.ascontiguousarray(a, np.uint16) if a is not None else None
+            for a in (scale_bits, bias_bits, effective_scale_bits, per_expert_scale_bits)]
+        ptrs = [C.c_void_p(a.ctypes.data) if a is not None else None for a in keep]
+        _check(self.L.ffmoe_upload_router_int8(self._h, layer, *ptrs, C.byref(err)), err)
+
+    def dequant_expert(self, layer: int, expert: int, which: int):
+        import torch
+        rows, cols = (self.shape.d, self.shape.f) if which == DOWN else (self.shape.f, self.shape.d)
+        out = torch.empty((rows, cols), dtype=torch.bfloat16, device=f"cuda:{self.device}")
+        err = C.c_char_p()
+        _check(self.L.ffmoe_dequant_expert(self._h, _stream(), layer, expert, which, _ptr(out), C.byref(err)), err)
+        return out
+
+    # -- router ----------------------------------------------------------------------------------
+    def router(self, layer: int, router_x, want_logits: bool = False):
+        """router_x: bf16 [T, stride>=d] CUDA tensor (rows may be strided). Returns (idx i32 [T,K], w bf16 [T,K][, logits])."""
+        import torch
+        assert router_x.dtype == torch.bfloat16 and router_x.is_cuda and router_x.stride(1) == 1
+        t = router_x.shape[0]
+        k, e = self.shape.top_k, self.shape.n_experts
+        idx = torch.empty((t, k), dtype=torch.int32, device=router_x.device)
+        w = torch.empty((t, k), dtype=torch.bfloat16, device=router_x.device)
+        logits = torch.empty((t, e), dtype=torch.float32, device=router_x.device) if want_logits else None
+        err = C.c_char_p()
+        _check(self.L.ffmoe_router(self._h, _stream(), layer, _ptr(router_x), _row_stride(router_x), t, _ptr(idx), _ptr(w),
+                                   _ptr(logits), C.byref(err)), err)
+        return (idx, w, logits) if want_logits else (idx, w)
+
+    # -- routed experts --------------------------------------------------------------------------
+    def verify(self, layer: int, x, idx, w, residual=None, out=None):
+        """Decode step (T = 1) or verify block (T <= 16): fused experts + weighted combine. x bf16 [T, stride]."""
+        import torch
+        t = x.shape[0]
+        y = out if out is not None else torch.empty((t, self.shape.d), dtype=torch.bfloat16, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_verify(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(idx), _ptr(w), _ptr(residual),
+                                   _ptr(y), C.byref(err)), err)
+        return y
+
+    def verify_partials(self, layer: int, x, idx, w, partials=None):
+        import torch
+        t = x.shape[0]
+        if partials is None:
+            partials = torch.zeros((t, self.shape.top_k, self.shape.d), dtype=torch.bfloat16, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_verify_partials(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(idx), _ptr(w),
+                                            _ptr(partials), C.byref(err)), err)
+        return partials
+
+    def last_live_experts(self) -> int:
+        n = C.c_uint32()
+        err = C.c_char_p()
+        _check(self.L.ffmoe_last_live_experts(self._h, _stream(), C.byref(n), C.byref(err)), err)
+        return int(n.value)
+
+    def reduce_token_major(self, partials, weights):
+        import torch
+        t, k, d = partials.shape
+        h2 = torch.empty((t, d), dtype=torch.bfloat16, device=partials.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_reduce_token_major(self._h, _stream(), _ptr(partials), _ptr(weights), _ptr(h2), t, k, d,
+                                               C.byref(err)), err)
+        return h2
+
+    # -- prefill ---------------------------------------------------------------------------------
+    def prefill(self, layer: int, x, idx, w, out=None):
+        import torch
+        t = x.shape[0]
+        y = out if out is not None else torch.empty((t, self.shape.d), dtype=torch.bfloat16, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_prefill(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(idx), _ptr(w), _ptr(y),
+                                    C.byref(err)), err)
+        return y
+
+    def prefill_pairs(self, layer: int, x, sorted_pairs, t: int, partials):
+        """Guest contract: sorted_pairs int32 [n, 4] CUDA tensor of (token, expert, rank, weight bits)."""
+        err = C.c_char_p()
+        _check(self.L.ffmoe_prefill_pairs(self._h, _stream(), layer, _ptr(x), _row_stride(x), _ptr(sorted_pairs),
+                                          sorted_pairs.shape[0], t, _ptr(partials), C.byref(err)), err)
+        return partials
+
+    # -- generic GEMV ----------------------------------------------------------------------------
+    def gemv_int4(self, W, S, B, x, f32_out: bool = False, w_byte_offset: int = 0):
+        """W uint8 [M, N/2] (optionally starting `w_byte_offset` bytes into a larger buffer), S/B bf16-bit
+        int16/uint16 tensors [M, N/64], x bf16 [R, stride]. Returns y [R, M]."""
+        import torch
+        m, n = S.shape[0], S.shape[1] * GROUP
+        rows = x.shape[0]
+        y = torch.empty((rows, m), dtype=torch.float32 if f32_out else torch.bfloat16, device=x.device)
+        err = C.c_char_p()
+        wp = C.c_void_p(W.data_ptr() + w_byte_offset)
+        _check(self.L.ffmoe_gemv_int4(self._h, _stream(), wp, _ptr(S), _ptr(B), _ptr(x), _ptr(y), m, n, rows,
+                                      _row_stride(x), m, int(f32_out), C.byref(err)), err)
+        return y

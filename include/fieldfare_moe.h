@@ -1,0 +1,174 @@
+/*
+ * fieldfare_moe.h - C ABI of libfieldfare_moe_hip.so: the quantized-MoE hot path of
+ * zw5/ane-fieldfare (router top-8 -> INT4 gate/up + GELU-tanh -> INT4 down -> weighted combine,
+ * plus the generic INT4 GEMV) as hand-written CDNA4 (gfx950) HIP kernels.
+ *
+ * Conventions (modelled on Sources/ANEFieldfareANECarrier/include/ANEExpertCarrier.h:14-38 and on
+ * the "encode" methods of the Swift operators this replaces):
+ *   - every compute call ENQUEUES work on the caller's HIP stream (`stream` is a hipStream_t passed
+ *     as void*, NULL = the default stream), returns without waiting, and allocates nothing; the
+ *     stream plays the part of the reference's MTLCommandBuffer;
+ *   - device buffers are caller-owned raw device pointers; scratch lives in the context;
+ *   - return value: FFMOE_OK (0) or a negative status; when `err` is non-NULL and the call fails,
+ *     `*err` receives a strdup'd message the caller releases with free();
+ *   - a context belongs to one host thread at a time (the reference's operators are not Sendable).
+ * Activations, routing weights and outputs are 16-bit: bf16 (FFMOE_BF16), which every kernel
+ * computes in with fp32 accumulation.
+ * All paths below are relative to the reference repository root.
+ */
+#ifndef FIELDFARE_MOE_H
+#define FIELDFARE_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    FFMOE_OK = 0,
+    FFMOE_ERR_INVALID = -1,   /* shape or argument misuse (a Swift precondition in the reference) */
+    FFMOE_ERR_RUNTIME = -2,   /* HIP runtime failure (MetalError / command-buffer error in the reference) */
+    FFMOE_ERR_ALLOC = -3,     /* PrefillGroupedRoutedMoEError.allocationFailed */
+    FFMOE_ERR_NO_LAYER = -4   /* layer not uploaded */
+};
+
+enum { FFMOE_BF16 = 0 };
+
+enum { FFMOE_GATE = 0, FFMOE_UP = 1, FFMOE_DOWN = 2 };
+
+#define FFMOE_GROUP 64          /* Quantization.groupSize, Infrastructure/ModelIO/Quantization.swift:2 */
+#define FFMOE_MAX_VERIFY_ROWS 16 /* maxVerifyTokens, Runtime/Inference/RealForwardRunner.swift:414 */
+#define FFMOE_MAX_EXPERTS 256    /* router limit, Kernels/MoE/MoE.swift:137 */
+
+typedef struct ffmoe_ctx ffmoe_ctx;
+
+/* Model shape of the routed-expert stage. Replaces the Metal function constants of
+ * Kernels/MoE/MoE.swift:34-46 (D = 2816, F = 704, top-k = 8, 128 experts for Gemma-4-26B-A4B). */
+typedef struct {
+    uint32_t d;            /* hidden size, multiple of 64 */
+    uint32_t f;            /* routed intermediate size, multiple of 64 */
+    uint32_t n_experts;    /* <= FFMOE_MAX_EXPERTS */
+    uint32_t top_k;        /* 1..8; the decode/verify kernels of the reference require 8 */
+    uint32_t n_layers;     /* layers the HBM expert arena holds */
+    uint32_t max_tokens;   /* largest T of a prefill call (PrefillRuntimeConfig.maxChunkTokens = 4096) */
+} ffmoe_shape;
+
+/* Byte offsets of the nine sub-tensors inside one expert blob.
+ * Replaces MoEExpertOffsets, Kernels/MoE/MoE.swift:4-29. */
+typedef struct {
+    uint32_t gate_w, gate_s, gate_b;
+    uint32_t up_w, up_s, up_b;
+    uint32_t down_w, down_s, down_b;
+} ffmoe_offsets;
+
+/* One routed (token, expert) pair, 16 bytes.
+ * Replaces PrefillTokenExpertPair, Kernels/Prefill/MoE/PrefillRouter.swift:5-21. */
+typedef struct {
+    uint32_t token, expert, rank, weight_bits_and_reserved;
+} ffmoe_pair;
+
+/* ---- lifetime -------------------------------------------------------------------------------- */
+
+/* Creates the context on HIP device `device`: the HBM expert arena for `n_layers` layers and all
+ * scratch. Replaces the operator constructors MoE.init / PrefillGroupedRoutedMoE.init
+ * (Kernels/MoE/MoE.swift:72-123, Kernels/Prefill/MoE/PrefillGroupedRoutedMoE.swift:208-241). */
+int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **err);
+void ffmoe_destroy(ffmoe_ctx *ctx);
+
+/* Bytes of HBM one layer's experts occupy in the arena (= n_experts * payload). */
+size_t ffmoe_layer_arena_bytes(const ffmoe_ctx *ctx);
+
+/* ---- weights --------------------------------------------------------------------------------- */
+
+/* Copies one layer's expert blobs (reference byte layout: `n_experts` blobs `stride` bytes apart
+ * starting at `blobs`, sub-tensors at `offsets`) into the HBM arena, re-tiled for the MFMA kernels.
+ * `blobs` is host memory (e.g. the mmap of a layer file) when `src_is_device` == 0, else a device
+ * pointer. Blocks until the copy is done. Replaces MappedExpertLayer + the per-expert MTLBuffer
+ * binding (Infrastructure/Streaming/MappedExpertLayer.swift:118-128) and makeReusedRoutedArgumentBuffer
+ * (Kernels/MoE/MoE.swift:302-310): with every expert resident, slots are base + expert * stride. */
+int ffmoe_upload_layer(ffmoe_ctx *ctx, uint32_t layer, const void *blobs, size_t stride,
+                       const ffmoe_offsets *offsets, int src_is_device, char **err);
+
+/* Router weights of one layer: bf16 [n_experts][d] (the benchmark configs' form). Optional bf16
+ * `effective_scale` [d] and `per_expert_scale` [n_experts] (NULL = 1), host pointers.
+ * Replaces the router tensors bound by MoE.encodeRouterGemma4 (Kernels/MoE/MoE.swift:168-180). */
+int ffmoe_upload_router_bf16(ffmoe_ctx *ctx, uint32_t layer, const uint16_t *w,
+                             const uint16_t *effective_scale, const uint16_t *per_expert_scale, char **err);
+/* Same for the reference's INT8-affine router (uint8 [E][d] + bf16 scale/bias per 64,
+ * Metal/MoE/moe.metal:65-103): dequantised once to fp32(q*s + b) at upload. */
+int ffmoe_upload_router_int8(ffmoe_ctx *ctx, uint32_t layer, const uint8_t *w, const uint16_t *scales,
+                             const uint16_t *biases, const uint16_t *effective_scale,
+                             const uint16_t *per_expert_scale, char **err);
+
+/* Expands one sub-tensor (FFMOE_GATE / UP / DOWN) of one expert from the arena to bf16
+ * [rows][cols], each element bf16(q*scale + bias) - the value a matrix-unit tile holds. Replaces
+ * ane_expert_weights (Metal/ANE/ane_prefill.metal:17-36) as the exact-expansion check
+ * (Tests/ANEFieldfareHotpathTests/ANEQuantizedCarrierTests.swift:59-67). */
+int ffmoe_dequant_expert(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint32_t expert, int which,
+                         uint16_t *out_bf16, char **err);
+
+/* ---- router ---------------------------------------------------------------------------------- */
+
+/* logits = W_router . (router_x * effective_scale); top-k by (score desc, index asc); weights =
+ * softmax over the selected scores * per_expert_scale, rounded to bf16. `router_x` is bf16
+ * [t][x_stride]. Writes out_idx uint32 [t][top_k] and out_w bf16 [t][top_k]; out_logits (fp32
+ * [t][n_experts]) may be NULL. Replaces MoE.encodeRouterGemma4 (Kernels/MoE/MoE.swift:168-237),
+ * MoE.encodeRouterRowsGemma4 (:249-300) and PrefillRouter.encodeGemma4Block
+ * (Kernels/Prefill/MoE/PrefillRouter.swift:30-73). */
+int ffmoe_router(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *router_x,
+                 uint32_t x_stride, uint32_t t, uint32_t *out_idx, uint16_t *out_w, float *out_logits,
+                 char **err);
+
+/* ---- routed experts, decode and verify block (t <= 16) ---------------------------------------- */
+
+/* y[t] = bf16(residual[t] + sum_r w[t][r] * down_e(gelu_tanh(gate_e x[t]) * up_e x[t])), e = idx[t][r].
+ * Tokens that share an expert are batched against one read of its weights. `x` bf16 [t][x_stride],
+ * `idx` uint32 [t][top_k], `w` bf16 [t][top_k], `residual` bf16 [t][d] or NULL, `y` bf16 [t][d]; all
+ * device pointers. t == 1 replaces MoE.encodeRoutedPersistentPhase1U16Load + ...Phase2Reduce and
+ * encodeGatherRoutedSlots / encodeRoutedPersistentGPUSlots (Kernels/MoE/MoE.swift:312-496); t <= 16
+ * replaces PrefillGroupedRoutedMoE.encodeVerifyBound / encodeVerifyRows
+ * (Kernels/Prefill/MoE/PrefillGroupedRoutedMoE.swift:331-448) followed by
+ * PrefillMoE.encodeReduceTokenMajor. Routes whose weight is exactly zero are skipped. */
+int ffmoe_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
+                 uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual,
+                 uint16_t *y, char **err);
+
+/* Same expert pass, but writes the un-weighted per-route rows bf16 partials[(token*top_k+rank)*d ...]
+ * the way the reference's verify and prefill kernels hand them to the reduce
+ * (Metal/Prefill/prefill.metal:1372-1374, Runtime/Supervisor/DeviceSupervisor.swift:14-17). */
+int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x,
+                          uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
+                          uint16_t *partials, char **err);
+
+/* Number of distinct experts the last ffmoe_verify* call on `stream` ran (reads back 4 bytes; waits
+ * for the stream). For reporting only. */
+int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char **err);
+
+/* ---- weighted combine ------------------------------------------------------------------------- */
+
+/* h2[t][c] = bf16(sum_r w[t][r] * partials[t][r][c]), fma in rank order.
+ * Replaces PrefillMoE.encodeReduceTokenMajor (Kernels/Prefill/MoE/PrefillMoE.swift:11-32,
+ * Metal/Prefill/prefill.metal:544-565). */
+int ffmoe_reduce_token_major(ffmoe_ctx *ctx, void *stream, const uint16_t *partials,
+                             const uint16_t *weights, uint16_t *h2, uint32_t t, uint32_t top_k,
+                             uint32_t d, char **err);
+
+/* ---- generic INT4 GEMV (reference layout: W uint8 [m][n/2], S/B bf16 [m][n/64]) ---------------- */
+
+/* y[r][row] = bf16(sum_k (q*scale + bias)[row][k] * x[r][k]) for r < rows <= 16, weights read once.
+ * Row r equals the rows == 1 result bit for bit. Replaces DequantInt4GEMV.encode / encodeRows
+ * (Kernels/Quant/DequantInt4GEMV.swift:72-123,184-224) and the LM-head GEMV
+ * (Metal/Sampling/logit.metal:614-667). `w` needs 2-byte alignment only; 16-byte aligned rows take
+ * the wide-load path. y_f32 != 0 writes fp32 logits instead of bf16 (RowsTypes.f16ToF32). */
+int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16_t *scales,
+                    const uint16_t *biases, const uint16_t *x, void *y, uint32_t m, uint32_t n,
+                    uint32_t rows, uint32_t x_stride, uint32_t y_stride, int y_f32, char **err);
+
+const char *ffmoe_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
