@@ -35,6 +35,7 @@ struct ffmoe_ctx {
     float *xsum = nullptr;           // [16][D/64]
     uint16_t *acts = nullptr;        // [16*top_k][F]
     float *partials = nullptr;       // [16*top_k][D]
+    KernelTimer timer;
 };
 
 namespace {
@@ -144,6 +145,8 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (ctx->xsum) (void)hipFree(ctx->xsum);
     if (ctx->acts) (void)hipFree(ctx->acts);
     if (ctx->partials) (void)hipFree(ctx->partials);
+    for (auto &ev : ctx->timer.ev)
+        if (ev) (void)hipEventDestroy(ev);
     delete ctx;
 }
 
@@ -257,7 +260,7 @@ int ffmoe_router(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *r
     const ffmoe_layer &l = ctx->layers[layer];
     RouterWeights rw{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale};
     FF_HIP(launch_router(static_cast<hipStream_t>(stream), rw, router_x, x_stride, t, ctx->shape.n_experts,
-                         ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w));
+                         ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w, &ctx->timer));
     return FFMOE_OK;
 }
 
@@ -274,7 +277,7 @@ static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uin
         return fail(err, FFMOE_ERR_INVALID, "y and residual must be 8-byte aligned");
     FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                         ctx->plan, ctx->xsum, ctx->acts, ctx->partials));
+                         ctx->plan, ctx->xsum, ctx->acts, ctx->partials, &ctx->timer));
     return FFMOE_OK;
 }
 
@@ -295,6 +298,24 @@ int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char
     if (!n_live) return fail(err, FFMOE_ERR_INVALID, "null argument");
     FF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     FF_HIP(hipMemcpy(n_live, &ctx->plan->n_live, sizeof(uint32_t), hipMemcpyDeviceToHost));
+    return FFMOE_OK;
+}
+
+int ffmoe_set_profiling(ffmoe_ctx *ctx, int enabled, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (enabled && !ctx->timer.ev[0])
+        for (auto &ev : ctx->timer.ev) FF_HIP(hipEventCreate(&ev));
+    ctx->timer.on = enabled != 0;
+    return FFMOE_OK;
+}
+
+int ffmoe_get_profile(ffmoe_ctx *ctx, ffmoe_profile *out, int reset, char **err) {
+    if (!ctx || !out) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    for (int i = 0; i < FFMOE_PROFILE_SLOTS; ++i) {
+        out->ms[i] = ctx->timer.ms[i];
+        out->launches[i] = ctx->timer.launches[i];
+        if (reset) { ctx->timer.ms[i] = 0; ctx->timer.launches[i] = 0; }
+    }
     return FFMOE_OK;
 }
 
@@ -319,7 +340,10 @@ int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16
     if (m == 0) return fail(err, FFMOE_ERR_INVALID, "M must be positive");
     if (rows == 0 || rows > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows=%u outside 1...%d", rows, FFMOE_MAX_VERIFY_ROWS);
     if (x_stride < n || y_stride < m) return fail(err, FFMOE_ERR_INVALID, "stride smaller than the row");
+    ctx->timer.begin(static_cast<hipStream_t>(stream));
     FF_HIP(launch_gemv_int4(static_cast<hipStream_t>(stream), w, scales, biases, x, y, m, n, rows, x_stride, y_stride, y_f32));
+    ctx->timer.mark(static_cast<hipStream_t>(stream), FFMOE_K_GEMV);
+    ctx->timer.finish();
     return FFMOE_OK;
 }
 

@@ -43,6 +43,40 @@ struct VerifyPlan {
     uint32_t route_valid[FFMOE_MAX_VERIFY_ROWS * 8];   // 1 when the route was planned (weight != 0, expert in range)
 };
 
+// Per-kernel GPU timing with HIP events on the caller's stream, switched on by ffmoe_set_profiling.
+// The counterpart of the reference's traced compute encoders (Infrastructure/Metal/GPUTrace.swift:19-115).
+struct KernelTimer {
+    bool on = false;
+    hipEvent_t ev[12] = {};
+    int ids[12] = {};
+    int n = 0;
+    double ms[FFMOE_PROFILE_SLOTS] = {};
+    uint64_t launches[FFMOE_PROFILE_SLOTS] = {};
+    void begin(hipStream_t s) {
+        n = 0;
+        if (on) (void)hipEventRecord(ev[0], s);
+    }
+    // call right after launching kernel `id`
+    void mark(hipStream_t s, int id) {
+        if (!on || n >= 11) return;
+        ids[n] = id;
+        (void)hipEventRecord(ev[++n], s);
+    }
+    // waits for the stream: profiling mode trades asynchrony for per-kernel times
+    void finish() {
+        if (!on || n == 0) return;
+        (void)hipEventSynchronize(ev[n]);
+        for (int i = 0; i < n; ++i) {
+            float t = 0.f;
+            if (hipEventElapsedTime(&t, ev[i], ev[i + 1]) == hipSuccess) {
+                ms[ids[i]] += t;
+                launches[ids[i]] += 1;
+            }
+        }
+        n = 0;
+    }
+};
+
 struct RouterWeights {
     const void *w;          // bf16 [E][D] or float [E][D]
     int w_is_f32;
@@ -59,13 +93,13 @@ hipError_t launch_dequant_expert(hipStream_t s, const uint8_t *arena_expert, Are
 // router.hip
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w);
+                         uint16_t *out_w, KernelTimer *timer);
 
 // skinny.hip
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
-                         VerifyPlan *plan, float *xsum, uint16_t *acts, float *partials_f32);
+                         VerifyPlan *plan, float *xsum, uint16_t *acts, float *partials_f32, KernelTimer *timer);
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,
                                      uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d);
 

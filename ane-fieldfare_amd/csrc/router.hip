@@ -113,7 +113,8 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *__restrict
 
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w) {
+                         uint16_t *out_w, KernelTimer *timer) {
+    timer->begin(s);
     const dim3 grid((n_experts + 3) / 4, (t + kRouterTokens - 1) / kRouterTokens);
     if (rw.w_is_f32)
         hipLaunchKernelGGL(router_logits_kernel<true>, grid, dim3(256), 0, s, rw.w, rw.effective_scale, x,
@@ -123,8 +124,11 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
                            x_stride, t, n_experts, d, logits);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
+    timer->mark(s, FFMOE_K_ROUTER_LOGITS);
     hipLaunchKernelGGL(router_topk_kernel, dim3(t), dim3(64), 0, s, logits, rw.per_expert_scale, n_experts,
                        top_k, out_idx, out_w);
+    timer->mark(s, FFMOE_K_ROUTER_TOPK);
+    timer->finish();
     return hipGetLastError();
 }
 

@@ -320,11 +320,13 @@ __global__ __launch_bounds__(256) void reduce_token_major_kernel(const uint16_t 
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
-                         VerifyPlan *plan, float *xsum, uint16_t *acts, float *partials_f32) {
+                         VerifyPlan *plan, float *xsum, uint16_t *acts, float *partials_f32, KernelTimer *timer) {
+    timer->begin(s);
     hipLaunchKernelGGL(verify_plan_kernel, dim3(1), dim3(256), 0, s, idx, w, t, top_k, n_experts, x, x_stride,
                        g.gd, plan, xsum);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
+    timer->mark(s, FFMOE_K_PLAN);
     const uint32_t slots = min(n_experts, t * top_k);
     const size_t sum_bytes_gu = (size_t)g.gd * kMaxRows * sizeof(float);
     if (slots <= 16) {
@@ -338,19 +340,25 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
     }
     e = hipGetLastError();
     if (e != hipSuccess) return e;
+    timer->mark(s, FFMOE_K_GATE_UP);
     const size_t sum_bytes_dn = (size_t)g.gf * kMaxRows * sizeof(float);
     const dim3 dn_grid((g.dn_rbp + 3) / 4, slots);
     if (partials_bf16) {
         hipLaunchKernelGGL(skinny_down_kernel<true>, dn_grid, dim3(256), sum_bytes_dn, s, arena_layer, g, plan,
                            acts, partials_f32, partials_bf16);
+        timer->mark(s, FFMOE_K_DOWN);
+        timer->finish();
         return hipGetLastError();
     }
     hipLaunchKernelGGL(skinny_down_kernel<false>, dn_grid, dim3(256), sum_bytes_dn, s, arena_layer, g, plan, acts,
                        partials_f32, partials_bf16);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
+    timer->mark(s, FFMOE_K_DOWN);
     hipLaunchKernelGGL(combine_kernel, dim3((g.d / 4 + 255) / 256, t), dim3(256), 0, s, partials_f32, w,
                        plan->route_valid, residual, top_k, g.d, y);
+    timer->mark(s, FFMOE_K_COMBINE);
+    timer->finish();
     return hipGetLastError();
 }
 

@@ -41,8 +41,16 @@ EXPORTS = [
     "ffmoe_version", "ffmoe_create", "ffmoe_destroy", "ffmoe_layer_arena_bytes", "ffmoe_upload_layer",
     "ffmoe_upload_router_bf16", "ffmoe_upload_router_int8", "ffmoe_dequant_expert", "ffmoe_router",
     "ffmoe_verify", "ffmoe_verify_partials", "ffmoe_last_live_experts", "ffmoe_reduce_token_major",
-    "ffmoe_gemv_int4",
+    "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile",
 ]
+
+PROFILE_SLOTS = 12
+KERNEL_NAMES = ["router_logits", "router_topk", "plan", "gate_up", "down", "combine", "prefill_sort",
+                "prefill_gate_up", "prefill_down", "prefill_combine", "gemv", "reserved"]
+
+
+class Profile(C.Structure):
+    _fields_ = [("ms", C.c_double * PROFILE_SLOTS), ("launches", C.c_uint64 * PROFILE_SLOTS)]
 
 
 def build() -> Path:
@@ -80,6 +88,8 @@ def lib() -> C.CDLL:
     L.ffmoe_last_live_experts.argtypes = [vp, vp, C.POINTER(u32), errp]
     L.ffmoe_reduce_token_major.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, errp]
     L.ffmoe_gemv_int4.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, i32, errp]
+    L.ffmoe_set_profiling.argtypes = [vp, i32, errp]
+    L.ffmoe_get_profile.argtypes = [vp, C.POINTER(Profile), i32, errp]
     if hasattr(L, "ffmoe_prefill"):
         L.ffmoe_prefill.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
         L.ffmoe_prefill_pairs.argtypes = [vp, vp, u32, vp, u32, vp, u32, u32, vp, errp]
@@ -137,6 +147,18 @@ class Context:
     @property
     def layer_arena_bytes(self) -> int:
         return int(self.L.ffmoe_layer_arena_bytes(self._h))
+
+    # -- per-kernel timing -----------------------------------------------------------------------
+    def set_profiling(self, enabled: bool):
+        err = C.c_char_p()
+        _check(self.L.ffmoe_set_profiling(self._h, int(enabled), C.byref(err)), err)
+
+    def profile(self, reset: bool = True) -> dict:
+        """{kernel: (total ms, launches)} accumulated while profiling was enabled."""
+        p = Profile()
+        err = C.c_char_p()
+        _check(self.L.ffmoe_get_profile(self._h, C.byref(p), int(reset), C.byref(err)), err)
+        return {KERNEL_NAMES[i]: (p.ms[i], int(p.launches[i])) for i in range(PROFILE_SLOTS) if p.launches[i]}
 
     # -- weights ---------------------------------------------------------------------------------
     def upload_layer(self, layer: int, blobs, stride: int, offsets: Offsets):

@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-MoE hot path on one MI355X.
+
+Workload (BASELINE.json config 3, the one the metric is quoted on): a 16-token DFlash verify block
+through one Gemma-4-26B-A4B-shaped MoE layer (hidden 2816, 128 experts of intermediate 704, top-8
+softmax router, MLX-affine INT4 g64 experts), synthetic seeded weights and inputs. A step is one pass
+of the hot path over one block: router logits + top-8, GPU-side route planning, gate/up + GELU-tanh
+gating, down projection, router-weighted combine. Steps cycle over `--layers` distinct resident layers
+(default 30 = 12.85 GB of experts) so that no step finds its experts in the 256 MB Infinity Cache.
+
+Prints ONE JSON line. `value` = INT4 expert bytes the step streams (distinct experts x 3,345,408 B)
+divided by the whole step time, inputs resident in HBM. `roofline` prices the dominant kernel
+(gate/up) against the 8 TB/s HBM peak from HIP-event timings; `cpu_baseline` times the CPU oracle
+(a C restatement of the reference's Swift test-support CPU path) on the same block.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (ROOT, ROOT / "ane-fieldfare_amd"):
+    if str(p) not in sys.path:
+        sys.path.insert(0, str(p))
+
+import numpy as np
+
+D, F, E, K = 2816, 704, 128, 8
+STRIDE = 3_358_720                       # 205 x 16 KiB per expert blob (reference layout)
+EXPERT_BYTES = 3_345_408                 # gate + up + down weights, scales and biases of one expert
+GATE_UP_BYTES = 2_230_272                # the share the gate/up kernel streams per expert
+DOWN_BYTES = 1_115_136
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+TOKEN_CORRELATION = 0.45                 # shared component of the block's tokens -> 40-60 distinct experts
+
+
+def synth_layer_gpu(torch, gen, offsets):
+    """One layer of experts in the reference blob layout, generated on the GPU: q ~ U{0..15},
+    scale = bf16(|N(0, 0.01)|), bias = bf16(-8 scale + N(0, 1e-3))."""
+    blob = torch.zeros((E, STRIDE), dtype=torch.uint8, device="cuda")
+    offs = offsets.as_tuple()
+    for i, (rows, cols) in enumerate(((F, D), (F, D), (D, F))):
+        wo, so, bo = offs[3 * i:3 * i + 3]
+        nw, ns = rows * cols // 2, rows * (cols // 64)
+        blob[:, wo:wo + nw] = torch.randint(0, 256, (E, nw), dtype=torch.uint8, device="cuda", generator=gen)
+        s = (torch.randn((E, ns), device="cuda", generator=gen) * 0.01).abs().to(torch.bfloat16)
+        b = (-8.0 * s.float() + torch.randn((E, ns), device="cuda", generator=gen) * 1e-3).to(torch.bfloat16)
+        blob[:, so:so + 2 * ns] = s.view(torch.uint8).view(E, 2 * ns)
+        blob[:, bo:bo + 2 * ns] = b.view(torch.uint8).view(E, 2 * ns)
+    return blob
+
+
+def block_tokens(rng, t):
+    c = rng.normal(0, 1, D)
+    n = rng.normal(0, 1, (t, D))
+    return (np.sqrt(TOKEN_CORRELATION) * c + np.sqrt(1 - TOKEN_CORRELATION) * n).astype(np.float32)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=120)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--layers", type=int, default=30)
+    ap.add_argument("--tokens", type=int, default=16)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the one-GPU hot path only; --gpus must be 1 "
+              "(the path has no collective: see DESIGN.md on how it would shard)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import fieldfare_moe as ff
+    from oracle import oracle
+
+    assert torch.cuda.is_available(), "bench.py needs a HIP device"
+    torch.cuda.set_device(0)
+    L, T = args.layers, args.tokens
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    rng = np.random.default_rng(0)
+    offsets, payload = oracle.layout_offsets(D, F, align=16)
+    assert payload == EXPERT_BYTES
+    ff_off = ff.Offsets(*offsets.as_tuple())
+
+    ctx = ff.Context(D, F, E, K, n_layers=L, max_tokens=4096)
+    host_layer0 = None
+    routers = []
+    for layer in range(L):
+        blob = synth_layer_gpu(torch, gen, offsets)
+        ctx.upload_layer(layer, blob.view(-1), STRIDE, ff_off)
+        if layer == 0:
+            host_layer0 = blob.view(-1).cpu().numpy()
+        del blob
+        r = oracle.bf16_bits(rng.normal(0, 0.02, (E, D)).astype(np.float32))
+        routers.append(r)
+        ctx.upload_router_bf16(layer, r)
+    torch.cuda.empty_cache()
+
+    xb = oracle.bf16_bits(block_tokens(rng, T))
+    x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
+    idx = torch.empty((T, K), dtype=torch.int32, device="cuda")
+    w = torch.empty((T, K), dtype=torch.bfloat16, device="cuda")
+    y = torch.empty((T, D), dtype=torch.bfloat16, device="cuda")
+
+    import ctypes as C
+    Lib, h = ctx.L, ctx._h
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    px, pidx, pw, py = (C.c_void_p(t_.data_ptr()) for t_ in (x, idx, w, y))
+    err = C.c_char_p()
+
+    def step(layer):
+        rc = Lib.ffmoe_router(h, stream, layer, px, D, T, pidx, pw, None, C.byref(err))
+        rc |= Lib.ffmoe_verify(h, stream, layer, px, D, T, pidx, pw, None, py, C.byref(err))
+        if rc:
+            raise RuntimeError(err.value)
+
+    # distinct experts per layer for this block (decides the algorithmic bytes of each step)
+    live = []
+    for layer in range(L):
+        step(layer)
+        live.append(ctx.last_live_experts())
+    for i in range(args.warmup):
+        step(i % L)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i % L)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    bytes_total = sum(live[i % L] for i in range(args.steps)) * EXPERT_BYTES
+    value = bytes_total / elapsed / 1e9
+
+    # per-kernel times (HIP events on the launch stream) for the same steps
+    ctx.set_profiling(True)
+    ctx.profile(reset=True)
+    for i in range(args.steps):
+        step(i % L)
+    prof = ctx.profile(reset=True)
+    ctx.set_profiling(False)
+    gu_ms, gu_n = prof["gate_up"]
+    gu_bytes = sum(live[i % L] for i in range(args.steps)) * GATE_UP_BYTES
+    achieved = gu_bytes / (gu_ms * 1e-3) / 1e9
+    kernel_us = {k: round(v[0] / v[1] * 1e3, 2) for k, v in prof.items()}
+    dn_ms, _ = prof["down"]
+    down_gbs = sum(live[i % L] for i in range(args.steps)) * DOWN_BYTES / (dn_ms * 1e-3) / 1e9
+
+    # secondary figures: decode step (T = 1) and config-1 GEMV
+    extra = {}
+    x1 = x[:1].contiguous()
+    px1 = C.c_void_p(x1.data_ptr())
+
+    def decode(layer):
+        Lib.ffmoe_router(h, stream, layer, px1, D, 1, pidx, pw, None, C.byref(err))
+        Lib.ffmoe_verify(h, stream, layer, px1, D, 1, pidx, pw, None, py, C.byref(err))
+    for i in range(L):
+        decode(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(4 * L):
+        decode(i % L)
+    torch.cuda.synchronize()
+    dec = (time.perf_counter() - t0) / (4 * L)
+    extra["decode_us_per_layer"] = round(dec * 1e6, 2)
+    extra["decode_expert_GBs"] = round(K * EXPERT_BYTES / dec / 1e9, 1)
+
+    cpu = None
+    if not args.no_cpu:
+        pool = oracle.ExpertPool(host_layer0, offsets, STRIDE, D, F)
+        threads = min(16, oracle.max_threads())
+        t0 = time.perf_counter()
+        ridx, rw, ry = oracle.moe_layer(pool, routers[0], xb, K, threads=1)
+        single = time.perf_counter() - t0
+        reps = 0
+        t0 = time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0) * threads < 12.0:
+            oracle.moe_layer(pool, routers[0], xb, K, threads=threads)
+            reps += 1
+        multi = (time.perf_counter() - t0) / reps
+        cpu_bytes = len(np.unique(ridx)) * EXPERT_BYTES
+        cpu = {"value": round(cpu_bytes / multi / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+               "sample": f"layer 0 of the same 16-token block, {reps} reps on {threads} threads "
+                         f"({multi * 1e3:.1f} ms each); 1 thread: {single * 1e3:.0f} ms = "
+                         f"{cpu_bytes / single / 1e9:.3f} GB/s; C restatement of the reference's Swift CPU "
+                         f"dequant+matmul path, gcc -O3 -march=x86-64-v3"}
+        # the GPU result of layer 0 against that CPU result: the bench measures a correct path
+        step(0)
+        torch.cuda.synchronize()
+        got = oracle.bf16_to_float(y.view(torch.int16).cpu().numpy().view(np.uint16))
+        assert np.array_equal(idx.cpu().numpy().astype(np.uint32), ridx), "top-k indices differ from the oracle"
+        rel = float(np.abs(got - ry).max() / np.abs(ry).max())
+        assert rel <= 1e-2, f"layer output differs from the oracle: rel err {rel}"
+        extra["parity_rel_err_layer0"] = round(rel, 5)
+
+    out = {
+        "metric": "MoE-layer INT4 weight GB/s (% HBM peak) @16-tok verify; prefill MoE tok/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config 3: {T}-token DFlash verify block through one MoE layer, hidden {D}, "
+                               f"{E} experts x intermediate {F}, top-{K}, INT4 g64; steps cycle {L} resident layers",
+                   "tokens": T, "layers_resident": L, "distinct_experts_mean": round(float(np.mean(live)), 1),
+                   "distinct_experts_min": int(min(live)), "distinct_experts_max": int(max(live)),
+                   "expert_bytes_per_step_mean": int(np.mean(live) * EXPERT_BYTES)},
+        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "roofline": {"bound": "hbm", "kernel": "skinny_gate_up_kernel", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "avg_kernel_us": kernel_us.get("gate_up")},
+        "kernel_us": kernel_us,
+        "down_kernel_GBs": round(down_gbs, 1),
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(out))
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -166,6 +166,27 @@ int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16
                     const uint16_t *biases, const uint16_t *x, void *y, uint32_t m, uint32_t n,
                     uint32_t rows, uint32_t x_stride, uint32_t y_stride, int y_f32, char **err);
 
+/* ---- per-kernel timing ------------------------------------------------------------------------ */
+
+/* Kernel slots of ffmoe_profile. */
+enum {
+    FFMOE_K_ROUTER_LOGITS = 0, FFMOE_K_ROUTER_TOPK, FFMOE_K_PLAN, FFMOE_K_GATE_UP, FFMOE_K_DOWN,
+    FFMOE_K_COMBINE, FFMOE_K_PREFILL_SORT, FFMOE_K_PREFILL_GATE_UP, FFMOE_K_PREFILL_DOWN,
+    FFMOE_K_PREFILL_COMBINE, FFMOE_K_GEMV, FFMOE_PROFILE_SLOTS = 12
+};
+typedef struct {
+    double ms[FFMOE_PROFILE_SLOTS];          /* summed GPU time per kernel slot */
+    uint64_t launches[FFMOE_PROFILE_SLOTS];
+} ffmoe_profile;
+
+/* While enabled, every compute call brackets each of its kernels with HIP events on the caller's
+ * stream and WAITS for the call to finish, adding the elapsed times to the context's profile.
+ * Replaces ANE_FIELDFARE_GPU_TRACE / makeTracedComputeEncoder
+ * (Infrastructure/Metal/GPUTrace.swift:19-115) and the runner's cumulative nanosecond counters
+ * (Runtime/Inference/RealForwardRunner.swift:171-203). */
+int ffmoe_set_profiling(ffmoe_ctx *ctx, int enabled, char **err);
+int ffmoe_get_profile(ffmoe_ctx *ctx, ffmoe_profile *out, int reset, char **err);
+
 const char *ffmoe_version(void);
 
 #ifdef __cplusplus
