@@ -32,7 +32,7 @@ struct ffmoe_ctx {
     // scratch (owned by the context, sized at creation; calls on one context must not overlap)
     float *logits = nullptr;         // [max(max_tokens,16)][E]
     VerifyPlan *plan = nullptr;
-    float *xsum = nullptr;           // [16][D/64]
+    uint32_t *counters = nullptr;    // completion counters of the fused router (self-resetting)
     uint16_t *acts = nullptr;        // [16*top_k][F]
     float *partials = nullptr;       // [16*top_k][D]
     KernelTimer timer;
@@ -118,7 +118,8 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->logits), (size_t)router_rows * shape->n_experts * sizeof(float));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->plan), sizeof(VerifyPlan));
     if (e == hipSuccess) e = hipMemset(ctx->plan, 0, sizeof(VerifyPlan));
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->xsum), (size_t)FFMOE_MAX_VERIFY_ROWS * ctx->geom.gd * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->counters), 64 * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMemset(ctx->counters, 0, 64 * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->acts), routes * shape->f * sizeof(uint16_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->partials), routes * shape->d * sizeof(float));
     if (e != hipSuccess) {
@@ -142,7 +143,7 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (ctx->arena) (void)hipFree(ctx->arena);
     if (ctx->logits) (void)hipFree(ctx->logits);
     if (ctx->plan) (void)hipFree(ctx->plan);
-    if (ctx->xsum) (void)hipFree(ctx->xsum);
+    if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->acts) (void)hipFree(ctx->acts);
     if (ctx->partials) (void)hipFree(ctx->partials);
     for (auto &ev : ctx->timer.ev)
@@ -260,7 +261,7 @@ int ffmoe_router(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *r
     const ffmoe_layer &l = ctx->layers[layer];
     RouterWeights rw{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale};
     FF_HIP(launch_router(static_cast<hipStream_t>(stream), rw, router_x, x_stride, t, ctx->shape.n_experts,
-                         ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w, &ctx->timer));
+                         ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w, ctx->counters, &ctx->timer));
     return FFMOE_OK;
 }
 
@@ -277,7 +278,7 @@ static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uin
         return fail(err, FFMOE_ERR_INVALID, "y and residual must be 8-byte aligned");
     FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                         ctx->plan, ctx->xsum, ctx->acts, ctx->partials, &ctx->timer));
+                         ctx->plan, ctx->acts, ctx->partials, &ctx->timer));
     return FFMOE_OK;
 }
 

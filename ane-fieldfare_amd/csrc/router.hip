@@ -4,129 +4,247 @@
 // prefill_router_gemma4_block (Metal/Prefill/prefill.metal:447-542).
 //
 // Summation order (fixed so that a CPU restatement reproduces every logit bit for bit, which makes the
-// selected indices exact): lane l of a 64-lane wave accumulates k = l + 64 i for increasing i with
-// fmaf, then a xor-butterfly (masks 32..1) of plain adds combines the 64 partials.
+// selected indices exact): lane l of a 64-lane wave owns the elements k = 256 i + 4 l + j (j = 0..3) and
+// accumulates them with fmaf in increasing i, then j; a xor-butterfly (masks 32..1) of plain adds
+// combines the 64 partials. Four consecutive elements per lane make every load 8 bytes wide.
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace ffmoe {
 namespace {
 
-constexpr int kRouterTokens = 16;   // tokens per block row
-
-template <bool W_F32>
-__global__ __launch_bounds__(256) void router_logits_kernel(const void *__restrict__ w_, const uint16_t *__restrict__ es,
-                                                            const uint16_t *__restrict__ x, uint32_t x_stride,
-                                                            uint32_t t, uint32_t n_experts, uint32_t d,
-                                                            float *__restrict__ logits) {
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t e = blockIdx.x * 4 + wave;
-    const uint32_t t0 = blockIdx.y * kRouterTokens;
-    if (e >= n_experts) return;
-    const uint32_t nt = min((uint32_t)kRouterTokens, t - t0);
-    float acc[kRouterTokens];
-#pragma unroll
-    for (int r = 0; r < kRouterTokens; ++r) acc[r] = 0.0f;
-    const uint32_t steps = d / 64;
-    for (uint32_t i = 0; i < steps; ++i) {
-        const uint32_t k = lane + 64 * i;
-        float wv;
-        if (W_F32) wv = reinterpret_cast<const float *>(w_)[(size_t)e * d + k];
-        else wv = bf16_to_f32(reinterpret_cast<const uint16_t *>(w_)[(size_t)e * d + k]);
-        const float sc = es ? bf16_to_f32(es[k]) : 1.0f;
-#pragma unroll
-        for (int r = 0; r < kRouterTokens; ++r) {
-            // rows past the block's last token re-read that token: same arithmetic, result unused
-            const uint32_t row = t0 + min((uint32_t)r, nt - 1);
-            float xv = bf16_to_f32(x[(size_t)row * x_stride + k]);
-            if (es) xv = xv * sc;     // product of two bf16 values: exact in fp32 (moe.metal:96-97)
-            acc[r] = __builtin_fmaf(wv, xv, acc[r]);
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < kRouterTokens; ++r) {
-        const float v = wave_butterfly_sum(acc[r]);
-        if (lane == 0 && (uint32_t)r < nt) logits[(size_t)(t0 + r) * n_experts + e] = v;
-    }
-}
+constexpr int kChunkTokens = 4;      // token rows a wave keeps in flight at once
 
 __device__ __forceinline__ uint32_t orderable(float v) {
     const uint32_t u = __float_as_uint(v);
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-// One wave per token. Candidate e lives in lane e % 64, slot e / 64 (E <= 256). top_k rounds of a
-// wave-wide argmax over the total order (score desc, index asc); scores <= -inf and NaN are never
-// taken; empty rounds give (index 0, -inf) and weight 0 (moe.metal:194-236).
-__global__ __launch_bounds__(64) void router_topk_kernel(const float *__restrict__ logits,
-                                                         const uint16_t *__restrict__ per_expert_scale,
-                                                         uint32_t n_experts, uint32_t top_k,
-                                                         uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w) {
-    const uint32_t lane = threadIdx.x, tok = blockIdx.x;
-    const float *row = logits + (size_t)tok * n_experts;
+// One wave: candidate e lives in lane e % 64, slot e / 64 (E <= 256). top_k rounds of a wave-wide
+// argmax over the total order (score desc, index asc); scores <= -inf and NaN are never taken; empty
+// rounds give (index 0, -inf) and weight 0 (moe.metal:194-236). 
+__device__ __forceinline__ void wave_topk(const float *row, const uint16_t *__restrict__ per_expert_scale,
+                                          uint32_t n_experts, uint32_t top_k, uint32_t *__restrict__ out_idx,
+                                          uint16_t *__restrict__ out_w, uint32_t lane) {
     unsigned long long key[4];
+    float val[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         const uint32_t e = c * 64 + lane;
-        float v = e < n_experts ? row[e] : -INFINITY;
-        const bool live = (v > -INFINITY);   // false for NaN and -inf
-        key[c] = live ? (((unsigned long long)orderable(v) << 32) | (0xFFFFFFFFu - e)) : 0ull;
+        val[c] = e < n_experts ? row[e] : -INFINITY;
+        const bool live = (val[c] > -INFINITY);   // false for NaN and -inf
+        key[c] = live ? (((unsigned long long)orderable(val[c]) << 32) | (0xFFFFFFFFu - e)) : 0ull;
     }
     uint32_t top_idx[8];
     float top_score[8];
-    for (uint32_t r = 0; r < top_k; ++r) {
-        unsigned long long best = key[0];
 #pragma unroll
-        for (int c = 1; c < 4; ++c) best = key[c] > best ? key[c] : best;
+    for (uint32_t r = 0; r < 8; ++r) {
+        if (r < top_k) {
+            unsigned long long best = key[0];
 #pragma unroll
-        for (int m = 32; m >= 1; m >>= 1) {
-            const unsigned long long o = __shfl_xor(best, m, 64);
-            best = o > best ? o : best;
-        }
-        if (best == 0ull) {
-            top_idx[r] = 0;
-            top_score[r] = -INFINITY;
-        } else {
-            const uint32_t e = 0xFFFFFFFFu - (uint32_t)best;
-            top_idx[r] = e;
-            top_score[r] = row[e];
+            for (int c = 1; c < 4; ++c) best = key[c] > best ? key[c] : best;
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
-                if (key[c] == best) key[c] = 0ull;
+            for (int m = 32; m >= 1; m >>= 1) {
+                const unsigned long long o = __shfl_xor(best, m, 64);
+                best = o > best ? o : best;
+            }
+            if (best == 0ull) {
+                top_idx[r] = 0;
+                top_score[r] = -INFINITY;
+            } else {
+                const uint32_t e = 0xFFFFFFFFu - (uint32_t)best;
+                top_idx[r] = e;
+                // recover the score from the key: orderable() is a bijection
+                const uint32_t o = (uint32_t)(best >> 32);
+                top_score[r] = __uint_as_float((o & 0x80000000u) ? (o & 0x7FFFFFFFu) : ~o);
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    if (key[c] == best) key[c] = 0ull;
+            }
         }
     }
     if (lane != 0) return;
     const float max_s = top_score[0];
     float sum = 0.0f, ex[8];
-    for (uint32_t i = 0; i < top_k; ++i) {
-        ex[i] = expf(top_score[i] - max_s);
-        sum += ex[i];
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) {
+        if (i < top_k) {
+            ex[i] = expf(top_score[i] - max_s);
+            sum += ex[i];
+        }
     }
-    for (uint32_t i = 0; i < top_k; ++i) {
-        const float gain = per_expert_scale ? bf16_to_f32(per_expert_scale[top_idx[i]]) : 1.0f;
-        out_idx[(size_t)tok * top_k + i] = top_idx[i];
-        out_w[(size_t)tok * top_k + i] = f32_to_bf16(ex[i] / sum * gain);
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) {
+        if (i < top_k) {
+            const float gain = per_expert_scale ? bf16_to_f32(per_expert_scale[top_idx[i]]) : 1.0f;
+            out_idx[i] = top_idx[i];
+            out_w[i] = f32_to_bf16(ex[i] / sum * gain);
+        }
     }
+}
+
+template <bool W_F32>
+__device__ __forceinline__ void load_w4(const void *w_, size_t off, bool ok, float (&out)[4]) {
+    if (!ok) {
+        out[0] = out[1] = out[2] = out[3] = 0.0f;
+        return;
+    }
+    if (W_F32) {
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(w_) + off);
+        out[0] = v[0]; out[1] = v[1]; out[2] = v[2]; out[3] = v[3];
+    } else {
+        const uint2 v = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(w_) + off);
+        out[0] = bf16lo_to_f32(v.x); out[1] = bf16hi_to_f32(v.x);
+        out[2] = bf16lo_to_f32(v.y); out[3] = bf16hi_to_f32(v.y);
+    }
+}
+
+// Four bf16 inputs starting at element `off` of a row that needs 2-byte alignment only.
+template <bool X_ALIGNED>
+__device__ __forceinline__ uint2 load_x4(const uint16_t *p) {
+    if (X_ALIGNED) return *reinterpret_cast<const uint2 *>(p);
+    uint2 r;
+    r.x = (uint32_t)p[0] | ((uint32_t)p[1] << 16);
+    r.y = (uint32_t)p[2] | ((uint32_t)p[3] << 16);
+    return r;
+}
+
+// Per-lane accumulation shared by both logits kernels: sub-accumulator `s` of lane `lane` over the
+// elements k = 1024 i + 256 s + 4 lane + j, i ascending then j, for kChunkTokens token rows at once.
+template <bool W_F32, bool X_ALIGNED>
+__device__ __forceinline__ void accumulate_sub(const void *__restrict__ w_, const uint16_t *__restrict__ es,
+                                               const uint16_t *__restrict__ x, uint32_t x_stride, uint32_t e,
+                                               uint32_t d, uint32_t s, uint32_t lane, uint32_t t0, uint32_t t_last,
+                                               float (&acc)[kChunkTokens]) {
+    const uint32_t steps = (d + 1023) / 1024;
+#pragma unroll 3
+    for (uint32_t i = 0; i < steps; ++i) {
+        const uint32_t k = 1024 * i + 256 * s + 4 * lane;
+        if (k < d) {
+            float wv[4], sc[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            load_w4<W_F32>(w_, (size_t)e * d + k, true, wv);
+            if (es) {
+                const uint2 v = *reinterpret_cast<const uint2 *>(es + k);
+                sc[0] = bf16lo_to_f32(v.x); sc[1] = bf16hi_to_f32(v.x);
+                sc[2] = bf16lo_to_f32(v.y); sc[3] = bf16hi_to_f32(v.y);
+            }
+#pragma unroll
+            for (int r = 0; r < kChunkTokens; ++r) {
+                // rows past the last token re-read it: same arithmetic, result unused
+                const uint32_t row = min(t0 + r, t_last);
+                const uint2 xv = load_x4<X_ALIGNED>(x + (size_t)row * x_stride + k);
+                const float xf[4] = {bf16lo_to_f32(xv.x), bf16hi_to_f32(xv.x), bf16lo_to_f32(xv.y), bf16hi_to_f32(xv.y)};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    // x * effective_scale: product of two bf16 values, exact in fp32 (moe.metal:96-97)
+                    const float xe = es ? xf[j] * sc[j] : xf[j];
+                    acc[r] = __builtin_fmaf(wv[j], xe, acc[r]);
+                }
+            }
+        }
+    }
+}
+
+// Decode / verify router logits (T <= 16). grid = (E, ceil(T / 4)); the four waves of a block are the
+// four sub-accumulators of one expert row for four tokens; wave 0 combines them. (A variant whose last
+// block also selected the top-k behind a device-scope counter measured 2.5x slower: every block paid
+// for the same-address atomic and the L2 write-back of its release fence.)
+template <bool W_F32, bool X_ALIGNED>
+__global__ __launch_bounds__(256) void router_small_kernel(const void *__restrict__ w_, const uint16_t *__restrict__ es,
+                                                           const uint16_t *__restrict__ x, uint32_t x_stride,
+                                                           uint32_t t, uint32_t n_experts, uint32_t d,
+                                                           float *__restrict__ logits) {
+    __shared__ float s_part[4][kChunkTokens][64];
+    const uint32_t lane = threadIdx.x & 63, s = threadIdx.x >> 6;
+    const uint32_t e = blockIdx.x;
+    const uint32_t t0 = blockIdx.y * kChunkTokens;
+    const uint32_t t_end = min(t, t0 + kChunkTokens);
+    float acc[kChunkTokens] = {0.f, 0.f, 0.f, 0.f};
+    accumulate_sub<W_F32, X_ALIGNED>(w_, es, x, x_stride, e, d, s, lane, t0, t_end - 1, acc);
+#pragma unroll
+    for (int r = 0; r < kChunkTokens; ++r) s_part[s][r][lane] = acc[r];
+    __syncthreads();
+    if (s != 0) return;
+#pragma unroll
+    for (int r = 0; r < kChunkTokens; ++r) {
+        const float v = wave_butterfly_sum((s_part[0][r][lane] + s_part[1][r][lane]) +
+                                           (s_part[2][r][lane] + s_part[3][r][lane]));
+        if (lane == 0 && t0 + r < t_end) logits[(size_t)(t0 + r) * n_experts + e] = v;
+    }
+}
+
+// Prefill router logits. grid = (ceil(E / 4), ceil(T / tokens_per_wave)); one wave per expert row keeps
+// all four sub-accumulators itself and walks its tokens in chunks of four.
+template <bool W_F32, bool X_ALIGNED>
+__global__ __launch_bounds__(256) void router_logits_kernel(const void *__restrict__ w_, const uint16_t *__restrict__ es,
+                                                            const uint16_t *__restrict__ x, uint32_t x_stride,
+                                                            uint32_t t, uint32_t n_experts, uint32_t d,
+                                                            uint32_t tokens_per_wave, float *__restrict__ logits) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t e = blockIdx.x * 4 + wave;
+    if (e >= n_experts) return;
+    const uint32_t t_begin = blockIdx.y * tokens_per_wave;
+    const uint32_t t_end = min(t, t_begin + tokens_per_wave);
+    for (uint32_t t0 = t_begin; t0 < t_end; t0 += kChunkTokens) {
+        float sub[4][kChunkTokens];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+#pragma unroll
+            for (int r = 0; r < kChunkTokens; ++r) sub[s][r] = 0.0f;
+            accumulate_sub<W_F32, X_ALIGNED>(w_, es, x, x_stride, e, d, s, lane, t0, t_end - 1, sub[s]);
+        }
+#pragma unroll
+        for (int r = 0; r < kChunkTokens; ++r) {
+            const float v = wave_butterfly_sum((sub[0][r] + sub[1][r]) + (sub[2][r] + sub[3][r]));
+            if (lane == 0 && t0 + r < t_end) logits[(size_t)(t0 + r) * n_experts + e] = v;
+        }
+    }
+}
+
+__global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, const uint16_t *__restrict__ per_expert_scale,
+                                                         uint32_t n_experts, uint32_t top_k,
+                                                         uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w) {
+    const uint32_t tok = blockIdx.x;
+    wave_topk(logits + (size_t)tok * n_experts, per_expert_scale, n_experts, top_k, out_idx + (size_t)tok * top_k,
+              out_w + (size_t)tok * top_k, threadIdx.x);
 }
 
 }  // namespace
 
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w, KernelTimer *timer) {
+                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer) {
+    (void)counters;
     timer->begin(s);
-    const dim3 grid((n_experts + 3) / 4, (t + kRouterTokens - 1) / kRouterTokens);
-    if (rw.w_is_f32)
-        hipLaunchKernelGGL(router_logits_kernel<true>, grid, dim3(256), 0, s, rw.w, rw.effective_scale, x,
-                           x_stride, t, n_experts, d, logits);
-    else
-        hipLaunchKernelGGL(router_logits_kernel<false>, grid, dim3(256), 0, s, rw.w, rw.effective_scale, x,
-                           x_stride, t, n_experts, d, logits);
+    const bool x_aligned = (reinterpret_cast<uintptr_t>(x) % 8 == 0) && (x_stride % 4 == 0);
+    if (t <= FFMOE_MAX_VERIFY_ROWS) {
+        const dim3 grid(n_experts, (t + kChunkTokens - 1) / kChunkTokens);
+#define FFMOE_ROUTER(WF, XA)                                                                                 \
+    hipLaunchKernelGGL((router_small_kernel<WF, XA>), grid, dim3(256), 0, s, rw.w, rw.effective_scale, x,   \
+                       x_stride, t, n_experts, d, logits)
+        if (rw.w_is_f32) { if (x_aligned) FFMOE_ROUTER(true, true); else FFMOE_ROUTER(true, false); }
+        else { if (x_aligned) FFMOE_ROUTER(false, true); else FFMOE_ROUTER(false, false); }
+#undef FFMOE_ROUTER
+        timer->mark(s, FFMOE_K_ROUTER_LOGITS);
+        hipLaunchKernelGGL(router_topk_kernel, dim3(t), dim3(64), 0, s, logits, rw.per_expert_scale, n_experts, top_k,
+                           out_idx, out_w);
+        timer->mark(s, FFMOE_K_ROUTER_TOPK);
+        timer->finish();
+        return hipGetLastError();
+    }
+    const uint32_t tpw = 64;
+    const dim3 grid((n_experts + 3) / 4, (t + tpw - 1) / tpw);
+#define FFMOE_ROUTER(WF, XA)                                                                                 \
+    hipLaunchKernelGGL((router_logits_kernel<WF, XA>), grid, dim3(256), 0, s, rw.w, rw.effective_scale, x,   \
+                       x_stride, t, n_experts, d, tpw, logits)
+    if (rw.w_is_f32) { if (x_aligned) FFMOE_ROUTER(true, true); else FFMOE_ROUTER(true, false); }
+    else { if (x_aligned) FFMOE_ROUTER(false, true); else FFMOE_ROUTER(false, false); }
+#undef FFMOE_ROUTER
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_ROUTER_LOGITS);
-    hipLaunchKernelGGL(router_topk_kernel, dim3(t), dim3(64), 0, s, logits, rw.per_expert_scale, n_experts,
-                       top_k, out_idx, out_w);
+    hipLaunchKernelGGL(router_topk_kernel, dim3(t), dim3(64), 0, s, logits, rw.per_expert_scale, n_experts, top_k,
+                       out_idx, out_w);
     timer->mark(s, FFMOE_K_ROUTER_TOPK);
     timer->finish();
     return hipGetLastError();

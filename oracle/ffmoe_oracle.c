@@ -344,10 +344,12 @@ void ffo_reduce_token_major(const void *partials, int partial_dtype, const uint1
     }
 }
 
-/* Router logits in this build's pinned order: 64 lane partials, lane l takes k = l + 64*i in
- * increasing i with fmaf, then a xor-butterfly (32,16,8,4,2,1) of plain adds. The input is
- * x[k] * effective_scale[k] as at Metal/MoE/moe.metal:96-97 (product of two bf16 values: exact in
- * fp32). Mathematically the row dot of moe.metal:65-103 with dequantized weights. */
+/* Router logits in this build's pinned order: 64 lanes x 4 sub-accumulators; sub-accumulator s of
+ * lane l owns k = 1024*i + 256*s + 4*l + j (j = 0..3) and accumulates with fmaf in increasing i, then
+ * j; the lane's value is (sub0 + sub1) + (sub2 + sub3); a xor-butterfly (32,16,8,4,2,1) of plain adds
+ * combines the 64 lane values. The input is x[k] * effective_scale[k] as at
+ * Metal/MoE/moe.metal:96-97 (product of two bf16 values: exact in fp32). Mathematically the row dot
+ * of moe.metal:65-103 with dequantized weights. */
 void ffo_router_logits_pinned(const void *W, int w_is_f32, const uint16_t *x, int x_dtype,
                               const uint16_t *es, int e, int d, float *logits) {
     float *xe = (float *)malloc((size_t)d * sizeof(float));
@@ -355,18 +357,26 @@ void ffo_router_logits_pinned(const void *W, int w_is_f32, const uint16_t *x, in
         float xv = ffo_from_bits16(x[k], x_dtype);
         xe[k] = es ? xv * ffo_bf16_to_float(es[k]) : xv;
     }
-    int steps = d / 64;
+    int steps = (d + 1023) / 1024;
     for (int row = 0; row < e; ++row) {
         float p[64], q[64];
         for (int l = 0; l < 64; ++l) {
-            float acc = 0.0f;
-            for (int i = 0; i < steps; ++i) {
-                int k = l + 64 * i;
-                float w = w_is_f32 ? ((const float *)W)[(size_t)row * d + k]
-                                   : ffo_bf16_to_float(((const uint16_t *)W)[(size_t)row * d + k]);
-                acc = fmaf(w, xe[k], acc);
+            float sub[4];
+            for (int s = 0; s < 4; ++s) {
+                float acc = 0.0f;
+                for (int i = 0; i < steps; ++i) {
+                    for (int j = 0; j < 4; ++j) {
+                        int k = 1024 * i + 256 * s + 4 * l + j;
+                        if (k >= d) continue;
+                        float w = w_is_f32 ? ((const float *)W)[(size_t)row * d + k]
+                                           : ffo_bf16_to_float(((const uint16_t *)W)[(size_t)row * d + k]);
+                        acc = fmaf(w, xe[k], acc);
+                    }
+                }
+                sub[s] = acc;
             }
-            p[l] = acc;
+            float lo = sub[0] + sub[1], hi = sub[2] + sub[3];
+            p[l] = lo + hi;
         }
         for (int m = 32; m >= 1; m >>= 1) {
             for (int l = 0; l < 64; ++l) q[l] = p[l] + p[l ^ m];

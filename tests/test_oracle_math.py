@@ -150,11 +150,19 @@ def test_router_pinned_order_definition(oracle):
     W = oracle.bf16_to_float(Wb).astype(np.float64)
     x = oracle.bf16_to_float(xb).astype(np.float64)
     assert np.abs(got - W @ x).max() < 2e-5
-    # lanes: fp32 fma chain over k = l + 64 i. bf16*bf16 products are exact in fp32, so fma == mul+add here.
+    # sub-accumulator s of lane l: fp32 chain over k = 1024 i + 256 s + 4 l + j. bf16*bf16 products are
+    # exact in fp32, so fma == mul+add here.
     Wf, xf = oracle.bf16_to_float(Wb), oracle.bf16_to_float(xb)
-    p = np.zeros((e, 64), np.float32)
-    for i in range(d // 64):
-        p = (Wf[:, 64 * i:64 * i + 64] * xf[64 * i:64 * i + 64] + p).astype(np.float32)
+    sub = np.zeros((4, e, 64), np.float32)
+    for i in range((d + 1023) // 1024):
+        for s in range(4):
+            for j in range(4):
+                ks = 1024 * i + 256 * s + 4 * np.arange(64) + j
+                ok = ks < d
+                term = np.zeros((e, 64), np.float32)
+                term[:, ok] = Wf[:, ks[ok]] * xf[ks[ok]]
+                sub[s] = np.where(ok[None, :], (term + sub[s]).astype(np.float32), sub[s])
+    p = ((sub[0] + sub[1]).astype(np.float32) + (sub[2] + sub[3]).astype(np.float32)).astype(np.float32)
     for m in (32, 16, 8, 4, 2, 1):
         p = (p + p[:, np.arange(64) ^ m]).astype(np.float32)
     assert np.array_equal(got, p[:, 0])
