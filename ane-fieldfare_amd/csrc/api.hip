@@ -35,6 +35,8 @@ struct ffmoe_ctx {
     uint32_t *counters = nullptr;    // completion counters of the fused router (self-resetting)
     uint16_t *acts = nullptr;        // [16*top_k][F]
     float *partials = nullptr;       // [16*top_k][D]
+    PrefillScratch pf{};
+    uint32_t max_pairs = 0;
     KernelTimer timer;
 };
 
@@ -122,6 +124,18 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     if (e == hipSuccess) e = hipMemset(ctx->counters, 0, 64 * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->acts), routes * shape->f * sizeof(uint16_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->partials), routes * shape->d * sizeof(float));
+    // prefill scratch: sort tables, pair lists, activations and per-route rows for max_tokens tokens
+    ctx->max_pairs = (shape->max_tokens > FFMOE_MAX_VERIFY_ROWS ? shape->max_tokens : FFMOE_MAX_VERIFY_ROWS) * shape->top_k;
+    const size_t sort_blocks = (ctx->max_pairs + 255) / 256;
+    ctx->pf.max_tiles = ctx->max_pairs / FFMOE_PREFILL_TILE_M + shape->n_experts + 1;
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.block_cnt), sort_blocks * shape->n_experts * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.plan), sizeof(PrefillPlan));
+    if (e == hipSuccess) e = hipMemset(ctx->pf.plan, 0, sizeof(PrefillPlan));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.tiles), (size_t)ctx->pf.max_tiles * sizeof(PrefillTile));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.sorted_token), (size_t)ctx->max_pairs * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.sorted_out_row), (size_t)ctx->max_pairs * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.acts), (size_t)ctx->max_pairs * shape->f * sizeof(uint16_t));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.partials), (size_t)ctx->max_pairs * shape->d * sizeof(uint16_t));
     if (e != hipSuccess) {
         ffmoe_destroy(ctx);
         return fail(err, FFMOE_ERR_ALLOC, "failed to allocate the expert arena (%zu bytes) or scratch: %s",
@@ -146,6 +160,13 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->acts) (void)hipFree(ctx->acts);
     if (ctx->partials) (void)hipFree(ctx->partials);
+    if (ctx->pf.block_cnt) (void)hipFree(ctx->pf.block_cnt);
+    if (ctx->pf.plan) (void)hipFree(ctx->pf.plan);
+    if (ctx->pf.tiles) (void)hipFree(ctx->pf.tiles);
+    if (ctx->pf.sorted_token) (void)hipFree(ctx->pf.sorted_token);
+    if (ctx->pf.sorted_out_row) (void)hipFree(ctx->pf.sorted_out_row);
+    if (ctx->pf.acts) (void)hipFree(ctx->pf.acts);
+    if (ctx->pf.partials) (void)hipFree(ctx->pf.partials);
     for (auto &ev : ctx->timer.ev)
         if (ev) (void)hipEventDestroy(ev);
     delete ctx;
@@ -299,6 +320,53 @@ int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char
     if (!n_live) return fail(err, FFMOE_ERR_INVALID, "null argument");
     FF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     FF_HIP(hipMemcpy(n_live, &ctx->plan->n_live, sizeof(uint32_t), hipMemcpyDeviceToHost));
+    return FFMOE_OK;
+}
+
+static int prefill_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride, uint32_t t,
+                          const uint32_t *idx, const uint16_t *w, const ffmoe_pair *pairs, uint32_t n_pairs, uint16_t *y,
+                          uint16_t *partials, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, true, false, err)) return rc;
+    if (!x) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (t == 0) return fail(err, FFMOE_ERR_INVALID, "queryCount must be positive");
+    if ((size_t)t * ctx->shape.top_k > ctx->max_pairs)
+        return fail(err, FFMOE_ERR_INVALID, "t = %u exceeds max_tokens = %u", t, ctx->shape.max_tokens);
+    if (pairs && n_pairs > ctx->max_pairs)
+        return fail(err, FFMOE_ERR_ALLOC, "prefill sorted route pairs exceed reusable capacity (%u > %u)", n_pairs, ctx->max_pairs);
+    if (x_stride < ctx->shape.d || x_stride % 8 || reinterpret_cast<uintptr_t>(x) % 16)
+        return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
+    if ((y && reinterpret_cast<uintptr_t>(y) % 16) || (partials && reinterpret_cast<uintptr_t>(partials) % 2))
+        return fail(err, FFMOE_ERR_INVALID, "output alignment");
+    FF_HIP(launch_prefill(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
+                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, pairs, n_pairs, y, partials,
+                          ctx->pf, &ctx->timer));
+    return FFMOE_OK;
+}
+
+int ffmoe_prefill(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride, uint32_t t,
+                  const uint32_t *idx, const uint16_t *w, uint16_t *y, char **err) {
+    if (!idx || !w || !y) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    return prefill_common(ctx, stream, layer, x, x_stride, t, idx, w, nullptr, 0, y, nullptr, err);
+}
+
+int ffmoe_prefill_pairs(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
+                        const ffmoe_pair *pairs, uint32_t n_pairs, uint32_t t, uint16_t *partials, char **err) {
+    if (!partials) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (n_pairs == 0) return FFMOE_OK;
+    if (!pairs) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    return prefill_common(ctx, stream, layer, x, x_stride, t, nullptr, nullptr, pairs, n_pairs, nullptr, partials, err);
+}
+
+int ffmoe_prefill_plan_stats(ffmoe_ctx *ctx, void *stream, uint32_t *n_pairs, uint32_t *n_tiles, uint32_t *counts,
+                             char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    FF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    PrefillPlan host;
+    FF_HIP(hipMemcpy(&host, ctx->pf.plan, sizeof(PrefillPlan), hipMemcpyDeviceToHost));
+    if (n_pairs) *n_pairs = host.n_pairs;
+    if (n_tiles) *n_tiles = host.n_tiles;
+    if (counts) memcpy(counts, host.expert_count, ctx->shape.n_experts * sizeof(uint32_t));
     return FFMOE_OK;
 }
 

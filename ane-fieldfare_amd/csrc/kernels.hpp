@@ -77,6 +77,27 @@ struct KernelTimer {
     }
 };
 
+// Prefill: expert-sorted pairs and their M-tiles, built on the GPU.
+#define FFMOE_PREFILL_TILE_M 128
+struct PrefillTile {
+    uint32_t expert, row_start, rows, pad;     // rows [row_start, row_start + rows) of the sorted pair list
+};
+struct PrefillPlan {
+    uint32_t n_pairs, n_tiles, pad[2];
+    uint32_t expert_count[FFMOE_MAX_EXPERTS];
+    uint32_t expert_offset[FFMOE_MAX_EXPERTS + 1];
+};
+struct PrefillScratch {
+    uint32_t *block_cnt;        // [sort blocks][E]: counts, then bases
+    PrefillPlan *plan;
+    PrefillTile *tiles;
+    uint32_t max_tiles;
+    uint32_t *sorted_token;     // [max pairs]
+    uint32_t *sorted_out_row;   // [max pairs]: token * top_k + rank
+    uint16_t *acts;             // [max pairs][F] bf16
+    uint16_t *partials;         // [max pairs][D] bf16 (used when the caller wants the combined output)
+};
+
 struct RouterWeights {
     const void *w;          // bf16 [E][D] or float [E][D]
     int w_is_f32;
@@ -102,6 +123,13 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
                          VerifyPlan *plan, uint16_t *acts, float *partials_f32, KernelTimer *timer);
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,
                                      uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d);
+
+// prefill.hip: routes come from (idx, w) [t][top_k], or from an explicit pair list when `pairs` != nullptr.
+// Writes y [t][d] (combined) when y != nullptr; un-weighted bf16 rows go to partials_out or to scratch.
+hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
+                          const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
+                          const ffmoe_pair *pairs, uint32_t n_pairs_in, uint16_t *y, uint16_t *partials_out,
+                          PrefillScratch sc, KernelTimer *timer);
 
 // gemv.hip
 hipError_t launch_gemv_int4(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,

@@ -41,7 +41,8 @@ EXPORTS = [
     "ffmoe_version", "ffmoe_create", "ffmoe_destroy", "ffmoe_layer_arena_bytes", "ffmoe_upload_layer",
     "ffmoe_upload_router_bf16", "ffmoe_upload_router_int8", "ffmoe_dequant_expert", "ffmoe_router",
     "ffmoe_verify", "ffmoe_verify_partials", "ffmoe_last_live_experts", "ffmoe_reduce_token_major",
-    "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile",
+    "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
+    "ffmoe_prefill_plan_stats",
 ]
 
 PROFILE_SLOTS = 12
@@ -69,6 +70,9 @@ def lib() -> C.CDLL:
         return _lib
     if not LIB_PATH.exists():
         raise FileNotFoundError(f"{LIB_PATH} is not built; run __graft_entry__.build() (there is no fallback path)")
+    # torch ships its own HIP runtime: it has to be in the process before this library resolves
+    # libamdhip64, or two runtimes end up loaded and the second one finds no device
+    import torch  # noqa: F401
     L = C.CDLL(str(LIB_PATH))
     vp, u32, sz, i32 = C.c_void_p, C.c_uint32, C.c_size_t, C.c_int
     errp = C.POINTER(C.c_char_p)
@@ -90,10 +94,9 @@ def lib() -> C.CDLL:
     L.ffmoe_gemv_int4.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, i32, errp]
     L.ffmoe_set_profiling.argtypes = [vp, i32, errp]
     L.ffmoe_get_profile.argtypes = [vp, C.POINTER(Profile), i32, errp]
-    if hasattr(L, "ffmoe_prefill"):
-        L.ffmoe_prefill.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
-        L.ffmoe_prefill_pairs.argtypes = [vp, vp, u32, vp, u32, vp, u32, u32, vp, errp]
-        L.ffmoe_prefill_plan_stats.argtypes = [vp, vp, vp, errp]
+    L.ffmoe_prefill.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
+    L.ffmoe_prefill_pairs.argtypes = [vp, vp, u32, vp, u32, vp, u32, u32, vp, errp]
+    L.ffmoe_prefill_plan_stats.argtypes = [vp, vp, C.POINTER(u32), C.POINTER(u32), vp, errp]
     _lib = L
     return L
 
@@ -268,6 +271,16 @@ class Context:
         _check(self.L.ffmoe_prefill_pairs(self._h, _stream(), layer, _ptr(x), _row_stride(x), _ptr(sorted_pairs),
                                           sorted_pairs.shape[0], t, _ptr(partials), C.byref(err)), err)
         return partials
+
+    def prefill_stats(self):
+        """(pairs kept, M-tiles, pairs per expert) of the last prefill call."""
+        import numpy as np
+        n_pairs, n_tiles = C.c_uint32(), C.c_uint32()
+        counts = np.zeros(self.shape.n_experts, np.uint32)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_prefill_plan_stats(self._h, _stream(), C.byref(n_pairs), C.byref(n_tiles),
+                                               C.c_void_p(counts.ctypes.data), C.byref(err)), err)
+        return int(n_pairs.value), int(n_tiles.value), counts
 
     # -- generic GEMV ----------------------------------------------------------------------------
     def gemv_int4(self, W, S, B, x, f32_out: bool = False, w_byte_offset: int = 0):

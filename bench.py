@@ -66,6 +66,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--layers", type=int, default=30)
     ap.add_argument("--tokens", type=int, default=16)
+    ap.add_argument("--prefill-tokens", type=int, default=3072, help="0 skips the prefill leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -169,6 +170,50 @@ def main():
     extra["decode_us_per_layer"] = round(dec * 1e6, 2)
     extra["decode_expert_GBs"] = round(K * EXPERT_BYTES / dec / 1e9, 1)
 
+    # prefill half of the metric (BASELINE.json config 4): 3,072 tokens through one MoE layer, router
+    # included, near-uniform routing from the Gaussian router; layers cycle as above
+    TP = args.prefill_tokens
+    prefill = None
+    if TP > 0:
+        xp = torch.from_numpy(oracle.bf16_bits(rng.normal(0, 1, (TP, D)).astype(np.float32)).view(np.int16)).cuda().view(torch.bfloat16)
+        pidx_t = torch.empty((TP, K), dtype=torch.int32, device="cuda")
+        pw_t = torch.empty((TP, K), dtype=torch.bfloat16, device="cuda")
+        py_t = torch.empty((TP, D), dtype=torch.bfloat16, device="cuda")
+        pxp, ppi, ppw, ppy = (C.c_void_p(t_.data_ptr()) for t_ in (xp, pidx_t, pw_t, py_t))
+
+        def pstep(layer):
+            rc = Lib.ffmoe_router(h, stream, layer, pxp, D, TP, ppi, ppw, None, C.byref(err))
+            rc |= Lib.ffmoe_prefill(h, stream, layer, pxp, D, TP, ppi, ppw, ppy, C.byref(err))
+            if rc:
+                raise RuntimeError(err.value)
+        psteps = max(4, min(args.steps, 2 * L))
+        for i in range(min(L, 8)):
+            pstep(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(psteps):
+            pstep(i % L)
+        torch.cuda.synchronize()
+        pel = (time.perf_counter() - t0) / psteps
+        n_pairs, n_tiles, counts = ctx.prefill_stats()
+        ctx.set_profiling(True)
+        ctx.profile(reset=True)
+        for i in range(psteps):
+            pstep(i % L)
+        pprof = ctx.profile(reset=True)
+        ctx.set_profiling(False)
+        pk_us = {k: round(v[0] / v[1] * 1e3, 2) for k, v in pprof.items()}
+        flops_gu = n_pairs * 2.0 * (2 * F * D)
+        flops_dn = n_pairs * 2.0 * (D * F)
+        gemm_s = (pprof["prefill_gate_up"][0] + pprof["prefill_down"][0]) / psteps * 1e-3
+        prefill = {"tokens": TP, "tok_per_s": round(TP / pel, 1), "ms_per_layer": round(pel * 1e3, 4),
+                   "pairs": n_pairs, "m_tiles": n_tiles, "pairs_per_expert_min": int(counts.min()),
+                   "pairs_per_expert_max": int(counts.max()), "kernel_us": pk_us,
+                   "roofline": {"bound": "mfma", "kernel": "prefill_gemm_kernel (gate_up + down)",
+                                "achieved": round((flops_gu + flops_dn) / gemm_s / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                                "unit": "TFLOP/s", "frac": round((flops_gu + flops_dn) / gemm_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                "traffic": None}}
+
     cpu = None
     if not args.no_cpu:
         pool = oracle.ExpertPool(host_layer0, offsets, STRIDE, D, F)
@@ -213,6 +258,8 @@ def main():
                      "traffic": None, "avg_kernel_us": kernel_us.get("gate_up")},
         "kernel_us": kernel_us,
         "down_kernel_GBs": round(down_gbs, 1),
+        "prefill_tok_s": prefill["tok_per_s"] if prefill else None,
+        "prefill": prefill,
         "cpu_baseline": cpu,
         "extra": extra,
     }

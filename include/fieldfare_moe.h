@@ -146,6 +146,33 @@ int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const ui
  * for the stream). For reporting only. */
 int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char **err);
 
+/* ---- routed experts, prefill chunk (t <= max_tokens) ------------------------------------------- */
+
+/* y[t] = bf16(sum_r w[t][r] * partial[t][r]) with partial = bf16(down_e(gelu_tanh(gate_e x[t]) * up_e x[t])),
+ * e = idx[t][r], for a whole prefill chunk: the routes are sorted by expert ON THE GPU (no read-back of
+ * the router output), each expert's pairs run as M-tiles of a grouped GEMM on the matrix units with
+ * INT4 -> bf16 tiles dequantised into LDS, and the per-route rows are combined in rank order. Routes
+ * whose weight is exactly zero are dropped. Replaces makeTokenExpertPairs + groupTokenExpertPairs
+ * (Kernels/Prefill/MoE/PrefillRouter.swift:75-95, PrefillMoEGrouping.swift:49-110),
+ * PrefillGroupedRoutedMoE.encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:275-326) and
+ * PrefillMoE.encodeReduceTokenMajor, i.e. RealForwardRunner.swift:1520-1599 without the host wait. */
+int ffmoe_prefill(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
+                  uint32_t t, const uint32_t *idx, const uint16_t *w, uint16_t *y, char **err);
+
+/* The guest contract of RoutedPrefillGuest.runLayer (Runtime/Supervisor/DeviceSupervisor.swift:14-22):
+ * for every pair of `pairs` (device array, any order; the reference passes them expert-sorted) write
+ * the UN-weighted row bf16 partials[(token * top_k + rank) * d ...]; rows of other routes are left
+ * untouched (the host zeroes `partials` first, RealForwardRunner.swift:1502-1506). Replaces
+ * ANERoutedPrefillBackend.runLayer (Runtime/Inference/ANERoutedPrefillBackend.swift:348-427). */
+int ffmoe_prefill_pairs(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
+                        const ffmoe_pair *pairs, uint32_t n_pairs, uint32_t t, uint16_t *partials, char **err);
+
+/* Pairs kept and M-tiles run by the last prefill call on `stream`, and pairs per expert (`counts`,
+ * n_experts entries, may be NULL). Waits for the stream. For reporting (the reference's
+ * prefillRouted* counters, RealForwardRunner.swift:171-203). */
+int ffmoe_prefill_plan_stats(ffmoe_ctx *ctx, void *stream, uint32_t *n_pairs, uint32_t *n_tiles,
+                             uint32_t *counts, char **err);
+
 /* ---- weighted combine ------------------------------------------------------------------------- */
 
 /* h2[t][c] = bf16(sum_r w[t][r] * partials[t][r][c]), fma in rank order.
