@@ -1,0 +1,412 @@
+// Host-side mirror of the reference's Swift operator surface for the routed-expert stage, written
+// over the C ABI of include/fieldfare_moe.h only (no HIP types: a stream is an opaque void*).
+//
+// The reference's host code is Swift; this image has no Swift toolchain, so the mirror is C++17 with
+// the same names, argument meaning and error behaviour. Shape misuse, a Swift `precondition` trap in
+// the reference, throws std::invalid_argument here; resource failures throw FieldfareError carrying
+// the library's message (the reference throws MetalError / PrefillGroupedRoutedMoEError).
+//
+//   reference type (file)                                              -> here
+//   MoEExpertOffsets              Kernels/MoE/MoE.swift:4-29            -> ffmoe_offsets (C ABI)
+//   PrefillTokenExpertPair        Kernels/Prefill/MoE/PrefillRouter.swift:5-21 -> PrefillTokenExpertPair
+//   PrefillRouter.makeTokenExpertPairs            PrefillRouter.swift:75-95    -> PrefillRouter::makeTokenExpertPairs
+//   PrefillMoEGrouping.groupTokenExpertPairs      PrefillMoEGrouping.swift:49-110 -> PrefillMoEGrouping::groupTokenExpertPairs
+//   PrefillStreamedTileBinding    PrefillGroupedRoutedMoE.swift:121-166 -> PrefillStreamedTileBinding
+//   MoE (router, decode phases)   Kernels/MoE/MoE.swift:31-507          -> MoE
+//   PrefillRouter.encodeGemma4Block               PrefillRouter.swift:30-73    -> PrefillRouter::encodeGemma4Block
+//   PrefillGroupedRoutedMoE       PrefillGroupedRoutedMoE.swift:183-448 -> PrefillGroupedRoutedMoE
+//   PrefillMoE.encodeReduceTokenMajor             PrefillMoE.swift:11-32       -> PrefillMoE::encodeReduceTokenMajor
+//   DequantInt4GEMV               Kernels/Quant/DequantInt4GEMV.swift   -> DequantInt4GEMV
+//   RoutedPrefillGuest, DeviceSupervisor, RuntimeFaultPolicy, GuestFault
+//                                 Runtime/Supervisor/DeviceSupervisor.swift:5-125 -> same names
+#pragma once
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdlib>
+#include <functional>
+#include <memory>
+#include <optional>
+#include <set>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/fieldfare_moe.h"
+
+namespace fieldfare {
+
+struct FieldfareError : std::runtime_error {
+    int code;
+    FieldfareError(int c, const std::string &m) : std::runtime_error(m), code(c) {}
+};
+
+inline void check(int rc, char *err) {
+    if (rc == FFMOE_OK) return;
+    std::string msg = err ? err : "(no message)";
+    std::free(err);
+    throw FieldfareError(rc, msg);
+}
+
+// One ffmoe_ctx. Plays the part of MetalContext + the resident expert store for the operators below.
+class Context {
+public:
+    Context(int device, const ffmoe_shape &shape) : shape_(shape) {
+        char *err = nullptr;
+        check(ffmoe_create(device, &shape, &ctx_, &err), err);
+    }
+    ~Context() { ffmoe_destroy(ctx_); }
+    Context(const Context &) = delete;
+    Context &operator=(const Context &) = delete;
+    ffmoe_ctx *raw() const { return ctx_; }
+    const ffmoe_shape &shape() const { return shape_; }
+
+    void uploadLayer(uint32_t layer, const void *blobs, size_t stride, const ffmoe_offsets &offsets, bool onDevice = false) {
+        char *err = nullptr;
+        check(ffmoe_upload_layer(ctx_, layer, blobs, stride, &offsets, onDevice ? 1 : 0, &err), err);
+    }
+    void uploadRouterBF16(uint32_t layer, const uint16_t *w, const uint16_t *effectiveScale = nullptr,
+                          const uint16_t *perExpertScale = nullptr) {
+        char *err = nullptr;
+        check(ffmoe_upload_router_bf16(ctx_, layer, w, effectiveScale, perExpertScale, &err), err);
+    }
+    void uploadRouterInt8(uint32_t layer, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                          const uint16_t *effectiveScale = nullptr, const uint16_t *perExpertScale = nullptr) {
+        char *err = nullptr;
+        check(ffmoe_upload_router_int8(ctx_, layer, w, scales, biases, effectiveScale, perExpertScale, &err), err);
+    }
+
+private:
+    ffmoe_ctx *ctx_ = nullptr;
+    ffmoe_shape shape_;
+};
+
+// ---------------------------------------------------------------------------------------------------
+// Pair building and grouping: pure host logic (no GPU).
+// ---------------------------------------------------------------------------------------------------
+struct PrefillTokenExpertPair {
+    uint32_t token, expert, rank, weightBitsAndReserved;
+    bool operator==(const PrefillTokenExpertPair &o) const {
+        return token == o.token && expert == o.expert && rank == o.rank && weightBitsAndReserved == o.weightBitsAndReserved;
+    }
+};
+static_assert(sizeof(PrefillTokenExpertPair) == sizeof(ffmoe_pair), "pairs cross the C ABI as they are");
+
+struct PrefillMoEGroup {
+    uint32_t expert, pairStart, pairCount;
+    bool operator==(const PrefillMoEGroup &o) const { return expert == o.expert && pairStart == o.pairStart && pairCount == o.pairCount; }
+};
+
+struct PrefillMoETile {
+    uint32_t groupStart, groupCount, pairStart, pairCount;
+    bool operator==(const PrefillMoETile &o) const {
+        return groupStart == o.groupStart && groupCount == o.groupCount && pairStart == o.pairStart && pairCount == o.pairCount;
+    }
+};
+
+struct PrefillMoEGroupedRoutes {
+    std::vector<PrefillTokenExpertPair> sortedPairs;
+    std::vector<PrefillMoEGroup> groups;
+    std::vector<PrefillMoETile> tiles;
+};
+
+struct PrefillMoEGroupingError : std::runtime_error {
+    uint32_t expert;
+    explicit PrefillMoEGroupingError(uint32_t e)
+        : std::runtime_error("route expert " + std::to_string(e) + " is out of range"), expert(e) {}
+};
+
+struct PrefillMoEGrouping {
+    // PrefillMoEGrouping.swift:49-110. Sort key: (expertSortKeys[expert] if given, expert, token, rank).
+    static PrefillMoEGroupedRoutes groupTokenExpertPairs(const std::vector<PrefillTokenExpertPair> &pairs, int queryCount,
+                                                         int topK, int numExperts, int tileExpertCount,
+                                                         const std::vector<uint64_t> *expertSortKeys = nullptr) {
+        if (!(queryCount >= 0 && topK > 0 && numExperts > 0 && tileExpertCount >= 1 && tileExpertCount <= 16))
+            throw std::invalid_argument("groupTokenExpertPairs: bad arguments");
+        if (pairs.size() > (size_t)queryCount * (size_t)topK) throw std::invalid_argument("more pairs than queryCount * topK");
+        if (expertSortKeys && expertSortKeys->size() != (size_t)numExperts) throw std::invalid_argument("expertSortKeys count mismatch");
+        for (const auto &p : pairs)
+            if (p.expert >= (uint32_t)numExperts) throw PrefillMoEGroupingError(p.expert);
+        PrefillMoEGroupedRoutes out;
+        out.sortedPairs = pairs;
+        std::sort(out.sortedPairs.begin(), out.sortedPairs.end(),
+                  [&](const PrefillTokenExpertPair &a, const PrefillTokenExpertPair &b) {
+                      if (expertSortKeys) {
+                          const uint64_t ka = (*expertSortKeys)[a.expert], kb = (*expertSortKeys)[b.expert];
+                          if (ka != kb) return ka < kb;
+                      }
+                      if (a.expert != b.expert) return a.expert < b.expert;
+                      if (a.token != b.token) return a.token < b.token;
+                      return a.rank < b.rank;
+                  });
+        size_t i = 0;
+        while (i < out.sortedPairs.size()) {
+            const uint32_t expert = out.sortedPairs[i].expert;
+            const size_t start = i;
+            while (i < out.sortedPairs.size() && out.sortedPairs[i].expert == expert) ++i;
+            out.groups.push_back({expert, (uint32_t)start, (uint32_t)(i - start)});
+        }
+        size_t groupStart = 0;
+        while (groupStart < out.groups.size()) {
+            const size_t groupEnd = std::min(out.groups.size(), groupStart + (size_t)tileExpertCount);
+            const auto &first = out.groups[groupStart];
+            const auto &last = out.groups[groupEnd - 1];
+            out.tiles.push_back({(uint32_t)groupStart, (uint32_t)(groupEnd - groupStart), first.pairStart,
+                                 last.pairStart + last.pairCount - first.pairStart});
+            groupStart = groupEnd;
+        }
+        return out;
+    }
+};
+
+struct PrefillGroupedRoutedMoEError : std::runtime_error {
+    enum Kind { invalidStreamedTileBinding, allocationFailed } kind;
+    PrefillGroupedRoutedMoEError(Kind k, const std::string &reason)
+        : std::runtime_error((k == invalidStreamedTileBinding ? "invalid streamed tile binding: " : "failed to allocate ") + reason), kind(k) {}
+};
+
+// PrefillGroupedRoutedMoE.swift:121-166. With every expert resident in HBM a binding carries expert ids
+// only (the reference also carries one TensorView per expert); the validation rules are the same.
+struct PrefillStreamedTileBinding {
+    std::vector<int> expertIDs;
+    explicit PrefillStreamedTileBinding(std::vector<int> ids) : expertIDs(std::move(ids)) {
+        using E = PrefillGroupedRoutedMoEError;
+        if (expertIDs.empty()) throw E(E::invalidStreamedTileBinding, "tile binding must include at least one expert");
+        if (expertIDs.size() > 16)
+            throw E(E::invalidStreamedTileBinding, "tile binding has " + std::to_string(expertIDs.size()) + " experts; maximum is 16");
+        std::set<int> seen;
+        for (int e : expertIDs) {
+            if (e < 0) throw E(E::invalidStreamedTileBinding, "expert id " + std::to_string(e) + " must be non-negative");
+            if (!seen.insert(e).second) throw E(E::invalidStreamedTileBinding, "duplicate expert id " + std::to_string(e) + " in tile binding");
+        }
+    }
+    static std::vector<int> expertIDsForTile(int tileIndex, const PrefillMoEGroupedRoutes &routes) {
+        const auto &tile = routes.tiles.at(tileIndex);
+        std::vector<int> ids;
+        for (uint32_t g = tile.groupStart; g < tile.groupStart + tile.groupCount; ++g) ids.push_back((int)routes.groups[g].expert);
+        return ids;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------
+// Operators. Every encode... enqueues on `stream` and returns; device pointers are caller-owned.
+// ---------------------------------------------------------------------------------------------------
+class PrefillRouter {
+public:
+    explicit PrefillRouter(Context &c) : c_(c) {}
+    // PrefillRouter.swift:30-73
+    void encodeGemma4Block(void *stream, uint32_t layer, const uint16_t *hidden, uint32_t *outIndices, uint16_t *outWeights,
+                           uint32_t queryCount, uint32_t hiddenStrideElements) {
+        if (queryCount == 0) throw std::invalid_argument("queryCount must be positive");
+        if (hiddenStrideElements < c_.shape().d) throw std::invalid_argument("hidden stride is too small");
+        char *err = nullptr;
+        check(ffmoe_router(c_.raw(), stream, layer, hidden, hiddenStrideElements, queryCount, outIndices, outWeights, nullptr, &err), err);
+    }
+    // PrefillRouter.swift:75-95: token-major pairs; weights are 16-bit patterns
+    static std::vector<PrefillTokenExpertPair> makeTokenExpertPairs(const std::vector<uint32_t> &indices,
+                                                                    const std::vector<uint16_t> &weights, int queryCount, int topK) {
+        if (queryCount < 0) throw std::invalid_argument("queryCount must be non-negative");
+        if (topK < 0) throw std::invalid_argument("topK must be non-negative");
+        if (indices.size() != (size_t)queryCount * topK) throw std::invalid_argument("indices count mismatch");
+        if (weights.size() != (size_t)queryCount * topK) throw std::invalid_argument("weights count mismatch");
+        std::vector<PrefillTokenExpertPair> pairs;
+        pairs.reserve(indices.size());
+        for (int token = 0; token < queryCount; ++token)
+            for (int rank = 0; rank < topK; ++rank) {
+                const size_t i = (size_t)token * topK + rank;
+                pairs.push_back({(uint32_t)token, indices[i], (uint32_t)rank, (uint32_t)weights[i]});
+            }
+        return pairs;
+    }
+
+private:
+    Context &c_;
+};
+
+class MoE {
+public:
+    static constexpr int maxStreamedExperts = 8;
+    static constexpr int maxRouterRows = 16;
+    explicit MoE(Context &c) : c_(c) {}
+    // MoE.encodeRouterGemma4 (MoE.swift:168-237): one hidden row
+    void encodeRouterGemma4(void *stream, uint32_t layer, const uint16_t *hidden, uint32_t *outIndices, uint16_t *outWeights) {
+        encodeRouterRowsGemma4(stream, layer, hidden, c_.shape().d, 1, outIndices, outWeights);
+    }
+    // MoE.encodeRouterRowsGemma4 (MoE.swift:249-300): rows <= 16 hidden rows of a block
+    void encodeRouterRowsGemma4(void *stream, uint32_t layer, const uint16_t *hidden, uint32_t hiddenStrideElements, int rows,
+                                uint32_t *outIndices, uint16_t *outWeights) {
+        if (rows < 1 || rows > maxRouterRows) throw std::invalid_argument("rows outside 1...16");
+        char *err = nullptr;
+        check(ffmoe_router(c_.raw(), stream, layer, hidden, hiddenStrideElements, (uint32_t)rows, outIndices, outWeights, nullptr, &err), err);
+    }
+    // encodeRoutedPersistentPhase1U16Load + encodeRoutedPersistentPhase2Reduce, and the GPU-routed form
+    // encodeGatherRoutedSlots + encodeRoutedPersistentGPUSlots (MoE.swift:312-496): the slots are the router's
+    // `indices` on the device; no host read-back, no address table (every expert is resident).
+    void encodeRoutedPersistentGPUSlots(void *stream, uint32_t layer, const uint16_t *x, const uint32_t *indices,
+                                        const uint16_t *routingWeights, const uint16_t *residual, uint16_t *y) {
+        char *err = nullptr;
+        check(ffmoe_verify(c_.raw(), stream, layer, x, c_.shape().d, 1, indices, routingWeights, residual, y, &err), err);
+    }
+
+private:
+    Context &c_;
+};
+
+class PrefillGroupedRoutedMoE {
+public:
+    static constexpr int verifyMaxRows = 16;
+    explicit PrefillGroupedRoutedMoE(Context &c) : c_(c) {}
+    // encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:275-326): `sortedPairs` on the device, un-weighted rows out
+    void encodeStreamedBatched(void *stream, uint32_t layer, const uint16_t *hidden, uint32_t hiddenStrideElements,
+                               const PrefillTokenExpertPair *sortedPairs, uint32_t pairCount, uint32_t queryCount,
+                               uint16_t *routePartials) {
+        char *err = nullptr;
+        check(ffmoe_prefill_pairs(c_.raw(), stream, layer, hidden, hiddenStrideElements,
+                                  reinterpret_cast<const ffmoe_pair *>(sortedPairs), pairCount, queryCount, routePartials, &err), err);
+    }
+    // encodeVerifyBound / encodeVerifyRows (PrefillGroupedRoutedMoE.swift:331-448): rows <= 16, routes on the device
+    void encodeVerifyBound(void *stream, uint32_t layer, const uint16_t *hidden, uint32_t hiddenStrideElements, int rows,
+                           const uint32_t *routeIDs, const uint16_t *routeWeights, uint16_t *routePartials) {
+        if (rows <= 0 || rows > verifyMaxRows) throw std::invalid_argument("rows outside 1...16");
+        char *err = nullptr;
+        check(ffmoe_verify_partials(c_.raw(), stream, layer, hidden, hiddenStrideElements, (uint32_t)rows, routeIDs, routeWeights,
+                                    routePartials, &err), err);
+    }
+    // the whole prefill stage on the GPU: sort + experts + reduce, no host wait between router and experts
+    void encodeGPURouted(void *stream, uint32_t layer, const uint16_t *hidden, uint32_t hiddenStrideElements, uint32_t queryCount,
+                         const uint32_t *routeIDs, const uint16_t *routeWeights, uint16_t *h2) {
+        char *err = nullptr;
+        check(ffmoe_prefill(c_.raw(), stream, layer, hidden, hiddenStrideElements, queryCount, routeIDs, routeWeights, h2, &err), err);
+    }
+
+private:
+    Context &c_;
+};
+
+class PrefillMoE {
+public:
+    explicit PrefillMoE(Context &c) : c_(c) {}
+    // PrefillMoE.swift:11-32
+    void encodeReduceTokenMajor(void *stream, const uint16_t *routePartials, const uint16_t *routeWeights, uint16_t *h2,
+                                uint32_t queryCount, uint32_t topK, uint32_t d) {
+        if (queryCount == 0) throw std::invalid_argument("queryCount must be positive");
+        if (topK == 0) throw std::invalid_argument("topK must be positive");
+        if (d == 0) throw std::invalid_argument("D must be positive");
+        char *err = nullptr;
+        check(ffmoe_reduce_token_major(c_.raw(), stream, routePartials, routeWeights, h2, queryCount, topK, d, &err), err);
+    }
+
+private:
+    Context &c_;
+};
+
+class DequantInt4GEMV {
+public:
+    static constexpr int maxBatchRows = 16;
+    enum class RowsTypes { bf16, bf16ToF32 };
+    explicit DequantInt4GEMV(Context &c) : c_(c) {}
+    // DequantInt4GEMV.encode (DequantInt4GEMV.swift:184-224)
+    void encode(void *stream, const uint8_t *weights, const uint16_t *scales, const uint16_t *biases, const uint16_t *x, uint16_t *y,
+                uint32_t m, uint32_t n) {
+        encodeRows(stream, weights, scales, biases, x, y, m, n, 1, n, m, RowsTypes::bf16);
+    }
+    // DequantInt4GEMV.encodeRows (DequantInt4GEMV.swift:72-123)
+    void encodeRows(void *stream, const uint8_t *weights, const uint16_t *scales, const uint16_t *biases, const uint16_t *x, void *y,
+                    uint32_t m, uint32_t n, int rows, uint32_t xStrideElements, uint32_t yStrideElements, RowsTypes types) {
+        if (rows <= 0 || rows > maxBatchRows) throw std::invalid_argument("rows outside 1...16");
+        if (n % FFMOE_GROUP) throw std::invalid_argument("N must be a multiple of 64");
+        char *err = nullptr;
+        check(ffmoe_gemv_int4(c_.raw(), stream, weights, scales, biases, x, y, m, n, (uint32_t)rows, xStrideElements, yStrideElements,
+                              types == RowsTypes::bf16ToF32 ? 1 : 0, &err), err);
+    }
+
+private:
+    Context &c_;
+};
+
+// ---------------------------------------------------------------------------------------------------
+// Guest plugin and supervisor (Runtime/Supervisor/DeviceSupervisor.swift:5-125).
+// ---------------------------------------------------------------------------------------------------
+enum class RuntimeFaultPolicy { failClosed, failoverHost };   // reference: .failClosed / .failoverMetal
+
+struct CancellationError : std::runtime_error {
+    CancellationError() : std::runtime_error("cancelled") {}
+};
+
+// Routed top-k prefill for one layer on a rail other than the host's. On return every routed (token, rank)
+// row named by `pairs` has been written to `partials`; on throw the guest has drained its own work, so the
+// host may overwrite `partials` at once.
+struct RoutedPrefillGuest {
+    virtual ~RoutedPrefillGuest() = default;
+    virtual void runLayer(int layer, const uint16_t *hidden, uint16_t *partials, const PrefillMoEGroupedRoutes &routes,
+                          const PrefillTokenExpertPair *pairsOnDevice) = 0;
+    virtual std::string profile() const { return "{}"; }
+};
+
+// The guest that runs routed prefill on this library's kernels (stands where ANERoutedPrefillBackend stood).
+class HipRoutedPrefillGuest : public RoutedPrefillGuest {
+public:
+    HipRoutedPrefillGuest(Context &c, void *stream, uint32_t queryCount, uint32_t hiddenStrideElements,
+                          std::function<void(void *)> synchronize)
+        : moe_(c), stream_(stream), queryCount_(queryCount), stride_(hiddenStrideElements), sync_(std::move(synchronize)) {}
+    void runLayer(int layer, const uint16_t *hidden, uint16_t *partials, const PrefillMoEGroupedRoutes &routes,
+                  const PrefillTokenExpertPair *pairsOnDevice) override {
+        moe_.encodeStreamedBatched(stream_, (uint32_t)layer, hidden, stride_, pairsOnDevice, (uint32_t)routes.sortedPairs.size(),
+                                   queryCount_, partials);
+        if (sync_) sync_(stream_);   // the contract: rows are written when runLayer returns
+        ++layers_;
+    }
+    std::string profile() const override { return "{\"layers_run\": " + std::to_string(layers_) + "}"; }
+
+private:
+    PrefillGroupedRoutedMoE moe_;
+    void *stream_;
+    uint32_t queryCount_, stride_;
+    std::function<void(void *)> sync_;
+    int layers_ = 0;
+};
+
+struct GuestFault {
+    enum class Action { failedClosed, evictedToHost };
+    int layer;
+    std::string message;
+    Action action;
+    bool operator==(const GuestFault &o) const { return layer == o.layer && message == o.message && action == o.action; }
+};
+
+class DeviceSupervisor {
+public:
+    DeviceSupervisor(int guestLayers, RuntimeFaultPolicy policy, std::shared_ptr<RoutedPrefillGuest> guest)
+        : guestLayers_(guest ? guestLayers : 0), faultPolicy_(policy), guest_(std::move(guest)) {}
+    int guestLayers() const { return guestLayers_; }
+    RuntimeFaultPolicy faultPolicy() const { return faultPolicy_; }
+    bool evicted() const { return evicted_; }
+    const std::vector<GuestFault> &faults() const { return faults_; }
+    // nullptr when the layer is the host's: never admitted again after an eviction
+    RoutedPrefillGuest *routedPrefill(int layer) const { return (!evicted_ && layer < guestLayers_) ? guest_.get() : nullptr; }
+    // true: the guest completed. false: evicted, the host must run the layer. failClosed rethrows; cancellation
+    // always propagates (DeviceSupervisor.swift:94-109).
+    bool supervise(int layer, const std::function<void()> &body) {
+        try {
+            body();
+            return true;
+        } catch (const CancellationError &) {
+            throw;
+        } catch (const std::exception &e) {
+            const bool closed = faultPolicy_ == RuntimeFaultPolicy::failClosed;
+            faults_.push_back({layer, e.what(), closed ? GuestFault::Action::failedClosed : GuestFault::Action::evictedToHost});
+            if (closed) throw;
+            evicted_ = true;
+            return false;
+        }
+    }
+
+private:
+    int guestLayers_;
+    RuntimeFaultPolicy faultPolicy_;
+    std::shared_ptr<RoutedPrefillGuest> guest_;
+    bool evicted_ = false;
+    std::vector<GuestFault> faults_;
+};
+
+}  // namespace fieldfare

@@ -1,0 +1,199 @@
+// GPU test of the C++ operator mirror: the reference's call sequence for one prefill layer
+// (RealForwardRunner.swift:1487-1599) and one decode layer (:1846-1923) driven through the mirrored
+// classes, checked against the CPU oracle. Built with hipcc, run by tests/test_host_cpp.py.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+#include "../../ane-fieldfare_amd/host/fieldfare_host.hpp"
+#include "../../oracle/ffmoe_oracle.h"
+
+using namespace fieldfare;
+
+static int failures = 0;
+#define EXPECT(cond)                                                              \
+    do {                                                                          \
+        if (!(cond)) { std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond); ++failures; } \
+    } while (0)
+#define HIP(x)                                                                                   \
+    do {                                                                                         \
+        hipError_t e_ = (x);                                                                     \
+        if (e_ != hipSuccess) { std::printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); return 2; } \
+    } while (0)
+
+template <typename T>
+static T *toDevice(const std::vector<T> &v) {
+    T *p = nullptr;
+    if (hipMalloc(reinterpret_cast<void **>(&p), v.size() * sizeof(T)) != hipSuccess) return nullptr;
+    (void)hipMemcpy(p, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice);
+    return p;
+}
+template <typename T>
+static std::vector<T> toHost(const T *p, size_t n) {
+    std::vector<T> v(n);
+    (void)hipMemcpy(v.data(), p, n * sizeof(T), hipMemcpyDeviceToHost);
+    return v;
+}
+
+static void errorStats(const std::vector<uint16_t> &got, const std::vector<float> &ref, double &rel, double &cosine) {
+    double maxd = 0, maxr = 0, dot = 0, ng = 0, nr = 0;
+    for (size_t i = 0; i < ref.size(); ++i) {
+        const double g = ffo_bf16_to_float(got[i]), r = ref[i];
+        maxd = std::fmax(maxd, std::fabs(g - r));
+        maxr = std::fmax(maxr, std::fabs(r));
+        dot += g * r; ng += g * g; nr += r * r;
+    }
+    rel = maxd / std::fmax(maxr, 1e-6);
+    cosine = dot / std::sqrt(ng * nr);
+}
+
+struct FaultingGuest : RoutedPrefillGuest {
+    void runLayer(int, const uint16_t *, uint16_t *, const PrefillMoEGroupedRoutes &, const PrefillTokenExpertPair *) override {
+        throw std::runtime_error("injected guest fault");
+    }
+};
+
+int main() {
+    const int d = 128, f = 64, E = 16, K = 8, T = 40;
+    // synthetic experts: uniform weights quantised with the reference quantiser, blob layout of makeBlob
+    // (MoEFusedFFNTests.swift:221-257)
+    const size_t guW = (size_t)f * d / 2, guS = (size_t)f * (d / 64) * 2, dnW = (size_t)d * f / 2, dnS = (size_t)d * (f / 64) * 2;
+    ffmoe_offsets off{};
+    uint32_t cur = 0;
+    auto take = [&](size_t n) { uint32_t o = cur; cur += (uint32_t)n; return o; };
+    off.gate_w = take(guW); off.gate_s = take(guS); off.gate_b = take(guS);
+    off.up_w = take(guW);   off.up_s = take(guS);   off.up_b = take(guS);
+    off.down_w = take(dnW); off.down_s = take(dnS); off.down_b = take(dnS);
+    const size_t stride = cur;
+    std::vector<uint8_t> pool(stride * E);
+    uint64_t rng = 0x5EED;
+    auto fill = [&](uint8_t *blob, uint32_t wOff, uint32_t sOff, uint32_t bOff, int rows, int cols) {
+        std::vector<float> row(cols);
+        for (int r = 0; r < rows; ++r) {
+            ffo_splitmix64_fill_uniform(&rng, -0.4f, 0.4f, row.data(), cols);
+            ffo_quantize_int4_affine(row.data(), cols, blob + wOff + (size_t)r * cols / 2,
+                                     reinterpret_cast<uint16_t *>(blob + sOff) + (size_t)r * (cols / 64),
+                                     reinterpret_cast<uint16_t *>(blob + bOff) + (size_t)r * (cols / 64));
+        }
+    };
+    for (int e = 0; e < E; ++e) {
+        uint8_t *blob = pool.data() + e * stride;
+        fill(blob, off.gate_w, off.gate_s, off.gate_b, f, d);
+        fill(blob, off.up_w, off.up_s, off.up_b, f, d);
+        fill(blob, off.down_w, off.down_s, off.down_b, d, f);
+    }
+    std::vector<uint16_t> router((size_t)E * d), x((size_t)T * d);
+    for (auto &v : router) v = ffo_bf16_bits(ffo_splitmix64_uniform(&rng, -0.05f, 0.05f));
+    for (auto &v : x) v = ffo_bf16_bits(ffo_splitmix64_uniform(&rng, -1.0f, 1.0f));
+
+    ffmoe_shape shape{(uint32_t)d, (uint32_t)f, (uint32_t)E, (uint32_t)K, 1, 64};
+    Context ctx(0, shape);
+    ctx.uploadLayer(0, pool.data(), stride, off);
+    ctx.uploadRouterBF16(0, router.data());
+    hipStream_t stream;
+    HIP(hipStreamCreate(&stream));
+
+    uint16_t *dx = toDevice(x);
+    uint32_t *dIdx = nullptr;
+    uint16_t *dW = nullptr, *dPartials = nullptr, *dH2 = nullptr, *dH2b = nullptr;
+    HIP(hipMalloc(reinterpret_cast<void **>(&dIdx), (size_t)T * K * 4));
+    HIP(hipMalloc(reinterpret_cast<void **>(&dW), (size_t)T * K * 2));
+    HIP(hipMalloc(reinterpret_cast<void **>(&dPartials), (size_t)T * K * d * 2));
+    HIP(hipMalloc(reinterpret_cast<void **>(&dH2), (size_t)T * d * 2));
+    HIP(hipMalloc(reinterpret_cast<void **>(&dH2b), (size_t)T * d * 2));
+
+    // --- prefill layer, host-routed through the guest (the reference's sequence) ---
+    PrefillRouter prefillRouter(ctx);
+    PrefillGroupedRoutedMoE grouped(ctx);
+    PrefillMoE prefillMoE(ctx);
+    prefillRouter.encodeGemma4Block(stream, 0, dx, dIdx, dW, T, d);
+    HIP(hipStreamSynchronize(stream));                       // the reference's waitForCompletion(cb)
+    auto idx = toHost(dIdx, (size_t)T * K);
+    auto w = toHost(dW, (size_t)T * K);
+    auto pairs = PrefillRouter::makeTokenExpertPairs(idx, w, T, K);
+    auto routes = PrefillMoEGrouping::groupTokenExpertPairs(pairs, T, K, E, 16);
+    PrefillTokenExpertPair *dPairs = toDevice(routes.sortedPairs);
+    auto sync = [](void *s) { (void)hipStreamSynchronize(static_cast<hipStream_t>(s)); };
+    DeviceSupervisor supervisor(1, RuntimeFaultPolicy::failoverHost,
+                                std::make_shared<HipRoutedPrefillGuest>(ctx, stream, T, d, sync));
+    HIP(hipMemsetAsync(dPartials, 0, (size_t)T * K * d * 2, stream));   // the host zeroes partials first
+    bool done = false;
+    if (auto *guest = supervisor.routedPrefill(0))
+        done = supervisor.supervise(0, [&] { guest->runLayer(0, dx, dPartials, routes, dPairs); });
+    EXPECT(done && !supervisor.evicted());
+    prefillMoE.encodeReduceTokenMajor(stream, dPartials, dW, dH2, T, K, d);
+    HIP(hipStreamSynchronize(stream));
+    auto h2 = toHost(dH2, (size_t)T * d);
+
+    std::vector<float> wf(w.size()), ref((size_t)T * d);
+    for (size_t i = 0; i < w.size(); ++i) wf[i] = ffo_bf16_to_float(w[i]);
+    ffo_offsets ooff;
+    std::memcpy(&ooff, &off, sizeof ooff);
+    ffo_moe_experts(pool.data(), stride, &ooff, d, f, x.data(), d, T, K, FFO_BF16, idx.data(), wf.data(), ref.data(), 0);
+    double rel, cosine;
+    errorStats(h2, ref, rel, cosine);
+    std::printf("prefill via guest: rel err %.2e cosine %.6f\n", rel, cosine);
+    EXPECT(rel <= 1e-2 && cosine >= 0.9999);
+    // router indices are the oracle's
+    std::vector<float> logits(E), ow(K);
+    std::vector<uint32_t> oidx(K);
+    for (int t = 0; t < T; ++t) {
+        ffo_router_logits_pinned(router.data(), 0, x.data() + (size_t)t * d, FFO_BF16, nullptr, E, d, logits.data());
+        ffo_topk_softmax(logits.data(), E, K, nullptr, oidx.data(), ow.data());
+        EXPECT(std::memcmp(oidx.data(), idx.data() + (size_t)t * K, K * 4) == 0);
+    }
+
+    // --- the same layer GPU-routed: bit-identical to the host-routed result ---
+    grouped.encodeGPURouted(stream, 0, dx, d, T, dIdx, dW, dH2b);
+    HIP(hipStreamSynchronize(stream));
+    EXPECT(toHost(dH2b, (size_t)T * d) == h2);
+
+    // --- a faulting guest under failover: the host clears the rows and runs the layer itself ---
+    DeviceSupervisor failing(1, RuntimeFaultPolicy::failoverHost, std::make_shared<FaultingGuest>());
+    done = failing.supervise(0, [&] { failing.routedPrefill(0)->runLayer(0, dx, dPartials, routes, dPairs); });
+    EXPECT(!done && failing.evicted() && failing.faults().size() == 1 && failing.routedPrefill(0) == nullptr);
+    HIP(hipMemsetAsync(dPartials, 0, (size_t)T * K * d * 2, stream));
+    grouped.encodeStreamedBatched(stream, 0, dx, d, dPairs, (uint32_t)routes.sortedPairs.size(), T, dPartials);
+    prefillMoE.encodeReduceTokenMajor(stream, dPartials, dW, dH2b, T, K, d);
+    HIP(hipStreamSynchronize(stream));
+    EXPECT(toHost(dH2b, (size_t)T * d) == h2);
+
+    // --- decode layer: router + GPU slots ---
+    MoE moe(ctx);
+    moe.encodeRouterGemma4(stream, 0, dx, dIdx, dW);
+    moe.encodeRoutedPersistentGPUSlots(stream, 0, dx, dIdx, dW, nullptr, dH2b);
+    HIP(hipStreamSynchronize(stream));
+    auto y1 = toHost(dH2b, d);
+    auto idx1 = toHost(dIdx, K);
+    auto w1 = toHost(dW, K);
+    std::vector<float> w1f(K), ref1(d);
+    for (int i = 0; i < K; ++i) w1f[i] = ffo_bf16_to_float(w1[i]);
+    ffo_moe_experts(pool.data(), stride, &ooff, d, f, x.data(), d, 1, K, FFO_BF16, idx1.data(), w1f.data(), ref1.data(), 0);
+    errorStats(y1, ref1, rel, cosine);
+    std::printf("decode: rel err %.2e cosine %.6f\n", rel, cosine);
+    EXPECT(rel <= 1e-2 && cosine >= 0.9999);
+    bool threw = false;
+    try { moe.encodeRouterRowsGemma4(stream, 0, dx, d, 17, dIdx, dW); } catch (const std::invalid_argument &) { threw = true; }
+    EXPECT(threw);
+
+    // --- DequantInt4GEMV on one expert's gate matrix (reference layout, device copy of the blob) ---
+    uint8_t *dPool = toDevice(pool);
+    uint16_t *dY = nullptr;
+    HIP(hipMalloc(reinterpret_cast<void **>(&dY), f * 2));
+    DequantInt4GEMV gemv(ctx);
+    gemv.encode(stream, dPool + off.gate_w, reinterpret_cast<uint16_t *>(dPool + off.gate_s),
+                reinterpret_cast<uint16_t *>(dPool + off.gate_b), dx, dY, f, d);
+    HIP(hipStreamSynchronize(stream));
+    auto yg = toHost(dY, f);
+    std::vector<float> xf(d), refg(f);
+    for (int i = 0; i < d; ++i) xf[i] = ffo_bf16_to_float(x[i]);
+    ffo_gemv_int4_ref(pool.data() + off.gate_w, reinterpret_cast<uint16_t *>(pool.data() + off.gate_s),
+                      reinterpret_cast<uint16_t *>(pool.data() + off.gate_b), f, d, xf.data(), refg.data());
+    errorStats(yg, refg, rel, cosine);
+    EXPECT(rel <= 1e-2);
+
+    std::printf(failures ? "%d FAILURES\n" : "host gpu ok\n", failures);
+    return failures ? 1 : 0;
+}
