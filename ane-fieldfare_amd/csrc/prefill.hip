@@ -72,8 +72,10 @@ __global__ __launch_bounds__(256) void prefill_scan_kernel(uint32_t n_blocks, ui
     __shared__ uint32_t tile_off[FFMOE_MAX_EXPERTS + 1];
     const uint32_t e = threadIdx.x;
     uint32_t sum = 0;
-    if (e < n_experts)
+    if (e < n_experts) {
+#pragma unroll 16
         for (uint32_t b = 0; b < n_blocks; ++b) sum += block_cnt[(size_t)b * n_experts + e];
+    }
     total[e] = e < n_experts ? sum : 0;
     __syncthreads();
     if (e == 0) {
@@ -94,10 +96,15 @@ __global__ __launch_bounds__(256) void prefill_scan_kernel(uint32_t n_blocks, ui
         uint32_t run = offset[e];
         plan->expert_offset[e] = run;
         plan->expert_count[e] = total[e];
-        for (uint32_t b = 0; b < n_blocks; ++b) {
-            const uint32_t c = block_cnt[(size_t)b * n_experts + e];
-            block_cnt[(size_t)b * n_experts + e] = run;      // count -> base, in place
-            run += c;
+        for (uint32_t b0 = 0; b0 < n_blocks; b0 += 16) {
+            uint32_t c[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) c[u] = b0 + u < n_blocks ? block_cnt[(size_t)(b0 + u) * n_experts + e] : 0;
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                if (b0 + u < n_blocks) block_cnt[(size_t)(b0 + u) * n_experts + e] = run;      // count -> base, in place
+                run += c[u];
+            }
         }
         const uint32_t nt = (total[e] + kBM - 1) / kBM;
         for (uint32_t i = 0; i < nt; ++i) {

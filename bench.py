@@ -68,6 +68,7 @@ def main():
     ap.add_argument("--tokens", type=int, default=16)
     ap.add_argument("--prefill-tokens", type=int, default=3072, help="0 skips the prefill leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode (T = 1) leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only; --gpus must be 1 "
@@ -159,16 +160,17 @@ def main():
     def decode(layer):
         Lib.ffmoe_router(h, stream, layer, px1, D, 1, pidx, pw, None, C.byref(err))
         Lib.ffmoe_verify(h, stream, layer, px1, D, 1, pidx, pw, None, py, C.byref(err))
-    for i in range(L):
-        decode(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(4 * L):
-        decode(i % L)
-    torch.cuda.synchronize()
-    dec = (time.perf_counter() - t0) / (4 * L)
-    extra["decode_us_per_layer"] = round(dec * 1e6, 2)
-    extra["decode_expert_GBs"] = round(K * EXPERT_BYTES / dec / 1e9, 1)
+    if not args.no_decode:
+        for i in range(L):
+            decode(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(4 * L):
+            decode(i % L)
+        torch.cuda.synchronize()
+        dec = (time.perf_counter() - t0) / (4 * L)
+        extra["decode_us_per_layer"] = round(dec * 1e6, 2)
+        extra["decode_expert_GBs"] = round(K * EXPERT_BYTES / dec / 1e9, 1)
 
     # prefill half of the metric (BASELINE.json config 4): 3,072 tokens through one MoE layer, router
     # included, near-uniform routing from the Gaussian router; layers cycle as above
