@@ -173,31 +173,126 @@ __global__ __launch_bounds__(256) void router_small_kernel(const void *__restric
     }
 }
 
-// Prefill router logits. grid = (ceil(E / 4), ceil(T / tokens_per_wave)); one wave per expert row keeps
-// all four sub-accumulators itself and walks its tokens in chunks of four.
+// Prefill router logits: a register-tiled fp32 GEMM that keeps the pinned order. A block owns a tile of
+// 8 tokens x 8 experts; its four waves are the four sub-accumulators, each walking its own k-blocks with
+// the next block's operands already in flight, so every x and W load feeds 8 rows of fmaf. The partials
+// meet in LDS, each wave then finishes 16 of the 64 outputs: (s0 + s1) + (s2 + s3) per lane and the
+// xor-butterfly done as a halving exchange (a lane keeps half of its values and receives the partner's
+// matching half; fp addition is commutative, so every sum has the same operands as the full butterfly).
+// Blocks are numbered so that all expert groups of one token group run on the same XCD and share its L2.
+constexpr int kTileTok = 8, kTileExp = 8;
+
+template <bool W_F32> struct WRaw { uint2 v; };
+template <> struct WRaw<true> { f32x4 v; };
+
 template <bool W_F32, bool X_ALIGNED>
-__global__ __launch_bounds__(256) void router_logits_kernel(const void *__restrict__ w_, const uint16_t *__restrict__ es,
-                                                            const uint16_t *__restrict__ x, uint32_t x_stride,
-                                                            uint32_t t, uint32_t n_experts, uint32_t d,
-                                                            uint32_t tokens_per_wave, float *__restrict__ logits) {
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t e = blockIdx.x * 4 + wave;
-    if (e >= n_experts) return;
-    const uint32_t t_begin = blockIdx.y * tokens_per_wave;
-    const uint32_t t_end = min(t, t_begin + tokens_per_wave);
-    for (uint32_t t0 = t_begin; t0 < t_end; t0 += kChunkTokens) {
-        float sub[4][kChunkTokens];
+__global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict__ w_, const uint16_t *__restrict__ es,
+                                                          const uint16_t *__restrict__ x, uint32_t x_stride,
+                                                          uint32_t t, uint32_t n_experts, uint32_t d,
+                                                          uint32_t n_egroups, uint32_t n_tgroups,
+                                                          float *__restrict__ logits) {
+    __shared__ float s_part[4][kTileTok * kTileExp][64];
+    const uint32_t lane = threadIdx.x & 63, s = threadIdx.x >> 6;
+    const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const uint32_t tg = (slot / n_egroups) * 8 + xcd, eg = slot % n_egroups;
+    if (tg >= n_tgroups) return;
+    const uint32_t t0 = tg * kTileTok, e0 = eg * kTileExp;
+
+    const uint16_t *xrow[kTileTok];
+    size_t wrow[kTileExp];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
+    for (int r = 0; r < kTileTok; ++r) xrow[r] = x + (size_t)min(t0 + r, t - 1) * x_stride;
 #pragma unroll
-            for (int r = 0; r < kChunkTokens; ++r) sub[s][r] = 0.0f;
-            accumulate_sub<W_F32, X_ALIGNED>(w_, es, x, x_stride, e, d, s, lane, t0, t_end - 1, sub[s]);
+    for (int c = 0; c < kTileExp; ++c) wrow[c] = (size_t)min(e0 + c, n_experts - 1) * d;
+
+    float acc[kTileTok][kTileExp];
+#pragma unroll
+    for (int r = 0; r < kTileTok; ++r)
+#pragma unroll
+        for (int c = 0; c < kTileExp; ++c) acc[r][c] = 0.0f;
+
+    WRaw<W_F32> wn[kTileExp];
+    uint2 xn[kTileTok], en = make_uint2(0x3F803F80u, 0x3F803F80u);
+    auto fetch = [&](uint32_t k) {
+        if (k >= d) return;
+#pragma unroll
+        for (int c = 0; c < kTileExp; ++c) {
+            if (W_F32) wn[c].v = *reinterpret_cast<const decltype(wn[c].v) *>(reinterpret_cast<const float *>(w_) + wrow[c] + k);
+            else wn[c].v = *reinterpret_cast<const decltype(wn[c].v) *>(reinterpret_cast<const uint16_t *>(w_) + wrow[c] + k);
         }
 #pragma unroll
-        for (int r = 0; r < kChunkTokens; ++r) {
-            const float v = wave_butterfly_sum((sub[0][r] + sub[1][r]) + (sub[2][r] + sub[3][r]));
-            if (lane == 0 && t0 + r < t_end) logits[(size_t)(t0 + r) * n_experts + e] = v;
+        for (int r = 0; r < kTileTok; ++r) xn[r] = load_x4<X_ALIGNED>(xrow[r] + k);
+        if (es) en = *reinterpret_cast<const uint2 *>(es + k);
+    };
+
+    const uint32_t steps = (d + 1023) / 1024;
+    uint32_t k = 256 * s + 4 * lane;
+    fetch(k);
+    for (uint32_t i = 0; i < steps; ++i, k += 1024) {
+        const bool live = k < d;
+        float wv[kTileExp][4];
+        uint2 xc[kTileTok];
+#pragma unroll
+        for (int c = 0; c < kTileExp; ++c) {
+            if constexpr (W_F32) {
+                wv[c][0] = wn[c].v[0]; wv[c][1] = wn[c].v[1]; wv[c][2] = wn[c].v[2]; wv[c][3] = wn[c].v[3];
+            } else {
+                wv[c][0] = bf16lo_to_f32(wn[c].v.x); wv[c][1] = bf16hi_to_f32(wn[c].v.x);
+                wv[c][2] = bf16lo_to_f32(wn[c].v.y); wv[c][3] = bf16hi_to_f32(wn[c].v.y);
+            }
         }
+#pragma unroll
+        for (int r = 0; r < kTileTok; ++r) xc[r] = xn[r];
+        const float sc[4] = {bf16lo_to_f32(en.x), bf16hi_to_f32(en.x), bf16lo_to_f32(en.y), bf16hi_to_f32(en.y)};
+        if (i + 1 < steps) fetch(k + 1024);
+        if (live) {
+#pragma unroll
+            for (int r = 0; r < kTileTok; ++r) {
+                const float xf[4] = {bf16lo_to_f32(xc[r].x), bf16hi_to_f32(xc[r].x), bf16lo_to_f32(xc[r].y),
+                                     bf16hi_to_f32(xc[r].y)};
+                float xe[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xe[j] = es ? xf[j] * sc[j] : xf[j];   // exact: product of two bf16
+#pragma unroll
+                for (int c = 0; c < kTileExp; ++c)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[r][c] = __builtin_fmaf(wv[c][j], xe[j], acc[r][c]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kTileTok; ++r)
+#pragma unroll
+        for (int c = 0; c < kTileExp; ++c) s_part[s][r * kTileExp + c][lane] = acc[r][c];
+    __syncthreads();
+
+    // wave s finishes outputs 16 s .. 16 s + 15
+    float v[16];
+#pragma unroll
+    for (int o = 0; o < 16; ++o) {
+        const uint32_t q = 16 * s + o;
+        v[o] = (s_part[0][q][lane] + s_part[1][q][lane]) + (s_part[2][q][lane] + s_part[3][q][lane]);
+    }
+    // halving exchange: after the step with mask m the lane keeps the outputs whose index bit matches
+    // its own lane bit; four steps leave output (lane >> 2) & 15, two plain butterfly steps finish it.
+#pragma unroll
+    for (int step = 0; step < 4; ++step) {
+        const int m = 32 >> step, half = 8 >> step;
+        const bool upper = (lane & m) != 0;
+#pragma unroll
+        for (int o = 0; o < half; ++o) {
+            const float keep = upper ? v[o + half] : v[o];
+            const float send = upper ? v[o] : v[o + half];
+            v[o] = keep + __shfl_xor(send, m, 64);
+        }
+    }
+    float r0 = v[0];
+    r0 = r0 + __shfl_xor(r0, 2, 64);
+    r0 = r0 + __shfl_xor(r0, 1, 64);
+    if ((lane & 3) == 0) {
+        const uint32_t q = 16 * s + (lane >> 2);
+        const uint32_t tok = t0 + q / kTileExp, e = e0 + q % kTileExp;
+        if (tok < t && e < n_experts) logits[(size_t)tok * n_experts + e] = r0;
     }
 }
 
@@ -232,11 +327,11 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
         timer->finish();
         return hipGetLastError();
     }
-    const uint32_t tpw = 64;
-    const dim3 grid((n_experts + 3) / 4, (t + tpw - 1) / tpw);
+    const uint32_t n_egroups = (n_experts + kTileExp - 1) / kTileExp, n_tgroups = (t + kTileTok - 1) / kTileTok;
+    const dim3 grid(n_egroups * ((n_tgroups + 7) / 8) * 8);
 #define FFMOE_ROUTER(WF, XA)                                                                                 \
-    hipLaunchKernelGGL((router_logits_kernel<WF, XA>), grid, dim3(256), 0, s, rw.w, rw.effective_scale, x,   \
-                       x_stride, t, n_experts, d, tpw, logits)
+    hipLaunchKernelGGL((router_tile_kernel<WF, XA>), grid, dim3(256), 0, s, rw.w, rw.effective_scale, x,     \
+                       x_stride, t, n_experts, d, n_egroups, n_tgroups, logits)
     if (rw.w_is_f32) { if (x_aligned) FFMOE_ROUTER(true, true); else FFMOE_ROUTER(true, false); }
     else { if (x_aligned) FFMOE_ROUTER(false, true); else FFMOE_ROUTER(false, false); }
 #undef FFMOE_ROUTER

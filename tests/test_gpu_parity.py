@@ -175,6 +175,43 @@ def test_router_strided_rows_and_special_scores(small, oracle, torch):
         assert np.array_equal(idx[tok].cpu().numpy().astype(np.uint32), ridx)
 
 
+@pytest.mark.parametrize("t,d,e,pad,kind", [
+    (37, 320, 13, 0, "bf16"),      # ragged token and expert tiles, d not a multiple of 256
+    (64, 1344, 20, 13, "bf16"),    # stride d + 13: rows only 2-byte aligned
+    (130, 1088, 128, 8, "int8"),   # fp32 router weights with effective and per-expert scales
+    (17, 64, 1, 0, "bf16"),        # a single expert, top-1
+])
+def test_router_prefill_tiles_bit_exact(oracle, ff, torch, t, d, e, pad, kind):
+    # more than 16 rows take the tiled logits kernel; every logit must still match the pinned order
+    rng = np.random.default_rng(t * 1000 + d)
+    k = min(8, e)
+    ctx = ff.Context(d, 64, e, k, n_layers=1, max_tokens=t)
+    W = rng.normal(0, 0.2, (e, d)).astype(np.float32)
+    esb = pesb = None
+    if kind == "int8":
+        P, S, B = oracle.quantize_int8(W)
+        esb = oracle.bf16_bits(rng.uniform(0.5, 1.5, d).astype(np.float32))
+        pesb = oracle.bf16_bits(rng.uniform(0.6, 1.4, e).astype(np.float32))
+        ctx.upload_router_int8(0, P, S, B, esb, pesb)
+        Wref = oracle.dequantize_int8(P, S, B)
+    else:
+        Wref = oracle.bf16_bits(W)
+        ctx.upload_router_bf16(0, Wref)
+    buf = np.full((t, d + pad), 7.5, np.float32)
+    buf[:, :d] = rng.normal(0, 1, (t, d))
+    xb = oracle.bf16_bits(buf)
+    x = bf16_tensor(torch, xb)[:, :d]
+    idx, w, logits = ctx.router(0, x, want_logits=True)
+    logits = logits.cpu().numpy()
+    for tok in range(t):
+        ref = oracle.router_logits_pinned(Wref, xb[tok, :d], oracle.BF16, esb)
+        assert np.array_equal(logits[tok].view(np.uint32), ref.view(np.uint32)), f"token {tok}"
+        ridx, rw = oracle.topk_softmax(ref, k, pesb)
+        assert np.array_equal(idx[tok].cpu().numpy().astype(np.uint32), ridx)
+        assert np.abs(oracle.bf16_to_float(bits_of(w[tok])) - rw).max() <= np.abs(rw).max() * 2 ** -7
+    ctx.close()
+
+
 def _run_verify_case(case, oracle, torch, t, seed, mode="fused"):
     d, e = case["d"], case["n_experts"] if "n_experts" in case else case["e"]
     rng = np.random.default_rng(seed)
