@@ -20,16 +20,16 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_floa
 __device__ __forceinline__ float bf16lo_to_f32(uint32_t pair) { return __uint_as_float(pair << 16); }
 __device__ __forceinline__ float bf16hi_to_f32(uint32_t pair) { return __uint_as_float(pair & 0xFFFF0000u); }
 
-// Round-to-nearest-even fp32 -> bf16 with no NaN special case: the exact integer recipe of
-// Quantization.bf16Bits (Infrastructure/ModelIO/Quantization.swift:9-15), so the bits match the
-// reference's encoder for every input.
-__device__ __forceinline__ uint16_t f32_to_bf16(float x) {
-    uint32_t bits = __float_as_uint(x);
-    uint32_t lsb = (bits >> 16) & 1u;
-    return (uint16_t)((bits + (0x7FFFu + lsb)) >> 16);
-}
+// Round-to-nearest-even fp32 -> bf16 on the gfx950 converter (v_cvt_pk_bf16_f32). For every non-NaN
+// input the bits equal the integer recipe of Quantization.bf16Bits
+// (Infrastructure/ModelIO/Quantization.swift:9-15): add 0x7FFF + lsb, keep the high half.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint16_t f32_to_bf16(float x) { return __builtin_bit_cast(uint16_t, (__bf16)x); }
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+    bf16x2 v;
+    v[0] = (__bf16)lo;
+    v[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, v);
 }
 
 // gelu_pytorch_tanh, Metal/MoE/moe.metal:40-47 (clamp kept: it guards tanh at large magnitudes).
@@ -38,6 +38,15 @@ __device__ __forceinline__ float gelu_tanh(float x) {
     float inner = 0.7978845608028654f * (x + 0.044715f * x3);
     inner = fminf(fmaxf(inner, -20.0f), 20.0f);
     return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+// The same function through 0.5 (1 + tanh z) = 1 / (1 + exp(-2 z)) on the hardware exp2 and reciprocal:
+// about ten instructions instead of a tanhf call, relative error ~1e-6 (the result is rounded to bf16).
+__device__ __forceinline__ float gelu_tanh_fast(float x) {
+    const float x3 = x * x * x;
+    float inner = 0.7978845608028654f * (x + 0.044715f * x3);
+    inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-2.8853900817779268f * inner));
 }
 
 // Arena nibble order inside one dword: nibble position m (m = 0..3) holds element 2m of the lane's
@@ -59,20 +68,26 @@ __device__ __forceinline__ bf16x8 unpack8_offset128(uint32_t w) {
 // (Metal/Prefill/prefill.metal:581-590 with half replaced by bfloat as Metal/TensorCore/tensorops.metal:267).
 // q * scale is exact in fp32 (4-bit x 8-bit significands), so fma and mul-then-add agree.
 __device__ __forceinline__ uint4 dequant8_bf16(uint32_t w, float scale, float bias) {
+    // even nibbles / odd nibbles as bytes; the empty asm keeps the two masks as written so that each
+    // byte converts with one v_cvt_f32_ubyteN instead of a bit-field extract plus a convert
+    uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+    asm("" : "+v"(lo), "+v"(hi));
     uint4 r;
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-        const float q0 = (float)((w >> (4 * m)) & 0xFu);
-        const float q1 = (float)((w >> (4 * m + 16)) & 0xFu);
-        const uint32_t p = pack_bf16x2(__builtin_fmaf(q0, scale, bias), __builtin_fmaf(q1, scale, bias));
-        if (m == 0) r.x = p; else if (m == 1) r.y = p; else if (m == 2) r.z = p; else r.w = p;
-    }
+    r.x = pack_bf16x2(__builtin_fmaf((float)(lo & 0xFFu), scale, bias), __builtin_fmaf((float)((lo >> 16) & 0xFFu), scale, bias));
+    r.y = pack_bf16x2(__builtin_fmaf((float)(hi & 0xFFu), scale, bias), __builtin_fmaf((float)((hi >> 16) & 0xFFu), scale, bias));
+    r.z = pack_bf16x2(__builtin_fmaf((float)((lo >> 8) & 0xFFu), scale, bias), __builtin_fmaf((float)(lo >> 24), scale, bias));
+    r.w = pack_bf16x2(__builtin_fmaf((float)((hi >> 8) & 0xFFu), scale, bias), __builtin_fmaf((float)(hi >> 24), scale, bias));
     return r;
 }
 
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
+
+// Workgroup barrier that waits for this wave's LDS traffic only. __syncthreads() also drains every
+// outstanding global load, which would serialise a register prefetch that is meant to stay in flight
+// across the barrier; here the compiler's own counters still guard each prefetched register at its use.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // xor-butterfly sum across the 64 lanes (masks 32,16,8,4,2,1): every lane ends with the same value.
 __device__ __forceinline__ float wave_butterfly_sum(float v) {

@@ -78,7 +78,6 @@ struct KernelTimer {
 };
 
 // Prefill: expert-sorted pairs and their M-tiles, built on the GPU.
-#define FFMOE_PREFILL_TILE_M 128
 struct PrefillTile {
     uint32_t expert, row_start, rows, pad;     // rows [row_start, row_start + rows) of the sorted pair list
 };

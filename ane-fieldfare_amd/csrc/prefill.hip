@@ -11,11 +11,11 @@
 // order the reference's comparator produces (PrefillMoEGrouping.swift:66-75). Only integer counting uses
 // LDS atomics; every position comes from prefix sums, so the result does not depend on timing.
 //
-// GEMM: one block = one M-tile of up to 128 same-expert pairs x 128 weight rows (4 arena tiles per
-// 64-wide group). Per group the block stages the pairs' inputs (bf16) and the four tiles' weights,
-// each expanded once to bf16(fma(q, scale, bias)) - the reference's 16-bit tile weight
-// (prefill.metal:581-590) - in the register layout v_mfma_f32_16x16x32_bf16 wants, so every wave reads
-// its operands with 16-byte LDS loads. fp32 accumulation; GELU-tanh(gate) * up in the epilogue.
+// GEMM: one block = one M-tile of up to 256 same-expert pairs x 128 weight rows (4 arena tiles per
+// 64-wide group). Per group the four tiles' weights are expanded once to bf16(fma(q, scale, bias)) - the
+// reference's 16-bit tile weight (prefill.metal:581-590) - into LDS in the register layout
+// v_mfma_f32_16x16x32_bf16 wants; the pairs' inputs go from global memory straight into that layout.
+// fp32 accumulation; GELU-tanh(gate) * up in the epilogue.
 // bf16 activations make the reference's power-of-two block scaling (prefill.metal:593-598, an FP16 range
 // fix) unnecessary.
 #include "common.hpp"
@@ -148,110 +148,174 @@ __global__ __launch_bounds__(kSortBlock) void prefill_scatter_kernel(ItemSource 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Grouped GEMM. grid = (N-blocks, tile capacity); block = 4 waves. Wave w expands arena tile w of the
-// N-block per group and owns pairs [32 w, 32 w + 32) of the M-tile against all 128 weight rows.
+// Grouped GEMM. One block = one M-tile (up to 256 pairs of one expert) x one N-block (4 arena tiles =
+// 128 weight rows); block ids are laid out so that all N-blocks of an M-tile run on one XCD and find the
+// tile's A rows in that XCD's L2. The M-tile's 16-row blocks are dealt round-robin to the four waves
+// (wave w owns blocks w, w + 4, ...), so a short tile still loads all four matrix units evenly.
+//   A: every lane loads its own MFMA fragments straight from global memory (16 B per fragment), one
+//      64-wide group ahead, into registers - the rows are private to the wave, LDS would add nothing.
+//   B: wave w expands arena tile w of the next group to bf16(fma(q, scale, bias)) into the other half of
+//      a double-buffered LDS area while all waves multiply from the current half; one barrier per group.
 // GATE_UP: A rows are gathered token rows of x; streams are gate / up; out = acts[pair][F].
 // else:    A rows are acts[pair][F]; streams are two 16-row blocks; out = partials[out_row][D] (bf16).
 // ---------------------------------------------------------------------------------------------------
-template <bool GATE_UP>
-__global__ __launch_bounds__(256) void prefill_gemm_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
-                                                           const PrefillPlan *__restrict__ plan,
-                                                           const PrefillTile *__restrict__ tiles,
-                                                           const uint32_t *__restrict__ sorted_token,
-                                                           const uint32_t *__restrict__ sorted_out_row,
-                                                           const uint16_t *__restrict__ a, uint32_t a_stride,
-                                                           uint16_t *__restrict__ out) {
-    constexpr uint32_t kRowElems = kGroup + 8;      // +16 B per row: 16-row fragments spread over the banks
-    __shared__ __align__(16) uint16_t xs[kBM][kRowElems];
-    __shared__ __align__(16) uint4 wb[kTilesPerBlock][2][2][kWave];   // [tile][stream][k-half][lane]
-    __shared__ uint32_t s_src[kBM];
+constexpr int kMbPerWave = kBM / 16 / 4;
 
-    if (blockIdx.y >= plan->n_tiles) return;
-    const PrefillTile tile = tiles[blockIdx.y];
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t j = lane & 15, jq = lane >> 4;
-    const uint32_t n_groups = GATE_UP ? g.gd : g.gf;
-    const uint32_t n_arena_tiles = GATE_UP ? g.gu_rb : g.dn_rbp;
-    const uint32_t at = blockIdx.x * kTilesPerBlock + wave;            // this wave's arena tile row
-    const bool at_ok = at < n_arena_tiles;
-    const uint8_t *expert_base = arena_layer + (size_t)tile.expert * g.expert_bytes;
-    const uint8_t *w_tiles = expert_base + (GATE_UP ? g.gu_tiles_off : g.dn_tiles_off) + (size_t)at * n_groups * kTileBytes;
-    const uint8_t *w_scales = expert_base + (GATE_UP ? g.gu_scales_off : g.dn_scales_off) + (size_t)at * n_groups * kTileScaleBytes;
+struct GemmWave {
+    const uint8_t *w_tiles, *w_scales;    // this wave's arena tile row
+    const uint16_t *a;                    // A matrix
+    uint32_t a_stride, n_groups, n_arena_tiles, nb, wave, lane;
+    PrefillTile tile;
+};
 
-    // source row of every pair of the tile: a token row of x, or the pair's own activation row
-    if (tid < (uint32_t)kBM) {
-        const uint32_t row = tile.row_start + min(tid, tile.rows - 1);
-        s_src[tid] = GATE_UP ? sorted_token[row] : row;
+// The k-loop and epilogue of one wave that owns NMB 16-row blocks (a compile-time count: the MFMA
+// sequence has no branches, so the scheduler can interleave it with the expansion of the next tile).
+template <bool GATE_UP, int NMB>
+__device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g, uint4 (*wb)[kTilesPerBlock][2][2][kWave],
+                                          const uint32_t *__restrict__ sorted_token,
+                                          const uint32_t *__restrict__ sorted_out_row, uint16_t *__restrict__ out) {
+    constexpr int NA = NMB > 0 ? NMB : 1;
+    const uint32_t lane = gw.lane, wave = gw.wave, j = lane & 15, jq = lane >> 4;
+    const uint32_t n_groups = gw.n_groups;
+    const uint16_t *arow[NA];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        const uint32_t prow = min((wave + 4 * i) * 16 + j, gw.tile.rows - 1);
+        const uint32_t src = GATE_UP ? sorted_token[gw.tile.row_start + prow] : gw.tile.row_start + prow;
+        arow[i] = gw.a + (size_t)src * gw.a_stride + 8 * jq;
     }
-    __syncthreads();
+    f32x4 acc[NA][2 * kTilesPerBlock];
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+#pragma unroll
+        for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) acc[i][nf] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    f32x4 acc[2][2 * kTilesPerBlock];
+    uint4 wraw = {0, 0, 0, 0};
+    uint2 sraw = {0, 0};
+    auto load_b = [&](uint32_t grp) {
+        wraw = reinterpret_cast<const uint4 *>(gw.w_tiles + (size_t)grp * kTileBytes)[lane];
+        sraw = reinterpret_cast<const uint2 *>(gw.w_scales + (size_t)grp * kTileScaleBytes)[j];
+    };
+    auto expand_b = [&](int buf) {
+        const float s0 = bf16lo_to_f32(sraw.x), b0 = bf16hi_to_f32(sraw.x);
+        const float s1 = bf16lo_to_f32(sraw.y), b1 = bf16hi_to_f32(sraw.y);
+        wb[buf][wave][0][0][lane] = dequant8_bf16(wraw.x, s0, b0);
+        wb[buf][wave][0][1][lane] = dequant8_bf16(wraw.y, s0, b0);
+        wb[buf][wave][1][0][lane] = dequant8_bf16(wraw.z, s1, b1);
+        wb[buf][wave][1][1][lane] = dequant8_bf16(wraw.w, s1, b1);
+    };
+    auto load_a = [&](uint32_t grp, uint4 (&dst)[NA][2]) {
+        if (NMB == 0) return;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) acc[mb][nf] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    for (uint32_t grp = 0; grp < n_groups; ++grp) {
-        // A: 128 rows x 64 k = 1024 16-byte chunks, four per thread
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint32_t i = tid + 256 * c, row = i >> 3, ch = i & 7;
-            const uint4 v = *reinterpret_cast<const uint4 *>(a + (size_t)s_src[row] * a_stride + grp * kGroup + ch * 8);
-            *reinterpret_cast<uint4 *>(&xs[row][ch * 8]) = v;
+        for (int i = 0; i < NA; ++i) {
+            dst[i][0] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup);
+            dst[i][1] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup + 32);
         }
-        // B: one arena tile per wave, expanded to bf16 in MFMA operand order
-        uint4 wt = {0, 0, 0, 0};
-        uint2 sc = {0, 0};
-        if (at_ok) {
-            wt = reinterpret_cast<const uint4 *>(w_tiles + (size_t)grp * kTileBytes)[lane];
-            sc = reinterpret_cast<const uint2 *>(w_scales + (size_t)grp * kTileScaleBytes)[j];
-        }
-        wb[wave][0][0][lane] = dequant8_bf16(wt.x, bf16lo_to_f32(sc.x), bf16hi_to_f32(sc.x));
-        wb[wave][0][1][lane] = dequant8_bf16(wt.y, bf16lo_to_f32(sc.x), bf16hi_to_f32(sc.x));
-        wb[wave][1][0][lane] = dequant8_bf16(wt.z, bf16lo_to_f32(sc.y), bf16hi_to_f32(sc.y));
-        wb[wave][1][1][lane] = dequant8_bf16(wt.w, bf16lo_to_f32(sc.y), bf16hi_to_f32(sc.y));
-        __syncthreads();
-        bf16x8 af[2][2];
+    };
+    // one 64-wide group: fetch A of the next group, expand B of the next group, multiply the current one
+    auto step = [&](uint32_t grp, uint4 (&a_use)[NA][2], uint4 (&a_next)[NA][2]) {
+        // Past the last group the same loads and expansion run once more on clamped indices and are never
+        // used: with no branch around them the compiler counts the loads in flight exactly and lets the
+        // prefetch stay outstanding while the matrix unit works.
+        const int buf = grp & 1;
+        load_a(min(grp + 1, n_groups - 1), a_next);
+        __builtin_amdgcn_sched_barrier(0);      // keep the A loads at the top of the step: a full step of latency
+        expand_b(buf ^ 1);
+        load_b(min(grp + 2, n_groups - 1));
+        if (NMB > 0) {
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+            for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) {
+                const bf16x8 b0 = __builtin_bit_cast(bf16x8, wb[buf][nf >> 1][nf & 1][0][lane]);
+                const bf16x8 b1 = __builtin_bit_cast(bf16x8, wb[buf][nf >> 1][nf & 1][1][lane]);
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
-                af[mb][h] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(&xs[32 * wave + 16 * mb + j][32 * h + 8 * jq]));
-#pragma unroll
-        for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) {
-            const bf16x8 b0 = __builtin_bit_cast(bf16x8, wb[nf >> 1][nf & 1][0][lane]);
-            const bf16x8 b1 = __builtin_bit_cast(bf16x8, wb[nf >> 1][nf & 1][1][lane]);
-#pragma unroll
-            for (int mb = 0; mb < 2; ++mb) {
-                acc[mb][nf] = mfma16(af[mb][0], b0, acc[mb][nf]);
-                acc[mb][nf] = mfma16(af[mb][1], b1, acc[mb][nf]);
-            }
-        }
-        __syncthreads();
-    }
-
-    // epilogue: lane holds pairs 32 w + 16 mb + 4 jq + r, weight row j of every fragment
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t prow = 32 * wave + 16 * mb + 4 * jq + r;
-            if (prow >= tile.rows) continue;
-            const uint32_t pair = tile.row_start + prow;
-#pragma unroll
-            for (int tl = 0; tl < kTilesPerBlock; ++tl) {
-                const uint32_t atl = blockIdx.x * kTilesPerBlock + tl;
-                if (atl >= n_arena_tiles) continue;
-                if (GATE_UP) {
-                    const uint32_t f = atl * kTileRows + j;
-                    out[(size_t)pair * g.f + f] = f32_to_bf16(gelu_tanh(acc[mb][2 * tl][r]) * acc[mb][2 * tl + 1][r]);
-                } else {
-                    const size_t base = (size_t)sorted_out_row[pair] * g.d + (size_t)atl * 2 * kTileRows + j;
-                    out[base] = f32_to_bf16(acc[mb][2 * tl][r]);
-                    out[base + kTileRows] = f32_to_bf16(acc[mb][2 * tl + 1][r]);
+                for (int i = 0; i < NA; ++i) {
+                    acc[i][nf] = mfma16(__builtin_bit_cast(bf16x8, a_use[i][0]), b0, acc[i][nf]);
+                    acc[i][nf] = mfma16(__builtin_bit_cast(bf16x8, a_use[i][1]), b1, acc[i][nf]);
                 }
             }
         }
+        __builtin_amdgcn_sched_barrier(0);      // nothing of the next step may start before the barrier
+        lds_barrier();
+    };
+
+    uint4 a0[NA][2], a1[NA][2];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) a0[i][0] = a0[i][1] = a1[i][0] = a1[i][1] = uint4{0, 0, 0, 0};
+    load_b(0);
+    load_a(0, a0);
+    expand_b(0);
+    load_b(min(1u, n_groups - 1));
+    lds_barrier();
+    uint32_t grp = 0;
+    for (; grp + 1 < n_groups; grp += 2) {
+        step(grp, a0, a1);
+        step(grp + 1, a1, a0);
+    }
+    if (grp < n_groups) step(grp, a0, a1);
+    if (NMB == 0) return;
+
+    // epilogue: lane holds pairs 16 (w + 4 i) + 4 jq + r, weight row j of every fragment
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t prow = (wave + 4 * i) * 16 + 4 * jq + r;
+            if (prow >= gw.tile.rows) continue;
+            const uint32_t pair = gw.tile.row_start + prow;
+            const size_t dn_base = GATE_UP ? 0 : (size_t)sorted_out_row[pair] * g.d;
+#pragma unroll
+            for (int tl = 0; tl < kTilesPerBlock; ++tl) {
+                const uint32_t atl = gw.nb * kTilesPerBlock + tl;
+                if (atl >= gw.n_arena_tiles) continue;
+                if (GATE_UP) {
+                    const uint32_t f = atl * kTileRows + j;
+                    out[(size_t)pair * g.f + f] = f32_to_bf16(gelu_tanh_fast(acc[i][2 * tl][r]) * acc[i][2 * tl + 1][r]);
+                } else {
+                    const size_t base = dn_base + (size_t)atl * 2 * kTileRows + j;
+                    out[base] = f32_to_bf16(acc[i][2 * tl][r]);
+                    out[base + kTileRows] = f32_to_bf16(acc[i][2 * tl + 1][r]);
+                }
+            }
+        }
+    }
+}
+
+template <bool GATE_UP>
+__global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                              const PrefillPlan *__restrict__ plan,
+                                                              const PrefillTile *__restrict__ tiles,
+                                                              const uint32_t *__restrict__ sorted_token,
+                                                              const uint32_t *__restrict__ sorted_out_row,
+                                                              const uint16_t *__restrict__ a, uint32_t a_stride,
+                                                              uint16_t *__restrict__ out, uint32_t n_nblocks) {
+    __shared__ __align__(16) uint4 wb[2][kTilesPerBlock][2][2][kWave];   // [buffer][tile][stream][k-half][lane]
+
+    const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const uint32_t ti = (slot / n_nblocks) * 8 + xcd, nb = slot % n_nblocks;
+    if (ti >= plan->n_tiles) return;
+    GemmWave gw;
+    gw.tile = tiles[ti];
+    gw.lane = threadIdx.x & 63;
+    gw.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // wave-uniform: branches on it stay scalar
+    gw.n_groups = GATE_UP ? g.gd : g.gf;
+    gw.n_arena_tiles = GATE_UP ? g.gu_rb : g.dn_rbp;
+    gw.nb = nb;
+    gw.a = a;
+    gw.a_stride = a_stride;
+    // the arena tile row this wave expands; past the last one it expands the last again (never stored)
+    const uint32_t at = min(nb * kTilesPerBlock + gw.wave, gw.n_arena_tiles - 1);
+    const uint8_t *expert_base = arena_layer + (size_t)gw.tile.expert * g.expert_bytes;
+    gw.w_tiles = expert_base + (GATE_UP ? g.gu_tiles_off : g.dn_tiles_off) + (size_t)at * gw.n_groups * kTileBytes;
+    gw.w_scales = expert_base + (GATE_UP ? g.gu_scales_off : g.dn_scales_off) + (size_t)at * gw.n_groups * kTileScaleBytes;
+
+    const uint32_t n_mb = (gw.tile.rows + 15) / 16;
+    const uint32_t my_mb = n_mb > gw.wave ? (n_mb - gw.wave + 3) / 4 : 0;    // 16-row blocks of this wave
+    switch (my_mb) {
+        case 0: gemm_wave<GATE_UP, 0>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        case 1: gemm_wave<GATE_UP, 1>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        case 2: gemm_wave<GATE_UP, 2>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        case 3: gemm_wave<GATE_UP, 3>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        default: gemm_wave<GATE_UP, 4>(gw, g, wb, sorted_token, sorted_out_row, out); break;
     }
 }
 
@@ -313,13 +377,14 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_PREFILL_SORT);
     const uint32_t tile_cap = min(sc.max_tiles, (src.n_items + kBM - 1) / kBM + n_experts);
-    hipLaunchKernelGGL(prefill_gemm_kernel<true>, dim3((g.gu_rb + kTilesPerBlock - 1) / kTilesPerBlock, tile_cap), dim3(256),
-                       0, s, arena_layer, g, sc.plan, sc.tiles, sc.sorted_token, sc.sorted_out_row, x, x_stride, sc.acts);
+    const uint32_t tile_slots = (tile_cap + 7) / 8 * 8;
+    const uint32_t nb_gu = (g.gu_rb + kTilesPerBlock - 1) / kTilesPerBlock, nb_dn = (g.dn_rbp + kTilesPerBlock - 1) / kTilesPerBlock;
+    hipLaunchKernelGGL(prefill_gemm_kernel<true>, dim3(nb_gu * tile_slots), dim3(256), 0, s, arena_layer, g, sc.plan,
+                       sc.tiles, sc.sorted_token, sc.sorted_out_row, x, x_stride, sc.acts, nb_gu);
     timer->mark(s, FFMOE_K_PREFILL_GATE_UP);
     uint16_t *partials = partials_out ? partials_out : sc.partials;
-    hipLaunchKernelGGL(prefill_gemm_kernel<false>, dim3((g.dn_rbp + kTilesPerBlock - 1) / kTilesPerBlock, tile_cap),
-                       dim3(256), 0, s, arena_layer, g, sc.plan, sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f,
-                       partials);
+    hipLaunchKernelGGL(prefill_gemm_kernel<false>, dim3(nb_dn * tile_slots), dim3(256), 0, s, arena_layer, g, sc.plan,
+                       sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_PREFILL_DOWN);

@@ -18,6 +18,7 @@ OK = 0
 GATE, UP, DOWN = 0, 1, 2
 GROUP = 64
 MAX_VERIFY_ROWS = 16
+PREFILL_TILE_M = 256      # FFMOE_PREFILL_TILE_M
 
 
 class FieldfareError(RuntimeError):

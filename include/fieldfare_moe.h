@@ -41,6 +41,8 @@ enum { FFMOE_GATE = 0, FFMOE_UP = 1, FFMOE_DOWN = 2 };
 #define FFMOE_GROUP 64          /* Quantization.groupSize, Infrastructure/ModelIO/Quantization.swift:2 */
 #define FFMOE_MAX_VERIFY_ROWS 16 /* maxVerifyTokens, Runtime/Inference/RealForwardRunner.swift:414 */
 #define FFMOE_MAX_EXPERTS 256    /* router limit, Kernels/MoE/MoE.swift:137 */
+#define FFMOE_PREFILL_TILE_M 256 /* pairs per M-tile of the prefill GEMMs (the role of groupTokenExpertPairs' tileM,
+                                    Kernels/Prefill/MoE/PrefillMoEGrouping.swift:49); ffmoe_prefill_plan_stats counts these */
 
 typedef struct ffmoe_ctx ffmoe_ctx;
 

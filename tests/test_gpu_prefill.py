@@ -25,7 +25,7 @@ def ff():
 def small(oracle, ff, torch):
     d, f, e = 128, 64, 16
     rng, pool, router = make_layer(oracle, 23, d, f, e, align=1)
-    ctx = ff.Context(d, f, e, 8, n_layers=1, max_tokens=512)
+    ctx = ff.Context(d, f, e, 8, n_layers=1, max_tokens=1024)
     ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
     ctx.upload_router_bf16(0, router)
     yield dict(rng=rng, pool=pool, router=router, ctx=ctx, d=d, f=f, e=e)
@@ -47,8 +47,8 @@ def _pairs_tensor(torch, pairs):
     return torch.from_numpy(raw.view(np.int32)).cuda()
 
 
-@pytest.mark.parametrize("t", [1, 7, 40, 300])
-def test_prefill_small_shape_against_oracle(small, oracle, torch, t):
+@pytest.mark.parametrize("t", [1, 7, 40, 300, 700])
+def test_prefill_small_shape_against_oracle(small, oracle, ff, torch, t):
     rng = np.random.default_rng(200 + t)
     xb = oracle.bf16_bits(rng.normal(0, 1, (t, small["d"])).astype(np.float32))
     x = bf16_tensor(torch, xb)
@@ -61,7 +61,8 @@ def test_prefill_small_shape_against_oracle(small, oracle, torch, t):
     n_pairs, n_tiles, counts = small["ctx"].prefill_stats()
     assert n_pairs == t * 8
     assert np.array_equal(counts, np.bincount(idx_np.ravel(), minlength=small["e"]))
-    assert n_tiles == int(np.sum((counts + 127) // 128))
+    tm = ff.PREFILL_TILE_M
+    assert n_tiles == int(np.sum((counts + tm - 1) // tm))
 
 
 def test_prefill_matches_mirror_rounding(small, oracle, torch):
@@ -133,9 +134,9 @@ def test_prefill_token_permutation_is_bit_exact(small, oracle, torch):
     assert np.array_equal(yp, y[perm])
 
 
-def test_prefill_edge_routes(small, oracle, torch):
+def test_prefill_edge_routes(small, oracle, ff, torch):
     # every token to the same experts (several M-tiles per expert), zero weights dropped, bad indices ignored
-    t, d = 300, small["d"]
+    t, d = 600, small["d"]
     rng = np.random.default_rng(8)
     xb = oracle.bf16_bits(rng.normal(0, 1, (t, d)).astype(np.float32))
     x = bf16_tensor(torch, xb)
@@ -154,7 +155,8 @@ def test_prefill_edge_routes(small, oracle, torch):
     assert rel_err(got, ref) <= 1e-2 and cosine(got, ref) >= 0.9999
     n_pairs, n_tiles, counts = small["ctx"].prefill_stats()
     assert n_pairs == t * 8 - t // 2 - len(range(1, t, 3))
-    assert counts[3] == t and n_tiles >= 3 * 7
+    tm = ff.PREFILL_TILE_M
+    assert counts[3] == t and n_tiles == int(np.sum((counts + tm - 1) // tm)) and n_tiles >= 3 * 6
     # all weights zero: nothing runs, the output is exactly zero
     z = small["ctx"].prefill(0, x, torch.from_numpy(idx_np.view(np.int32)).cuda(),
                              torch.zeros((t, 8), dtype=torch.bfloat16, device="cuda"))
