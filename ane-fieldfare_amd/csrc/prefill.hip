@@ -180,10 +180,22 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     const uint16_t *arow[NA];
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-        const uint32_t prow = min((wave + 4 * i) * 16 + j, gw.tile.rows - 1);
+        // load layout: four neighbouring lanes read 64 contiguous bytes of one row (row lane / 4, 8-element
+        // chunk lane % 4), so a load touches 16 half-lines instead of 64 scattered 16-byte pieces
+        const uint32_t prow = min((wave + 4 * i) * 16 + (lane >> 2), gw.tile.rows - 1);
         const uint32_t src = GATE_UP ? sorted_token[gw.tile.row_start + prow] : gw.tile.row_start + prow;
-        arow[i] = gw.a + (size_t)src * gw.a_stride + 8 * jq;
+        arow[i] = gw.a + (size_t)src * gw.a_stride + 8 * (lane & 3);
     }
+    // MFMA layout: lane (j, jq) needs row j, chunk jq = what load-layout lane 4 j + jq holds
+    const int pull = (int)((4 * j + jq) * 4);
+    auto to_frag = [&](const uint4 &v) {
+        uint4 r;
+        r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x);
+        r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y);
+        r.z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z);
+        r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w);
+        return __builtin_bit_cast(bf16x8, r);
+    };
     f32x4 acc[NA][2 * kTilesPerBlock];
 #pragma unroll
     for (int i = 0; i < NA; ++i)
@@ -204,54 +216,69 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
         wb[buf][wave][1][0][lane] = dequant8_bf16(wraw.z, s1, b1);
         wb[buf][wave][1][1][lane] = dequant8_bf16(wraw.w, s1, b1);
     };
-    auto load_a = [&](uint32_t grp, uint4 (&dst)[NA][2]) {
+    uint4 araw[NA][2];      // A of the next group in load layout (in flight during the step)
+    bf16x8 af[NA][2];       // A of the current group as MFMA fragments
+    auto load_a = [&](uint32_t grp) {
         if (NMB == 0) return;
 #pragma unroll
         for (int i = 0; i < NA; ++i) {
-            dst[i][0] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup);
-            dst[i][1] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup + 32);
+            araw[i][0] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup);
+            araw[i][1] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup + 32);
         }
     };
-    // one 64-wide group: fetch A of the next group, expand B of the next group, multiply the current one
-    auto step = [&](uint32_t grp, uint4 (&a_use)[NA][2], uint4 (&a_next)[NA][2]) {
-        // Past the last group the same loads and expansion run once more on clamped indices and are never
-        // used: with no branch around them the compiler counts the loads in flight exactly and lets the
-        // prefetch stay outstanding while the matrix unit works.
+    auto frag_a = [&]() {
+        if (NMB == 0) return;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            af[i][0] = to_frag(araw[i][0]);
+            af[i][1] = to_frag(araw[i][1]);
+        }
+    };
+    // One 64-wide group. On entry: af = fragments of this group, araw = loads of the next group in flight,
+    // wraw/sraw = this wave's packed tile of the next group in flight, wb[buf] = expanded tiles of this group.
+    // The step expands the next tiles into wb[buf ^ 1] between the MFMAs, then turns araw into the next
+    // fragments (its loads have had the whole step to land) and issues the loads of the group after.
+    // Past the last group the same loads and expansion run once more on clamped indices and are never used:
+    // with no branch around them the compiler counts the loads in flight exactly.
+    auto step = [&](uint32_t grp) {
         const int buf = grp & 1;
-        load_a(min(grp + 1, n_groups - 1), a_next);
-        __builtin_amdgcn_sched_barrier(0);      // keep the A loads at the top of the step: a full step of latency
         expand_b(buf ^ 1);
         load_b(min(grp + 2, n_groups - 1));
         if (NMB > 0) {
+            // B fragments are read one fragment pair ahead of the MFMAs that use them
+            uint4 bq[2][2];
+            bq[0][0] = wb[buf][0][0][0][lane];
+            bq[0][1] = wb[buf][0][0][1][lane];
 #pragma unroll
             for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) {
-                const bf16x8 b0 = __builtin_bit_cast(bf16x8, wb[buf][nf >> 1][nf & 1][0][lane]);
-                const bf16x8 b1 = __builtin_bit_cast(bf16x8, wb[buf][nf >> 1][nf & 1][1][lane]);
+                if (nf + 1 < 2 * kTilesPerBlock) {
+                    bq[(nf + 1) & 1][0] = wb[buf][(nf + 1) >> 1][(nf + 1) & 1][0][lane];
+                    bq[(nf + 1) & 1][1] = wb[buf][(nf + 1) >> 1][(nf + 1) & 1][1][lane];
+                }
+                const bf16x8 b0 = __builtin_bit_cast(bf16x8, bq[nf & 1][0]);
+                const bf16x8 b1 = __builtin_bit_cast(bf16x8, bq[nf & 1][1]);
 #pragma unroll
                 for (int i = 0; i < NA; ++i) {
-                    acc[i][nf] = mfma16(__builtin_bit_cast(bf16x8, a_use[i][0]), b0, acc[i][nf]);
-                    acc[i][nf] = mfma16(__builtin_bit_cast(bf16x8, a_use[i][1]), b1, acc[i][nf]);
+                    acc[i][nf] = mfma16(af[i][0], b0, acc[i][nf]);
+                    acc[i][nf] = mfma16(af[i][1], b1, acc[i][nf]);
                 }
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        frag_a();
+        load_a(min(grp + 2, n_groups - 1));
         __builtin_amdgcn_sched_barrier(0);      // nothing of the next step may start before the barrier
         lds_barrier();
     };
 
-    uint4 a0[NA][2], a1[NA][2];
-#pragma unroll
-    for (int i = 0; i < NA; ++i) a0[i][0] = a0[i][1] = a1[i][0] = a1[i][1] = uint4{0, 0, 0, 0};
     load_b(0);
-    load_a(0, a0);
+    load_a(0);
     expand_b(0);
     load_b(min(1u, n_groups - 1));
+    frag_a();
+    load_a(min(1u, n_groups - 1));
     lds_barrier();
-    uint32_t grp = 0;
-    for (; grp + 1 < n_groups; grp += 2) {
-        step(grp, a0, a1);
-        step(grp + 1, a1, a0);
-    }
-    if (grp < n_groups) step(grp, a0, a1);
+    for (uint32_t grp = 0; grp < n_groups; ++grp) step(grp);
     if (NMB == 0) return;
 
     // epilogue: lane holds pairs 16 (w + 4 i) + 4 jq + r, weight row j of every fragment
