@@ -259,8 +259,10 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
                 const bf16x8 b1 = __builtin_bit_cast(bf16x8, bq[nf & 1][1]);
 #pragma unroll
                 for (int i = 0; i < NA; ++i) {
-                    acc[i][nf] = mfma16(af[i][0], b0, acc[i][nf]);
-                    acc[i][nf] = mfma16(af[i][1], b1, acc[i][nf]);
+                    // weights as the first operand: the lane ends up with four consecutive weight rows of
+                    // one pair, which the epilogue stores as one 8-byte piece of that pair's output row
+                    acc[i][nf] = mfma16(b0, af[i][0], acc[i][nf]);
+                    acc[i][nf] = mfma16(b1, af[i][1], acc[i][nf]);
                 }
             }
         }
@@ -281,26 +283,28 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     for (uint32_t grp = 0; grp < n_groups; ++grp) step(grp);
     if (NMB == 0) return;
 
-    // epilogue: lane holds pairs 16 (w + 4 i) + 4 jq + r, weight row j of every fragment
+    // epilogue: lane (j, jq) holds pair 16 (w + 4 i) + j, weight rows 4 jq .. 4 jq + 3 of every fragment
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
+        const uint32_t prow = (wave + 4 * i) * 16 + j;
+        if (prow >= gw.tile.rows) continue;
+        const uint32_t pair = gw.tile.row_start + prow;
+        uint16_t *orow = GATE_UP ? out + (size_t)pair * g.f : out + (size_t)sorted_out_row[pair] * g.d;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t prow = (wave + 4 * i) * 16 + 4 * jq + r;
-            if (prow >= gw.tile.rows) continue;
-            const uint32_t pair = gw.tile.row_start + prow;
-            const size_t dn_base = GATE_UP ? 0 : (size_t)sorted_out_row[pair] * g.d;
+        for (int tl = 0; tl < kTilesPerBlock; ++tl) {
+            const uint32_t atl = gw.nb * kTilesPerBlock + tl;
+            if (atl >= gw.n_arena_tiles) continue;
+            if (GATE_UP) {
+                float h[4];
 #pragma unroll
-            for (int tl = 0; tl < kTilesPerBlock; ++tl) {
-                const uint32_t atl = gw.nb * kTilesPerBlock + tl;
-                if (atl >= gw.n_arena_tiles) continue;
-                if (GATE_UP) {
-                    const uint32_t f = atl * kTileRows + j;
-                    out[(size_t)pair * g.f + f] = f32_to_bf16(gelu_tanh_fast(acc[i][2 * tl][r]) * acc[i][2 * tl + 1][r]);
-                } else {
-                    const size_t base = dn_base + (size_t)atl * 2 * kTileRows + j;
-                    out[base] = f32_to_bf16(acc[i][2 * tl][r]);
-                    out[base + kTileRows] = f32_to_bf16(acc[i][2 * tl + 1][r]);
+                for (int r = 0; r < 4; ++r) h[r] = gelu_tanh_fast(acc[i][2 * tl][r]) * acc[i][2 * tl + 1][r];
+                *reinterpret_cast<uint2 *>(orow + atl * kTileRows + 4 * jq) = make_uint2(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]));
+            } else {
+#pragma unroll
+                for (int sdx = 0; sdx < 2; ++sdx) {
+                    const f32x4 v = acc[i][2 * tl + sdx];
+                    *reinterpret_cast<uint2 *>(orow + atl * 2 * kTileRows + sdx * kTileRows + 4 * jq) =
+                        make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
                 }
             }
         }
