@@ -24,6 +24,7 @@ struct ffmoe_layer {
 
 struct ffmoe_ctx {
     int device = 0;
+    uint32_t n_cus = 0;       // compute units: sizes the persistent grids
     ffmoe_shape shape{};
     ArenaGeom geom{};
     uint8_t *arena = nullptr;
@@ -110,6 +111,11 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     ffmoe_ctx *ctx = new (std::nothrow) ffmoe_ctx();
     if (!ctx) return fail(err, FFMOE_ERR_ALLOC, "out of host memory");
     ctx->device = device;
+    {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
+        ctx->n_cus = (uint32_t)cus;
+    }
     ctx->shape = *shape;
     ctx->geom = make_geom(shape->d, shape->f);
     ctx->layer_bytes = (size_t)shape->n_experts * ctx->geom.expert_bytes;
@@ -299,7 +305,7 @@ static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uin
         return fail(err, FFMOE_ERR_INVALID, "y and residual must be 8-byte aligned");
     FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                         ctx->plan, ctx->acts, ctx->partials, &ctx->timer));
+                         ctx->plan, ctx->acts, ctx->partials, ctx->n_cus, &ctx->timer));
     return FFMOE_OK;
 }
 

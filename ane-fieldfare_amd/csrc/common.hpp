@@ -55,12 +55,18 @@ __device__ __forceinline__ float gelu_tanh_fast(float x) {
 //
 // unpack8_offset128: the eight nibbles as bf16 values 128 + q (0x4300 | q is exact: the bf16 ulp at
 // 128 is 1). The matrix unit then accumulates sum (128 + q) x; the caller removes 128 * sum x.
+// One v_and_or_b32 per pair: gfx9 VOP3 takes no literals and one scalar operand, so the mask has to sit in a
+// scalar register and the constant in a vector register. The empty asm statements only hide the two
+// values' constness, which makes the compiler itself select v_and_or_b32 (it otherwise emits and + or).
 __device__ __forceinline__ bf16x8 unpack8_offset128(uint32_t w) {
+    uint32_t mask = 0x000F000Fu, c = 0x43004300u;
+    asm("" : "+s"(mask));
+    asm("" : "+v"(c));
     uint4 r;
-    r.x = (w & 0x000F000Fu) | 0x43004300u;
-    r.y = ((w >> 4) & 0x000F000Fu) | 0x43004300u;
-    r.z = ((w >> 8) & 0x000F000Fu) | 0x43004300u;
-    r.w = ((w >> 12) & 0x000F000Fu) | 0x43004300u;
+    r.x = (w & mask) | c;
+    r.y = ((w >> 4) & mask) | c;
+    r.z = ((w >> 8) & mask) | c;
+    r.w = ((w >> 12) & mask) | c;
     return __builtin_bit_cast(bf16x8, r);
 }
 

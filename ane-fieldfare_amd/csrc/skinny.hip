@@ -197,7 +197,7 @@ __global__ __launch_bounds__(256) void skinny_gate_up_kernel(const uint8_t *__re
     for (int r = 0; r < 4; ++r) {
         const uint32_t ts = 4 * jq + r;
         // one rounding to 16 bits, gate and up themselves stay fp32 (moe.metal:496)
-        if (ts < n) acts[(size_t)slot.routes[ts] * g.f + row] = f32_to_bf16(gelu_tanh(tot.a[r]) * tot.b[r]);
+        if (ts < n) acts[(size_t)slot.routes[ts] * g.f + row] = f32_to_bf16(gelu_tanh_fast(tot.a[r]) * tot.b[r]);
     }
 }
 
@@ -234,6 +234,226 @@ __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restr
             } else {
                 partials_f32[base + row_a] = tot.a[r];
                 partials_f32[base + row_b] = tot.b[r];
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Persistent forms of the two kernels above for experts whose K-slice fits the register ring
+// (D <= 4 * 11 * 64 and F <= 11 * 64, which covers the reference model). The grid is sized to what the
+// chip holds at once; every wave keeps its token operand in registers and walks several row blocks with
+// the weight ring refilled across row-block boundaries, so from its first instruction to its last a wave
+// has one full K-slice (about 12 KiB) of weights in flight and never pays the load latency again.
+// Groups past the end of a short K-slice are read from the last valid tile and enter with zero scales.
+// ---------------------------------------------------------------------------------------------------
+struct WeightRing {
+    uint4 t[kRing];
+    uint2 s[kRing];
+};
+
+// `tiles` / `scales` are wave-uniform (scalar registers); the lane part is a 32-bit offset, so every ring load is
+// one instruction with a scalar base and no per-load 64-bit address arithmetic.
+__device__ __forceinline__ void ring_fill(WeightRing &ring, int u, const uint8_t *tiles, const uint8_t *scales,
+                                          uint32_t g_clamped, uint32_t lane) {
+    const uint8_t *tg = tiles + (size_t)g_clamped * kTileBytes, *sg = scales + (size_t)g_clamped * kTileScaleBytes;
+    ring.t[u] = *reinterpret_cast<const uint4 *>(tg + lane * 16u);
+    ring.s[u] = *reinterpret_cast<const uint2 *>(sg + (lane & 15u) * 8u);
+}
+
+// Consume ring slot u against the resident token operand, then start the load that refills the slot.
+__device__ __forceinline__ void ring_step(WeightRing &ring, int u, bool live, const uint4 &x0, const uint4 &x1,
+                                          TwoStreamAcc &tot, const uint8_t *next_tiles, const uint8_t *next_scales,
+                                          uint32_t next_g, uint32_t lane) {
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    const uint4 ones_bits = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+    const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
+    const uint4 tile = ring.t[u];
+    uint2 sc = ring.s[u];
+    if (!live) sc = make_uint2(0u, 0u);
+    ring_fill(ring, u, next_tiles, next_scales, next_g, lane);
+    const bf16x8 a0 = __builtin_bit_cast(bf16x8, x0), a1 = __builtin_bit_cast(bf16x8, x1);
+    f32x4 acc_a = mfma16(a0, unpack8_offset128(tile.x), zero);
+    acc_a = mfma16(a1, unpack8_offset128(tile.y), acc_a);
+    f32x4 acc_b = mfma16(a0, unpack8_offset128(tile.z), zero);
+    acc_b = mfma16(a1, unpack8_offset128(tile.w), acc_b);
+    f32x4 sx = mfma16(a0, ones, zero);
+    sx = mfma16(a1, ones, sx);
+    const float sa = bf16lo_to_f32(sc.x), ba = bf16hi_to_f32(sc.x);
+    const float sb = bf16lo_to_f32(sc.y), bb = bf16hi_to_f32(sc.y);
+    const float ta = __builtin_fmaf(-128.0f, sa, ba), tb = __builtin_fmaf(-128.0f, sb, bb);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        tot.a[r] = __builtin_fmaf(sa, acc_a[r], tot.a[r]);
+        tot.a[r] = __builtin_fmaf(ta, sx[r], tot.a[r]);
+        tot.b[r] = __builtin_fmaf(sb, acc_b[r], tot.b[r]);
+        tot.b[r] = __builtin_fmaf(tb, sx[r], tot.b[r]);
+    }
+}
+
+// Split `n_items` of one expert over `parts` workers: worker `sub` gets [first, last).
+__device__ __forceinline__ void split_range(uint32_t n_items, uint32_t parts, uint32_t sub, uint32_t &first,
+                                            uint32_t &last) {
+    first = (uint32_t)((uint64_t)sub * n_items / parts);
+    last = (uint32_t)((uint64_t)(sub + 1) * n_items / parts);
+}
+
+// gate/up + GELU-tanh gating, persistent. grid = (blocks); the blocks are dealt to the live experts, each
+// block walks a range of 16-row blocks of its expert; its four waves split K and meet in LDS per row block
+// (partials added in wave order), each wave finishing a quarter of the token slots.
+__global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                                    uint32_t top_k, const VerifyPlan *__restrict__ plan,
+                                                                    const uint16_t *__restrict__ x, uint32_t x_stride,
+                                                                    uint16_t *__restrict__ acts) {
+    __shared__ float s_red[2][kKSplit][8][64];
+    const uint32_t n_live = plan->n_live;
+    if (n_live == 0) return;
+    const uint32_t blocks_per_slot = max(1u, min(g.gu_rb, gridDim.x / n_live));
+    const uint32_t slot_id = blockIdx.x / blocks_per_slot;
+    if (slot_id >= n_live) return;
+    uint32_t rb0, rb1;
+    split_range(g.gu_rb, blocks_per_slot, blockIdx.x % blocks_per_slot, rb0, rb1);
+    if (rb0 >= rb1) return;
+    const PlanSlot &slot = plan->slots[slot_id];
+    const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
+    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint8_t *expert_base = arena_layer + (size_t)__builtin_amdgcn_readfirstlane(slot.expert) * g.expert_bytes;
+    const uint32_t per = (g.gd + kKSplit - 1) / kKSplit;
+    const uint32_t g0 = min(ks * per, g.gd), g1 = min(g.gd, g0 + per), ng = g1 - g0;
+    const uint32_t g_last = g1 > g0 ? g1 - 1 : g.gd - 1;
+    const uint8_t *tiles = expert_base + g.gu_tiles_off;
+    const uint8_t *scales = expert_base + g.gu_scales_off;
+    const size_t tile_row = (size_t)g.gd * kTileBytes, scale_row = (size_t)g.gd * kTileScaleBytes;
+
+    WeightRing ring;
+#pragma unroll
+    for (int u = 0; u < kRing; ++u)
+        ring_fill(ring, u, tiles + rb0 * tile_row, scales + rb0 * scale_row, min(g0 + u, g_last), lane);
+    // token operand of this wave's K-slice: token slot j (clamped), k-quarter jq of every group
+    const uint32_t tok = slot.routes[min(j, n - 1)] / top_k;
+    const uint16_t *xrow = x + (size_t)tok * x_stride + 8 * jq;
+    uint4 x0[kRing], x1[kRing];
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) {
+        const bool live = (uint32_t)u < ng;
+        const uint32_t gg = min(g0 + u, g_last);
+        x0[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup) : uint4{0, 0, 0, 0};
+        x1[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
+    }
+    const uint32_t my_ts = 4 * jq + ks;     // the token slot this lane finishes
+    const uint32_t my_route = slot.routes[min(my_ts, n - 1)];
+
+    for (uint32_t rb = rb0; rb < rb1; ++rb) {
+        // the refill targets the next row block; past the last one it re-reads the current tiles (cache hits)
+        const uint32_t rbn = min(rb + 1, rb1 - 1);
+        const uint8_t *nt = tiles + rbn * tile_row, *ns = scales + rbn * scale_row;
+        TwoStreamAcc tot;
+        tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
+        tot.b = tot.a;
+#pragma unroll
+        for (int u = 0; u < kRing; ++u)
+            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, nt, ns, min(g0 + u, g_last), lane);
+        const int buf = (rb - rb0) & 1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            s_red[buf][ks][r][lane] = tot.a[r];
+            s_red[buf][ks][4 + r][lane] = tot.b[r];
+        }
+        lds_barrier();
+        float ga = s_red[buf][0][ks][lane], ub = s_red[buf][0][4 + ks][lane];
+#pragma unroll
+        for (int o = 1; o < kKSplit; ++o) {
+            ga += s_red[buf][o][ks][lane];
+            ub += s_red[buf][o][4 + ks][lane];
+        }
+        // one rounding to 16 bits, gate and up themselves stay fp32 (moe.metal:496)
+        if (my_ts < n) acts[(size_t)my_route * g.f + rb * kTileRows + j] = f32_to_bf16(gelu_tanh_fast(ga) * ub);
+    }
+}
+
+// down projection, persistent. grid = (blocks); the blocks are dealt to the live experts. A block stages
+// its expert's (<= 16) activation rows in LDS once (rows padded by 16 bytes so that the 16 rows of a
+// fragment read fall into different banks) and its waves walk disjoint ranges of 32-row blocks. With the
+// token operand in LDS a wave needs few registers, so three blocks fit a CU and the chip keeps most of
+// the layer's down weights in flight at once.
+constexpr int kXsStride = kRing * kGroup + 8;
+
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256, 2) void skinny_down_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                                 const VerifyPlan *__restrict__ plan,
+                                                                 const uint16_t *__restrict__ acts,
+                                                                 float *__restrict__ partials_f32,
+                                                                 uint16_t *__restrict__ partials_bf16) {
+    __shared__ __align__(16) uint16_t xs[kMaxRows][kXsStride];
+    const uint32_t n_live = plan->n_live;
+    if (n_live == 0) return;
+    const uint32_t blocks_per_slot = max(1u, min((g.dn_rbp + 3) / 4, gridDim.x / n_live));
+    const uint32_t slot_id = blockIdx.x / blocks_per_slot;
+    if (slot_id >= n_live) return;
+    uint32_t b0, b1, rb0, rb1;
+    split_range(g.dn_rbp, blocks_per_slot, blockIdx.x % blocks_per_slot, b0, b1);
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    split_range(b1 - b0, 4, wave, rb0, rb1);
+    rb0 += b0;
+    rb1 += b0;
+    const PlanSlot &slot = plan->slots[slot_id];
+    const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint8_t *expert_base = arena_layer + (size_t)__builtin_amdgcn_readfirstlane(slot.expert) * g.expert_bytes;
+    const uint8_t *tiles = expert_base + g.dn_tiles_off;
+    const uint8_t *scales = expert_base + g.dn_scales_off;
+    const size_t tile_row = (size_t)g.gf * kTileBytes, scale_row = (size_t)g.gf * kTileScaleBytes;
+    const uint32_t ng = g.gf, g_last = g.gf - 1;
+    const uint32_t rb_first = min(rb0, g.dn_rbp - 1);       // a wave without row blocks still loads valid memory
+
+    WeightRing ring;
+#pragma unroll
+    for (int u = 0; u < kRing; ++u)
+        ring_fill(ring, u, tiles + rb_first * tile_row, scales + rb_first * scale_row, min((uint32_t)u, g_last), lane);
+    // stage the activation rows while the first tiles are on their way
+    // (columns past F, read by the groups of a short K that enter with zero scales, are cleared)
+    constexpr uint32_t kChunksPerRow = kRing * kGroup / 8;
+    const uint32_t live_chunks = g.f / 8;
+    for (uint32_t i = threadIdx.x; i < n * kChunksPerRow; i += 256) {
+        const uint32_t row = i / kChunksPerRow, c = i % kChunksPerRow;
+        uint4 v = {0, 0, 0, 0};
+        if (c < live_chunks) v = *reinterpret_cast<const uint4 *>(acts + (size_t)slot.routes[row] * g.f + c * 8);
+        *reinterpret_cast<uint4 *>(&xs[row][c * 8]) = v;
+    }
+    lds_barrier();
+    const uint16_t *xrow = &xs[min(j, n - 1)][8 * jq];
+    size_t out_base[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) out_base[r] = (size_t)slot.routes[min(4 * jq + r, n - 1)] * g.d;
+
+    for (uint32_t rb = rb0; rb < rb1; ++rb) {
+        const uint32_t rbn = min(rb + 1, rb1 - 1);
+        const uint8_t *nt = tiles + rbn * tile_row, *ns = scales + rbn * scale_row;
+        TwoStreamAcc tot;
+        tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
+        tot.b = tot.a;
+        // the token operand is re-read from LDS for every row block: the clobber keeps the compiler from
+        // hoisting 22 fragment reads out of the loop into registers it does not have
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) {
+            const uint4 x0 = *reinterpret_cast<const uint4 *>(xrow + u * kGroup);
+            const uint4 x1 = *reinterpret_cast<const uint4 *>(xrow + u * kGroup + 32);
+            ring_step(ring, u, (uint32_t)u < ng, x0, x1, tot, nt, ns, min((uint32_t)u, g_last), lane);
+            if (u & 1) __builtin_amdgcn_sched_barrier(0);   // bound how many groups the scheduler unpacks ahead
+        }
+        const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            if (4 * jq + r < n) {
+                if (OUT_BF16) {
+                    partials_bf16[out_base[r] + row_a] = f32_to_bf16(tot.a[r]);
+                    partials_bf16[out_base[r] + row_b] = f32_to_bf16(tot.b[r]);
+                } else {
+                    partials_f32[out_base[r] + row_a] = tot.a[r];
+                    partials_f32[out_base[r] + row_b] = tot.b[r];
+                }
             }
         }
     }
@@ -291,26 +511,43 @@ __global__ __launch_bounds__(256) void reduce_token_major_kernel(const uint16_t 
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
-                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, KernelTimer *timer) {
+                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer) {
     timer->begin(s);
     hipLaunchKernelGGL(verify_plan_kernel, dim3(1), dim3(256), 0, s, idx, w, t * top_k, n_experts, plan);
     timer->mark(s, FFMOE_K_PLAN);
     const uint32_t slots = min(n_experts, t * top_k);
-    hipLaunchKernelGGL(skinny_gate_up_kernel, dim3(g.gu_rb, slots), dim3(256), 0, s, arena_layer, g, top_k, plan, x,
-                       x_stride, acts);
+    // the persistent kernels hold a K-slice of kRing groups per wave; larger experts take the one-shot grids
+    const bool persistent = (g.gd + kKSplit - 1) / kKSplit <= (uint32_t)kRing && g.gf <= (uint32_t)kRing;
+    const uint32_t resident = 2 * n_cus;       // blocks the chip holds at once (__launch_bounds__(256, 2))
+    if (persistent) {
+        const uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
+        hipLaunchKernelGGL(skinny_gate_up_persistent, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k,
+                           plan, x, x_stride, acts);
+    } else {
+        hipLaunchKernelGGL(skinny_gate_up_kernel, dim3(g.gu_rb, slots), dim3(256), 0, s, arena_layer, g, top_k, plan, x,
+                           x_stride, acts);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_GATE_UP);
-    const dim3 dn_grid((g.dn_rbp + 3) / 4, slots);
+    const bool dn_persistent = false;
+    const dim3 dn_grid = dn_persistent ? dim3(max(slots, min(2 * n_cus, slots * ((g.dn_rbp + 3) / 4))))
+                                       : dim3((g.dn_rbp + 3) / 4, slots);
+#define FFMOE_DOWN(BF)                                                                                          \
+    if (dn_persistent)                                                                                          \
+        hipLaunchKernelGGL(skinny_down_persistent<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,    \
+                           partials_f32, partials_bf16);                                                        \
+    else                                                                                                        \
+        hipLaunchKernelGGL(skinny_down_kernel<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,        \
+                           partials_f32, partials_bf16)
     if (partials_bf16) {
-        hipLaunchKernelGGL(skinny_down_kernel<true>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts, partials_f32,
-                           partials_bf16);
+        FFMOE_DOWN(true);
         timer->mark(s, FFMOE_K_DOWN);
         timer->finish();
         return hipGetLastError();
     }
-    hipLaunchKernelGGL(skinny_down_kernel<false>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts, partials_f32,
-                       partials_bf16);
+    FFMOE_DOWN(false);
+#undef FFMOE_DOWN
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_DOWN);
