@@ -32,49 +32,78 @@ constexpr int kRing = 11;       // groups in flight per wave (= one K-slice of D
 // route order. A route takes part when its weight is not +-0 and its expert is in range; an expert
 // keeps its first 16 routes. Slots past the last live expert get n = 0.
 // ---------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void verify_plan_kernel(const uint32_t *__restrict__ idx,
-                                                          const uint16_t *__restrict__ w, uint32_t n_routes,
-                                                          uint32_t n_experts, VerifyPlan *__restrict__ plan) {
-    __shared__ uint32_t cnt[FFMOE_MAX_EXPERTS];
-    __shared__ uint32_t slot_of[FFMOE_MAX_EXPERTS];
-    __shared__ uint32_t route_expert[kMaxRoutes];
-    __shared__ uint32_t wave_total[4];
+struct PlanScratch {
+    uint32_t cnt[FFMOE_MAX_EXPERTS];
+    uint32_t slot_of[FFMOE_MAX_EXPERTS];
+    uint32_t expert_of[FFMOE_MAX_EXPERTS];
+    uint32_t route_expert[kMaxRoutes];
+    uint32_t wave_total[4];
+    uint32_t my_routes[kMaxRows];
+};
+
+// Run by all 256 threads of a block. Builds the plan in LDS; writes it to `plan_out` when that is not
+// null; when `my_slot` is a live slot, leaves that slot's route list in ps.my_routes. Returns n_live.
+// `slot_from_total` maps the number of live experts to the caller's slot (or to ~0u for none).
+template <typename SlotFn>
+__device__ __forceinline__ uint32_t build_plan(PlanScratch &ps, const uint32_t *__restrict__ idx,
+                                               const uint16_t *__restrict__ w, uint32_t n_routes, uint32_t n_experts,
+                                               VerifyPlan *plan_out, SlotFn slot_from_total, uint32_t &my_slot) {
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    cnt[tid] = 0;
+    ps.cnt[tid] = 0;
     __syncthreads();
     uint32_t e = 0xFFFFFFFFu;
     if (tid < n_routes) {
         const uint32_t ee = idx[tid];
         if ((w[tid] & 0x7FFFu) != 0 && ee < n_experts) e = ee;
-        route_expert[tid] = e;
-        if (e != 0xFFFFFFFFu) atomicAdd(&cnt[e], 1u);
+        ps.route_expert[tid] = e;
+        if (e != 0xFFFFFFFFu) atomicAdd(&ps.cnt[e], 1u);
     }
     __syncthreads();
-    const bool live = tid < n_experts && cnt[tid] > 0;
+    const bool live = tid < n_experts && ps.cnt[tid] > 0;
     const unsigned long long mask = __ballot(live);
     const uint32_t before = __popcll(mask & ((1ull << lane) - 1ull));
-    if (lane == 0) wave_total[wave] = __popcll(mask);
+    if (lane == 0) ps.wave_total[wave] = __popcll(mask);
     __syncthreads();
     uint32_t base = 0, total = 0;
 #pragma unroll
     for (uint32_t v = 0; v < 4; ++v) {
-        const uint32_t c = wave_total[v];
+        const uint32_t c = ps.wave_total[v];
         base += v < wave ? c : 0;
         total += c;
     }
     if (live) {
-        slot_of[tid] = base + before;
-        plan->slots[base + before].expert = tid;
-        plan->slots[base + before].n = min(cnt[tid], (uint32_t)kMaxRows);
+        ps.slot_of[tid] = base + before;
+        ps.expert_of[base + before] = tid;
+        if (plan_out) {
+            plan_out->slots[base + before].expert = tid;
+            plan_out->slots[base + before].n = min(ps.cnt[tid], (uint32_t)kMaxRows);
+        }
     }
-    if (tid >= total) plan->slots[tid].n = 0;
-    if (tid == 0) plan->n_live = total;
+    if (plan_out) {
+        if (tid >= total) plan_out->slots[tid].n = 0;
+        if (tid == 0) plan_out->n_live = total;
+    }
+    my_slot = slot_from_total(total);
     __syncthreads();
     if (tid < n_routes && e != 0xFFFFFFFFu) {
         uint32_t pos = 0;
-        for (uint32_t j = 0; j < tid; ++j) pos += route_expert[j] == e ? 1u : 0u;
-        if (pos < (uint32_t)kMaxRows) plan->slots[slot_of[e]].routes[pos] = tid;
+        for (uint32_t j = 0; j < tid; ++j) pos += ps.route_expert[j] == e ? 1u : 0u;
+        if (pos < (uint32_t)kMaxRows) {
+            const uint32_t sl = ps.slot_of[e];
+            if (plan_out) plan_out->slots[sl].routes[pos] = tid;
+            if (sl == my_slot) ps.my_routes[pos] = tid;
+        }
     }
+    __syncthreads();
+    return total;
+}
+
+__global__ __launch_bounds__(256) void verify_plan_kernel(const uint32_t *__restrict__ idx,
+                                                          const uint16_t *__restrict__ w, uint32_t n_routes,
+                                                          uint32_t n_experts, VerifyPlan *__restrict__ plan) {
+    __shared__ PlanScratch ps;
+    uint32_t my_slot;
+    build_plan(ps, idx, w, n_routes, n_experts, plan, [](uint32_t) { return 0xFFFFFFFFu; }, my_slot);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -302,23 +331,33 @@ __device__ __forceinline__ void split_range(uint32_t n_items, uint32_t parts, ui
 // block walks a range of 16-row blocks of its expert; its four waves split K and meet in LDS per row block
 // (partials added in wave order), each wave finishing a quarter of the token slots.
 __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
-                                                                    uint32_t top_k, const VerifyPlan *__restrict__ plan,
+                                                                    uint32_t top_k, uint32_t n_experts,
+                                                                    const uint32_t *__restrict__ idx,
+                                                                    const uint16_t *__restrict__ w, uint32_t n_routes,
+                                                                    VerifyPlan *__restrict__ plan,
                                                                     const uint16_t *__restrict__ x, uint32_t x_stride,
                                                                     uint16_t *__restrict__ acts) {
     __shared__ float s_red[2][kKSplit][8][64];
-    const uint32_t n_live = plan->n_live;
-    if (n_live == 0) return;
-    const uint32_t blocks_per_slot = max(1u, min(g.gu_rb, gridDim.x / n_live));
-    const uint32_t slot_id = blockIdx.x / blocks_per_slot;
-    if (slot_id >= n_live) return;
+    __shared__ PlanScratch ps;
+    // Every block derives the routing plan itself from the (at most 128) routes: a few hundred LDS
+    // operations, against a separate launch plus two dependent global reads per block. Block 0 also
+    // writes the plan out for the down kernel.
+    const uint32_t gu_rb = g.gu_rb, n_blocks = gridDim.x, bid = blockIdx.x;
+    uint32_t slot_id;
+    const uint32_t n_live = build_plan(
+        ps, idx, w, n_routes, n_experts, bid == 0 ? plan : nullptr,
+        [=](uint32_t total) { return total ? bid / max(1u, min(gu_rb, n_blocks / total)) : 0xFFFFFFFFu; }, slot_id);
+    if (n_live == 0 || slot_id >= n_live) return;
+    const uint32_t blocks_per_slot = max(1u, min(gu_rb, n_blocks / n_live));
     uint32_t rb0, rb1;
-    split_range(g.gu_rb, blocks_per_slot, blockIdx.x % blocks_per_slot, rb0, rb1);
+    split_range(gu_rb, blocks_per_slot, bid % blocks_per_slot, rb0, rb1);
     if (rb0 >= rb1) return;
-    const PlanSlot &slot = plan->slots[slot_id];
-    const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
+    const uint32_t slot_expert = __builtin_amdgcn_readfirstlane(ps.expert_of[slot_id]);
+    const uint32_t n = min(__builtin_amdgcn_readfirstlane(ps.cnt[slot_expert]), (uint32_t)kMaxRows);
+    struct { const uint32_t *routes; } slot = {ps.my_routes};
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15, jq = lane >> 4;
-    const uint8_t *expert_base = arena_layer + (size_t)__builtin_amdgcn_readfirstlane(slot.expert) * g.expert_bytes;
+    const uint8_t *expert_base = arena_layer + (size_t)slot_expert * g.expert_bytes;
     const uint32_t per = (g.gd + kKSplit - 1) / kKSplit;
     const uint32_t g0 = min(ks * per, g.gd), g1 = min(g.gd, g0 + per), ng = g1 - g0;
     const uint32_t g_last = g1 > g0 ? g1 - 1 : g.gd - 1;
@@ -513,17 +552,18 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
                          VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer) {
     timer->begin(s);
-    hipLaunchKernelGGL(verify_plan_kernel, dim3(1), dim3(256), 0, s, idx, w, t * top_k, n_experts, plan);
-    timer->mark(s, FFMOE_K_PLAN);
     const uint32_t slots = min(n_experts, t * top_k);
     // the persistent kernels hold a K-slice of kRing groups per wave; larger experts take the one-shot grids
     const bool persistent = (g.gd + kKSplit - 1) / kKSplit <= (uint32_t)kRing && g.gf <= (uint32_t)kRing;
     const uint32_t resident = 2 * n_cus;       // blocks the chip holds at once (__launch_bounds__(256, 2))
     if (persistent) {
+        // plan slot of the profile stays empty: the gate/up kernel builds the plan itself
         const uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
-        hipLaunchKernelGGL(skinny_gate_up_persistent, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k,
-                           plan, x, x_stride, acts);
+        hipLaunchKernelGGL(skinny_gate_up_persistent, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts,
+                           idx, w, t * top_k, plan, x, x_stride, acts);
     } else {
+        hipLaunchKernelGGL(verify_plan_kernel, dim3(1), dim3(256), 0, s, idx, w, t * top_k, n_experts, plan);
+        timer->mark(s, FFMOE_K_PLAN);
         hipLaunchKernelGGL(skinny_gate_up_kernel, dim3(g.gu_rb, slots), dim3(256), 0, s, arena_layer, g, top_k, plan, x,
                            x_stride, acts);
     }
