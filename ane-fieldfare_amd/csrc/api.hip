@@ -22,6 +22,15 @@ struct ffmoe_layer {
     uint16_t *per_expert_scale = nullptr;
 };
 
+// A resident matrix: the re-tiled copy of one [m][n] INT4 weight plus the scratch of its greedy choice.
+struct ffmoe_matrix {
+    ffmoe_ctx *ctx = nullptr;
+    uint32_t m = 0, n = 0;
+    uint8_t *tiles = nullptr, *scales = nullptr;
+    float *logits = nullptr;                  // [16][m] fp32, allocated with the first greedy call's matrix
+    unsigned long long *partials = nullptr;   // [16][segments]
+};
+
 struct ffmoe_ctx {
     int device = 0;
     uint32_t n_cus = 0;       // compute units: sizes the persistent grids
@@ -418,6 +427,123 @@ int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16
     ctx->timer.begin(static_cast<hipStream_t>(stream));
     FF_HIP(launch_gemv_int4(static_cast<hipStream_t>(stream), w, scales, biases, x, y, m, n, rows, x_stride, y_stride, y_f32));
     ctx->timer.mark(static_cast<hipStream_t>(stream), FFMOE_K_GEMV);
+    ctx->timer.finish();
+    return FFMOE_OK;
+}
+
+int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases, uint32_t m,
+                        uint32_t n, int with_greedy, ffmoe_matrix **out, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!w || !scales || !biases || !out) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    *out = nullptr;
+    if (m == 0) return fail(err, FFMOE_ERR_INVALID, "M must be positive");
+    if (n == 0 || !matrix_shape_ok(n))
+        return fail(err, FFMOE_ERR_INVALID, "N = %u must be a multiple of %d and at most %d", n, FFMOE_GROUP,
+                    FFMOE_MATRIX_MAX_N);
+    if (reinterpret_cast<uintptr_t>(w) % 2) return fail(err, FFMOE_ERR_INVALID, "weights need a 2-aligned offset");
+    ffmoe_matrix *mx = new (std::nothrow) ffmoe_matrix();
+    if (!mx) return fail(err, FFMOE_ERR_ALLOC, "out of host memory");
+    mx->ctx = ctx;
+    mx->m = m;
+    mx->n = n;
+    const size_t w_bytes = (size_t)m * n / 2, s_bytes = (size_t)m * (n / FFMOE_GROUP) * 2;
+    uint8_t *stage = nullptr;
+    auto cleanup = [&]() {
+        if (stage) (void)hipFree(stage);
+        if (mx->tiles) (void)hipFree(mx->tiles);
+        if (mx->scales) (void)hipFree(mx->scales);
+        if (mx->logits) (void)hipFree(mx->logits);
+        if (mx->partials) (void)hipFree(mx->partials);
+        delete mx;
+    };
+#define FF_MX(call)                                                                                   \
+    do {                                                                                              \
+        hipError_t e_ = (call);                                                                       \
+        if (e_ != hipSuccess) {                                                                       \
+            cleanup();                                                                                \
+            return fail(err, e_ == hipErrorOutOfMemory ? FFMOE_ERR_ALLOC : FFMOE_ERR_RUNTIME,         \
+                        "%s: %s", #call, hipGetErrorString(e_));                                      \
+        }                                                                                             \
+    } while (0)
+    FF_MX(hipMalloc(&mx->tiles, matrix_tiles_bytes(m, n)));
+    FF_MX(hipMalloc(&mx->scales, matrix_scales_bytes(m, n)));
+    if (with_greedy) {
+        FF_MX(hipMalloc(&mx->logits, (size_t)FFMOE_MAX_VERIFY_ROWS * m * sizeof(float)));
+        FF_MX(hipMalloc(&mx->partials, (size_t)FFMOE_MAX_VERIFY_ROWS * argmax_segments(m) * sizeof(unsigned long long)));
+    }
+    // the source may live on the host (an mmap of the checkpoint) or on the device
+    const uint8_t *dw = w;
+    const uint16_t *ds = scales, *db = biases;
+    hipPointerAttribute_t attr{};
+    const bool on_device = hipPointerGetAttributes(&attr, w) == hipSuccess && attr.type == hipMemoryTypeDevice;
+    (void)hipGetLastError();
+    if (!on_device) {
+        const size_t w_pad = (w_bytes + 15) / 16 * 16, s_pad = (s_bytes + 15) / 16 * 16;
+        FF_MX(hipMalloc(&stage, w_pad + 2 * s_pad));
+        FF_MX(hipMemcpy(stage, w, w_bytes, hipMemcpyHostToDevice));
+        FF_MX(hipMemcpy(stage + w_pad, scales, s_bytes, hipMemcpyHostToDevice));
+        FF_MX(hipMemcpy(stage + w_pad + s_pad, biases, s_bytes, hipMemcpyHostToDevice));
+        dw = stage;
+        ds = reinterpret_cast<const uint16_t *>(stage + w_pad);
+        db = reinterpret_cast<const uint16_t *>(stage + w_pad + s_pad);
+    }
+    FF_MX(launch_matrix_repack(nullptr, dw, ds, db, m, n, mx->tiles, mx->scales));
+    FF_MX(hipDeviceSynchronize());
+#undef FF_MX
+    if (stage) (void)hipFree(stage);
+    *out = mx;
+    return FFMOE_OK;
+}
+
+void ffmoe_matrix_destroy(ffmoe_matrix *mx) {
+    if (!mx) return;
+    (void)hipSetDevice(mx->ctx->device);
+    (void)hipDeviceSynchronize();
+    if (mx->tiles) (void)hipFree(mx->tiles);
+    if (mx->scales) (void)hipFree(mx->scales);
+    if (mx->logits) (void)hipFree(mx->logits);
+    if (mx->partials) (void)hipFree(mx->partials);
+    delete mx;
+}
+
+static int check_matrix_call(ffmoe_matrix *mx, const uint16_t *x, uint32_t x_stride, uint32_t rows, char **err) {
+    if (!mx || !mx->ctx) return fail(err, FFMOE_ERR_INVALID, "null matrix");
+    if (int rc = check_ctx(mx->ctx, err)) return rc;
+    if (!x) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (rows == 0 || rows > FFMOE_MAX_VERIFY_ROWS)
+        return fail(err, FFMOE_ERR_INVALID, "rows=%u outside 1...%d", rows, FFMOE_MAX_VERIFY_ROWS);
+    if (x_stride < mx->n || x_stride % 8 || reinterpret_cast<uintptr_t>(x) % 16)
+        return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a row stride that is a multiple of 8 and >= N");
+    return FFMOE_OK;
+}
+
+int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y,
+                      uint32_t y_stride, int y_f32, char **err) {
+    if (int rc = check_matrix_call(mx, x, x_stride, rows, err)) return rc;
+    if (!y) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (y_stride < mx->m) return fail(err, FFMOE_ERR_INVALID, "stride smaller than the row");
+    ffmoe_ctx *ctx = mx->ctx;
+    ctx->timer.begin(static_cast<hipStream_t>(stream));
+    FF_HIP(launch_matrix_gemv(static_cast<hipStream_t>(stream), mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows,
+                              y, y_stride, y_f32 != 0, ctx->n_cus));
+    ctx->timer.mark(static_cast<hipStream_t>(stream), FFMOE_K_GEMV);
+    ctx->timer.finish();
+    return FFMOE_OK;
+}
+
+int ffmoe_matrix_greedy(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
+                        uint32_t *out_tokens, char **err) {
+    if (int rc = check_matrix_call(mx, x, x_stride, rows, err)) return rc;
+    if (!out_tokens) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (!mx->logits) return fail(err, FFMOE_ERR_INVALID, "matrix was created without the greedy scratch");
+    ffmoe_ctx *ctx = mx->ctx;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    ctx->timer.begin(s);
+    FF_HIP(launch_matrix_gemv(s, mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows, mx->logits, mx->m, true,
+                              ctx->n_cus));
+    ctx->timer.mark(s, FFMOE_K_GEMV);
+    FF_HIP(launch_argmax_rows(s, mx->logits, mx->m, mx->m, rows, mx->partials, out_tokens));
+    ctx->timer.mark(s, FFMOE_K_ARGMAX);
     ctx->timer.finish();
     return FFMOE_OK;
 }

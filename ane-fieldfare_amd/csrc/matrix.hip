@@ -1,0 +1,236 @@
+// Resident INT4 matrix: a [M][N] weight in the reference's row-major layout is re-tiled once into
+// two-stream tiles and then serves 1..16 input rows per call at streaming speed, with an optional
+// greedy choice (argmax) over the outputs.
+//
+// Replaces the LM head of LMHeadChainInt4.encodeGreedyDecode / encodeGreedyRows
+// (Kernels/Fusions/LMHeadChainInt4.swift:94-139,225-284; Metal/Sampling/logit.metal:614-720,952-1005) and the
+// static-weight uses of DequantInt4GEMV.encodeRows (Kernels/Quant/DequantInt4GEMV.swift:72-182).
+// A tile holds rows a = 32 p + l % 16 (stream A) and a + 16 (stream B) of one 64-wide group, in the
+// same lane order as the expert arena, so the kernels share the expert path's register-ring code.
+#include "common.hpp"
+#include "kernels.hpp"
+#include "stream.hpp"
+
+namespace ffmoe {
+namespace {
+
+__device__ __forceinline__ uint32_t ref_nibbles8(const uint8_t *row, uint32_t k0) {
+    const uint8_t *p = row + (k0 >> 1);
+    return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+
+// reference order (nibble j = element j) -> arena order (position m = element 2m, m + 4 = element 2m + 1)
+__device__ __forceinline__ uint32_t to_arena_order(uint32_t v) {
+    uint32_t out = 0;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        out |= ((v >> (8 * m)) & 0xFu) << (4 * m);
+        out |= ((v >> (8 * m + 4)) & 0xFu) << (4 * m + 16);
+    }
+    return out;
+}
+
+__device__ __forceinline__ uint16_t load_u16(const uint8_t *p) { return (uint16_t)(p[0] | ((uint16_t)p[1] << 8)); }
+
+// One thread per (tile, lane). Rows past M (M is padded up to a multiple of 32) become zero weights
+// with zero scale and bias.
+__global__ __launch_bounds__(256) void repack_matrix_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ s,
+                                                            const uint8_t *__restrict__ b, uint32_t m, uint32_t n,
+                                                            uint8_t *__restrict__ tiles, uint8_t *__restrict__ scales) {
+    const uint32_t n_groups = n / kGroup, row_bytes = n / 2;
+    const size_t n_tiles = (size_t)((m + 31) / 32) * n_groups;
+    const size_t total = n_tiles * kWave;
+    for (size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x; gid < total;
+         gid += (size_t)gridDim.x * blockDim.x) {
+        const uint32_t lane = gid & 63, i = lane & 15, jq = lane >> 4;
+        const size_t tile = gid >> 6;
+        const uint32_t rbp = tile / n_groups, grp = tile % n_groups;
+        const uint32_t row_a = rbp * 2 * kTileRows + i, row_b = row_a + kTileRows;
+        const uint32_t k0 = grp * kGroup + 8 * jq;
+        uint4 chunk = {0, 0, 0, 0};
+        if (row_a < m) {
+            chunk.x = to_arena_order(ref_nibbles8(w + (size_t)row_a * row_bytes, k0));
+            chunk.y = to_arena_order(ref_nibbles8(w + (size_t)row_a * row_bytes, k0 + 32));
+        }
+        if (row_b < m) {
+            chunk.z = to_arena_order(ref_nibbles8(w + (size_t)row_b * row_bytes, k0));
+            chunk.w = to_arena_order(ref_nibbles8(w + (size_t)row_b * row_bytes, k0 + 32));
+        }
+        reinterpret_cast<uint4 *>(tiles + tile * kTileBytes)[lane] = chunk;
+        if (jq == 0) {
+            uint2 sc = {0, 0};
+            const size_t ia = ((size_t)row_a * n_groups + grp) * 2, ib = ((size_t)row_b * n_groups + grp) * 2;
+            if (row_a < m) sc.x = (uint32_t)load_u16(s + ia) | ((uint32_t)load_u16(b + ia) << 16);
+            if (row_b < m) sc.y = (uint32_t)load_u16(s + ib) | ((uint32_t)load_u16(b + ib) << 16);
+            reinterpret_cast<uint2 *>(scales + tile * kTileScaleBytes)[i] = sc;
+        }
+    }
+}
+
+// y[r][m] = sum_g [ s_g * sum_k q_k x_k + b_g * sum_k x_k ] (moe.metal:323-378, logit.metal:614-667) for all
+// input rows at once. grid = (blocks): every block walks a range of 32-row tiles; its four waves split K
+// (at most kRing groups each), keep their slice of the input rows in registers and refill the weight
+// ring across tiles; per tile the partial sums meet in LDS, are added in wave order, and each wave
+// stores a quarter of the input rows.
+template <bool Y_F32>
+__global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__restrict__ tiles,
+                                                             const uint8_t *__restrict__ scales, uint32_t m,
+                                                             uint32_t n_groups, const uint16_t *__restrict__ x,
+                                                             uint32_t x_stride, uint32_t rows, void *__restrict__ y_,
+                                                             uint32_t y_stride) {
+    __shared__ float s_red[2][kKSplit][8][64];
+    const uint32_t n_tiles = (m + 31) / 32;
+    uint32_t rb0, rb1;
+    split_range(n_tiles, gridDim.x, blockIdx.x, rb0, rb1);
+    if (rb0 >= rb1) return;
+    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint32_t per = (n_groups + kKSplit - 1) / kKSplit;
+    const uint32_t g0 = min(ks * per, n_groups), g1 = min(n_groups, g0 + per), ng = g1 - g0;
+    const uint32_t g_last = g1 > g0 ? g1 - 1 : n_groups - 1;
+    const size_t tile_row = (size_t)n_groups * kTileBytes, scale_row = (size_t)n_groups * kTileScaleBytes;
+
+    WeightRing ring;
+#pragma unroll
+    for (int u = 0; u < kRing; ++u)
+        ring_fill(ring, u, tiles + rb0 * tile_row, scales + rb0 * scale_row, min(g0 + u, g_last), lane);
+    const uint16_t *xrow = x + (size_t)min(j, rows - 1) * x_stride + 8 * jq;
+    uint4 x0[kRing], x1[kRing];
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) {
+        const bool live = (uint32_t)u < ng;
+        const uint32_t gg = min(g0 + u, g_last);
+        x0[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup) : uint4{0, 0, 0, 0};
+        x1[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
+    }
+    const uint32_t my_row = 4 * jq + ks;        // the input row this lane finishes
+    float *y32 = reinterpret_cast<float *>(y_);
+    uint16_t *y16 = reinterpret_cast<uint16_t *>(y_);
+
+    for (uint32_t rb = rb0; rb < rb1; ++rb) {
+        const uint32_t rbn = min(rb + 1, rb1 - 1);
+        const uint8_t *nt = tiles + rbn * tile_row, *ns = scales + rbn * scale_row;
+        TwoStreamAcc tot;
+        tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
+        tot.b = tot.a;
+#pragma unroll
+        for (int u = 0; u < kRing; ++u)
+            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, nt, ns, min(g0 + u, g_last), lane);
+        const int buf = (rb - rb0) & 1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            s_red[buf][ks][r][lane] = tot.a[r];
+            s_red[buf][ks][4 + r][lane] = tot.b[r];
+        }
+        lds_barrier();
+        float va = s_red[buf][0][ks][lane], vb = s_red[buf][0][4 + ks][lane];
+#pragma unroll
+        for (int o = 1; o < kKSplit; ++o) {
+            va += s_red[buf][o][ks][lane];
+            vb += s_red[buf][o][4 + ks][lane];
+        }
+        if (my_row < rows) {
+            const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
+            const size_t base = (size_t)my_row * y_stride;
+            if (Y_F32) {
+                if (row_a < m) y32[base + row_a] = va;
+                if (row_b < m) y32[base + row_b] = vb;
+            } else {
+                if (row_a < m) y16[base + row_a] = f32_to_bf16(va);
+                if (row_b < m) y16[base + row_b] = f32_to_bf16(vb);
+            }
+        }
+    }
+}
+
+// Greedy choice per row: the largest finite value wins, ties go to the lowest index, NaN and +-inf never
+// win; a row with no candidate yields index 0 (Metal/Sampling/logit.metal:689-720, 916-921). Two stages so that the
+// vocabulary-sized scan uses the whole chip: per (row, segment) partial winners, then one block per row.
+__device__ __forceinline__ unsigned long long argmax_key(float v, uint32_t i) {
+    if (!(__builtin_fabsf(v) < INFINITY)) return 0ull;       // NaN or +-inf: never chosen
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t ord = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    return ((unsigned long long)ord << 32) | (0xFFFFFFFFu - i);
+}
+
+__device__ __forceinline__ unsigned long long block_max_key(unsigned long long k, unsigned long long *s_k) {
+#pragma unroll
+    for (int mk = 32; mk >= 1; mk >>= 1) {
+        const unsigned long long o = __shfl_xor(k, mk, 64);
+        k = o > k ? o : k;
+    }
+    if ((threadIdx.x & 63) == 0) s_k[threadIdx.x >> 6] = k;
+    __syncthreads();
+    k = s_k[0];
+    for (uint32_t v = 1; v < blockDim.x / 64; ++v) k = s_k[v] > k ? s_k[v] : k;
+    return k;
+}
+
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__restrict__ y, uint32_t y_stride, uint32_t m,
+                                                             uint32_t seg_len, unsigned long long *__restrict__ part) {
+    __shared__ unsigned long long s_k[4];
+    const uint32_t row = blockIdx.y, seg = blockIdx.x;
+    const uint32_t i0 = seg * seg_len, i1 = min(m, i0 + seg_len);
+    unsigned long long best = 0ull;
+    for (uint32_t i = i0 + threadIdx.x; i < i1; i += 256) {
+        const unsigned long long k = argmax_key(y[(size_t)row * y_stride + i], i);
+        best = k > best ? k : best;
+    }
+    best = block_max_key(best, s_k);
+    if (threadIdx.x == 0) part[(size_t)row * gridDim.x + seg] = best;
+}
+
+__global__ __launch_bounds__(256) void argmax_final_kernel(const unsigned long long *__restrict__ part, uint32_t n_seg,
+                                                           uint32_t *__restrict__ out) {
+    __shared__ unsigned long long s_k[4];
+    const uint32_t row = blockIdx.x;
+    unsigned long long best = 0ull;
+    for (uint32_t i = threadIdx.x; i < n_seg; i += 256) {
+        const unsigned long long k = part[(size_t)row * n_seg + i];
+        best = k > best ? k : best;
+    }
+    best = block_max_key(best, s_k);
+    if (threadIdx.x == 0) out[row] = best ? 0xFFFFFFFFu - (uint32_t)best : 0u;
+}
+
+}  // namespace
+
+size_t matrix_tiles_bytes(uint32_t m, uint32_t n) { return (size_t)((m + 31) / 32) * (n / kGroup) * kTileBytes; }
+size_t matrix_scales_bytes(uint32_t m, uint32_t n) { return (size_t)((m + 31) / 32) * (n / kGroup) * kTileScaleBytes; }
+bool matrix_shape_ok(uint32_t n) { return n % kGroup == 0 && (n / kGroup + kKSplit - 1) / kKSplit <= (uint32_t)kRing; }
+
+hipError_t launch_matrix_repack(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                                uint32_t m, uint32_t n, uint8_t *tiles_out, uint8_t *scales_out) {
+    const size_t total = matrix_tiles_bytes(m, n) / kTileBytes * kWave;
+    const uint32_t blocks = (uint32_t)min((size_t)65535 * 16, (total + 255) / 256);
+    hipLaunchKernelGGL(repack_matrix_kernel, dim3(blocks), dim3(256), 0, s, w, reinterpret_cast<const uint8_t *>(scales),
+                       reinterpret_cast<const uint8_t *>(biases), m, n, tiles_out, scales_out);
+    return hipGetLastError();
+}
+
+hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
+                              const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
+                              bool y_f32, uint32_t n_cus) {
+    const uint32_t n_tiles = (m + 31) / 32;
+    const dim3 grid(min(2 * n_cus, n_tiles));
+    if (y_f32)
+        hipLaunchKernelGGL(matrix_gemv_kernel<true>, grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, rows,
+                           y, y_stride);
+    else
+        hipLaunchKernelGGL(matrix_gemv_kernel<false>, grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride,
+                           rows, y, y_stride);
+    return hipGetLastError();
+}
+
+uint32_t argmax_segments(uint32_t m) { return min(256u, (m + 4095) / 4096); }
+
+hipError_t launch_argmax_rows(hipStream_t s, const float *y, uint32_t y_stride, uint32_t m, uint32_t rows,
+                              unsigned long long *partials, uint32_t *out) {
+    const uint32_t n_seg = argmax_segments(m);
+    const uint32_t seg_len = (m + n_seg - 1) / n_seg;
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(n_seg, rows), dim3(256), 0, s, y, y_stride, m, seg_len, partials);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, partials, n_seg, out);
+    return hipGetLastError();
+}
+
+}  // namespace ffmoe

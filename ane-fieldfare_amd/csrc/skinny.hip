@@ -17,14 +17,13 @@
 // wave has PD KiB of weights in flight from its first instruction.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "stream.hpp"
 
 namespace ffmoe {
 namespace {
 
 constexpr int kMaxRows = FFMOE_MAX_VERIFY_ROWS;
 constexpr int kMaxRoutes = kMaxRows * 8;
-constexpr int kKSplit = 4;      // waves of a gate/up block that split K
-constexpr int kRing = 11;       // groups in flight per wave (= one K-slice of D = 2816)
 
 // ---------------------------------------------------------------------------------------------------
 // Plan: invert routes [t][top_k] into per-expert route lists and compact the live experts in expert
@@ -112,10 +111,6 @@ __global__ __launch_bounds__(256) void verify_plan_kernel(const uint32_t *__rest
 // the token operand it supplies token slot l % 16 (`xrow` = that token's row, already offset by
 // 8 * (l / 16) elements); it ends up holding token slots 4 * (l / 16) + 0..3.
 // ---------------------------------------------------------------------------------------------------
-struct TwoStreamAcc {
-    f32x4 a, b;
-};
-
 template <int PD>
 __device__ __forceinline__ TwoStreamAcc stream_tiles(const uint8_t *__restrict__ tiles,
                                                      const uint8_t *__restrict__ scales,
@@ -276,57 +271,6 @@ __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restr
 // has one full K-slice (about 12 KiB) of weights in flight and never pays the load latency again.
 // Groups past the end of a short K-slice are read from the last valid tile and enter with zero scales.
 // ---------------------------------------------------------------------------------------------------
-struct WeightRing {
-    uint4 t[kRing];
-    uint2 s[kRing];
-};
-
-// `tiles` / `scales` are wave-uniform (scalar registers); the lane part is a 32-bit offset, so every ring load is
-// one instruction with a scalar base and no per-load 64-bit address arithmetic.
-__device__ __forceinline__ void ring_fill(WeightRing &ring, int u, const uint8_t *tiles, const uint8_t *scales,
-                                          uint32_t g_clamped, uint32_t lane) {
-    const uint8_t *tg = tiles + (size_t)g_clamped * kTileBytes, *sg = scales + (size_t)g_clamped * kTileScaleBytes;
-    ring.t[u] = *reinterpret_cast<const uint4 *>(tg + lane * 16u);
-    ring.s[u] = *reinterpret_cast<const uint2 *>(sg + (lane & 15u) * 8u);
-}
-
-// Consume ring slot u against the resident token operand, then start the load that refills the slot.
-__device__ __forceinline__ void ring_step(WeightRing &ring, int u, bool live, const uint4 &x0, const uint4 &x1,
-                                          TwoStreamAcc &tot, const uint8_t *next_tiles, const uint8_t *next_scales,
-                                          uint32_t next_g, uint32_t lane) {
-    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-    const uint4 ones_bits = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-    const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
-    const uint4 tile = ring.t[u];
-    uint2 sc = ring.s[u];
-    if (!live) sc = make_uint2(0u, 0u);
-    ring_fill(ring, u, next_tiles, next_scales, next_g, lane);
-    const bf16x8 a0 = __builtin_bit_cast(bf16x8, x0), a1 = __builtin_bit_cast(bf16x8, x1);
-    f32x4 acc_a = mfma16(a0, unpack8_offset128(tile.x), zero);
-    acc_a = mfma16(a1, unpack8_offset128(tile.y), acc_a);
-    f32x4 acc_b = mfma16(a0, unpack8_offset128(tile.z), zero);
-    acc_b = mfma16(a1, unpack8_offset128(tile.w), acc_b);
-    f32x4 sx = mfma16(a0, ones, zero);
-    sx = mfma16(a1, ones, sx);
-    const float sa = bf16lo_to_f32(sc.x), ba = bf16hi_to_f32(sc.x);
-    const float sb = bf16lo_to_f32(sc.y), bb = bf16hi_to_f32(sc.y);
-    const float ta = __builtin_fmaf(-128.0f, sa, ba), tb = __builtin_fmaf(-128.0f, sb, bb);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        tot.a[r] = __builtin_fmaf(sa, acc_a[r], tot.a[r]);
-        tot.a[r] = __builtin_fmaf(ta, sx[r], tot.a[r]);
-        tot.b[r] = __builtin_fmaf(sb, acc_b[r], tot.b[r]);
-        tot.b[r] = __builtin_fmaf(tb, sx[r], tot.b[r]);
-    }
-}
-
-// Split `n_items` of one expert over `parts` workers: worker `sub` gets [first, last).
-__device__ __forceinline__ void split_range(uint32_t n_items, uint32_t parts, uint32_t sub, uint32_t &first,
-                                            uint32_t &last) {
-    first = (uint32_t)((uint64_t)sub * n_items / parts);
-    last = (uint32_t)((uint64_t)(sub + 1) * n_items / parts);
-}
-
 // gate/up + GELU-tanh gating, persistent. grid = (blocks); the blocks are dealt to the live experts, each
 // block walks a range of 16-row blocks of its expert; its four waves split K and meet in LDS per row block
 // (partials added in wave order), each wave finishing a quarter of the token slots.

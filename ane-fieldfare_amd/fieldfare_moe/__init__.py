@@ -43,16 +43,69 @@ EXPORTS = [
     "ffmoe_upload_router_bf16", "ffmoe_upload_router_int8", "ffmoe_dequant_expert", "ffmoe_router",
     "ffmoe_verify", "ffmoe_verify_partials", "ffmoe_last_live_experts", "ffmoe_reduce_token_major",
     "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
-    "ffmoe_prefill_plan_stats",
+    "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
+    "ffmoe_matrix_greedy",
 ]
 
 PROFILE_SLOTS = 12
 KERNEL_NAMES = ["router_logits", "router_topk", "plan", "gate_up", "down", "combine", "prefill_sort",
-                "prefill_gate_up", "prefill_down", "prefill_combine", "gemv", "reserved"]
+                "prefill_gate_up", "prefill_down", "prefill_combine", "gemv", "argmax"]
 
 
 class Profile(C.Structure):
     _fields_ = [("ms", C.c_double * PROFILE_SLOTS), ("launches", C.c_uint64 * PROFILE_SLOTS)]
+
+
+class Matrix:
+    """ffmoe_matrix: the LM head (or any static INT4 weight) kept re-tiled in HBM."""
+
+    def __init__(self, ctx, W, S, B, greedy: bool, w_byte_offset: int = 0):
+        import numpy as np
+        self.ctx, self.L = ctx, ctx.L
+        self.m, self.n = int(S.shape[0]), int(S.shape[1]) * GROUP
+        keep = []
+
+        def raw(a, off=0):
+            if isinstance(a, np.ndarray):
+                a = np.ascontiguousarray(a)
+                keep.append(a)
+                return C.c_void_p(a.ctypes.data + off)
+            keep.append(a)
+            return C.c_void_p(a.data_ptr() + off)
+
+        h, err = C.c_void_p(), C.c_char_p()
+        _check(self.L.ffmoe_matrix_create(ctx._h, raw(W, w_byte_offset), raw(S), raw(B), self.m, self.n, int(greedy),
+                                          C.byref(h), C.byref(err)), err)
+        self._h = h
+
+    def gemv(self, x, f32_out: bool = False):
+        import torch
+        rows = x.shape[0]
+        y = torch.empty((rows, self.m), dtype=torch.float32 if f32_out else torch.bfloat16, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_matrix_gemv(self._h, _stream(), _ptr(x), _row_stride(x), rows, _ptr(y), self.m,
+                                        int(f32_out), C.byref(err)), err)
+        return y
+
+    def greedy(self, x):
+        import torch
+        rows = x.shape[0]
+        out = torch.empty((rows,), dtype=torch.int32, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_matrix_greedy(self._h, _stream(), _ptr(x), _row_stride(x), rows, _ptr(out), C.byref(err)),
+               err)
+        return out
+
+    def close(self):
+        if self._h:
+            self.L.ffmoe_matrix_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 def build() -> Path:
@@ -98,6 +151,11 @@ def lib() -> C.CDLL:
     L.ffmoe_prefill.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
     L.ffmoe_prefill_pairs.argtypes = [vp, vp, u32, vp, u32, vp, u32, u32, vp, errp]
     L.ffmoe_prefill_plan_stats.argtypes = [vp, vp, C.POINTER(u32), C.POINTER(u32), vp, errp]
+    L.ffmoe_matrix_create.argtypes = [vp, vp, vp, vp, u32, u32, i32, C.POINTER(vp), errp]
+    L.ffmoe_matrix_destroy.argtypes = [vp]
+    L.ffmoe_matrix_destroy.restype = None
+    L.ffmoe_matrix_gemv.argtypes = [vp, vp, vp, u32, u32, vp, u32, i32, errp]
+    L.ffmoe_matrix_greedy.argtypes = [vp, vp, vp, u32, u32, vp, errp]
     _lib = L
     return L
 
@@ -284,6 +342,10 @@ class Context:
         return int(n_pairs.value), int(n_tiles.value), counts
 
     # -- generic GEMV ----------------------------------------------------------------------------
+    def matrix(self, W, S, B, greedy: bool = False, w_byte_offset: int = 0):
+        """Resident re-tiled copy of W uint8 [M, N/2], S/B bf16 bits [M, N/64] (numpy arrays or tensors)."""
+        return Matrix(self, W, S, B, greedy, w_byte_offset)
+
     def gemv_int4(self, W, S, B, x, f32_out: bool = False, w_byte_offset: int = 0):
         """W uint8 [M, N/2] (optionally starting `w_byte_offset` bytes into a larger buffer), S/B bf16-bit
         int16/uint16 tensors [M, N/64], x bf16 [R, stride]. Returns y [R, M]."""

@@ -195,13 +195,42 @@ int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16
                     const uint16_t *biases, const uint16_t *x, void *y, uint32_t m, uint32_t n,
                     uint32_t rows, uint32_t x_stride, uint32_t y_stride, int y_f32, char **err);
 
+/* ---- resident INT4 matrix (LM head and other static weights) ------------------------------------ */
+
+#define FFMOE_MATRIX_MAX_N 2816  /* K kept in registers: 4 waves x 11 groups of 64 */
+
+typedef struct ffmoe_matrix ffmoe_matrix;
+
+/* Re-tiles one weight in the reference layout (W uint8 [m][n/2] with 2-byte alignment, S/B bf16
+ * [m][n/64]; host or device memory) into HBM once, as LMHeadChainInt4 keeps the head's table and
+ * scratch for its lifetime (Kernels/Fusions/LMHeadChainInt4.swift:57-88). n must be a multiple of 64,
+ * at most FFMOE_MATRIX_MAX_N; m is free (the reference's head tests use 4,099 rows). with_greedy != 0
+ * also allocates the fp32 logits of ffmoe_matrix_greedy ([16][m]). Blocking; not a hot-path call. */
+int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                        uint32_t m, uint32_t n, int with_greedy, ffmoe_matrix **out, char **err);
+void ffmoe_matrix_destroy(ffmoe_matrix *mx);
+
+/* y[r][row] = sum_g [ s_g * sum_k q_k x_k + b_g * sum_k x_k ] for r < rows <= 16 with the matrix read
+ * once: DequantInt4GEMV.encodeRows on a static weight (Kernels/Quant/DequantInt4GEMV.swift:72-123) and
+ * the head projection of LMHeadChainInt4.encodeGreedyRows (LMHeadChainInt4.swift:122-131). x bf16
+ * [rows][x_stride], 16-byte aligned, stride a multiple of 8; y bf16 or (y_f32 != 0) fp32 [rows][y_stride]. */
+int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
+                      void *y, uint32_t y_stride, int y_f32, char **err);
+
+/* Greedy token per row: fp32 logits from the GEMV above, then the index of the largest finite logit,
+ * ties to the lowest index, non-finite values never chosen (Metal/Sampling/logit.metal:689-720,916-921;
+ * LMHeadChainInt4.encodeGreedyDecode / encodeGreedyRows, LMHeadChainInt4.swift:94-139,225-284). The
+ * input rows are the already normalised hidden rows (the reference runs its RMSNorm operator first). */
+int ffmoe_matrix_greedy(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
+                        uint32_t *out_tokens, char **err);
+
 /* ---- per-kernel timing ------------------------------------------------------------------------ */
 
 /* Kernel slots of ffmoe_profile. */
 enum {
     FFMOE_K_ROUTER_LOGITS = 0, FFMOE_K_ROUTER_TOPK, FFMOE_K_PLAN, FFMOE_K_GATE_UP, FFMOE_K_DOWN,
     FFMOE_K_COMBINE, FFMOE_K_PREFILL_SORT, FFMOE_K_PREFILL_GATE_UP, FFMOE_K_PREFILL_DOWN,
-    FFMOE_K_PREFILL_COMBINE, FFMOE_K_GEMV, FFMOE_PROFILE_SLOTS = 12
+    FFMOE_K_PREFILL_COMBINE, FFMOE_K_GEMV, FFMOE_K_ARGMAX, FFMOE_PROFILE_SLOTS = 12
 };
 typedef struct {
     double ms[FFMOE_PROFILE_SLOTS];          /* summed GPU time per kernel slot */

@@ -1,0 +1,161 @@
+"""Resident INT4 matrix (LM head): re-tiling, multi-row GEMV and greedy choice against the CPU oracle,
+through the C ABI. Run on the GPU box: pytest -m gpu."""
+import numpy as np
+import pytest
+
+from helpers import bf16_tensor, bits_of, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+@pytest.fixture(scope="module")
+def ff():
+    import fieldfare_moe
+    fieldfare_moe.lib()
+    return fieldfare_moe
+
+
+@pytest.fixture(scope="module")
+def ctx(ff, torch):
+    c = ff.Context(128, 64, 16, 8, n_layers=1, max_tokens=16)
+    yield c
+    c.close()
+
+
+def _i16(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda()
+
+
+@pytest.mark.parametrize("m,n,rows,off,src", [(300, 2112, 3, 0, "host"), (301, 2816, 4, 2, "device"),
+                                              (256, 2112, 12, 0, "device"), (384, 2816, 13, 0, "host"),
+                                              (1408, 2816, 1, 0, "device"), (1408, 2816, 16, 0, "device"),
+                                              (64, 128, 1, 0, "host"), (4099, 2816, 4, 0, "device")])
+def test_matrix_gemv_reference_shapes(ctx, oracle, torch, m, n, rows, off, src):
+    # DequantInt4SmallBatchTests.swift:66-119 shapes (incl. the 2-byte weight offset), config 1 (1408 x 2816),
+    # StreamingKernelIntegrationTests.swift:84-161 (64 x 128) and the 4,099-row head of
+    # LMHeadChainInt4Tests.swift:118-160; the weight comes from host memory or from device memory
+    g = oracle.seed_tree_key(0xE1 + rows, f"matrix-m{m}-n{n}-r{rows}-off{off}")
+    W, S, B = oracle.quantize_int4(g.uniform(-0.5, 0.5, m * n).reshape(m, n))
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, rows * n)).reshape(rows, n)
+    raw = np.concatenate([np.zeros(off, np.uint8), W.ravel()])
+    if src == "device":
+        mx = ctx.matrix(torch.from_numpy(raw).cuda(), _i16(torch, S), _i16(torch, B), w_byte_offset=off)
+    else:
+        mx = ctx.matrix(raw, S, B, w_byte_offset=off)
+    x = bf16_tensor(torch, xb)
+    y16 = bits_of(mx.gemv(x))
+    y32 = mx.gemv(x, f32_out=True).cpu().numpy()
+    for r in range(rows):
+        ref = oracle.gemv_int4_ref(W, S, B, oracle.bf16_to_float(xb[r]))
+        assert rel_err(y32[r], ref) < 5e-3, f"row {r}"         # Tolerance.fp16Reduction on the unrounded sum
+        assert rel_err(oracle.bf16_to_float(y16[r]), ref) < 1e-2, f"row {r}"
+        # the 16-bit output is the rounding of the fp32 output
+        assert np.array_equal(y16[r], oracle.bf16_bits(y32[r]))
+    # row r of a multi-row call equals the single-row call bit for bit (matchesSingleRowGEMVBitwise)
+    for r in range(rows):
+        single = mx.gemv(x[r:r + 1], f32_out=True).cpu().numpy()[0]
+        assert np.array_equal(single.view(np.uint32), y32[r].view(np.uint32)), f"row {r}"
+    mx.close()
+
+
+def test_matrix_equals_raw_layout_gemv(ctx, oracle, torch):
+    # the same weight through the reference-layout GEMV and through the resident tiles
+    m, n, rows = 512, 1408, 5
+    g = oracle.SplitMix64(77)
+    W, S, B = oracle.quantize_int4(g.uniform(-0.4, 0.4, m * n).reshape(m, n))
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, rows * n)).reshape(rows, n)
+    x = bf16_tensor(torch, xb)
+    mx = ctx.matrix(W, S, B)
+    a = mx.gemv(x, f32_out=True).cpu().numpy()
+    b = ctx.gemv_int4(torch.from_numpy(W).cuda(), _i16(torch, S), _i16(torch, B), x, f32_out=True).cpu().numpy()
+    assert rel_err(a, b) < 1e-4
+    mx.close()
+
+
+def _cpu_greedy(oracle, W, S, B, x_f32):
+    # cpuGreedy of LMHeadChainInt4Tests.swift:10-39 after its RMSNorm: first strictly larger dot wins
+    return int(np.argmax(oracle.gemv_int4_ref(W, S, B, x_f32)))
+
+
+def test_greedy_matches_cpu_reference(ctx, oracle, torch):
+    # rawGreedyMatchesCPUReference (LMHeadChainInt4Tests.swift:77-100): d = 64, v = 1024, same seed
+    d, v = 64, 1024
+    rng = oracle.SplitMix64(0x1A4E_4EAD_2026_0603)
+    hidden = rng.uniform(-1.0, 1.0, d)
+    rng.uniform(0.5, 1.5, d)                                # the norm weights of the Swift test: drawn, not used here
+    W, S, B = oracle.quantize_int4(np.stack([rng.uniform(-1.0, 1.0, d) for _ in range(v)]))
+    xb = oracle.bf16_bits(hidden)
+    mx = ctx.matrix(W, S, B, greedy=True)
+    got = int(mx.greedy(bf16_tensor(torch, xb[None, :]))[0])
+    logits = oracle.gemv_int4_ref(W, S, B, oracle.bf16_to_float(xb))
+    order = np.argsort(-logits)
+    assert logits[order[0]] - logits[order[1]] > 1e-4       # the case is not a near-tie
+    assert got == order[0] == _cpu_greedy(oracle, W, S, B, oracle.bf16_to_float(xb))
+    mx.close()
+
+
+def test_greedy_ties_and_non_finite(ctx, oracle, torch):
+    # tiesResolveToLowestIndex (LMHeadChainInt4Tests.swift:102-116): rows 17 and 311 carry the same weights
+    d, v = 64, 1024
+    hidden = np.array([0.2 + (i % 5) * 0.02 for i in range(d)], np.float32)
+    rows = np.full((v, d), -0.25, np.float32)
+    rows[17] = rows[311] = 1.0
+    W, S, B = oracle.quantize_int4(rows)
+    x = bf16_tensor(torch, oracle.bf16_bits(hidden)[None, :])
+    mx = ctx.matrix(W, S, B, greedy=True)
+    assert int(mx.greedy(x)[0]) == 17
+    mx.close()
+    # a row whose logit is +inf or NaN never wins (logit.metal:916-921): scale = +inf makes row 5 non-finite
+    S2, B2 = S.copy(), B.copy()
+    S2[5, 0] = 0x7F80
+    S2[9, 0] = 0x7FC0
+    mx = ctx.matrix(W, S2, B2, greedy=True)
+    logits = mx.gemv(x, f32_out=True).cpu().numpy()[0]
+    assert not np.isfinite(logits[5]) and not np.isfinite(logits[9])
+    assert int(mx.greedy(x)[0]) == 17
+    mx.close()
+
+
+def test_greedy_rows_large_head(ctx, oracle, torch):
+    # decode's shape (D = 2816) against a 4,099-row head with a tied pair, four rows at once
+    # (checkAndHotGuessMatchSingleRowHead, LMHeadChainInt4Tests.swift:118-160)
+    d, v, rows = 2816, 4099, 4
+    rng = oracle.SplitMix64(0xC4EC_4EAD)
+    Wf = rng.uniform(-1.0, 1.0, v * d).reshape(v, d)
+    Wf[4001] = Wf[1203]                                     # a tied pair: the lower index must win when it leads
+    W, S, B = oracle.quantize_int4(Wf)
+    xb = oracle.bf16_bits(rng.uniform(-1.0, 1.0, rows * d)).reshape(rows, d)
+    xb[2] = oracle.bf16_bits(oracle.dequantize_int4(W[1203:1204], S[1203:1204], B[1203:1204])[0])   # row 2 points at the pair
+    mx = ctx.matrix(W, S, B, greedy=True)
+    got = mx.greedy(bf16_tensor(torch, xb)).cpu().numpy()
+    for r in range(rows):
+        logits = oracle.gemv_int4_ref(W, S, B, oracle.bf16_to_float(xb[r]))
+        order = np.argsort(-logits, kind="stable")
+        if order[0] in (1203, 4001):
+            assert got[r] == 1203
+        else:
+            assert logits[order[0]] - logits[order[1]] > 1e-3 * abs(logits[order[0]])
+            assert got[r] == order[0]
+    assert got[2] == 1203
+    mx.close()
+
+
+def test_matrix_argument_errors(ctx, ff, oracle, torch):
+    W, S, B = oracle.quantize_int4(np.zeros((32, 64), np.float32))
+    with pytest.raises(ff.FieldfareError, match="at most"):
+        big = np.zeros((32, 2880 // 2), np.uint8)
+        ctx.matrix(big, np.zeros((32, 45), np.uint16), np.zeros((32, 45), np.uint16))
+    mx = ctx.matrix(W, S, B)
+    x = torch.zeros((1, 64), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ff.FieldfareError, match="greedy scratch"):
+        mx.greedy(x)
+    with pytest.raises(ff.FieldfareError, match="outside 1...16"):
+        mx.gemv(torch.zeros((17, 64), dtype=torch.bfloat16, device="cuda"))
+    mx.close()
