@@ -88,12 +88,12 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
     const uint32_t per = (n_groups + kKSplit - 1) / kKSplit;
     const uint32_t g0 = min(ks * per, n_groups), g1 = min(n_groups, g0 + per), ng = g1 - g0;
     const uint32_t g_last = g1 > g0 ? g1 - 1 : n_groups - 1;
-    const size_t tile_row = (size_t)n_groups * kTileBytes, scale_row = (size_t)n_groups * kTileScaleBytes;
+    const TileSource src = make_tile_source(tiles, (size_t)n_tiles * n_groups * kTileBytes, scales,
+                                            (size_t)n_tiles * n_groups * kTileScaleBytes);
 
     WeightRing ring;
 #pragma unroll
-    for (int u = 0; u < kRing; ++u)
-        ring_fill(ring, u, tiles + rb0 * tile_row, scales + rb0 * scale_row, min(g0 + u, g_last), lane);
+    for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb0 * n_groups + min(g0 + u, g_last), lane);
     const uint16_t *xrow = x + (size_t)min(j, rows - 1) * x_stride + 8 * jq;
     uint4 x0[kRing], x1[kRing];
 #pragma unroll
@@ -108,14 +108,13 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
     uint16_t *y16 = reinterpret_cast<uint16_t *>(y_);
 
     for (uint32_t rb = rb0; rb < rb1; ++rb) {
-        const uint32_t rbn = min(rb + 1, rb1 - 1);
-        const uint8_t *nt = tiles + rbn * tile_row, *ns = scales + rbn * scale_row;
+        const uint32_t next_row = min(rb + 1, rb1 - 1) * n_groups;
         TwoStreamAcc tot;
         tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, nt, ns, min(g0 + u, g_last), lane);
+            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min(g0 + u, g_last), lane);
         const int buf = (rb - rb0) & 1;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {

@@ -82,6 +82,9 @@ __device__ __forceinline__ uint32_t build_plan(PlanScratch &ps, const uint32_t *
         if (tid >= total) plan_out->slots[tid].n = 0;
         if (tid == 0) plan_out->n_live = total;
     }
+    // every thread read the same four counts from LDS; say so, or all that derives from the total (slot,
+    // row ranges, loop bounds, load offsets) is treated as per-lane data and computed in vector registers
+    total = __builtin_amdgcn_readfirstlane(total);
     my_slot = slot_from_total(total);
     __syncthreads();
     if (tid < n_routes && e != 0xFFFFFFFFu) {
@@ -305,14 +308,12 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     const uint32_t per = (g.gd + kKSplit - 1) / kKSplit;
     const uint32_t g0 = min(ks * per, g.gd), g1 = min(g.gd, g0 + per), ng = g1 - g0;
     const uint32_t g_last = g1 > g0 ? g1 - 1 : g.gd - 1;
-    const uint8_t *tiles = expert_base + g.gu_tiles_off;
-    const uint8_t *scales = expert_base + g.gu_scales_off;
-    const size_t tile_row = (size_t)g.gd * kTileBytes, scale_row = (size_t)g.gd * kTileScaleBytes;
+    const TileSource gu_src = make_tile_source(expert_base + g.gu_tiles_off, (size_t)g.gu_rb * g.gd * kTileBytes,
+                                               expert_base + g.gu_scales_off, (size_t)g.gu_rb * g.gd * kTileScaleBytes);
 
     WeightRing ring;
 #pragma unroll
-    for (int u = 0; u < kRing; ++u)
-        ring_fill(ring, u, tiles + rb0 * tile_row, scales + rb0 * scale_row, min(g0 + u, g_last), lane);
+    for (int u = 0; u < kRing; ++u) ring_fill(ring, u, gu_src, rb0 * g.gd + min(g0 + u, g_last), lane);
     // token operand of this wave's K-slice: token slot j (clamped), k-quarter jq of every group
     const uint32_t tok = slot.routes[min(j, n - 1)] / top_k;
     const uint16_t *xrow = x + (size_t)tok * x_stride + 8 * jq;
@@ -329,14 +330,13 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
 
     for (uint32_t rb = rb0; rb < rb1; ++rb) {
         // the refill targets the next row block; past the last one it re-reads the current tiles (cache hits)
-        const uint32_t rbn = min(rb + 1, rb1 - 1);
-        const uint8_t *nt = tiles + rbn * tile_row, *ns = scales + rbn * scale_row;
+        const uint32_t next_row = min(rb + 1, rb1 - 1) * g.gd;
         TwoStreamAcc tot;
         tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, nt, ns, min(g0 + u, g_last), lane);
+            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, gu_src, next_row + min(g0 + u, g_last), lane);
         const int buf = (rb - rb0) & 1;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -352,93 +352,6 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
         }
         // one rounding to 16 bits, gate and up themselves stay fp32 (moe.metal:496)
         if (my_ts < n) acts[(size_t)my_route * g.f + rb * kTileRows + j] = f32_to_bf16(gelu_tanh_fast(ga) * ub);
-    }
-}
-
-// down projection, persistent. grid = (blocks); the blocks are dealt to the live experts. A block stages
-// its expert's (<= 16) activation rows in LDS once (rows padded by 16 bytes so that the 16 rows of a
-// fragment read fall into different banks) and its waves walk disjoint ranges of 32-row blocks. With the
-// token operand in LDS a wave needs few registers, so three blocks fit a CU and the chip keeps most of
-// the layer's down weights in flight at once.
-constexpr int kXsStride = kRing * kGroup + 8;
-
-template <bool OUT_BF16>
-__global__ __launch_bounds__(256, 2) void skinny_down_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
-                                                                 const VerifyPlan *__restrict__ plan,
-                                                                 const uint16_t *__restrict__ acts,
-                                                                 float *__restrict__ partials_f32,
-                                                                 uint16_t *__restrict__ partials_bf16) {
-    __shared__ __align__(16) uint16_t xs[kMaxRows][kXsStride];
-    const uint32_t n_live = plan->n_live;
-    if (n_live == 0) return;
-    const uint32_t blocks_per_slot = max(1u, min((g.dn_rbp + 3) / 4, gridDim.x / n_live));
-    const uint32_t slot_id = blockIdx.x / blocks_per_slot;
-    if (slot_id >= n_live) return;
-    uint32_t b0, b1, rb0, rb1;
-    split_range(g.dn_rbp, blocks_per_slot, blockIdx.x % blocks_per_slot, b0, b1);
-    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    split_range(b1 - b0, 4, wave, rb0, rb1);
-    rb0 += b0;
-    rb1 += b0;
-    const PlanSlot &slot = plan->slots[slot_id];
-    const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
-    const uint32_t j = lane & 15, jq = lane >> 4;
-    const uint8_t *expert_base = arena_layer + (size_t)__builtin_amdgcn_readfirstlane(slot.expert) * g.expert_bytes;
-    const uint8_t *tiles = expert_base + g.dn_tiles_off;
-    const uint8_t *scales = expert_base + g.dn_scales_off;
-    const size_t tile_row = (size_t)g.gf * kTileBytes, scale_row = (size_t)g.gf * kTileScaleBytes;
-    const uint32_t ng = g.gf, g_last = g.gf - 1;
-    const uint32_t rb_first = min(rb0, g.dn_rbp - 1);       // a wave without row blocks still loads valid memory
-
-    WeightRing ring;
-#pragma unroll
-    for (int u = 0; u < kRing; ++u)
-        ring_fill(ring, u, tiles + rb_first * tile_row, scales + rb_first * scale_row, min((uint32_t)u, g_last), lane);
-    // stage the activation rows while the first tiles are on their way
-    // (columns past F, read by the groups of a short K that enter with zero scales, are cleared)
-    constexpr uint32_t kChunksPerRow = kRing * kGroup / 8;
-    const uint32_t live_chunks = g.f / 8;
-    for (uint32_t i = threadIdx.x; i < n * kChunksPerRow; i += 256) {
-        const uint32_t row = i / kChunksPerRow, c = i % kChunksPerRow;
-        uint4 v = {0, 0, 0, 0};
-        if (c < live_chunks) v = *reinterpret_cast<const uint4 *>(acts + (size_t)slot.routes[row] * g.f + c * 8);
-        *reinterpret_cast<uint4 *>(&xs[row][c * 8]) = v;
-    }
-    lds_barrier();
-    const uint16_t *xrow = &xs[min(j, n - 1)][8 * jq];
-    size_t out_base[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) out_base[r] = (size_t)slot.routes[min(4 * jq + r, n - 1)] * g.d;
-
-    for (uint32_t rb = rb0; rb < rb1; ++rb) {
-        const uint32_t rbn = min(rb + 1, rb1 - 1);
-        const uint8_t *nt = tiles + rbn * tile_row, *ns = scales + rbn * scale_row;
-        TwoStreamAcc tot;
-        tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
-        tot.b = tot.a;
-        // the token operand is re-read from LDS for every row block: the clobber keeps the compiler from
-        // hoisting 22 fragment reads out of the loop into registers it does not have
-        asm volatile("" ::: "memory");
-#pragma unroll
-        for (int u = 0; u < kRing; ++u) {
-            const uint4 x0 = *reinterpret_cast<const uint4 *>(xrow + u * kGroup);
-            const uint4 x1 = *reinterpret_cast<const uint4 *>(xrow + u * kGroup + 32);
-            ring_step(ring, u, (uint32_t)u < ng, x0, x1, tot, nt, ns, min((uint32_t)u, g_last), lane);
-            if (u & 1) __builtin_amdgcn_sched_barrier(0);   // bound how many groups the scheduler unpacks ahead
-        }
-        const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            if (4 * jq + r < n) {
-                if (OUT_BF16) {
-                    partials_bf16[out_base[r] + row_a] = f32_to_bf16(tot.a[r]);
-                    partials_bf16[out_base[r] + row_b] = f32_to_bf16(tot.b[r]);
-                } else {
-                    partials_f32[out_base[r] + row_a] = tot.a[r];
-                    partials_f32[out_base[r] + row_b] = tot.b[r];
-                }
-            }
-        }
     }
 }
 
@@ -514,16 +427,10 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_GATE_UP);
-    const bool dn_persistent = false;
-    const dim3 dn_grid = dn_persistent ? dim3(max(slots, min(2 * n_cus, slots * ((g.dn_rbp + 3) / 4))))
-                                       : dim3((g.dn_rbp + 3) / 4, slots);
+    const dim3 dn_grid((g.dn_rbp + 3) / 4, slots);
 #define FFMOE_DOWN(BF)                                                                                          \
-    if (dn_persistent)                                                                                          \
-        hipLaunchKernelGGL(skinny_down_persistent<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,    \
-                           partials_f32, partials_bf16);                                                        \
-    else                                                                                                        \
-        hipLaunchKernelGGL(skinny_down_kernel<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,        \
-                           partials_f32, partials_bf16)
+    hipLaunchKernelGGL(skinny_down_kernel<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts, partials_f32, \
+                       partials_bf16)
     if (partials_bf16) {
         FFMOE_DOWN(true);
         timer->mark(s, FFMOE_K_DOWN);

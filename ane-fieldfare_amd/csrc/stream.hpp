@@ -19,26 +19,49 @@ struct WeightRing {
     uint2 s[kRing];
 };
 
-// `tiles` / `scales` are wave-uniform (scalar registers); the lane part is a 32-bit offset, so every ring load is
-// one instruction with a scalar base and no per-load 64-bit address arithmetic.
-__device__ __forceinline__ void ring_fill(WeightRing &ring, int u, const uint8_t *tiles, const uint8_t *scales,
-                                          uint32_t g_clamped, uint32_t lane) {
-    const uint8_t *tg = tiles + (size_t)g_clamped * kTileBytes, *sg = scales + (size_t)g_clamped * kTileScaleBytes;
-    ring.t[u] = *reinterpret_cast<const uint4 *>(tg + lane * 16u);
-    ring.s[u] = *reinterpret_cast<const uint2 *>(sg + (lane & 15u) * 8u);
+// Where a wave's tiles come from: two buffer descriptors (scalar registers). A ring load is then a single
+// buffer_load with the lane's fixed 32-bit offset and a scalar byte offset - no per-load 64-bit address
+// arithmetic in vector registers, which otherwise costs two registers per load in flight - and a load
+// past the end of the region returns zero instead of faulting.
+struct TileSource {
+    __amdgpu_buffer_rsrc_t tiles, scales;
+};
+
+__device__ __forceinline__ TileSource make_tile_source(const uint8_t *tiles, size_t tile_bytes, const uint8_t *scales,
+                                                       size_t scale_bytes) {
+    TileSource src;
+    src.tiles = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(tiles), 0, (int)(uint32_t)tile_bytes, 0x00020000);
+    src.scales = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(scales), 0, (int)(uint32_t)scale_bytes, 0x00020000);
+    return src;
+}
+
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+// `tile_index` = index of the 1 KiB tile inside the region (wave-uniform).
+__device__ __forceinline__ void ring_fill(WeightRing &ring, int u, const TileSource &src, uint32_t tile_index,
+                                          uint32_t lane) {
+    // the index is wave-uniform by contract; pinning it to a scalar register spares the waterfall loop the
+    // compiler emits whenever it happened to compute a uniform value in a vector register
+    tile_index = __builtin_amdgcn_readfirstlane(tile_index);
+    const u32x4_t t = __builtin_amdgcn_raw_buffer_load_b128(src.tiles, (int)(lane * 16u), (int)(tile_index * kTileBytes), 0);
+    const u32x2_t s = __builtin_amdgcn_raw_buffer_load_b64(src.scales, (int)((lane & 15u) * 8u),
+                                                           (int)(tile_index * kTileScaleBytes), 0);
+    ring.t[u] = make_uint4(t.x, t.y, t.z, t.w);
+    ring.s[u] = make_uint2(s.x, s.y);
 }
 
 // Consume ring slot u against the resident token operand, then start the load that refills the slot.
 __device__ __forceinline__ void ring_step(WeightRing &ring, int u, bool live, const uint4 &x0, const uint4 &x1,
-                                          TwoStreamAcc &tot, const uint8_t *next_tiles, const uint8_t *next_scales,
-                                          uint32_t next_g, uint32_t lane) {
+                                          TwoStreamAcc &tot, const TileSource &src, uint32_t next_tile_index,
+                                          uint32_t lane) {
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     const uint4 ones_bits = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
     const uint4 tile = ring.t[u];
     uint2 sc = ring.s[u];
     if (!live) sc = make_uint2(0u, 0u);
-    ring_fill(ring, u, next_tiles, next_scales, next_g, lane);
+    ring_fill(ring, u, src, next_tile_index, lane);
     const bf16x8 a0 = __builtin_bit_cast(bf16x8, x0), a1 = __builtin_bit_cast(bf16x8, x1);
     f32x4 acc_a = mfma16(a0, unpack8_offset128(tile.x), zero);
     acc_a = mfma16(a1, unpack8_offset128(tile.y), acc_a);
