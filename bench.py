@@ -69,6 +69,10 @@ def main():
     ap.add_argument("--prefill-tokens", type=int, default=3072, help="0 skips the prefill leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode (T = 1) leg")
+    ap.add_argument("--no-gemv", action="store_true", help="skip the INT4 GEMV legs (config 1 and the LM head)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="also run BASELINE.json config 5: 8,192-token Zipf prefill over all layers, then 256 decode "
+                         "steps as 16 verify blocks with the LM head once per block")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only; --gpus must be 1 "
@@ -89,7 +93,7 @@ def main():
     assert payload == EXPERT_BYTES
     ff_off = ff.Offsets(*offsets.as_tuple())
 
-    ctx = ff.Context(D, F, E, K, n_layers=L, max_tokens=4096)
+    ctx = ff.Context(D, F, E, K, n_layers=L, max_tokens=8192 if args.sweep else 4096)
     host_layer0 = None
     routers = []
     for layer in range(L):
@@ -223,6 +227,111 @@ def main():
                                 "unit": "TFLOP/s", "frac": round((flops_gu + flops_dn) / gemm_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                                 "traffic": None}}
 
+    def timed(fn, reps, warm=3):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        t0_ = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0_) / reps
+
+    # INT4 GEMV: BASELINE.json config 1 ([1408 x 2816], one input row) and the LM head of config 5
+    # ([262144 x 2816]) as resident matrices; synthetic weights as in synth_layer_gpu
+    head = None
+    if not args.no_gemv:
+        def synth_matrix(m):
+            W = torch.randint(0, 256, (m, D // 2), dtype=torch.uint8, device="cuda", generator=gen)
+            S = (torch.randn((m, D // 64), device="cuda", generator=gen) * 0.01).abs().to(torch.bfloat16)
+            Bq = (-8.0 * S.float() + torch.randn((m, D // 64), device="cuda", generator=gen) * 1e-3).to(torch.bfloat16)
+            return W, S, Bq
+        gemv = {}
+        W1, S1, B1 = synth_matrix(2 * F)
+        m1 = ctx.matrix(W1, S1, B1)
+        bytes1 = 2 * F * D // 2 + 2 * (2 * F) * (D // 64) * 2
+        x1row = x[:1].contiguous()
+        t_res = timed(lambda: m1.gemv(x1row), 200)
+        t_raw = timed(lambda: ctx.gemv_int4(W1, S1, B1, x1row), 200)
+        gemv["config1_1408x2816"] = {"resident_us": round(t_res * 1e6, 2), "resident_GBs": round(bytes1 / t_res / 1e9, 1),
+                                     "reference_layout_us": round(t_raw * 1e6, 2), "bytes": bytes1,
+                                     "note": "host-timed back-to-back calls: launch latency, not bandwidth, bounds a 2.2 MB GEMV"}
+        m1.close()
+        V = 262144
+        Wh, Sh, Bh = synth_matrix(V)
+        head = ctx.matrix(Wh, Sh, Bh, greedy=True)
+        del Wh, Sh, Bh
+        torch.cuda.empty_cache()
+        head_bytes = V * D // 2 + 2 * V * (D // 64) * 2
+        for rows in (1, 16):
+            xr = x[:rows].contiguous()
+            tg = timed(lambda: head.gemv(xr, f32_out=True), 20)
+            gemv[f"lm_head_262144x2816_rows{rows}"] = {"us": round(tg * 1e6, 1), "GBs": round(head_bytes / tg / 1e9, 1),
+                                                        "pct_hbm_peak": round(100 * head_bytes / tg / 1e9 / HBM_PEAK_GBS, 1)}
+        tg = timed(lambda: head.greedy(x), 20)
+        gemv["lm_head_greedy_rows16_us"] = round(tg * 1e6, 1)
+        extra["gemv"] = gemv
+
+    # BASELINE.json config 5: all layers resident, one 8,192-token prefill with Zipf(1.1) routing imposed on
+    # the experts, then 256 decode steps as 16 verify blocks of 16 tokens, the LM head once per block
+    sweep = None
+    if args.sweep:
+        TS = 8192
+        zr = np.random.default_rng(5)
+        pz = 1.0 / np.arange(1, E + 1) ** 1.1
+        pz /= pz.sum()
+        perm = zr.permutation(E)
+        zidx = np.stack([perm[zr.choice(E, K, replace=False, p=pz)] for _ in range(TS)]).astype(np.int32)
+        zw = zr.random((TS, K)).astype(np.float32)
+        zw = zw / zw.sum(1, keepdims=True)
+        xs_ = torch.from_numpy(oracle.bf16_bits(zr.normal(0, 1, (TS, D)).astype(np.float32)).view(np.int16)).cuda().view(torch.bfloat16)
+        zi = torch.from_numpy(zidx).cuda()
+        zwt = torch.from_numpy(oracle.bf16_bits(zw).view(np.int16)).cuda().view(torch.bfloat16)
+        ys_ = torch.empty((TS, D), dtype=torch.bfloat16, device="cuda")
+        pzx, pzi, pzw, pzy = (C.c_void_p(t_.data_ptr()) for t_ in (xs_, zi, zwt, ys_))
+
+        def prefill_all():
+            for layer in range(L):
+                rc = Lib.ffmoe_prefill(h, stream, layer, pzx, D, TS, pzi, pzw, pzy, C.byref(err))
+                if rc:
+                    raise RuntimeError(err.value)
+        t_pf = timed(prefill_all, 2, warm=1)
+        counts_z = np.bincount(zidx.ravel(), minlength=E)
+        ctx.set_profiling(True)
+        ctx.profile(reset=True)
+        prefill_all()
+        zprof = ctx.profile(reset=True)
+        ctx.set_profiling(False)
+
+        def decode_blocks():
+            for _ in range(16):
+                for layer in range(L):
+                    step(layer)
+                if head is not None:
+                    head.greedy(x)
+        t_dec = timed(decode_blocks, 2, warm=1)
+        ctx.set_profiling(True)
+        ctx.profile(reset=True)
+        decode_blocks()
+        dprof = ctx.profile(reset=True)
+        ctx.set_profiling(False)
+        flops_pf = L * TS * K * 2.0 * (3 * F * D)
+        sweep = {
+            "layers": L, "prefill_tokens": TS, "routing": "Zipf s=1.1 over a permuted expert order, 8 distinct experts per token",
+            "pairs_per_expert_min": int(counts_z.min()), "pairs_per_expert_max": int(counts_z.max()),
+            "prefill_ms_all_layers": round(t_pf * 1e3, 2), "prefill_tok_per_s_per_layer": round(TS * L / t_pf, 1),
+            "prefill_expert_TFLOPs": round(flops_pf / t_pf / 1e12, 1),
+            "prefill_kernel_ms": {k_: round(v[0], 3) for k_, v in zprof.items()},
+            "decode_steps": 256, "decode_ms_256_steps": round(t_dec * 1e3, 2),
+            "decode_us_per_block_layer": round(t_dec * 1e6 / (16 * L), 2),
+            "decode_kernel_ms": {k_: round(v[0], 3) for k_, v in dprof.items()},
+            "lm_head_included": head is not None,
+            "note": "router of the prefill is imposed (not run); decode blocks run router + experts per layer and the "
+                    "LM-head greedy choice once per block; times are host-timed whole phases, kernel_ms are HIP-event sums",
+        }
+    if head is not None:
+        head.close()
+
     cpu = None
     if not args.no_cpu:
         pool = oracle.ExpertPool(host_layer0, offsets, STRIDE, D, F)
@@ -271,6 +380,7 @@ def main():
         "prefill": prefill,
         "cpu_baseline": cpu,
         "extra": extra,
+        "sweep": sweep,
     }
     print(json.dumps(out))
     ctx.close()
