@@ -324,6 +324,49 @@ private:
     Context &c_;
 };
 
+// LMHeadChainInt4 (Kernels/Fusions/LMHeadChainInt4.swift:57-139,225-284): owns the head's INT4 table for its
+// lifetime - here the re-tiled resident copy - plus the fp32 logits scratch, and returns greedy tokens for
+// 1...maxGreedyRows normalised hidden rows with one pass over the table. The RMSNorm the Swift chain runs
+// first is a separate operator there too (rms.encodeBF16W) and stays with the caller.
+class LMHeadChainInt4 {
+public:
+    static constexpr int maxGreedyRows = 16;
+    // weights uint8 [vocab][d/2], scales/biases bf16 [vocab][d/64], in host or device memory
+    LMHeadChainInt4(Context &c, const uint8_t *weights, const uint16_t *scales, const uint16_t *biases, uint32_t d, uint32_t vocab)
+        : d_(d), vocab_(vocab) {
+        if (d % 64) throw std::invalid_argument("d must be a multiple of 64");
+        char *err = nullptr;
+        check(ffmoe_matrix_create(c.raw(), weights, scales, biases, vocab, d, 1, &mx_, &err), err);
+    }
+    ~LMHeadChainInt4() { ffmoe_matrix_destroy(mx_); }
+    LMHeadChainInt4(const LMHeadChainInt4 &) = delete;
+    LMHeadChainInt4 &operator=(const LMHeadChainInt4 &) = delete;
+    // encodeGreedyDecode (LMHeadChainInt4.swift:225-284): one row
+    void encodeGreedyDecode(void *stream, const uint16_t *normedHidden, uint32_t *outToken) {
+        encodeGreedyRows(stream, normedHidden, d_, 1, outToken);
+    }
+    // encodeGreedyRows (LMHeadChainInt4.swift:94-139)
+    void encodeGreedyRows(void *stream, const uint16_t *normedHidden, uint32_t hiddenStrideElements, int rowCount,
+                          uint32_t *outTokens) {
+        if (rowCount <= 0 || rowCount > maxGreedyRows) throw std::invalid_argument("rowCount outside 1...16");
+        char *err = nullptr;
+        check(ffmoe_matrix_greedy(mx_, stream, normedHidden, hiddenStrideElements, (uint32_t)rowCount, outTokens, &err), err);
+    }
+    // fp32 logits of the same rows (rowsProjection.encodeRows with .f16ToF32, LMHeadChainInt4.swift:122-131)
+    void encodeLogitsRows(void *stream, const uint16_t *normedHidden, uint32_t hiddenStrideElements, int rowCount, float *logits,
+                          uint32_t logitsStrideElements) {
+        if (rowCount <= 0 || rowCount > maxGreedyRows) throw std::invalid_argument("rowCount outside 1...16");
+        char *err = nullptr;
+        check(ffmoe_matrix_gemv(mx_, stream, normedHidden, hiddenStrideElements, (uint32_t)rowCount, logits, logitsStrideElements, 1,
+                                &err), err);
+    }
+    uint32_t vocab() const { return vocab_; }
+
+private:
+    ffmoe_matrix *mx_ = nullptr;
+    uint32_t d_, vocab_;
+};
+
 // ---------------------------------------------------------------------------------------------------
 // Guest plugin and supervisor (Runtime/Supervisor/DeviceSupervisor.swift:5-125).
 // ---------------------------------------------------------------------------------------------------

@@ -194,6 +194,31 @@ int main() {
     errorStats(yg, refg, rel, cosine);
     EXPECT(rel <= 1e-2);
 
+    // --- LMHeadChainInt4 over the same matrix as a 64-token "vocabulary": greedy token == CPU argmax ---
+    {
+        LMHeadChainInt4 head(ctx, pool.data() + off.gate_w, reinterpret_cast<uint16_t *>(pool.data() + off.gate_s),
+                             reinterpret_cast<uint16_t *>(pool.data() + off.gate_b), d, f);
+        uint32_t *dTok = nullptr;
+        HIP(hipMalloc(reinterpret_cast<void **>(&dTok), 4 * sizeof(uint32_t)));
+        head.encodeGreedyRows(stream, dx, d, 3, dTok);
+        HIP(hipStreamSynchronize(stream));
+        auto tok = toHost(dTok, 3);
+        for (int r = 0; r < 3; ++r) {
+            std::vector<float> xr(d), ref(f);
+            for (int i = 0; i < d; ++i) xr[i] = ffo_bf16_to_float(x[(size_t)r * d + i]);
+            ffo_gemv_int4_ref(pool.data() + off.gate_w, reinterpret_cast<uint16_t *>(pool.data() + off.gate_s),
+                              reinterpret_cast<uint16_t *>(pool.data() + off.gate_b), f, d, xr.data(), ref.data());
+            uint32_t best = 0;
+            for (int i = 1; i < f; ++i)
+                if (ref[i] > ref[best]) best = i;
+            EXPECT(tok[r] == best);
+        }
+        bool threwRows = false;
+        try { head.encodeGreedyRows(stream, dx, d, 17, dTok); } catch (const std::invalid_argument &) { threwRows = true; }
+        EXPECT(threwRows);
+        HIP(hipFree(dTok));
+    }
+
     std::printf(failures ? "%d FAILURES\n" : "host gpu ok\n", failures);
     return failures ? 1 : 0;
 }
