@@ -176,7 +176,8 @@ __global__ __launch_bounds__(256) void router_small_kernel(const void *__restric
 // Prefill router logits: a register-tiled fp32 GEMM that keeps the pinned order. A block owns a tile of
 // 8 tokens x 8 experts; its four waves are the four sub-accumulators, each walking its own k-blocks with
 // the next block's operands already in flight, so every x and W load feeds 8 rows of fmaf. The partials
-// meet in LDS, each wave then finishes 16 of the 64 outputs: (s0 + s1) + (s2 + s3) per lane and the
+// meet in LDS (pairwise first, which halves the space and lets three blocks share a CU), each wave
+// then finishes 16 of the 64 outputs: (s0 + s1) + (s2 + s3) per lane and the
 // xor-butterfly done as a halving exchange (a lane keeps half of its values and receives the partner's
 // matching half; fp addition is commutative, so every sum has the same operands as the full butterfly).
 // Blocks are numbered so that all expert groups of one token group run on the same XCD and share its L2.
@@ -191,7 +192,7 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict
                                                           uint32_t t, uint32_t n_experts, uint32_t d,
                                                           uint32_t n_egroups, uint32_t n_tgroups,
                                                           float *__restrict__ logits) {
-    __shared__ float s_part[4][kTileTok * kTileExp][64];
+    __shared__ float s_part[2][kTileTok * kTileExp][64];
     const uint32_t lane = threadIdx.x & 63, s = threadIdx.x >> 6;
     const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const uint32_t tg = (slot / n_egroups) * 8 + xcd, eg = slot % n_egroups;
@@ -260,10 +261,23 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict
             }
         }
     }
+    // (s0 + s1) and (s2 + s3) first, each in the even wave of the pair, through two 16 KiB regions
+    if (s & 1) {
 #pragma unroll
-    for (int r = 0; r < kTileTok; ++r)
+        for (int r = 0; r < kTileTok; ++r)
 #pragma unroll
-        for (int c = 0; c < kTileExp; ++c) s_part[s][r * kTileExp + c][lane] = acc[r][c];
+            for (int c = 0; c < kTileExp; ++c) s_part[s >> 1][r * kTileExp + c][lane] = acc[r][c];
+    }
+    __syncthreads();
+    if (!(s & 1)) {
+#pragma unroll
+        for (int r = 0; r < kTileTok; ++r)
+#pragma unroll
+            for (int c = 0; c < kTileExp; ++c) {
+                float *cell = &s_part[s >> 1][r * kTileExp + c][lane];
+                *cell = acc[r][c] + *cell;
+            }
+    }
     __syncthreads();
 
     // wave s finishes outputs 16 s .. 16 s + 15
@@ -271,7 +285,7 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict
 #pragma unroll
     for (int o = 0; o < 16; ++o) {
         const uint32_t q = 16 * s + o;
-        v[o] = (s_part[0][q][lane] + s_part[1][q][lane]) + (s_part[2][q][lane] + s_part[3][q][lane]);
+        v[o] = s_part[0][q][lane] + s_part[1][q][lane];
     }
     // halving exchange: after the step with mask m the lane keeps the outputs whose index bit matches
     // its own lane bit; four steps leave output (lane >> 2) & 15, two plain butterfly steps finish it.
