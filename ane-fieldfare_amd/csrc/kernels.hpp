@@ -47,24 +47,31 @@ struct VerifyPlan {
 // The counterpart of the reference's traced compute encoders (Infrastructure/Metal/GPUTrace.swift:19-115).
 struct KernelTimer {
     bool on = false;
-    hipEvent_t ev[12] = {};
-    int ids[12] = {};
+    hipEvent_t ev[14] = {};      // ev[0], ev[1]: an empty interval; ev[1] also opens the first kernel's interval
+    int ids[14] = {};
     int n = 0;
     double ms[FFMOE_PROFILE_SLOTS] = {};
     uint64_t launches[FFMOE_PROFILE_SLOTS] = {};
     void begin(hipStream_t s) {
         n = 0;
-        if (on) (void)hipEventRecord(ev[0], s);
+        if (!on) return;
+        (void)hipEventRecord(ev[0], s);
+        ids[0] = FFMOE_K_EVENT_GAP;
+        (void)hipEventRecord(ev[1], s);
+        n = 1;
     }
     // call right after launching kernel `id`
     void mark(hipStream_t s, int id) {
-        if (!on || n >= 11) return;
+        if (!on || n >= 13) return;
         ids[n] = id;
         (void)hipEventRecord(ev[++n], s);
     }
     // waits for the stream: profiling mode trades asynchrony for per-kernel times
     void finish() {
-        if (!on || n == 0) return;
+        if (!on || n <= 1) {
+            n = 0;
+            return;
+        }
         (void)hipEventSynchronize(ev[n]);
         for (int i = 0; i < n; ++i) {
             float t = 0.f;

@@ -47,9 +47,10 @@ EXPORTS = [
     "ffmoe_matrix_greedy",
 ]
 
-PROFILE_SLOTS = 12
+PROFILE_SLOTS = 16
 KERNEL_NAMES = ["router_logits", "router_topk", "plan", "gate_up", "down", "combine", "prefill_sort",
-                "prefill_gate_up", "prefill_down", "prefill_combine", "gemv", "argmax"]
+                "prefill_gate_up", "prefill_down", "prefill_combine", "gemv", "argmax", "event_gap", "reserved13",
+                "reserved14", "reserved15"]
 
 
 class Profile(C.Structure):

@@ -34,6 +34,10 @@ GATE_UP_BYTES = 2_230_272                # the share the gate/up kernel streams 
 DOWN_BYTES = 1_115_136
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this same workload (seeded, so
+# the launches are the same ones), scaled by a plain 1 GiB copy: see profiles/hbm_traffic_verify16_prefill3072.txt
+TRAFFIC_GATE_UP_VERIFY16 = 113.1e6 + 0.3e6
+TRAFFIC_PREFILL_GEMMS_3072 = (439.9e6 + 34.6e6) + (181.4e6 + 138.4e6)
 TOKEN_CORRELATION = 0.45                 # shared component of the block's tokens -> 40-60 distinct experts
 
 
@@ -70,6 +74,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode (T = 1) leg")
     ap.add_argument("--no-gemv", action="store_true", help="skip the INT4 GEMV legs (config 1 and the LM head)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 1 GiB device-to-device copy three times: the known-size kernel that "
+                         "FETCH_SIZE / WRITE_SIZE readings of a rocprofv3 --pmc run are scaled by")
     ap.add_argument("--sweep", action="store_true",
                     help="also run BASELINE.json config 5: 8,192-token Zipf prefill over all layers, then 256 decode "
                          "steps as 16 verify blocks with the LM head once per block")
@@ -142,6 +149,15 @@ def main():
     bytes_total = sum(live[i % L] for i in range(args.steps)) * EXPERT_BYTES
     value = bytes_total / elapsed / 1e9
 
+    if args.copy_probe:
+        src_c = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst_c = torch.empty_like(src_c)
+        for _ in range(3):
+            dst_c.copy_(src_c)
+        torch.cuda.synchronize()
+        del src_c, dst_c
+        torch.cuda.empty_cache()
+
     # per-kernel times (HIP events on the launch stream) for the same steps
     ctx.set_profiling(True)
     ctx.profile(reset=True)
@@ -149,14 +165,22 @@ def main():
         step(i % L)
     prof = ctx.profile(reset=True)
     ctx.set_profiling(False)
-    gu_ms, gu_n = prof["gate_up"]
-    kernel_us = {k: round(v[0] / v[1] * 1e3, 2) for k, v in prof.items()}
+    # An event record costs the stream a few microseconds. The library measures an empty interval (two
+    # records with nothing between them, once per call); a kernel's interval carries half of that - one
+    # record's worth - on top of the kernel's own duration, which is what rocprofv3 --kernel-trace shows
+    # (gate/up: 33.1 us raw, 5.1 us empty interval, 30.5 us corrected, 30.3 us in the trace).
+    gap_ms = 0.5 * prof["event_gap"][0] / prof["event_gap"][1] if "event_gap" in prof else 0.0
+
+    def kernel_times(pr):
+        return {k_: round((v[0] / v[1] - gap_ms) * 1e3, 2) for k_, v in pr.items() if k_ != "event_gap"}
+    kernel_us = kernel_times(prof)
+    gu_ms = prof["gate_up"][0] - gap_ms * prof["gate_up"][1]
     live_sum = sum(live[i % L] for i in range(args.steps))
     if "down" in prof:
         # two launches: gate/up is the dominant kernel
         dominant = "skinny_gate_up_persistent"
         achieved = live_sum * GATE_UP_BYTES / (gu_ms * 1e-3) / 1e9
-        down_gbs = live_sum * DOWN_BYTES / (prof["down"][0] * 1e-3) / 1e9
+        down_gbs = live_sum * DOWN_BYTES / ((prof["down"][0] - gap_ms * prof["down"][1]) * 1e-3) / 1e9
     else:
         # gate/up and down share one launch (its time sits in the gate_up slot): all expert bytes
         dominant = "skinny_gate_up_persistent<1> (gate/up + down in one launch)"
@@ -164,7 +188,7 @@ def main():
         down_gbs = None
 
     # secondary figures: decode step (T = 1) and config-1 GEMV
-    extra = {}
+    extra = {"event_record_us": round(gap_ms * 1e3, 2)}
     x1 = x[:1].contiguous()
     px1 = C.c_void_p(x1.data_ptr())
 
@@ -215,17 +239,18 @@ def main():
             pstep(i % L)
         pprof = ctx.profile(reset=True)
         ctx.set_profiling(False)
-        pk_us = {k: round(v[0] / v[1] * 1e3, 2) for k, v in pprof.items()}
+        pk_us = kernel_times(pprof)
         flops_gu = n_pairs * 2.0 * (2 * F * D)
         flops_dn = n_pairs * 2.0 * (D * F)
-        gemm_s = (pprof["prefill_gate_up"][0] + pprof["prefill_down"][0]) / psteps * 1e-3
+        gemm_s = ((pprof["prefill_gate_up"][0] + pprof["prefill_down"][0]) / psteps - 2 * gap_ms) * 1e-3
         prefill = {"tokens": TP, "tok_per_s": round(TP / pel, 1), "ms_per_layer": round(pel * 1e3, 4),
                    "pairs": n_pairs, "m_tiles": n_tiles, "pairs_per_expert_min": int(counts.min()),
                    "pairs_per_expert_max": int(counts.max()), "kernel_us": pk_us,
                    "roofline": {"bound": "mfma", "kernel": "prefill_gemm_kernel (gate_up + down)",
                                 "achieved": round((flops_gu + flops_dn) / gemm_s / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                                 "unit": "TFLOP/s", "frac": round((flops_gu + flops_dn) / gemm_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-                                "traffic": None}}
+                                "traffic": TRAFFIC_PREFILL_GEMMS_3072 if TP == 3072 else None,
+                                "traffic_unit": "HBM bytes of the two launches (rocprofv3 --pmc, same profile file)"}}
 
     def timed(fn, reps, warm=3):
         for _ in range(warm):
@@ -373,7 +398,10 @@ def main():
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "avg_kernel_us": kernel_us.get("gate_up")},
+                     "traffic": TRAFFIC_GATE_UP_VERIFY16 if (T == 16 and L == 30 and "down" in prof) else None,
+                     "traffic_unit": "bytes per launch (rocprofv3 --pmc, profiles/hbm_traffic_verify16_prefill3072.txt)",
+                     "algorithmic_bytes_per_launch": int(live_sum / args.steps * GATE_UP_BYTES),
+                     "avg_kernel_us": kernel_us.get("gate_up")},
         "kernel_us": kernel_us,
         "down_kernel_GBs": None if down_gbs is None else round(down_gbs, 1),
         "prefill_tok_s": prefill["tok_per_s"] if prefill else None,

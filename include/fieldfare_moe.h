@@ -230,7 +230,9 @@ int ffmoe_matrix_greedy(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint3
 enum {
     FFMOE_K_ROUTER_LOGITS = 0, FFMOE_K_ROUTER_TOPK, FFMOE_K_PLAN, FFMOE_K_GATE_UP, FFMOE_K_DOWN,
     FFMOE_K_COMBINE, FFMOE_K_PREFILL_SORT, FFMOE_K_PREFILL_GATE_UP, FFMOE_K_PREFILL_DOWN,
-    FFMOE_K_PREFILL_COMBINE, FFMOE_K_GEMV, FFMOE_K_ARGMAX, FFMOE_PROFILE_SLOTS = 12
+    FFMOE_K_PREFILL_COMBINE, FFMOE_K_GEMV, FFMOE_K_ARGMAX,
+    FFMOE_K_EVENT_GAP, /* two event records with nothing between them: what an event pair adds to every slot above */
+    FFMOE_PROFILE_SLOTS = 16
 };
 typedef struct {
     double ms[FFMOE_PROFILE_SLOTS];          /* summed GPU time per kernel slot */
