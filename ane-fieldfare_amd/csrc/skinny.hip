@@ -355,6 +355,85 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     }
 }
 
+// down projection, persistent: the waves of the grid are dealt to the live experts; a wave keeps the
+// expert's (<= 16) activation rows in registers (all of K = F: at most kRing groups) and walks a range of
+// 32-row tile rows with the weight ring refilled across them. No K-split, so no LDS and no barrier.
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                                 const VerifyPlan *__restrict__ plan,
+                                                                 const uint16_t *__restrict__ acts,
+                                                                 float *__restrict__ partials_f32,
+                                                                 uint16_t *__restrict__ partials_bf16) {
+    __shared__ float s_tmp[4][8][64];
+    const uint32_t n_live = __builtin_amdgcn_readfirstlane(plan->n_live);
+    if (n_live == 0) return;
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t gwave = blockIdx.x * 4 + wave;
+    const uint32_t waves_per_slot = max(1u, min(g.dn_rbp, gridDim.x * 4 / n_live));
+    const uint32_t slot_id = gwave / waves_per_slot;
+    if (slot_id >= n_live) return;
+    uint32_t rb0, rb1;
+    split_range(g.dn_rbp, waves_per_slot, gwave % waves_per_slot, rb0, rb1);
+    if (rb0 >= rb1) return;
+    const PlanSlot &slot = plan->slots[slot_id];
+    const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
+    const uint32_t expert = __builtin_amdgcn_readfirstlane(slot.expert);
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint8_t *expert_base = arena_layer + (size_t)expert * g.expert_bytes;
+    const TileSource src = make_tile_source(expert_base + g.dn_tiles_off, (size_t)g.dn_rbp * g.gf * kTileBytes,
+                                            expert_base + g.dn_scales_off, (size_t)g.dn_rbp * g.gf * kTileScaleBytes);
+    const uint32_t ng = g.gf, g_last = g.gf - 1;
+
+    WeightRing ring;
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb0 * ng + min((uint32_t)u, g_last), lane);
+    const uint16_t *arow = acts + (size_t)slot.routes[min(j, n - 1)] * g.f + 8 * jq;
+    uint4 x0[kRing], x1[kRing];
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) {
+        const bool live = (uint32_t)u < ng;
+        const uint32_t gg = min((uint32_t)u, g_last);
+        x0[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup) : uint4{0, 0, 0, 0};
+        x1[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
+    }
+    uint32_t out_base[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) out_base[r] = slot.routes[min(4 * jq + r, n - 1)] * g.d;
+
+    for (uint32_t rb = rb0; rb < rb1; ++rb) {
+        const uint32_t next_row = min(rb + 1, rb1 - 1) * ng;
+        TwoStreamAcc tot;
+        tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
+        tot.b = tot.a;
+#pragma unroll
+        for (int u = 0; u < kRing; ++u)
+            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min((uint32_t)u, g_last), lane);
+        // The sums take a detour through a wave-private LDS slot. It costs sixteen LDS operations per tile
+        // row and changes nothing arithmetically, but it is what keeps the register allocation of this loop
+        // sane: with the sums used directly the compiler keeps every group's matrix results alive to the end
+        // of the row and spills 180 registers (the K-split kernels get the same effect from their LDS merge).
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            s_tmp[wave][r][lane] = tot.a[r];
+            s_tmp[wave][4 + r][lane] = tot.b[r];
+        }
+        const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float va = s_tmp[wave][r][lane], vb = s_tmp[wave][4 + r][lane];
+            if (4 * jq + r < n) {
+                if (OUT_BF16) {
+                    partials_bf16[(size_t)out_base[r] + row_a] = f32_to_bf16(va);
+                    partials_bf16[(size_t)out_base[r] + row_b] = f32_to_bf16(vb);
+                } else {
+                    partials_f32[(size_t)out_base[r] + row_a] = va;
+                    partials_f32[(size_t)out_base[r] + row_b] = vb;
+                }
+            }
+        }
+    }
+}
+
 // y[t][c] = bf16(residual + sum_r w[t][r] * partial[t*k + r][c]) in rank order with fmaf, fp32 partials,
 // one rounding at the end (the decode form, moe.metal:627-636). Routes the plan skips (zero weight or
 // expert out of range) add nothing.
@@ -427,10 +506,15 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_GATE_UP);
-    const dim3 dn_grid((g.dn_rbp + 3) / 4, slots);
+    const dim3 dn_grid = persistent ? dim3(max((slots + 3) / 4, min(n_cus, (slots * g.dn_rbp + 3) / 4)))
+                                    : dim3((g.dn_rbp + 3) / 4, slots);
 #define FFMOE_DOWN(BF)                                                                                          \
-    hipLaunchKernelGGL(skinny_down_kernel<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts, partials_f32, \
-                       partials_bf16)
+    if (persistent)                                                                                             \
+        hipLaunchKernelGGL(skinny_down_persistent<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,    \
+                           partials_f32, partials_bf16);                                                        \
+    else                                                                                                        \
+        hipLaunchKernelGGL(skinny_down_kernel<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,        \
+                           partials_f32, partials_bf16)
     if (partials_bf16) {
         FFMOE_DOWN(true);
         timer->mark(s, FFMOE_K_DOWN);
