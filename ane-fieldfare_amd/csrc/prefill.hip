@@ -284,30 +284,61 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     if (NMB == 0) return;
 
     // epilogue: lane (j, jq) holds pair 16 (w + 4 i) + j, weight rows 4 jq .. 4 jq + 3 of every fragment
+    if (GATE_UP) {
 #pragma unroll
-    for (int i = 0; i < NA; ++i) {
-        const uint32_t prow = (wave + 4 * i) * 16 + j;
-        if (prow >= gw.tile.rows) continue;
-        const uint32_t pair = gw.tile.row_start + prow;
-        uint16_t *orow = GATE_UP ? out + (size_t)pair * g.f : out + (size_t)sorted_out_row[pair] * g.d;
+        for (int i = 0; i < NA; ++i) {
+            const uint32_t prow = (wave + 4 * i) * 16 + j;
+            if (prow >= gw.tile.rows) continue;
+            uint16_t *orow = out + (size_t)(gw.tile.row_start + prow) * g.f;
 #pragma unroll
-        for (int tl = 0; tl < kTilesPerBlock; ++tl) {
-            const uint32_t atl = gw.nb * kTilesPerBlock + tl;
-            if (atl >= gw.n_arena_tiles) continue;
-            if (GATE_UP) {
+            for (int tl = 0; tl < kTilesPerBlock; ++tl) {
+                const uint32_t atl = gw.nb * kTilesPerBlock + tl;
+                if (atl >= gw.n_arena_tiles) continue;
                 float h[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) h[r] = gelu_tanh_fast(acc[i][2 * tl][r]) * acc[i][2 * tl + 1][r];
                 *reinterpret_cast<uint2 *>(orow + atl * kTileRows + 4 * jq) = make_uint2(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]));
-            } else {
-#pragma unroll
-                for (int sdx = 0; sdx < 2; ++sdx) {
-                    const f32x4 v = acc[i][2 * tl + sdx];
-                    *reinterpret_cast<uint2 *>(orow + atl * 2 * kTileRows + sdx * kTileRows + 4 * jq) =
-                        make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-                }
             }
         }
+        return;
+    }
+    // Down projection: a 16-pair block of this N-block is 16 rows x 256 B. Each wave turns its blocks
+    // through a private LDS area (the weight buffers are free: the last step ended with a barrier) so that
+    // 16 lanes store one row's 256 contiguous bytes, instead of 8-byte pieces 32 B apart per instruction.
+    constexpr uint32_t kStageRow = 2 * kTilesPerBlock * kTileRows * 2 + 16;     // bytes: 128 columns + padding
+    static_assert(4 * 16 * kStageRow <= sizeof(uint4) * 2 * kTilesPerBlock * 2 * 2 * kWave, "staging fits the weight buffers");
+    uint8_t *stage = reinterpret_cast<uint8_t *>(wb) + wave * 16 * kStageRow;
+    const uint32_t rsub = lane >> 4, chunk = lane & 15;                         // read side: row 4 p + rsub, columns 8 chunk ..
+    const bool col_ok = gw.nb * kTilesPerBlock + (chunk >> 2) < gw.n_arena_tiles;
+    uint32_t orow_idx[NA][4];
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const uint32_t prow = (wave + 4 * i) * 16 + 4 * p + rsub;
+            orow_idx[i][p] = sorted_out_row[gw.tile.row_start + min(prow, gw.tile.rows - 1)];
+        }
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+#pragma unroll
+        for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) {
+            const f32x4 v = acc[i][nf];
+            *reinterpret_cast<uint2 *>(stage + j * kStageRow + nf * 32 + 8 * jq) =
+                make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const uint32_t row = 4 * p + rsub, prow = (wave + 4 * i) * 16 + row;
+            const uint4 v = *reinterpret_cast<const uint4 *>(stage + row * kStageRow + 16 * chunk);
+            if (prow < gw.tile.rows && col_ok)
+                *reinterpret_cast<uint4 *>(out + (size_t)orow_idx[i][p] * g.d + gw.nb * (2 * kTilesPerBlock * kTileRows) + 8 * chunk) = v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 }
 
