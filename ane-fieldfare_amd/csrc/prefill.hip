@@ -202,83 +202,107 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
 #pragma unroll
         for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) acc[i][nf] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    uint4 wraw = {0, 0, 0, 0};
+    uint4 wraw = {0, 0, 0, 0};      // this wave's packed tile, in flight: the group after the one being expanded
     uint2 sraw = {0, 0};
     auto load_b = [&](uint32_t grp) {
         wraw = reinterpret_cast<const uint4 *>(gw.w_tiles + (size_t)grp * kTileBytes)[lane];
         sraw = reinterpret_cast<const uint2 *>(gw.w_scales + (size_t)grp * kTileScaleBytes)[j];
     };
-    auto expand_b = [&](int buf) {
-        const float s0 = bf16lo_to_f32(sraw.x), b0 = bf16hi_to_f32(sraw.x);
-        const float s1 = bf16lo_to_f32(sraw.y), b1 = bf16hi_to_f32(sraw.y);
-        wb[buf][wave][0][0][lane] = dequant8_bf16(wraw.x, s0, b0);
-        wb[buf][wave][0][1][lane] = dequant8_bf16(wraw.y, s0, b0);
-        wb[buf][wave][1][0][lane] = dequant8_bf16(wraw.z, s1, b1);
-        wb[buf][wave][1][1][lane] = dequant8_bf16(wraw.w, s1, b1);
+    // Expansion of the packed tile in `wcur` into wb[buf], cut into 16 pieces of about five VALU
+    // instructions (piece 4 c + q = output dword q of packed word c; the word's last piece stores it).
+    uint32_t wcur[4];
+    float sc[2], bi[2];
+    uint32_t lo = 0, hi = 0;
+    uint4 ex = {0, 0, 0, 0};
+    auto expand_begin = [&]() {
+        wcur[0] = wraw.x, wcur[1] = wraw.y, wcur[2] = wraw.z, wcur[3] = wraw.w;
+        sc[0] = bf16lo_to_f32(sraw.x), bi[0] = bf16hi_to_f32(sraw.x);
+        sc[1] = bf16lo_to_f32(sraw.y), bi[1] = bf16hi_to_f32(sraw.y);
     };
-    uint4 araw[NA][2];      // A of the next group in load layout (in flight during the step)
-    bf16x8 af[NA][2];       // A of the current group as MFMA fragments
-    auto load_a = [&](uint32_t grp) {
-        if (NMB == 0) return;
-#pragma unroll
-        for (int i = 0; i < NA; ++i) {
-            araw[i][0] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup);
-            araw[i][1] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup + 32);
+    auto expand_piece = [&](int buf, int piece) {
+        const int c = piece >> 2, q = piece & 3;
+        const float s_ = sc[c >> 1], b_ = bi[c >> 1];
+        if (q == 0) {
+            // even / odd nibbles as bytes; the empty asm keeps the masks as written (one v_cvt_f32_ubyteN per byte)
+            lo = wcur[c] & 0x0F0F0F0Fu, hi = (wcur[c] >> 4) & 0x0F0F0F0Fu;
+            asm("" : "+v"(lo), "+v"(hi));
+            ex.x = pack_bf16x2(__builtin_fmaf((float)(lo & 0xFFu), s_, b_), __builtin_fmaf((float)((lo >> 16) & 0xFFu), s_, b_));
+        } else if (q == 1) {
+            ex.y = pack_bf16x2(__builtin_fmaf((float)(hi & 0xFFu), s_, b_), __builtin_fmaf((float)((hi >> 16) & 0xFFu), s_, b_));
+        } else if (q == 2) {
+            ex.z = pack_bf16x2(__builtin_fmaf((float)((lo >> 8) & 0xFFu), s_, b_), __builtin_fmaf((float)(lo >> 24), s_, b_));
+        } else {
+            ex.w = pack_bf16x2(__builtin_fmaf((float)((hi >> 8) & 0xFFu), s_, b_), __builtin_fmaf((float)(hi >> 24), s_, b_));
+            wb[buf][wave][c >> 1][c & 1][lane] = ex;
         }
     };
-    auto frag_a = [&]() {
+    uint4 araw[NA][2];      // A in load layout, in flight: [.][0] k-half 0, [.][1] k-half 1
+    bf16x8 af[NA][2];       // A as MFMA fragments
+    auto load_a = [&](uint32_t grp, int half) {
         if (NMB == 0) return;
 #pragma unroll
-        for (int i = 0; i < NA; ++i) {
-            af[i][0] = to_frag(araw[i][0]);
-            af[i][1] = to_frag(araw[i][1]);
-        }
+        for (int i = 0; i < NA; ++i) araw[i][half] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup + 32 * half);
     };
-    // One 64-wide group. On entry: af = fragments of this group, araw = loads of the next group in flight,
-    // wraw/sraw = this wave's packed tile of the next group in flight, wb[buf] = expanded tiles of this group.
-    // The step expands the next tiles into wb[buf ^ 1] between the MFMAs, then turns araw into the next
-    // fragments (its loads have had the whole step to land) and issues the loads of the group after.
-    // Past the last group the same loads and expansion run once more on clamped indices and are never used:
-    // with no branch around them the compiler counts the loads in flight exactly.
+    auto frag_a = [&](int half) {
+        if (NMB == 0) return;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) af[i][half] = to_frag(araw[i][half]);
+    };
+    // One 64-wide group = 16 units; unit u multiplies weight fragment (nf = u % 8, k-half u / 8) with the NA
+    // row blocks, and is followed by one piece of the next group's expansion, so the matrix pipe and the
+    // VALU run side by side inside the wave (a scheduling fence after every unit keeps the order as
+    // written). On entry: af[.][0] = k-half 0 of this group; araw[.][1] = its k-half 1 in load layout;
+    // araw[.][0] = k-half 0 of the next group in flight; wraw/sraw = packed tile of the next group in
+    // flight; wb[buf] = expanded tiles of this group. The k-half 1 fragments are made at the start of the
+    // step and the next k-half 0 fragments in its middle, each as soon as the registers they replace have
+    // had their last use, with 8 units of MFMAs to cover the cross-lane latency; every register that a
+    // conversion frees is reloaded at once for the following group. Past the last group the loads and the
+    // expansion run once more on clamped indices and are never used: with no branch around them the
+    // compiler counts the loads in flight exactly.
     auto step = [&](uint32_t grp) {
         const int buf = grp & 1;
-        expand_b(buf ^ 1);
+        frag_a(1);
+        load_a(min(grp + 1, n_groups - 1), 1);
+        expand_begin();
         load_b(min(grp + 2, n_groups - 1));
+        uint4 bq[3];
+        auto read_b = [&](int u) { bq[u % 3] = wb[buf][(u & 7) >> 1][u & 1][u >> 3][lane]; };
         if (NMB > 0) {
-            // B fragments are read one fragment pair ahead of the MFMAs that use them
-            uint4 bq[2][2];
-            bq[0][0] = wb[buf][0][0][0][lane];
-            bq[0][1] = wb[buf][0][0][1][lane];
-#pragma unroll
-            for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) {
-                if (nf + 1 < 2 * kTilesPerBlock) {
-                    bq[(nf + 1) & 1][0] = wb[buf][(nf + 1) >> 1][(nf + 1) & 1][0][lane];
-                    bq[(nf + 1) & 1][1] = wb[buf][(nf + 1) >> 1][(nf + 1) & 1][1][lane];
-                }
-                const bf16x8 b0 = __builtin_bit_cast(bf16x8, bq[nf & 1][0]);
-                const bf16x8 b1 = __builtin_bit_cast(bf16x8, bq[nf & 1][1]);
-#pragma unroll
-                for (int i = 0; i < NA; ++i) {
-                    // weights as the first operand: the lane ends up with four consecutive weight rows of
-                    // one pair, which the epilogue stores as one 8-byte piece of that pair's output row
-                    acc[i][nf] = mfma16(b0, af[i][0], acc[i][nf]);
-                    acc[i][nf] = mfma16(b1, af[i][1], acc[i][nf]);
-                }
-            }
+            read_b(0);
+            read_b(1);
         }
         __builtin_amdgcn_sched_barrier(0);
-        frag_a();
-        load_a(min(grp + 2, n_groups - 1));
-        __builtin_amdgcn_sched_barrier(0);      // nothing of the next step may start before the barrier
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            if (NMB > 0) {
+                if (u + 2 < 16) read_b(u + 2);
+                const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bq[u % 3]);
+#pragma unroll
+                for (int i = 0; i < NA; ++i)
+                    // weights as the first operand: the lane ends up with four consecutive weight rows of
+                    // one pair, which the epilogue packs into one 8-byte piece of that pair's output row
+                    acc[i][u & 7] = mfma16(bfrag, af[i][u >> 3], acc[i][u & 7]);
+            }
+            expand_piece(buf ^ 1, u);
+            __builtin_amdgcn_sched_barrier(0);
+            if (u == 7) {
+                frag_a(0);
+                load_a(min(grp + 2, n_groups - 1), 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
         lds_barrier();
     };
 
     load_b(0);
-    load_a(0);
-    expand_b(0);
+    load_a(0, 0);
+    load_a(0, 1);
+    expand_begin();
     load_b(min(1u, n_groups - 1));
-    frag_a();
-    load_a(min(1u, n_groups - 1));
+#pragma unroll
+    for (int piece = 0; piece < 16; ++piece) expand_piece(0, piece);
+    frag_a(0);
+    load_a(min(1u, n_groups - 1), 0);
     lds_barrier();
     for (uint32_t grp = 0; grp < n_groups; ++grp) step(grp);
     if (NMB == 0) return;
