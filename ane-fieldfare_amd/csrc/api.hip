@@ -16,6 +16,7 @@ using namespace ffmoe;
 
 struct ffmoe_layer {
     bool experts_loaded = false;
+    std::vector<bool> part_loaded;  // experts uploaded one at a time (ffmoe_upload_expert_parts)
     void *router_w = nullptr;       // bf16 or float [E][D]
     int router_is_f32 = 0;
     uint16_t *effective_scale = nullptr;
@@ -47,6 +48,9 @@ struct ffmoe_ctx {
     float *partials = nullptr;       // [16*top_k][D]
     PrefillScratch pf{};
     uint32_t max_pairs = 0;
+    // dense FFN (n_experts == 1, top_k == 1): every row routes to expert 0 with weight 1
+    uint32_t *dense_idx = nullptr;   // [max(max_tokens,16)] zeros
+    uint16_t *dense_w = nullptr;     // [max(max_tokens,16)] bf16 1.0
     KernelTimer timer;
 };
 
@@ -151,6 +155,12 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.sorted_out_row), (size_t)ctx->max_pairs * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.acts), (size_t)ctx->max_pairs * shape->f * sizeof(uint16_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.partials), (size_t)ctx->max_pairs * shape->d * sizeof(uint16_t));
+    if (e == hipSuccess && shape->n_experts == 1 && shape->top_k == 1) {
+        e = hipMalloc(reinterpret_cast<void **>(&ctx->dense_idx), (size_t)router_rows * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipMemset(ctx->dense_idx, 0, (size_t)router_rows * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->dense_w), (size_t)router_rows * sizeof(uint16_t));
+        if (e == hipSuccess) e = hipMemsetD16(reinterpret_cast<hipDeviceptr_t>(ctx->dense_w), 0x3F80, router_rows);
+    }
     if (e != hipSuccess) {
         ffmoe_destroy(ctx);
         return fail(err, FFMOE_ERR_ALLOC, "failed to allocate the expert arena (%zu bytes) or scratch: %s",
@@ -182,6 +192,8 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (ctx->pf.sorted_out_row) (void)hipFree(ctx->pf.sorted_out_row);
     if (ctx->pf.acts) (void)hipFree(ctx->pf.acts);
     if (ctx->pf.partials) (void)hipFree(ctx->pf.partials);
+    if (ctx->dense_idx) (void)hipFree(ctx->dense_idx);
+    if (ctx->dense_w) (void)hipFree(ctx->dense_w);
     for (auto &ev : ctx->timer.ev)
         if (ev) (void)hipEventDestroy(ev);
     delete ctx;
@@ -225,6 +237,50 @@ int ffmoe_upload_layer(ffmoe_ctx *ctx, uint32_t layer, const void *blobs, size_t
     if (staging) (void)hipFree(staging);
     if (e != hipSuccess) return fail(err, FFMOE_ERR_RUNTIME, "re-tiling layer %u failed: %s", layer, hipGetErrorString(e));
     ctx->layers[layer].experts_loaded = true;
+    return FFMOE_OK;
+}
+
+int ffmoe_upload_expert_parts(ffmoe_ctx *ctx, uint32_t layer, uint32_t expert, const ffmoe_projection *gate,
+                              const ffmoe_projection *up, const ffmoe_projection *down, int src_is_device,
+                              char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, false, false, err)) return rc;
+    const ffmoe_shape &sh = ctx->shape;
+    if (expert >= sh.n_experts) return fail(err, FFMOE_ERR_INVALID, "expert %u out of range", expert);
+    const ffmoe_projection *proj[3] = {gate, up, down};
+    for (const ffmoe_projection *p : proj)
+        if (!p || !p->w || !p->scales || !p->biases) return fail(err, FFMOE_ERR_INVALID, "null projection");
+    // stage the nine arrays as one blob in the order gate W/S/B, up W/S/B, down W/S/B, 16-byte aligned
+    const size_t gu_w = (size_t)sh.f * sh.d / 2, gu_s = (size_t)sh.f * (sh.d / FFMOE_GROUP) * 2;
+    const size_t dn_w = (size_t)sh.d * sh.f / 2, dn_s = (size_t)sh.d * (sh.f / FFMOE_GROUP) * 2;
+    const size_t len[9] = {gu_w, gu_s, gu_s, gu_w, gu_s, gu_s, dn_w, dn_s, dn_s};
+    const void *src[9] = {gate->w, gate->scales, gate->biases, up->w, up->scales, up->biases,
+                          down->w, down->scales, down->biases};
+    uint32_t off[9];
+    size_t total = 0;
+    for (int i = 0; i < 9; ++i) {
+        off[i] = (uint32_t)total;
+        total += (len[i] + 15) & ~(size_t)15;
+    }
+    uint8_t *staging = nullptr;
+    FF_HIP(hipMalloc(reinterpret_cast<void **>(&staging), total));
+    hipError_t e = hipSuccess;
+    for (int i = 0; i < 9 && e == hipSuccess; ++i)
+        e = hipMemcpy(staging + off[i], src[i], len[i], src_is_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice);
+    const ffmoe_offsets offsets = {off[0], off[1], off[2], off[3], off[4], off[5], off[6], off[7], off[8]};
+    if (e == hipSuccess)
+        e = launch_repack_layer(nullptr, staging, total, offsets, 1, ctx->geom,
+                                ctx->arena + (size_t)layer * ctx->layer_bytes + (size_t)expert * ctx->geom.expert_bytes);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    (void)hipFree(staging);
+    if (e != hipSuccess)
+        return fail(err, FFMOE_ERR_RUNTIME, "upload of expert %u of layer %u failed: %s", expert, layer, hipGetErrorString(e));
+    ffmoe_layer &l = ctx->layers[layer];
+    if (l.part_loaded.size() != sh.n_experts) l.part_loaded.assign(sh.n_experts, false);
+    l.part_loaded[expert] = true;
+    bool all = true;
+    for (bool b : l.part_loaded) all = all && b;
+    if (all) l.experts_loaded = true;
     return FFMOE_OK;
 }
 
@@ -351,8 +407,8 @@ static int prefill_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const ui
         return fail(err, FFMOE_ERR_ALLOC, "prefill sorted route pairs exceed reusable capacity (%u > %u)", n_pairs, ctx->max_pairs);
     if (x_stride < ctx->shape.d || x_stride % 8 || reinterpret_cast<uintptr_t>(x) % 16)
         return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
-    if ((y && reinterpret_cast<uintptr_t>(y) % 16) || (partials && reinterpret_cast<uintptr_t>(partials) % 2))
-        return fail(err, FFMOE_ERR_INVALID, "output alignment");
+    if ((y && reinterpret_cast<uintptr_t>(y) % 16) || (partials && reinterpret_cast<uintptr_t>(partials) % 16))
+        return fail(err, FFMOE_ERR_INVALID, "outputs must be 16-byte aligned");
     FF_HIP(launch_prefill(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                           ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, pairs, n_pairs, y, partials,
                           ctx->pf, &ctx->timer));
@@ -371,6 +427,20 @@ int ffmoe_prefill_pairs(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint
     if (n_pairs == 0) return FFMOE_OK;
     if (!pairs) return fail(err, FFMOE_ERR_INVALID, "null argument");
     return prefill_common(ctx, stream, layer, x, x_stride, t, nullptr, nullptr, pairs, n_pairs, nullptr, partials, err);
+}
+
+int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride, uint32_t t,
+                    uint16_t *y, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!ctx->dense_idx)
+        return fail(err, FFMOE_ERR_INVALID, "the dense FFN needs a context with n_experts = 1 and top_k = 1");
+    if (!y) return fail(err, FFMOE_ERR_INVALID, "null output");
+    if (reinterpret_cast<uintptr_t>(y) % 16) return fail(err, FFMOE_ERR_INVALID, "y must be 16-byte aligned");
+    // With one route per row at weight 1, the un-weighted bf16 row of route t is the output row t: the
+    // down projection writes y itself and the combine pass has nothing to add.
+    if (t <= FFMOE_MAX_VERIFY_ROWS)
+        return verify_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, nullptr, y, err);
+    return prefill_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, 0, nullptr, y, err);
 }
 
 int ffmoe_prefill_plan_stats(ffmoe_ctx *ctx, void *stream, uint32_t *n_pairs, uint32_t *n_tiles, uint32_t *counts,

@@ -159,7 +159,6 @@ __global__ __launch_bounds__(kSortBlock) void prefill_scatter_kernel(ItemSource 
 // GATE_UP: A rows are gathered token rows of x; streams are gate / up; out = acts[pair][F].
 // else:    A rows are acts[pair][F]; streams are two 16-row blocks; out = partials[out_row][D] (bf16).
 // ---------------------------------------------------------------------------------------------------
-constexpr int kMbPerWave = kBM / 16 / 4;
 
 struct GemmWave {
     const uint8_t *w_tiles, *w_scales;    // this wave's arena tile row

@@ -434,6 +434,86 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
     }
 }
 
+// down projection, persistent, for K = F of more than kRing groups (a wide dense expert): the blocks of the
+// grid are dealt to the live experts and the four waves of a block split K as in the gate/up kernel, each
+// with its slice of the activation rows in registers; the partial sums meet in LDS and wave ks finishes
+// token slots 4 * (lane / 16) + ks.
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                                        const VerifyPlan *__restrict__ plan,
+                                                                        const uint16_t *__restrict__ acts,
+                                                                        float *__restrict__ partials_f32,
+                                                                        uint16_t *__restrict__ partials_bf16) {
+    __shared__ float s_red[2][kKSplit][8][64];
+    const uint32_t n_live = __builtin_amdgcn_readfirstlane(plan->n_live);
+    if (n_live == 0) return;
+    const uint32_t bid = blockIdx.x;
+    const uint32_t blocks_per_slot = max(1u, min(g.dn_rbp, gridDim.x / n_live));
+    const uint32_t slot_id = bid / blocks_per_slot;
+    if (slot_id >= n_live) return;
+    uint32_t rb0, rb1;
+    split_range(g.dn_rbp, blocks_per_slot, bid % blocks_per_slot, rb0, rb1);
+    if (rb0 >= rb1) return;
+    const PlanSlot &slot = plan->slots[slot_id];
+    const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
+    const uint32_t expert = __builtin_amdgcn_readfirstlane(slot.expert);
+    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint8_t *expert_base = arena_layer + (size_t)expert * g.expert_bytes;
+    const uint32_t per = (g.gf + kKSplit - 1) / kKSplit;
+    const uint32_t g0 = min(ks * per, g.gf), g1 = min(g.gf, g0 + per), ng = g1 - g0;
+    const uint32_t g_last = g1 > g0 ? g1 - 1 : g.gf - 1;
+    const TileSource src = make_tile_source(expert_base + g.dn_tiles_off, (size_t)g.dn_rbp * g.gf * kTileBytes,
+                                            expert_base + g.dn_scales_off, (size_t)g.dn_rbp * g.gf * kTileScaleBytes);
+    WeightRing ring;
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb0 * g.gf + min(g0 + u, g_last), lane);
+    const uint16_t *arow = acts + (size_t)slot.routes[min(j, n - 1)] * g.f + 8 * jq;
+    uint4 x0[kRing], x1[kRing];
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) {
+        const bool live = (uint32_t)u < ng;
+        const uint32_t gg = min(g0 + u, g_last);
+        x0[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup) : uint4{0, 0, 0, 0};
+        x1[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
+    }
+    const uint32_t my_ts = 4 * jq + ks;     // the token slot this lane finishes
+    const size_t out_base = (size_t)slot.routes[min(my_ts, n - 1)] * g.d;
+
+    for (uint32_t rb = rb0; rb < rb1; ++rb) {
+        const uint32_t next_row = min(rb + 1, rb1 - 1) * g.gf;
+        TwoStreamAcc tot;
+        tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
+        tot.b = tot.a;
+#pragma unroll
+        for (int u = 0; u < kRing; ++u)
+            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min(g0 + u, g_last), lane);
+        const int buf = (rb - rb0) & 1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            s_red[buf][ks][r][lane] = tot.a[r];
+            s_red[buf][ks][4 + r][lane] = tot.b[r];
+        }
+        lds_barrier();
+        float va = s_red[buf][0][ks][lane], vb = s_red[buf][0][4 + ks][lane];
+#pragma unroll
+        for (int o = 1; o < kKSplit; ++o) {
+            va += s_red[buf][o][ks][lane];
+            vb += s_red[buf][o][4 + ks][lane];
+        }
+        const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
+        if (my_ts < n) {
+            if (OUT_BF16) {
+                partials_bf16[out_base + row_a] = f32_to_bf16(va);
+                partials_bf16[out_base + row_b] = f32_to_bf16(vb);
+            } else {
+                partials_f32[out_base + row_a] = va;
+                partials_f32[out_base + row_b] = vb;
+            }
+        }
+    }
+}
+
 // y[t][c] = bf16(residual + sum_r w[t][r] * partial[t*k + r][c]) in rank order with fmaf, fp32 partials,
 // one rounding at the end (the decode form, moe.metal:627-636). Routes the plan skips (zero weight or
 // expert out of range) add nothing.
@@ -490,9 +570,11 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
     timer->begin(s);
     const uint32_t slots = min(n_experts, t * top_k);
     // the persistent kernels hold a K-slice of kRing groups per wave; larger experts take the one-shot grids
-    const bool persistent = (g.gd + kKSplit - 1) / kKSplit <= (uint32_t)kRing && g.gf <= (uint32_t)kRing;
+    const bool gu_persistent = (g.gd + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
+    const bool dn_whole = g.gf <= (uint32_t)kRing;                                     // a wave holds all of K
+    const bool dn_ksplit = !dn_whole && (g.gf + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
     const uint32_t resident = 2 * n_cus;       // blocks the chip holds at once (__launch_bounds__(256, 2))
-    if (persistent) {
+    if (gu_persistent) {
         // plan slot of the profile stays empty: the gate/up kernel builds the plan itself
         const uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
         hipLaunchKernelGGL(skinny_gate_up_persistent, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts,
@@ -506,14 +588,18 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_GATE_UP);
-    const dim3 dn_grid = persistent ? dim3(max((slots + 3) / 4, min(n_cus, (slots * g.dn_rbp + 3) / 4)))
-                                    : dim3((g.dn_rbp + 3) / 4, slots);
-#define FFMOE_DOWN(BF)                                                                                          \
-    if (persistent)                                                                                             \
-        hipLaunchKernelGGL(skinny_down_persistent<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,    \
-                           partials_f32, partials_bf16);                                                        \
-    else                                                                                                        \
-        hipLaunchKernelGGL(skinny_down_kernel<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,        \
+    const dim3 dn_grid = dn_whole    ? dim3(max((slots + 3) / 4, min(n_cus, (slots * g.dn_rbp + 3) / 4)))
+                         : dn_ksplit ? dim3(max(slots, min(resident, slots * g.dn_rbp)))
+                                     : dim3((g.dn_rbp + 3) / 4, slots);
+#define FFMOE_DOWN(BF)                                                                                            \
+    if (dn_whole)                                                                                                 \
+        hipLaunchKernelGGL(skinny_down_persistent<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,      \
+                           partials_f32, partials_bf16);                                                          \
+    else if (dn_ksplit)                                                                                           \
+        hipLaunchKernelGGL(skinny_down_ksplit_persistent<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan,     \
+                           acts, partials_f32, partials_bf16);                                                    \
+    else                                                                                                          \
+        hipLaunchKernelGGL(skinny_down_kernel<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,          \
                            partials_f32, partials_bf16)
     if (partials_bf16) {
         FFMOE_DOWN(true);

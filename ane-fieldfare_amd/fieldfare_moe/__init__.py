@@ -44,13 +44,18 @@ EXPORTS = [
     "ffmoe_verify", "ffmoe_verify_partials", "ffmoe_last_live_experts", "ffmoe_reduce_token_major",
     "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
-    "ffmoe_matrix_greedy",
+    "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn",
 ]
 
 PROFILE_SLOTS = 16
 KERNEL_NAMES = ["router_logits", "router_topk", "plan", "gate_up", "down", "combine", "prefill_sort",
                 "prefill_gate_up", "prefill_down", "prefill_combine", "gemv", "argmax", "event_gap", "reserved13",
                 "reserved14", "reserved15"]
+
+
+class Projection(C.Structure):
+    """SharedExpertProjection: W uint8 [rows][cols/2], S/B bf16 [rows][cols/64] (Kernels/MoE/SharedExpertInt4.swift:32-40)."""
+    _fields_ = [("w", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p)]
 
 
 class Profile(C.Structure):
@@ -157,6 +162,9 @@ def lib() -> C.CDLL:
     L.ffmoe_matrix_destroy.restype = None
     L.ffmoe_matrix_gemv.argtypes = [vp, vp, vp, u32, u32, vp, u32, i32, errp]
     L.ffmoe_matrix_greedy.argtypes = [vp, vp, vp, u32, u32, vp, errp]
+    L.ffmoe_upload_expert_parts.argtypes = [vp, u32, u32, C.POINTER(Projection), C.POINTER(Projection),
+                                            C.POINTER(Projection), i32, errp]
+    L.ffmoe_dense_ffn.argtypes = [vp, vp, u32, vp, u32, u32, vp, errp]
     _lib = L
     return L
 
@@ -236,6 +244,31 @@ class Context:
             assert blobs.dtype == torch.uint8 and blobs.is_contiguous()
             p, on_dev = C.c_void_p(blobs.data_ptr()), int(blobs.is_cuda)
         _check(self.L.ffmoe_upload_layer(self._h, layer, p, stride, C.byref(offsets), on_dev, C.byref(err)), err)
+
+    def upload_expert_parts(self, layer: int, expert: int, gate, up, down):
+        """One expert from three (W uint8, S bf16 bits, B bf16 bits) triples: all numpy arrays or all CUDA tensors."""
+        import numpy as np
+        keep, kinds = [], set()
+
+        def proj(triple):
+            ptrs = []
+            for a in triple:
+                if isinstance(a, np.ndarray):
+                    a = np.ascontiguousarray(a)
+                    ptrs.append(a.ctypes.data)
+                    kinds.add(0)
+                else:
+                    assert a.is_contiguous()
+                    ptrs.append(a.data_ptr())
+                    kinds.add(int(a.is_cuda))
+                keep.append(a)
+            return Projection(*ptrs)
+
+        g, u, dn = proj(gate), proj(up), proj(down)
+        assert len(kinds) == 1, "all nine arrays must live on the same side"
+        err = C.c_char_p()
+        _check(self.L.ffmoe_upload_expert_parts(self._h, layer, expert, C.byref(g), C.byref(u), C.byref(dn),
+                                                kinds.pop(), C.byref(err)), err)
 
     def upload_router_bf16(self, layer: int, w_bits, effective_scale_bits=None, per_expert_scale_bits=None):
         """numpy uint16 arrays (bf16 bit patterns), host side."""
@@ -323,6 +356,15 @@ class Context:
         err = C.c_char_p()
         _check(self.L.ffmoe_prefill(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(idx), _ptr(w), _ptr(y),
                                     C.byref(err)), err)
+        return y
+
+    def dense_ffn(self, layer: int, x, out=None):
+        """Shared expert: every row of x through expert 0 with weight 1 (context with n_experts = top_k = 1)."""
+        import torch
+        t = x.shape[0]
+        y = out if out is not None else torch.empty((t, self.shape.d), dtype=torch.bfloat16, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_dense_ffn(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(y), C.byref(err)), err)
         return y
 
     def prefill_pairs(self, layer: int, x, sorted_pairs, t: int, partials):

@@ -368,6 +368,91 @@ private:
 };
 
 // ---------------------------------------------------------------------------------------------------
+// Shared expert (Kernels/MoE/SharedExpertInt4.swift, Kernels/Prefill/MoE/PrefillSharedExpert.swift): the dense
+// INT4 FFN every token passes through. The Swift operators bind the three projections on every call; here
+// they are uploaded once per layer into a context of one expert (n_experts = top_k = 1, f = the shared
+// width) and the calls name the layer.
+// ---------------------------------------------------------------------------------------------------
+struct SharedExpertProjection {   // weights uint8 [rows][cols/2], scales/biases bf16 [rows][cols/64]
+    const uint8_t *weights;
+    const uint16_t *scales, *biases;
+    uint32_t rows, cols;
+};
+
+struct SharedExpertError : std::runtime_error {
+    enum Kind { unsupportedWeightBits, dimensionMismatch, scratchTooSmall } kind;
+    SharedExpertError(Kind k, const std::string &m) : std::runtime_error(m), kind(k) {}
+};
+
+class SharedExpertInt4 {
+public:
+    explicit SharedExpertInt4(Context &dense) : c_(dense) {
+        if (dense.shape().n_experts != 1 || dense.shape().top_k != 1)
+            throw std::invalid_argument("the shared expert needs a context with n_experts = 1 and top_k = 1");
+    }
+    // the guard of SharedExpertInt4.encode (SharedExpertInt4.swift:41-46), then the upload
+    void load(uint32_t layer, const SharedExpertProjection &gate, const SharedExpertProjection &up,
+              const SharedExpertProjection &down, bool onDevice = false) {
+        const ffmoe_shape &sh = c_.shape();
+        if (gate.rows != up.rows || gate.cols != up.cols || down.rows != gate.cols || down.cols != gate.rows ||
+            gate.rows != sh.f || gate.cols != sh.d)
+            throw SharedExpertError(SharedExpertError::dimensionMismatch,
+                                    "SharedExpert dimension mismatch: gate=(" + std::to_string(gate.rows) + "," +
+                                        std::to_string(gate.cols) + ") up=(" + std::to_string(up.rows) + "," +
+                                        std::to_string(up.cols) + ") down=(" + std::to_string(down.rows) + "," +
+                                        std::to_string(down.cols) + ")");
+        const ffmoe_projection g{gate.weights, gate.scales, gate.biases}, u{up.weights, up.scales, up.biases},
+            dn{down.weights, down.scales, down.biases};
+        char *err = nullptr;
+        check(ffmoe_upload_expert_parts(c_.raw(), layer, 0, &g, &u, &dn, onDevice ? 1 : 0, &err), err);
+    }
+    // encode (SharedExpertInt4.swift:32-89): one row; the activation scratch is the context's
+    void encode(void *stream, uint32_t layer, const uint16_t *x, uint16_t *y) {
+        char *err = nullptr;
+        check(ffmoe_dense_ffn(c_.raw(), stream, layer, x, c_.shape().d, 1, y, &err), err);
+    }
+
+protected:
+    Context &c_;
+};
+
+// SharedExpertRuntime (SharedExpertInt4.swift:92-130): picks the implementation by weight width; only the
+// 4-bit one is part of this library.
+class SharedExpertRuntime : public SharedExpertInt4 {
+public:
+    SharedExpertRuntime(Context &dense, int weightBits) : SharedExpertInt4(dense) {
+        if (weightBits != 4)
+            throw SharedExpertError(SharedExpertError::unsupportedWeightBits,
+                                    "SharedExpert unsupported weight bits: " + std::to_string(weightBits));
+    }
+};
+
+// PrefillSharedExpert.encodeBlock (PrefillSharedExpert.swift:94-137): a block of rows. The Swift class loops
+// its single-row operator below 32 tokens and batches above; here rows <= 16 stream the weights once for
+// all rows and more rows run the grouped GEMMs.
+class PrefillSharedExpert : public SharedExpertInt4 {
+public:
+    static constexpr int batchedMinimumTokens = 17;
+    using SharedExpertInt4::SharedExpertInt4;
+    void encodeBlock(void *stream, uint32_t layer, const uint16_t *x, uint16_t *y, int queryCount, int d, int intermediate,
+                     int xStrideElements, int yStrideElements) {
+        if (queryCount < 0) throw std::invalid_argument("queryCount must be non-negative");
+        if (d <= 0) throw std::invalid_argument("d must be positive");
+        if (intermediate <= 0) throw std::invalid_argument("intermediate must be positive");
+        if (xStrideElements < d) throw std::invalid_argument("x stride is too small");
+        if (yStrideElements < d) throw std::invalid_argument("y stride is too small");
+        if ((uint32_t)d != c_.shape().d || (uint32_t)intermediate != c_.shape().f)
+            throw SharedExpertError(SharedExpertError::dimensionMismatch,
+                                    "SharedExpert dimension mismatch: expected gate/up=(" + std::to_string(c_.shape().f) + "," +
+                                        std::to_string(c_.shape().d) + ")");
+        if (yStrideElements != d) throw std::invalid_argument("y rows must be contiguous");
+        if (queryCount == 0) return;
+        char *err = nullptr;
+        check(ffmoe_dense_ffn(c_.raw(), stream, layer, x, (uint32_t)xStrideElements, (uint32_t)queryCount, y, &err), err);
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------
 // Guest plugin and supervisor (Runtime/Supervisor/DeviceSupervisor.swift:5-125).
 // ---------------------------------------------------------------------------------------------------
 enum class RuntimeFaultPolicy { failClosed, failoverHost };   // reference: .failClosed / .failoverMetal

@@ -74,6 +74,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode (T = 1) leg")
     ap.add_argument("--no-gemv", action="store_true", help="skip the INT4 GEMV legs (config 1 and the LM head)")
+    ap.add_argument("--no-shared", action="store_true", help="skip the shared-expert (dense INT4 FFN, width 2112) leg")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy three times: the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE readings of a rocprofv3 --pmc run are scaled by")
@@ -296,6 +297,49 @@ def main():
         tg = timed(lambda: head.greedy(x), 20)
         gemv["lm_head_greedy_rows16_us"] = round(tg * 1e6, 1)
         extra["gemv"] = gemv
+
+    # Shared expert: the model's dense INT4 FFN (2816 -> 2112 -> 2816) that every token passes beside the
+    # routed experts, as a context of one expert; 16 rows (verify block) and the prefill chunk
+    if not args.no_shared:
+        FS, LS = 2112, 8
+        s_off, s_payload = oracle.layout_offsets(D, FS, align=16)
+        dense = ff.Context(D, FS, 1, 1, n_layers=LS, max_tokens=max(args.prefill_tokens, 16))
+        for layer in range(LS):
+            blob = torch.empty(s_payload, dtype=torch.uint8, device="cuda")
+            for (w_o, s_o, b_o), (rows, cols) in (((s_off.gate_w, s_off.gate_s, s_off.gate_b), (FS, D)),
+                                                  ((s_off.up_w, s_off.up_s, s_off.up_b), (FS, D)),
+                                                  ((s_off.down_w, s_off.down_s, s_off.down_b), (D, FS))):
+                g_ = cols // 64
+                blob[w_o:w_o + rows * cols // 2] = torch.randint(0, 256, (rows * cols // 2,), dtype=torch.uint8, device="cuda", generator=gen)
+                sc = (torch.randn((rows, g_), device="cuda", generator=gen) * 0.01).abs().to(torch.bfloat16)
+                bi = (-8.0 * sc.float() + torch.randn((rows, g_), device="cuda", generator=gen) * 1e-3).to(torch.bfloat16)
+                blob[s_o:s_o + rows * g_ * 2] = sc.view(torch.uint8).view(-1)
+                blob[b_o:b_o + rows * g_ * 2] = bi.view(torch.uint8).view(-1)
+            dense.upload_layer(layer, blob, s_payload, ff.Offsets(*s_off.as_tuple()))
+            del blob
+        state = {"i": 0}
+
+        def dense_step(xin, yout):
+            dense.dense_ffn(state["i"] % LS, xin, out=yout)
+            state["i"] += 1
+        shared = {"shape": f"{D} -> {FS} -> {D}, INT4 g64", "bytes_per_layer": s_payload, "layers_cycled": LS}
+        y16 = torch.empty((T, D), dtype=torch.bfloat16, device="cuda")
+        t16 = timed(lambda: dense_step(x, y16), 200, warm=10)
+        shared["rows16"] = {"us": round(t16 * 1e6, 2), "GBs": round(s_payload / t16 / 1e9, 1)}
+        x1s, y1s = x[:1].contiguous(), torch.empty((1, D), dtype=torch.bfloat16, device="cuda")
+        t1 = timed(lambda: dense_step(x1s, y1s), 200, warm=10)
+        shared["rows1"] = {"us": round(t1 * 1e6, 2), "GBs": round(s_payload / t1 / 1e9, 1)}
+        if args.prefill_tokens:
+            TPs = args.prefill_tokens
+            xps = torch.randn((TPs, D), device="cuda", generator=gen).to(torch.bfloat16)
+            yps = torch.empty((TPs, D), dtype=torch.bfloat16, device="cuda")
+            tp_ = timed(lambda: dense_step(xps, yps), 20)
+            fl = 2.0 * 3 * D * FS * TPs
+            shared[f"rows{TPs}"] = {"us": round(tp_ * 1e6, 1), "TFLOPs": round(fl / tp_ / 1e12, 1),
+                                    "frac_mfma_peak": round(fl / tp_ / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+            del xps, yps
+        extra["shared_expert"] = shared
+        dense.close()
 
     # BASELINE.json config 5: all layers resident, one 8,192-token prefill with Zipf(1.1) routing imposed on
     # the experts, then 256 decode steps as 16 verify blocks of 16 tokens, the LM head once per block

@@ -164,8 +164,9 @@ int ffmoe_prefill(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *
 /* The guest contract of RoutedPrefillGuest.runLayer (Runtime/Supervisor/DeviceSupervisor.swift:14-22):
  * for every pair of `pairs` (device array, any order; the reference passes them expert-sorted) write
  * the UN-weighted row bf16 partials[(token * top_k + rank) * d ...]; rows of other routes are left
- * untouched (the host zeroes `partials` first, RealForwardRunner.swift:1502-1506). Replaces
- * ANERoutedPrefillBackend.runLayer (Runtime/Inference/ANERoutedPrefillBackend.swift:348-427). */
+ * untouched (the host zeroes `partials` first, RealForwardRunner.swift:1502-1506). `partials` is
+ * 16-byte aligned. Replaces ANERoutedPrefillBackend.runLayer
+ * (Runtime/Inference/ANERoutedPrefillBackend.swift:348-427). */
 int ffmoe_prefill_pairs(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
                         const ffmoe_pair *pairs, uint32_t n_pairs, uint32_t t, uint16_t *partials, char **err);
 
@@ -223,6 +224,38 @@ int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_
  * input rows are the already normalised hidden rows (the reference runs its RMSNorm operator first). */
 int ffmoe_matrix_greedy(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
                         uint32_t *out_tokens, char **err);
+
+/* ---- dense (shared-expert) FFN ------------------------------------------------------------------ */
+
+/* One projection in the reference layout: W uint8 [rows][cols/2], S/B bf16 [rows][cols/64]
+ * (SharedExpertProjection: Kernels/MoE/SharedExpertInt8.swift, used by SharedExpertInt4.encode,
+ * Kernels/MoE/SharedExpertInt4.swift:32-40). Host or device pointers, all three of the same kind. */
+typedef struct {
+    const uint8_t *w;
+    const uint16_t *scales;
+    const uint16_t *biases;
+} ffmoe_projection;
+
+/* Uploads one expert from three separate projections (gate, up [f][d]; down [d][f]) instead of a blob:
+ * the form in which the reference holds its shared expert (TensorView triples from
+ * Model.sharedExpertGate / Up / Down, bound per call by SharedExpertInt4.encode,
+ * Kernels/MoE/SharedExpertInt4.swift:67-72). The layer counts as loaded once each of its experts has
+ * been uploaded this way (or ffmoe_upload_layer ran). Blocking. */
+int ffmoe_upload_expert_parts(ffmoe_ctx *ctx, uint32_t layer, uint32_t expert, const ffmoe_projection *gate,
+                              const ffmoe_projection *up, const ffmoe_projection *down, int src_is_device,
+                              char **err);
+
+/* y[t] = down( bf16( gelu_tanh(gate x[t]) * (up x[t]) ) ) for every row, weight 1, no routing: the
+ * shared expert. Needs a context created with n_experts = 1 and top_k = 1 (f = the shared width).
+ * Rows <= 16 run the streaming kernels of ffmoe_verify, more rows the grouped GEMMs of ffmoe_prefill
+ * (the reference switches from its per-token GEMV loop to batched GEMMs at 32 tokens). Replaces
+ * SharedExpertInt4.encode (Kernels/MoE/SharedExpertInt4.swift:32-89, kernel shared_gate_up_act_int4,
+ * Metal/MoE/moe.metal:548-570) and PrefillSharedExpert.encodeBlock
+ * (Kernels/Prefill/MoE/PrefillSharedExpert.swift:94-137). Gate and up stay fp32 in front of the
+ * activation; the reference rounds them to FP16 there only to match its own unfused path bit for bit.
+ * x bf16 [t][x_stride], y bf16 [t][d]; both 16-byte aligned. */
+int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
+                    uint32_t t, uint16_t *y, char **err);
 
 /* ---- per-kernel timing ------------------------------------------------------------------------ */
 

@@ -219,6 +219,39 @@ int main() {
         HIP(hipFree(dTok));
     }
 
+    // --- shared expert: expert 3's projections as the dense FFN, one row and a 40-row block ---
+    {
+        ffmoe_shape denseShape{(uint32_t)d, (uint32_t)f, 1, 1, 1, 64};
+        Context dense(0, denseShape);
+        const uint8_t *blob = pool.data() + 3 * stride;
+        auto u16 = [&](uint32_t o) { return reinterpret_cast<const uint16_t *>(blob + o); };
+        const SharedExpertProjection gate{blob + off.gate_w, u16(off.gate_s), u16(off.gate_b), (uint32_t)f, (uint32_t)d};
+        const SharedExpertProjection up{blob + off.up_w, u16(off.up_s), u16(off.up_b), (uint32_t)f, (uint32_t)d};
+        const SharedExpertProjection down{blob + off.down_w, u16(off.down_s), u16(off.down_b), (uint32_t)d, (uint32_t)f};
+        PrefillSharedExpert shared(dense);
+        bool threwDims = false;
+        try { shared.load(0, gate, down, down); } catch (const SharedExpertError &e) { threwDims = e.kind == SharedExpertError::dimensionMismatch; }
+        EXPECT(threwDims);
+        bool threwBits = false;
+        try { SharedExpertRuntime bad(dense, 8); } catch (const SharedExpertError &e) { threwBits = e.kind == SharedExpertError::unsupportedWeightBits; }
+        EXPECT(threwBits);
+        shared.load(0, gate, up, down);
+        ffo_offsets fo{off.gate_w, off.gate_s, off.gate_b, off.up_w, off.up_s, off.up_b, off.down_w, off.down_s, off.down_b};
+        std::vector<float> refAll((size_t)T * d), xr(d);
+        for (int r = 0; r < T; ++r) {
+            for (int i = 0; i < d; ++i) xr[i] = ffo_bf16_to_float(x[(size_t)r * d + i]);
+            ffo_run_ffn(blob, &fo, d, f, xr.data(), refAll.data() + (size_t)r * d);
+        }
+        shared.encode(stream, 0, dx, dH2);
+        shared.encodeBlock(stream, 0, dx, dH2b, T, d, f, d, d);
+        HIP(hipStreamSynchronize(stream));
+        double relS = 0, cosS = 0;
+        errorStats(toHost(dH2, (size_t)d), std::vector<float>(refAll.begin(), refAll.begin() + d), relS, cosS);
+        EXPECT(relS <= 1e-2 && cosS >= 0.9999);
+        errorStats(toHost(dH2b, (size_t)T * d), refAll, relS, cosS);
+        EXPECT(relS <= 1e-2 && cosS >= 0.9999);
+    }
+
     std::printf(failures ? "%d FAILURES\n" : "host gpu ok\n", failures);
     return failures ? 1 : 0;
 }

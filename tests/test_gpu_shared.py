@@ -1,0 +1,153 @@
+"""Dense (shared-expert) FFN through the C ABI against the CPU oracle: the single-row operator, its
+multi-row and batched forms, and the upload from separate projections. Run on the GPU box: pytest -m gpu."""
+import numpy as np
+import pytest
+
+from helpers import bf16_tensor, bits_of, cosine, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+@pytest.fixture(scope="module")
+def ff():
+    import fieldfare_moe
+    fieldfare_moe.lib()
+    return fieldfare_moe
+
+
+def _reference_rows(oracle, parts, x_bits):
+    """SharedExpertInt4Tests.swift:24-31 per row: dequant GEMV for gate and up, the activation rounded
+    to 16 bits once, dequant GEMV for down."""
+    (gW, gS, gB), (uW, uS, uB), (dW, dS, dB) = parts
+    out = []
+    for row in x_bits:
+        x = oracle.bf16_to_float(row)
+        g = oracle.gemv_int4_ref(gW, gS, gB, x)
+        u = oracle.gemv_int4_ref(uW, uS, uB, x)
+        act = oracle.bf16_to_float(oracle.bf16_bits(oracle.gelu_tanh(g) * u))
+        out.append(oracle.gemv_int4_ref(dW, dS, dB, act))
+    return np.stack(out)
+
+
+def _context(ff, parts, d, f, max_tokens):
+    ctx = ff.Context(d, f, 1, 1, n_layers=1, max_tokens=max_tokens)
+    ctx.upload_expert_parts(0, 0, *parts)
+    return ctx
+
+
+def test_shared_expert_matches_affine_reference(ff, oracle, torch):
+    # sharedExpertInt4MatchesAffineReference (SharedExpertInt4Tests.swift:13-50): same seed and draw order
+    d, f = 128, 64
+    rng = oracle.seed_tree_key(0x604, "shared-expert-int4")
+    x = rng.uniform(-0.4, 0.4, d)
+    gate = np.stack([rng.uniform(-0.4, 0.4, d) for _ in range(f)])
+    up = np.stack([rng.uniform(-0.4, 0.4, d) for _ in range(f)])
+    down = np.stack([rng.uniform(-0.4, 0.4, f) for _ in range(d)])
+    parts = (oracle.quantize_int4(gate), oracle.quantize_int4(up), oracle.quantize_int4(down))
+    xb = oracle.bf16_bits(x)[None, :]
+    ref = _reference_rows(oracle, parts, xb)
+    ctx = _context(ff, parts, d, f, 16)
+    y = oracle.bf16_to_float(bits_of(ctx.dense_ffn(0, bf16_tensor(torch, xb))))
+    # Tolerance.quantInt4 * 4 (Tolerances.swift:16) is the reference's FP16 bound; bf16 outputs carry 2^-9
+    assert rel_err(y, ref) < 1e-2
+    assert cosine(y, ref) > 0.9999
+    ctx.close()
+
+
+@pytest.mark.parametrize("d,f,t", [(128, 64, 5), (256, 192, 16), (2816, 2112, 1), (2816, 2112, 16)])
+def test_shared_expert_rows(ff, oracle, torch, d, f, t):
+    # rows <= 16: the streaming kernels; (2816, 2112) is the model's shared expert
+    g = oracle.seed_tree_key(0x5EED, f"shared-ffn-d{d}-f{f}-t{t}")
+    scale = 0.4 if d < 1024 else 0.08
+    parts = tuple(oracle.quantize_int4(g.uniform(-scale, scale, r * c).reshape(r, c)) for r, c in ((f, d), (f, d), (d, f)))
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    ref = _reference_rows(oracle, parts, xb)
+    ctx = _context(ff, parts, d, f, 16)
+    x = bf16_tensor(torch, xb)
+    y = bits_of(ctx.dense_ffn(0, x))
+    yf = oracle.bf16_to_float(y)
+    assert rel_err(yf, ref) < 1e-2
+    assert cosine(yf, ref) > 0.9999
+    # a row of a block equals the same row run alone, bit for bit
+    for r in range(0, t, max(1, t // 3)):
+        single = bits_of(ctx.dense_ffn(0, x[r:r + 1]))
+        assert np.array_equal(single[0], y[r]), f"row {r}"
+    ctx.close()
+
+
+@pytest.mark.parametrize("d,f,t", [(128, 64, 40), (256, 192, 300), (2816, 2112, 64)])
+def test_shared_expert_batched(ff, oracle, torch, d, f, t):
+    # more than 16 rows: the grouped GEMMs. 64 rows of U(-2, 2) at the model's shape restate
+    # batchedIsNoLessAccurateThanPerToken (PrefillSharedExpertBatchedTests.swift:47-101), whose reference is
+    # MoeRef.runFFN per token and whose bound is a relative L2 error below 5e-3 on FP16 outputs.
+    g = oracle.seed_tree_key(0x5EED, f"shared-ffn-batched-d{d}-f{f}-t{t}")
+    scale = 0.4 if d < 1024 else 0.05
+    parts = tuple(oracle.quantize_int4(g.uniform(-scale, scale, r * c).reshape(r, c)) for r, c in ((f, d), (f, d), (d, f)))
+    xb = oracle.bf16_bits(g.uniform(-2.0, 2.0, t * d)).reshape(t, d)
+    pool = oracle.pool_from_parts([parts], d, f, align=16)
+    ref = np.stack([oracle.run_ffn(pool, 0, oracle.bf16_to_float(row)) for row in xb])
+    ctx = _context(ff, parts, d, f, max(t, 64))
+    yf = oracle.bf16_to_float(bits_of(ctx.dense_ffn(0, bf16_tensor(torch, xb))))
+    l2 = float(np.sqrt(((yf - ref) ** 2).sum() / (ref ** 2).sum()))
+    assert l2 < 5e-3
+    assert rel_err(yf, ref) < 1e-2
+    assert cosine(yf, ref) > 0.9999
+    # the streaming path on the first rows agrees with the GEMM path to the same bar
+    head = oracle.bf16_to_float(bits_of(ctx.dense_ffn(0, bf16_tensor(torch, xb[:8]))))
+    assert rel_err(head, yf[:8]) < 1e-2
+    ctx.close()
+
+
+def test_parts_upload_equals_blob_upload(ff, oracle, torch):
+    # the same expert through ffmoe_upload_expert_parts (host and device sources) and through a blob
+    d, f = 256, 128
+    rng = np.random.default_rng(11)
+    pool = oracle.random_pool(rng, 2, d, f, align=16)
+    blob = ff.Context(d, f, 2, 2, n_layers=1, max_tokens=16)
+    blob.upload_layer(0, pool.bytes, pool.stride, ff.Offsets(*pool.offsets.as_tuple()))
+    host = ff.Context(d, f, 2, 2, n_layers=1, max_tokens=16)
+    dev = ff.Context(d, f, 2, 2, n_layers=1, max_tokens=16)
+    x = torch.zeros((1, d), dtype=torch.bfloat16, device="cuda")
+    idx = torch.zeros((1, 2), dtype=torch.int32, device="cuda")
+    w = torch.ones((1, 2), dtype=torch.bfloat16, device="cuda")
+    for e in range(2):
+        parts = tuple(pool.sub(e, which) for which in ("gate", "up", "down"))
+        if e == 0:
+            # one of two experts uploaded: the layer is not ready yet
+            host.upload_expert_parts(0, 1, *tuple(pool.sub(1, which) for which in ("gate", "up", "down")))
+            with pytest.raises(ff.FieldfareError, match="not uploaded"):
+                host.verify(0, x, idx, w)
+        host.upload_expert_parts(0, e, *parts)
+        dev.upload_expert_parts(0, e, *tuple(tuple(torch.from_numpy(np.ascontiguousarray(a).view(np.uint8)).cuda()
+                                                   for a in tr) for tr in parts))
+    for e in range(2):
+        for which in (0, 1, 2):
+            ref = bits_of(blob.dequant_expert(0, e, which))
+            assert np.array_equal(bits_of(host.dequant_expert(0, e, which)), ref)
+            assert np.array_equal(bits_of(dev.dequant_expert(0, e, which)), ref)
+    for c in (blob, host, dev):
+        c.close()
+
+
+def test_dense_ffn_argument_errors(ff, oracle, torch):
+    routed = ff.Context(128, 64, 4, 2, n_layers=1, max_tokens=16)
+    x = torch.zeros((1, 128), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ff.FieldfareError, match="n_experts = 1"):
+        routed.dense_ffn(0, x)
+    routed.close()
+    dense = ff.Context(128, 64, 1, 1, n_layers=1, max_tokens=32)
+    with pytest.raises(ff.FieldfareError, match="not uploaded"):
+        dense.dense_ffn(0, x)
+    parts = tuple(oracle.quantize_int4(np.zeros((r, c), np.float32)) for r, c in ((64, 128), (64, 128), (128, 64)))
+    dense.upload_expert_parts(0, 0, *parts)
+    with pytest.raises(ff.FieldfareError, match="exceeds max_tokens"):
+        dense.dense_ffn(0, torch.zeros((33, 128), dtype=torch.bfloat16, device="cuda"))
+    assert float(dense.dense_ffn(0, x).abs().max()) == 0.0
+    dense.close()
