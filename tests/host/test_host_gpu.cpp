@@ -5,9 +5,12 @@
 
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <fstream>
 
 #include "../../ane-fieldfare_amd/host/fieldfare_host.hpp"
+#include "../../ane-fieldfare_amd/host/packed_experts.hpp"
 #include "../../oracle/ffmoe_oracle.h"
 
 using namespace fieldfare;
@@ -250,6 +253,81 @@ int main() {
         EXPECT(relS <= 1e-2 && cosS >= 0.9999);
         errorStats(toHost(dH2b, (size_t)T * d), refAll, relS, cosS);
         EXPECT(relS <= 1e-2 && cosS >= 0.9999);
+    }
+
+    // --- packed experts: a two-layer checkpoint directory written as ModelLoaderTests.swift:204-241 writes its
+    // toy one (16 KiB stride, layout.json with explicit ids), layer 1 with reversed physical ranks; after
+    // uploadPackedExperts every expert expands to the same bf16 weights as the directly uploaded blobs ---
+    {
+        char tmpl[] = "/tmp/ffmoe_ckpt_XXXXXX";
+        const char *dir = mkdtemp(tmpl);
+        EXPECT(dir != nullptr);
+        const std::string root = dir ? dir : "/tmp";
+        EXPECT(std::system(("mkdir -p " + root + "/packed_experts").c_str()) == 0);
+        const uint64_t ckStride = 16384;
+        EXPECT(stride <= ckStride);
+        auto tensorsJson = [&]() {
+            const char *roles[9] = {"gate", "gate_scales", "gate_biases", "up", "up_scales", "up_biases", "down", "down_scales", "down_biases"};
+            const uint32_t offs[9] = {off.gate_w, off.gate_s, off.gate_b, off.up_w, off.up_s, off.up_b, off.down_w, off.down_s, off.down_b};
+            const size_t sizes[9] = {guW, guS, guS, guW, guS, guS, dnW, dnS, dnS};
+            std::string t = "{";
+            for (int i = 0; i < 9; ++i) {
+                const bool wt = i % 3 == 0;
+                const int rows = i < 6 ? f : d, cols = i < 6 ? d : f;
+                t += (i ? "," : "") + std::string("\"") + roles[i] + "\":{\"offset\":" + std::to_string(offs[i]) + ",\"size\":" + std::to_string(sizes[i]) +
+                     ",\"dtype\":\"" + (wt ? "U32" : "BF16") + "\",\"shape\":[" + std::to_string(rows) + "," + std::to_string(wt ? cols : cols / 64) + "]" +
+                     (wt ? ",\"bits\":4" : "") + "}";
+            }
+            return t + "}";
+        };
+        std::string layersJson;
+        for (int L = 0; L < 2; ++L) {
+            std::vector<uint8_t> payload(ckStride * E, 0);
+            std::string expertsJson;
+            for (int e = 0; e < E; ++e) {
+                const int rank = L == 0 ? e : E - 1 - e;
+                std::memcpy(payload.data() + (size_t)rank * ckStride, pool.data() + (size_t)e * stride, stride);
+                expertsJson += (e ? "," : "") + std::string("{\"expert\":") + std::to_string(e) + ",\"physicalRank\":" + std::to_string(rank) +
+                               ",\"offset\":" + std::to_string((uint64_t)rank * ckStride) + ",\"size\":" + std::to_string(ckStride) + ",\"tensors\":" + tensorsJson() + "}";
+            }
+            const std::string file = "layer_0" + std::to_string(L) + ".bin";
+            std::ofstream(root + "/packed_experts/" + file, std::ios::binary).write(reinterpret_cast<const char *>(payload.data()), (std::streamsize)payload.size());
+            layersJson += (L ? "," : "") + std::string("{\"layer\":") + std::to_string(L) + ",\"file\":\"" + file + "\",\"experts\":[" + expertsJson + "]}";
+        }
+        std::ofstream(root + "/packed_experts/layout.json") << "{\"expertStride\":" << ckStride << ",\"numLayers\":2,\"expertsPerLayer\":" << E
+                                                             << ",\"layers\":[" << layersJson << "]}";
+        const PackedExpertsLayout layout = PackedExpertsLayoutReader::read(root);
+        EXPECT(layout.numLayers == 2 && layout.expertsPerLayer == E && layout.expert(1, 0).physicalRank == E - 1);
+        ffmoe_shape ckShape{(uint32_t)d, (uint32_t)f, (uint32_t)E, (uint32_t)K, 2, 64};
+        Context ck(0, ckShape);
+        EXPECT(uploadPackedExperts(ck, root, layout) == 2 * ckStride * E);
+        uint16_t *dA = nullptr, *dB = nullptr;
+        HIP(hipMalloc(reinterpret_cast<void **>(&dA), (size_t)f * d * 2));
+        HIP(hipMalloc(reinterpret_cast<void **>(&dB), (size_t)f * d * 2));
+        int mismatches = 0;
+        for (int L = 0; L < 2; ++L)
+            for (int e = 0; e < E; ++e)
+                for (int which = 0; which < 3; ++which) {
+                    char *err = nullptr;
+                    check(ffmoe_dequant_expert(ctx.raw(), stream, 0, (uint32_t)e, which, dA, &err), err);
+                    check(ffmoe_dequant_expert(ck.raw(), stream, (uint32_t)L, (uint32_t)e, which, dB, &err), err);
+                    HIP(hipStreamSynchronize(stream));
+                    if (toHost(dA, (size_t)f * d) != toHost(dB, (size_t)f * d)) ++mismatches;
+                }
+        EXPECT(mismatches == 0);
+        // a layer file shorter than the layout says, and a shape the context does not have
+        bool threwSize = false;
+        EXPECT(truncate((root + "/packed_experts/layer_01.bin").c_str(), (off_t)(ckStride * (E - 1))) == 0);
+        try { uploadPackedExperts(ck, root, layout); } catch (const MappedExpertLayerError &e) { threwSize = e.kind == MappedExpertLayerError::sizeMismatch; }
+        EXPECT(threwSize);
+        bool threwShape = false;
+        ffmoe_shape other{(uint32_t)d, (uint32_t)(2 * f), (uint32_t)E, (uint32_t)K, 2, 64};
+        Context wrong(0, other);
+        try { uploadPackedExperts(wrong, root, layout); } catch (const GTurboFormatError &) { threwShape = true; }
+        EXPECT(threwShape);
+        HIP(hipFree(dA));
+        HIP(hipFree(dB));
+        EXPECT(std::system(("rm -rf " + root).c_str()) == 0);
     }
 
     std::printf(failures ? "%d FAILURES\n" : "host gpu ok\n", failures);

@@ -1,10 +1,12 @@
 // Host-logic tests of the C++ operator mirror (no GPU): exact expected arrays restated from the reference's
 // PrefillMoEGroupingTests.swift, PrefillRouterTests.swift:12-22, PrefillGroupedRoutedMoETests+Binding.swift and
-// the fault policy of DeviceSupervisorFailoverTests.swift:19-81.
+// the fault policy of DeviceSupervisorFailoverTests.swift:19-81, and the packed-experts layout cases of
+// GTurboFormatCodecTests.swift:47-66,136-183 and ModelLoaderTests.swift:56-90,204-241.
 #include <cstdio>
 #include <cstring>
 
 #include "../../ane-fieldfare_amd/host/fieldfare_host.hpp"
+#include "../../ane-fieldfare_amd/host/packed_experts.hpp"
 
 using namespace fieldfare;
 
@@ -139,6 +141,108 @@ static void supervisorPolicies() {
     }
 }
 
+// FormatFixture.layout (GTurboFormatCodecTests.swift:47-66) as the JSON its encoder writes: one layer, two
+// experts of one 16 KiB stride, one tensor "gate" {offset 0, size 32, U32, [8, 8], bits 4}.
+static std::string fixtureLayoutJson(bool explicitIDs, bool explicitRanks, const std::string &file = "layer_00.bin",
+                                     const std::string &tensor = "{\"offset\":0,\"size\":32,\"dtype\":\"U32\",\"shape\":[8,8],\"bits\":4}") {
+    std::string experts;
+    for (int e = 0; e < 2; ++e) {
+        experts += e ? "," : "";
+        experts += "{";
+        if (explicitIDs) experts += "\"expert\":" + std::to_string(e) + ",";
+        if (explicitRanks) experts += "\"physicalRank\":" + std::to_string(e) + ",";
+        experts += "\"offset\":" + std::to_string(e * 16384) + ",\"size\":16384,\"tensors\":{\"gate\":" + tensor + "}}";
+    }
+    return "{\"expertStride\":16384,\"numLayers\":1,\"expertsPerLayer\":2,\"layers\":[{\"layer\":0,\"file\":\"" + file +
+           "\",\"experts\":[" + experts + "]}]}";
+}
+
+static bool rejects(const std::string &json, const char *needle) {
+    try {
+        PackedExpertsLayoutReader::decode(json);
+    } catch (const GTurboFormatError &e) {
+        return std::string(e.what()).find(needle) != std::string::npos;
+    }
+    return false;
+}
+
+static void packedExpertsLayoutCodec() {
+    // roundTripPreservesIdentityFallback (GTurboFormatCodecTests.swift:137-141): positional ids and ranks
+    for (int mode = 0; mode < 4; ++mode) {
+        const auto layout = PackedExpertsLayoutReader::decode(fixtureLayoutJson(mode & 1, mode & 2));
+        EXPECT(layout.expertStride == 16384 && layout.numLayers == 1 && layout.expertsPerLayer == 2);
+        EXPECT(layout.layers.size() == 1 && layout.layers[0].file == "layer_00.bin" && layout.layers[0].experts.size() == 2);
+        for (int e = 0; e < 2; ++e) {
+            const ExpertEntry &ex = layout.expert(0, e);
+            EXPECT(ex.expert == e && ex.physicalRank == e && ex.offset == (uint64_t)e * 16384 && ex.size == 16384);
+            const SubTensorEntry &t = ex.subTensors.at("gate");
+            EXPECT(t.offset == 0 && t.size == 32 && t.dtype == "U32" && t.shape == std::vector<uint32_t>({8, 8}) && t.bits == 4);
+        }
+        EXPECT(layout.routedExpertPhysicalOffsets(0) == std::vector<uint64_t>({0, 16384}));
+    }
+    // rejectsSlashBearingLayerBasename (:143-152)
+    EXPECT(rejects(fixtureLayoutJson(true, true, "nested/layer.bin"), "expected basename"));
+    EXPECT(rejects(fixtureLayoutJson(true, true, "../layer.bin"), "non-canonical path"));
+    EXPECT(rejects(fixtureLayoutJson(true, true, "/layer.bin"), "unsafe relative path"));
+    EXPECT(rejects(fixtureLayoutJson(true, true, "Layout.JSON"), "reserved packed-expert filename"));
+    // rejectsTensorOutsideExpertBlob (:167-181): offset stride - 8, size 16
+    EXPECT(rejects(fixtureLayoutJson(true, true, "layer_00.bin", "{\"offset\":16376,\"size\":16,\"dtype\":\"U32\",\"shape\":[1],\"bits\":4}"),
+                   "range exceeds expert blob"));
+    // the validator's other guards (GTurboPackedExpertsLayoutV1.swift:73-160)
+    EXPECT(rejects(fixtureLayoutJson(true, true, "layer_00.bin", "{\"offset\":0,\"size\":32,\"dtype\":\"F32\",\"shape\":[8,8]}"), "invalid dtype or shape"));
+    EXPECT(rejects(fixtureLayoutJson(true, true, "layer_00.bin", "{\"offset\":0,\"size\":32,\"dtype\":\"U32\",\"shape\":[8,0]}"), "invalid dtype or shape"));
+    EXPECT(rejects(fixtureLayoutJson(true, true, "layer_00.bin", "{\"offset\":0,\"size\":32,\"dtype\":\"U32\",\"shape\":[8,8],\"bits\":33}"), "invalid dtype or shape"));
+    EXPECT(rejects("{\"expertStride\":1000,\"numLayers\":1,\"expertsPerLayer\":2,\"layers\":[]}", "invalid dimensions or stride"));
+    EXPECT(rejects("{\"expertStride\":16384,\"numLayers\":2,\"expertsPerLayer\":2,\"layers\":[]}", "invalid dimensions or stride"));
+    {   // ids must be all explicit or all positional; offsets must follow the physical rank
+        std::string mixed = fixtureLayoutJson(true, false);
+        mixed.replace(mixed.find("\"expert\":1,"), 11, "");
+        EXPECT(rejects(mixed, "either all explicit or all positional"));
+        std::string moved = fixtureLayoutJson(true, true);
+        moved.replace(moved.find("\"offset\":16384"), 14, "\"offset\":32768");
+        EXPECT(rejects(moved, "offset or size does not match physical rank"));
+        std::string dup = fixtureLayoutJson(true, true);
+        dup.replace(dup.find("\"expert\":1"), 10, "\"expert\":0");
+        EXPECT(rejects(dup, "duplicate or invalid expert mapping"));
+    }
+    {   // two tensors that overlap
+        const std::string two = "{\"expertStride\":16384,\"numLayers\":1,\"expertsPerLayer\":1,\"layers\":[{\"layer\":0,\"file\":\"l.bin\",\"experts\":["
+                                "{\"offset\":0,\"size\":16384,\"tensors\":{\"gate\":{\"offset\":0,\"size\":32,\"dtype\":\"U32\",\"shape\":[8,8]},"
+                                "\"gate_scales\":{\"offset\":16,\"size\":32,\"dtype\":\"BF16\",\"shape\":[8,2]}}}]}]}";
+        EXPECT(rejects(two, "overlapping ranges gate and gate_scales"));
+    }
+    {   // truncated and malformed documents
+        bool truncated = false;
+        try { PackedExpertsLayoutReader::decode("{\"expertStride\":16384,"); } catch (const GTurboFormatError &e) { truncated = e.kind == GTurboFormatError::truncated; }
+        EXPECT(truncated);
+        EXPECT(rejects("[1,2]", "expected an object"));
+        bool overflow = false;
+        try { PackedExpertsLayoutReader::decode("{\"expertStride\":99999999999999999999999}"); } catch (const GTurboFormatError &e) { overflow = e.kind == GTurboFormatError::overflow; }
+        EXPECT(overflow);
+    }
+    {   // a permuted layer: logical expert 0 at physical rank 1; experts come back sorted by logical id, and the
+        // nine routed offsets are read from expert 0 (Model.routedExpertOffsets, ModelExpertIO.swift:11-30)
+        auto tensors = [](int base) {
+            const char *roles[9] = {"gate", "gate_scales", "gate_biases", "up", "up_scales", "up_biases", "down", "down_scales", "down_biases"};
+            std::string t = "{";
+            for (int i = 0; i < 9; ++i) {
+                t += i ? "," : "";
+                t += std::string("\"") + roles[i] + "\":{\"offset\":" + std::to_string(base + 64 * i) + ",\"size\":64,\"dtype\":\"" +
+                     (i % 3 == 0 ? "U32" : "BF16") + "\",\"shape\":[4,4]}";
+            }
+            return t + "}";
+        };
+        const std::string json = "{\"expertStride\":16384,\"numLayers\":1,\"expertsPerLayer\":2,\"layers\":[{\"layer\":0,\"file\":\"layer_00.bin\",\"experts\":["
+                                 "{\"expert\":1,\"physicalRank\":0,\"offset\":0,\"size\":16384,\"tensors\":" + tensors(0) + "},"
+                                 "{\"expert\":0,\"physicalRank\":1,\"offset\":16384,\"size\":16384,\"tensors\":" + tensors(128) + "}]}]}";
+        const auto layout = PackedExpertsLayoutReader::decode(json);
+        EXPECT(layout.expert(0, 0).physicalRank == 1 && layout.expert(0, 1).physicalRank == 0);
+        EXPECT(layout.routedExpertPhysicalOffsets(0) == std::vector<uint64_t>({16384, 0}));
+        const ffmoe_offsets o = layout.routedExpertOffsets(0);
+        EXPECT(o.gate_w == 128 && o.gate_s == 192 && o.gate_b == 256 && o.up_w == 320 && o.down_b == 128 + 64 * 8);
+    }
+}
+
 int main() {
     groupingSortsPairsAndBuildsOffsetsCountsAndTiles();
     groupingCanOrderTilesByExpertSortKeys();
@@ -146,6 +250,7 @@ int main() {
     tokenExpertPairsAreTokenMajor();
     streamedTileBinding();
     supervisorPolicies();
+    packedExpertsLayoutCodec();
     std::printf(failures ? "%d FAILURES\n" : "host logic ok\n", failures);
     return failures ? 1 : 0;
 }
