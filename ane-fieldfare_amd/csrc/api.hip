@@ -455,6 +455,42 @@ int ffmoe_prefill_plan_stats(ffmoe_ctx *ctx, void *stream, uint32_t *n_pairs, ui
     return FFMOE_OK;
 }
 
+static int check_rows(uint32_t t, uint32_t d, const uint32_t *strides, int n_strides, char **err) {
+    if (t == 0) return fail(err, FFMOE_ERR_INVALID, "queryCount must be positive");
+    if (d == 0 || d > FFMOE_ROW_MAX_D || d % 8) return fail(err, FFMOE_ERR_INVALID, "D must be a multiple of 8 in 8...%d", FFMOE_ROW_MAX_D);
+    for (int i = 0; i < n_strides; ++i)
+        if (strides[i] < d) return fail(err, FFMOE_ERR_INVALID, "a row stride is too small");
+    return FFMOE_OK;
+}
+
+int ffmoe_post_attn_setup(ffmoe_ctx *ctx, void *stream, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *attn,
+                          uint32_t attn_stride, uint16_t *dense_x, uint32_t dense_stride, uint16_t *routed_x,
+                          uint32_t routed_stride, uint16_t *router_x, uint32_t router_stride, const uint16_t *w_post_attn,
+                          const uint16_t *w_pre_ffn, const uint16_t *w_pre_ffn2, uint32_t t, uint32_t d, float eps,
+                          char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!hidden || !attn || !dense_x || !routed_x || !router_x || !w_post_attn || !w_pre_ffn || !w_pre_ffn2)
+        return fail(err, FFMOE_ERR_INVALID, "null argument");
+    const uint32_t strides[5] = {hidden_stride, attn_stride, dense_stride, routed_stride, router_stride};
+    if (int rc = check_rows(t, d, strides, 5, err)) return rc;
+    FF_HIP(launch_post_attn_setup(static_cast<hipStream_t>(stream), hidden, hidden_stride, attn, attn_stride, dense_x,
+                                  dense_stride, routed_x, routed_stride, router_x, router_stride, w_post_attn, w_pre_ffn,
+                                  w_pre_ffn2, t, d, eps));
+    return FFMOE_OK;
+}
+
+int ffmoe_layer_tail(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1,
+                     uint32_t h1_stride, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2,
+                     const uint16_t *w_postffn, uint32_t t, uint32_t d, float eps, float layer_scalar, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!h2 || !h1 || !hidden || !w_postffn2 || !w_postffn) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    const uint32_t strides[3] = {h2_stride, h1_stride, hidden_stride};
+    if (int rc = check_rows(t, d, strides, 3, err)) return rc;
+    FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), h2, h2_stride, h1, h1_stride, hidden, hidden_stride,
+                             w_postffn2, w_postffn, t, d, eps, layer_scalar));
+    return FFMOE_OK;
+}
+
 int ffmoe_set_profiling(ffmoe_ctx *ctx, int enabled, char **err) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (enabled && !ctx->timer.ev[0])

@@ -1,0 +1,202 @@
+// The steps either side of the MoE stage, one block per token row:
+//   post-attention setup  fused_post_attn_setup (Metal/Fusions/fused.metal:210-296) and its block form
+//                         prefill_post_attn_setup_block (Metal/Prefill/prefill.metal:243-318)
+//   layer tail            prefill_layer_tail_block (Metal/Prefill/prefill.metal:320-399) and the decode
+//                         tail of Kernels/Fusions/FusedLayerTail.swift
+// Both are RMS norms around residual adds with every intermediate rounded to 16 bits where the reference
+// rounds to FP16. A thread keeps its elements in registers from the first read to the last write (the
+// reference stages rows in threadgroup memory); a row is read once and written once: HBM-bound.
+//
+// Summation order of the squares (the reference's simd_sum leaves it open): thread t owns the 8-element
+// chunks t, t + 256, ... and adds their squares in index order with fmaf; the wave meets in a
+// xor-butterfly; the four wave sums combine as (w0 + w1) + (w2 + w3); inv = 1 / sqrt(sum / D + eps) with
+// IEEE division and square root. Rows that are not 16-byte aligned take scalar loads of the same elements,
+// so both paths give the same bits.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace ffmoe {
+namespace {
+
+constexpr int kRowThreads = 256;
+constexpr int kMaxChunks = 2;        // D <= 4096: at most two 8-element chunks per thread
+
+struct Row8 {
+    float v[8];
+};
+
+template <bool VEC>
+__device__ __forceinline__ Row8 load8(const uint16_t *__restrict__ row, uint32_t chunk) {
+    Row8 r;
+    if (VEC) {
+        const uint4 q = reinterpret_cast<const uint4 *>(row)[chunk];
+        r.v[0] = bf16lo_to_f32(q.x); r.v[1] = bf16hi_to_f32(q.x);
+        r.v[2] = bf16lo_to_f32(q.y); r.v[3] = bf16hi_to_f32(q.y);
+        r.v[4] = bf16lo_to_f32(q.z); r.v[5] = bf16hi_to_f32(q.z);
+        r.v[6] = bf16lo_to_f32(q.w); r.v[7] = bf16hi_to_f32(q.w);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r.v[e] = bf16_to_f32(row[8 * chunk + e]);
+    }
+    return r;
+}
+
+template <bool VEC>
+__device__ __forceinline__ void store8(uint16_t *__restrict__ row, uint32_t chunk, const Row8 &r) {
+    if (VEC) {
+        uint4 q;
+        q.x = pack_bf16x2(r.v[0], r.v[1]);
+        q.y = pack_bf16x2(r.v[2], r.v[3]);
+        q.z = pack_bf16x2(r.v[4], r.v[5]);
+        q.w = pack_bf16x2(r.v[6], r.v[7]);
+        reinterpret_cast<uint4 *>(row)[chunk] = q;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) row[8 * chunk + e] = f32_to_bf16(r.v[e]);
+    }
+}
+
+__device__ __forceinline__ float round_bf16(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+
+// 1 / sqrt(mean of squares + eps) over the block's row; `slot` is a 4-float LDS area of its own
+__device__ __forceinline__ float block_rms_inv(const Row8 (&x)[kMaxChunks], uint32_t n_mine, uint32_t d, float eps,
+                                               float *slot) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if ((uint32_t)c < n_mine)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(x[c].v[e], x[c].v[e], acc);
+    acc = wave_butterfly_sum(acc);
+    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    const float total = (slot[0] + slot[1]) + (slot[2] + slot[3]);
+    return 1.0f / sqrtf(total / (float)d + eps);
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kRowThreads) void post_attn_setup_kernel(
+    uint16_t *__restrict__ hidden, uint32_t hidden_stride, const uint16_t *__restrict__ attn, uint32_t attn_stride,
+    uint16_t *__restrict__ dense_x, uint32_t dense_stride, uint16_t *__restrict__ routed_x, uint32_t routed_stride,
+    uint16_t *__restrict__ router_x, uint32_t router_stride, const uint16_t *__restrict__ w_post_attn,
+    const uint16_t *__restrict__ w_pre_ffn, const uint16_t *__restrict__ w_pre_ffn2, uint32_t d, float eps) {
+    __shared__ float s_sum[2][4];
+    const uint32_t row = blockIdx.x, t = threadIdx.x, chunks = d / 8;
+    const uint32_t n_mine = t < chunks ? (chunks - t + kRowThreads - 1) / kRowThreads : 0;
+    uint16_t *hrow = hidden + (size_t)row * hidden_stride;
+    const uint16_t *arow = attn + (size_t)row * attn_stride;
+    Row8 a[kMaxChunks], h[kMaxChunks];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if ((uint32_t)c < n_mine) {
+            a[c] = load8<VEC>(arow, t + c * kRowThreads);
+            h[c] = load8<VEC>(hrow, t + c * kRowThreads);
+        }
+    const float attn_inv = block_rms_inv(a, n_mine, d, eps, s_sum[0]);
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if ((uint32_t)c < n_mine) {
+            const Row8 w = load8<VEC>(w_post_attn, t + c * kRowThreads);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[c].v[e] = round_bf16(h[c].v[e] + round_bf16(a[c].v[e] * attn_inv * w.v[e]));
+            store8<VEC>(hrow, t + c * kRowThreads, h[c]);
+        }
+    const float hidden_inv = block_rms_inv(h, n_mine, d, eps, s_sum[1]);
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if ((uint32_t)c < n_mine) {
+            const uint32_t chunk = t + c * kRowThreads;
+            const Row8 w1 = load8<VEC>(w_pre_ffn, chunk), w2 = load8<VEC>(w_pre_ffn2, chunk);
+            Row8 o_dense, o_routed, o_router;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float v = h[c].v[e] * hidden_inv;
+                o_dense.v[e] = v * w1.v[e];
+                o_routed.v[e] = v * w2.v[e];
+                o_router.v[e] = v;
+            }
+            store8<VEC>(dense_x + (size_t)row * dense_stride, chunk, o_dense);
+            store8<VEC>(routed_x + (size_t)row * routed_stride, chunk, o_routed);
+            store8<VEC>(router_x + (size_t)row * router_stride, chunk, o_router);
+        }
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kRowThreads) void layer_tail_kernel(const uint16_t *__restrict__ h2, uint32_t h2_stride,
+                                                                 const uint16_t *__restrict__ h1, uint32_t h1_stride,
+                                                                 uint16_t *__restrict__ hidden, uint32_t hidden_stride,
+                                                                 const uint16_t *__restrict__ w_postffn2,
+                                                                 const uint16_t *__restrict__ w_postffn, uint32_t d,
+                                                                 float eps, float layer_scalar) {
+    __shared__ float s_sum[2][4];
+    const uint32_t row = blockIdx.x, t = threadIdx.x, chunks = d / 8;
+    const uint32_t n_mine = t < chunks ? (chunks - t + kRowThreads - 1) / kRowThreads : 0;
+    uint16_t *hrow = hidden + (size_t)row * hidden_stride;
+    Row8 a[kMaxChunks], h12[kMaxChunks];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if ((uint32_t)c < n_mine) {
+            a[c] = load8<VEC>(h2 + (size_t)row * h2_stride, t + c * kRowThreads);
+            h12[c] = load8<VEC>(h1 + (size_t)row * h1_stride, t + c * kRowThreads);
+        }
+    const float inv_h2 = block_rms_inv(a, n_mine, d, eps, s_sum[0]);
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if ((uint32_t)c < n_mine) {
+            const Row8 w = load8<VEC>(w_postffn2, t + c * kRowThreads);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h12[c].v[e] = round_bf16(h12[c].v[e] + round_bf16(a[c].v[e] * inv_h2 * w.v[e]));
+        }
+    const float inv_h12 = block_rms_inv(h12, n_mine, d, eps, s_sum[1]);
+    const float scale = round_bf16(layer_scalar);
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if ((uint32_t)c < n_mine) {
+            const uint32_t chunk = t + c * kRowThreads;
+            const Row8 w = load8<VEC>(w_postffn, chunk);
+            Row8 hv = load8<VEC>(hrow, chunk);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                hv.v[e] = round_bf16(hv.v[e] + round_bf16(h12[c].v[e] * inv_h12 * w.v[e])) * scale;
+            store8<VEC>(hrow, chunk, hv);
+        }
+}
+
+bool aligned16(const void *p, uint32_t stride) { return reinterpret_cast<uintptr_t>(p) % 16 == 0 && stride % 8 == 0; }
+
+}  // namespace
+
+hipError_t launch_post_attn_setup(hipStream_t s, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *attn,
+                                  uint32_t attn_stride, uint16_t *dense_x, uint32_t dense_stride, uint16_t *routed_x,
+                                  uint32_t routed_stride, uint16_t *router_x, uint32_t router_stride,
+                                  const uint16_t *w_post_attn, const uint16_t *w_pre_ffn, const uint16_t *w_pre_ffn2,
+                                  uint32_t t, uint32_t d, float eps) {
+    const bool vec = aligned16(hidden, hidden_stride) && aligned16(attn, attn_stride) && aligned16(dense_x, dense_stride) &&
+                     aligned16(routed_x, routed_stride) && aligned16(router_x, router_stride) && aligned16(w_post_attn, 8) &&
+                     aligned16(w_pre_ffn, 8) && aligned16(w_pre_ffn2, 8);
+    if (vec)
+        hipLaunchKernelGGL(post_attn_setup_kernel<true>, dim3(t), dim3(kRowThreads), 0, s, hidden, hidden_stride, attn, attn_stride,
+                           dense_x, dense_stride, routed_x, routed_stride, router_x, router_stride, w_post_attn, w_pre_ffn,
+                           w_pre_ffn2, d, eps);
+    else
+        hipLaunchKernelGGL(post_attn_setup_kernel<false>, dim3(t), dim3(kRowThreads), 0, s, hidden, hidden_stride, attn, attn_stride,
+                           dense_x, dense_stride, routed_x, routed_stride, router_x, router_stride, w_post_attn, w_pre_ffn,
+                           w_pre_ffn2, d, eps);
+    return hipGetLastError();
+}
+
+hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1, uint32_t h1_stride,
+                             uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
+                             uint32_t t, uint32_t d, float eps, float layer_scalar) {
+    const bool vec = aligned16(h2, h2_stride) && aligned16(h1, h1_stride) && aligned16(hidden, hidden_stride) &&
+                     aligned16(w_postffn2, 8) && aligned16(w_postffn, 8);
+    if (vec)
+        hipLaunchKernelGGL(layer_tail_kernel<true>, dim3(t), dim3(kRowThreads), 0, s, h2, h2_stride, h1, h1_stride, hidden,
+                           hidden_stride, w_postffn2, w_postffn, d, eps, layer_scalar);
+    else
+        hipLaunchKernelGGL(layer_tail_kernel<false>, dim3(t), dim3(kRowThreads), 0, s, h2, h2_stride, h1, h1_stride, hidden,
+                           hidden_stride, w_postffn2, w_postffn, d, eps, layer_scalar);
+    return hipGetLastError();
+}
+
+}  // namespace ffmoe

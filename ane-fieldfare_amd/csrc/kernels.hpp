@@ -150,6 +150,16 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
                           const ffmoe_pair *pairs, uint32_t n_pairs_in, uint16_t *y, uint16_t *partials_out,
                           PrefillScratch sc, KernelTimer *timer);
 
+// epilogue.hip: row-wise steps either side of the MoE stage
+hipError_t launch_post_attn_setup(hipStream_t s, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *attn,
+                                  uint32_t attn_stride, uint16_t *dense_x, uint32_t dense_stride, uint16_t *routed_x,
+                                  uint32_t routed_stride, uint16_t *router_x, uint32_t router_stride,
+                                  const uint16_t *w_post_attn, const uint16_t *w_pre_ffn, const uint16_t *w_pre_ffn2,
+                                  uint32_t t, uint32_t d, float eps);
+hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1, uint32_t h1_stride,
+                             uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
+                             uint32_t t, uint32_t d, float eps, float layer_scalar);
+
 // gemv.hip
 hipError_t launch_gemv_int4(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                             const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows,

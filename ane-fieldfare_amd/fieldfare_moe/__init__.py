@@ -44,7 +44,8 @@ EXPORTS = [
     "ffmoe_verify", "ffmoe_verify_partials", "ffmoe_last_live_experts", "ffmoe_reduce_token_major",
     "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
-    "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn",
+    "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
+    "ffmoe_layer_tail",
 ]
 
 PROFILE_SLOTS = 16
@@ -165,6 +166,9 @@ def lib() -> C.CDLL:
     L.ffmoe_upload_expert_parts.argtypes = [vp, u32, u32, C.POINTER(Projection), C.POINTER(Projection),
                                             C.POINTER(Projection), i32, errp]
     L.ffmoe_dense_ffn.argtypes = [vp, vp, u32, vp, u32, u32, vp, errp]
+    L.ffmoe_post_attn_setup.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, u32, vp, u32, vp, vp, vp, u32, u32,
+                                        C.c_float, errp]
+    L.ffmoe_layer_tail.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, vp, u32, u32, C.c_float, C.c_float, errp]
     _lib = L
     return L
 
@@ -383,6 +387,32 @@ class Context:
         _check(self.L.ffmoe_prefill_plan_stats(self._h, _stream(), C.byref(n_pairs), C.byref(n_tiles),
                                                C.c_void_p(counts.ctypes.data), C.byref(err)), err)
         return int(n_pairs.value), int(n_tiles.value), counts
+
+    # -- steps either side of the MoE stage ------------------------------------------------------
+    def post_attn_setup(self, hidden, attn, w_post_attn, w_pre_ffn, w_pre_ffn2, eps: float = 1e-6, d: int | None = None,
+                        out=None):
+        """hidden (updated in place), attn: bf16 CUDA tensors [t, >= d] (row stride = their second stride);
+        returns (dense_x, routed_x, router_x), each [t, d] unless `out` gives three tensors to fill."""
+        import torch
+        t = hidden.shape[0]
+        d = d or self.shape.d
+        outs = out if out is not None else tuple(torch.empty((t, d), dtype=torch.bfloat16, device=hidden.device) for _ in range(3))
+        err = C.c_char_p()
+        _check(self.L.ffmoe_post_attn_setup(self._h, _stream(), _ptr(hidden), _row_stride(hidden), _ptr(attn), _row_stride(attn),
+                                            _ptr(outs[0]), _row_stride(outs[0]), _ptr(outs[1]), _row_stride(outs[1]),
+                                            _ptr(outs[2]), _row_stride(outs[2]), _ptr(w_post_attn), _ptr(w_pre_ffn),
+                                            _ptr(w_pre_ffn2), t, d, eps, C.byref(err)), err)
+        return outs
+
+    def layer_tail(self, h2, h1, hidden, w_postffn2, w_postffn, layer_scalar: float, eps: float = 1e-6, d: int | None = None):
+        """hidden = (hidden + norm(h1 + norm(h2))) * layer_scalar, in place; bf16 CUDA tensors [t, >= d]."""
+        t = hidden.shape[0]
+        d = d or self.shape.d
+        err = C.c_char_p()
+        _check(self.L.ffmoe_layer_tail(self._h, _stream(), _ptr(h2), _row_stride(h2), _ptr(h1), _row_stride(h1), _ptr(hidden),
+                                       _row_stride(hidden), _ptr(w_postffn2), _ptr(w_postffn), t, d, eps, layer_scalar,
+                                       C.byref(err)), err)
+        return hidden
 
     # -- generic GEMV ----------------------------------------------------------------------------
     def matrix(self, W, S, B, greedy: bool = False, w_byte_offset: int = 0):

@@ -453,6 +453,70 @@ public:
 };
 
 // ---------------------------------------------------------------------------------------------------
+// The steps either side of the MoE stage. PrefillPostAttentionSetup / PrefillLayerTail
+// (Kernels/Prefill/Epilogues/) take blocks of rows; FusedPostAttentionSetup / FusedLayerTail
+// (Kernels/Fusions/) are their one-row decode forms. Same preconditions as the Swift classes.
+// ---------------------------------------------------------------------------------------------------
+class PrefillPostAttentionSetup {
+public:
+    explicit PrefillPostAttentionSetup(Context &c) : c_(c) {}
+    void encode(void *stream, uint16_t *hidden, const uint16_t *attn, uint16_t *denseX, uint16_t *routedX, uint16_t *routerX,
+                const uint16_t *postAttnWeight, const uint16_t *preFFNWeight, const uint16_t *preFFN2Weight, uint32_t queryCount,
+                uint32_t d, uint32_t hiddenStrideElements, uint32_t attnStrideElements, uint32_t denseStrideElements,
+                uint32_t routedStrideElements, uint32_t routerStrideElements, float eps) {
+        if (queryCount == 0) throw std::invalid_argument("queryCount must be positive");
+        if (d == 0 || d > FFMOE_ROW_MAX_D) throw std::invalid_argument("D must be in 1...4096");
+        char *err = nullptr;
+        check(ffmoe_post_attn_setup(c_.raw(), stream, hidden, hiddenStrideElements, attn, attnStrideElements, denseX,
+                                    denseStrideElements, routedX, routedStrideElements, routerX, routerStrideElements, postAttnWeight,
+                                    preFFNWeight, preFFN2Weight, queryCount, d, eps, &err), err);
+    }
+
+protected:
+    Context &c_;
+};
+
+class FusedPostAttentionSetup : public PrefillPostAttentionSetup {
+public:
+    using PrefillPostAttentionSetup::PrefillPostAttentionSetup;
+    void encode(void *stream, uint16_t *hidden, const uint16_t *attn, uint16_t *denseX, uint16_t *routedX, uint16_t *routerX,
+                const uint16_t *postAttnWeight, const uint16_t *preFFNWeight, const uint16_t *preFFN2Weight, uint32_t d, float eps) {
+        PrefillPostAttentionSetup::encode(stream, hidden, attn, denseX, routedX, routerX, postAttnWeight, preFFNWeight, preFFN2Weight,
+                                          1, d, d, d, d, d, d, eps);
+    }
+};
+
+class PrefillLayerTail {
+public:
+    explicit PrefillLayerTail(Context &c) : c_(c) {}
+    // encode (PrefillLayerTail.swift:11-51)
+    void encode(void *stream, const uint16_t *h2, const uint16_t *h1, uint16_t *hidden, const uint16_t *postFFN2Weight,
+                const uint16_t *postFFNWeight, uint32_t queryCount, uint32_t d, uint32_t h2StrideElements, uint32_t h1StrideElements,
+                uint32_t hiddenStrideElements, float eps, float layerScalar) {
+        if (queryCount == 0) throw std::invalid_argument("queryCount must be positive");
+        if (d == 0 || d > FFMOE_ROW_MAX_D) throw std::invalid_argument("D must be in 1...4096");
+        if (h2StrideElements < d) throw std::invalid_argument("h2 stride is too small");
+        if (h1StrideElements < d) throw std::invalid_argument("h1 stride is too small");
+        if (hiddenStrideElements < d) throw std::invalid_argument("hidden stride is too small");
+        char *err = nullptr;
+        check(ffmoe_layer_tail(c_.raw(), stream, h2, h2StrideElements, h1, h1StrideElements, hidden, hiddenStrideElements, postFFN2Weight,
+                               postFFNWeight, queryCount, d, eps, layerScalar, &err), err);
+    }
+
+protected:
+    Context &c_;
+};
+
+class FusedLayerTail : public PrefillLayerTail {
+public:
+    using PrefillLayerTail::PrefillLayerTail;
+    void encode(void *stream, const uint16_t *h2, const uint16_t *h1, uint16_t *hidden, const uint16_t *postFFN2Weight,
+                const uint16_t *postFFNWeight, uint32_t d, float eps, float layerScalar) {
+        PrefillLayerTail::encode(stream, h2, h1, hidden, postFFN2Weight, postFFNWeight, 1, d, d, d, d, eps, layerScalar);
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------
 // Guest plugin and supervisor (Runtime/Supervisor/DeviceSupervisor.swift:5-125).
 // ---------------------------------------------------------------------------------------------------
 enum class RuntimeFaultPolicy { failClosed, failoverHost };   // reference: .failClosed / .failoverMetal

@@ -341,6 +341,24 @@ def main():
         extra["shared_expert"] = shared
         dense.close()
 
+    # The row-wise steps either side of the MoE stage at the prefill chunk and at a verify block:
+    # 2 row reads + 4 row writes (setup), 3 reads + 1 write (tail); weights stay in cache
+    if not args.no_shared:
+        rowk = {}
+        for rows_ in sorted({T, args.prefill_tokens} - {0}):
+            hid = torch.randn((rows_, D), device="cuda", generator=gen).to(torch.bfloat16)
+            att = torch.randn((rows_, D), device="cuda", generator=gen).to(torch.bfloat16)
+            h1_ = torch.randn((rows_, D), device="cuda", generator=gen).to(torch.bfloat16)
+            wn = [(torch.rand((D,), device="cuda", generator=gen) + 0.5).to(torch.bfloat16) for _ in range(5)]
+            outs_ = tuple(torch.empty((rows_, D), dtype=torch.bfloat16, device="cuda") for _ in range(3))
+            ts = timed(lambda: ctx.post_attn_setup(hid, att, wn[0], wn[1], wn[2], out=outs_), 50)
+            tt = timed(lambda: ctx.layer_tail(att, h1_, hid, wn[3], wn[4], 1.0), 50)
+            row_bytes = rows_ * D * 2
+            rowk[f"rows{rows_}"] = {"post_attn_setup_us": round(ts * 1e6, 2), "post_attn_setup_GBs": round(6 * row_bytes / ts / 1e9, 1),
+                                    "layer_tail_us": round(tt * 1e6, 2), "layer_tail_GBs": round(4 * row_bytes / tt / 1e9, 1)}
+            del hid, att, h1_, outs_
+        extra["row_kernels"] = rowk
+
     # BASELINE.json config 5: all layers resident, one 8,192-token prefill with Zipf(1.1) routing imposed on
     # the experts, then 256 decode steps as 16 verify blocks of 16 tokens, the LM head once per block
     sweep = None

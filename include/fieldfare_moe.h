@@ -257,6 +257,37 @@ int ffmoe_upload_expert_parts(ffmoe_ctx *ctx, uint32_t layer, uint32_t expert, c
 int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
                     uint32_t t, uint16_t *y, char **err);
 
+/* ---- the steps either side of the MoE stage ------------------------------------------------------ */
+
+#define FFMOE_ROW_MAX_D 4096  /* kFusedMaxD / kPrefillPostMaxD: Kernels/Prefill/Epilogues/PrefillLayerTail.swift:27 */
+
+/* After attention and its output projection, for each of t rows:
+ *   attn = rmsnorm(attn, w_post_attn); hidden += attn (in place);
+ *   dense_x = rmsnorm(hidden, w_pre_ffn); routed_x = rmsnorm(hidden, w_pre_ffn2); router_x = rmsnorm(hidden)
+ * every result rounded to bf16 where the reference rounds to FP16. dense_x feeds the shared expert
+ * (ffmoe_dense_ffn), routed_x the routed experts, router_x the router. Replaces fused_post_attn_setup
+ * (Metal/Fusions/fused.metal:210-296, Kernels/Fusions/FusedPostAttentionSetup.swift) for t = 1 and
+ * prefill_post_attn_setup_block (Metal/Prefill/prefill.metal:243-318,
+ * Kernels/Prefill/Epilogues/PrefillPostAttentionSetup.swift) for a block. All pointers are device memory;
+ * rows are bf16 with strides in elements (>= d, any 2-byte alignment: 16-byte aligned rows take the fast
+ * path, the bits are the same); weights are bf16 [d]; d is a multiple of 8, at most FFMOE_ROW_MAX_D.
+ * Bytes outside the d used elements of a row are left alone. Needs no uploaded layer. */
+int ffmoe_post_attn_setup(ffmoe_ctx *ctx, void *stream, uint16_t *hidden, uint32_t hidden_stride,
+                          const uint16_t *attn, uint32_t attn_stride, uint16_t *dense_x, uint32_t dense_stride,
+                          uint16_t *routed_x, uint32_t routed_stride, uint16_t *router_x, uint32_t router_stride,
+                          const uint16_t *w_post_attn, const uint16_t *w_pre_ffn, const uint16_t *w_pre_ffn2,
+                          uint32_t t, uint32_t d, float eps, char **err);
+
+/* After the FFNs, for each of t rows (h1 = shared-expert output, h2 = combined routed output):
+ *   h12 = h1 + rmsnorm(h2, w_postffn2); hidden = (hidden + rmsnorm(h12, w_postffn)) * layer_scalar
+ * in place, every step rounded to bf16 as the reference rounds to FP16 (cpuReference,
+ * Tests/.../Kernels/Fusions/FusedLayerTailTests.swift:96-110). Replaces prefill_layer_tail_block
+ * (Metal/Prefill/prefill.metal:320-399, Kernels/Prefill/Epilogues/PrefillLayerTail.swift:11-51) and
+ * FusedLayerTail.encode (Kernels/Fusions/FusedLayerTail.swift). Same pointer rules as above. */
+int ffmoe_layer_tail(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1,
+                     uint32_t h1_stride, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2,
+                     const uint16_t *w_postffn, uint32_t t, uint32_t d, float eps, float layer_scalar, char **err);
+
 /* ---- per-kernel timing ------------------------------------------------------------------------ */
 
 /* Kernel slots of ffmoe_profile. */

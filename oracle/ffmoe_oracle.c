@@ -465,6 +465,84 @@ void ffo_moe_layer(const uint8_t *pool, size_t stride, const ffo_offsets *o, int
     ffo_moe_experts(pool, stride, o, d, f, x, x_stride, t, top_k, dtype, idx_out, w_out, y, n_threads);
 }
 
+/* --- the steps either side of the MoE stage: post-attention setup and layer tail ---
+ * Row-wise RMS norms around residual adds. The reference reduces the squares with simd_sum, whose
+ * order is unspecified; this build pins one: thread t of 256 owns the 8-element chunks t, t + 256, ...
+ * and sums their squares in index order with fmaf; the 64 threads of a wave meet in a xor-butterfly
+ * (32,16,8,4,2,1) of plain adds; the four wave sums combine as (w0 + w1) + (w2 + w3);
+ * inv = 1 / sqrt(sum / D + eps) with IEEE division and square root. d is a multiple of 8. */
+static float rms_inv_pinned(const float *x, int d, float eps) {
+    float lane[256];
+    const int chunks = d / 8;
+    for (int t = 0; t < 256; ++t) {
+        float acc = 0.0f;
+        for (int c = t; c < chunks; c += 256)
+            for (int e = 0; e < 8; ++e) acc = fmaf(x[8 * c + e], x[8 * c + e], acc);
+        lane[t] = acc;
+    }
+    float wave[4];
+    for (int w = 0; w < 4; ++w) {
+        float v[64];
+        memcpy(v, lane + 64 * w, sizeof v);
+        for (int m = 32; m >= 1; m >>= 1) {
+            float nv[64];
+            for (int l = 0; l < 64; ++l) nv[l] = v[l] + v[l ^ m];
+            memcpy(v, nv, sizeof v);
+        }
+        wave[w] = v[0];
+    }
+    const float total = (wave[0] + wave[1]) + (wave[2] + wave[3]);
+    return 1.0f / sqrtf(total / (float)d + eps);
+}
+
+/* fused_post_attn_setup (Metal/Fusions/fused.metal:210-296) = one row of prefill_post_attn_setup_block
+ * (Metal/Prefill/prefill.metal:243-318): attn = norm(attn, w_post_attn) rounded; hidden += attn, rounded,
+ * in place; from the norm of that hidden: dense_x (w_pre_ffn), routed_x (w_pre_ffn2), router_x (no weight). */
+void ffo_post_attn_setup(uint16_t *hidden, const uint16_t *attn, uint16_t *dense_x, uint16_t *routed_x,
+                         uint16_t *router_x, const uint16_t *w_post_attn, const uint16_t *w_pre_ffn,
+                         const uint16_t *w_pre_ffn2, int d, float eps, int dtype) {
+    float *a = (float *)calloc((size_t)d, sizeof(float)), *h = (float *)calloc((size_t)d, sizeof(float));
+    for (int i = 0; i < d; ++i) a[i] = ffo_from_bits16(attn[i], dtype);
+    const float attn_inv = rms_inv_pinned(a, d, eps);
+    for (int i = 0; i < d; ++i) {
+        const float an = ffo_round16(a[i] * attn_inv * ffo_bf16_to_float(w_post_attn[i]), dtype);
+        hidden[i] = ffo_bits16(ffo_from_bits16(hidden[i], dtype) + an, dtype);
+        h[i] = ffo_from_bits16(hidden[i], dtype);
+    }
+    const float hidden_inv = rms_inv_pinned(h, d, eps);
+    for (int i = 0; i < d; ++i) {
+        const float v = h[i] * hidden_inv;
+        dense_x[i] = ffo_bits16(v * ffo_bf16_to_float(w_pre_ffn[i]), dtype);
+        routed_x[i] = ffo_bits16(v * ffo_bf16_to_float(w_pre_ffn2[i]), dtype);
+        router_x[i] = ffo_bits16(v, dtype);
+    }
+    free(a);
+    free(h);
+}
+
+/* fused layer tail = one row of prefill_layer_tail_block (Metal/Prefill/prefill.metal:320-399), the
+ * arithmetic of cpuReference in FusedLayerTailTests.swift:96-110: h12 = r(h1 + r(norm(h2, w_postffn2)));
+ * hidden = r(r(hidden + r(norm(h12, w_postffn))) * r(layer_scalar)), every r a rounding to 16 bits. */
+void ffo_layer_tail(const uint16_t *h2, const uint16_t *h1, uint16_t *hidden, const uint16_t *w_postffn2,
+                    const uint16_t *w_postffn, int d, float eps, float layer_scalar, int dtype) {
+    float *a = (float *)calloc((size_t)d, sizeof(float)), *h12 = (float *)calloc((size_t)d, sizeof(float));
+    for (int i = 0; i < d; ++i) a[i] = ffo_from_bits16(h2[i], dtype);
+    const float inv_h2 = rms_inv_pinned(a, d, eps);
+    for (int i = 0; i < d; ++i) {
+        const float tmp = ffo_round16(a[i] * inv_h2 * ffo_bf16_to_float(w_postffn2[i]), dtype);
+        h12[i] = ffo_round16(ffo_from_bits16(h1[i], dtype) + tmp, dtype);
+    }
+    const float inv_h12 = rms_inv_pinned(h12, d, eps);
+    const float scale = ffo_round16(layer_scalar, dtype);
+    for (int i = 0; i < d; ++i) {
+        const float tmp = ffo_round16(h12[i] * inv_h12 * ffo_bf16_to_float(w_postffn[i]), dtype);
+        const float sum = ffo_round16(ffo_from_bits16(hidden[i], dtype) + tmp, dtype);
+        hidden[i] = ffo_bits16(sum * scale, dtype);
+    }
+    free(a);
+    free(h12);
+}
+
 int ffo_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

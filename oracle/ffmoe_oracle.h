@@ -31,6 +31,10 @@
  *   combine               one-hot weights reproduce the selected partial;
  *                         cpuReduce of PrefillMoETests.swift:46-64
  *   PRNG                  SplitMix64 published test vector (seed 1234567)
+ *   setup / layer tail    fp64 restatement of RmsNormRef (Reference/Primitives/RmsNorm.swift)
+ *                         composed as cpuReference of FusedLayerTailTests.swift:96-110;
+ *                         unit weights make the three setup outputs equal; router_x has
+ *                         unit RMS; zero attention leaves hidden untouched
  * The pinned-order router logits (ffo_router_logits_pinned) define a summation
  * order of this build, not of the reference (Apple's simd_sum order is
  * unspecified); they are checked against a fp64 dot within rounding noise.
@@ -133,6 +137,15 @@ void ffo_moe_layer(const uint8_t *pool, size_t stride, const ffo_offsets *o, int
 void ffo_moe_experts(const uint8_t *pool, size_t stride, const ffo_offsets *o, int d, int f,
                      const uint16_t *x, size_t x_stride, int t, int top_k, int dtype,
                      const uint32_t *idx, const float *w, float *y, int n_threads);
+
+/* --- steps either side of the MoE stage (summation order pinned by this build, see the .c file) ---
+   Metal/Fusions/fused.metal:210-296, Metal/Prefill/prefill.metal:243-399. One row per call; 16-bit
+   patterns of `dtype`, weights bf16 [d]; hidden is updated in place. d is a multiple of 8. */
+void ffo_post_attn_setup(uint16_t *hidden, const uint16_t *attn, uint16_t *dense_x, uint16_t *routed_x,
+                         uint16_t *router_x, const uint16_t *w_post_attn, const uint16_t *w_pre_ffn,
+                         const uint16_t *w_pre_ffn2, int d, float eps, int dtype);
+void ffo_layer_tail(const uint16_t *h2, const uint16_t *h1, uint16_t *hidden, const uint16_t *w_postffn2,
+                    const uint16_t *w_postffn, int d, float eps, float layer_scalar, int dtype);
 
 int ffo_max_threads(void);
 

@@ -97,6 +97,10 @@ def lib():
         L.ffo_moe_experts.restype = None
         L.ffo_moe_experts.argtypes = [vp, C.c_size_t, C.POINTER(Offsets), C.c_int, C.c_int, vp, C.c_size_t,
                                       C.c_int, C.c_int, C.c_int, vp, vp, vp, C.c_int]
+        L.ffo_post_attn_setup.restype = None
+        L.ffo_post_attn_setup.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_float, C.c_int]
+        L.ffo_layer_tail.restype = None
+        L.ffo_layer_tail.argtypes = [vp, vp, vp, vp, vp, C.c_int, C.c_float, C.c_float, C.c_int]
         L.ffo_max_threads.restype = C.c_int
         _lib = L
     return _lib
@@ -410,6 +414,32 @@ def moe_experts(pool: ExpertPool, x_bits, idx, w, dtype: int = BF16, threads: in
     lib().ffo_moe_experts(_p(pool.bytes), pool.stride, C.byref(pool.offsets), pool.d, pool.f, _p(x_bits), stride,
                           t, idx.shape[1], dtype, _p(idx), _p(w), _p(y), threads)
     return y
+
+
+def post_attn_setup(hidden_bits, attn_bits, w_post_attn, w_pre_ffn, w_pre_ffn2, eps: float = 1e-6, dtype: int = BF16):
+    """Rows [T, D] of 16-bit patterns -> (hidden, dense_x, routed_x, router_x), each [T, D]; hidden is the updated copy."""
+    hidden = np.array(hidden_bits, np.uint16, ndmin=2, copy=True)
+    attn = np.ascontiguousarray(np.array(attn_bits, np.uint16, ndmin=2))
+    ws = [np.ascontiguousarray(w, np.uint16) for w in (w_post_attn, w_pre_ffn, w_pre_ffn2)]
+    t, d = hidden.shape
+    outs = [np.empty((t, d), np.uint16) for _ in range(3)]
+    for r in range(t):
+        lib().ffo_post_attn_setup(_p(hidden[r]), _p(attn[r]), _p(outs[0][r]), _p(outs[1][r]), _p(outs[2][r]),
+                                  _p(ws[0]), _p(ws[1]), _p(ws[2]), d, eps, dtype)
+    return hidden, outs[0], outs[1], outs[2]
+
+
+def layer_tail(h2_bits, h1_bits, hidden_bits, w_postffn2, w_postffn, layer_scalar: float, eps: float = 1e-6,
+               dtype: int = BF16) -> np.ndarray:
+    """Rows [T, D] of 16-bit patterns -> the updated hidden rows."""
+    hidden = np.array(hidden_bits, np.uint16, ndmin=2, copy=True)
+    h2 = np.ascontiguousarray(np.array(h2_bits, np.uint16, ndmin=2))
+    h1 = np.ascontiguousarray(np.array(h1_bits, np.uint16, ndmin=2))
+    w2, w1 = np.ascontiguousarray(w_postffn2, np.uint16), np.ascontiguousarray(w_postffn, np.uint16)
+    t, d = hidden.shape
+    for r in range(t):
+        lib().ffo_layer_tail(_p(h2[r]), _p(h1[r]), _p(hidden[r]), _p(w2), _p(w1), d, eps, layer_scalar, dtype)
+    return hidden
 
 
 def max_threads() -> int:

@@ -255,6 +255,57 @@ int main() {
         EXPECT(relS <= 1e-2 && cosS >= 0.9999);
     }
 
+    // --- post-attention setup and layer tail through the mirrored classes: a 5-row block against the oracle's
+    // rows, bit for bit, and the one-row forms against row 0 ---
+    {
+        const int R = 5;
+        auto draw = [&](size_t n, float lo, float hi) {
+            std::vector<uint16_t> v(n);
+            for (auto &b : v) b = ffo_bf16_bits(ffo_splitmix64_uniform(&rng, lo, hi));
+            return v;
+        };
+        auto hid = draw((size_t)R * d, -2.f, 2.f), att = draw((size_t)R * d, -1.f, 1.f), h2v = draw((size_t)R * d, -1.f, 1.f),
+             h1v = draw((size_t)R * d, -3.f, 3.f);
+        std::vector<std::vector<uint16_t>> wts;
+        for (int i = 0; i < 5; ++i) wts.push_back(draw(d, 0.5f, 1.5f));
+        std::vector<uint16_t> refH = hid, refDense((size_t)R * d), refRouted((size_t)R * d), refRouter((size_t)R * d);
+        for (int r = 0; r < R; ++r)
+            ffo_post_attn_setup(refH.data() + (size_t)r * d, att.data() + (size_t)r * d, refDense.data() + (size_t)r * d,
+                                refRouted.data() + (size_t)r * d, refRouter.data() + (size_t)r * d, wts[0].data(), wts[1].data(),
+                                wts[2].data(), d, 1e-6f, FFO_BF16);
+        std::vector<uint16_t> refT = refH;
+        for (int r = 0; r < R; ++r)
+            ffo_layer_tail(h2v.data() + (size_t)r * d, h1v.data() + (size_t)r * d, refT.data() + (size_t)r * d, wts[3].data(),
+                           wts[4].data(), d, 1e-6f, 0.875f, FFO_BF16);
+        uint16_t *dHid = toDevice(hid), *dAtt = toDevice(att), *dH2v = toDevice(h2v), *dH1v = toDevice(h1v);
+        uint16_t *dWt[5];
+        for (int i = 0; i < 5; ++i) dWt[i] = toDevice(wts[i]);
+        uint16_t *dOut[3];
+        for (auto &p : dOut) HIP(hipMalloc(reinterpret_cast<void **>(&p), (size_t)R * d * 2));
+        PrefillPostAttentionSetup setup(ctx);
+        PrefillLayerTail tail(ctx);
+        setup.encode(stream, dHid, dAtt, dOut[0], dOut[1], dOut[2], dWt[0], dWt[1], dWt[2], R, d, d, d, d, d, d, 1e-6f);
+        HIP(hipStreamSynchronize(stream));
+        EXPECT(toHost(dHid, (size_t)R * d) == refH && toHost(dOut[0], (size_t)R * d) == refDense);
+        EXPECT(toHost(dOut[1], (size_t)R * d) == refRouted && toHost(dOut[2], (size_t)R * d) == refRouter);
+        tail.encode(stream, dH2v, dH1v, dHid, dWt[3], dWt[4], R, d, d, d, d, 1e-6f, 0.875f);
+        HIP(hipStreamSynchronize(stream));
+        EXPECT(toHost(dHid, (size_t)R * d) == refT);
+        // decode forms on row 0
+        uint16_t *dRow = toDevice(std::vector<uint16_t>(hid.begin(), hid.begin() + d));
+        FusedPostAttentionSetup setup1(ctx);
+        FusedLayerTail tail1(ctx);
+        setup1.encode(stream, dRow, dAtt, dOut[0], dOut[1], dOut[2], dWt[0], dWt[1], dWt[2], d, 1e-6f);
+        tail1.encode(stream, dH2v, dH1v, dRow, dWt[3], dWt[4], d, 1e-6f, 0.875f);
+        HIP(hipStreamSynchronize(stream));
+        EXPECT(toHost(dRow, (size_t)d) == std::vector<uint16_t>(refT.begin(), refT.begin() + d));
+        bool threwStride = false;
+        try { tail.encode(stream, dH2v, dH1v, dHid, dWt[3], dWt[4], R, d, d - 8, d, d, 1e-6f, 1.f); } catch (const std::invalid_argument &) { threwStride = true; }
+        EXPECT(threwStride);
+        for (auto p : {dHid, dAtt, dH2v, dH1v, dRow, dOut[0], dOut[1], dOut[2]}) HIP(hipFree(p));
+        for (auto p : dWt) HIP(hipFree(p));
+    }
+
     // --- packed experts: a two-layer checkpoint directory written as ModelLoaderTests.swift:204-241 writes its
     // toy one (16 KiB stride, layout.json with explicit ids), layer 1 with reversed physical ranks; after
     // uploadPackedExperts every expert expands to the same bf16 weights as the directly uploaded blobs ---

@@ -320,3 +320,81 @@ def test_route_partials_reference_test_restated(oracle):
         ref = D @ act
         got = out[t, r].view(np.float16).astype(np.float64)
         assert np.abs(got - ref).max() <= 0.0015
+
+
+def _rms_norm_ref64(x, w, eps):
+    """RmsNormRef.apply (Tests/Support/Validation/Reference/Primitives/RmsNorm.swift:9-41) in float64."""
+    x = np.asarray(x, np.float64)
+    return x * np.asarray(w, np.float64) / np.sqrt((x * x).mean() + eps)
+
+
+def test_layer_tail_against_cpu_reference_restated(oracle):
+    # fusedLayerTailNorms_matchSeparateDispatchesAndReference (FusedLayerTailTests.swift:15-61): same seed and
+    # draw order (h2, h1, hidden, four weight vectors, the scalar); cpuReference (:96-110) restated in float64
+    # with its roundings; the reference's bound on FP16 data is 4e-3 relative, bf16 carries 2^-9 per rounding
+    d, eps = 2816, 1e-6
+    for dtype, bound in ((oracle.FP16, 4e-3), (oracle.BF16, 2e-2)):
+        rng = oracle.SplitMix64(0x7A11_0001)
+        h2 = oracle.bits16(rng.uniform(-1, 1, d), dtype)
+        h1 = oracle.bits16(rng.uniform(-3, 3, d), dtype)
+        hidden = oracle.bits16(rng.uniform(-2, 2, d), dtype)
+        weights = [oracle.bf16_bits(rng.uniform(0.5, 1.5, d)) for _ in range(4)]
+        scalar = float(rng.uniform(0.75, 1.25, 1)[0])
+        r16 = lambda v: oracle.from_bits16(oracle.bits16(np.asarray(v, np.float32), dtype), dtype).astype(np.float64)
+        w2, w1 = oracle.bf16_to_float(weights[1]), oracle.bf16_to_float(weights[2])
+        h2n = r16(_rms_norm_ref64(oracle.from_bits16(h2, dtype), w2, eps))
+        h12 = r16(oracle.from_bits16(h1, dtype).astype(np.float64) + h2n)
+        h12n = r16(_rms_norm_ref64(h12, w1, eps))
+        ref = r16(r16(oracle.from_bits16(hidden, dtype).astype(np.float64) + h12n) * r16(scalar))
+        got = oracle.from_bits16(oracle.layer_tail(h2, h1, hidden, weights[1], weights[2], scalar, eps, dtype)[0], dtype)
+        assert np.abs(got - ref).max() / np.abs(ref).max() < bound
+        # almost every element agrees to the bit; the rest are one rounding step apart
+        assert (got == ref).mean() > 0.95
+
+
+def test_post_attn_setup_against_primitive_chain(oracle):
+    # fusedPostAttentionSetup_matchesPrimitiveChainBitwise_realShape (FusedPostAttentionSetupTests.swift:11-100):
+    # the chain norm(attn) -> hidden += -> three norms of hidden, the router's with a unit weight; same seed
+    d, eps = 2816, 1e-6
+    rng = oracle.SplitMix64(0x9057_A77E)
+    hidden = oracle.bf16_bits(rng.uniform(-1, 1, d))
+    attn = oracle.bf16_bits(rng.uniform(-1, 1, d))
+    w_post, w_pre, w_pre2 = (oracle.bf16_bits(rng.uniform(0.5, 1.5, d)) for _ in range(3))
+    new_hidden, dense, routed, router = oracle.post_attn_setup(hidden, attn, w_post, w_pre, w_pre2, eps)
+    r16 = lambda v: oracle.bf16_to_float(oracle.bf16_bits(np.asarray(v, np.float32))).astype(np.float64)
+    an = r16(_rms_norm_ref64(oracle.bf16_to_float(attn), oracle.bf16_to_float(w_post), eps))
+    h = r16(oracle.bf16_to_float(hidden).astype(np.float64) + an)
+    close = lambda got, ref: (np.abs(oracle.bf16_to_float(got[0]) - ref).max() / np.abs(ref).max() < 1e-2
+                              and (oracle.bf16_to_float(got[0]) == ref).mean() > 0.95)
+    assert close(new_hidden, h)
+    hf = oracle.bf16_to_float(new_hidden[0])
+    assert close(dense, r16(_rms_norm_ref64(hf, oracle.bf16_to_float(w_pre), eps)))
+    assert close(routed, r16(_rms_norm_ref64(hf, oracle.bf16_to_float(w_pre2), eps)))
+    assert close(router, r16(_rms_norm_ref64(hf, np.ones(d), eps)))
+    # what the arithmetic fixes: router_x has unit RMS; unit weights make the three outputs the same bits;
+    # zero attention leaves hidden alone; scaling hidden and attn by 2 leaves the normalised outputs alone
+    assert abs(np.sqrt((oracle.bf16_to_float(router[0]).astype(np.float64) ** 2).mean()) - 1.0) < 2e-3
+    ones = oracle.bf16_bits(np.ones(d, np.float32))
+    _, a, b, c = oracle.post_attn_setup(hidden, attn, w_post, ones, ones, eps)
+    assert np.array_equal(a, b) and np.array_equal(b, c)
+    h0, *_ = oracle.post_attn_setup(hidden, np.zeros(d, np.uint16), w_post, w_pre, w_pre2, eps)
+    assert np.array_equal(h0[0], hidden)
+    two = lambda bits: oracle.bf16_bits(2.0 * oracle.bf16_to_float(bits))
+    _, d2, r2, q2 = oracle.post_attn_setup(two(new_hidden[0]), np.zeros(d, np.uint16), w_post, w_pre, w_pre2, 0.0)
+    _, d1, r1, q1 = oracle.post_attn_setup(new_hidden[0], np.zeros(d, np.uint16), w_post, w_pre, w_pre2, 0.0)
+    assert np.array_equal(d1, d2) and np.array_equal(r1, r2) and np.array_equal(q1, q2)
+
+
+def test_layer_tail_invariants(oracle):
+    d, eps = 512, 1e-6
+    rng = oracle.SplitMix64(0x7A11_B10C)
+    h2, h1, hidden = (oracle.bf16_bits(rng.uniform(-1, 1, d)) for _ in range(3))
+    w2, w1 = (oracle.bf16_bits(rng.uniform(0.5, 1.5, d)) for _ in range(2))
+    base = oracle.layer_tail(h2, h1, hidden, w2, w1, 1.0, eps)
+    # a power-of-two scalar only shifts exponents; a scalar is rounded to 16 bits before use
+    assert np.array_equal(oracle.bf16_to_float(oracle.layer_tail(h2, h1, hidden, w2, w1, 2.0, eps)), 2.0 * oracle.bf16_to_float(base))
+    assert np.array_equal(oracle.layer_tail(h2, h1, hidden, w2, w1, 1.0 + 2.0 ** -10, eps), base)
+    # rows are independent: a block equals its rows one at a time (PrefillLayerTailTests.swift:11-118)
+    blk = oracle.layer_tail(np.stack([h2, h1]), np.stack([h1, h2]), np.stack([hidden, hidden]), w2, w1, 0.9, eps)
+    assert np.array_equal(blk[0], oracle.layer_tail(h2, h1, hidden, w2, w1, 0.9, eps)[0])
+    assert np.array_equal(blk[1], oracle.layer_tail(h1, h2, hidden, w2, w1, 0.9, eps)[0])
