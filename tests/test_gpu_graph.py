@@ -1,0 +1,76 @@
+"""The hot-path entry points only enqueue kernels (no allocation, no memset, no synchronisation), so a caller
+may capture them into a HIP graph. A captured chain of layers is replayed several times, with eager work and
+synchronisations of the same context between the replays, and every replay must equal the eager result bit for bit.
+Run on the GPU box: pytest -m gpu."""
+import numpy as np
+import pytest
+
+from helpers import bf16_tensor, bits_of, make_layer, to_ff_offsets
+
+pytestmark = pytest.mark.gpu
+
+
+def test_router_verify_and_dense_chain_in_a_graph(oracle):
+    import torch
+    import fieldfare_moe as ff
+    ff.lib()
+    d, f, e, k, layers, t = 256, 128, 32, 8, 3, 16
+    ctx = ff.Context(d, f, e, k, n_layers=layers, max_tokens=64)
+    dense = ff.Context(d, 2 * f, 1, 1, n_layers=layers, max_tokens=64)
+    rng = np.random.default_rng(5)
+    for layer in range(layers):
+        _, pool, router = make_layer(oracle, 40 + layer, d, f, e)
+        ctx.upload_layer(layer, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
+        ctx.upload_router_bf16(layer, router)
+        _, dpool, _ = make_layer(oracle, 70 + layer, d, 2 * f, 1)
+        dense.upload_layer(layer, dpool.bytes, dpool.stride, to_ff_offsets(ff, dpool.offsets))
+    x = bf16_tensor(torch, oracle.bf16_bits(rng.normal(0, 1, (t, d)).astype(np.float32)))
+    ws = [bf16_tensor(torch, oracle.bf16_bits(rng.uniform(0.5, 1.5, d).astype(np.float32))) for _ in range(5)]
+    hidden0 = bf16_tensor(torch, oracle.bf16_bits(rng.normal(0, 1, (t, d)).astype(np.float32)))
+    hidden = hidden0.clone()
+    idx = torch.empty((t, k), dtype=torch.int32, device="cuda")
+    w = torch.empty((t, k), dtype=torch.bfloat16, device="cuda")
+    outs = tuple(torch.empty((t, d), dtype=torch.bfloat16, device="cuda") for _ in range(3))
+    h1 = torch.empty((t, d), dtype=torch.bfloat16, device="cuda")
+    h2 = torch.empty((t, d), dtype=torch.bfloat16, device="cuda")
+
+    def chain():
+        # one decoder-layer MoE block per layer: setup -> (shared expert, router -> routed experts) -> tail
+        for layer in range(layers):
+            ctx.post_attn_setup(hidden, x, ws[0], ws[1], ws[2], out=outs)
+            dense.dense_ffn(layer, outs[0], out=h1)
+            i_, w_ = ctx.router(layer, outs[2])
+            idx.copy_(i_)
+            w.copy_(w_)
+            ctx.verify(layer, outs[1], idx, w, out=h2)
+            ctx.layer_tail(h2, h1, hidden, ws[3], ws[4], 0.9)
+
+    chain()
+    torch.cuda.synchronize()
+    eager = bits_of(hidden)
+    assert np.isfinite(oracle.bf16_to_float(eager)).all()
+
+    # warm the allocator on the capture stream, then capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        hidden.copy_(hidden0)
+        chain()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    hidden.copy_(hidden0)
+    with torch.cuda.graph(graph, stream=side):
+        chain()
+    for replay in range(4):
+        hidden.copy_(hidden0)
+        h2.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(bits_of(hidden), eager), f"replay {replay}"
+        # eager work of the same contexts between replays
+        ctx.verify(replay % layers, x, idx, w)
+        dense.dense_ffn(replay % layers, x)
+        torch.cuda.synchronize()
+    ctx.close()
+    dense.close()
