@@ -384,10 +384,15 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
                                             expert_base + g.dn_scales_off, (size_t)g.dn_rbp * g.gf * kTileScaleBytes);
     const uint32_t ng = g.gf, g_last = g.gf - 1;
 
+    // the route list is read in the same round trip as the slot's count: every entry of the fixed-size
+    // list is addressable, entries past the count are stale and replaced by route 0 after the fact
+    const uint32_t route_j = slot.routes[j];
     WeightRing ring;
 #pragma unroll
     for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb0 * ng + min((uint32_t)u, g_last), lane);
-    const uint16_t *arow = acts + (size_t)slot.routes[min(j, n - 1)] * g.f + 8 * jq;
+    const uint32_t route_0 = __builtin_amdgcn_readfirstlane(route_j);
+    const uint32_t my_route = j < n ? route_j : route_0;
+    const uint16_t *arow = acts + (size_t)my_route * g.f + 8 * jq;
     uint4 x0[kRing], x1[kRing];
 #pragma unroll
     for (int u = 0; u < kRing; ++u) {
@@ -398,7 +403,11 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
     }
     uint32_t out_base[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) out_base[r] = slot.routes[min(4 * jq + r, n - 1)] * g.d;
+    for (int r = 0; r < 4; ++r) {
+        // route of token slot 4 jq + r: lane 4 jq + r holds it (its j is that slot)
+        const uint32_t rt = (uint32_t)__shfl((int)route_j, (int)(4 * jq + r), 64);
+        out_base[r] = (4 * jq + r < n ? rt : route_0) * g.d;
+    }
 
     for (uint32_t rb = rb0; rb < rb1; ++rb) {
         const uint32_t next_row = min(rb + 1, rb1 - 1) * ng;
