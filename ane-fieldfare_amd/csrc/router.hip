@@ -295,8 +295,12 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict
         const bool upper = (lane & m) != 0;
 #pragma unroll
         for (int o = 0; o < half; ++o) {
-            const float keep = upper ? v[o + half] : v[o];
-            const float send = upper ? v[o] : v[o + half];
+            // both candidates are pinned in registers first: left alone, the compiler folds the two selects
+            // into one load of v[] at a lane-dependent index, i.e. a 16-way compare-and-select chain
+            float lo = v[o], hi = v[o + half];
+            asm("" : "+v"(lo), "+v"(hi));
+            const float keep = upper ? hi : lo;
+            const float send = upper ? lo : hi;
             v[o] = keep + __shfl_xor(send, m, 64);
         }
     }
