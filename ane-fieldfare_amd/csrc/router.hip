@@ -186,7 +186,7 @@ constexpr int kTileTok = 8, kTileExp = 8;
 template <bool W_F32> struct WRaw { uint2 v; };
 template <> struct WRaw<true> { f32x4 v; };
 
-template <bool W_F32, bool X_ALIGNED>
+template <bool W_F32, bool X_ALIGNED, bool HAS_ES>
 __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict__ w_, const uint16_t *__restrict__ es,
                                                           const uint16_t *__restrict__ x, uint32_t x_stride,
                                                           uint32_t t, uint32_t n_experts, uint32_t d,
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict
         }
 #pragma unroll
         for (int r = 0; r < kTileTok; ++r) xn[r] = load_x4<X_ALIGNED>(xrow[r] + k);
-        if (es) en = *reinterpret_cast<const uint2 *>(es + k);
+        if (HAS_ES) en = *reinterpret_cast<const uint2 *>(es + k);
     };
 
     const uint32_t steps = (d + 1023) / 1024;
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict
                                      bf16hi_to_f32(xc[r].y)};
                 float xe[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) xe[j] = es ? xf[j] * sc[j] : xf[j];   // exact: product of two bf16
+                for (int j = 0; j < 4; ++j) xe[j] = HAS_ES ? xf[j] * sc[j] : xf[j];   // exact: product of two bf16
 #pragma unroll
                 for (int c = 0; c < kTileExp; ++c)
 #pragma unroll
@@ -348,8 +348,14 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
     const uint32_t n_egroups = (n_experts + kTileExp - 1) / kTileExp, n_tgroups = (t + kTileTok - 1) / kTileTok;
     const dim3 grid(n_egroups * ((n_tgroups + 7) / 8) * 8);
 #define FFMOE_ROUTER(WF, XA)                                                                                 \
-    hipLaunchKernelGGL((router_tile_kernel<WF, XA>), grid, dim3(256), 0, s, rw.w, rw.effective_scale, x,     \
-                       x_stride, t, n_experts, d, n_egroups, n_tgroups, logits)
+    do {                                                                                                     \
+        if (rw.effective_scale)                                                                              \
+            hipLaunchKernelGGL((router_tile_kernel<WF, XA, true>), grid, dim3(256), 0, s, rw.w,              \
+                               rw.effective_scale, x, x_stride, t, n_experts, d, n_egroups, n_tgroups, logits); \
+        else                                                                                                 \
+            hipLaunchKernelGGL((router_tile_kernel<WF, XA, false>), grid, dim3(256), 0, s, rw.w,             \
+                               rw.effective_scale, x, x_stride, t, n_experts, d, n_egroups, n_tgroups, logits); \
+    } while (0)
     if (rw.w_is_f32) { if (x_aligned) FFMOE_ROUTER(true, true); else FFMOE_ROUTER(true, false); }
     else { if (x_aligned) FFMOE_ROUTER(false, true); else FFMOE_ROUTER(false, false); }
 #undef FFMOE_ROUTER
