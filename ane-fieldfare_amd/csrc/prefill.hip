@@ -62,23 +62,48 @@ __global__ __launch_bounds__(kSortBlock) void prefill_hist_kernel(ItemSource src
     if (threadIdx.x < src.n_experts) block_cnt[(size_t)blockIdx.x * src.n_experts + threadIdx.x] = cnt[threadIdx.x];
 }
 
-// One block: per expert, turn the per-block counts into per-block bases, then lay out the experts one
-// after the other and cut each into M-tiles.
-__global__ __launch_bounds__(256) void prefill_scan_kernel(uint32_t n_blocks, uint32_t n_experts,
-                                                           uint32_t *__restrict__ block_cnt, PrefillPlan *__restrict__ plan,
-                                                           PrefillTile *__restrict__ tiles, uint32_t max_tiles) {
+// One block of 1024 threads: per expert, turn the per-block counts into per-block bases, then lay out the
+// experts one after the other and cut each into M-tiles. Thread (expert e, chunk c) owns a contiguous run
+// of sort blocks, so the counts of a whole column are in flight at once and - up to kScanKeep per thread -
+// stay in registers between the summing pass and the pass that writes the bases.
+constexpr int kScanThreads = 1024;
+constexpr int kScanKeep = 16;
+
+__global__ __launch_bounds__(kScanThreads) void prefill_scan_kernel(uint32_t n_blocks, uint32_t n_experts, uint32_t e_pad,
+                                                                    uint32_t *__restrict__ block_cnt,
+                                                                    PrefillPlan *__restrict__ plan,
+                                                                    PrefillTile *__restrict__ tiles, uint32_t max_tiles) {
     __shared__ uint32_t total[FFMOE_MAX_EXPERTS];
     __shared__ uint32_t offset[FFMOE_MAX_EXPERTS + 1];
     __shared__ uint32_t tile_off[FFMOE_MAX_EXPERTS + 1];
-    const uint32_t e = threadIdx.x;
+    __shared__ uint32_t part[kScanThreads];                 // [chunk][e_pad]: chunk sums, then chunk bases
+    const uint32_t e = threadIdx.x % e_pad, ch = threadIdx.x / e_pad, chunks = kScanThreads / e_pad;
+    const uint32_t per = (n_blocks + chunks - 1) / chunks;
+    const uint32_t b_lo = min(n_blocks, ch * per), b_hi = min(n_blocks, b_lo + per);
+    const bool live = e < n_experts;
+    uint32_t keep[kScanKeep];
     uint32_t sum = 0;
-    if (e < n_experts) {
-#pragma unroll 16
-        for (uint32_t b = 0; b < n_blocks; ++b) sum += block_cnt[(size_t)b * n_experts + e];
+#pragma unroll
+    for (int u = 0; u < kScanKeep; ++u) {
+        keep[u] = live && b_lo + u < b_hi ? block_cnt[(size_t)(b_lo + u) * n_experts + e] : 0;
+        sum += keep[u];
     }
-    total[e] = e < n_experts ? sum : 0;
+    if (live)
+        for (uint32_t b = b_lo + kScanKeep; b < b_hi; ++b) sum += block_cnt[(size_t)b * n_experts + e];
+    part[threadIdx.x] = sum;
+    if (threadIdx.x < FFMOE_MAX_EXPERTS) total[threadIdx.x] = 0;
     __syncthreads();
-    if (e == 0) {
+    if (ch == 0 && live) {
+        uint32_t run = 0;
+        for (uint32_t c = 0; c < chunks; ++c) {
+            const uint32_t v = part[c * e_pad + e];
+            part[c * e_pad + e] = run;
+            run += v;
+        }
+        total[e] = run;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
         uint32_t run = 0, trun = 0;
         for (uint32_t i = 0; i < n_experts; ++i) {
             offset[i] = run;
@@ -90,36 +115,36 @@ __global__ __launch_bounds__(256) void prefill_scan_kernel(uint32_t n_blocks, ui
         tile_off[n_experts] = trun;
         plan->n_pairs = run;
         plan->n_tiles = min(trun, max_tiles);
+        plan->expert_offset[n_experts] = run;
     }
     __syncthreads();
-    if (e < n_experts) {
-        uint32_t run = offset[e];
-        plan->expert_offset[e] = run;
-        plan->expert_count[e] = total[e];
-        for (uint32_t b0 = 0; b0 < n_blocks; b0 += 16) {
-            uint32_t c[16];
+    if (!live) return;
+    uint32_t run = offset[e] + part[threadIdx.x];
 #pragma unroll
-            for (int u = 0; u < 16; ++u) c[u] = b0 + u < n_blocks ? block_cnt[(size_t)(b0 + u) * n_experts + e] : 0;
-#pragma unroll
-            for (int u = 0; u < 16; ++u) {
-                if (b0 + u < n_blocks) block_cnt[(size_t)(b0 + u) * n_experts + e] = run;      // count -> base, in place
-                run += c[u];
-            }
-        }
-        const uint32_t nt = (total[e] + kBM - 1) / kBM;
-        for (uint32_t i = 0; i < nt; ++i) {
-            const uint32_t ti = tile_off[e] + i;
-            if (ti < max_tiles) {
-                PrefillTile tl;
-                tl.expert = e;
-                tl.row_start = offset[e] + i * kBM;
-                tl.rows = min((uint32_t)kBM, total[e] - i * kBM);
-                tl.pad = 0;
-                tiles[ti] = tl;
-            }
+    for (int u = 0; u < kScanKeep; ++u) {
+        if (b_lo + u < b_hi) block_cnt[(size_t)(b_lo + u) * n_experts + e] = run;      // count -> base, in place
+        run += keep[u];
+    }
+    for (uint32_t b = b_lo + kScanKeep; b < b_hi; ++b) {
+        const uint32_t c = block_cnt[(size_t)b * n_experts + e];
+        block_cnt[(size_t)b * n_experts + e] = run;
+        run += c;
+    }
+    if (ch != 0) return;
+    plan->expert_offset[e] = offset[e];
+    plan->expert_count[e] = total[e];
+    const uint32_t nt = (total[e] + kBM - 1) / kBM;
+    for (uint32_t i = 0; i < nt; ++i) {
+        const uint32_t ti = tile_off[e] + i;
+        if (ti < max_tiles) {
+            PrefillTile tl;
+            tl.expert = e;
+            tl.row_start = offset[e] + i * kBM;
+            tl.rows = min((uint32_t)kBM, total[e] - i * kBM);
+            tl.pad = 0;
+            tiles[ti] = tl;
         }
     }
-    if (e == 0) plan->expert_offset[n_experts] = offset[n_experts];
 }
 
 __global__ __launch_bounds__(kSortBlock) void prefill_scatter_kernel(ItemSource src, const uint32_t *__restrict__ block_base,
@@ -454,8 +479,10 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
     if (src.n_items == 0) return hipSuccess;
     const uint32_t n_blocks = (src.n_items + kSortBlock - 1) / kSortBlock;
     hipLaunchKernelGGL(prefill_hist_kernel, dim3(n_blocks), dim3(kSortBlock), 0, s, src, sc.block_cnt);
-    hipLaunchKernelGGL(prefill_scan_kernel, dim3(1), dim3(256), 0, s, n_blocks, n_experts, sc.block_cnt, sc.plan, sc.tiles,
-                       sc.max_tiles);
+    uint32_t e_pad = 1;
+    while (e_pad < n_experts) e_pad <<= 1;          // n_experts <= FFMOE_MAX_EXPERTS = 256 <= kScanThreads
+    hipLaunchKernelGGL(prefill_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, n_blocks, n_experts, e_pad, sc.block_cnt, sc.plan,
+                       sc.tiles, sc.max_tiles);
     hipLaunchKernelGGL(prefill_scatter_kernel, dim3(n_blocks), dim3(kSortBlock), 0, s, src, sc.block_cnt, sc.sorted_token,
                        sc.sorted_out_row);
     hipError_t e = hipGetLastError();
