@@ -45,7 +45,7 @@ EXPORTS = [
     "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
     "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
-    "ffmoe_layer_tail",
+    "ffmoe_layer_tail", "ffmoe_route_verify",
 ]
 
 PROFILE_SLOTS = 16
@@ -150,6 +150,7 @@ def lib() -> C.CDLL:
     L.ffmoe_router.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
     L.ffmoe_verify.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, vp, errp]
     L.ffmoe_verify_partials.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
+    L.ffmoe_route_verify.argtypes = [vp, vp, u32, vp, u32, vp, u32, u32, vp, vp, vp, vp, errp]
     L.ffmoe_last_live_experts.argtypes = [vp, vp, C.POINTER(u32), errp]
     L.ffmoe_reduce_token_major.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, errp]
     L.ffmoe_gemv_int4.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, i32, errp]
@@ -326,6 +327,18 @@ class Context:
         _check(self.L.ffmoe_verify(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(idx), _ptr(w), _ptr(residual),
                                    _ptr(y), C.byref(err)), err)
         return y
+
+    def route_verify(self, layer: int, router_x, x, residual=None, out=None):
+        """Router + expert pass of a block of <= 16 rows in one call. Returns (y, idx, w)."""
+        import torch
+        t, k = x.shape[0], self.shape.top_k
+        y = out if out is not None else torch.empty((t, self.shape.d), dtype=torch.bfloat16, device=x.device)
+        idx = torch.empty((t, k), dtype=torch.int32, device=x.device)
+        w = torch.empty((t, k), dtype=torch.bfloat16, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_route_verify(self._h, _stream(), layer, _ptr(router_x), _row_stride(router_x), _ptr(x), _row_stride(x),
+                                         t, _ptr(residual), _ptr(y), _ptr(idx), _ptr(w), C.byref(err)), err)
+        return y, idx, w
 
     def verify_partials(self, layer: int, x, idx, w, partials=None):
         import torch

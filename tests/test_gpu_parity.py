@@ -359,3 +359,27 @@ def test_gemv_int4_reference_shapes(small, oracle, torch, m, n, rows, off):
     for r in range(rows):
         single = small["ctx"].gemv_int4(Wd, Sd, Bd, x[r:r + 1], f32_out=True, w_byte_offset=off).cpu().numpy()[0]
         assert np.array_equal(single.view(np.uint32), y32[r].view(np.uint32)), f"row {r} differs from the GEMV"
+
+
+@pytest.mark.parametrize("which,t", [("small", 1), ("small", 3), ("small", 8), ("small", 9), ("real", 1), ("real", 4),
+                                     ("real", 8), ("real", 16)])
+def test_route_verify_equals_router_then_verify(small, real, oracle, torch, which, t):
+    # one call (up to 8 rows the select runs inside the gate/up kernel) against the two calls: routes,
+    # weights and outputs bit for bit; the routes are the oracle's
+    fx = small if which == "small" else real
+    ctx, d, layer = fx["ctx"], fx["d"], 1 if which == "small" else 0
+    g = oracle.seed_tree_key(0x207E, f"route-verify-{which}-{t}")
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    rb = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    res = oracle.bf16_bits(g.uniform(-0.5, 0.5, t * d)).reshape(t, d)
+    x, router_x, residual = bf16_tensor(torch, xb), bf16_tensor(torch, rb), bf16_tensor(torch, res)
+    idx2, w2 = ctx.router(layer, router_x)
+    y2 = ctx.verify(layer, x, idx2, w2, residual=residual)
+    y1, idx1, w1 = ctx.route_verify(layer, router_x, x, residual=residual)
+    assert np.array_equal(idx1.cpu().numpy(), idx2.cpu().numpy())
+    assert np.array_equal(bits_of(w1), bits_of(w2))
+    assert np.array_equal(bits_of(y1), bits_of(y2))
+    got = idx1.cpu().numpy().astype(np.uint32)
+    for r in range(t):
+        ref_idx, _ = oracle.topk_softmax(oracle.router_logits_pinned(fx["router"], rb[r]), 8)
+        assert np.array_equal(got[r], ref_idx), f"row {r}"
