@@ -257,6 +257,33 @@ def main():
                                 "unit": "TFLOP/s", "frac": round((flops_gu + flops_dn) / gemm_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                                 "traffic": TRAFFIC_PREFILL_GEMMS_3072 if TP == 3072 else None,
                                 "traffic_unit": "HBM bytes of the two launches (rocprofv3 --pmc, same profile file)"}}
+        # BASELINE.json config 4 (ii): the same chunk with Zipf(1.1) routing imposed on the experts
+        # (indices and weights given, no router): a few experts hold most pairs, many hold a handful
+        zr_ = np.random.default_rng(4)
+        pz_ = 1.0 / np.arange(1, E + 1) ** 1.1
+        pz_ /= pz_.sum()
+        perm_ = zr_.permutation(E)
+        zidx_ = np.stack([perm_[zr_.choice(E, K, replace=False, p=pz_)] for _ in range(TP)]).astype(np.int32)
+        zw_ = zr_.random((TP, K)).astype(np.float32)
+        zw_ = zw_ / zw_.sum(1, keepdims=True)
+        pidx_t.copy_(torch.from_numpy(zidx_))
+        pw_t.copy_(torch.from_numpy(oracle.bf16_bits(zw_).view(np.int16)).view(torch.bfloat16))
+
+        def zstep(layer):
+            if Lib.ffmoe_prefill(h, stream, layer, pxp, D, TP, ppi, ppw, ppy, C.byref(err)):
+                raise RuntimeError(err.value)
+        for i in range(4):
+            zstep(i % L)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(psteps):
+            zstep(i % L)
+        torch.cuda.synchronize()
+        zel = (time.perf_counter() - t0) / psteps
+        _, z_tiles, zcounts = ctx.prefill_stats()
+        prefill["zipf_1p1"] = {"tok_per_s": round(TP / zel, 1), "ms_per_layer": round(zel * 1e3, 4), "m_tiles": z_tiles,
+                               "pairs_per_expert_min": int(zcounts.min()), "pairs_per_expert_max": int(zcounts.max()),
+                               "pairs_per_expert_median": int(np.median(zcounts)), "router": "not run (routes imposed)"}
 
     def timed(fn, reps, warm=3):
         for _ in range(warm):
