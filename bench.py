@@ -371,6 +371,63 @@ def main():
                                     "frac_mfma_peak": round(fl / tp_ / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
             del xps, yps
         extra["shared_expert"] = shared
+
+        # One decoder layer's MoE block for a 16-token verify block, as the reference schedules it
+        # (RealForwardRunner.swift:454-756): post-attention setup, then the shared expert beside router +
+        # routed experts (two streams, as the reference runs them concurrently), then the layer tail.
+        main_s, side_s = torch.cuda.current_stream(), torch.cuda.Stream()
+        hid_b = x.clone()
+        att_b = torch.randn((T, D), device="cuda", generator=gen).to(torch.bfloat16)
+        wn_b = [(torch.rand((D,), device="cuda", generator=gen) + 0.5).to(torch.bfloat16) for _ in range(5)]
+        outs_b = tuple(torch.empty((T, D), dtype=torch.bfloat16, device="cuda") for _ in range(3))
+        h1_b = torch.empty((T, D), dtype=torch.bfloat16, device="cuda")
+        ev_fork, ev_join = torch.cuda.Event(), torch.cuda.Event()
+        pouts = [C.c_void_p(o.data_ptr()) for o in outs_b]
+
+        def layer_block(i, concurrent):
+            layer = i % L
+            ctx.post_attn_setup(hid_b, att_b, wn_b[0], wn_b[1], wn_b[2], out=outs_b)
+            if concurrent:
+                ev_fork.record(main_s)
+                with torch.cuda.stream(side_s):
+                    side_s.wait_event(ev_fork)
+                    dense.dense_ffn(i % LS, outs_b[0], out=h1_b)
+                    ev_join.record(side_s)
+            else:
+                dense.dense_ffn(i % LS, outs_b[0], out=h1_b)
+            rc = Lib.ffmoe_router(h, stream, layer, pouts[2], D, T, pidx, pw, None, C.byref(err))
+            rc |= Lib.ffmoe_verify(h, stream, layer, pouts[1], D, T, pidx, pw, None, py, C.byref(err))
+            if rc:
+                raise RuntimeError(err.value)
+            if concurrent:
+                main_s.wait_event(ev_join)
+            ctx.layer_tail(y, h1_b, hid_b, wn_b[3], wn_b[4], 1.0)
+        counter = {"i": 0}
+
+        def run_block(concurrent):
+            layer_block(counter["i"], concurrent)
+            counter["i"] += 1
+        t_seq = timed(lambda: run_block(False), 120, warm=30)
+        t_con = timed(lambda: run_block(True), 120, warm=30)
+        # the same chain of L layers as a HIP graph: nine launches per layer from Python are host-bound,
+        # a replay shows the device time (the library only enqueues kernels, so the chain captures as it is)
+        graph_us = {}
+        for label, conc in (("one_stream", False), ("shared_expert_on_second_stream", True)):
+            gph = torch.cuda.CUDAGraph()
+            cap = torch.cuda.Stream()
+            cap.wait_stream(main_s)
+            with torch.cuda.graph(gph, stream=cap):
+                main_s = torch.cuda.current_stream()
+                stream = C.c_void_p(main_s.cuda_stream)
+                for i in range(L):
+                    layer_block(i, conc)
+            main_s = torch.cuda.current_stream()
+            stream = C.c_void_p(main_s.cuda_stream)
+            graph_us[label] = round(timed(gph.replay, 8, warm=2) / L * 1e6, 2)
+            del gph
+        extra["layer_block_rows16"] = {"one_stream_us": round(t_seq * 1e6, 2), "shared_expert_on_second_stream_us": round(t_con * 1e6, 2),
+                                       "hip_graph_replay_us": graph_us,
+                                       "steps": "post-attention setup, shared expert, router, routed experts, layer tail"}
         dense.close()
 
     # The row-wise steps either side of the MoE stage at the prefill chunk and at a verify block:
