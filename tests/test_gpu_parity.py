@@ -383,3 +383,28 @@ def test_route_verify_equals_router_then_verify(small, real, oracle, torch, whic
     for r in range(t):
         ref_idx, _ = oracle.topk_softmax(oracle.router_logits_pinned(fx["router"], rb[r]), 8)
         assert np.array_equal(got[r], ref_idx), f"row {r}"
+
+
+@pytest.mark.parametrize("which", ["small", "real"])
+def test_decode_sized_blocks_equal_rows_of_a_larger_block(small, real, oracle, torch, which):
+    # rows are independent of the block they arrive in: a block of two rows and a block of one row give the
+    # bits of the same rows inside a three-row block, with and without a residual, with a skipped route
+    fx = small if which == "small" else real
+    ctx, d, layer = fx["ctx"], fx["d"], 1 if which == "small" else 0
+    g = oracle.seed_tree_key(0xDEC0, f"decode-rows-{which}")
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, 3 * d)).reshape(3, d)
+    res = oracle.bf16_bits(g.uniform(-0.5, 0.5, 3 * d)).reshape(3, d)
+    x, residual = bf16_tensor(torch, xb), bf16_tensor(torch, res)
+    idx, w = ctx.router(layer, x)
+    w[1, 3] = 0.0                       # a skipped route inside the small blocks
+    for resid in (None, residual):
+        y3 = bits_of(ctx.verify(layer, x, idx, w, residual=resid))
+        y2 = bits_of(ctx.verify(layer, x[:2], idx[:2], w[:2], residual=None if resid is None else resid[:2]))
+        y1 = bits_of(ctx.verify(layer, x[2:3], idx[2:3], w[2:3], residual=None if resid is None else resid[2:3]))
+        assert np.array_equal(y2, y3[:2])
+        assert np.array_equal(y1[0], y3[2])
+    # and the oracle on the small block
+    w_np = oracle.bf16_to_float(bits_of(w[:2]))
+    ref = oracle.moe_experts(fx["pool"], xb[:2], idx[:2].cpu().numpy().astype(np.uint32), w_np)
+    got = oracle.bf16_to_float(bits_of(ctx.verify(layer, x[:2], idx[:2], w[:2])))
+    assert rel_err(got, ref) < 1e-2 and cosine(got, ref) > 0.9999
