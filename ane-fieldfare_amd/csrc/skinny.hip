@@ -44,14 +44,18 @@ struct PlanScratch {
 // Run by all 256 threads of a block. Builds the plan in LDS; writes it to `plan_out` when that is not
 // null; when `my_slot` is a live slot, leaves that slot's route list in ps.my_routes. Returns n_live.
 // `slot_from_total` maps the number of live experts to the caller's slot (or to ~0u for none).
+// Phase A: live experts compacted in expert order (ps.expert_of, ps.slot_of, ps.cnt); returns n_live and
+// leaves the calling thread's own route expert in `e`. Phase B: the route lists. A caller that streams
+// weights can start its loads between the two: the expert of its slot is known after phase A.
 template <typename SlotFn>
-__device__ __forceinline__ uint32_t build_plan(PlanScratch &ps, const uint32_t *__restrict__ idx,
-                                               const uint16_t *__restrict__ w, uint32_t n_routes, uint32_t n_experts,
-                                               VerifyPlan *plan_out, SlotFn slot_from_total, uint32_t &my_slot) {
+__device__ __forceinline__ uint32_t build_plan_experts(PlanScratch &ps, const uint32_t *__restrict__ idx,
+                                                       const uint16_t *__restrict__ w, uint32_t n_routes, uint32_t n_experts,
+                                                       VerifyPlan *plan_out, SlotFn slot_from_total, uint32_t &my_slot,
+                                                       uint32_t &e) {
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     ps.cnt[tid] = 0;
     __syncthreads();
-    uint32_t e = 0xFFFFFFFFu;
+    e = 0xFFFFFFFFu;
     if (tid < n_routes) {
         const uint32_t ee = idx[tid];
         if ((w[tid] & 0x7FFFu) != 0 && ee < n_experts) e = ee;
@@ -88,6 +92,12 @@ __device__ __forceinline__ uint32_t build_plan(PlanScratch &ps, const uint32_t *
     total = __builtin_amdgcn_readfirstlane(total);
     my_slot = slot_from_total(total);
     __syncthreads();
+    return total;
+}
+
+__device__ __forceinline__ void build_plan_routes(PlanScratch &ps, uint32_t n_routes, VerifyPlan *plan_out, uint32_t my_slot,
+                                                  uint32_t e) {
+    const uint32_t tid = threadIdx.x;
     if (tid < n_routes && e != 0xFFFFFFFFu) {
         uint32_t pos = 0;
         for (uint32_t j = 0; j < tid; ++j) pos += ps.route_expert[j] == e ? 1u : 0u;
@@ -97,7 +107,16 @@ __device__ __forceinline__ uint32_t build_plan(PlanScratch &ps, const uint32_t *
             if (sl == my_slot) ps.my_routes[pos] = tid;
         }
     }
-    __syncthreads();
+    lds_barrier();      // LDS only: the caller's weight loads stay in flight across it
+}
+
+template <typename SlotFn>
+__device__ __forceinline__ uint32_t build_plan(PlanScratch &ps, const uint32_t *__restrict__ idx,
+                                               const uint16_t *__restrict__ w, uint32_t n_routes, uint32_t n_experts,
+                                               VerifyPlan *plan_out, SlotFn slot_from_total, uint32_t &my_slot) {
+    uint32_t e;
+    const uint32_t total = build_plan_experts(ps, idx, w, n_routes, n_experts, plan_out, slot_from_total, my_slot, e);
+    build_plan_routes(ps, n_routes, plan_out, my_slot, e);
     return total;
 }
 
@@ -320,17 +339,20 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     // operations, against a separate launch plus two dependent global reads per block. Block 0 also
     // writes the plan out for the down kernel.
     const uint32_t gu_rb = g.gu_rb, n_blocks = gridDim.x, bid = blockIdx.x;
-    uint32_t slot_id;
-    const uint32_t n_live = build_plan(
-        ps, idx, w, n_routes, n_experts, bid == 0 ? plan : nullptr,
-        [=](uint32_t total) { return total ? bid / max(1u, min(gu_rb, n_blocks / total)) : 0xFFFFFFFFu; }, slot_id);
-    if (n_live == 0 || slot_id >= n_live) return;
-    const uint32_t blocks_per_slot = max(1u, min(gu_rb, n_blocks / n_live));
-    uint32_t rb0, rb1;
-    split_range(gu_rb, blocks_per_slot, bid % blocks_per_slot, rb0, rb1);
-    if (rb0 >= rb1) return;
-    const uint32_t slot_expert = __builtin_amdgcn_readfirstlane(ps.expert_of[slot_id]);
-    const uint32_t n = min(__builtin_amdgcn_readfirstlane(ps.cnt[slot_expert]), (uint32_t)kMaxRows);
+    uint32_t slot_id, route_expert;
+    VerifyPlan *plan_out = bid == 0 ? plan : nullptr;
+    const uint32_t n_live = build_plan_experts(
+        ps, idx, w, n_routes, n_experts, plan_out,
+        [=](uint32_t total) { return total ? bid / max(1u, min(gu_rb, n_blocks / total)) : 0xFFFFFFFFu; }, slot_id,
+        route_expert);
+    // a block with no work still takes part in the barriers of the second phase (block 0 publishes the plan)
+    const bool has_slot = n_live != 0 && slot_id < n_live;
+    const uint32_t blocks_per_slot = max(1u, min(gu_rb, n_blocks / max(1u, n_live)));
+    uint32_t rb0 = 0, rb1 = 0;
+    if (has_slot) split_range(gu_rb, blocks_per_slot, bid % blocks_per_slot, rb0, rb1);
+    const bool has_rows = has_slot && rb0 < rb1;
+    const uint32_t slot_expert = has_slot ? __builtin_amdgcn_readfirstlane(ps.expert_of[slot_id]) : 0;
+    const uint32_t n = has_slot ? min(__builtin_amdgcn_readfirstlane(ps.cnt[slot_expert]), (uint32_t)kMaxRows) : 1;
     struct { const uint32_t *routes; } slot = {ps.my_routes};
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15, jq = lane >> 4;
@@ -341,9 +363,15 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     const TileSource gu_src = make_tile_source(expert_base + g.gu_tiles_off, (size_t)g.gu_rb * g.gd * kTileBytes,
                                                expert_base + g.gu_scales_off, (size_t)g.gu_rb * g.gd * kTileScaleBytes);
 
+    // the weights of the first tile row are requested as soon as the slot's expert is known; the route lists
+    // are worked out while those loads are in flight
     WeightRing ring;
+    if (has_rows) {
 #pragma unroll
-    for (int u = 0; u < kRing; ++u) ring_fill(ring, u, gu_src, rb0 * g.gd + min(g0 + u, g_last), lane);
+        for (int u = 0; u < kRing; ++u) ring_fill(ring, u, gu_src, rb0 * g.gd + min(g0 + u, g_last), lane);
+    }
+    build_plan_routes(ps, n_routes, plan_out, slot_id, route_expert);
+    if (!has_rows) return;
     // token operand of this wave's K-slice: token slot j (clamped), k-quarter jq of every group
     const uint32_t tok = slot.routes[min(j, n - 1)] / top_k;
     const uint16_t *xrow = x + (size_t)tok * x_stride + 8 * jq;
