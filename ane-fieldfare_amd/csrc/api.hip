@@ -548,9 +548,9 @@ int ffmoe_reduce_token_major(ffmoe_ctx *ctx, void *stream, const uint16_t *parti
     return FFMOE_OK;
 }
 
-int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
-                    const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows, uint32_t x_stride,
-                    uint32_t y_stride, int y_f32, char **err) {
+static int gemv_common(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                       const uint32_t *ids, const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows,
+                       uint32_t x_stride, uint32_t y_stride, int y_f32, char **err) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (!w || !scales || !biases || !x || !y) return fail(err, FFMOE_ERR_INVALID, "null argument");
     if (n == 0 || n % FFMOE_GROUP) return fail(err, FFMOE_ERR_INVALID, "N must be a multiple of %d", FFMOE_GROUP);
@@ -559,10 +559,23 @@ int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16
     if (rows == 0 || rows > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows=%u outside 1...%d", rows, FFMOE_MAX_VERIFY_ROWS);
     if (x_stride < n || y_stride < m) return fail(err, FFMOE_ERR_INVALID, "stride smaller than the row");
     ctx->timer.begin(static_cast<hipStream_t>(stream));
-    FF_HIP(launch_gemv_int4(static_cast<hipStream_t>(stream), w, scales, biases, x, y, m, n, rows, x_stride, y_stride, y_f32));
+    FF_HIP(launch_gemv_int4(static_cast<hipStream_t>(stream), w, scales, biases, x, y, m, n, rows, x_stride, y_stride, y_f32, ids));
     ctx->timer.mark(static_cast<hipStream_t>(stream), FFMOE_K_GEMV);
     ctx->timer.finish();
     return FFMOE_OK;
+}
+
+int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                    const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows, uint32_t x_stride,
+                    uint32_t y_stride, int y_f32, char **err) {
+    return gemv_common(ctx, stream, w, scales, biases, nullptr, x, y, m, n, rows, x_stride, y_stride, y_f32, err);
+}
+
+int ffmoe_gemv_int4_listed(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                           const uint32_t *ids, const uint16_t *x, float *y, uint32_t m, uint32_t n, uint32_t rows,
+                           uint32_t x_stride, uint32_t y_stride, char **err) {
+    if (!ids) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    return gemv_common(ctx, stream, w, scales, biases, ids, x, y, m, n, rows, x_stride, y_stride, 1, err);
 }
 
 int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases, uint32_t m,

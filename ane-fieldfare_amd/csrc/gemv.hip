@@ -56,10 +56,17 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const uint8_t *__restric
                                                         const uint16_t *__restrict__ biases,
                                                         const uint16_t *__restrict__ x, void *__restrict__ y_,
                                                         uint32_t m, uint32_t n, uint32_t rows, uint32_t x_stride,
-                                                        uint32_t y_stride) {
+                                                        uint32_t y_stride, const uint32_t *__restrict__ ids) {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t m0 = (blockIdx.x * 4 + wave) * kRowsPerWave;
     if (m0 >= m) return;
+    // output o is weight row o, or row ids[o] of the table when a list is given (encodeRowsListed)
+    uint32_t wrow[kRowsPerWave];
+#pragma unroll
+    for (int mi = 0; mi < kRowsPerWave; ++mi) {
+        const uint32_t o = min(m0 + mi, m - 1);
+        wrow[mi] = ids ? ids[o] : o;
+    }
     const uint32_t row_bytes = n / 2, n_groups = n / kGroup, chunks = n / 32;
     const uint32_t rounds = (chunks + 63) / 64;
 
@@ -98,7 +105,7 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const uint8_t *__restric
             uint32_t sb[kRowsPerWave];
 #pragma unroll
             for (int mi = 0; mi < kRowsPerWave; ++mi) {
-                const uint32_t row = min(m0 + mi, m - 1);
+                const uint32_t row = wrow[mi];
                 wv[mi] = load_chunk<ALIGNED>(w + (size_t)row * row_bytes + (size_t)c * 16);
                 const size_t gi = (size_t)row * n_groups + (c >> 1);
                 sb[mi] = (uint32_t)scales[gi] | ((uint32_t)biases[gi] << 16);
@@ -143,13 +150,13 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const uint8_t *__restric
 
 hipError_t launch_gemv_int4(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                             const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows,
-                            uint32_t x_stride, uint32_t y_stride, int y_f32) {
+                            uint32_t x_stride, uint32_t y_stride, int y_f32, const uint32_t *ids) {
     const uint32_t waves = (m + kRowsPerWave - 1) / kRowsPerWave;
     const dim3 grid((waves + 3) / 4), block(256);
     const bool aligned = (reinterpret_cast<uintptr_t>(w) % 16 == 0) && ((n / 2) % 16 == 0);
     const bool x_aligned = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (x_stride % 8 == 0);
 #define FFMOE_GEMV(A, X, F) \
-    hipLaunchKernelGGL((gemv_int4_kernel<A, X, F>), grid, block, 0, s, w, scales, biases, x, y, m, n, rows, x_stride, y_stride)
+    hipLaunchKernelGGL((gemv_int4_kernel<A, X, F>), grid, block, 0, s, w, scales, biases, x, y, m, n, rows, x_stride, y_stride, ids)
     if (aligned && x_aligned) { if (y_f32) FFMOE_GEMV(true, true, true); else FFMOE_GEMV(true, true, false); }
     else if (aligned) { if (y_f32) FFMOE_GEMV(true, false, true); else FFMOE_GEMV(true, false, false); }
     else if (x_aligned) { if (y_f32) FFMOE_GEMV(false, true, true); else FFMOE_GEMV(false, true, false); }

@@ -166,6 +166,6 @@ hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stri
 // gemv.hip
 hipError_t launch_gemv_int4(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                             const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows,
-                            uint32_t x_stride, uint32_t y_stride, int y_f32);
+                            uint32_t x_stride, uint32_t y_stride, int y_f32, const uint32_t *ids = nullptr);
 
 }  // namespace ffmoe

@@ -45,7 +45,7 @@ EXPORTS = [
     "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
     "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
-    "ffmoe_layer_tail", "ffmoe_route_verify",
+    "ffmoe_layer_tail", "ffmoe_route_verify", "ffmoe_gemv_int4_listed",
 ]
 
 PROFILE_SLOTS = 16
@@ -154,6 +154,7 @@ def lib() -> C.CDLL:
     L.ffmoe_last_live_experts.argtypes = [vp, vp, C.POINTER(u32), errp]
     L.ffmoe_reduce_token_major.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, errp]
     L.ffmoe_gemv_int4.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, i32, errp]
+    L.ffmoe_gemv_int4_listed.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, errp]
     L.ffmoe_set_profiling.argtypes = [vp, i32, errp]
     L.ffmoe_get_profile.argtypes = [vp, C.POINTER(Profile), i32, errp]
     L.ffmoe_prefill.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
@@ -431,6 +432,16 @@ class Context:
     def matrix(self, W, S, B, greedy: bool = False, w_byte_offset: int = 0):
         """Resident re-tiled copy of W uint8 [M, N/2], S/B bf16 bits [M, N/64] (numpy arrays or tensors)."""
         return Matrix(self, W, S, B, greedy, w_byte_offset)
+
+    def gemv_int4_listed(self, W, S, B, ids, x):
+        """GEMV over the weight rows listed in `ids` (int32 CUDA tensor [m]): y fp32 [R, m], y[:, o] = row ids[o]."""
+        import torch
+        m, n, rows = ids.shape[0], S.shape[1] * GROUP, x.shape[0]
+        y = torch.empty((rows, m), dtype=torch.float32, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_gemv_int4_listed(self._h, _stream(), _ptr(W), _ptr(S), _ptr(B), _ptr(ids), _ptr(x), _ptr(y), m, n,
+                                             rows, _row_stride(x), m, C.byref(err)), err)
+        return y
 
     def gemv_int4(self, W, S, B, x, f32_out: bool = False, w_byte_offset: int = 0):
         """W uint8 [M, N/2] (optionally starting `w_byte_offset` bytes into a larger buffer), S/B bf16-bit

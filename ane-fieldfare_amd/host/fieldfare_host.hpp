@@ -319,6 +319,16 @@ public:
         check(ffmoe_gemv_int4(c_.raw(), stream, weights, scales, biases, x, y, m, n, (uint32_t)rows, xStrideElements, yStrideElements,
                               types == RowsTypes::bf16ToF32 ? 1 : 0, &err), err);
     }
+    // DequantInt4GEMV.encodeRowsListed (DequantInt4GEMV.swift:124-145): output o is weight row ids[o]; fp32 out
+    void encodeRowsListed(void *stream, const uint8_t *weights, const uint16_t *scales, const uint16_t *biases, const uint32_t *ids,
+                          const uint16_t *x, float *y, uint32_t m, uint32_t n, int rows, uint32_t xStrideElements,
+                          uint32_t yStrideElements) {
+        if (rows <= 0 || rows > maxBatchRows) throw std::invalid_argument("rows outside 1...16");
+        if (n % FFMOE_GROUP) throw std::invalid_argument("N must be a multiple of 64");
+        char *err = nullptr;
+        check(ffmoe_gemv_int4_listed(c_.raw(), stream, weights, scales, biases, ids, x, y, m, n, (uint32_t)rows, xStrideElements,
+                                     yStrideElements, &err), err);
+    }
 
 private:
     Context &c_;

@@ -206,6 +206,14 @@ int ffmoe_gemv_int4(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16
                     const uint16_t *biases, const uint16_t *x, void *y, uint32_t m, uint32_t n,
                     uint32_t rows, uint32_t x_stride, uint32_t y_stride, int y_f32, char **err);
 
+/* The same over the m weight rows listed in `ids` (device, uint32): output o of each input row is the
+ * dot product with weight row ids[o]; fp32 out. The caller keeps every id inside the table.
+ * Replaces DequantInt4GEMV.encodeRowsListed (Kernels/Quant/DequantInt4GEMV.swift:124-145), the
+ * projection of the LM head's hot-vocabulary guess (Kernels/Fusions/LMHeadChainInt4.swift:171-177). */
+int ffmoe_gemv_int4_listed(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uint16_t *scales,
+                           const uint16_t *biases, const uint32_t *ids, const uint16_t *x, float *y, uint32_t m,
+                           uint32_t n, uint32_t rows, uint32_t x_stride, uint32_t y_stride, char **err);
+
 /* ---- resident INT4 matrix (LM head and other static weights) ------------------------------------ */
 
 #define FFMOE_MATRIX_MAX_N 2816  /* K kept in registers: 4 waves x 11 groups of 64 */

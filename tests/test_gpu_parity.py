@@ -408,3 +408,23 @@ def test_decode_sized_blocks_equal_rows_of_a_larger_block(small, real, oracle, t
     ref = oracle.moe_experts(fx["pool"], xb[:2], idx[:2].cpu().numpy().astype(np.uint32), w_np)
     got = oracle.bf16_to_float(bits_of(ctx.verify(layer, x[:2], idx[:2], w[:2])))
     assert rel_err(got, ref) < 1e-2 and cosine(got, ref) > 0.9999
+
+
+def test_gemv_int4_listed_rows(small, oracle, torch):
+    # encodeRowsListed (DequantInt4GEMV.swift:124-145): output o is weight row ids[o]; the hot-vocabulary
+    # projection of LMHeadChainInt4.swift:171-177. Same arithmetic per row as the full GEMV: equal bits.
+    ctx = small["ctx"]
+    m, n, rows = 1031, 1408, 5
+    g = oracle.seed_tree_key(0x11D5, "listed-gemv")
+    W, S, B = oracle.quantize_int4(g.uniform(-0.5, 0.5, m * n).reshape(m, n))
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, rows * n)).reshape(rows, n)
+    ids = np.array([7, 0, 1030, 512, 7, 64, 65, 1, 999], np.int32)          # unordered, with a repeat
+    tW, tS, tB = torch.from_numpy(W).cuda(), torch.from_numpy(S.view(np.int16)).cuda(), torch.from_numpy(B.view(np.int16)).cuda()
+    x = bf16_tensor(torch, xb)
+    full = ctx.gemv_int4(tW, tS, tB, x, f32_out=True).cpu().numpy()
+    listed = ctx.gemv_int4_listed(tW, tS, tB, torch.from_numpy(ids).cuda(), x).cpu().numpy()
+    assert listed.shape == (rows, ids.size)
+    assert np.array_equal(listed.view(np.uint32), full[:, ids].view(np.uint32))
+    for r in range(rows):
+        ref = oracle.gemv_int4_ref(W[ids], S[ids], B[ids], oracle.bf16_to_float(xb[r]))
+        assert rel_err(listed[r], ref) < 5e-3
