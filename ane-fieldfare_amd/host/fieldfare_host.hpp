@@ -247,6 +247,16 @@ public:
         char *err = nullptr;
         check(ffmoe_verify(c_.raw(), stream, layer, x, c_.shape().d, 1, indices, routingWeights, residual, y, &err), err);
     }
+    // encodeRouterRowsGemma4 followed by the routed experts of the same rows, as the decode and verify loops
+    // issue them back to back (RealForwardRunner.swift:1846-1923): one call, the routes also left on the device
+    void encodeRouterAndRoutedExperts(void *stream, uint32_t layer, const uint16_t *routerHidden, uint32_t routerStrideElements,
+                                      const uint16_t *x, uint32_t xStrideElements, int rows, const uint16_t *residual, uint16_t *y,
+                                      uint32_t *outIndices, uint16_t *outWeights) {
+        if (rows < 1 || rows > maxRouterRows) throw std::invalid_argument("rows outside 1...16");
+        char *err = nullptr;
+        check(ffmoe_route_verify(c_.raw(), stream, layer, routerHidden, routerStrideElements, x, xStrideElements, (uint32_t)rows,
+                                 residual, y, outIndices, outWeights, &err), err);
+    }
 
 private:
     Context &c_;
