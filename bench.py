@@ -150,6 +150,22 @@ def main():
     bytes_total = sum(live[i % L] for i in range(args.steps)) * EXPERT_BYTES
     value = bytes_total / elapsed / 1e9
 
+    # spread of the step time: one event after every step (a record costs the stream a few microseconds, so
+    # these intervals sit above ms_per_step by about one record; the spread is what they are for)
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    evs[0].record()
+    for i in range(args.steps):
+        step(i % L)
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    per_step = np.array([evs[i].elapsed_time(evs[i + 1]) * 1e3 for i in range(args.steps)])
+    step_spread = {"median": round(float(np.median(per_step)), 2), "p10": round(float(np.percentile(per_step, 10)), 2),
+                   "p90": round(float(np.percentile(per_step, 90)), 2), "n": int(args.steps),
+                   "note": "per-step HIP-event intervals, each including one event record"}
+    props = torch.cuda.get_device_properties(0)
+    device_info = {"name": props.name, "compute_units": props.multi_processor_count,
+                   "hbm_GiB": round(props.total_memory / 2 ** 30, 1), "torch": torch.__version__, "hip": torch.version.hip}
+
     if args.copy_probe:
         src_c = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
         dst_c = torch.empty_like(src_c)
@@ -547,6 +563,8 @@ def main():
                    "distinct_experts_min": int(min(live)), "distinct_experts_max": int(max(live)),
                    "expert_bytes_per_step_mean": int(np.mean(live) * EXPERT_BYTES)},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "step_us": step_spread,
+        "device": device_info,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": TRAFFIC_GATE_UP_VERIFY16 if (T == 16 and L == 30 and "down" in prof) else None,
