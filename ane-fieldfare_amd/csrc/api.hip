@@ -519,6 +519,31 @@ int ffmoe_layer_tail(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uint32_t 
     return FFMOE_OK;
 }
 
+int ffmoe_layer_tail_norms(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1,
+                           uint32_t h1_stride, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn1,
+                           const uint16_t *w_postffn2, const uint16_t *w_postffn, const uint16_t *w_next, uint16_t *normed,
+                           uint32_t normed_stride, uint32_t t, uint32_t d, float eps, float layer_scalar, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!h2 || !h1 || !hidden || !w_postffn1 || !w_postffn2 || !w_postffn) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if ((w_next == nullptr) != (normed == nullptr))
+        return fail(err, FFMOE_ERR_INVALID, "the next layer's norm weight and its output go together");
+    const uint32_t strides[4] = {h2_stride, h1_stride, hidden_stride, normed ? normed_stride : d};
+    if (int rc = check_rows(t, d, strides, 4, err)) return rc;
+    FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), h2, h2_stride, h1, h1_stride, hidden, hidden_stride, w_postffn2,
+                             w_postffn, t, d, eps, layer_scalar, w_postffn1, w_next, normed, normed_stride));
+    return FFMOE_OK;
+}
+
+int ffmoe_rmsnorm(ffmoe_ctx *ctx, void *stream, const uint16_t *x, uint32_t x_stride, const uint16_t *w, uint16_t *out,
+                  uint32_t out_stride, uint32_t t, uint32_t d, float eps, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!x || !w || !out) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    const uint32_t strides[2] = {x_stride, out_stride};
+    if (int rc = check_rows(t, d, strides, 2, err)) return rc;
+    FF_HIP(launch_rmsnorm(static_cast<hipStream_t>(stream), x, x_stride, w, out, out_stride, t, d, eps));
+    return FFMOE_OK;
+}
+
 int ffmoe_set_profiling(ffmoe_ctx *ctx, int enabled, char **err) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (enabled && !ctx->timer.ev[0])

@@ -121,14 +121,20 @@ __global__ __launch_bounds__(kRowThreads) void post_attn_setup_kernel(
         }
 }
 
-template <bool VEC>
+// NORMS: h1 arrives before its own norm (w_postffn1) and, when w_next is given, the norm of the new hidden
+// row under w_next goes to `normed` (the next layer's input norm): fused_layer_tail_norms
+// (Kernels/Fusions/FusedLayerTail.swift:74-117). h1 itself is left as it was found.
+template <bool VEC, bool NORMS>
 __global__ __launch_bounds__(kRowThreads) void layer_tail_kernel(const uint16_t *__restrict__ h2, uint32_t h2_stride,
                                                                  const uint16_t *__restrict__ h1, uint32_t h1_stride,
                                                                  uint16_t *__restrict__ hidden, uint32_t hidden_stride,
                                                                  const uint16_t *__restrict__ w_postffn2,
                                                                  const uint16_t *__restrict__ w_postffn, uint32_t d,
-                                                                 float eps, float layer_scalar) {
-    __shared__ float s_sum[2][4];
+                                                                 float eps, float layer_scalar,
+                                                                 const uint16_t *__restrict__ w_postffn1,
+                                                                 const uint16_t *__restrict__ w_next,
+                                                                 uint16_t *__restrict__ normed, uint32_t normed_stride) {
+    __shared__ float s_sum[4][4];
     const uint32_t row = blockIdx.x, t = threadIdx.x, chunks = d / 8;
     const uint32_t n_mine = t < chunks ? (chunks - t + kRowThreads - 1) / kRowThreads : 0;
     uint16_t *hrow = hidden + (size_t)row * hidden_stride;
@@ -139,6 +145,16 @@ __global__ __launch_bounds__(kRowThreads) void layer_tail_kernel(const uint16_t 
             a[c] = load8<VEC>(h2 + (size_t)row * h2_stride, t + c * kRowThreads);
             h12[c] = load8<VEC>(h1 + (size_t)row * h1_stride, t + c * kRowThreads);
         }
+    if (NORMS) {
+        const float inv_h1 = block_rms_inv(h12, n_mine, d, eps, s_sum[2]);
+#pragma unroll
+        for (int c = 0; c < kMaxChunks; ++c)
+            if ((uint32_t)c < n_mine) {
+                const Row8 w = load8<VEC>(w_postffn1, t + c * kRowThreads);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) h12[c].v[e] = round_bf16(h12[c].v[e] * inv_h1 * w.v[e]);
+            }
+    }
     const float inv_h2 = block_rms_inv(a, n_mine, d, eps, s_sum[0]);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
@@ -157,8 +173,46 @@ __global__ __launch_bounds__(kRowThreads) void layer_tail_kernel(const uint16_t 
             Row8 hv = load8<VEC>(hrow, chunk);
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-                hv.v[e] = round_bf16(hv.v[e] + round_bf16(h12[c].v[e] * inv_h12 * w.v[e])) * scale;
+                hv.v[e] = round_bf16(round_bf16(hv.v[e] + round_bf16(h12[c].v[e] * inv_h12 * w.v[e])) * scale);
             store8<VEC>(hrow, chunk, hv);
+            a[c] = hv;          // the new hidden row, as stored
+        }
+    if (NORMS && w_next) {
+        const float inv_next = block_rms_inv(a, n_mine, d, eps, s_sum[3]);
+#pragma unroll
+        for (int c = 0; c < kMaxChunks; ++c)
+            if ((uint32_t)c < n_mine) {
+                const uint32_t chunk = t + c * kRowThreads;
+                const Row8 w = load8<VEC>(w_next, chunk);
+                Row8 o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o.v[e] = a[c].v[e] * inv_next * w.v[e];
+                store8<VEC>(normed + (size_t)row * normed_stride, chunk, o);
+            }
+    }
+}
+
+// rmsnorm_bf16w (RMSNorm.encodeBF16W): out = round((x * inv) * w) per row; out may be x.
+template <bool VEC>
+__global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(const uint16_t *x, uint32_t x_stride, const uint16_t *__restrict__ w,
+                                                              uint16_t *out, uint32_t out_stride, uint32_t d, float eps) {
+    __shared__ float s_sum[4];
+    const uint32_t row = blockIdx.x, t = threadIdx.x, chunks = d / 8;
+    const uint32_t n_mine = t < chunks ? (chunks - t + kRowThreads - 1) / kRowThreads : 0;
+    Row8 a[kMaxChunks];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if ((uint32_t)c < n_mine) a[c] = load8<VEC>(x + (size_t)row * x_stride, t + c * kRowThreads);
+    const float inv = block_rms_inv(a, n_mine, d, eps, s_sum);
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if ((uint32_t)c < n_mine) {
+            const uint32_t chunk = t + c * kRowThreads;
+            const Row8 wv = load8<VEC>(w, chunk);
+            Row8 o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o.v[e] = a[c].v[e] * inv * wv.v[e];
+            store8<VEC>(out + (size_t)row * out_stride, chunk, o);
         }
 }
 
@@ -187,15 +241,27 @@ hipError_t launch_post_attn_setup(hipStream_t s, uint16_t *hidden, uint32_t hidd
 
 hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1, uint32_t h1_stride,
                              uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
-                             uint32_t t, uint32_t d, float eps, float layer_scalar) {
+                             uint32_t t, uint32_t d, float eps, float layer_scalar, const uint16_t *w_postffn1,
+                             const uint16_t *w_next, uint16_t *normed, uint32_t normed_stride) {
+    const bool norms = w_postffn1 != nullptr;
     const bool vec = aligned16(h2, h2_stride) && aligned16(h1, h1_stride) && aligned16(hidden, hidden_stride) &&
-                     aligned16(w_postffn2, 8) && aligned16(w_postffn, 8);
-    if (vec)
-        hipLaunchKernelGGL(layer_tail_kernel<true>, dim3(t), dim3(kRowThreads), 0, s, h2, h2_stride, h1, h1_stride, hidden,
-                           hidden_stride, w_postffn2, w_postffn, d, eps, layer_scalar);
+                     aligned16(w_postffn2, 8) && aligned16(w_postffn, 8) &&
+                     (!norms || (aligned16(w_postffn1, 8) && (!w_next || (aligned16(w_next, 8) && aligned16(normed, normed_stride)))));
+#define FFMOE_TAIL(V, N)                                                                                              \
+    hipLaunchKernelGGL((layer_tail_kernel<V, N>), dim3(t), dim3(kRowThreads), 0, s, h2, h2_stride, h1, h1_stride, hidden, \
+                       hidden_stride, w_postffn2, w_postffn, d, eps, layer_scalar, w_postffn1, w_next, normed, normed_stride)
+    if (vec) { if (norms) FFMOE_TAIL(true, true); else FFMOE_TAIL(true, false); }
+    else { if (norms) FFMOE_TAIL(false, true); else FFMOE_TAIL(false, false); }
+#undef FFMOE_TAIL
+    return hipGetLastError();
+}
+
+hipError_t launch_rmsnorm(hipStream_t s, const uint16_t *x, uint32_t x_stride, const uint16_t *w, uint16_t *out,
+                          uint32_t out_stride, uint32_t t, uint32_t d, float eps) {
+    if (aligned16(x, x_stride) && aligned16(out, out_stride) && aligned16(w, 8))
+        hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3(t), dim3(kRowThreads), 0, s, x, x_stride, w, out, out_stride, d, eps);
     else
-        hipLaunchKernelGGL(layer_tail_kernel<false>, dim3(t), dim3(kRowThreads), 0, s, h2, h2_stride, h1, h1_stride, hidden,
-                           hidden_stride, w_postffn2, w_postffn, d, eps, layer_scalar);
+        hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3(t), dim3(kRowThreads), 0, s, x, x_stride, w, out, out_stride, d, eps);
     return hipGetLastError();
 }
 

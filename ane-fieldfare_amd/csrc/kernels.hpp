@@ -161,7 +161,10 @@ hipError_t launch_post_attn_setup(hipStream_t s, uint16_t *hidden, uint32_t hidd
                                   uint32_t t, uint32_t d, float eps);
 hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1, uint32_t h1_stride,
                              uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
-                             uint32_t t, uint32_t d, float eps, float layer_scalar);
+                             uint32_t t, uint32_t d, float eps, float layer_scalar, const uint16_t *w_postffn1 = nullptr,
+                             const uint16_t *w_next = nullptr, uint16_t *normed = nullptr, uint32_t normed_stride = 0);
+hipError_t launch_rmsnorm(hipStream_t s, const uint16_t *x, uint32_t x_stride, const uint16_t *w, uint16_t *out,
+                          uint32_t out_stride, uint32_t t, uint32_t d, float eps);
 
 // gemv.hip
 hipError_t launch_gemv_int4(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,

@@ -46,6 +46,7 @@ EXPORTS = [
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
     "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
     "ffmoe_layer_tail", "ffmoe_route_verify", "ffmoe_gemv_int4_listed",
+    "ffmoe_layer_tail_norms", "ffmoe_rmsnorm",
 ]
 
 PROFILE_SLOTS = 16
@@ -154,6 +155,9 @@ def lib() -> C.CDLL:
     L.ffmoe_last_live_experts.argtypes = [vp, vp, C.POINTER(u32), errp]
     L.ffmoe_reduce_token_major.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, errp]
     L.ffmoe_gemv_int4.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, i32, errp]
+    L.ffmoe_layer_tail_norms.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, vp, vp, vp, vp, u32, u32, u32, C.c_float,
+                                         C.c_float, errp]
+    L.ffmoe_rmsnorm.argtypes = [vp, vp, vp, u32, vp, vp, u32, u32, u32, C.c_float, errp]
     L.ffmoe_gemv_int4_listed.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, errp]
     L.ffmoe_set_profiling.argtypes = [vp, i32, errp]
     L.ffmoe_get_profile.argtypes = [vp, C.POINTER(Profile), i32, errp]
@@ -427,6 +431,29 @@ class Context:
                                        _row_stride(hidden), _ptr(w_postffn2), _ptr(w_postffn), t, d, eps, layer_scalar,
                                        C.byref(err)), err)
         return hidden
+
+    def layer_tail_norms(self, h2, h1, hidden, w_postffn1, w_postffn2, w_postffn, layer_scalar: float, w_next=None,
+                         eps: float = 1e-6, d: int | None = None):
+        """The tail with h1 taken before its post-FFN-1 norm; with w_next also returns the next layer's input norm."""
+        import torch
+        t = hidden.shape[0]
+        d = d or self.shape.d
+        normed = torch.empty((t, d), dtype=torch.bfloat16, device=hidden.device) if w_next is not None else None
+        err = C.c_char_p()
+        _check(self.L.ffmoe_layer_tail_norms(self._h, _stream(), _ptr(h2), _row_stride(h2), _ptr(h1), _row_stride(h1), _ptr(hidden),
+                                             _row_stride(hidden), _ptr(w_postffn1), _ptr(w_postffn2), _ptr(w_postffn), _ptr(w_next),
+                                             _ptr(normed), d, t, d, eps, layer_scalar, C.byref(err)), err)
+        return normed
+
+    def rmsnorm(self, x, w, eps: float = 1e-6, d: int | None = None, out=None):
+        import torch
+        t = x.shape[0]
+        d = d or self.shape.d
+        y = out if out is not None else torch.empty((t, d), dtype=torch.bfloat16, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_rmsnorm(self._h, _stream(), _ptr(x), _row_stride(x), _ptr(w), _ptr(y), _row_stride(y), t, d, eps,
+                                    C.byref(err)), err)
+        return y
 
     # -- generic GEMV ----------------------------------------------------------------------------
     def matrix(self, W, S, B, greedy: bool = False, w_byte_offset: int = 0):

@@ -530,10 +530,38 @@ protected:
 class FusedLayerTail : public PrefillLayerTail {
 public:
     using PrefillLayerTail::PrefillLayerTail;
+    static constexpr bool fusesNorms = true;
     void encode(void *stream, const uint16_t *h2, const uint16_t *h1, uint16_t *hidden, const uint16_t *postFFN2Weight,
                 const uint16_t *postFFNWeight, uint32_t d, float eps, float layerScalar) {
         PrefillLayerTail::encode(stream, h2, h1, hidden, postFFN2Weight, postFFNWeight, 1, d, d, d, d, eps, layerScalar);
     }
+    // encodeWithNorms (FusedLayerTail.swift:74-117): h1 before its post-FFN-1 norm; nextInputNorm / nextNormed
+    // may both be null (no next layer)
+    void encodeWithNorms(void *stream, const uint16_t *h2, const uint16_t *h1, uint16_t *hidden, const uint16_t *postFFN1Weight,
+                         const uint16_t *postFFN2Weight, const uint16_t *postFFNWeight, const uint16_t *nextInputNorm,
+                         uint16_t *nextNormed, uint32_t d, float eps, float layerScalar) {
+        if (d == 0 || d > FFMOE_ROW_MAX_D) throw std::invalid_argument("D > 4096 exceeds the fused-tail row limit");
+        if ((nextInputNorm == nullptr) != (nextNormed == nullptr))
+            throw std::invalid_argument("nextInputNorm and nextNormed go together");
+        char *err = nullptr;
+        check(ffmoe_layer_tail_norms(c_.raw(), stream, h2, d, h1, d, hidden, d, postFFN1Weight, postFFN2Weight, postFFNWeight,
+                                     nextInputNorm, nextNormed, d, 1, d, eps, layerScalar, &err), err);
+    }
+};
+
+// RMSNorm.encodeBF16W: rows of x normalised under a bf16 weight; `out` may be `x`
+class RMSNorm {
+public:
+    explicit RMSNorm(Context &c) : c_(c) {}
+    void encodeBF16W(void *stream, const uint16_t *x, const uint16_t *weight, uint16_t *out, uint32_t d, float eps, uint32_t rows = 1,
+                     uint32_t xStrideElements = 0, uint32_t outStrideElements = 0) {
+        char *err = nullptr;
+        check(ffmoe_rmsnorm(c_.raw(), stream, x, xStrideElements ? xStrideElements : d, weight, out,
+                            outStrideElements ? outStrideElements : d, rows, d, eps, &err), err);
+    }
+
+private:
+    Context &c_;
 };
 
 // ---------------------------------------------------------------------------------------------------

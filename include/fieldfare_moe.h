@@ -306,6 +306,23 @@ int ffmoe_layer_tail(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uint32_t 
                      uint32_t h1_stride, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2,
                      const uint16_t *w_postffn, uint32_t t, uint32_t d, float eps, float layer_scalar, char **err);
 
+/* The layer tail with the two decode norms either side of it folded in: h1 arrives BEFORE its own norm
+ * (w_postffn1, the shared expert's post-FFN-1 norm; h1 is left as found), and when w_next / normed are
+ * given the norm of the new hidden row under w_next (the next layer's input norm) is written to normed.
+ * Bit for bit ffmoe_rmsnorm(h1), ffmoe_layer_tail, ffmoe_rmsnorm(hidden). Replaces
+ * FusedLayerTail.encodeWithNorms (Kernels/Fusions/FusedLayerTail.swift:74-117). */
+int ffmoe_layer_tail_norms(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1,
+                           uint32_t h1_stride, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn1,
+                           const uint16_t *w_postffn2, const uint16_t *w_postffn, const uint16_t *w_next,
+                           uint16_t *normed, uint32_t normed_stride, uint32_t t, uint32_t d, float eps,
+                           float layer_scalar, char **err);
+
+/* out[r] = round((x[r] * rsqrt(mean(x[r]^2) + eps)) * w) for t rows; out may be x. Replaces
+ * RMSNorm.encodeBF16W (kernel rmsnorm_bf16w), the operator the reference runs in front of the LM head
+ * (Kernels/Fusions/LMHeadChainInt4.swift:165-170) and around the tail. Same pointer rules as above. */
+int ffmoe_rmsnorm(ffmoe_ctx *ctx, void *stream, const uint16_t *x, uint32_t x_stride, const uint16_t *w,
+                  uint16_t *out, uint32_t out_stride, uint32_t t, uint32_t d, float eps, char **err);
+
 /* ---- per-kernel timing ------------------------------------------------------------------------ */
 
 /* Kernel slots of ffmoe_profile. */

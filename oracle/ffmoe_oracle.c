@@ -520,6 +520,15 @@ void ffo_post_attn_setup(uint16_t *hidden, const uint16_t *attn, uint16_t *dense
     free(h);
 }
 
+/* rmsnorm_bf16w (Metal/Norms/rmsnorm.metal; RMSNorm.encodeBF16W): out = r((x * inv) * w), one row. */
+void ffo_rmsnorm(const uint16_t *x, const uint16_t *w, uint16_t *out, int d, float eps, int dtype) {
+    float *a = (float *)calloc((size_t)d, sizeof(float));
+    for (int i = 0; i < d; ++i) a[i] = ffo_from_bits16(x[i], dtype);
+    const float inv = rms_inv_pinned(a, d, eps);
+    for (int i = 0; i < d; ++i) out[i] = ffo_bits16(a[i] * inv * ffo_bf16_to_float(w[i]), dtype);
+    free(a);
+}
+
 /* fused layer tail = one row of prefill_layer_tail_block (Metal/Prefill/prefill.metal:320-399), the
  * arithmetic of cpuReference in FusedLayerTailTests.swift:96-110: h12 = r(h1 + r(norm(h2, w_postffn2)));
  * hidden = r(r(hidden + r(norm(h12, w_postffn))) * r(layer_scalar)), every r a rounding to 16 bits. */

@@ -144,6 +144,7 @@ void ffo_moe_experts(const uint8_t *pool, size_t stride, const ffo_offsets *o, i
 void ffo_post_attn_setup(uint16_t *hidden, const uint16_t *attn, uint16_t *dense_x, uint16_t *routed_x,
                          uint16_t *router_x, const uint16_t *w_post_attn, const uint16_t *w_pre_ffn,
                          const uint16_t *w_pre_ffn2, int d, float eps, int dtype);
+void ffo_rmsnorm(const uint16_t *x, const uint16_t *w, uint16_t *out, int d, float eps, int dtype);
 void ffo_layer_tail(const uint16_t *h2, const uint16_t *h1, uint16_t *hidden, const uint16_t *w_postffn2,
                     const uint16_t *w_postffn, int d, float eps, float layer_scalar, int dtype);
 

@@ -99,6 +99,8 @@ def lib():
                                       C.c_int, C.c_int, C.c_int, vp, vp, vp, C.c_int]
         L.ffo_post_attn_setup.restype = None
         L.ffo_post_attn_setup.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int, C.c_float, C.c_int]
+        L.ffo_rmsnorm.restype = None
+        L.ffo_rmsnorm.argtypes = [vp, vp, vp, C.c_int, C.c_float, C.c_int]
         L.ffo_layer_tail.restype = None
         L.ffo_layer_tail.argtypes = [vp, vp, vp, vp, vp, C.c_int, C.c_float, C.c_float, C.c_int]
         L.ffo_max_threads.restype = C.c_int
@@ -427,6 +429,16 @@ def post_attn_setup(hidden_bits, attn_bits, w_post_attn, w_pre_ffn, w_pre_ffn2, 
         lib().ffo_post_attn_setup(_p(hidden[r]), _p(attn[r]), _p(outs[0][r]), _p(outs[1][r]), _p(outs[2][r]),
                                   _p(ws[0]), _p(ws[1]), _p(ws[2]), d, eps, dtype)
     return hidden, outs[0], outs[1], outs[2]
+
+
+def rmsnorm(x_bits, w_bits, eps: float = 1e-6, dtype: int = BF16) -> np.ndarray:
+    """Rows [T, D] of 16-bit patterns, bf16 weight [D] -> normalised rows."""
+    x = np.ascontiguousarray(np.array(x_bits, np.uint16, ndmin=2))
+    w = np.ascontiguousarray(w_bits, np.uint16)
+    out = np.empty_like(x)
+    for r in range(x.shape[0]):
+        lib().ffo_rmsnorm(_p(x[r]), _p(w), _p(out[r]), x.shape[1], eps, dtype)
+    return out
 
 
 def layer_tail(h2_bits, h1_bits, hidden_bits, w_postffn2, w_postffn, layer_scalar: float, eps: float = 1e-6,

@@ -299,6 +299,27 @@ int main() {
         tail1.encode(stream, dH2v, dH1v, dRow, dWt[3], dWt[4], d, 1e-6f, 0.875f);
         HIP(hipStreamSynchronize(stream));
         EXPECT(toHost(dRow, (size_t)d) == std::vector<uint16_t>(refT.begin(), refT.begin() + d));
+        // encodeWithNorms on row 0 equals RMSNorm(h1), encode, RMSNorm(hidden) bit for bit and leaves h1 alone
+        {
+            RMSNorm norm(ctx);
+            uint16_t *sepHid = toDevice(std::vector<uint16_t>(hid.begin(), hid.begin() + d));
+            uint16_t *fusHid = toDevice(std::vector<uint16_t>(hid.begin(), hid.begin() + d));
+            const std::vector<uint16_t> h1Before = toHost(dH1v, (size_t)d);
+            norm.encodeBF16W(stream, dH1v, dWt[0], dOut[0], d, 1e-6f);
+            tail1.encode(stream, dH2v, dOut[0], sepHid, dWt[3], dWt[4], d, 1e-6f, 0.875f);
+            norm.encodeBF16W(stream, sepHid, dWt[1], dOut[1], d, 1e-6f);
+            tail1.encodeWithNorms(stream, dH2v, dH1v, fusHid, dWt[0], dWt[3], dWt[4], dWt[1], dOut[2], d, 1e-6f, 0.875f);
+            HIP(hipStreamSynchronize(stream));
+            EXPECT(toHost(fusHid, (size_t)d) == toHost(sepHid, (size_t)d));
+            EXPECT(toHost(dOut[2], (size_t)d) == toHost(dOut[1], (size_t)d));
+            EXPECT(toHost(dH1v, (size_t)d) == h1Before);
+            bool threwPair = false;
+            try { tail1.encodeWithNorms(stream, dH2v, dH1v, fusHid, dWt[0], dWt[3], dWt[4], dWt[1], nullptr, d, 1e-6f, 1.f); }
+            catch (const std::invalid_argument &) { threwPair = true; }
+            EXPECT(threwPair);
+            HIP(hipFree(sepHid));
+            HIP(hipFree(fusHid));
+        }
         bool threwStride = false;
         try { tail.encode(stream, dH2v, dH1v, dHid, dWt[3], dWt[4], R, d, d - 8, d, d, 1e-6f, 1.f); } catch (const std::invalid_argument &) { threwStride = true; }
         EXPECT(threwStride);

@@ -128,3 +128,58 @@ def test_epilogue_argument_errors(ctx, torch):
         ctx.post_attn_setup(x.clone(), x, w, w, w, d=4104)
     with pytest.raises(ff.FieldfareError, match="stride is too small"):
         ctx.layer_tail(torch.zeros((2, 64), dtype=torch.bfloat16, device="cuda"), x, x.clone(), w, w, 1.0, d=136)
+
+
+def test_layer_tail_with_norms_equals_separate_steps(ctx, oracle, torch):
+    # fusedLayerTailNorms_matchSeparateDispatchesAndReference (FusedLayerTailTests.swift:15-93): same seed and
+    # ranges; the fused call equals rmsnorm(h1) -> tail -> rmsnorm(hidden) bit for bit, on the GPU and in the
+    # oracle, and leaves h1 as it found it
+    rng = oracle.SplitMix64(0x7A11_0001)
+    h2 = oracle.bf16_bits(rng.uniform(-1, 1, D))[None, :]
+    h1 = oracle.bf16_bits(rng.uniform(-3, 3, D))[None, :]
+    hidden = oracle.bf16_bits(rng.uniform(-2, 2, D))[None, :]
+    w = [oracle.bf16_bits(rng.uniform(0.5, 1.5, D)) for _ in range(4)]      # post 1, post 2, post, next input
+    scalar = float(rng.uniform(0.75, 1.25, 1)[0])
+    tw = [bf16_tensor(torch, x) for x in w]
+    # separate steps on the GPU
+    h1n = ctx.rmsnorm(bf16_tensor(torch, h1), tw[0], EPS, d=D)
+    sep_hidden = bf16_tensor(torch, hidden)
+    ctx.layer_tail(bf16_tensor(torch, h2), h1n, sep_hidden, tw[1], tw[2], scalar, EPS, d=D)
+    sep_normed = ctx.rmsnorm(sep_hidden, tw[3], EPS, d=D)
+    # the oracle's chain
+    ref_h1n = oracle.rmsnorm(h1, w[0], EPS)
+    ref_hidden = oracle.layer_tail(h2, ref_h1n, hidden, w[1], w[2], scalar, EPS)
+    ref_normed = oracle.rmsnorm(ref_hidden, w[3], EPS)
+    assert np.array_equal(bits_of(h1n), ref_h1n)
+    assert np.array_equal(bits_of(sep_hidden), ref_hidden) and np.array_equal(bits_of(sep_normed), ref_normed)
+    # fused
+    th1, fused_hidden = bf16_tensor(torch, h1), bf16_tensor(torch, hidden)
+    normed = ctx.layer_tail_norms(bf16_tensor(torch, h2), th1, fused_hidden, tw[0], tw[1], tw[2], scalar, w_next=tw[3], eps=EPS, d=D)
+    assert np.array_equal(bits_of(fused_hidden), ref_hidden) and np.array_equal(bits_of(normed), ref_normed)
+    assert np.array_equal(bits_of(th1), h1)
+    # without a next layer; several rows; rows that are only 2-byte aligned
+    rows = 3
+    blk = lambda lo, hi, stride: np.concatenate([oracle.bf16_bits(rng.uniform(lo, hi, rows * D)).reshape(rows, D),
+                                                 np.full((rows, stride - D), 0xC1A8, np.uint16)], axis=1)
+    bh2, bh1, bhid = blk(-1, 1, D + 9), blk(-3, 3, D + 13), blk(-2, 2, D + 17)
+    ref = oracle.layer_tail(bh2[:, :D], oracle.rmsnorm(bh1[:, :D], w[0], EPS), bhid[:, :D], w[1], w[2], scalar, EPS)
+    tb = bf16_tensor(torch, bhid)
+    assert ctx.layer_tail_norms(bf16_tensor(torch, bh2), bf16_tensor(torch, bh1), tb, tw[0], tw[1], tw[2], scalar, eps=EPS, d=D) is None
+    exp = bhid.copy()
+    exp[:, :D] = ref
+    assert np.array_equal(bits_of(tb), exp)
+
+
+def test_rmsnorm_rows_in_place_and_unit_rms(ctx, oracle, torch):
+    g = oracle.seed_tree_key(0x2A5, "rmsnorm")
+    for d, rows in ((64, 1), (2816, 16), (4096, 3)):
+        xb = oracle.bf16_bits(g.uniform(-4, 4, rows * d)).reshape(rows, d)
+        wb = oracle.bf16_bits(g.uniform(0.5, 1.5, d))
+        x = bf16_tensor(torch, xb)
+        out = ctx.rmsnorm(x, bf16_tensor(torch, wb), EPS, d=d)
+        ref = oracle.rmsnorm(xb, wb, EPS)
+        assert np.array_equal(bits_of(out), ref)
+        ctx.rmsnorm(x, bf16_tensor(torch, wb), EPS, d=d, out=x)               # in place
+        assert np.array_equal(bits_of(x), ref)
+        unit = oracle.bf16_to_float(bits_of(ctx.rmsnorm(bf16_tensor(torch, xb), bf16_tensor(torch, oracle.bf16_bits(np.ones(d, np.float32))), 0.0, d=d)))
+        assert np.allclose(np.sqrt((unit.astype(np.float64) ** 2).mean(axis=1)), 1.0, atol=3e-3)

@@ -352,6 +352,50 @@ def test_layer_tail_against_cpu_reference_restated(oracle):
         assert (got == ref).mean() > 0.95
 
 
+def test_rmsnorm_against_float64_and_tail_with_norms_chain(oracle):
+    # the plain norm against RmsNormRef in float64 (every element within one rounding step), the closed form
+    # for a constant row, and the reference test's full chain (cpuReference, FusedLayerTailTests.swift:96-110,
+    # with the post-FFN-1 norm in front and the next layer's norm behind) restated in float64
+    d, eps = 2816, 1e-6
+    for dtype, ulp in ((oracle.FP16, 2.0 ** -10), (oracle.BF16, 2.0 ** -7)):
+        rng = oracle.SplitMix64(0x7A11_0001)
+        h2 = oracle.bits16(rng.uniform(-1, 1, d), dtype)
+        h1 = oracle.bits16(rng.uniform(-3, 3, d), dtype)
+        hidden = oracle.bits16(rng.uniform(-2, 2, d), dtype)
+        weights = [oracle.bf16_bits(rng.uniform(0.5, 1.5, d)) for _ in range(4)]
+        scalar = float(rng.uniform(0.75, 1.25, 1)[0])
+        f = lambda bits: oracle.from_bits16(bits, dtype).astype(np.float64)
+        wf = [oracle.bf16_to_float(w).astype(np.float64) for w in weights]
+        got = f(oracle.rmsnorm(h1, weights[0], eps, dtype)[0])
+        ref = _rms_norm_ref64(f(h1), wf[0], eps)
+        assert np.all(np.abs(got - ref) <= np.abs(ref) * ulp)
+        r16 = lambda v: f(oracle.bits16(np.asarray(v, np.float32), dtype))
+        h1n = r16(ref)
+        h2n = r16(_rms_norm_ref64(f(h2), wf[1], eps))
+        h12n = r16(_rms_norm_ref64(r16(h1n + h2n), wf[2], eps))
+        new_hidden = r16(r16(f(hidden) + h12n) * r16(scalar))
+        normed = r16(_rms_norm_ref64(new_hidden, wf[3], eps))
+        o_hidden = oracle.layer_tail(h2, oracle.rmsnorm(h1, weights[0], eps, dtype), hidden, weights[1], weights[2], scalar, eps, dtype)
+        o_normed = f(oracle.rmsnorm(o_hidden, weights[3], eps, dtype)[0])
+        bound = 4e-3 if dtype == oracle.FP16 else 2e-2
+        assert np.abs(f(o_hidden[0]) - new_hidden).max() / np.abs(new_hidden).max() < bound
+        assert np.abs(o_normed - normed).max() / np.abs(normed).max() < bound
+    # a constant row c with unit weight normalises to sign(c) (eps = 0), whatever c
+    for c in (0.37, -5.0, 1024.0):
+        row = oracle.bf16_bits(np.full(256, c, np.float32))
+        out = oracle.bf16_to_float(oracle.rmsnorm(row, oracle.bf16_bits(np.ones(256, np.float32)), 0.0)[0])
+        assert np.array_equal(out, np.full(256, np.sign(c), np.float32))
+    # scaling the row by a power of two leaves the result unchanged (eps = 0); the weight scales it linearly
+    g = np.random.default_rng(5)
+    row = oracle.bf16_bits(g.uniform(-1, 1, 512).astype(np.float32))
+    w = oracle.bf16_bits(g.uniform(0.5, 1.5, 512).astype(np.float32))
+    base = oracle.rmsnorm(row, w, 0.0)
+    row4 = oracle.bf16_bits(oracle.bf16_to_float(row) * 4.0)
+    assert np.array_equal(oracle.rmsnorm(row4, w, 0.0), base)
+    w2 = oracle.bf16_bits(oracle.bf16_to_float(w) * 2.0)
+    assert np.array_equal(oracle.bf16_to_float(oracle.rmsnorm(row, w2, 0.0)), oracle.bf16_to_float(base) * 2.0)
+
+
 def test_post_attn_setup_against_primitive_chain(oracle):
     # fusedPostAttentionSetup_matchesPrimitiveChainBitwise_realShape (FusedPostAttentionSetupTests.swift:11-100):
     # the chain norm(attn) -> hidden += -> three norms of hidden, the router's with a unit weight; same seed
