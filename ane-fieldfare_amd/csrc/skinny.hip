@@ -28,42 +28,42 @@ constexpr int kMaxRoutes = kMaxRows * 8;
 
 // ---------------------------------------------------------------------------------------------------
 // Plan: invert routes [t][top_k] into per-expert route lists and compact the live experts in expert
-// order. Deterministic: LDS integer atomics only count; every ordering comes from ballot prefixes and
-// route order. A route takes part when its weight is not +-0 and its expert is in range; an expert
+// order. Deterministic: the LDS atomics only build sets; every ordering comes from ballot prefixes and
+// bit positions. A route takes part when its weight is not +-0 and its expert is in range; an expert
 // keeps its first 16 routes. Slots past the last live expert get n = 0.
 // ---------------------------------------------------------------------------------------------------
+static_assert(kMaxRoutes <= 128, "an expert's routes are kept as one 128-bit set");
+
 struct PlanScratch {
+    uint4 routes_of[FFMOE_MAX_EXPERTS];     // bit r set: route r goes to this expert
     uint32_t cnt[FFMOE_MAX_EXPERTS];
     uint32_t slot_of[FFMOE_MAX_EXPERTS];
     uint32_t expert_of[FFMOE_MAX_EXPERTS];
-    uint32_t route_expert[kMaxRoutes];
     uint32_t wave_total[4];
-    uint32_t my_routes[kMaxRows];
 };
 
-// Run by all 256 threads of a block. Builds the plan in LDS; writes it to `plan_out` when that is not
-// null; when `my_slot` is a live slot, leaves that slot's route list in ps.my_routes. Returns n_live.
-// `slot_from_total` maps the number of live experts to the caller's slot (or to ~0u for none).
-// Phase A: live experts compacted in expert order (ps.expert_of, ps.slot_of, ps.cnt); returns n_live and
-// leaves the calling thread's own route expert in `e`. Phase B: the route lists. A caller that streams
-// weights can start its loads between the two: the expert of its slot is known after phase A.
+// Run by all 256 threads of a block. Builds the plan in LDS and writes it to `plan_out` when that is not
+// null. Returns n_live. `slot_from_total` maps the number of live experts to the caller's slot (or to ~0u
+// for none). Thread r < n_routes brings route r's expert and weight (`route_idx`, `route_w`), so that the
+// caller decides when that load is issued.
+// Phase A: every expert's set of routes (one LDS or per route; a set has no order to get wrong), live
+// experts compacted in expert order (ps.expert_of, ps.slot_of, ps.cnt); returns n_live and leaves the
+// calling thread's own route expert in `e`. Phase B: the route lists, a route's place being the number of
+// lower routes in its expert's set; only a block that writes the plan out needs it.
 template <typename SlotFn>
-__device__ __forceinline__ uint32_t build_plan_experts(PlanScratch &ps, const uint32_t *__restrict__ idx,
-                                                       const uint16_t *__restrict__ w, uint32_t n_routes, uint32_t n_experts,
-                                                       VerifyPlan *plan_out, SlotFn slot_from_total, uint32_t &my_slot,
-                                                       uint32_t &e) {
+__device__ __forceinline__ uint32_t build_plan_experts(PlanScratch &ps, uint32_t route_idx, uint16_t route_w, uint32_t n_routes,
+                                                       uint32_t n_experts, VerifyPlan *plan_out, SlotFn slot_from_total,
+                                                       uint32_t &my_slot, uint32_t &e) {
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    ps.cnt[tid] = 0;
+    e = tid < n_routes && (route_w & 0x7FFFu) != 0 && route_idx < n_experts ? route_idx : 0xFFFFFFFFu;
+    ps.routes_of[tid] = uint4{0, 0, 0, 0};
     __syncthreads();
-    e = 0xFFFFFFFFu;
-    if (tid < n_routes) {
-        const uint32_t ee = idx[tid];
-        if ((w[tid] & 0x7FFFu) != 0 && ee < n_experts) e = ee;
-        ps.route_expert[tid] = e;
-        if (e != 0xFFFFFFFFu) atomicAdd(&ps.cnt[e], 1u);
-    }
+    if (e != 0xFFFFFFFFu) atomicOr(reinterpret_cast<uint32_t *>(&ps.routes_of[e]) + (tid >> 5), 1u << (tid & 31));
     __syncthreads();
-    const bool live = tid < n_experts && ps.cnt[tid] > 0;
+    const uint4 mine = ps.routes_of[tid];
+    const uint32_t count = tid < n_experts ? __popc(mine.x) + __popc(mine.y) + __popc(mine.z) + __popc(mine.w) : 0;
+    ps.cnt[tid] = count;
+    const bool live = count > 0;
     const unsigned long long mask = __ballot(live);
     const uint32_t before = __popcll(mask & ((1ull << lane) - 1ull));
     if (lane == 0) ps.wave_total[wave] = __popcll(mask);
@@ -80,7 +80,7 @@ __device__ __forceinline__ uint32_t build_plan_experts(PlanScratch &ps, const ui
         ps.expert_of[base + before] = tid;
         if (plan_out) {
             plan_out->slots[base + before].expert = tid;
-            plan_out->slots[base + before].n = min(ps.cnt[tid], (uint32_t)kMaxRows);
+            plan_out->slots[base + before].n = min(count, (uint32_t)kMaxRows);
         }
     }
     if (plan_out) {
@@ -95,37 +95,28 @@ __device__ __forceinline__ uint32_t build_plan_experts(PlanScratch &ps, const ui
     return total;
 }
 
-__device__ __forceinline__ void build_plan_routes(PlanScratch &ps, uint32_t n_routes, VerifyPlan *plan_out, uint32_t my_slot,
-                                                  uint32_t e) {
+__device__ __forceinline__ void build_plan_routes(PlanScratch &ps, uint32_t n_routes, VerifyPlan *plan_out, uint32_t e) {
     const uint32_t tid = threadIdx.x;
     if (tid < n_routes && e != 0xFFFFFFFFu) {
-        uint32_t pos = 0;
-        for (uint32_t j = 0; j < tid; ++j) pos += ps.route_expert[j] == e ? 1u : 0u;
-        if (pos < (uint32_t)kMaxRows) {
-            const uint32_t sl = ps.slot_of[e];
-            if (plan_out) plan_out->slots[sl].routes[pos] = tid;
-            if (sl == my_slot) ps.my_routes[pos] = tid;
-        }
+        const uint4 set = ps.routes_of[e];
+        const uint32_t word = tid >> 5, below = (1u << (tid & 31)) - 1u;
+        const uint32_t pos = __popc(set.x & (word > 0 ? 0xFFFFFFFFu : below)) +
+                             (word >= 1 ? __popc(set.y & (word > 1 ? 0xFFFFFFFFu : below)) : 0) +
+                             (word >= 2 ? __popc(set.z & (word > 2 ? 0xFFFFFFFFu : below)) : 0) +
+                             (word >= 3 ? __popc(set.w & below) : 0);
+        if (pos < (uint32_t)kMaxRows) plan_out->slots[ps.slot_of[e]].routes[pos] = tid;
     }
-    lds_barrier();      // LDS only: the caller's weight loads stay in flight across it
-}
-
-template <typename SlotFn>
-__device__ __forceinline__ uint32_t build_plan(PlanScratch &ps, const uint32_t *__restrict__ idx,
-                                               const uint16_t *__restrict__ w, uint32_t n_routes, uint32_t n_experts,
-                                               VerifyPlan *plan_out, SlotFn slot_from_total, uint32_t &my_slot) {
-    uint32_t e;
-    const uint32_t total = build_plan_experts(ps, idx, w, n_routes, n_experts, plan_out, slot_from_total, my_slot, e);
-    build_plan_routes(ps, n_routes, plan_out, my_slot, e);
-    return total;
 }
 
 __global__ __launch_bounds__(256) void verify_plan_kernel(const uint32_t *__restrict__ idx,
                                                           const uint16_t *__restrict__ w, uint32_t n_routes,
                                                           uint32_t n_experts, VerifyPlan *__restrict__ plan) {
     __shared__ PlanScratch ps;
-    uint32_t my_slot;
-    build_plan(ps, idx, w, n_routes, n_experts, plan, [](uint32_t) { return 0xFFFFFFFFu; }, my_slot);
+    uint32_t my_slot, e;
+    const bool has_route = threadIdx.x < n_routes;
+    build_plan_experts(ps, has_route ? idx[threadIdx.x] : 0u, has_route ? w[threadIdx.x] : (uint16_t)0, n_routes, n_experts, plan,
+                       [](uint32_t) { return 0xFFFFFFFFu; }, my_slot, e);
+    build_plan_routes(ps, n_routes, plan, e);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -319,62 +310,22 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     __shared__ PlanScratch ps;
     __shared__ uint32_t s_idx[ROUTE ? kRoutedRows * 8 : 1];
     __shared__ uint16_t s_w[ROUTE ? kRoutedRows * 8 : 1];
-    if (ROUTE) {
-        // Every block selects the top-k of the (at most kRoutedRows) rows itself, one wave per row: about a
-        // microsecond in front of the plan, against a launch of its own for the select. Block 0 writes the
-        // routes out for the combine pass and the caller.
-        const uint32_t rows = n_routes / top_k, wv = threadIdx.x >> 6;
-        for (uint32_t r = wv; r < rows; r += 4)
-            wave_topk(route.logits + (size_t)r * n_experts, route.per_expert_scale, n_experts, top_k, s_idx + r * top_k,
-                      s_w + r * top_k, threadIdx.x & 63);
-        __syncthreads();
-        if (blockIdx.x == 0 && threadIdx.x < n_routes) {
-            route.out_idx[threadIdx.x] = s_idx[threadIdx.x];
-            route.out_w[threadIdx.x] = s_w[threadIdx.x];
-        }
-        idx = s_idx;
-        w = s_w;
-    }
-    // Every block derives the routing plan itself from the (at most 128) routes: a few hundred LDS
-    // operations, against a separate launch plus two dependent global reads per block. Block 0 also
-    // writes the plan out for the down kernel.
-    const uint32_t gu_rb = g.gu_rb, n_blocks = gridDim.x, bid = blockIdx.x;
-    uint32_t slot_id, route_expert;
-    VerifyPlan *plan_out = bid == 0 ? plan : nullptr;
-    const uint32_t n_live = build_plan_experts(
-        ps, idx, w, n_routes, n_experts, plan_out,
-        [=](uint32_t total) { return total ? bid / max(1u, min(gu_rb, n_blocks / total)) : 0xFFFFFFFFu; }, slot_id,
-        route_expert);
-    // a block with no work still takes part in the barriers of the second phase (block 0 publishes the plan)
-    const bool has_slot = n_live != 0 && slot_id < n_live;
-    const uint32_t blocks_per_slot = max(1u, min(gu_rb, n_blocks / max(1u, n_live)));
-    uint32_t rb0 = 0, rb1 = 0;
-    if (has_slot) split_range(gu_rb, blocks_per_slot, bid % blocks_per_slot, rb0, rb1);
-    const bool has_rows = has_slot && rb0 < rb1;
-    const uint32_t slot_expert = has_slot ? __builtin_amdgcn_readfirstlane(ps.expert_of[slot_id]) : 0;
-    const uint32_t n = has_slot ? min(__builtin_amdgcn_readfirstlane(ps.cnt[slot_expert]), (uint32_t)kMaxRows) : 1;
-    struct { const uint32_t *routes; } slot = {ps.my_routes};
+    // The token operand is the block's rows themselves, row min(j, rows - 1) in token column j: which expert a
+    // block serves does not matter for fetching them, so they are requested first and are there when the plan
+    // is. An expert's routes only decide which columns of the result are stored.
+    const uint32_t rows = n_routes / top_k;
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15, jq = lane >> 4;
-    const uint8_t *expert_base = arena_layer + (size_t)slot_expert * g.expert_bytes;
     const uint32_t per = (g.gd + kKSplit - 1) / kKSplit;
     const uint32_t g0 = min(ks * per, g.gd), g1 = min(g.gd, g0 + per), ng = g1 - g0;
     const uint32_t g_last = g1 > g0 ? g1 - 1 : g.gd - 1;
-    const TileSource gu_src = make_tile_source(expert_base + g.gu_tiles_off, (size_t)g.gu_rb * g.gd * kTileBytes,
-                                               expert_base + g.gu_scales_off, (size_t)g.gu_rb * g.gd * kTileScaleBytes);
-
-    // the weights of the first tile row are requested as soon as the slot's expert is known; the route lists
-    // are worked out while those loads are in flight
-    WeightRing ring;
-    if (has_rows) {
-#pragma unroll
-        for (int u = 0; u < kRing; ++u) ring_fill(ring, u, gu_src, rb0 * g.gd + min(g0 + u, g_last), lane);
+    uint32_t route_idx = 0;
+    uint16_t route_w = 0;
+    if (!ROUTE && threadIdx.x < n_routes) {
+        route_idx = idx[threadIdx.x];
+        route_w = w[threadIdx.x];
     }
-    build_plan_routes(ps, n_routes, plan_out, slot_id, route_expert);
-    if (!has_rows) return;
-    // token operand of this wave's K-slice: token slot j (clamped), k-quarter jq of every group
-    const uint32_t tok = slot.routes[min(j, n - 1)] / top_k;
-    const uint16_t *xrow = x + (size_t)tok * x_stride + 8 * jq;
+    const uint16_t *xrow = x + (size_t)min(j, rows - 1) * x_stride + 8 * jq;
     uint4 x0[kRing], x1[kRing];
 #pragma unroll
     for (int u = 0; u < kRing; ++u) {
@@ -383,8 +334,61 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
         x0[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup) : uint4{0, 0, 0, 0};
         x1[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
     }
-    const uint32_t my_ts = 4 * jq + ks;     // the token slot this lane finishes
-    const uint32_t my_route = slot.routes[min(my_ts, n - 1)];
+    if (ROUTE) {
+        // Every block selects the top-k of the (at most kRoutedRows) rows itself, one wave per row: about a
+        // microsecond in front of the plan, against a launch of its own for the select. Block 0 writes the
+        // routes out for the combine pass and the caller.
+        const uint32_t wv = threadIdx.x >> 6;
+        for (uint32_t r = wv; r < rows; r += 4)
+            wave_topk(route.logits + (size_t)r * n_experts, route.per_expert_scale, n_experts, top_k, s_idx + r * top_k,
+                      s_w + r * top_k, lane);
+        __syncthreads();
+        if (threadIdx.x < n_routes) {
+            route_idx = s_idx[threadIdx.x];
+            route_w = s_w[threadIdx.x];
+            if (blockIdx.x == 0) {
+                route.out_idx[threadIdx.x] = route_idx;
+                route.out_w[threadIdx.x] = route_w;
+            }
+        }
+    }
+    // Every block derives the routing plan itself from the (at most 128) routes: a few dozen LDS
+    // operations, against a separate launch plus two dependent global reads per block. Block 0 also
+    // writes the plan out for the down kernel.
+    const uint32_t gu_rb = g.gu_rb, n_blocks = gridDim.x, bid = blockIdx.x;
+    uint32_t slot_id, route_expert;
+    VerifyPlan *plan_out = bid == 0 ? plan : nullptr;
+    const uint32_t n_live = build_plan_experts(
+        ps, route_idx, route_w, n_routes, n_experts, plan_out,
+        [=](uint32_t total) { return total ? bid / max(1u, min(gu_rb, n_blocks / total)) : 0xFFFFFFFFu; }, slot_id,
+        route_expert);
+    const bool has_slot = n_live != 0 && slot_id < n_live;
+    const uint32_t blocks_per_slot = max(1u, min(gu_rb, n_blocks / max(1u, n_live)));
+    uint32_t rb0 = 0, rb1 = 0;
+    if (has_slot) split_range(gu_rb, blocks_per_slot, bid % blocks_per_slot, rb0, rb1);
+    const bool has_rows = has_slot && rb0 < rb1;
+    const uint32_t slot_expert = has_slot ? __builtin_amdgcn_readfirstlane(ps.expert_of[slot_id]) : 0;
+    const uint8_t *expert_base = arena_layer + (size_t)slot_expert * g.expert_bytes;
+    const TileSource gu_src = make_tile_source(expert_base + g.gu_tiles_off, (size_t)g.gu_rb * g.gd * kTileBytes,
+                                               expert_base + g.gu_scales_off, (size_t)g.gu_rb * g.gd * kTileScaleBytes);
+    WeightRing ring;
+    if (has_rows) {
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) ring_fill(ring, u, gu_src, rb0 * g.gd + min(g0 + u, g_last), lane);
+    }
+    if (plan_out) build_plan_routes(ps, n_routes, plan_out, route_expert);
+    if (!has_rows) return;
+    // this lane finishes token column 4 jq + ks; `stores` = which of that row's top_k routes go to the expert
+    // (one bit at most unless a row names an expert twice)
+    const uint32_t col = 4 * jq + ks;
+    uint32_t stores = 0;
+    if (col < rows) {
+        const uint32_t *set = reinterpret_cast<const uint32_t *>(&ps.routes_of[slot_expert]);
+        const uint32_t first = col * top_k, word = first >> 5;
+        const uint64_t pair = (uint64_t)set[word] | ((uint64_t)(word < 3 ? set[word + 1] : 0u) << 32);
+        stores = (uint32_t)(pair >> (first & 31)) & ((1u << top_k) - 1u);
+    }
+    uint16_t *out_col = acts + (size_t)col * top_k * g.f + j;
 
     for (uint32_t rb = rb0; rb < rb1; ++rb) {
         // the refill targets the next row block; past the last one it re-reads the current tiles (cache hits)
@@ -409,7 +413,9 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
             ub += s_red[buf][o][4 + ks][lane];
         }
         // one rounding to 16 bits, gate and up themselves stay fp32 (moe.metal:496)
-        if (my_ts < n) acts[(size_t)my_route * g.f + rb * kTileRows + j] = f32_to_bf16(gelu_tanh_fast(ga) * ub);
+        const uint16_t v = f32_to_bf16(gelu_tanh_fast(ga) * ub);
+        for (uint32_t todo = stores; todo; todo &= todo - 1)
+            out_col[(size_t)__builtin_ctz(todo) * g.f + rb * kTileRows] = v;
     }
 }
 
