@@ -385,27 +385,8 @@ int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint1
                        uint32_t *out_idx, uint16_t *out_w, char **err) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (!out_idx || !out_w || !y) return fail(err, FFMOE_ERR_INVALID, "null argument");
-    if (t == 0 || t > FFMOE_MAX_VERIFY_ROWS || !verify_routes_in_kernel(ctx->geom, t, ctx->shape.top_k)) {
-        // larger blocks: the select keeps its own launch
-        if (int rc = ffmoe_router(ctx, stream, layer, router_x, router_x_stride, t, out_idx, out_w, nullptr, err)) return rc;
-        return ffmoe_verify(ctx, stream, layer, x, x_stride, t, out_idx, out_w, residual, y, err);
-    }
-    if (int rc = check_layer(ctx, layer, true, true, err)) return rc;
-    if (!router_x || !x) return fail(err, FFMOE_ERR_INVALID, "null argument");
-    if (router_x_stride < ctx->shape.d) return fail(err, FFMOE_ERR_INVALID, "hidden stride is too small");
-    if (x_stride < ctx->shape.d || x_stride % 8 || reinterpret_cast<uintptr_t>(x) % 16)
-        return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
-    if (reinterpret_cast<uintptr_t>(y) % 8 || (residual && reinterpret_cast<uintptr_t>(residual) % 8))
-        return fail(err, FFMOE_ERR_INVALID, "y and residual must be 8-byte aligned");
-    const ffmoe_layer &l = ctx->layers[layer];
-    RouterWeights rw{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale};
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    FF_HIP(launch_router(s, rw, router_x, router_x_stride, t, ctx->shape.n_experts, ctx->shape.d, ctx->shape.top_k, ctx->logits,
-                         out_idx, out_w, ctx->counters, &ctx->timer, true));
-    FF_HIP(launch_verify(s, ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom, ctx->shape.n_experts, ctx->shape.top_k, x,
-                         x_stride, t, out_idx, out_w, residual, y, nullptr, ctx->plan, ctx->acts, ctx->partials, ctx->n_cus,
-                         &ctx->timer, ctx->logits, l.per_expert_scale));
-    return FFMOE_OK;
+    if (int rc = ffmoe_router(ctx, stream, layer, router_x, router_x_stride, t, out_idx, out_w, nullptr, err)) return rc;
+    return ffmoe_verify(ctx, stream, layer, x, x_stride, t, out_idx, out_w, residual, y, err);
 }
 
 int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,

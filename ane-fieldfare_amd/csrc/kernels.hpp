@@ -120,16 +120,13 @@ hipError_t launch_dequant_expert(hipStream_t s, const uint8_t *arena_expert, Are
 // router.hip
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer, bool logits_only = false);
+                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer);
 
 // skinny.hip
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
-                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer,
-                         const float *route_logits = nullptr, const uint16_t *per_expert_scale = nullptr);
-// true when launch_verify can select the routes of a t-row block inside its gate/up kernel (route_logits given)
-bool verify_routes_in_kernel(ArenaGeom g, uint32_t t, uint32_t top_k);
+                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer);
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,
                                      uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d);
 

@@ -259,7 +259,7 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, co
 
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer, bool logits_only) {
+                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer) {
     (void)counters;
     timer->begin(s);
     const bool x_aligned = (reinterpret_cast<uintptr_t>(x) % 8 == 0) && (x_stride % 4 == 0);
@@ -272,11 +272,9 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
         else { if (x_aligned) FFMOE_ROUTER(false, true); else FFMOE_ROUTER(false, false); }
 #undef FFMOE_ROUTER
         timer->mark(s, FFMOE_K_ROUTER_LOGITS);
-        if (!logits_only) {
-            hipLaunchKernelGGL(router_topk_kernel, dim3(t), dim3(64), 0, s, logits, rw.per_expert_scale, n_experts, top_k,
-                               out_idx, out_w);
-            timer->mark(s, FFMOE_K_ROUTER_TOPK);
-        }
+        hipLaunchKernelGGL(router_topk_kernel, dim3(t), dim3(64), 0, s, logits, rw.per_expert_scale, n_experts, top_k, out_idx,
+                           out_w);
+        timer->mark(s, FFMOE_K_ROUTER_TOPK);
         timer->finish();
         return hipGetLastError();
     }

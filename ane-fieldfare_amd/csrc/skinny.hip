@@ -18,7 +18,6 @@
 #include "common.hpp"
 #include "kernels.hpp"
 #include "stream.hpp"
-#include "topk.hpp"
 
 namespace ffmoe {
 namespace {
@@ -288,28 +287,15 @@ __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restr
 // gate/up + GELU-tanh gating, persistent. grid = (blocks); the blocks are dealt to the live experts, each
 // block walks a range of 16-row blocks of its expert; its four waves split K and meet in LDS per row block
 // (partials added in wave order), each wave finishing a quarter of the token slots.
-// Router inputs of a block that selects its own routes: fp32 logits [t][n_experts] of the launch before.
-struct RouteSource {
-    const float *logits;
-    const uint16_t *per_expert_scale;   // bf16 [n_experts] or nullptr
-    uint32_t *out_idx;                  // [t][top_k], written by block 0
-    uint16_t *out_w;
-};
-
-constexpr int kRoutedRows = 8;          // rows a block routes itself: two per wave
-
-template <bool ROUTE>
 __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                                     uint32_t top_k, uint32_t n_experts,
                                                                     const uint32_t *__restrict__ idx,
                                                                     const uint16_t *__restrict__ w, uint32_t n_routes,
                                                                     VerifyPlan *__restrict__ plan,
                                                                     const uint16_t *__restrict__ x, uint32_t x_stride,
-                                                                    uint16_t *__restrict__ acts, RouteSource route) {
+                                                                    uint16_t *__restrict__ acts) {
     __shared__ float s_red[2][kKSplit][8][64];
     __shared__ PlanScratch ps;
-    __shared__ uint32_t s_idx[ROUTE ? kRoutedRows * 8 : 1];
-    __shared__ uint16_t s_w[ROUTE ? kRoutedRows * 8 : 1];
     // The token operand is the block's rows themselves, row min(j, rows - 1) in token column j: which expert a
     // block serves does not matter for fetching them, so they are requested first and are there when the plan
     // is. An expert's routes only decide which columns of the result are stored.
@@ -321,7 +307,7 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     const uint32_t g_last = g1 > g0 ? g1 - 1 : g.gd - 1;
     uint32_t route_idx = 0;
     uint16_t route_w = 0;
-    if (!ROUTE && threadIdx.x < n_routes) {
+    if (threadIdx.x < n_routes) {
         route_idx = idx[threadIdx.x];
         route_w = w[threadIdx.x];
     }
@@ -333,24 +319,6 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
         const uint32_t gg = min(g0 + u, g_last);
         x0[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup) : uint4{0, 0, 0, 0};
         x1[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
-    }
-    if (ROUTE) {
-        // Every block selects the top-k of the (at most kRoutedRows) rows itself, one wave per row: about a
-        // microsecond in front of the plan, against a launch of its own for the select. Block 0 writes the
-        // routes out for the combine pass and the caller.
-        const uint32_t wv = threadIdx.x >> 6;
-        for (uint32_t r = wv; r < rows; r += 4)
-            wave_topk(route.logits + (size_t)r * n_experts, route.per_expert_scale, n_experts, top_k, s_idx + r * top_k,
-                      s_w + r * top_k, lane);
-        __syncthreads();
-        if (threadIdx.x < n_routes) {
-            route_idx = s_idx[threadIdx.x];
-            route_w = s_w[threadIdx.x];
-            if (blockIdx.x == 0) {
-                route.out_idx[threadIdx.x] = route_idx;
-                route.out_w[threadIdx.x] = route_w;
-            }
-        }
     }
     // Every block derives the routing plan itself from the (at most 128) routes: a few dozen LDS
     // operations, against a separate launch plus two dependent global reads per block. Block 0 also
@@ -636,16 +604,10 @@ __global__ __launch_bounds__(256) void reduce_token_major_kernel(const uint16_t 
 
 }  // namespace
 
-bool verify_routes_in_kernel(ArenaGeom g, uint32_t t, uint32_t top_k) {
-    return (g.gd + kKSplit - 1) / kKSplit <= (uint32_t)kRing && t <= (uint32_t)kRoutedRows && top_k <= 8;
-}
-
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
-                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer,
-                         const float *route_logits, const uint16_t *per_expert_scale) {
-    if (route_logits && !verify_routes_in_kernel(g, t, top_k)) return hipErrorInvalidValue;
+                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer) {
     timer->begin(s);
     const uint32_t slots = min(n_experts, t * top_k);
     // the persistent kernels hold a K-slice of kRing groups per wave; larger experts take the one-shot grids
@@ -656,13 +618,8 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
     if (gu_persistent) {
         // plan slot of the profile stays empty: the gate/up kernel builds the plan itself
         const uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
-        if (route_logits)
-            hipLaunchKernelGGL(skinny_gate_up_persistent<true>, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts,
-                               nullptr, nullptr, t * top_k, plan, x, x_stride, acts,
-                               RouteSource{route_logits, per_expert_scale, const_cast<uint32_t *>(idx), const_cast<uint16_t *>(w)});
-        else
-            hipLaunchKernelGGL(skinny_gate_up_persistent<false>, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts,
-                               idx, w, t * top_k, plan, x, x_stride, acts, RouteSource{});
+        hipLaunchKernelGGL(skinny_gate_up_persistent, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, idx, w,
+                           t * top_k, plan, x, x_stride, acts);
     } else {
         hipLaunchKernelGGL(verify_plan_kernel, dim3(1), dim3(256), 0, s, idx, w, t * top_k, n_experts, plan);
         timer->mark(s, FFMOE_K_PLAN);

@@ -1,6 +1,7 @@
-// Top-k select + softmax weights of one row of router logits by one wave; shared by the router's own
-// kernel and by the gate/up kernel when it routes small blocks of rows itself.
+// Top-k select + softmax weights of one row of router logits by one wave.
 #pragma once
+
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -12,67 +13,99 @@ __device__ __forceinline__ uint32_t orderable(float v) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// Largest value of an unsigned quantity over the 64 lanes (zero if all are zero), the same in every lane:
+// four shifts inside each row of 16 lanes, two row broadcasts, one lane read. These are register-to-register
+// moves of a few cycles each; a butterfly of __shfl_xor would go through the LDS crossbar at more than a
+// hundred cycles a step, and the eight rounds of a select are one dependent chain.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    auto shifted = [](uint32_t x, auto ctrl, auto rows) {
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, decltype(ctrl)::value, decltype(rows)::value, 0xF, false);
+    };
+    using std::integral_constant;
+    v = max(v, shifted(v, integral_constant<int, 0x111>{}, integral_constant<int, 0xF>{}));   // row_shr:1
+    v = max(v, shifted(v, integral_constant<int, 0x112>{}, integral_constant<int, 0xF>{}));   // row_shr:2
+    v = max(v, shifted(v, integral_constant<int, 0x114>{}, integral_constant<int, 0xF>{}));   // row_shr:4
+    v = max(v, shifted(v, integral_constant<int, 0x118>{}, integral_constant<int, 0xF>{}));   // row_shr:8: lane 15 of a row holds the row
+    v = max(v, shifted(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xA>{}));   // row_bcast:15 into rows 1 and 3
+    v = max(v, shifted(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xC>{}));   // row_bcast:31 into rows 2 and 3
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
 // One wave: candidate e lives in lane e % 64, slot e / 64 (E <= 256). top_k rounds of a wave-wide
-// argmax over the total order (score desc, index asc); scores <= -inf and NaN are never taken; empty
-// rounds give (index 0, -inf) and weight 0 (moe.metal:194-236). 
-__device__ __forceinline__ void wave_topk(const float *row, const uint16_t *__restrict__ per_expert_scale,
-                                          uint32_t n_experts, uint32_t top_k, uint32_t *__restrict__ out_idx,
-                                          uint16_t *__restrict__ out_w, uint32_t lane) {
-    unsigned long long key[4];
-    float val[4];
+// argmax over the total order (score desc, index asc): the largest score by wave_max_u32, then the lowest
+// index that holds it by ballots, slot by slot. Scores <= -inf and NaN are never taken; empty rounds give
+// (index 0, -inf) and weight 0 (moe.metal:194-236). The weights: lane i takes exp(score_i - max) and the
+// division for rank i, the sum runs over the ranks in order as a serial loop would.
+// The three parts of a row's select: load, select, store.
+struct TopkRow {
+    uint32_t key[4];        // in: orderable score of candidate 64 c + lane, 0 = not a candidate
+    float ex, sum;          // out: lane i: exp(score_i - max); the sum over the ranks in order
+    uint32_t idx;           // out: lane i: index of rank i
+};
+
+__device__ __forceinline__ void topk_load(TopkRow &t, const float *row, uint32_t n_experts, uint32_t lane) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         const uint32_t e = c * 64 + lane;
-        val[c] = e < n_experts ? row[e] : -INFINITY;
-        const bool live = (val[c] > -INFINITY);   // false for NaN and -inf
-        key[c] = live ? (((unsigned long long)orderable(val[c]) << 32) | (0xFFFFFFFFu - e)) : 0ull;
+        const float v = e < n_experts ? row[e] : -INFINITY;
+        t.key[c] = v > -INFINITY ? orderable(v) : 0u;     // the comparison is false for NaN and -inf (every candidate's key is above 0x007FFFFF)
     }
-    uint32_t top_idx[8];
-    float top_score[8];
+}
+
+__device__ __forceinline__ void topk_select(TopkRow &t, uint32_t top_k, uint32_t lane) {
+    float mine = -INFINITY, max_s = -INFINITY;      // lane i: score of rank i
+    t.idx = 0;
 #pragma unroll
     for (uint32_t r = 0; r < 8; ++r) {
         if (r < top_k) {
-            unsigned long long best = key[0];
-#pragma unroll
-            for (int c = 1; c < 4; ++c) best = key[c] > best ? key[c] : best;
-#pragma unroll
-            for (int m = 32; m >= 1; m >>= 1) {
-                const unsigned long long o = __shfl_xor(best, m, 64);
-                best = o > best ? o : best;
-            }
-            if (best == 0ull) {
-                top_idx[r] = 0;
-                top_score[r] = -INFINITY;
-            } else {
-                const uint32_t e = 0xFFFFFFFFu - (uint32_t)best;
-                top_idx[r] = e;
+            const uint32_t best = wave_max_u32(max(max(t.key[0], t.key[1]), max(t.key[2], t.key[3])));
+            uint32_t e = 0;
+            float score = -INFINITY;
+            if (best != 0u) {
                 // recover the score from the key: orderable() is a bijection
-                const uint32_t o = (uint32_t)(best >> 32);
-                top_score[r] = __uint_as_float((o & 0x80000000u) ? (o & 0x7FFFFFFFu) : ~o);
+                score = __uint_as_float((best & 0x80000000u) ? (best & 0x7FFFFFFFu) : ~best);
+                bool found = false;
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    if (key[c] == best) key[c] = 0ull;
+                for (int c = 0; c < 4; ++c) {
+                    const unsigned long long holders = __ballot(t.key[c] == best);
+                    if (!found && holders != 0ull) {
+                        const uint32_t l = (uint32_t)__builtin_ctzll(holders);
+                        e = c * 64 + l;
+                        if (lane == l) t.key[c] = 0u;
+                        found = true;
+                    }
+                }
+            }
+            if (r == 0) max_s = score;
+            if (lane == r) {
+                mine = score;
+                t.idx = e;
             }
         }
     }
-    if (lane != 0) return;
-    const float max_s = top_score[0];
-    float sum = 0.0f, ex[8];
+    t.ex = expf(mine - max_s);
+    t.sum = 0.0f;
 #pragma unroll
-    for (uint32_t i = 0; i < 8; ++i) {
-        if (i < top_k) {
-            ex[i] = expf(top_score[i] - max_s);
-            sum += ex[i];
-        }
+    for (uint32_t i = 0; i < 8; ++i)
+        if (i < top_k) t.sum += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(t.ex), (int)i));
+}
+
+__device__ __forceinline__ void topk_store(const TopkRow &t, const uint16_t *__restrict__ per_expert_scale, uint32_t top_k,
+                                           uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w, uint32_t lane) {
+    if (lane < top_k) {
+        const float gain = per_expert_scale ? bf16_to_f32(per_expert_scale[t.idx]) : 1.0f;
+        out_idx[lane] = t.idx;
+        out_w[lane] = f32_to_bf16(t.ex / t.sum * gain);
     }
-#pragma unroll
-    for (uint32_t i = 0; i < 8; ++i) {
-        if (i < top_k) {
-            const float gain = per_expert_scale ? bf16_to_f32(per_expert_scale[top_idx[i]]) : 1.0f;
-            out_idx[i] = top_idx[i];
-            out_w[i] = f32_to_bf16(ex[i] / sum * gain);
-        }
-    }
+}
+
+__device__ __forceinline__ void wave_topk(const float *row, const uint16_t *__restrict__ per_expert_scale,
+                                          uint32_t n_experts, uint32_t top_k, uint32_t *__restrict__ out_idx,
+                                          uint16_t *__restrict__ out_w, uint32_t lane) {
+    TopkRow t;
+    topk_load(t, row, n_experts, lane);
+    topk_select(t, top_k, lane);
+    topk_store(t, per_expert_scale, top_k, out_idx, out_w, lane);
 }
 
 }  // namespace

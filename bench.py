@@ -213,11 +213,8 @@ def main():
         Lib.ffmoe_router(h, stream, layer, px1, D, 1, pidx, pw, None, C.byref(err))
         Lib.ffmoe_verify(h, stream, layer, px1, D, 1, pidx, pw, None, py, C.byref(err))
 
-    def decode_one_call(layer):
-        # router + experts in one call: the top-8 select runs inside the gate/up kernel (one launch fewer)
-        Lib.ffmoe_route_verify(h, stream, layer, px1, D, px1, D, 1, None, py, pidx, pw, C.byref(err))
     if not args.no_decode:
-        for name_, fn_ in (("decode_two_calls_us_per_layer", decode), ("decode_us_per_layer", decode_one_call)):
+        for name_, fn_ in (("decode_us_per_layer", decode),):
             for i in range(L):
                 fn_(i)
             torch.cuda.synchronize()

@@ -144,18 +144,17 @@ int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const ui
                           uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
                           uint16_t *partials, char **err);
 
-/* Number of distinct experts the last ffmoe_verify* call on `stream` ran (reads back 4 bytes; waits
- * for the stream). For reporting only. */
 /* Router and expert pass of one block in one call, for the decode loop that never shows the routes to
- * the host: ffmoe_router followed by ffmoe_verify, same results bit for bit, with the selected routes
- * also written to out_idx / out_w ([t][top_k], device). Up to 8 rows the top-k select runs inside the
- * gate/up kernel (one launch fewer); larger blocks are the two calls. Replaces the pair
- * MoE.encodeRouterGemma4 + encodeRoutedPersistentGPUSlots (Kernels/MoE/MoE.swift:168-247,454-496), where
- * the GPU routes the persistent kernels without a host round trip. */
+ * the host: ffmoe_router followed by ffmoe_verify on the same stream, with the selected routes also
+ * written to out_idx / out_w ([t][top_k], device). Replaces the pair MoE.encodeRouterGemma4 +
+ * encodeRoutedPersistentGPUSlots (Kernels/MoE/MoE.swift:168-247,454-496), where the GPU routes the
+ * persistent kernels without a host round trip. */
 int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *router_x,
                        uint32_t router_x_stride, const uint16_t *x, uint32_t x_stride, uint32_t t,
                        const uint16_t *residual, uint16_t *y, uint32_t *out_idx, uint16_t *out_w, char **err);
 
+/* Number of distinct experts the last ffmoe_verify* call on `stream` ran (reads back 4 bytes; waits
+ * for the stream). For reporting only. */
 int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char **err);
 
 /* ---- routed experts, prefill chunk (t <= max_tokens) ------------------------------------------- */

@@ -364,7 +364,7 @@ def test_gemv_int4_reference_shapes(small, oracle, torch, m, n, rows, off):
 @pytest.mark.parametrize("which,t", [("small", 1), ("small", 3), ("small", 8), ("small", 9), ("real", 1), ("real", 4),
                                      ("real", 8), ("real", 16)])
 def test_route_verify_equals_router_then_verify(small, real, oracle, torch, which, t):
-    # one call (up to 8 rows the select runs inside the gate/up kernel) against the two calls: routes,
+    # one call against the two calls: routes,
     # weights and outputs bit for bit; the routes are the oracle's
     fx = small if which == "small" else real
     ctx, d, layer = fx["ctx"], fx["d"], 1 if which == "small" else 0
