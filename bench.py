@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this same workload (seeded, so
 # the launches are the same ones), scaled by a plain 1 GiB copy: see profiles/hbm_traffic_verify16_prefill3072.txt
-TRAFFIC_GATE_UP_VERIFY16 = 113.1e6 + 0.3e6
+TRAFFIC_GATE_UP_VERIFY16 = 113.3e6 + 0.3e6
 TRAFFIC_PREFILL_GEMMS_3072 = (447.7e6 + 34.6e6) + (179.7e6 + 138.4e6)
 TOKEN_CORRELATION = 0.45                 # shared component of the block's tokens -> 40-60 distinct experts
 
