@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace ffmoe {
 
 constexpr int kGroup = 64;     // MLX-affine group size (Infrastructure/ModelIO/Quantization.swift:2)
@@ -95,8 +97,39 @@ __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
 // across the barrier; here the compiler's own counters still guard each prefetched register at its use.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// xor-butterfly sum across the 64 lanes (masks 32,16,8,4,2,1): every lane ends with the same value.
+// xor-butterfly sum across the 64 lanes (masks 32,16,8,4,2,1): every lane ends with the same value, and
+// every addition has the operands v[i] and v[i ^ mask] - the order the CPU oracle restates. The partners
+// come through register-to-register lane moves (gfx950 row swaps for 32 and 16, DPP rotations and quad
+// permutations below that) at a few cycles a step; __shfl_xor goes through the LDS crossbar at more than
+// a hundred, six times in a row on the critical path of every row reduction.
 __device__ __forceinline__ float wave_butterfly_sum(float v) {
+    auto dpp = [](float x, auto ctrl, auto banks, float old) {
+        return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp((int)__float_as_uint(old), (int)__float_as_uint(x),
+                                                                      decltype(ctrl)::value, 0xF, decltype(banks)::value, false));
+    };
+    using std::integral_constant;
+    // 32: the swap leaves (lower half, lower half) and (upper half, upper half) in the two registers
+    auto h = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(h[0]) + __uint_as_float(h[1]);
+    // 16: the same with the odd rows of one register and the even rows of the other
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    // 8: rotation by half a row
+    v = v + dpp(v, integral_constant<int, 0x128>{}, integral_constant<int, 0xF>{}, v);
+    // 4: lanes 0-3 and 8-11 of a row take from four lanes up (rotate right by 12), the others from four down
+    float p = dpp(v, integral_constant<int, 0x12C>{}, integral_constant<int, 0x5>{}, v);
+    p = dpp(v, integral_constant<int, 0x124>{}, integral_constant<int, 0xA>{}, p);
+    v = v + p;
+    // 2 and 1: permutations inside each quad
+    v = v + dpp(v, integral_constant<int, 0x4E>{}, integral_constant<int, 0xF>{}, v);
+    v = v + dpp(v, integral_constant<int, 0xB1>{}, integral_constant<int, 0xF>{}, v);
+    return v;
+}
+
+// The same sums (same operands in every addition) through the LDS crossbar: for kernels that reduce many
+// independent values per wave and have the vector ALU busy with other work, where throughput counts and the
+// latency of a step does not.
+__device__ __forceinline__ float wave_butterfly_sum_shuffle(float v) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) v = v + __shfl_xor(v, m, 64);
     return v;

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const uint8_t *__restric
         for (int mi = 0; mi < kRowsPerWave; ++mi) {
 #pragma unroll
             for (int r = 0; r < kRowTile; ++r) {
-                const float v = wave_butterfly_sum(acc[mi][r]);
+                const float v = wave_butterfly_sum_shuffle(acc[mi][r]);
                 if (lane == 0 && m0 + mi < m && r0 + r < rows) {
                     const size_t o = (size_t)(r0 + r) * y_stride + m0 + mi;
                     if (Y_F32) reinterpret_cast<float *>(y_)[o] = v;
