@@ -50,7 +50,8 @@ struct ffmoe_ctx {
     uint32_t max_pairs = 0;
     // dense FFN (n_experts == 1, top_k == 1): every row routes to expert 0 with weight 1
     uint32_t *dense_idx = nullptr;   // [max(max_tokens,16)] zeros
-    uint16_t *dense_w = nullptr;     // [max(max_tokens,16)] bf16 1.0
+    uint16_t *dense_w = nullptr;     // [max(max_tokens,16)] 1.0 in the activation type
+    bool f16 = false;                // activations are FP16 (ffmoe_set_activation_dtype)
     KernelTimer timer;
 };
 
@@ -192,6 +193,7 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (ctx->pf.sorted_out_row) (void)hipFree(ctx->pf.sorted_out_row);
     if (ctx->pf.acts) (void)hipFree(ctx->pf.acts);
     if (ctx->pf.partials) (void)hipFree(ctx->pf.partials);
+    if (ctx->pf.x16) (void)hipFree(ctx->pf.x16);
     if (ctx->dense_idx) (void)hipFree(ctx->dense_idx);
     if (ctx->dense_w) (void)hipFree(ctx->dense_w);
     for (auto &ev : ctx->timer.ev)
@@ -348,12 +350,15 @@ int ffmoe_router(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *r
     if (!router_x || !out_idx || !out_w) return fail(err, FFMOE_ERR_INVALID, "null argument");
     if (t == 0) return fail(err, FFMOE_ERR_INVALID, "queryCount must be positive");
     if (x_stride < ctx->shape.d) return fail(err, FFMOE_ERR_INVALID, "hidden stride is too small");
+    if (ctx->f16 && (reinterpret_cast<uintptr_t>(router_x) % 8 || x_stride % 4))
+        return fail(err, FFMOE_ERR_INVALID, "FP16 router rows must be 8-byte aligned with a stride that is a multiple of 4");
     const uint32_t cap = ctx->shape.max_tokens > FFMOE_MAX_VERIFY_ROWS ? ctx->shape.max_tokens : FFMOE_MAX_VERIFY_ROWS;
     if (!out_logits && t > cap) return fail(err, FFMOE_ERR_INVALID, "t = %u exceeds max_tokens = %u", t, cap);
     const ffmoe_layer &l = ctx->layers[layer];
     RouterWeights rw{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale};
     FF_HIP(launch_router(static_cast<hipStream_t>(stream), rw, router_x, x_stride, t, ctx->shape.n_experts,
-                         ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w, ctx->counters, &ctx->timer));
+                         ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w, ctx->counters, &ctx->timer,
+                         ctx->f16));
     return FFMOE_OK;
 }
 
@@ -370,7 +375,7 @@ static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uin
         return fail(err, FFMOE_ERR_INVALID, "y and residual must be 8-byte aligned");
     FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                         ctx->plan, ctx->acts, ctx->partials, ctx->n_cus, &ctx->timer));
+                         ctx->plan, ctx->acts, ctx->partials, ctx->n_cus, &ctx->timer, ctx->f16));
     return FFMOE_OK;
 }
 
@@ -420,7 +425,7 @@ static int prefill_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const ui
         return fail(err, FFMOE_ERR_INVALID, "outputs must be 16-byte aligned");
     FF_HIP(launch_prefill(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                           ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, pairs, n_pairs, y, partials,
-                          ctx->pf, &ctx->timer));
+                          ctx->pf, &ctx->timer, ctx->f16));
     return FFMOE_OK;
 }
 
@@ -484,7 +489,7 @@ int ffmoe_post_attn_setup(ffmoe_ctx *ctx, void *stream, uint16_t *hidden, uint32
     if (int rc = check_rows(t, d, strides, 5, err)) return rc;
     FF_HIP(launch_post_attn_setup(static_cast<hipStream_t>(stream), hidden, hidden_stride, attn, attn_stride, dense_x,
                                   dense_stride, routed_x, routed_stride, router_x, router_stride, w_post_attn, w_pre_ffn,
-                                  w_pre_ffn2, t, d, eps));
+                                  w_pre_ffn2, t, d, eps, ctx->f16));
     return FFMOE_OK;
 }
 
@@ -496,7 +501,7 @@ int ffmoe_layer_tail(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uint32_t 
     const uint32_t strides[3] = {h2_stride, h1_stride, hidden_stride};
     if (int rc = check_rows(t, d, strides, 3, err)) return rc;
     FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), h2, h2_stride, h1, h1_stride, hidden, hidden_stride,
-                             w_postffn2, w_postffn, t, d, eps, layer_scalar));
+                             w_postffn2, w_postffn, t, d, eps, layer_scalar, nullptr, nullptr, nullptr, 0, ctx->f16));
     return FFMOE_OK;
 }
 
@@ -511,7 +516,7 @@ int ffmoe_layer_tail_norms(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uin
     const uint32_t strides[4] = {h2_stride, h1_stride, hidden_stride, normed ? normed_stride : d};
     if (int rc = check_rows(t, d, strides, 4, err)) return rc;
     FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), h2, h2_stride, h1, h1_stride, hidden, hidden_stride, w_postffn2,
-                             w_postffn, t, d, eps, layer_scalar, w_postffn1, w_next, normed, normed_stride));
+                             w_postffn, t, d, eps, layer_scalar, w_postffn1, w_next, normed, normed_stride, ctx->f16));
     return FFMOE_OK;
 }
 
@@ -521,7 +526,27 @@ int ffmoe_rmsnorm(ffmoe_ctx *ctx, void *stream, const uint16_t *x, uint32_t x_st
     if (!x || !w || !out) return fail(err, FFMOE_ERR_INVALID, "null argument");
     const uint32_t strides[2] = {x_stride, out_stride};
     if (int rc = check_rows(t, d, strides, 2, err)) return rc;
-    FF_HIP(launch_rmsnorm(static_cast<hipStream_t>(stream), x, x_stride, w, out, out_stride, t, d, eps));
+    FF_HIP(launch_rmsnorm(static_cast<hipStream_t>(stream), x, x_stride, w, out, out_stride, t, d, eps, ctx->f16));
+    return FFMOE_OK;
+}
+
+int ffmoe_set_activation_dtype(ffmoe_ctx *ctx, int dtype, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (dtype != FFMOE_BF16 && dtype != FFMOE_FP16) return fail(err, FFMOE_ERR_INVALID, "activation dtype %d is neither FFMOE_BF16 nor FFMOE_FP16", dtype);
+    const bool f16 = dtype == FFMOE_FP16;
+    if (f16 && !ctx->pf.x16) {
+        // the prefill GEMMs run on bf16 tiles: room for the converted input rows of the largest chunk
+        const uint32_t cap = ctx->shape.max_tokens > FFMOE_MAX_VERIFY_ROWS ? ctx->shape.max_tokens : FFMOE_MAX_VERIFY_ROWS;
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.x16), (size_t)cap * ctx->shape.d * sizeof(uint16_t));
+        if (e != hipSuccess) return fail(err, FFMOE_ERR_ALLOC, "hipMalloc of the FP16 conversion rows: %s", hipGetErrorString(e));
+    }
+    if (ctx->dense_w) {
+        // the dense FFN's unit route weights follow the type
+        const uint32_t cap = ctx->shape.max_tokens > FFMOE_MAX_VERIFY_ROWS ? ctx->shape.max_tokens : FFMOE_MAX_VERIFY_ROWS;
+        FF_HIP(hipDeviceSynchronize());
+        FF_HIP(hipMemsetD16(reinterpret_cast<hipDeviceptr_t>(ctx->dense_w), f16 ? 0x3C00 : 0x3F80, cap));
+    }
+    ctx->f16 = f16;
     return FFMOE_OK;
 }
 
@@ -550,7 +575,7 @@ int ffmoe_reduce_token_major(ffmoe_ctx *ctx, void *stream, const uint16_t *parti
     if (t == 0) return fail(err, FFMOE_ERR_INVALID, "queryCount must be positive");
     if (top_k == 0) return fail(err, FFMOE_ERR_INVALID, "topK must be positive");
     if (d == 0) return fail(err, FFMOE_ERR_INVALID, "D must be positive");
-    FF_HIP(launch_reduce_token_major(static_cast<hipStream_t>(stream), partials, weights, h2, t, top_k, d));
+    FF_HIP(launch_reduce_token_major(static_cast<hipStream_t>(stream), partials, weights, h2, t, top_k, d, ctx->f16));
     return FFMOE_OK;
 }
 
@@ -565,7 +590,10 @@ static int gemv_common(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const uin
     if (rows == 0 || rows > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows=%u outside 1...%d", rows, FFMOE_MAX_VERIFY_ROWS);
     if (x_stride < n || y_stride < m) return fail(err, FFMOE_ERR_INVALID, "stride smaller than the row");
     ctx->timer.begin(static_cast<hipStream_t>(stream));
-    FF_HIP(launch_gemv_int4(static_cast<hipStream_t>(stream), w, scales, biases, x, y, m, n, rows, x_stride, y_stride, y_f32, ids));
+    if (ctx->f16 && (reinterpret_cast<uintptr_t>(x) % 16 || x_stride % 8))
+        return fail(err, FFMOE_ERR_INVALID, "FP16 input rows must be 16-byte aligned with a stride that is a multiple of 8");
+    FF_HIP(launch_gemv_int4(static_cast<hipStream_t>(stream), w, scales, biases, x, y, m, n, rows, x_stride, y_stride, y_f32, ids,
+                            ctx->f16));
     ctx->timer.mark(static_cast<hipStream_t>(stream), FFMOE_K_GEMV);
     ctx->timer.finish();
     return FFMOE_OK;
@@ -678,7 +706,7 @@ int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_
     ffmoe_ctx *ctx = mx->ctx;
     ctx->timer.begin(static_cast<hipStream_t>(stream));
     FF_HIP(launch_matrix_gemv(static_cast<hipStream_t>(stream), mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows,
-                              y, y_stride, y_f32 != 0, ctx->n_cus));
+                              y, y_stride, y_f32 != 0, ctx->n_cus, ctx->f16));
     ctx->timer.mark(static_cast<hipStream_t>(stream), FFMOE_K_GEMV);
     ctx->timer.finish();
     return FFMOE_OK;
@@ -693,7 +721,7 @@ int ffmoe_matrix_greedy(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint3
     hipStream_t s = static_cast<hipStream_t>(stream);
     ctx->timer.begin(s);
     FF_HIP(launch_matrix_gemv(s, mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows, mx->logits, mx->m, true,
-                              ctx->n_cus));
+                              ctx->n_cus, ctx->f16));
     ctx->timer.mark(s, FFMOE_K_GEMV);
     FF_HIP(launch_argmax_rows(s, mx->logits, mx->m, mx->m, rows, mx->partials, out_tokens));
     ctx->timer.mark(s, FFMOE_K_ARGMAX);

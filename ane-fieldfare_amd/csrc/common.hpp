@@ -92,6 +92,58 @@ __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
+// The two 16-bit activation types a context can run in (FFMOE_BF16, FFMOE_FP16): conversions, the offset
+// form of an INT4 weight for the streaming kernels and the matrix instruction that goes with it.
+// FP16 is the reference's text-path type (Metal/MoE/moe.metal:69,389,555). Offset form: 1024 + q is exact in
+// FP16 (ulp 1 at 1024) as 128 + q is in bf16, and 0x6400 | q needs no shift either.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+template <bool F16> struct Act;
+template <> struct Act<false> {
+    static constexpr uint32_t kOffsetBits = 0x43004300u, kOnesBits = 0x3F803F80u;
+    static constexpr float kOffset = 128.0f;
+    static __device__ __forceinline__ float lo(uint32_t pair) { return bf16lo_to_f32(pair); }
+    static __device__ __forceinline__ float hi(uint32_t pair) { return bf16hi_to_f32(pair); }
+    static __device__ __forceinline__ float widen(uint16_t b) { return bf16_to_f32(b); }
+    static __device__ __forceinline__ uint16_t round(float x) { return f32_to_bf16(x); }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) { return pack_bf16x2(a, b); }
+    static __device__ __forceinline__ f32x4 mfma(const uint4 &a, const uint4 &b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Act<true> {
+    static constexpr uint32_t kOffsetBits = 0x64006400u, kOnesBits = 0x3C003C00u;
+    static constexpr float kOffset = 1024.0f;
+    static __device__ __forceinline__ float lo(uint32_t pair) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xFFFFu)); }
+    static __device__ __forceinline__ float hi(uint32_t pair) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16)); }
+    static __device__ __forceinline__ float widen(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+    static __device__ __forceinline__ uint16_t round(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        f16x2 v;
+        v[0] = (_Float16)a;
+        v[1] = (_Float16)b;
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ f32x4 mfma(const uint4 &a, const uint4 &b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+// The eight nibbles of a dword as 16-bit values offset + q in the activation type (see unpack8_offset128).
+template <bool F16>
+__device__ __forceinline__ uint4 unpack8_offset(uint32_t w) {
+    uint32_t mask = 0x000F000Fu, c = Act<F16>::kOffsetBits;
+    asm("" : "+s"(mask));
+    asm("" : "+v"(c));
+    uint4 r;
+    r.x = (w & mask) | c;
+    r.y = ((w >> 4) & mask) | c;
+    r.z = ((w >> 8) & mask) | c;
+    r.w = ((w >> 12) & mask) | c;
+    return r;
+}
+
 // Workgroup barrier that waits for this wave's LDS traffic only. __syncthreads() also drains every
 // outstanding global load, which would serialise a register prefetch that is meant to stay in flight
 // across the barrier; here the compiler's own counters still guard each prefetched register at its use.

@@ -25,38 +25,45 @@ struct Row8 {
     float v[8];
 };
 
-template <bool VEC>
+// Rows are in the context's activation type (F16: FP16, else bf16); norm weights are always bf16 (loadw8).
+template <bool VEC, bool F16>
 __device__ __forceinline__ Row8 load8(const uint16_t *__restrict__ row, uint32_t chunk) {
     Row8 r;
     if (VEC) {
         const uint4 q = reinterpret_cast<const uint4 *>(row)[chunk];
-        r.v[0] = bf16lo_to_f32(q.x); r.v[1] = bf16hi_to_f32(q.x);
-        r.v[2] = bf16lo_to_f32(q.y); r.v[3] = bf16hi_to_f32(q.y);
-        r.v[4] = bf16lo_to_f32(q.z); r.v[5] = bf16hi_to_f32(q.z);
-        r.v[6] = bf16lo_to_f32(q.w); r.v[7] = bf16hi_to_f32(q.w);
+        r.v[0] = Act<F16>::lo(q.x); r.v[1] = Act<F16>::hi(q.x);
+        r.v[2] = Act<F16>::lo(q.y); r.v[3] = Act<F16>::hi(q.y);
+        r.v[4] = Act<F16>::lo(q.z); r.v[5] = Act<F16>::hi(q.z);
+        r.v[6] = Act<F16>::lo(q.w); r.v[7] = Act<F16>::hi(q.w);
     } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) r.v[e] = bf16_to_f32(row[8 * chunk + e]);
+        for (int e = 0; e < 8; ++e) r.v[e] = Act<F16>::widen(row[8 * chunk + e]);
     }
     return r;
 }
 
 template <bool VEC>
+__device__ __forceinline__ Row8 loadw8(const uint16_t *__restrict__ row, uint32_t chunk) {
+    return load8<VEC, false>(row, chunk);
+}
+
+template <bool VEC, bool F16>
 __device__ __forceinline__ void store8(uint16_t *__restrict__ row, uint32_t chunk, const Row8 &r) {
     if (VEC) {
         uint4 q;
-        q.x = pack_bf16x2(r.v[0], r.v[1]);
-        q.y = pack_bf16x2(r.v[2], r.v[3]);
-        q.z = pack_bf16x2(r.v[4], r.v[5]);
-        q.w = pack_bf16x2(r.v[6], r.v[7]);
+        q.x = Act<F16>::pack(r.v[0], r.v[1]);
+        q.y = Act<F16>::pack(r.v[2], r.v[3]);
+        q.z = Act<F16>::pack(r.v[4], r.v[5]);
+        q.w = Act<F16>::pack(r.v[6], r.v[7]);
         reinterpret_cast<uint4 *>(row)[chunk] = q;
     } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) row[8 * chunk + e] = f32_to_bf16(r.v[e]);
+        for (int e = 0; e < 8; ++e) row[8 * chunk + e] = Act<F16>::round(r.v[e]);
     }
 }
 
-__device__ __forceinline__ float round_bf16(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+template <bool F16>
+__device__ __forceinline__ float round16(float x) { return Act<F16>::widen(Act<F16>::round(x)); }
 
 // 1 / sqrt(mean of squares + eps) over the block's row; `slot` is a 4-float LDS area of its own
 __device__ __forceinline__ float block_rms_inv(const Row8 (&x)[kMaxChunks], uint32_t n_mine, uint32_t d, float eps,
@@ -74,7 +81,7 @@ __device__ __forceinline__ float block_rms_inv(const Row8 (&x)[kMaxChunks], uint
     return 1.0f / sqrtf(total / (float)d + eps);
 }
 
-template <bool VEC>
+template <bool VEC, bool F16>
 __global__ __launch_bounds__(kRowThreads) void post_attn_setup_kernel(
     uint16_t *__restrict__ hidden, uint32_t hidden_stride, const uint16_t *__restrict__ attn, uint32_t attn_stride,
     uint16_t *__restrict__ dense_x, uint32_t dense_stride, uint16_t *__restrict__ routed_x, uint32_t routed_stride,
@@ -89,24 +96,24 @@ __global__ __launch_bounds__(kRowThreads) void post_attn_setup_kernel(
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
         if ((uint32_t)c < n_mine) {
-            a[c] = load8<VEC>(arow, t + c * kRowThreads);
-            h[c] = load8<VEC>(hrow, t + c * kRowThreads);
+            a[c] = load8<VEC, F16>(arow, t + c * kRowThreads);
+            h[c] = load8<VEC, F16>(hrow, t + c * kRowThreads);
         }
     const float attn_inv = block_rms_inv(a, n_mine, d, eps, s_sum[0]);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
         if ((uint32_t)c < n_mine) {
-            const Row8 w = load8<VEC>(w_post_attn, t + c * kRowThreads);
+            const Row8 w = loadw8<VEC>(w_post_attn, t + c * kRowThreads);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) h[c].v[e] = round_bf16(h[c].v[e] + round_bf16(a[c].v[e] * attn_inv * w.v[e]));
-            store8<VEC>(hrow, t + c * kRowThreads, h[c]);
+            for (int e = 0; e < 8; ++e) h[c].v[e] = round16<F16>(h[c].v[e] + round16<F16>(a[c].v[e] * attn_inv * w.v[e]));
+            store8<VEC, F16>(hrow, t + c * kRowThreads, h[c]);
         }
     const float hidden_inv = block_rms_inv(h, n_mine, d, eps, s_sum[1]);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
         if ((uint32_t)c < n_mine) {
             const uint32_t chunk = t + c * kRowThreads;
-            const Row8 w1 = load8<VEC>(w_pre_ffn, chunk), w2 = load8<VEC>(w_pre_ffn2, chunk);
+            const Row8 w1 = loadw8<VEC>(w_pre_ffn, chunk), w2 = loadw8<VEC>(w_pre_ffn2, chunk);
             Row8 o_dense, o_routed, o_router;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -115,16 +122,16 @@ __global__ __launch_bounds__(kRowThreads) void post_attn_setup_kernel(
                 o_routed.v[e] = v * w2.v[e];
                 o_router.v[e] = v;
             }
-            store8<VEC>(dense_x + (size_t)row * dense_stride, chunk, o_dense);
-            store8<VEC>(routed_x + (size_t)row * routed_stride, chunk, o_routed);
-            store8<VEC>(router_x + (size_t)row * router_stride, chunk, o_router);
+            store8<VEC, F16>(dense_x + (size_t)row * dense_stride, chunk, o_dense);
+            store8<VEC, F16>(routed_x + (size_t)row * routed_stride, chunk, o_routed);
+            store8<VEC, F16>(router_x + (size_t)row * router_stride, chunk, o_router);
         }
 }
 
 // NORMS: h1 arrives before its own norm (w_postffn1) and, when w_next is given, the norm of the new hidden
 // row under w_next goes to `normed` (the next layer's input norm): fused_layer_tail_norms
 // (Kernels/Fusions/FusedLayerTail.swift:74-117). h1 itself is left as it was found.
-template <bool VEC, bool NORMS>
+template <bool VEC, bool NORMS, bool F16>
 __global__ __launch_bounds__(kRowThreads) void layer_tail_kernel(const uint16_t *__restrict__ h2, uint32_t h2_stride,
                                                                  const uint16_t *__restrict__ h1, uint32_t h1_stride,
                                                                  uint16_t *__restrict__ hidden, uint32_t hidden_stride,
@@ -142,39 +149,39 @@ __global__ __launch_bounds__(kRowThreads) void layer_tail_kernel(const uint16_t 
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
         if ((uint32_t)c < n_mine) {
-            a[c] = load8<VEC>(h2 + (size_t)row * h2_stride, t + c * kRowThreads);
-            h12[c] = load8<VEC>(h1 + (size_t)row * h1_stride, t + c * kRowThreads);
+            a[c] = load8<VEC, F16>(h2 + (size_t)row * h2_stride, t + c * kRowThreads);
+            h12[c] = load8<VEC, F16>(h1 + (size_t)row * h1_stride, t + c * kRowThreads);
         }
     if (NORMS) {
         const float inv_h1 = block_rms_inv(h12, n_mine, d, eps, s_sum[2]);
 #pragma unroll
         for (int c = 0; c < kMaxChunks; ++c)
             if ((uint32_t)c < n_mine) {
-                const Row8 w = load8<VEC>(w_postffn1, t + c * kRowThreads);
+                const Row8 w = loadw8<VEC>(w_postffn1, t + c * kRowThreads);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) h12[c].v[e] = round_bf16(h12[c].v[e] * inv_h1 * w.v[e]);
+                for (int e = 0; e < 8; ++e) h12[c].v[e] = round16<F16>(h12[c].v[e] * inv_h1 * w.v[e]);
             }
     }
     const float inv_h2 = block_rms_inv(a, n_mine, d, eps, s_sum[0]);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
         if ((uint32_t)c < n_mine) {
-            const Row8 w = load8<VEC>(w_postffn2, t + c * kRowThreads);
+            const Row8 w = loadw8<VEC>(w_postffn2, t + c * kRowThreads);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) h12[c].v[e] = round_bf16(h12[c].v[e] + round_bf16(a[c].v[e] * inv_h2 * w.v[e]));
+            for (int e = 0; e < 8; ++e) h12[c].v[e] = round16<F16>(h12[c].v[e] + round16<F16>(a[c].v[e] * inv_h2 * w.v[e]));
         }
     const float inv_h12 = block_rms_inv(h12, n_mine, d, eps, s_sum[1]);
-    const float scale = round_bf16(layer_scalar);
+    const float scale = round16<F16>(layer_scalar);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
         if ((uint32_t)c < n_mine) {
             const uint32_t chunk = t + c * kRowThreads;
-            const Row8 w = load8<VEC>(w_postffn, chunk);
-            Row8 hv = load8<VEC>(hrow, chunk);
+            const Row8 w = loadw8<VEC>(w_postffn, chunk);
+            Row8 hv = load8<VEC, F16>(hrow, chunk);
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-                hv.v[e] = round_bf16(round_bf16(hv.v[e] + round_bf16(h12[c].v[e] * inv_h12 * w.v[e])) * scale);
-            store8<VEC>(hrow, chunk, hv);
+                hv.v[e] = round16<F16>(round16<F16>(hv.v[e] + round16<F16>(h12[c].v[e] * inv_h12 * w.v[e])) * scale);
+            store8<VEC, F16>(hrow, chunk, hv);
             a[c] = hv;          // the new hidden row, as stored
         }
     if (NORMS && w_next) {
@@ -183,17 +190,17 @@ __global__ __launch_bounds__(kRowThreads) void layer_tail_kernel(const uint16_t 
         for (int c = 0; c < kMaxChunks; ++c)
             if ((uint32_t)c < n_mine) {
                 const uint32_t chunk = t + c * kRowThreads;
-                const Row8 w = load8<VEC>(w_next, chunk);
+                const Row8 w = loadw8<VEC>(w_next, chunk);
                 Row8 o;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) o.v[e] = a[c].v[e] * inv_next * w.v[e];
-                store8<VEC>(normed + (size_t)row * normed_stride, chunk, o);
+                store8<VEC, F16>(normed + (size_t)row * normed_stride, chunk, o);
             }
     }
 }
 
 // rmsnorm_bf16w (RMSNorm.encodeBF16W): out = round((x * inv) * w) per row; out may be x.
-template <bool VEC>
+template <bool VEC, bool F16>
 __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(const uint16_t *x, uint32_t x_stride, const uint16_t *__restrict__ w,
                                                               uint16_t *out, uint32_t out_stride, uint32_t d, float eps) {
     __shared__ float s_sum[4];
@@ -202,17 +209,17 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(const uint16_t *x,
     Row8 a[kMaxChunks];
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
-        if ((uint32_t)c < n_mine) a[c] = load8<VEC>(x + (size_t)row * x_stride, t + c * kRowThreads);
+        if ((uint32_t)c < n_mine) a[c] = load8<VEC, F16>(x + (size_t)row * x_stride, t + c * kRowThreads);
     const float inv = block_rms_inv(a, n_mine, d, eps, s_sum);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
         if ((uint32_t)c < n_mine) {
             const uint32_t chunk = t + c * kRowThreads;
-            const Row8 wv = load8<VEC>(w, chunk);
+            const Row8 wv = loadw8<VEC>(w, chunk);
             Row8 o;
 #pragma unroll
             for (int e = 0; e < 8; ++e) o.v[e] = a[c].v[e] * inv * wv.v[e];
-            store8<VEC>(out + (size_t)row * out_stride, chunk, o);
+            store8<VEC, F16>(out + (size_t)row * out_stride, chunk, o);
         }
 }
 
@@ -224,32 +231,39 @@ hipError_t launch_post_attn_setup(hipStream_t s, uint16_t *hidden, uint32_t hidd
                                   uint32_t attn_stride, uint16_t *dense_x, uint32_t dense_stride, uint16_t *routed_x,
                                   uint32_t routed_stride, uint16_t *router_x, uint32_t router_stride,
                                   const uint16_t *w_post_attn, const uint16_t *w_pre_ffn, const uint16_t *w_pre_ffn2,
-                                  uint32_t t, uint32_t d, float eps) {
+                                  uint32_t t, uint32_t d, float eps, bool f16) {
     const bool vec = aligned16(hidden, hidden_stride) && aligned16(attn, attn_stride) && aligned16(dense_x, dense_stride) &&
                      aligned16(routed_x, routed_stride) && aligned16(router_x, router_stride) && aligned16(w_post_attn, 8) &&
                      aligned16(w_pre_ffn, 8) && aligned16(w_pre_ffn2, 8);
-    if (vec)
-        hipLaunchKernelGGL(post_attn_setup_kernel<true>, dim3(t), dim3(kRowThreads), 0, s, hidden, hidden_stride, attn, attn_stride,
-                           dense_x, dense_stride, routed_x, routed_stride, router_x, router_stride, w_post_attn, w_pre_ffn,
-                           w_pre_ffn2, d, eps);
-    else
-        hipLaunchKernelGGL(post_attn_setup_kernel<false>, dim3(t), dim3(kRowThreads), 0, s, hidden, hidden_stride, attn, attn_stride,
-                           dense_x, dense_stride, routed_x, routed_stride, router_x, router_stride, w_post_attn, w_pre_ffn,
-                           w_pre_ffn2, d, eps);
+#define FFMOE_SETUP(V, H)                                                                                                  \
+    hipLaunchKernelGGL((post_attn_setup_kernel<V, H>), dim3(t), dim3(kRowThreads), 0, s, hidden, hidden_stride, attn, attn_stride, \
+                       dense_x, dense_stride, routed_x, routed_stride, router_x, router_stride, w_post_attn, w_pre_ffn,       \
+                       w_pre_ffn2, d, eps)
+    if (f16) { if (vec) FFMOE_SETUP(true, true); else FFMOE_SETUP(false, true); }
+    else { if (vec) FFMOE_SETUP(true, false); else FFMOE_SETUP(false, false); }
+#undef FFMOE_SETUP
     return hipGetLastError();
 }
 
 hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1, uint32_t h1_stride,
                              uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
                              uint32_t t, uint32_t d, float eps, float layer_scalar, const uint16_t *w_postffn1,
-                             const uint16_t *w_next, uint16_t *normed, uint32_t normed_stride) {
+                             const uint16_t *w_next, uint16_t *normed, uint32_t normed_stride, bool f16) {
     const bool norms = w_postffn1 != nullptr;
     const bool vec = aligned16(h2, h2_stride) && aligned16(h1, h1_stride) && aligned16(hidden, hidden_stride) &&
                      aligned16(w_postffn2, 8) && aligned16(w_postffn, 8) &&
                      (!norms || (aligned16(w_postffn1, 8) && (!w_next || (aligned16(w_next, 8) && aligned16(normed, normed_stride)))));
 #define FFMOE_TAIL(V, N)                                                                                              \
-    hipLaunchKernelGGL((layer_tail_kernel<V, N>), dim3(t), dim3(kRowThreads), 0, s, h2, h2_stride, h1, h1_stride, hidden, \
-                       hidden_stride, w_postffn2, w_postffn, d, eps, layer_scalar, w_postffn1, w_next, normed, normed_stride)
+    do {                                                                                                              \
+        if (f16)                                                                                                      \
+            hipLaunchKernelGGL((layer_tail_kernel<V, N, true>), dim3(t), dim3(kRowThreads), 0, s, h2, h2_stride, h1, h1_stride, \
+                               hidden, hidden_stride, w_postffn2, w_postffn, d, eps, layer_scalar, w_postffn1, w_next, normed, \
+                               normed_stride);                                                                        \
+        else                                                                                                          \
+            hipLaunchKernelGGL((layer_tail_kernel<V, N, false>), dim3(t), dim3(kRowThreads), 0, s, h2, h2_stride, h1, h1_stride, \
+                               hidden, hidden_stride, w_postffn2, w_postffn, d, eps, layer_scalar, w_postffn1, w_next, normed, \
+                               normed_stride);                                                                        \
+    } while (0)
     if (vec) { if (norms) FFMOE_TAIL(true, true); else FFMOE_TAIL(true, false); }
     else { if (norms) FFMOE_TAIL(false, true); else FFMOE_TAIL(false, false); }
 #undef FFMOE_TAIL
@@ -257,11 +271,13 @@ hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stri
 }
 
 hipError_t launch_rmsnorm(hipStream_t s, const uint16_t *x, uint32_t x_stride, const uint16_t *w, uint16_t *out,
-                          uint32_t out_stride, uint32_t t, uint32_t d, float eps) {
-    if (aligned16(x, x_stride) && aligned16(out, out_stride) && aligned16(w, 8))
-        hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3(t), dim3(kRowThreads), 0, s, x, x_stride, w, out, out_stride, d, eps);
-    else
-        hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3(t), dim3(kRowThreads), 0, s, x, x_stride, w, out, out_stride, d, eps);
+                          uint32_t out_stride, uint32_t t, uint32_t d, float eps, bool f16) {
+    const bool vec = aligned16(x, x_stride) && aligned16(out, out_stride) && aligned16(w, 8);
+#define FFMOE_NORM(V, H) \
+    hipLaunchKernelGGL((rmsnorm_kernel<V, H>), dim3(t), dim3(kRowThreads), 0, s, x, x_stride, w, out, out_stride, d, eps)
+    if (f16) { if (vec) FFMOE_NORM(true, true); else FFMOE_NORM(false, true); }
+    else { if (vec) FFMOE_NORM(true, false); else FFMOE_NORM(false, false); }
+#undef FFMOE_NORM
     return hipGetLastError();
 }
 

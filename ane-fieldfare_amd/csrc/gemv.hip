@@ -23,8 +23,10 @@ constexpr int kRowTile = 4;   // input rows held in registers per pass
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
+template <bool F16>
 __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+    if constexpr (F16) return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+    else return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
 }
 
 template <bool ALIGNED>
@@ -51,7 +53,8 @@ __device__ __forceinline__ uint4 load_x8(const uint16_t *src) {
     return r;
 }
 
-template <bool ALIGNED, bool X_ALIGNED, bool Y_F32>
+// F16: inputs and 16-bit outputs are FP16 (a context in FP16 mode); the offset form is then 1024 + q
+template <bool ALIGNED, bool X_ALIGNED, bool Y_F32, bool F16>
 __global__ __launch_bounds__(256) void gemv_int4_kernel(const uint8_t *__restrict__ w, const uint16_t *__restrict__ scales,
                                                         const uint16_t *__restrict__ biases,
                                                         const uint16_t *__restrict__ x, void *__restrict__ y_,
@@ -97,7 +100,7 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const uint8_t *__restric
                     xp[r][q * 4 + 2] = (d[1] & 0xFFFFu) | (d[3] << 16);
                     xp[r][q * 4 + 3] = (d[1] >> 16) | (d[3] & 0xFFFF0000u);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) { sum += bf16lo_to_f32(d[i]); sum += bf16hi_to_f32(d[i]); }
+                    for (int i = 0; i < 4; ++i) { sum += Act<F16>::lo(d[i]); sum += Act<F16>::hi(d[i]); }
                 }
                 sx[r] = sum;
             }
@@ -117,15 +120,15 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const uint8_t *__restric
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
 #pragma unroll
-                    for (int p = 0; p < 4; ++p) q[i * 4 + p] = ((ww[i] >> (4 * p)) & 0x000F000Fu) | 0x43004300u;
+                    for (int p = 0; p < 4; ++p) q[i * 4 + p] = ((ww[i] >> (4 * p)) & 0x000F000Fu) | Act<F16>::kOffsetBits;
                 }
                 const float s = bf16lo_to_f32(sb[mi]), b = bf16hi_to_f32(sb[mi]);
-                const float tb = __builtin_fmaf(-128.0f, s, b);
+                const float tb = __builtin_fmaf(-Act<F16>::kOffset, s, b);
 #pragma unroll
                 for (int r = 0; r < kRowTile; ++r) {
                     float dsum = 0.0f;
 #pragma unroll
-                    for (int p = 0; p < 16; ++p) dsum = dot2(q[p], xp[r][p], dsum);
+                    for (int p = 0; p < 16; ++p) dsum = dot2<F16>(q[p], xp[r][p], dsum);
                     acc[mi][r] = __builtin_fmaf(s, dsum, acc[mi][r]);
                     acc[mi][r] = __builtin_fmaf(tb, sx[r], acc[mi][r]);
                 }
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const uint8_t *__restric
                 if (lane == 0 && m0 + mi < m && r0 + r < rows) {
                     const size_t o = (size_t)(r0 + r) * y_stride + m0 + mi;
                     if (Y_F32) reinterpret_cast<float *>(y_)[o] = v;
-                    else reinterpret_cast<uint16_t *>(y_)[o] = f32_to_bf16(v);
+                    else reinterpret_cast<uint16_t *>(y_)[o] = Act<F16>::round(v);
                 }
             }
         }
@@ -150,13 +153,22 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const uint8_t *__restric
 
 hipError_t launch_gemv_int4(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                             const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows,
-                            uint32_t x_stride, uint32_t y_stride, int y_f32, const uint32_t *ids) {
+                            uint32_t x_stride, uint32_t y_stride, int y_f32, const uint32_t *ids, bool f16) {
     const uint32_t waves = (m + kRowsPerWave - 1) / kRowsPerWave;
     const dim3 grid((waves + 3) / 4), block(256);
     const bool aligned = (reinterpret_cast<uintptr_t>(w) % 16 == 0) && ((n / 2) % 16 == 0);
     const bool x_aligned = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (x_stride % 8 == 0);
+#define FFMOE_GEMV16(A, F) \
+    hipLaunchKernelGGL((gemv_int4_kernel<A, true, F, true>), grid, block, 0, s, w, scales, biases, x, y, m, n, rows, x_stride, y_stride, ids)
+    if (f16) {
+        if (!x_aligned) return hipErrorInvalidValue;     // FP16 rows come 16-byte aligned (checked at the boundary)
+        if (aligned) { if (y_f32) FFMOE_GEMV16(true, true); else FFMOE_GEMV16(true, false); }
+        else { if (y_f32) FFMOE_GEMV16(false, true); else FFMOE_GEMV16(false, false); }
+        return hipGetLastError();
+    }
+#undef FFMOE_GEMV16
 #define FFMOE_GEMV(A, X, F) \
-    hipLaunchKernelGGL((gemv_int4_kernel<A, X, F>), grid, block, 0, s, w, scales, biases, x, y, m, n, rows, x_stride, y_stride, ids)
+    hipLaunchKernelGGL((gemv_int4_kernel<A, X, F, false>), grid, block, 0, s, w, scales, biases, x, y, m, n, rows, x_stride, y_stride, ids)
     if (aligned && x_aligned) { if (y_f32) FFMOE_GEMV(true, true, true); else FFMOE_GEMV(true, true, false); }
     else if (aligned) { if (y_f32) FFMOE_GEMV(true, false, true); else FFMOE_GEMV(true, false, false); }
     else if (x_aligned) { if (y_f32) FFMOE_GEMV(false, true, true); else FFMOE_GEMV(false, true, false); }

@@ -101,7 +101,8 @@ struct PrefillScratch {
     uint32_t *sorted_token;     // [max pairs]
     uint32_t *sorted_out_row;   // [max pairs]: token * top_k + rank
     uint16_t *acts;             // [max pairs][F] bf16
-    uint16_t *partials;         // [max pairs][D] bf16 (used when the caller wants the combined output)
+    uint16_t *partials;         // [max pairs][D] 16-bit (used when the caller wants the combined output)
+    uint16_t *x16;              // [max tokens][D] bf16: the input rows of a context in FP16 mode, converted (else null)
 };
 
 struct RouterWeights {
@@ -120,15 +121,16 @@ hipError_t launch_dequant_expert(hipStream_t s, const uint8_t *arena_expert, Are
 // router.hip
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer);
+                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer, bool f16 = false);
 
 // skinny.hip
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
-                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer);
+                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer,
+                         bool f16 = false);
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,
-                                     uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d);
+                                     uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d, bool f16 = false);
 
 // matrix.hip: resident two-stream tiling of a [M][N] INT4 matrix, its multi-row GEMV and the greedy choice.
 size_t matrix_tiles_bytes(uint32_t m, uint32_t n);
@@ -139,7 +141,7 @@ hipError_t launch_matrix_repack(hipStream_t s, const uint8_t *w, const uint16_t 
                                 uint32_t m, uint32_t n, uint8_t *tiles_out, uint8_t *scales_out);
 hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                               const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
-                              bool y_f32, uint32_t n_cus);
+                              bool y_f32, uint32_t n_cus, bool f16 = false);
 hipError_t launch_argmax_rows(hipStream_t s, const float *y, uint32_t y_stride, uint32_t m, uint32_t rows,
                               unsigned long long *partials, uint32_t *out);
 
@@ -148,24 +150,25 @@ hipError_t launch_argmax_rows(hipStream_t s, const float *y, uint32_t y_stride, 
 hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
                           const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
                           const ffmoe_pair *pairs, uint32_t n_pairs_in, uint16_t *y, uint16_t *partials_out,
-                          PrefillScratch sc, KernelTimer *timer);
+                          PrefillScratch sc, KernelTimer *timer, bool f16 = false);
 
 // epilogue.hip: row-wise steps either side of the MoE stage
 hipError_t launch_post_attn_setup(hipStream_t s, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *attn,
                                   uint32_t attn_stride, uint16_t *dense_x, uint32_t dense_stride, uint16_t *routed_x,
                                   uint32_t routed_stride, uint16_t *router_x, uint32_t router_stride,
                                   const uint16_t *w_post_attn, const uint16_t *w_pre_ffn, const uint16_t *w_pre_ffn2,
-                                  uint32_t t, uint32_t d, float eps);
+                                  uint32_t t, uint32_t d, float eps, bool f16 = false);
 hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1, uint32_t h1_stride,
                              uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
                              uint32_t t, uint32_t d, float eps, float layer_scalar, const uint16_t *w_postffn1 = nullptr,
-                             const uint16_t *w_next = nullptr, uint16_t *normed = nullptr, uint32_t normed_stride = 0);
+                             const uint16_t *w_next = nullptr, uint16_t *normed = nullptr, uint32_t normed_stride = 0,
+                             bool f16 = false);
 hipError_t launch_rmsnorm(hipStream_t s, const uint16_t *x, uint32_t x_stride, const uint16_t *w, uint16_t *out,
-                          uint32_t out_stride, uint32_t t, uint32_t d, float eps);
+                          uint32_t out_stride, uint32_t t, uint32_t d, float eps, bool f16 = false);
 
 // gemv.hip
 hipError_t launch_gemv_int4(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                             const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows,
-                            uint32_t x_stride, uint32_t y_stride, int y_f32, const uint32_t *ids = nullptr);
+                            uint32_t x_stride, uint32_t y_stride, int y_f32, const uint32_t *ids = nullptr, bool f16 = false);
 
 }  // namespace ffmoe

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void repack_matrix_kernel(const uint8_t *__res
 // (at most kRing groups each), keep their slice of the input rows in registers and refill the weight
 // ring across tiles; per tile the partial sums meet in LDS, are added in wave order, and each wave
 // stores a quarter of the input rows.
-template <bool Y_F32>
+template <bool Y_F32, bool F16>
 __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__restrict__ tiles,
                                                              const uint8_t *__restrict__ scales, uint32_t m,
                                                              uint32_t n_groups, const uint16_t *__restrict__ x,
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min(g0 + u, g_last), lane);
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min(g0 + u, g_last), lane);
         const int buf = (rb - rb0) & 1;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -135,8 +135,8 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
                 if (row_a < m) y32[base + row_a] = va;
                 if (row_b < m) y32[base + row_b] = vb;
             } else {
-                if (row_a < m) y16[base + row_a] = f32_to_bf16(va);
-                if (row_b < m) y16[base + row_b] = f32_to_bf16(vb);
+                if (row_a < m) y16[base + row_a] = Act<F16>::round(va);
+                if (row_b < m) y16[base + row_b] = Act<F16>::round(vb);
             }
         }
     }
@@ -209,15 +209,14 @@ hipError_t launch_matrix_repack(hipStream_t s, const uint8_t *w, const uint16_t 
 
 hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                               const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
-                              bool y_f32, uint32_t n_cus) {
+                              bool y_f32, uint32_t n_cus, bool f16) {
     const uint32_t n_tiles = (m + 31) / 32;
     const dim3 grid(min(2 * n_cus, n_tiles));
-    if (y_f32)
-        hipLaunchKernelGGL(matrix_gemv_kernel<true>, grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, rows,
-                           y, y_stride);
-    else
-        hipLaunchKernelGGL(matrix_gemv_kernel<false>, grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride,
-                           rows, y, y_stride);
+#define FFMOE_MGEMV(Y, H) \
+    hipLaunchKernelGGL((matrix_gemv_kernel<Y, H>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, rows, y, y_stride)
+    if (f16) { if (y_f32) FFMOE_MGEMV(true, true); else FFMOE_MGEMV(false, true); }
+    else { if (y_f32) FFMOE_MGEMV(true, false); else FFMOE_MGEMV(false, false); }
+#undef FFMOE_MGEMV
     return hipGetLastError();
 }
 

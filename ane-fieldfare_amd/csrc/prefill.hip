@@ -194,7 +194,7 @@ struct GemmWave {
 
 // The k-loop and epilogue of one wave that owns NMB 16-row blocks (a compile-time count: the MFMA
 // sequence has no branches, so the scheduler can interleave it with the expansion of the next tile).
-template <bool GATE_UP, int NMB>
+template <bool GATE_UP, int NMB, bool OUT_F16>
 __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g, uint4 (*wb)[kTilesPerBlock][2][2][kWave],
                                           const uint32_t *__restrict__ sorted_token,
                                           const uint32_t *__restrict__ sorted_out_row, uint16_t *__restrict__ out) {
@@ -372,7 +372,7 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
         for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) {
             const f32x4 v = acc[i][nf];
             *reinterpret_cast<uint2 *>(stage + j * kStageRow + nf * 32 + 8 * jq) =
-                make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+                make_uint2(Act<OUT_F16>::pack(v[0], v[1]), Act<OUT_F16>::pack(v[2], v[3]));
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -390,7 +390,8 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     }
 }
 
-template <bool GATE_UP>
+// OUT_F16: the down projection's per-route rows leave as FP16 instead of bf16 (a context in FP16 mode)
+template <bool GATE_UP, bool OUT_F16 = false>
 __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                               const PrefillPlan *__restrict__ plan,
                                                               const PrefillTile *__restrict__ tiles,
@@ -421,17 +422,18 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__r
     const uint32_t n_mb = (gw.tile.rows + 15) / 16;
     const uint32_t my_mb = n_mb > gw.wave ? (n_mb - gw.wave + 3) / 4 : 0;    // 16-row blocks of this wave
     switch (my_mb) {
-        case 0: gemm_wave<GATE_UP, 0>(gw, g, wb, sorted_token, sorted_out_row, out); break;
-        case 1: gemm_wave<GATE_UP, 1>(gw, g, wb, sorted_token, sorted_out_row, out); break;
-        case 2: gemm_wave<GATE_UP, 2>(gw, g, wb, sorted_token, sorted_out_row, out); break;
-        case 3: gemm_wave<GATE_UP, 3>(gw, g, wb, sorted_token, sorted_out_row, out); break;
-        default: gemm_wave<GATE_UP, 4>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        case 0: gemm_wave<GATE_UP, 0, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        case 1: gemm_wave<GATE_UP, 1, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        case 2: gemm_wave<GATE_UP, 2, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        case 3: gemm_wave<GATE_UP, 3, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        default: gemm_wave<GATE_UP, 4, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
     }
 }
 
 // h2[t][c] = bf16(sum_r w[t][r] * partial[t][r][c]) over the routes the sort kept, fma in rank order
 // (prefill.metal:544-565); dropped routes (zero weight, expert out of range) add nothing, which equals
 // the reference's zero-filled partial rows without having to clear 138 MB first.
+template <bool F16>
 __global__ __launch_bounds__(256) void prefill_combine_kernel(const uint16_t *__restrict__ partials,
                                                               const uint16_t *__restrict__ w,
                                                               const uint32_t *__restrict__ idx, uint32_t n_experts,
@@ -444,21 +446,36 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(const uint16_t *__
         const uint32_t route = tok * top_k + r;
         const uint16_t wbits = w[route];
         if ((wbits & 0x7FFFu) == 0 || idx[route] >= n_experts) continue;
-        const float wv = bf16_to_f32(wbits);
+        const float wv = Act<F16>::widen(wbits);
         const uint4 p = *reinterpret_cast<const uint4 *>(partials + (size_t)route * d + c);
         const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            acc[2 * i] = __builtin_fmaf(wv, bf16lo_to_f32(pw[i]), acc[2 * i]);
-            acc[2 * i + 1] = __builtin_fmaf(wv, bf16hi_to_f32(pw[i]), acc[2 * i + 1]);
+            acc[2 * i] = __builtin_fmaf(wv, Act<F16>::lo(pw[i]), acc[2 * i]);
+            acc[2 * i + 1] = __builtin_fmaf(wv, Act<F16>::hi(pw[i]), acc[2 * i + 1]);
         }
     }
     uint4 o;
-    o.x = pack_bf16x2(acc[0], acc[1]);
-    o.y = pack_bf16x2(acc[2], acc[3]);
-    o.z = pack_bf16x2(acc[4], acc[5]);
-    o.w = pack_bf16x2(acc[6], acc[7]);
+    o.x = Act<F16>::pack(acc[0], acc[1]);
+    o.y = Act<F16>::pack(acc[2], acc[3]);
+    o.z = Act<F16>::pack(acc[4], acc[5]);
+    o.w = Act<F16>::pack(acc[6], acc[7]);
     *reinterpret_cast<uint4 *>(y + (size_t)tok * d + c) = o;
+}
+
+// FP16 rows -> bf16 rows (round to nearest even), 8 elements per thread: a context in FP16 mode feeds the
+// gate/up GEMM, whose tiles are bf16, through this pass.
+__global__ __launch_bounds__(256) void rows_f16_to_bf16_kernel(const uint16_t *__restrict__ x, uint32_t x_stride, uint32_t d,
+                                                               uint16_t *__restrict__ out) {
+    const uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (c >= d) return;
+    const uint4 q = *reinterpret_cast<const uint4 *>(x + (size_t)blockIdx.y * x_stride + c);
+    uint4 o;
+    o.x = pack_bf16x2(Act<true>::lo(q.x), Act<true>::hi(q.x));
+    o.y = pack_bf16x2(Act<true>::lo(q.y), Act<true>::hi(q.y));
+    o.z = pack_bf16x2(Act<true>::lo(q.z), Act<true>::hi(q.z));
+    o.w = pack_bf16x2(Act<true>::lo(q.w), Act<true>::hi(q.w));
+    *reinterpret_cast<uint4 *>(out + (size_t)blockIdx.y * d + c) = o;
 }
 
 }  // namespace
@@ -466,7 +483,7 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(const uint16_t *__
 hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
                           const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
                           const ffmoe_pair *pairs, uint32_t n_pairs_in, uint16_t *y, uint16_t *partials_out,
-                          PrefillScratch sc, KernelTimer *timer) {
+                          PrefillScratch sc, KernelTimer *timer, bool f16) {
     timer->begin(s);
     ItemSource src{};
     src.idx = pairs ? nullptr : idx;
@@ -491,18 +508,33 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
     const uint32_t tile_cap = min(sc.max_tiles, (src.n_items + kBM - 1) / kBM + n_experts);
     const uint32_t tile_slots = (tile_cap + 7) / 8 * 8;
     const uint32_t nb_gu = (g.gu_rb + kTilesPerBlock - 1) / kTilesPerBlock, nb_dn = (g.dn_rbp + kTilesPerBlock - 1) / kTilesPerBlock;
+    if (f16) {
+        // the GEMMs compute on bf16 tiles: FP16 inputs are rounded to bf16 once, outputs leave as FP16
+        if (!sc.x16) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(rows_f16_to_bf16_kernel, dim3((g.d / 8 + 255) / 256, t), dim3(256), 0, s, x, x_stride, g.d, sc.x16);
+        x = sc.x16;
+        x_stride = g.d;
+    }
     hipLaunchKernelGGL(prefill_gemm_kernel<true>, dim3(nb_gu * tile_slots), dim3(256), 0, s, arena_layer, g, sc.plan,
                        sc.tiles, sc.sorted_token, sc.sorted_out_row, x, x_stride, sc.acts, nb_gu);
     timer->mark(s, FFMOE_K_PREFILL_GATE_UP);
     uint16_t *partials = partials_out ? partials_out : sc.partials;
-    hipLaunchKernelGGL(prefill_gemm_kernel<false>, dim3(nb_dn * tile_slots), dim3(256), 0, s, arena_layer, g, sc.plan,
-                       sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn);
+    if (f16)
+        hipLaunchKernelGGL((prefill_gemm_kernel<false, true>), dim3(nb_dn * tile_slots), dim3(256), 0, s, arena_layer, g, sc.plan,
+                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn);
+    else
+        hipLaunchKernelGGL((prefill_gemm_kernel<false, false>), dim3(nb_dn * tile_slots), dim3(256), 0, s, arena_layer, g, sc.plan,
+                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_PREFILL_DOWN);
     if (y) {
-        hipLaunchKernelGGL(prefill_combine_kernel, dim3((g.d / 8 + 255) / 256, t), dim3(256), 0, s, partials, w, idx,
-                           n_experts, top_k, g.d, y);
+        if (f16)
+            hipLaunchKernelGGL(prefill_combine_kernel<true>, dim3((g.d / 8 + 255) / 256, t), dim3(256), 0, s, partials, w, idx,
+                               n_experts, top_k, g.d, y);
+        else
+            hipLaunchKernelGGL(prefill_combine_kernel<false>, dim3((g.d / 8 + 255) / 256, t), dim3(256), 0, s, partials, w, idx,
+                               n_experts, top_k, g.d, y);
         timer->mark(s, FFMOE_K_PREFILL_COMBINE);
     }
     timer->finish();

@@ -44,7 +44,8 @@ __device__ __forceinline__ uint2 load_x4(const uint16_t *p) {
 
 // Per-lane accumulation shared by both logits kernels: sub-accumulator `s` of lane `lane` over the
 // elements k = 1024 i + 256 s + 4 lane + j, i ascending then j, for kChunkTokens token rows at once.
-template <bool W_F32, bool X_ALIGNED>
+// XK: how the input rows arrive - 0: bf16, rows 2-byte aligned only; 1: bf16, 8-byte aligned; 2: FP16, 8-byte aligned.
+template <bool W_F32, int XK>
 __device__ __forceinline__ void accumulate_sub(const void *__restrict__ w_, const uint16_t *__restrict__ es,
                                                const uint16_t *__restrict__ x, uint32_t x_stride, uint32_t e,
                                                uint32_t d, uint32_t s, uint32_t lane, uint32_t t0, uint32_t t_last,
@@ -65,11 +66,11 @@ __device__ __forceinline__ void accumulate_sub(const void *__restrict__ w_, cons
             for (int r = 0; r < kChunkTokens; ++r) {
                 // rows past the last token re-read it: same arithmetic, result unused
                 const uint32_t row = min(t0 + r, t_last);
-                const uint2 xv = load_x4<X_ALIGNED>(x + (size_t)row * x_stride + k);
-                const float xf[4] = {bf16lo_to_f32(xv.x), bf16hi_to_f32(xv.x), bf16lo_to_f32(xv.y), bf16hi_to_f32(xv.y)};
+                const uint2 xv = load_x4<XK != 0>(x + (size_t)row * x_stride + k);
+                const float xf[4] = {Act<XK == 2>::lo(xv.x), Act<XK == 2>::hi(xv.x), Act<XK == 2>::lo(xv.y), Act<XK == 2>::hi(xv.y)};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    // x * effective_scale: product of two bf16 values, exact in fp32 (moe.metal:96-97)
+                    // x * effective_scale: 8 or 11 significant bits times 8, exact in fp32 (moe.metal:96-97)
                     const float xe = es ? xf[j] * sc[j] : xf[j];
                     acc[r] = __builtin_fmaf(wv[j], xe, acc[r]);
                 }
@@ -82,7 +83,7 @@ __device__ __forceinline__ void accumulate_sub(const void *__restrict__ w_, cons
 // four sub-accumulators of one expert row for four tokens; wave 0 combines them. (A variant whose last
 // block also selected the top-k behind a device-scope counter measured 2.5x slower: every block paid
 // for the same-address atomic and the L2 write-back of its release fence.)
-template <bool W_F32, bool X_ALIGNED>
+template <bool W_F32, int XK>
 __global__ __launch_bounds__(256) void router_small_kernel(const void *__restrict__ w_, const uint16_t *__restrict__ es,
                                                            const uint16_t *__restrict__ x, uint32_t x_stride,
                                                            uint32_t t, uint32_t n_experts, uint32_t d,
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(256) void router_small_kernel(const void *__restric
     const uint32_t t0 = blockIdx.y * kChunkTokens;
     const uint32_t t_end = min(t, t0 + kChunkTokens);
     float acc[kChunkTokens] = {0.f, 0.f, 0.f, 0.f};
-    accumulate_sub<W_F32, X_ALIGNED>(w_, es, x, x_stride, e, d, s, lane, t0, t_end - 1, acc);
+    accumulate_sub<W_F32, XK>(w_, es, x, x_stride, e, d, s, lane, t0, t_end - 1, acc);
 #pragma unroll
     for (int r = 0; r < kChunkTokens; ++r) s_part[s][r][lane] = acc[r];
     __syncthreads();
@@ -119,7 +120,7 @@ constexpr int kTileTok = 8, kTileExp = 8;
 template <bool W_F32> struct WRaw { uint2 v; };
 template <> struct WRaw<true> { f32x4 v; };
 
-template <bool W_F32, bool X_ALIGNED, bool HAS_ES>
+template <bool W_F32, int XK, bool HAS_ES>
 __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict__ w_, const uint16_t *__restrict__ es,
                                                           const uint16_t *__restrict__ x, uint32_t x_stride,
                                                           uint32_t t, uint32_t n_experts, uint32_t d,
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict
             else wn[c].v = *reinterpret_cast<const decltype(wn[c].v) *>(reinterpret_cast<const uint16_t *>(w_) + wrow[c] + k);
         }
 #pragma unroll
-        for (int r = 0; r < kTileTok; ++r) xn[r] = load_x4<X_ALIGNED>(xrow[r] + k);
+        for (int r = 0; r < kTileTok; ++r) xn[r] = load_x4<XK != 0>(xrow[r] + k);
         if (HAS_ES) en = *reinterpret_cast<const uint2 *>(es + k);
     };
 
@@ -182,11 +183,11 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict
         if (live) {
 #pragma unroll
             for (int r = 0; r < kTileTok; ++r) {
-                const float xf[4] = {bf16lo_to_f32(xc[r].x), bf16hi_to_f32(xc[r].x), bf16lo_to_f32(xc[r].y),
-                                     bf16hi_to_f32(xc[r].y)};
+                const float xf[4] = {Act<XK == 2>::lo(xc[r].x), Act<XK == 2>::hi(xc[r].x), Act<XK == 2>::lo(xc[r].y),
+                                     Act<XK == 2>::hi(xc[r].y)};
                 float xe[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) xe[j] = HAS_ES ? xf[j] * sc[j] : xf[j];   // exact: product of two bf16
+                for (int j = 0; j < 4; ++j) xe[j] = HAS_ES ? xf[j] * sc[j] : xf[j];   // exact: at most 11 + 8 significant bits
 #pragma unroll
                 for (int c = 0; c < kTileExp; ++c)
 #pragma unroll
@@ -249,31 +250,32 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const void *__restrict
 
 __global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, const uint16_t *__restrict__ per_expert_scale,
                                                          uint32_t n_experts, uint32_t top_k,
-                                                         uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w) {
+                                                         uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w, bool w_f16) {
     const uint32_t tok = blockIdx.x;
     wave_topk(logits + (size_t)tok * n_experts, per_expert_scale, n_experts, top_k, out_idx + (size_t)tok * top_k,
-              out_w + (size_t)tok * top_k, threadIdx.x);
+              out_w + (size_t)tok * top_k, threadIdx.x, w_f16);
 }
 
 }  // namespace
 
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer) {
+                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer, bool f16) {
     (void)counters;
     timer->begin(s);
     const bool x_aligned = (reinterpret_cast<uintptr_t>(x) % 8 == 0) && (x_stride % 4 == 0);
+    if (f16 && !x_aligned) return hipErrorInvalidValue;     // FP16 rows come 8-byte aligned (checked at the boundary)
     if (t <= FFMOE_MAX_VERIFY_ROWS) {
         const dim3 grid(n_experts, (t + kChunkTokens - 1) / kChunkTokens);
 #define FFMOE_ROUTER(WF, XA)                                                                                 \
     hipLaunchKernelGGL((router_small_kernel<WF, XA>), grid, dim3(256), 0, s, rw.w, rw.effective_scale, x,   \
                        x_stride, t, n_experts, d, logits)
-        if (rw.w_is_f32) { if (x_aligned) FFMOE_ROUTER(true, true); else FFMOE_ROUTER(true, false); }
-        else { if (x_aligned) FFMOE_ROUTER(false, true); else FFMOE_ROUTER(false, false); }
+        if (rw.w_is_f32) { if (f16) FFMOE_ROUTER(true, 2); else if (x_aligned) FFMOE_ROUTER(true, 1); else FFMOE_ROUTER(true, 0); }
+        else { if (f16) FFMOE_ROUTER(false, 2); else if (x_aligned) FFMOE_ROUTER(false, 1); else FFMOE_ROUTER(false, 0); }
 #undef FFMOE_ROUTER
         timer->mark(s, FFMOE_K_ROUTER_LOGITS);
         hipLaunchKernelGGL(router_topk_kernel, dim3(t), dim3(64), 0, s, logits, rw.per_expert_scale, n_experts, top_k, out_idx,
-                           out_w);
+                           out_w, f16);
         timer->mark(s, FFMOE_K_ROUTER_TOPK);
         timer->finish();
         return hipGetLastError();
@@ -289,14 +291,14 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
             hipLaunchKernelGGL((router_tile_kernel<WF, XA, false>), grid, dim3(256), 0, s, rw.w,             \
                                rw.effective_scale, x, x_stride, t, n_experts, d, n_egroups, n_tgroups, logits); \
     } while (0)
-    if (rw.w_is_f32) { if (x_aligned) FFMOE_ROUTER(true, true); else FFMOE_ROUTER(true, false); }
-    else { if (x_aligned) FFMOE_ROUTER(false, true); else FFMOE_ROUTER(false, false); }
+    if (rw.w_is_f32) { if (f16) FFMOE_ROUTER(true, 2); else if (x_aligned) FFMOE_ROUTER(true, 1); else FFMOE_ROUTER(true, 0); }
+    else { if (f16) FFMOE_ROUTER(false, 2); else if (x_aligned) FFMOE_ROUTER(false, 1); else FFMOE_ROUTER(false, 0); }
 #undef FFMOE_ROUTER
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_ROUTER_LOGITS);
     hipLaunchKernelGGL(router_topk_kernel, dim3(t), dim3(64), 0, s, logits, rw.per_expert_scale, n_experts, top_k,
-                       out_idx, out_w);
+                       out_idx, out_w, f16);
     timer->mark(s, FFMOE_K_ROUTER_TOPK);
     timer->finish();
     return hipGetLastError();

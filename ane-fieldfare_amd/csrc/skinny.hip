@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256) void verify_plan_kernel(const uint32_t *__rest
 // the token operand it supplies token slot l % 16 (`xrow` = that token's row, already offset by
 // 8 * (l / 16) elements); it ends up holding token slots 4 * (l / 16) + 0..3.
 // ---------------------------------------------------------------------------------------------------
-template <int PD>
+template <int PD, bool F16>
 __device__ __forceinline__ TwoStreamAcc stream_tiles(const uint8_t *__restrict__ tiles,
                                                      const uint8_t *__restrict__ scales,
                                                      const uint16_t *__restrict__ xrow, uint32_t g0, uint32_t g1,
@@ -134,8 +134,7 @@ __device__ __forceinline__ TwoStreamAcc stream_tiles(const uint8_t *__restrict__
     tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
     tot.b = f32x4{0.f, 0.f, 0.f, 0.f};
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-    const uint4 ones_bits = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-    const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
+    const uint4 ones = {Act<F16>::kOnesBits, Act<F16>::kOnesBits, Act<F16>::kOnesBits, Act<F16>::kOnesBits};
     uint4 tbuf[PD], xb0[PD], xb1[PD];
     uint2 sbuf[PD];
 #pragma unroll
@@ -164,16 +163,15 @@ __device__ __forceinline__ TwoStreamAcc stream_tiles(const uint8_t *__restrict__
                     xb0[u] = *reinterpret_cast<const uint4 *>(xrow + (g + PD) * kGroup);
                     xb1[u] = *reinterpret_cast<const uint4 *>(xrow + (g + PD) * kGroup + 32);
                 }
-                const bf16x8 a0 = __builtin_bit_cast(bf16x8, x0), a1 = __builtin_bit_cast(bf16x8, x1);
-                f32x4 acc_a = mfma16(a0, unpack8_offset128(tile.x), zero);
-                acc_a = mfma16(a1, unpack8_offset128(tile.y), acc_a);
-                f32x4 acc_b = mfma16(a0, unpack8_offset128(tile.z), zero);
-                acc_b = mfma16(a1, unpack8_offset128(tile.w), acc_b);
-                f32x4 sx = mfma16(a0, ones, zero);
-                sx = mfma16(a1, ones, sx);
+                f32x4 acc_a = Act<F16>::mfma(x0, unpack8_offset<F16>(tile.x), zero);
+                acc_a = Act<F16>::mfma(x1, unpack8_offset<F16>(tile.y), acc_a);
+                f32x4 acc_b = Act<F16>::mfma(x0, unpack8_offset<F16>(tile.z), zero);
+                acc_b = Act<F16>::mfma(x1, unpack8_offset<F16>(tile.w), acc_b);
+                f32x4 sx = Act<F16>::mfma(x0, ones, zero);
+                sx = Act<F16>::mfma(x1, ones, sx);
                 const float sa = bf16lo_to_f32(sc.x), ba = bf16hi_to_f32(sc.x);
                 const float sb = bf16lo_to_f32(sc.y), bb = bf16hi_to_f32(sc.y);
-                const float ta = __builtin_fmaf(-128.0f, sa, ba), tb = __builtin_fmaf(-128.0f, sb, bb);
+                const float ta = __builtin_fmaf(-Act<F16>::kOffset, sa, ba), tb = __builtin_fmaf(-Act<F16>::kOffset, sb, bb);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     tot.a[r] = __builtin_fmaf(sa, acc_a[r], tot.a[r]);
@@ -189,6 +187,7 @@ __device__ __forceinline__ TwoStreamAcc stream_tiles(const uint8_t *__restrict__
 
 // gate/up + GELU-tanh gating. grid = (F / 16, live-slot capacity); the four waves of a block share one
 // row block and split K four ways; their partial sums meet in LDS and are added in wave order.
+template <bool F16>
 __global__ __launch_bounds__(256) void skinny_gate_up_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                              uint32_t top_k, const VerifyPlan *__restrict__ plan,
                                                              const uint16_t *__restrict__ x, uint32_t x_stride,
@@ -210,7 +209,7 @@ __global__ __launch_bounds__(256) void skinny_gate_up_kernel(const uint8_t *__re
     tot.b = tot.a;
     if (g0 < g1) {
         const uint32_t tok = slot.routes[min(j, n - 1)] / top_k;
-        tot = stream_tiles<kRing>(tiles, scales, x + (size_t)tok * x_stride + 8 * jq, g0, g1, lane);
+        tot = stream_tiles<kRing, F16>(tiles, scales, x + (size_t)tok * x_stride + 8 * jq, g0, g1, lane);
     }
     if (ks != 0) {
 #pragma unroll
@@ -234,14 +233,14 @@ __global__ __launch_bounds__(256) void skinny_gate_up_kernel(const uint8_t *__re
     for (int r = 0; r < 4; ++r) {
         const uint32_t ts = 4 * jq + r;
         // one rounding to 16 bits, gate and up themselves stay fp32 (moe.metal:496)
-        if (ts < n) acts[(size_t)slot.routes[ts] * g.f + row] = f32_to_bf16(gelu_tanh_fast(tot.a[r]) * tot.b[r]);
+        if (ts < n) acts[(size_t)slot.routes[ts] * g.f + row] = Act<F16>::round(gelu_tanh_fast(tot.a[r]) * tot.b[r]);
     }
 }
 
 // down projection. grid = (ceil(D/32 / 4), live-slot capacity); each wave owns one pair of 16-row blocks,
 // the whole K = F, and all (<= 16) routes of the expert.
 // Output: un-weighted rows, fp32 into `partials_f32` (fused combine) or bf16 into `partials_bf16`.
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool F16>
 __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                           const VerifyPlan *__restrict__ plan,
                                                           const uint16_t *__restrict__ acts,
@@ -258,7 +257,7 @@ __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restr
     const uint8_t *tiles = expert_base + g.dn_tiles_off + (size_t)rbp * g.gf * kTileBytes;
     const uint8_t *scales = expert_base + g.dn_scales_off + (size_t)rbp * g.gf * kTileScaleBytes;
     const uint16_t *arow = acts + (size_t)slot.routes[min(j, n - 1)] * g.f + 8 * jq;
-    const TwoStreamAcc tot = stream_tiles<kRing>(tiles, scales, arow, 0, g.gf, lane);
+    const TwoStreamAcc tot = stream_tiles<kRing, F16>(tiles, scales, arow, 0, g.gf, lane);
     const uint32_t row_a = rbp * 2 * kTileRows + j, row_b = row_a + kTileRows;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -266,8 +265,8 @@ __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restr
         if (ts < n) {
             const size_t base = (size_t)slot.routes[ts] * g.d;
             if (OUT_BF16) {
-                partials_bf16[base + row_a] = f32_to_bf16(tot.a[r]);
-                partials_bf16[base + row_b] = f32_to_bf16(tot.b[r]);
+                partials_bf16[base + row_a] = Act<F16>::round(tot.a[r]);
+                partials_bf16[base + row_b] = Act<F16>::round(tot.b[r]);
             } else {
                 partials_f32[base + row_a] = tot.a[r];
                 partials_f32[base + row_b] = tot.b[r];
@@ -287,6 +286,7 @@ __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restr
 // gate/up + GELU-tanh gating, persistent. grid = (blocks); the blocks are dealt to the live experts, each
 // block walks a range of 16-row blocks of its expert; its four waves split K and meet in LDS per row block
 // (partials added in wave order), each wave finishing a quarter of the token slots.
+template <bool F16>
 __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                                     uint32_t top_k, uint32_t n_experts,
                                                                     const uint32_t *__restrict__ idx,
@@ -366,7 +366,7 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, gu_src, next_row + min(g0 + u, g_last), lane);
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, gu_src, next_row + min(g0 + u, g_last), lane);
         const int buf = (rb - rb0) & 1;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -381,7 +381,7 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
             ub += s_red[buf][o][4 + ks][lane];
         }
         // one rounding to 16 bits, gate and up themselves stay fp32 (moe.metal:496)
-        const uint16_t v = f32_to_bf16(gelu_tanh_fast(ga) * ub);
+        const uint16_t v = Act<F16>::round(gelu_tanh_fast(ga) * ub);
         for (uint32_t todo = stores; todo; todo &= todo - 1)
             out_col[(size_t)__builtin_ctz(todo) * g.f + rb * kTileRows] = v;
     }
@@ -390,7 +390,7 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
 // down projection, persistent: the waves of the grid are dealt to the live experts; a wave keeps the
 // expert's (<= 16) activation rows in registers (all of K = F: at most kRing groups) and walks a range of
 // 32-row tile rows with the weight ring refilled across them. No K-split, so no LDS and no barrier.
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool F16>
 __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                                  const VerifyPlan *__restrict__ plan,
                                                                  const uint16_t *__restrict__ acts,
@@ -448,7 +448,7 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min((uint32_t)u, g_last), lane);
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min((uint32_t)u, g_last), lane);
         // The sums take a detour through a wave-private LDS slot. It costs sixteen LDS operations per tile
         // row and changes nothing arithmetically, but it is what keeps the register allocation of this loop
         // sane: with the sums used directly the compiler keeps every group's matrix results alive to the end
@@ -464,8 +464,8 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
             const float va = s_tmp[wave][r][lane], vb = s_tmp[wave][4 + r][lane];
             if (4 * jq + r < n) {
                 if (OUT_BF16) {
-                    partials_bf16[(size_t)out_base[r] + row_a] = f32_to_bf16(va);
-                    partials_bf16[(size_t)out_base[r] + row_b] = f32_to_bf16(vb);
+                    partials_bf16[(size_t)out_base[r] + row_a] = Act<F16>::round(va);
+                    partials_bf16[(size_t)out_base[r] + row_b] = Act<F16>::round(vb);
                 } else {
                     partials_f32[(size_t)out_base[r] + row_a] = va;
                     partials_f32[(size_t)out_base[r] + row_b] = vb;
@@ -479,7 +479,7 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
 // grid are dealt to the live experts and the four waves of a block split K as in the gate/up kernel, each
 // with its slice of the activation rows in registers; the partial sums meet in LDS and wave ks finishes
 // token slots 4 * (lane / 16) + ks.
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool F16>
 __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                                         const VerifyPlan *__restrict__ plan,
                                                                         const uint16_t *__restrict__ acts,
@@ -528,7 +528,7 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min(g0 + u, g_last), lane);
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min(g0 + u, g_last), lane);
         const int buf = (rb - rb0) & 1;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -545,8 +545,8 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
         const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
         if (my_ts < n) {
             if (OUT_BF16) {
-                partials_bf16[out_base + row_a] = f32_to_bf16(va);
-                partials_bf16[out_base + row_b] = f32_to_bf16(vb);
+                partials_bf16[out_base + row_a] = Act<F16>::round(va);
+                partials_bf16[out_base + row_b] = Act<F16>::round(vb);
             } else {
                 partials_f32[out_base + row_a] = va;
                 partials_f32[out_base + row_b] = vb;
@@ -558,6 +558,7 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
 // y[t][c] = bf16(residual + sum_r w[t][r] * partial[t*k + r][c]) in rank order with fmaf, fp32 partials,
 // one rounding at the end (the decode form, moe.metal:627-636). Routes the plan skips (zero weight or
 // expert out of range) add nothing.
+template <bool F16>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ partials,
                                                       const uint16_t *__restrict__ w,
                                                       const uint32_t *__restrict__ idx, uint32_t n_experts,
@@ -569,25 +570,26 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (residual) {
         const uint2 rv = *reinterpret_cast<const uint2 *>(residual + (size_t)tok * d + c);
-        acc[0] = bf16lo_to_f32(rv.x); acc[1] = bf16hi_to_f32(rv.x);
-        acc[2] = bf16lo_to_f32(rv.y); acc[3] = bf16hi_to_f32(rv.y);
+        acc[0] = Act<F16>::lo(rv.x); acc[1] = Act<F16>::hi(rv.x);
+        acc[2] = Act<F16>::lo(rv.y); acc[3] = Act<F16>::hi(rv.y);
     }
     for (uint32_t r = 0; r < top_k; ++r) {
         const uint32_t route = tok * top_k + r;
         const uint16_t wb = w[route];
         if ((wb & 0x7FFFu) == 0 || idx[route] >= n_experts) continue;
-        const float wv = bf16_to_f32(wb);
+        const float wv = Act<F16>::widen(wb);
         const f32x4 p = *reinterpret_cast<const f32x4 *>(partials + (size_t)route * d + c);
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] = __builtin_fmaf(wv, p[i], acc[i]);
     }
     uint2 o;
-    o.x = pack_bf16x2(acc[0], acc[1]);
-    o.y = pack_bf16x2(acc[2], acc[3]);
+    o.x = Act<F16>::pack(acc[0], acc[1]);
+    o.y = Act<F16>::pack(acc[2], acc[3]);
     *reinterpret_cast<uint2 *>(y + (size_t)tok * d + c) = o;
 }
 
 // prefill_moe_reduce_token_major (prefill.metal:544-565) on 16-bit partials.
+template <bool F16>
 __global__ __launch_bounds__(256) void reduce_token_major_kernel(const uint16_t *__restrict__ partials,
                                                                  const uint16_t *__restrict__ w, uint32_t top_k,
                                                                  uint32_t d, uint16_t *__restrict__ h2) {
@@ -597,17 +599,20 @@ __global__ __launch_bounds__(256) void reduce_token_major_kernel(const uint16_t 
     float acc = 0.0f;
     for (uint32_t r = 0; r < top_k; ++r) {
         const size_t route = (size_t)tok * top_k + r;
-        acc = __builtin_fmaf(bf16_to_f32(w[route]), bf16_to_f32(partials[route * d + c]), acc);
+        acc = __builtin_fmaf(Act<F16>::widen(w[route]), Act<F16>::widen(partials[route * d + c]), acc);
     }
-    h2[(size_t)tok * d + c] = f32_to_bf16(acc);
+    h2[(size_t)tok * d + c] = Act<F16>::round(acc);
 }
 
 }  // namespace
 
-hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
-                         uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
-                         const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
-                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer) {
+namespace {
+
+template <bool F16>
+hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
+                            const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
+                            const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16, VerifyPlan *plan, uint16_t *acts,
+                            float *partials_f32, uint32_t n_cus, KernelTimer *timer) {
     timer->begin(s);
     const uint32_t slots = min(n_experts, t * top_k);
     // the persistent kernels hold a K-slice of kRing groups per wave; larger experts take the one-shot grids
@@ -618,12 +623,12 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
     if (gu_persistent) {
         // plan slot of the profile stays empty: the gate/up kernel builds the plan itself
         const uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
-        hipLaunchKernelGGL(skinny_gate_up_persistent, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, idx, w,
-                           t * top_k, plan, x, x_stride, acts);
+        hipLaunchKernelGGL(skinny_gate_up_persistent<F16>, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, idx,
+                           w, t * top_k, plan, x, x_stride, acts);
     } else {
         hipLaunchKernelGGL(verify_plan_kernel, dim3(1), dim3(256), 0, s, idx, w, t * top_k, n_experts, plan);
         timer->mark(s, FFMOE_K_PLAN);
-        hipLaunchKernelGGL(skinny_gate_up_kernel, dim3(g.gu_rb, slots), dim3(256), 0, s, arena_layer, g, top_k, plan, x,
+        hipLaunchKernelGGL(skinny_gate_up_kernel<F16>, dim3(g.gu_rb, slots), dim3(256), 0, s, arena_layer, g, top_k, plan, x,
                            x_stride, acts);
     }
     hipError_t e = hipGetLastError();
@@ -632,15 +637,15 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
     const dim3 dn_grid = dn_whole    ? dim3(max((slots + 3) / 4, min(n_cus, (slots * g.dn_rbp + 3) / 4)))
                          : dn_ksplit ? dim3(max(slots, min(resident, slots * g.dn_rbp)))
                                      : dim3((g.dn_rbp + 3) / 4, slots);
-#define FFMOE_DOWN(BF)                                                                                            \
-    if (dn_whole)                                                                                                 \
-        hipLaunchKernelGGL(skinny_down_persistent<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,      \
-                           partials_f32, partials_bf16);                                                          \
-    else if (dn_ksplit)                                                                                           \
-        hipLaunchKernelGGL(skinny_down_ksplit_persistent<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan,     \
-                           acts, partials_f32, partials_bf16);                                                    \
-    else                                                                                                          \
-        hipLaunchKernelGGL(skinny_down_kernel<BF>, dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,          \
+#define FFMOE_DOWN(BF)                                                                                                \
+    if (dn_whole)                                                                                                     \
+        hipLaunchKernelGGL((skinny_down_persistent<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,   \
+                           partials_f32, partials_bf16);                                                              \
+    else if (dn_ksplit)                                                                                               \
+        hipLaunchKernelGGL((skinny_down_ksplit_persistent<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan,  \
+                           acts, partials_f32, partials_bf16);                                                        \
+    else                                                                                                              \
+        hipLaunchKernelGGL((skinny_down_kernel<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,       \
                            partials_f32, partials_bf16)
     if (partials_bf16) {
         FFMOE_DOWN(true);
@@ -653,17 +658,34 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_DOWN);
-    hipLaunchKernelGGL(combine_kernel, dim3((g.d / 4 + 255) / 256, t), dim3(256), 0, s, partials_f32, w, idx, n_experts,
+    hipLaunchKernelGGL(combine_kernel<F16>, dim3((g.d / 4 + 255) / 256, t), dim3(256), 0, s, partials_f32, w, idx, n_experts,
                        residual, top_k, g.d, y);
     timer->mark(s, FFMOE_K_COMBINE);
     timer->finish();
     return hipGetLastError();
 }
 
+}  // namespace
+
+// x, w, residual, y and the 16-bit partial rows are FP16 when `f16`, bf16 otherwise
+hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
+                         uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
+                         const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
+                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer, bool f16) {
+    return f16 ? launch_verify_as<true>(s, arena_layer, g, n_experts, top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
+                                        plan, acts, partials_f32, n_cus, timer)
+               : launch_verify_as<false>(s, arena_layer, g, n_experts, top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
+                                         plan, acts, partials_f32, n_cus, timer);
+}
+
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,
-                                     uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d) {
-    hipLaunchKernelGGL(reduce_token_major_kernel, dim3((d + 255) / 256, t), dim3(256), 0, s, partials, weights,
-                       top_k, d, h2);
+                                     uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d, bool f16) {
+    if (f16)
+        hipLaunchKernelGGL(reduce_token_major_kernel<true>, dim3((d + 255) / 256, t), dim3(256), 0, s, partials, weights, top_k,
+                           d, h2);
+    else
+        hipLaunchKernelGGL(reduce_token_major_kernel<false>, dim3((d + 255) / 256, t), dim3(256), 0, s, partials, weights, top_k,
+                           d, h2);
     return hipGetLastError();
 }
 

@@ -52,26 +52,25 @@ __device__ __forceinline__ void ring_fill(WeightRing &ring, int u, const TileSou
 }
 
 // Consume ring slot u against the resident token operand, then start the load that refills the slot.
+template <bool F16 = false>
 __device__ __forceinline__ void ring_step(WeightRing &ring, int u, bool live, const uint4 &x0, const uint4 &x1,
                                           TwoStreamAcc &tot, const TileSource &src, uint32_t next_tile_index,
                                           uint32_t lane) {
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-    const uint4 ones_bits = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-    const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
+    const uint4 ones = {Act<F16>::kOnesBits, Act<F16>::kOnesBits, Act<F16>::kOnesBits, Act<F16>::kOnesBits};
     const uint4 tile = ring.t[u];
     uint2 sc = ring.s[u];
     if (!live) sc = make_uint2(0u, 0u);
     ring_fill(ring, u, src, next_tile_index, lane);
-    const bf16x8 a0 = __builtin_bit_cast(bf16x8, x0), a1 = __builtin_bit_cast(bf16x8, x1);
-    f32x4 acc_a = mfma16(a0, unpack8_offset128(tile.x), zero);
-    acc_a = mfma16(a1, unpack8_offset128(tile.y), acc_a);
-    f32x4 acc_b = mfma16(a0, unpack8_offset128(tile.z), zero);
-    acc_b = mfma16(a1, unpack8_offset128(tile.w), acc_b);
-    f32x4 sx = mfma16(a0, ones, zero);
-    sx = mfma16(a1, ones, sx);
+    f32x4 acc_a = Act<F16>::mfma(x0, unpack8_offset<F16>(tile.x), zero);
+    acc_a = Act<F16>::mfma(x1, unpack8_offset<F16>(tile.y), acc_a);
+    f32x4 acc_b = Act<F16>::mfma(x0, unpack8_offset<F16>(tile.z), zero);
+    acc_b = Act<F16>::mfma(x1, unpack8_offset<F16>(tile.w), acc_b);
+    f32x4 sx = Act<F16>::mfma(x0, ones, zero);
+    sx = Act<F16>::mfma(x1, ones, sx);
     const float sa = bf16lo_to_f32(sc.x), ba = bf16hi_to_f32(sc.x);
     const float sb = bf16lo_to_f32(sc.y), bb = bf16hi_to_f32(sc.y);
-    const float ta = __builtin_fmaf(-128.0f, sa, ba), tb = __builtin_fmaf(-128.0f, sb, bb);
+    const float ta = __builtin_fmaf(-Act<F16>::kOffset, sa, ba), tb = __builtin_fmaf(-Act<F16>::kOffset, sb, bb);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         tot.a[r] = __builtin_fmaf(sa, acc_a[r], tot.a[r]);

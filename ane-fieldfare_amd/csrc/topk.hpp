@@ -91,21 +91,23 @@ __device__ __forceinline__ void topk_select(TopkRow &t, uint32_t top_k, uint32_t
 }
 
 __device__ __forceinline__ void topk_store(const TopkRow &t, const uint16_t *__restrict__ per_expert_scale, uint32_t top_k,
-                                           uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w, uint32_t lane) {
+                                           uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w, uint32_t lane,
+                                           bool w_f16) {
     if (lane < top_k) {
         const float gain = per_expert_scale ? bf16_to_f32(per_expert_scale[t.idx]) : 1.0f;
+        const float weight = t.ex / t.sum * gain;
         out_idx[lane] = t.idx;
-        out_w[lane] = f32_to_bf16(t.ex / t.sum * gain);
+        out_w[lane] = w_f16 ? Act<true>::round(weight) : Act<false>::round(weight);
     }
 }
 
 __device__ __forceinline__ void wave_topk(const float *row, const uint16_t *__restrict__ per_expert_scale,
                                           uint32_t n_experts, uint32_t top_k, uint32_t *__restrict__ out_idx,
-                                          uint16_t *__restrict__ out_w, uint32_t lane) {
+                                          uint16_t *__restrict__ out_w, uint32_t lane, bool w_f16) {
     TopkRow t;
     topk_load(t, row, n_experts, lane);
     topk_select(t, top_k, lane);
-    topk_store(t, per_expert_scale, top_k, out_idx, out_w, lane);
+    topk_store(t, per_expert_scale, top_k, out_idx, out_w, lane, w_f16);
 }
 
 }  // namespace

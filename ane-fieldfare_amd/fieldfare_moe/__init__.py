@@ -38,6 +38,8 @@ class Offsets(C.Structure):
                 ("gate_w", "gate_s", "gate_b", "up_w", "up_s", "up_b", "down_w", "down_s", "down_b")]
 
 
+BF16, FP16 = 0, 1     # FFMOE_BF16, FFMOE_FP16
+
 EXPORTS = [
     "ffmoe_version", "ffmoe_create", "ffmoe_destroy", "ffmoe_layer_arena_bytes", "ffmoe_upload_layer",
     "ffmoe_upload_router_bf16", "ffmoe_upload_router_int8", "ffmoe_dequant_expert", "ffmoe_router",
@@ -46,7 +48,7 @@ EXPORTS = [
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
     "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
     "ffmoe_layer_tail", "ffmoe_route_verify", "ffmoe_gemv_int4_listed",
-    "ffmoe_layer_tail_norms", "ffmoe_rmsnorm",
+    "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype",
 ]
 
 PROFILE_SLOTS = 16
@@ -89,7 +91,7 @@ class Matrix:
     def gemv(self, x, f32_out: bool = False):
         import torch
         rows = x.shape[0]
-        y = torch.empty((rows, self.m), dtype=torch.float32 if f32_out else torch.bfloat16, device=x.device)
+        y = torch.empty((rows, self.m), dtype=torch.float32 if f32_out else self.ctx.act, device=x.device)
         err = C.c_char_p()
         _check(self.L.ffmoe_matrix_gemv(self._h, _stream(), _ptr(x), _row_stride(x), rows, _ptr(y), self.m,
                                         int(f32_out), C.byref(err)), err)
@@ -157,6 +159,7 @@ def lib() -> C.CDLL:
     L.ffmoe_gemv_int4.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, i32, errp]
     L.ffmoe_layer_tail_norms.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, vp, vp, vp, vp, u32, u32, u32, C.c_float,
                                          C.c_float, errp]
+    L.ffmoe_set_activation_dtype.argtypes = [vp, C.c_int, errp]
     L.ffmoe_rmsnorm.argtypes = [vp, vp, vp, u32, vp, vp, u32, u32, u32, C.c_float, errp]
     L.ffmoe_gemv_int4_listed.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, errp]
     L.ffmoe_set_profiling.argtypes = [vp, i32, errp]
@@ -203,16 +206,30 @@ class Context:
     """One ffmoe_ctx: the HBM expert arena of `n_layers` layers plus scratch, on one GPU."""
 
     def __init__(self, d: int, f: int, n_experts: int, top_k: int = 8, n_layers: int = 1, max_tokens: int = 4096,
-                 device: int = 0):
+                 device: int = 0, act_dtype: str = "bf16"):
         import torch
         if not torch.cuda.is_available():
             raise RuntimeError("no HIP device visible: the fieldfare MoE kernels have no CPU fallback")
+        if act_dtype not in ("bf16", "fp16"):
+            raise ValueError("act_dtype is 'bf16' or 'fp16'")
         self.L = lib()
         self.shape = Shape(d, f, n_experts, top_k, n_layers, max_tokens)
         self.device = device
+        self.act = torch.bfloat16 if act_dtype == "bf16" else torch.float16    # type of every 16-bit row in and out
         self._h = C.c_void_p()
         err = C.c_char_p()
         _check(self.L.ffmoe_create(device, C.byref(self.shape), C.byref(self._h), C.byref(err)), err)
+        if act_dtype == "fp16":
+            _check(self.L.ffmoe_set_activation_dtype(self._h, FP16, C.byref(err)), err)
+
+    def set_act_dtype(self, act_dtype: str):
+        """Switch the type of every 16-bit row in and out ('bf16' or 'fp16'); waits for the device."""
+        import torch
+        if act_dtype not in ("bf16", "fp16"):
+            raise ValueError("act_dtype is 'bf16' or 'fp16'")
+        err = C.c_char_p()
+        _check(self.L.ffmoe_set_activation_dtype(self._h, FP16 if act_dtype == "fp16" else BF16, C.byref(err)), err)
+        self.act = torch.bfloat16 if act_dtype == "bf16" else torch.float16
 
     def close(self):
         if getattr(self, "_h", None) and self._h.value:
@@ -311,11 +328,11 @@ class Context:
     def router(self, layer: int, router_x, want_logits: bool = False):
         """router_x: bf16 [T, stride>=d] CUDA tensor (rows may be strided). Returns (idx i32 [T,K], w bf16 [T,K][, logits])."""
         import torch
-        assert router_x.dtype == torch.bfloat16 and router_x.is_cuda and router_x.stride(1) == 1
+        assert router_x.dtype == self.act and router_x.is_cuda and router_x.stride(1) == 1
         t = router_x.shape[0]
         k, e = self.shape.top_k, self.shape.n_experts
         idx = torch.empty((t, k), dtype=torch.int32, device=router_x.device)
-        w = torch.empty((t, k), dtype=torch.bfloat16, device=router_x.device)
+        w = torch.empty((t, k), dtype=self.act, device=router_x.device)
         logits = torch.empty((t, e), dtype=torch.float32, device=router_x.device) if want_logits else None
         err = C.c_char_p()
         _check(self.L.ffmoe_router(self._h, _stream(), layer, _ptr(router_x), _row_stride(router_x), t, _ptr(idx), _ptr(w),
@@ -327,7 +344,7 @@ class Context:
         """Decode step (T = 1) or verify block (T <= 16): fused experts + weighted combine. x bf16 [T, stride]."""
         import torch
         t = x.shape[0]
-        y = out if out is not None else torch.empty((t, self.shape.d), dtype=torch.bfloat16, device=x.device)
+        y = out if out is not None else torch.empty((t, self.shape.d), dtype=self.act, device=x.device)
         err = C.c_char_p()
         _check(self.L.ffmoe_verify(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(idx), _ptr(w), _ptr(residual),
                                    _ptr(y), C.byref(err)), err)
@@ -337,9 +354,9 @@ class Context:
         """Router + expert pass of a block of <= 16 rows in one call. Returns (y, idx, w)."""
         import torch
         t, k = x.shape[0], self.shape.top_k
-        y = out if out is not None else torch.empty((t, self.shape.d), dtype=torch.bfloat16, device=x.device)
+        y = out if out is not None else torch.empty((t, self.shape.d), dtype=self.act, device=x.device)
         idx = torch.empty((t, k), dtype=torch.int32, device=x.device)
-        w = torch.empty((t, k), dtype=torch.bfloat16, device=x.device)
+        w = torch.empty((t, k), dtype=self.act, device=x.device)
         err = C.c_char_p()
         _check(self.L.ffmoe_route_verify(self._h, _stream(), layer, _ptr(router_x), _row_stride(router_x), _ptr(x), _row_stride(x),
                                          t, _ptr(residual), _ptr(y), _ptr(idx), _ptr(w), C.byref(err)), err)
@@ -349,7 +366,7 @@ class Context:
         import torch
         t = x.shape[0]
         if partials is None:
-            partials = torch.zeros((t, self.shape.top_k, self.shape.d), dtype=torch.bfloat16, device=x.device)
+            partials = torch.zeros((t, self.shape.top_k, self.shape.d), dtype=self.act, device=x.device)
         err = C.c_char_p()
         _check(self.L.ffmoe_verify_partials(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(idx), _ptr(w),
                                             _ptr(partials), C.byref(err)), err)
@@ -364,7 +381,7 @@ class Context:
     def reduce_token_major(self, partials, weights):
         import torch
         t, k, d = partials.shape
-        h2 = torch.empty((t, d), dtype=torch.bfloat16, device=partials.device)
+        h2 = torch.empty((t, d), dtype=self.act, device=partials.device)
         err = C.c_char_p()
         _check(self.L.ffmoe_reduce_token_major(self._h, _stream(), _ptr(partials), _ptr(weights), _ptr(h2), t, k, d,
                                                C.byref(err)), err)
@@ -374,7 +391,7 @@ class Context:
     def prefill(self, layer: int, x, idx, w, out=None):
         import torch
         t = x.shape[0]
-        y = out if out is not None else torch.empty((t, self.shape.d), dtype=torch.bfloat16, device=x.device)
+        y = out if out is not None else torch.empty((t, self.shape.d), dtype=self.act, device=x.device)
         err = C.c_char_p()
         _check(self.L.ffmoe_prefill(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(idx), _ptr(w), _ptr(y),
                                     C.byref(err)), err)
@@ -384,7 +401,7 @@ class Context:
         """Shared expert: every row of x through expert 0 with weight 1 (context with n_experts = top_k = 1)."""
         import torch
         t = x.shape[0]
-        y = out if out is not None else torch.empty((t, self.shape.d), dtype=torch.bfloat16, device=x.device)
+        y = out if out is not None else torch.empty((t, self.shape.d), dtype=self.act, device=x.device)
         err = C.c_char_p()
         _check(self.L.ffmoe_dense_ffn(self._h, _stream(), layer, _ptr(x), _row_stride(x), t, _ptr(y), C.byref(err)), err)
         return y
@@ -414,7 +431,7 @@ class Context:
         import torch
         t = hidden.shape[0]
         d = d or self.shape.d
-        outs = out if out is not None else tuple(torch.empty((t, d), dtype=torch.bfloat16, device=hidden.device) for _ in range(3))
+        outs = out if out is not None else tuple(torch.empty((t, d), dtype=self.act, device=hidden.device) for _ in range(3))
         err = C.c_char_p()
         _check(self.L.ffmoe_post_attn_setup(self._h, _stream(), _ptr(hidden), _row_stride(hidden), _ptr(attn), _row_stride(attn),
                                             _ptr(outs[0]), _row_stride(outs[0]), _ptr(outs[1]), _row_stride(outs[1]),
@@ -438,7 +455,7 @@ class Context:
         import torch
         t = hidden.shape[0]
         d = d or self.shape.d
-        normed = torch.empty((t, d), dtype=torch.bfloat16, device=hidden.device) if w_next is not None else None
+        normed = torch.empty((t, d), dtype=self.act, device=hidden.device) if w_next is not None else None
         err = C.c_char_p()
         _check(self.L.ffmoe_layer_tail_norms(self._h, _stream(), _ptr(h2), _row_stride(h2), _ptr(h1), _row_stride(h1), _ptr(hidden),
                                              _row_stride(hidden), _ptr(w_postffn1), _ptr(w_postffn2), _ptr(w_postffn), _ptr(w_next),
@@ -449,7 +466,7 @@ class Context:
         import torch
         t = x.shape[0]
         d = d or self.shape.d
-        y = out if out is not None else torch.empty((t, d), dtype=torch.bfloat16, device=x.device)
+        y = out if out is not None else torch.empty((t, d), dtype=self.act, device=x.device)
         err = C.c_char_p()
         _check(self.L.ffmoe_rmsnorm(self._h, _stream(), _ptr(x), _row_stride(x), _ptr(w), _ptr(y), _row_stride(y), t, d, eps,
                                     C.byref(err)), err)
@@ -476,7 +493,7 @@ class Context:
         import torch
         m, n = S.shape[0], S.shape[1] * GROUP
         rows = x.shape[0]
-        y = torch.empty((rows, m), dtype=torch.float32 if f32_out else torch.bfloat16, device=x.device)
+        y = torch.empty((rows, m), dtype=torch.float32 if f32_out else self.act, device=x.device)
         err = C.c_char_p()
         wp = C.c_void_p(W.data_ptr() + w_byte_offset)
         _check(self.L.ffmoe_gemv_int4(self._h, _stream(), wp, _ptr(S), _ptr(B), _ptr(x), _ptr(y), m, n, rows,

@@ -61,6 +61,14 @@ public:
     ffmoe_ctx *raw() const { return ctx_; }
     const ffmoe_shape &shape() const { return shape_; }
 
+    // FFMOE_BF16 (default) or FFMOE_FP16, the reference's text-path type: what every 16-bit row handed to or
+    // returned by the operators below is. Set before the first encode call.
+    void setActivationDtype(int dtype) {
+        char *err = nullptr;
+        if (dtype != FFMOE_BF16 && dtype != FFMOE_FP16) throw std::invalid_argument("activation dtype is FFMOE_BF16 or FFMOE_FP16");
+        check(ffmoe_set_activation_dtype(ctx_, dtype, &err), err);
+    }
+
     void uploadLayer(uint32_t layer, const void *blobs, size_t stride, const ffmoe_offsets &offsets, bool onDevice = false) {
         char *err = nullptr;
         check(ffmoe_upload_layer(ctx_, layer, blobs, stride, &offsets, onDevice ? 1 : 0, &err), err);

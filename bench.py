@@ -74,6 +74,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode (T = 1) leg")
     ap.add_argument("--no-gemv", action="store_true", help="skip the INT4 GEMV legs (config 1 and the LM head)")
+    ap.add_argument("--no-fp16", action="store_true", help="skip the FP16-activation leg (same context switched to FFMOE_FP16)")
     ap.add_argument("--no-shared", action="store_true", help="skip the shared-expert (dense INT4 FFN, width 2112) leg")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy three times: the known-size kernel that "
@@ -307,6 +308,61 @@ def main():
             fn()
         torch.cuda.synchronize()
         return (time.perf_counter() - t0_) / reps
+
+    # The same steps with FP16 rows (the reference's text-path type): the context is switched, run and switched back
+    if not args.no_fp16:
+        ctx.set_act_dtype("fp16")
+        xh = x.to(torch.float16)
+        wh = torch.empty((T, K), dtype=torch.float16, device="cuda")
+        yh = torch.empty((T, D), dtype=torch.float16, device="cuda")
+        pxh, pwh, pyh = (C.c_void_p(t_.data_ptr()) for t_ in (xh, wh, yh))
+
+        def step16(layer, rows):
+            rc = Lib.ffmoe_router(h, stream, layer, pxh, D, rows, pidx, pwh, None, C.byref(err))
+            rc |= Lib.ffmoe_verify(h, stream, layer, pxh, D, rows, pidx, pwh, None, pyh, C.byref(err))
+            if rc:
+                raise RuntimeError(err.value)
+        fp16 = {}
+        for name_, rows in (("verify16_us_per_layer", T), ("decode_us_per_layer", 1)):
+            for i in range(L):
+                step16(i, rows)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(4 * L):
+                step16(i % L, rows)
+            torch.cuda.synchronize()
+            fp16[name_] = round((time.perf_counter() - t0) / (4 * L) * 1e6, 2)
+        if args.prefill_tokens:
+            TPh = args.prefill_tokens
+            xph = torch.from_numpy(rng.normal(0, 1, (TPh, D)).astype(np.float16).view(np.int16)).cuda().view(torch.float16)
+            ih = torch.empty((TPh, K), dtype=torch.int32, device="cuda")
+            wph = torch.empty((TPh, K), dtype=torch.float16, device="cuda")
+            yph = torch.empty((TPh, D), dtype=torch.float16, device="cuda")
+            pxph, pih, pwph, pyph = (C.c_void_p(t_.data_ptr()) for t_ in (xph, ih, wph, yph))
+
+            def pstep16(layer):
+                rc = Lib.ffmoe_router(h, stream, layer, pxph, D, TPh, pih, pwph, None, C.byref(err))
+                rc |= Lib.ffmoe_prefill(h, stream, layer, pxph, D, TPh, pih, pwph, pyph, C.byref(err))
+                if rc:
+                    raise RuntimeError(err.value)
+            for i in range(4):
+                pstep16(i % L)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(12):
+                pstep16(i % L)
+            torch.cuda.synchronize()
+            fp16["prefill_ms_per_layer"] = round((time.perf_counter() - t0) / 12 * 1e3, 4)
+            ctx.set_profiling(True)
+            ctx.profile(reset=True)
+            for i in range(12):
+                pstep16(i % L)
+            fp16["prefill_kernel_us"] = kernel_times(ctx.profile(reset=True))
+            ctx.set_profiling(False)
+            del xph, ih, wph, yph
+        fp16["note"] = "FFMOE_FP16: router, experts and combine on FP16 rows; the prefill converts its input rows to bf16 once"
+        extra["fp16_mode"] = fp16
+        ctx.set_act_dtype("bf16")
 
     # INT4 GEMV: BASELINE.json config 1 ([1408 x 2816], one input row) and the LM head of config 5
     # ([262144 x 2816]) as resident matrices; synthetic weights as in synth_layer_gpu

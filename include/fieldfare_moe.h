@@ -12,8 +12,9 @@
  *   - return value: FFMOE_OK (0) or a negative status; when `err` is non-NULL and the call fails,
  *     `*err` receives a strdup'd message the caller releases with free();
  *   - a context belongs to one host thread at a time (the reference's operators are not Sendable).
- * Activations, routing weights and outputs are 16-bit: bf16 (FFMOE_BF16), which every kernel
- * computes in with fp32 accumulation.
+ * Activations, routing weights and outputs are 16-bit, all of one type per context: bf16 (FFMOE_BF16, the
+ * default and the type the benchmark configurations name) or FP16 (FFMOE_FP16, the reference's text-path
+ * type, Metal/MoE/moe.metal:69,389,555); see ffmoe_set_activation_dtype. Accumulation is fp32 in both.
  * All paths below are relative to the reference repository root.
  */
 #ifndef FIELDFARE_MOE_H
@@ -34,7 +35,7 @@ enum {
     FFMOE_ERR_NO_LAYER = -4   /* layer not uploaded */
 };
 
-enum { FFMOE_BF16 = 0 };
+enum { FFMOE_BF16 = 0, FFMOE_FP16 = 1 };
 
 enum { FFMOE_GATE = 0, FFMOE_UP = 1, FFMOE_DOWN = 2 };
 
@@ -321,6 +322,22 @@ int ffmoe_layer_tail_norms(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uin
  * (Kernels/Fusions/LMHeadChainInt4.swift:165-170) and around the tail. Same pointer rules as above. */
 int ffmoe_rmsnorm(ffmoe_ctx *ctx, void *stream, const uint16_t *x, uint32_t x_stride, const uint16_t *w,
                   uint16_t *out, uint32_t out_stride, uint32_t t, uint32_t d, float eps, char **err);
+
+/* ---- activation type ------------------------------------------------------------------------- */
+
+/* What the 16-bit values a caller hands over or gets back are: input rows, residual, route weights
+ * (the router's output), outputs, per-route rows, the rows of the setup / tail / norm calls and the
+ * 16-bit outputs of the GEMV calls. FFMOE_BF16 at creation. Norm weights, scales and biases of the
+ * quantized tensors, per-expert scales and effective scales are bf16 in both (as in the reference's
+ * checkpoints). FFMOE_FP16 reproduces the reference's text path: the router reads FP16 rows exactly, the
+ * decode / verify kernels multiply FP16 rows with the INT4 weights on the FP16 matrix instruction and
+ * round where the reference rounds to FP16 (activations, per-route rows, outputs); the prefill GEMMs
+ * keep their bf16 tiles - input rows are rounded to bf16 once, which also makes the reference's
+ * power-of-two block scaling (Metal/Prefill/prefill.metal:593-598,685-702, an FP16 range fix)
+ * unnecessary - and write FP16 rows. In FFMOE_FP16 input rows must be 16-byte aligned with strides
+ * that are multiples of 8 wherever a call accepts less otherwise (router, GEMV). Set it before the
+ * first compute call; switching waits for the device. May allocate (once). */
+int ffmoe_set_activation_dtype(ffmoe_ctx *ctx, int dtype, char **err);
 
 /* ---- per-kernel timing ------------------------------------------------------------------------ */
 

@@ -253,6 +253,43 @@ int main() {
         EXPECT(relS <= 1e-2 && cosS >= 0.9999);
         errorStats(toHost(dH2b, (size_t)T * d), refAll, relS, cosS);
         EXPECT(relS <= 1e-2 && cosS >= 0.9999);
+
+        // the same block with FP16 rows in and out (the reference's text-path type): the bf16 inputs above are
+        // exactly representable in FP16, so the reference rows are the same
+        Context dense16(0, denseShape);
+        bool threwType = false;
+        try { dense16.setActivationDtype(5); } catch (const std::invalid_argument &) { threwType = true; }
+        EXPECT(threwType);
+        dense16.setActivationDtype(FFMOE_FP16);
+        PrefillSharedExpert shared16(dense16);
+        shared16.load(0, gate, up, down);
+        std::vector<uint16_t> xh((size_t)T * d);
+        for (size_t i = 0; i < xh.size(); ++i) {
+            const _Float16 h = (_Float16)ffo_bf16_to_float(x[i]);
+            std::memcpy(&xh[i], &h, 2);
+        }
+        uint16_t *dxh = toDevice(xh);
+        shared16.encodeBlock(stream, 0, dxh, dH2b, T, d, f, d, d);
+        shared16.encode(stream, 0, dxh, dH2);
+        HIP(hipStreamSynchronize(stream));
+        auto asBf16Ref = [&](const std::vector<uint16_t> &halfBits, const std::vector<float> &ref, double &rel, double &cosine) {
+            double maxd = 0, maxr = 0, dot = 0, ng = 0, nr = 0;
+            for (size_t i = 0; i < ref.size(); ++i) {
+                _Float16 h;
+                std::memcpy(&h, &halfBits[i], 2);
+                const double g = (float)h, r = ref[i];
+                maxd = std::fmax(maxd, std::fabs(g - r));
+                maxr = std::fmax(maxr, std::fabs(r));
+                dot += g * r; ng += g * g; nr += r * r;
+            }
+            rel = maxd / std::fmax(maxr, 1e-6);
+            cosine = dot / std::sqrt(ng * nr);
+        };
+        asBf16Ref(toHost(dH2b, (size_t)T * d), refAll, relS, cosS);
+        EXPECT(relS <= 1e-2 && cosS >= 0.9999);
+        asBf16Ref(toHost(dH2, (size_t)d), std::vector<float>(refAll.begin(), refAll.begin() + d), relS, cosS);
+        EXPECT(relS <= 1e-2 && cosS >= 0.9999);
+        HIP(hipFree(dxh));
     }
 
     // --- post-attention setup and layer tail through the mirrored classes: a 5-row block against the oracle's
