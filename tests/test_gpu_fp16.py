@@ -218,3 +218,24 @@ def test_row_steps_fp16_bit_exact(ff, oracle, torch):
     for got, want in zip(outs, ref[1:]):
         assert got.dtype == torch.float16 and np.array_equal(bits_of(got), want)
     ctx.close()
+
+
+def test_guest_pairs_and_reduce_fp16(small, oracle, torch):
+    # the guest seam in FP16 mode (RoutedPrefillGuest.runLayer: sorted pairs in, un-weighted FP16 rows out), then
+    # prefill_moe_reduce_token_major on those rows: the GPU reduce is bit-exact against the oracle's reduce of
+    # the same rows and equals the fused call
+    t = 45
+    rng = np.random.default_rng(21)
+    xb = f16_bits(rng.normal(0, 1, (t, small["d"])))
+    x = f16_tensor(torch, xb)
+    ctx = small["ctx"]
+    idx, w = ctx.router(0, x)
+    pairs = oracle.make_token_expert_pairs(idx.cpu().numpy(), bits_of(w), t, 8)
+    want_partials = oracle.route_partials(small["pool"], pairs, xb, small["d"], t, 8, oracle.FP16)
+    partials = torch.zeros((t, 8, small["d"]), dtype=torch.float16, device="cuda")
+    raw = np.stack([pairs["token"], pairs["expert"], pairs["rank"], pairs["weight_bits"]], 1).astype(np.uint32)
+    ctx.prefill_pairs(0, x, torch.from_numpy(raw.view(np.int32)).cuda(), t, partials)
+    assert rel_err(f16_float(bits_of(partials)), f16_float(want_partials)) <= 1e-2
+    h2 = bits_of(ctx.reduce_token_major(partials, w))
+    assert np.array_equal(h2, oracle.reduce_token_major(bits_of(partials), oracle.FP16, bits_of(w), oracle.FP16))
+    assert np.array_equal(h2, bits_of(ctx.prefill(0, x, idx, w)))
