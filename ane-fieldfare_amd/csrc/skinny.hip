@@ -555,6 +555,71 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
     }
 }
 
+// Decode step (one row): down projection and combine in one launch. A block owns one 32-row tile row of the
+// output for ALL of the row's routes, wave r the expert of route r: every wave requests its 11 KiB of
+// weights and its activation row at once, the eight results meet in LDS and are added in rank order with
+// the arithmetic of combine_kernel (residual first, fmaf per route), so the output is bit for bit what the
+// two launches give. No plan is read: a wave takes its expert and weight straight from the routes.
+template <bool F16>
+__global__ __launch_bounds__(512, 1) void decode_down_combine_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                                     uint32_t n_experts, uint32_t top_k,
+                                                                     const uint32_t *__restrict__ idx,
+                                                                     const uint16_t *__restrict__ w,
+                                                                     const uint16_t *__restrict__ acts,
+                                                                     const uint16_t *__restrict__ residual,
+                                                                     uint16_t *__restrict__ y) {
+    __shared__ float s_row[8][2 * kTileRows];
+    __shared__ float s_w[8];
+    const uint32_t lane = threadIdx.x & 63, r = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t rb = blockIdx.x, j = lane & 15, jq = lane >> 4;
+    uint32_t expert = 0;
+    uint16_t wbits = 0;
+    if (r < top_k) {
+        expert = __builtin_amdgcn_readfirstlane(idx[r]);
+        wbits = (uint16_t)__builtin_amdgcn_readfirstlane((uint32_t)w[r]);
+    }
+    const bool live = r < top_k && (wbits & 0x7FFFu) != 0 && expert < n_experts;
+    if (lane == 0) s_w[r] = live ? Act<F16>::widen(wbits) : 0.0f;
+    if (live) {
+        const uint8_t *expert_base = arena_layer + (size_t)expert * g.expert_bytes;
+        const TileSource src = make_tile_source(expert_base + g.dn_tiles_off, (size_t)g.dn_rbp * g.gf * kTileBytes,
+                                                expert_base + g.dn_scales_off, (size_t)g.dn_rbp * g.gf * kTileScaleBytes);
+        const uint32_t ng = g.gf, g_last = g.gf - 1;
+        WeightRing ring;
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb * ng + min((uint32_t)u, g_last), lane);
+        const uint16_t *arow = acts + (size_t)r * g.f + 8 * jq;      // one row: every token column reads it
+        uint4 x0[kRing], x1[kRing];
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) {
+            const bool in = (uint32_t)u < ng;
+            const uint32_t gg = min((uint32_t)u, g_last);
+            x0[u] = in ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup) : uint4{0, 0, 0, 0};
+            x1[u] = in ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
+        }
+        TwoStreamAcc tot;
+        tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
+        tot.b = tot.a;
+#pragma unroll
+        for (int u = 0; u < kRing; ++u)
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, rb * ng + min((uint32_t)u, g_last), lane);
+        if (jq == 0) {          // token column 0 sits in the first element of lanes 0..15
+            s_row[r][j] = tot.a[0];
+            s_row[r][kTileRows + j] = tot.b[0];
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < 2 * kTileRows) {
+        const uint32_t row = rb * 2 * kTileRows + threadIdx.x;
+        float acc = residual ? Act<F16>::widen(residual[row]) : 0.0f;
+        for (uint32_t q = 0; q < top_k; ++q) {
+            const float wv = s_w[q];
+            if (wv != 0.0f) acc = __builtin_fmaf(wv, s_row[q][threadIdx.x], acc);      // a dead route left no row
+        }
+        y[row] = Act<F16>::round(acc);
+    }
+}
+
 // y[t][c] = bf16(residual + sum_r w[t][r] * partial[t*k + r][c]) in rank order with fmaf, fp32 partials,
 // one rounding at the end (the decode form, moe.metal:627-636). Routes the plan skips (zero weight or
 // expert out of range) add nothing.
@@ -634,6 +699,14 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_GATE_UP);
+    if (t == 1 && dn_whole && !partials_bf16 && top_k <= 8) {
+        // a decode step: down projection and combine in one launch (its time sits in the down slot)
+        hipLaunchKernelGGL(decode_down_combine_kernel<F16>, dim3(g.dn_rbp), dim3(512), 0, s, arena_layer, g, n_experts, top_k, idx,
+                           w, acts, residual, y);
+        timer->mark(s, FFMOE_K_DOWN);
+        timer->finish();
+        return hipGetLastError();
+    }
     const dim3 dn_grid = dn_whole    ? dim3(max((slots + 3) / 4, min(n_cus, (slots * g.dn_rbp + 3) / 4)))
                          : dn_ksplit ? dim3(max(slots, min(resident, slots * g.dn_rbp)))
                                      : dim3((g.dn_rbp + 3) / 4, slots);
