@@ -632,20 +632,35 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
     const uint32_t tok = blockIdx.y;
     const uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (c >= d) return;
+    // every load of the thread is requested before the first is used: the routes' weights and experts, then
+    // the rows of the live ones (a dead route's row may hold anything and is never touched)
+    float wv[8];
+    bool live[8];
+#pragma unroll
+    for (uint32_t r = 0; r < 8; ++r) {
+        const uint32_t route = tok * top_k + min(r, top_k - 1);
+        const uint16_t wb = w[route];
+        live[r] = r < top_k && (wb & 0x7FFFu) != 0 && idx[route] < n_experts;
+        wv[r] = Act<F16>::widen(wb);
+    }
+    f32x4 p[8];
+#pragma unroll
+    for (uint32_t r = 0; r < 8; ++r) {
+        const uint32_t route = tok * top_k + min(r, top_k - 1);
+        p[r] = live[r] ? *reinterpret_cast<const f32x4 *>(partials + (size_t)route * d + c) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (residual) {
         const uint2 rv = *reinterpret_cast<const uint2 *>(residual + (size_t)tok * d + c);
         acc[0] = Act<F16>::lo(rv.x); acc[1] = Act<F16>::hi(rv.x);
         acc[2] = Act<F16>::lo(rv.y); acc[3] = Act<F16>::hi(rv.y);
     }
-    for (uint32_t r = 0; r < top_k; ++r) {
-        const uint32_t route = tok * top_k + r;
-        const uint16_t wb = w[route];
-        if ((wb & 0x7FFFu) == 0 || idx[route] >= n_experts) continue;
-        const float wv = Act<F16>::widen(wb);
-        const f32x4 p = *reinterpret_cast<const f32x4 *>(partials + (size_t)route * d + c);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] = __builtin_fmaf(wv, p[i], acc[i]);
+    for (uint32_t r = 0; r < 8; ++r) {
+        if (live[r]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = __builtin_fmaf(wv[r], p[r][i], acc[i]);
+        }
     }
     uint2 o;
     o.x = Act<F16>::pack(acc[0], acc[1]);
