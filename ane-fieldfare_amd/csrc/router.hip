@@ -51,28 +51,43 @@ __device__ __forceinline__ void accumulate_sub(const void *__restrict__ w_, cons
                                                uint32_t d, uint32_t s, uint32_t lane, uint32_t t0, uint32_t t_last,
                                                float (&acc)[kChunkTokens]) {
     const uint32_t steps = (d + 1023) / 1024;
-#pragma unroll 3
-    for (uint32_t i = 0; i < steps; ++i) {
-        const uint32_t k = 1024 * i + 256 * s + 4 * lane;
-        if (k < d) {
-            float wv[4], sc[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-            load_w4<W_F32>(w_, (size_t)e * d + k, true, wv);
-            if (es) {
-                const uint2 v = *reinterpret_cast<const uint2 *>(es + k);
-                sc[0] = bf16lo_to_f32(v.x); sc[1] = bf16hi_to_f32(v.x);
-                sc[2] = bf16lo_to_f32(v.y); sc[3] = bf16hi_to_f32(v.y);
-            }
+    // Four steps at a time: all their loads (weights, scale, token rows) are requested before the first
+    // product, from clamped addresses so that no load sits behind a branch; the sums then run in the pinned
+    // order. (A load per loop turn behind `if (k < d)` is a serial chain of memory round trips in a kernel
+    // that is nothing but latency.)
+    constexpr int kBatch = 4;
+    for (uint32_t i0 = 0; i0 < steps; i0 += kBatch) {
+        float wv[kBatch][4];
+        uint2 ev[kBatch], xv[kBatch][kChunkTokens];
+        bool live[kBatch];
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const uint32_t k = 1024 * (i0 + b) + 256 * s + 4 * lane;
+            live[b] = k < d;
+            const uint32_t kc = live[b] ? k : 0;
+            load_w4<W_F32>(w_, (size_t)e * d + kc, true, wv[b]);
+            ev[b] = es ? *reinterpret_cast<const uint2 *>(es + kc) : make_uint2(0x3F803F80u, 0x3F803F80u);
 #pragma unroll
             for (int r = 0; r < kChunkTokens; ++r) {
                 // rows past the last token re-read it: same arithmetic, result unused
                 const uint32_t row = min(t0 + r, t_last);
-                const uint2 xv = load_x4<XK != 0>(x + (size_t)row * x_stride + k);
-                const float xf[4] = {Act<XK == 2>::lo(xv.x), Act<XK == 2>::hi(xv.x), Act<XK == 2>::lo(xv.y), Act<XK == 2>::hi(xv.y)};
+                xv[b][r] = load_x4<XK != 0>(x + (size_t)row * x_stride + kc);
+            }
+        }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    // x * effective_scale: 8 or 11 significant bits times 8, exact in fp32 (moe.metal:96-97)
-                    const float xe = es ? xf[j] * sc[j] : xf[j];
-                    acc[r] = __builtin_fmaf(wv[j], xe, acc[r]);
+        for (int b = 0; b < kBatch; ++b) {
+            if (live[b]) {
+                const float sc[4] = {bf16lo_to_f32(ev[b].x), bf16hi_to_f32(ev[b].x), bf16lo_to_f32(ev[b].y), bf16hi_to_f32(ev[b].y)};
+#pragma unroll
+                for (int r = 0; r < kChunkTokens; ++r) {
+                    const float xf[4] = {Act<XK == 2>::lo(xv[b][r].x), Act<XK == 2>::hi(xv[b][r].x), Act<XK == 2>::lo(xv[b][r].y),
+                                         Act<XK == 2>::hi(xv[b][r].y)};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        // x * effective_scale: 8 or 11 significant bits times 8, exact in fp32 (moe.metal:96-97)
+                        const float xe = es ? xf[j] * sc[j] : xf[j];
+                        acc[r] = __builtin_fmaf(wv[b][j], xe, acc[r]);
+                    }
                 }
             }
         }
