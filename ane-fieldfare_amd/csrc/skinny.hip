@@ -311,7 +311,12 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
         route_idx = idx[threadIdx.x];
         route_w = w[threadIdx.x];
     }
-    const uint16_t *xrow = x + (size_t)min(j, rows - 1) * x_stride + 8 * jq;
+    // Load layout: four neighbouring lanes read 64 contiguous bytes of one row (row lane / 4, 8-element chunk
+    // lane % 4), 16 requests of 64 bytes per instruction; with the matrix unit's own layout (row lane % 16)
+    // every lane would be a request of its own and the 22 loads of a wave would keep the address unit busy
+    // for microseconds. The rows are turned into the operand layout (lane (j, jq): row j, chunk jq) by
+    // cross-lane moves once the weight requests are out.
+    const uint16_t *xrow = x + (size_t)min(lane >> 2, rows - 1) * x_stride + 8 * (lane & 3);
     uint4 x0[kRing], x1[kRing];
 #pragma unroll
     for (int u = 0; u < kRing; ++u) {
@@ -346,6 +351,20 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     }
     if (plan_out) build_plan_routes(ps, n_routes, plan_out, route_expert);
     if (!has_rows) return;
+    {
+        const int pull = (int)((4 * j + jq) * 4);       // operand lane (j, jq) takes what load lane 4 j + jq holds
+        auto turn = [&](uint4 &v) {
+            v.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x);
+            v.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y);
+            v.z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z);
+            v.w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w);
+        };
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) {
+            turn(x0[u]);
+            turn(x1[u]);
+        }
+    }
     // this lane finishes token column 4 jq + ks; `stores` = which of that row's top_k routes go to the expert
     // (one bit at most unless a row names an expert twice)
     const uint32_t col = 4 * jq + ks;
