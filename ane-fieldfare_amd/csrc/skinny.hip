@@ -528,7 +528,12 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
     WeightRing ring;
 #pragma unroll
     for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb0 * g.gf + min(g0 + u, g_last), lane);
-    const uint16_t *arow = acts + (size_t)slot.routes[min(j, n - 1)] * g.f + 8 * jq;
+    // a wide expert is a dense one: up to 16 distinct activation rows, fetched four lanes per 64 contiguous
+    // bytes (slot lane / 4, chunk lane % 4) and turned into the operand layout by cross-lane moves
+    // (with one or two rows the operand layout itself is as cheap to load, and needs no moves)
+    const bool gather4 = n > 2;
+    const uint16_t *arow = gather4 ? acts + (size_t)slot.routes[min(lane >> 2, n - 1)] * g.f + 8 * (lane & 3)
+                                   : acts + (size_t)slot.routes[min(j, n - 1)] * g.f + 8 * jq;
     uint4 x0[kRing], x1[kRing];
 #pragma unroll
     for (int u = 0; u < kRing; ++u) {
@@ -536,6 +541,20 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
         const uint32_t gg = min(g0 + u, g_last);
         x0[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup) : uint4{0, 0, 0, 0};
         x1[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
+    }
+    if (gather4) {
+        const int pull = (int)((4 * j + jq) * 4);
+        auto turn = [&](uint4 &v) {
+            v.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x);
+            v.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y);
+            v.z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z);
+            v.w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w);
+        };
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) {
+            turn(x0[u]);
+            turn(x1[u]);
+        }
     }
     const uint32_t my_ts = 4 * jq + ks;     // the token slot this lane finishes
     const size_t out_base = (size_t)slot.routes[min(my_ts, n - 1)] * g.d;
