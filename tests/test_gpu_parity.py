@@ -238,6 +238,34 @@ def test_verify_small_shape(small, oracle, torch, t):
     assert rel_err(got, ref) <= 1e-2 and cosine(got, ref) >= 0.9999
 
 
+@pytest.mark.parametrize("d,f,t", [(3072, 64, 1), (3072, 64, 6), (128, 2880, 6), (128, 2880, 1)])
+def test_verify_shapes_beyond_the_register_ring(oracle, ff, torch, d, f, t):
+    # hidden > 2816: gate/up takes the one-shot grid behind the plan kernel; intermediate > 704: the down
+    # projection splits K over the waves of a block (<= 2816) - routed experts, not only the dense form
+    e, k = 8, 4
+    rng, pool, router = make_layer(oracle, 1000 + d + t, d, f, e, align=1)
+    ctx = ff.Context(d, f, e, k, n_layers=1, max_tokens=16)
+    try:
+        ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
+        ctx.upload_router_bf16(0, router)
+        xb = oracle.bf16_bits(rng.normal(0, 1, (t, d)).astype(np.float32))
+        x = bf16_tensor(torch, xb)
+        idx, w = ctx.router(0, x)
+        idx_np = idx.cpu().numpy().astype(np.uint32)
+        for tok in range(t):
+            ridx, _ = oracle.topk_softmax(oracle.router_logits_pinned(router, xb[tok]), k)
+            assert np.array_equal(idx_np[tok], ridx)
+        ref = oracle.moe_experts(pool, xb, idx_np, oracle.bf16_to_float(bits_of(w)))
+        got = oracle.bf16_to_float(bits_of(ctx.verify(0, x, idx, w)))
+        assert rel_err(got, ref) <= 1e-2 and cosine(got, ref) >= 0.9999
+        assert ctx.last_live_experts() == len(np.unique(idx_np))
+        partials = ctx.verify_partials(0, x, idx, w)
+        got = oracle.bf16_to_float(bits_of(ctx.reduce_token_major(partials, w)))
+        assert rel_err(got, ref) <= 1e-2 and cosine(got, ref) >= 0.9999
+    finally:
+        ctx.close()
+
+
 @pytest.mark.parametrize("t,mode", [(1, "fused"), (16, "fused"), (16, "partials"), (7, "fused")])
 def test_verify_real_shape(real, oracle, torch, t, mode):
     # layer outputs: max rel err <= 1e-2 and cosine >= 0.9999 against the fp32 reference composition

@@ -61,9 +61,11 @@ def test_shared_expert_matches_affine_reference(ff, oracle, torch):
     ctx.close()
 
 
-@pytest.mark.parametrize("d,f,t", [(128, 64, 5), (256, 192, 16), (2816, 2112, 1), (2816, 2112, 16)])
+@pytest.mark.parametrize("d,f,t", [(128, 64, 5), (256, 192, 16), (2816, 2112, 1), (2816, 2112, 16), (3072, 192, 5),
+                                   (192, 3072, 5), (3072, 2880, 16)])
 def test_shared_expert_rows(ff, oracle, torch, d, f, t):
-    # rows <= 16: the streaming kernels; (2816, 2112) is the model's shared expert
+    # rows <= 16: the streaming kernels; (2816, 2112) is the model's shared expert. A hidden size above 2816 or an
+    # intermediate size above 2816 is more than a wave's register ring holds: those take the one-shot grids
     g = oracle.seed_tree_key(0x5EED, f"shared-ffn-d{d}-f{f}-t{t}")
     scale = 0.4 if d < 1024 else 0.08
     parts = tuple(oracle.quantize_int4(g.uniform(-scale, scale, r * c).reshape(r, c)) for r, c in ((f, d), (f, d), (d, f)))
