@@ -28,8 +28,7 @@ struct ffmoe_matrix {
     ffmoe_ctx *ctx = nullptr;
     uint32_t m = 0, n = 0;
     uint8_t *tiles = nullptr, *scales = nullptr;
-    float *logits = nullptr;                  // [16][m] fp32, allocated with the first greedy call's matrix
-    unsigned long long *partials = nullptr;   // [16][segments]
+    unsigned long long *partials = nullptr;   // [16][blocks of the GEMV grid]: per-block winners of the greedy choice
 };
 
 struct ffmoe_ctx {
@@ -633,7 +632,6 @@ int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales
         if (stage) (void)hipFree(stage);
         if (mx->tiles) (void)hipFree(mx->tiles);
         if (mx->scales) (void)hipFree(mx->scales);
-        if (mx->logits) (void)hipFree(mx->logits);
         if (mx->partials) (void)hipFree(mx->partials);
         delete mx;
     };
@@ -649,8 +647,7 @@ int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales
     FF_MX(hipMalloc(&mx->tiles, matrix_tiles_bytes(m, n)));
     FF_MX(hipMalloc(&mx->scales, matrix_scales_bytes(m, n)));
     if (with_greedy) {
-        FF_MX(hipMalloc(&mx->logits, (size_t)FFMOE_MAX_VERIFY_ROWS * m * sizeof(float)));
-        FF_MX(hipMalloc(&mx->partials, (size_t)FFMOE_MAX_VERIFY_ROWS * argmax_segments(m) * sizeof(unsigned long long)));
+        FF_MX(hipMalloc(&mx->partials, (size_t)FFMOE_MAX_VERIFY_ROWS * greedy_segments(m, ctx->n_cus) * sizeof(unsigned long long)));
     }
     // the source may live on the host (an mmap of the checkpoint) or on the device
     const uint8_t *dw = w;
@@ -682,7 +679,6 @@ void ffmoe_matrix_destroy(ffmoe_matrix *mx) {
     (void)hipDeviceSynchronize();
     if (mx->tiles) (void)hipFree(mx->tiles);
     if (mx->scales) (void)hipFree(mx->scales);
-    if (mx->logits) (void)hipFree(mx->logits);
     if (mx->partials) (void)hipFree(mx->partials);
     delete mx;
 }
@@ -716,15 +712,12 @@ int ffmoe_matrix_greedy(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint3
                         uint32_t *out_tokens, char **err) {
     if (int rc = check_matrix_call(mx, x, x_stride, rows, err)) return rc;
     if (!out_tokens) return fail(err, FFMOE_ERR_INVALID, "null argument");
-    if (!mx->logits) return fail(err, FFMOE_ERR_INVALID, "matrix was created without the greedy scratch");
+    if (!mx->partials) return fail(err, FFMOE_ERR_INVALID, "matrix was created without the greedy scratch");
     ffmoe_ctx *ctx = mx->ctx;
     hipStream_t s = static_cast<hipStream_t>(stream);
     ctx->timer.begin(s);
-    FF_HIP(launch_matrix_gemv(s, mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows, mx->logits, mx->m, true,
-                              ctx->n_cus, ctx->f16));
-    ctx->timer.mark(s, FFMOE_K_GEMV);
-    FF_HIP(launch_argmax_rows(s, mx->logits, mx->m, mx->m, rows, mx->partials, out_tokens));
-    ctx->timer.mark(s, FFMOE_K_ARGMAX);
+    FF_HIP(launch_matrix_greedy(s, mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows, mx->partials, out_tokens,
+                                ctx->n_cus, ctx->f16, &ctx->timer));
     ctx->timer.finish();
     return FFMOE_OK;
 }

@@ -136,14 +136,16 @@ hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, co
 size_t matrix_tiles_bytes(uint32_t m, uint32_t n);
 size_t matrix_scales_bytes(uint32_t m, uint32_t n);
 bool matrix_shape_ok(uint32_t n);
-uint32_t argmax_segments(uint32_t m);
 hipError_t launch_matrix_repack(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                                 uint32_t m, uint32_t n, uint8_t *tiles_out, uint8_t *scales_out);
 hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                               const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
                               bool y_f32, uint32_t n_cus, bool f16 = false);
-hipError_t launch_argmax_rows(hipStream_t s, const float *y, uint32_t y_stride, uint32_t m, uint32_t rows,
-                              unsigned long long *partials, uint32_t *out);
+uint32_t greedy_segments(uint32_t m, uint32_t n_cus);
+// the GEMV with the greedy choice as its epilogue: per-block winners, then one block per input row
+hipError_t launch_matrix_greedy(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
+                                const uint16_t *x, uint32_t x_stride, uint32_t rows, unsigned long long *partials,
+                                uint32_t *out, uint32_t n_cus, bool f16, KernelTimer *timer);
 
 // prefill.hip: routes come from (idx, w) [t][top_k], or from an explicit pair list when `pairs` != nullptr.
 // Writes y [t][d] (combined) when y != nullptr; un-weighted bf16 rows go to partials_out or to scratch.

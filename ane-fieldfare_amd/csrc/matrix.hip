@@ -67,12 +67,25 @@ __global__ __launch_bounds__(256) void repack_matrix_kernel(const uint8_t *__res
     }
 }
 
+// Greedy choice per row: the largest finite value wins, ties go to the lowest index, NaN and +-inf never
+// win; a row with no candidate yields index 0 (Metal/Sampling/logit.metal:689-720, 916-921). Two stages: the
+// GEMV's blocks each leave the winner of the weight rows they walked, then one block per input row picks
+// among those. A key orders by value first and by lower index second, so the order of comparisons is free.
+__device__ __forceinline__ unsigned long long argmax_key(float v, uint32_t i) {
+    if (!(__builtin_fabsf(v) < INFINITY)) return 0ull;       // NaN or +-inf: never chosen
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t ord = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    return ((unsigned long long)ord << 32) | (0xFFFFFFFFu - i);
+}
+
 // y[r][m] = sum_g [ s_g * sum_k q_k x_k + b_g * sum_k x_k ] (moe.metal:323-378, logit.metal:614-667) for all
 // input rows at once. grid = (blocks): every block walks a range of 32-row tiles; its four waves split K
 // (at most kRing groups each), keep their slice of the input rows in registers and refill the weight
 // ring across tiles; per tile the partial sums meet in LDS, are added in wave order, and each wave
-// stores a quarter of the input rows.
-template <bool Y_F32, bool F16>
+// stores a quarter of the input rows. GREEDY: nothing is stored per weight row; every lane keeps the best
+// (value, index) key of the sums it finishes and the block leaves one key per input row in
+// y_[row * gridDim.x + block], so the [rows][m] fp32 logits never travel to memory and back.
+template <bool Y_F32, bool F16, bool GREEDY = false>
 __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__restrict__ tiles,
                                                              const uint8_t *__restrict__ scales, uint32_t m,
                                                              uint32_t n_groups, const uint16_t *__restrict__ x,
@@ -82,7 +95,10 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
     const uint32_t n_tiles = (m + 31) / 32;
     uint32_t rb0, rb1;
     split_range(n_tiles, gridDim.x, blockIdx.x, rb0, rb1);
-    if (rb0 >= rb1) return;
+    if (rb0 >= rb1) {
+        if (GREEDY && threadIdx.x < rows) reinterpret_cast<unsigned long long *>(y_)[(size_t)threadIdx.x * gridDim.x + blockIdx.x] = 0ull;
+        return;
+    }
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15, jq = lane >> 4;
     const uint32_t per = (n_groups + kKSplit - 1) / kKSplit;
@@ -106,6 +122,7 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
     const uint32_t my_row = 4 * jq + ks;        // the input row this lane finishes
     float *y32 = reinterpret_cast<float *>(y_);
     uint16_t *y16 = reinterpret_cast<uint16_t *>(y_);
+    unsigned long long best = 0ull;
 
     for (uint32_t rb = rb0; rb < rb1; ++rb) {
         const uint32_t next_row = min(rb + 1, rb1 - 1) * n_groups;
@@ -131,7 +148,11 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
         if (my_row < rows) {
             const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
             const size_t base = (size_t)my_row * y_stride;
-            if (Y_F32) {
+            if (GREEDY) {
+                const unsigned long long ka = row_a < m ? argmax_key(va, row_a) : 0ull;
+                const unsigned long long kb = row_b < m ? argmax_key(vb, row_b) : 0ull;
+                best = max(best, max(ka, kb));
+            } else if (Y_F32) {
                 if (row_a < m) y32[base + row_a] = va;
                 if (row_b < m) y32[base + row_b] = vb;
             } else {
@@ -140,16 +161,13 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
             }
         }
     }
-}
-
-// Greedy choice per row: the largest finite value wins, ties go to the lowest index, NaN and +-inf never
-// win; a row with no candidate yields index 0 (Metal/Sampling/logit.metal:689-720, 916-921). Two stages so that the
-// vocabulary-sized scan uses the whole chip: per (row, segment) partial winners, then one block per row.
-__device__ __forceinline__ unsigned long long argmax_key(float v, uint32_t i) {
-    if (!(__builtin_fabsf(v) < INFINITY)) return 0ull;       // NaN or +-inf: never chosen
-    const uint32_t u = __float_as_uint(v);
-    const uint32_t ord = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-    return ((unsigned long long)ord << 32) | (0xFFFFFFFFu - i);
+    if (GREEDY) {
+        // the 16 lanes that share lane / 16 finished the same input row
+#pragma unroll
+        for (int mk = 8; mk >= 1; mk >>= 1) best = max(best, (unsigned long long)__shfl_xor(best, mk, 64));
+        if (j == 0 && my_row < rows)
+            reinterpret_cast<unsigned long long *>(y_)[(size_t)my_row * gridDim.x + blockIdx.x] = best;
+    }
 }
 
 __device__ __forceinline__ unsigned long long block_max_key(unsigned long long k, unsigned long long *s_k) {
@@ -163,20 +181,6 @@ __device__ __forceinline__ unsigned long long block_max_key(unsigned long long k
     k = s_k[0];
     for (uint32_t v = 1; v < blockDim.x / 64; ++v) k = s_k[v] > k ? s_k[v] : k;
     return k;
-}
-
-__global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__restrict__ y, uint32_t y_stride, uint32_t m,
-                                                             uint32_t seg_len, unsigned long long *__restrict__ part) {
-    __shared__ unsigned long long s_k[4];
-    const uint32_t row = blockIdx.y, seg = blockIdx.x;
-    const uint32_t i0 = seg * seg_len, i1 = min(m, i0 + seg_len);
-    unsigned long long best = 0ull;
-    for (uint32_t i = i0 + threadIdx.x; i < i1; i += 256) {
-        const unsigned long long k = argmax_key(y[(size_t)row * y_stride + i], i);
-        best = k > best ? k : best;
-    }
-    best = block_max_key(best, s_k);
-    if (threadIdx.x == 0) part[(size_t)row * gridDim.x + seg] = best;
 }
 
 __global__ __launch_bounds__(256) void argmax_final_kernel(const unsigned long long *__restrict__ part, uint32_t n_seg,
@@ -220,14 +224,24 @@ hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t
     return hipGetLastError();
 }
 
-uint32_t argmax_segments(uint32_t m) { return min(256u, (m + 4095) / 4096); }
+// keys per input row that launch_matrix_greedy leaves between its two kernels
+uint32_t greedy_segments(uint32_t m, uint32_t n_cus) { return min(2 * n_cus, (m + 31) / 32); }
 
-hipError_t launch_argmax_rows(hipStream_t s, const float *y, uint32_t y_stride, uint32_t m, uint32_t rows,
-                              unsigned long long *partials, uint32_t *out) {
-    const uint32_t n_seg = argmax_segments(m);
-    const uint32_t seg_len = (m + n_seg - 1) / n_seg;
-    hipLaunchKernelGGL(argmax_partial_kernel, dim3(n_seg, rows), dim3(256), 0, s, y, y_stride, m, seg_len, partials);
-    hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, partials, n_seg, out);
+hipError_t launch_matrix_greedy(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
+                                const uint16_t *x, uint32_t x_stride, uint32_t rows, unsigned long long *partials,
+                                uint32_t *out, uint32_t n_cus, bool f16, KernelTimer *timer) {
+    const dim3 grid(greedy_segments(m, n_cus));
+    if (f16)
+        hipLaunchKernelGGL((matrix_gemv_kernel<true, true, true>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride,
+                           rows, partials, 0u);
+    else
+        hipLaunchKernelGGL((matrix_gemv_kernel<true, false, true>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride,
+                           rows, partials, 0u);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    timer->mark(s, FFMOE_K_GEMV);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, partials, grid.x, out);
+    timer->mark(s, FFMOE_K_ARGMAX);
     return hipGetLastError();
 }
 

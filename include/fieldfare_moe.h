@@ -224,7 +224,8 @@ typedef struct ffmoe_matrix ffmoe_matrix;
  * [m][n/64]; host or device memory) into HBM once, as LMHeadChainInt4 keeps the head's table and
  * scratch for its lifetime (Kernels/Fusions/LMHeadChainInt4.swift:57-88). n must be a multiple of 64,
  * at most FFMOE_MATRIX_MAX_N; m is free (the reference's head tests use 4,099 rows). with_greedy != 0
- * also allocates the fp32 logits of ffmoe_matrix_greedy ([16][m]). Blocking; not a hot-path call. */
+ * also allocates the scratch of ffmoe_matrix_greedy (a few KB of per-block winners). Blocking; not a
+ * hot-path call. */
 int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                         uint32_t m, uint32_t n, int with_greedy, ffmoe_matrix **out, char **err);
 void ffmoe_matrix_destroy(ffmoe_matrix *mx);
@@ -236,7 +237,8 @@ void ffmoe_matrix_destroy(ffmoe_matrix *mx);
 int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
                       void *y, uint32_t y_stride, int y_f32, char **err);
 
-/* Greedy token per row: fp32 logits from the GEMV above, then the index of the largest finite logit,
+/* Greedy token per row: the fp32 logits of the GEMV above and, as that kernel's epilogue (the logits are
+ * never written out), the index of the largest finite logit,
  * ties to the lowest index, non-finite values never chosen (Metal/Sampling/logit.metal:689-720,916-921;
  * LMHeadChainInt4.encodeGreedyDecode / encodeGreedyRows, LMHeadChainInt4.swift:94-139,225-284). The
  * input rows are the already normalised hidden rows (the reference runs its RMSNorm operator first). */
