@@ -63,6 +63,37 @@ def block_tokens(rng, t):
     return (np.sqrt(TOKEN_CORRELATION) * c + np.sqrt(1 - TOKEN_CORRELATION) * n).astype(np.float32)
 
 
+def clocks_under_load(burst, torch):
+    """Shader / memory clock and power cap as `rocm-smi` (a child process) reads them while the verify steps run.
+    Best effort: None when the tool is missing or prints something else."""
+    import shutil
+    import subprocess
+    exe = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
+    try:
+        child = subprocess.Popen([exe, "--showclocks", "--showpower", "--showmaxpower", "--json"], stdout=subprocess.PIPE,
+                                 stderr=subprocess.DEVNULL, text=True)
+        t_end = time.perf_counter() + 1.5
+        while child.poll() is None and time.perf_counter() < t_end:
+            burst()
+            torch.cuda.synchronize()
+        text, _ = child.communicate(timeout=20)
+        card = next(iter(json.loads(text[text.index("{"):]).values()))
+        pick = {}
+        for key, val in card.items():
+            k = key.lower()
+            if "sclk clock speed" in k:
+                pick["sclk"] = val.strip("()")
+            elif "mclk clock speed" in k:
+                pick["mclk"] = val.strip("()")
+            elif "max graphics package power" in k:
+                pick["power_cap_W"] = float(val)
+            elif "power" in k and "(w)" in k:
+                pick["power_W"] = float(val)
+        return pick or None
+    except Exception:
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -136,9 +167,13 @@ def main():
 
     # distinct experts per layer for this block (decides the algorithmic bytes of each step)
     live = []
+    tokens_per_expert = np.zeros(T * K + 1, np.int64)     # [n]: live experts that n of the block's routes go to
     for layer in range(L):
         step(layer)
         live.append(ctx.last_live_experts())
+        per_expert = np.bincount(idx.cpu().numpy().astype(np.int64).ravel(), minlength=E)
+        assert int((per_expert > 0).sum()) == live[-1], "plan and routes disagree on the live experts"
+        tokens_per_expert += np.bincount(per_expert[per_expert > 0], minlength=T * K + 1)
     for i in range(args.warmup):
         step(i % L)
     torch.cuda.synchronize()
@@ -165,7 +200,8 @@ def main():
                    "note": "per-step HIP-event intervals, each including one event record"}
     props = torch.cuda.get_device_properties(0)
     device_info = {"name": props.name, "compute_units": props.multi_processor_count,
-                   "hbm_GiB": round(props.total_memory / 2 ** 30, 1), "torch": torch.__version__, "hip": torch.version.hip}
+                   "hbm_GiB": round(props.total_memory / 2 ** 30, 1), "torch": torch.__version__, "hip": torch.version.hip,
+                   "clocks_under_load": clocks_under_load(lambda: [step(i % L) for i in range(4 * L)], torch)}
 
     if args.copy_probe:
         src_c = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
@@ -614,7 +650,9 @@ def main():
                                f"{E} experts x intermediate {F}, top-{K}, INT4 g64; steps cycle {L} resident layers",
                    "tokens": T, "layers_resident": L, "distinct_experts_mean": round(float(np.mean(live)), 1),
                    "distinct_experts_min": int(min(live)), "distinct_experts_max": int(max(live)),
-                   "expert_bytes_per_step_mean": int(np.mean(live) * EXPERT_BYTES)},
+                   "expert_bytes_per_step_mean": int(np.mean(live) * EXPERT_BYTES),
+                   "routes_per_live_expert_hist": {str(n): int(c) for n, c in enumerate(tokens_per_expert) if c},
+                   "routes_per_live_expert_note": f"over the {L} layers: how many live experts receive n of the block's {T * K} routes"},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "step_us": step_spread,
         "device": device_info,
