@@ -64,32 +64,35 @@ def block_tokens(rng, t):
 
 
 def clocks_under_load(burst, torch):
-    """Shader / memory clock and power cap as `rocm-smi` (a child process) reads them while the verify steps run.
-    Best effort: None when the tool is missing or prints something else."""
-    import shutil
-    import subprocess
-    exe = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
+    """Shader / memory clock and power cap from the amdgpu driver's sysfs files (what `rocm-smi --showclocks
+    --showmaxpower` prints), read while a queue of verify steps is still running. No child process is started.
+    Best effort: None when the files are not there or read differently."""
+    import glob
+
+    def current(path):
+        for line in open(path):
+            if line.strip().endswith("*"):
+                return line.split(":", 1)[1].replace("*", "").strip()
+        return None
+
     try:
-        child = subprocess.Popen([exe, "--showclocks", "--showpower", "--showmaxpower", "--json"], stdout=subprocess.PIPE,
-                                 stderr=subprocess.DEVNULL, text=True)
-        t_end = time.perf_counter() + 1.5
-        while child.poll() is None and time.perf_counter() < t_end:
+        cards = [os.path.dirname(f) for f in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))]
+        if not cards:
+            return None
+        for _ in range(3):                      # let the clocks ramp, then leave a backlog on the stream
             burst()
-            torch.cuda.synchronize()
-        text, _ = child.communicate(timeout=20)
-        card = next(iter(json.loads(text[text.index("{"):]).values()))
-        pick = {}
-        for key, val in card.items():
-            k = key.lower()
-            if "sclk clock speed" in k:
-                pick["sclk"] = val.strip("()")
-            elif "mclk clock speed" in k:
-                pick["mclk"] = val.strip("()")
-            elif "max graphics package power" in k:
-                pick["power_cap_W"] = float(val)
-            elif "power" in k and "(w)" in k:
-                pick["power_W"] = float(val)
-        return pick or None
+        torch.cuda.synchronize()
+        for _ in range(8):
+            burst()
+        seen = [(current(c + "/pp_dpm_sclk"), current(c + "/pp_dpm_mclk"), c) for c in cards]
+        torch.cuda.synchronize()
+        mhz = lambda v: int("".join(ch for ch in (v or "0") if ch.isdigit()) or 0)
+        sclk, mclk, card = max(seen, key=lambda r: mhz(r[0]))       # the busy card, should the box show several
+        pick = {"sclk": sclk, "mclk": mclk}
+        caps = glob.glob(card + "/hwmon/hwmon*/power1_cap")
+        if caps:
+            pick["power_cap_W"] = int(open(caps[0]).read()) / 1e6
+        return pick
     except Exception:
         return None
 
