@@ -119,6 +119,10 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
         x0[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup) : uint4{0, 0, 0, 0};
         x1[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
     }
+    // per group: the sum of its inputs per token column, once for all the tile rows this wave walks
+    f32x4 sx[kRing];
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) sx[u] = group_input_sum<F16>(x0[u], x1[u]);
     const uint32_t my_row = 4 * jq + ks;        // the input row this lane finishes
     float *y32 = reinterpret_cast<float *>(y_);
     uint16_t *y16 = reinterpret_cast<uint16_t *>(y_);
@@ -131,7 +135,7 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min(g0 + u, g_last), lane);
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], sx[u], tot, src, next_row + min(g0 + u, g_last), lane);
         const int buf = (rb - rb0) & 1;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {

@@ -365,6 +365,10 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
             turn(x1[u]);
         }
     }
+    // per group: the sum of its inputs per token column, once for all the tile rows this wave walks
+    f32x4 sx[kRing];
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) sx[u] = group_input_sum<F16>(x0[u], x1[u]);
     // this lane finishes token column 4 jq + ks; `stores` = which of that row's top_k routes go to the expert
     // (one bit at most unless a row names an expert twice)
     const uint32_t col = 4 * jq + ks;
@@ -385,7 +389,7 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, gu_src, next_row + min(g0 + u, g_last), lane);
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], sx[u], tot, gu_src, next_row + min(g0 + u, g_last), lane);
         const int buf = (rb - rb0) & 1;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -452,6 +456,10 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
         x0[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup) : uint4{0, 0, 0, 0};
         x1[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
     }
+    // per group: the sum of its inputs per token column, once for all the tile rows this wave walks
+    f32x4 sx[kRing];
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) sx[u] = group_input_sum<F16>(x0[u], x1[u]);
     uint32_t out_base[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -467,7 +475,7 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min((uint32_t)u, g_last), lane);
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], sx[u], tot, src, next_row + min((uint32_t)u, g_last), lane);
         // The sums take a detour through a wave-private LDS slot. It costs sixteen LDS operations per tile
         // row and changes nothing arithmetically, but it is what keeps the register allocation of this loop
         // sane: with the sums used directly the compiler keeps every group's matrix results alive to the end
@@ -556,6 +564,10 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
             turn(x1[u]);
         }
     }
+    // per group: the sum of its inputs per token column, once for all the tile rows this wave walks
+    f32x4 sx[kRing];
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) sx[u] = group_input_sum<F16>(x0[u], x1[u]);
     const uint32_t my_ts = 4 * jq + ks;     // the token slot this lane finishes
     const size_t out_base = (size_t)slot.routes[min(my_ts, n - 1)] * g.d;
 
@@ -566,7 +578,7 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, next_row + min(g0 + u, g_last), lane);
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], sx[u], tot, src, next_row + min(g0 + u, g_last), lane);
         const int buf = (rb - rb0) & 1;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -635,12 +647,16 @@ __global__ __launch_bounds__(512, 1) void decode_down_combine_kernel(const uint8
             x0[u] = in ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup) : uint4{0, 0, 0, 0};
             x1[u] = in ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
         }
+        // per group: the sum of its inputs per token column, once for all the tile rows this wave walks
+        f32x4 sx[kRing];
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) sx[u] = group_input_sum<F16>(x0[u], x1[u]);
         TwoStreamAcc tot;
         tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
         tot.b = tot.a;
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
-            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], tot, src, rb * ng + min((uint32_t)u, g_last), lane);
+            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], sx[u], tot, src, rb * ng + min((uint32_t)u, g_last), lane);
         if (jq == 0) {          // token column 0 sits in the first element of lanes 0..15
             s_row[r][j] = tot.a[0];
             s_row[r][kTileRows + j] = tot.b[0];

@@ -51,13 +51,23 @@ __device__ __forceinline__ void ring_fill(WeightRing &ring, int u, const TileSou
     ring.s[u] = make_uint2(s.x, s.y);
 }
 
-// Consume ring slot u against the resident token operand, then start the load that refills the slot.
+// Sum of a group's 64 inputs per token column, in the register layout of the matrix results: the product
+// with an all-ones operand. It depends on the token operand only, so a wave that walks several tile rows
+// with the same operand computes it once per group, not once per tile.
 template <bool F16 = false>
-__device__ __forceinline__ void ring_step(WeightRing &ring, int u, bool live, const uint4 &x0, const uint4 &x1,
-                                          TwoStreamAcc &tot, const TileSource &src, uint32_t next_tile_index,
-                                          uint32_t lane) {
+__device__ __forceinline__ f32x4 group_input_sum(const uint4 &x0, const uint4 &x1) {
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     const uint4 ones = {Act<F16>::kOnesBits, Act<F16>::kOnesBits, Act<F16>::kOnesBits, Act<F16>::kOnesBits};
+    return Act<F16>::mfma(x1, ones, Act<F16>::mfma(x0, ones, zero));
+}
+
+// Consume ring slot u against the resident token operand (`sx` = its group_input_sum), then start the load
+// that refills the slot.
+template <bool F16 = false>
+__device__ __forceinline__ void ring_step(WeightRing &ring, int u, bool live, const uint4 &x0, const uint4 &x1,
+                                          const f32x4 &sx, TwoStreamAcc &tot, const TileSource &src,
+                                          uint32_t next_tile_index, uint32_t lane) {
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     const uint4 tile = ring.t[u];
     uint2 sc = ring.s[u];
     if (!live) sc = make_uint2(0u, 0u);
@@ -66,8 +76,6 @@ __device__ __forceinline__ void ring_step(WeightRing &ring, int u, bool live, co
     acc_a = Act<F16>::mfma(x1, unpack8_offset<F16>(tile.y), acc_a);
     f32x4 acc_b = Act<F16>::mfma(x0, unpack8_offset<F16>(tile.z), zero);
     acc_b = Act<F16>::mfma(x1, unpack8_offset<F16>(tile.w), acc_b);
-    f32x4 sx = Act<F16>::mfma(x0, ones, zero);
-    sx = Act<F16>::mfma(x1, ones, sx);
     const float sa = bf16lo_to_f32(sc.x), ba = bf16hi_to_f32(sc.x);
     const float sb = bf16lo_to_f32(sc.y), bb = bf16hi_to_f32(sc.y);
     const float ta = __builtin_fmaf(-Act<F16>::kOffset, sa, ba), tb = __builtin_fmaf(-Act<F16>::kOffset, sb, bb);
