@@ -419,7 +419,6 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
                                                                  const uint16_t *__restrict__ acts,
                                                                  float *__restrict__ partials_f32,
                                                                  uint16_t *__restrict__ partials_bf16) {
-    __shared__ float s_tmp[4][8][64];
     const uint32_t n_live = __builtin_amdgcn_readfirstlane(plan->n_live);
     if (n_live == 0) return;
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -476,19 +475,14 @@ __global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *
 #pragma unroll
         for (int u = 0; u < kRing; ++u)
             ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], sx[u], tot, src, next_row + min((uint32_t)u, g_last), lane);
-        // The sums take a detour through a wave-private LDS slot. It costs sixteen LDS operations per tile
-        // row and changes nothing arithmetically, but it is what keeps the register allocation of this loop
-        // sane: with the sums used directly the compiler keeps every group's matrix results alive to the end
-        // of the row and spills 180 registers (the K-split kernels get the same effect from their LDS merge).
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            s_tmp[wave][r][lane] = tot.a[r];
-            s_tmp[wave][4 + r][lane] = tot.b[r];
-        }
+        // The compiler keeps every group's matrix results to the end of the tile row and applies scale and
+        // bias only inside the branch of a token slot that is stored: with the two or three slots an expert
+        // has on average most of those 16 fma per tile never run. That needs the 512 registers of one wave
+        // per SIMD; under the 256 of two it spills.
         const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float va = s_tmp[wave][r][lane], vb = s_tmp[wave][4 + r][lane];
+            const float va = tot.a[r], vb = tot.b[r];
             if (4 * jq + r < n) {
                 if (OUT_BF16) {
                     partials_bf16[(size_t)out_base[r] + row_a] = Act<F16>::round(va);
