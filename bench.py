@@ -258,12 +258,16 @@ def main():
             for i in range(L):
                 fn_(i)
             torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for i in range(4 * L):
-                fn_(i % L)
-            torch.cuda.synchronize()
-            dec = (time.perf_counter() - t0) / (4 * L)
+            runs = []
+            for _ in range(7):          # a run is 3 ms: the median of seven keeps a stray host hiccup out
+                t0 = time.perf_counter()
+                for i in range(4 * L):
+                    fn_(i % L)
+                torch.cuda.synchronize()
+                runs.append((time.perf_counter() - t0) / (4 * L))
+            dec = float(np.median(runs))
             extra[name_] = round(dec * 1e6, 2)
+            extra[name_ + "_min_max"] = [round(min(runs) * 1e6, 2), round(max(runs) * 1e6, 2)]
         extra["decode_expert_GBs"] = round(K * EXPERT_BYTES / dec / 1e9, 1)
 
     # prefill half of the metric (BASELINE.json config 4): 3,072 tokens through one MoE layer, router
