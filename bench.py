@@ -225,7 +225,7 @@ def main():
     # An event record costs the stream a few microseconds. The library measures an empty interval (two
     # records with nothing between them, once per call); a kernel's interval carries half of that - one
     # record's worth - on top of the kernel's own duration, which is what rocprofv3 --kernel-trace shows
-    # (gate/up: 33.1 us raw, 5.1 us empty interval, 30.5 us corrected, 30.3 us in the trace).
+    # (gate/up: 29.5 us raw, 5.2 us empty interval, 26.9 us corrected, 27.3 us in the trace).
     gap_ms = 0.5 * prof["event_gap"][0] / prof["event_gap"][1] if "event_gap" in prof else 0.0
 
     def kernel_times(pr):
