@@ -136,7 +136,7 @@ def main():
     assert payload == EXPERT_BYTES
     ff_off = ff.Offsets(*offsets.as_tuple())
 
-    ctx = ff.Context(D, F, E, K, n_layers=L, max_tokens=8192 if args.sweep else 4096)
+    ctx = ff.Context(D, F, E, K, n_layers=L, max_tokens=max(8192 if args.sweep else 4096, args.prefill_tokens))
     host_layer0 = None
     routers = []
     for layer in range(L):
