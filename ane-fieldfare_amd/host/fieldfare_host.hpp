@@ -353,7 +353,7 @@ private:
 };
 
 // LMHeadChainInt4 (Kernels/Fusions/LMHeadChainInt4.swift:57-139,225-284): owns the head's INT4 table for its
-// lifetime - here the re-tiled resident copy - plus the fp32 logits scratch, and returns greedy tokens for
+// lifetime - here the re-tiled resident copy - plus the scratch of the greedy choice, and returns greedy tokens for
 // 1...maxGreedyRows normalised hidden rows with one pass over the table. The RMSNorm the Swift chain runs
 // first is a separate operator there too (rms.encodeBF16W) and stays with the caller.
 class LMHeadChainInt4 {
