@@ -18,3 +18,12 @@ def oracle():
     from oracle import oracle as o
     o.build()
     return o
+
+
+@pytest.fixture(scope="session", autouse=True)
+def built_library():
+    """The tests load the HIP library that is built in-tree; only when none is there (a fresh checkout) is it
+    compiled first - hipcc cross-compiles gfx950 without a GPU."""
+    import fieldfare_moe
+    if not fieldfare_moe.LIB_PATH.exists():
+        fieldfare_moe.build()

@@ -21,7 +21,7 @@ def test_header_declares_the_expected_surface():
 
 def test_library_exports_every_declared_symbol():
     import fieldfare_moe
-    assert fieldfare_moe.LIB_PATH.exists(), "build the HIP library first: python -c 'import __graft_entry__ as g; g.build()'"
+    assert fieldfare_moe.LIB_PATH.exists(), "the session fixture builds the library when it is missing"
     lib = ctypes.CDLL(str(fieldfare_moe.LIB_PATH))
     missing = [s for s in declared_symbols() if not hasattr(lib, s)]
     assert not missing, f"not exported: {missing}"
