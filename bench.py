@@ -124,6 +124,8 @@ def main():
 
     import torch
     import fieldfare_moe as ff
+    if not ff.LIB_PATH.exists():          # nothing built in-tree: compile once, then load that
+        ff.build()
     from oracle import oracle
 
     assert torch.cuda.is_available(), "bench.py needs a HIP device"
