@@ -25,7 +25,8 @@ struct ffmoe_layer {
 
 // A resident matrix: the re-tiled copy of one [m][n] INT4 weight plus the scratch of its greedy choice.
 struct ffmoe_matrix {
-    ffmoe_ctx *ctx = nullptr;
+    ffmoe_ctx *ctx = nullptr;     // null once the owning context was destroyed (the device memory went with it)
+    int device = 0;
     uint32_t m = 0, n = 0;
     uint8_t *tiles = nullptr, *scales = nullptr;
     unsigned long long *partials = nullptr;   // [16][blocks of the GEMV grid]: per-block winners of the greedy choice
@@ -42,7 +43,6 @@ struct ffmoe_ctx {
     // scratch (owned by the context, sized at creation; calls on one context must not overlap)
     float *logits = nullptr;         // [max(max_tokens,16)][E]
     VerifyPlan *plan = nullptr;
-    uint32_t *counters = nullptr;    // completion counters of the fused router (self-resetting)
     uint16_t *acts = nullptr;        // [16*top_k][F]
     float *partials = nullptr;       // [16*top_k][D]
     PrefillScratch pf{};
@@ -52,6 +52,7 @@ struct ffmoe_ctx {
     uint16_t *dense_w = nullptr;     // [max(max_tokens,16)] 1.0 in the activation type
     bool f16 = false;                // activations are FP16 (ffmoe_set_activation_dtype)
     KernelTimer timer;
+    std::vector<ffmoe_matrix *> matrices;   // resident matrices created on this context and not yet destroyed
 };
 
 namespace {
@@ -131,6 +132,12 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     }
     ctx->shape = *shape;
     ctx->geom = make_geom(shape->d, shape->f);
+    // an expert's tile regions are addressed through buffer descriptors with 32-bit sizes and offsets
+    if ((size_t)shape->d * shape->f >= ((size_t)1 << 32)) {
+        delete ctx;
+        return fail(err, FFMOE_ERR_INVALID, "d = %u x f = %u: an expert's gate/up tile region must stay below 4 GiB", shape->d,
+                    shape->f);
+    }
     ctx->layer_bytes = (size_t)shape->n_experts * ctx->geom.expert_bytes;
     ctx->layers.resize(shape->n_layers);
     const uint32_t router_rows = shape->max_tokens > FFMOE_MAX_VERIFY_ROWS ? shape->max_tokens : FFMOE_MAX_VERIFY_ROWS;
@@ -139,8 +146,6 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->logits), (size_t)router_rows * shape->n_experts * sizeof(float));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->plan), sizeof(VerifyPlan));
     if (e == hipSuccess) e = hipMemset(ctx->plan, 0, sizeof(VerifyPlan));
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->counters), 64 * sizeof(uint32_t));
-    if (e == hipSuccess) e = hipMemset(ctx->counters, 0, 64 * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->acts), routes * shape->f * sizeof(uint16_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->partials), routes * shape->d * sizeof(float));
     // prefill scratch: sort tables, pair lists, activations and per-route rows for max_tokens tokens
@@ -162,9 +167,10 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
         if (e == hipSuccess) e = hipMemsetD16(reinterpret_cast<hipDeviceptr_t>(ctx->dense_w), 0x3F80, router_rows);
     }
     if (e != hipSuccess) {
+        const size_t want = ctx->layer_bytes * shape->n_layers;      // read before the context is gone
         ffmoe_destroy(ctx);
-        return fail(err, FFMOE_ERR_ALLOC, "failed to allocate the expert arena (%zu bytes) or scratch: %s",
-                    ctx->layer_bytes * shape->n_layers, hipGetErrorString(e));
+        return fail(err, FFMOE_ERR_ALLOC, "failed to allocate the expert arena (%zu bytes) or scratch: %s", want,
+                    hipGetErrorString(e));
     }
     *out = ctx;
     return FFMOE_OK;
@@ -182,7 +188,6 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (ctx->arena) (void)hipFree(ctx->arena);
     if (ctx->logits) (void)hipFree(ctx->logits);
     if (ctx->plan) (void)hipFree(ctx->plan);
-    if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->acts) (void)hipFree(ctx->acts);
     if (ctx->partials) (void)hipFree(ctx->partials);
     if (ctx->pf.block_cnt) (void)hipFree(ctx->pf.block_cnt);
@@ -195,6 +200,15 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (ctx->pf.x16) (void)hipFree(ctx->pf.x16);
     if (ctx->dense_idx) (void)hipFree(ctx->dense_idx);
     if (ctx->dense_w) (void)hipFree(ctx->dense_w);
+    // matrices that outlive their context lose their device memory here; the handles stay valid to destroy
+    for (ffmoe_matrix *mx : ctx->matrices) {
+        if (mx->tiles) (void)hipFree(mx->tiles);
+        if (mx->scales) (void)hipFree(mx->scales);
+        if (mx->partials) (void)hipFree(mx->partials);
+        mx->tiles = mx->scales = nullptr;
+        mx->partials = nullptr;
+        mx->ctx = nullptr;
+    }
     for (auto &ev : ctx->timer.ev)
         if (ev) (void)hipEventDestroy(ev);
     delete ctx;
@@ -356,14 +370,21 @@ int ffmoe_router(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *r
     const ffmoe_layer &l = ctx->layers[layer];
     RouterWeights rw{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale};
     FF_HIP(launch_router(static_cast<hipStream_t>(stream), rw, router_x, x_stride, t, ctx->shape.n_experts,
-                         ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w, ctx->counters, &ctx->timer,
+                         ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w, &ctx->timer,
                          ctx->f16));
     return FFMOE_OK;
 }
 
+// Scratch of one decode / verify call: the context's own allocations, or pieces of the static array.
+struct VerifyScratch {
+    VerifyPlan *plan;
+    uint16_t *acts;
+    float *partials;
+};
+
 static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
                          uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual, uint16_t *y,
-                         uint16_t *partials_bf16, char **err) {
+                         uint16_t *partials_bf16, char **err, const VerifyScratch *use = nullptr) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (int rc = check_layer(ctx, layer, true, false, err)) return rc;
     if (!x || !idx || !w || (!y && !partials_bf16)) return fail(err, FFMOE_ERR_INVALID, "null argument");
@@ -372,9 +393,11 @@ static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uin
         return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
     if ((y && reinterpret_cast<uintptr_t>(y) % 8) || (residual && reinterpret_cast<uintptr_t>(residual) % 8))
         return fail(err, FFMOE_ERR_INVALID, "y and residual must be 8-byte aligned");
+    const VerifyScratch own{ctx->plan, ctx->acts, ctx->partials};
+    const VerifyScratch &sc = use ? *use : own;
     FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                         ctx->plan, ctx->acts, ctx->partials, ctx->n_cus, &ctx->timer, ctx->f16));
+                         sc.plan, sc.acts, sc.partials, ctx->n_cus, &ctx->timer, ctx->f16));
     return FFMOE_OK;
 }
 
@@ -440,6 +463,19 @@ int ffmoe_prefill_pairs(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint
     if (n_pairs == 0) return FFMOE_OK;
     if (!pairs) return fail(err, FFMOE_ERR_INVALID, "null argument");
     return prefill_common(ctx, stream, layer, x, x_stride, t, nullptr, nullptr, pairs, n_pairs, nullptr, partials, err);
+}
+
+int ffmoe_prefill_dump_tiles(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint32_t expert, int gate_up, void *out,
+                             size_t out_bytes, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, true, false, err)) return rc;
+    if (expert >= ctx->shape.n_experts) return fail(err, FFMOE_ERR_INVALID, "expert %u out of range", expert);
+    if (!out || reinterpret_cast<uintptr_t>(out) % 16) return fail(err, FFMOE_ERR_INVALID, "output must be a 16-byte aligned device pointer");
+    const size_t need = (size_t)prefill_dump_fragments(ctx->geom, gate_up != 0) * 64 * sizeof(uint4);
+    if (out_bytes < need) return fail(err, FFMOE_ERR_INVALID, "output holds %zu bytes, the fragments take %zu", out_bytes, need);
+    FF_HIP(launch_prefill_dump_tiles(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
+                                     expert, gate_up != 0, ctx->pf, out));
+    return FFMOE_OK;
 }
 
 int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride, uint32_t t,
@@ -621,9 +657,14 @@ int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales
         return fail(err, FFMOE_ERR_INVALID, "N = %u must be a multiple of %d and at most %d", n, FFMOE_GROUP,
                     FFMOE_MATRIX_MAX_N);
     if (reinterpret_cast<uintptr_t>(w) % 2) return fail(err, FFMOE_ERR_INVALID, "weights need a 2-aligned offset");
+    // the kernels address the tile region through a buffer descriptor with 32-bit sizes and offsets
+    if (matrix_tiles_bytes(m, n) >= ((size_t)1 << 32))
+        return fail(err, FFMOE_ERR_INVALID, "M = %u x N = %u needs a tile region of %zu bytes; the limit is 4 GiB", m, n,
+                    matrix_tiles_bytes(m, n));
     ffmoe_matrix *mx = new (std::nothrow) ffmoe_matrix();
     if (!mx) return fail(err, FFMOE_ERR_ALLOC, "out of host memory");
     mx->ctx = ctx;
+    mx->device = ctx->device;
     mx->m = m;
     mx->n = n;
     const size_t w_bytes = (size_t)m * n / 2, s_bytes = (size_t)m * (n / FFMOE_GROUP) * 2;
@@ -669,22 +710,32 @@ int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales
     FF_MX(hipDeviceSynchronize());
 #undef FF_MX
     if (stage) (void)hipFree(stage);
+    ctx->matrices.push_back(mx);
     *out = mx;
     return FFMOE_OK;
 }
 
 void ffmoe_matrix_destroy(ffmoe_matrix *mx) {
     if (!mx) return;
-    (void)hipSetDevice(mx->ctx->device);
-    (void)hipDeviceSynchronize();
-    if (mx->tiles) (void)hipFree(mx->tiles);
-    if (mx->scales) (void)hipFree(mx->scales);
-    if (mx->partials) (void)hipFree(mx->partials);
+    if (mx->ctx) {      // still owned: release the device memory and leave the context's list
+        (void)hipSetDevice(mx->device);
+        (void)hipDeviceSynchronize();
+        if (mx->tiles) (void)hipFree(mx->tiles);
+        if (mx->scales) (void)hipFree(mx->scales);
+        if (mx->partials) (void)hipFree(mx->partials);
+        auto &list = mx->ctx->matrices;
+        for (size_t i = 0; i < list.size(); ++i)
+            if (list[i] == mx) {
+                list.erase(list.begin() + (long)i);
+                break;
+            }
+    }
     delete mx;
 }
 
 static int check_matrix_call(ffmoe_matrix *mx, const uint16_t *x, uint32_t x_stride, uint32_t rows, char **err) {
-    if (!mx || !mx->ctx) return fail(err, FFMOE_ERR_INVALID, "null matrix");
+    if (!mx) return fail(err, FFMOE_ERR_INVALID, "null matrix");
+    if (!mx->ctx) return fail(err, FFMOE_ERR_INVALID, "the matrix's context was destroyed");
     if (int rc = check_ctx(mx->ctx, err)) return rc;
     if (!x) return fail(err, FFMOE_ERR_INVALID, "null argument");
     if (rows == 0 || rows > FFMOE_MAX_VERIFY_ROWS)

@@ -34,15 +34,8 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, v);
 }
 
-// gelu_pytorch_tanh, Metal/MoE/moe.metal:40-47 (clamp kept: it guards tanh at large magnitudes).
-__device__ __forceinline__ float gelu_tanh(float x) {
-    const float x3 = x * x * x;
-    float inner = 0.7978845608028654f * (x + 0.044715f * x3);
-    inner = fminf(fmaxf(inner, -20.0f), 20.0f);
-    return 0.5f * x * (1.0f + tanhf(inner));
-}
-
-// The same function through 0.5 (1 + tanh z) = 1 / (1 + exp(-2 z)) on the hardware exp2 and reciprocal:
+// gelu_pytorch_tanh, Metal/MoE/moe.metal:40-47 (clamp kept: it guards the exponential at large magnitudes),
+// through 0.5 (1 + tanh z) = 1 / (1 + exp(-2 z)) on the hardware exp2 and reciprocal:
 // about ten instructions instead of a tanhf call, relative error ~1e-6 (the result is rounded to bf16).
 __device__ __forceinline__ float gelu_tanh_fast(float x) {
     const float x3 = x * x * x;
@@ -55,23 +48,6 @@ __device__ __forceinline__ float gelu_tanh_fast(float x) {
 // eight k-slots and position m + 4 holds element 2m + 1, so that ((w >> 4m) & 0x000F000F) is the
 // 16-bit pair (element 2m, element 2m + 1) with no cross-lane or cross-register shuffling.
 //
-// unpack8_offset128: the eight nibbles as bf16 values 128 + q (0x4300 | q is exact: the bf16 ulp at
-// 128 is 1). The matrix unit then accumulates sum (128 + q) x; the caller removes 128 * sum x.
-// One v_and_or_b32 per pair: gfx9 VOP3 takes no literals and one scalar operand, so the mask has to sit in a
-// scalar register and the constant in a vector register. The empty asm statements only hide the two
-// values' constness, which makes the compiler itself select v_and_or_b32 (it otherwise emits and + or).
-__device__ __forceinline__ bf16x8 unpack8_offset128(uint32_t w) {
-    uint32_t mask = 0x000F000Fu, c = 0x43004300u;
-    asm("" : "+s"(mask));
-    asm("" : "+v"(c));
-    uint4 r;
-    r.x = (w & mask) | c;
-    r.y = ((w >> 4) & mask) | c;
-    r.z = ((w >> 8) & mask) | c;
-    r.w = ((w >> 12) & mask) | c;
-    return __builtin_bit_cast(bf16x8, r);
-}
-
 // dequant8_bf16: the eight nibbles as bf16(fma(q, scale, bias)) - the reference's 16-bit tile weight
 // (Metal/Prefill/prefill.metal:581-590 with half replaced by bfloat as Metal/TensorCore/tensorops.metal:267).
 // q * scale is exact in fp32 (4-bit x 8-bit significands), so fma and mul-then-add agree.
@@ -130,7 +106,11 @@ template <> struct Act<true> {
     }
 };
 
-// The eight nibbles of a dword as 16-bit values offset + q in the activation type (see unpack8_offset128).
+// The eight nibbles of a dword as 16-bit values offset + q in the activation type (128 + q as bf16: 0x4300 | q
+// is exact, the bf16 ulp at 128 is 1). The matrix unit then accumulates sum (offset + q) x; the caller removes
+// offset * sum x. One v_and_or_b32 per pair: gfx9 VOP3 takes no literals and one scalar operand, so the mask has
+// to sit in a scalar register and the constant in a vector register. The empty asm statements only hide the two
+// values' constness, which makes the compiler itself select v_and_or_b32 (it otherwise emits and + or).
 template <bool F16>
 __device__ __forceinline__ uint4 unpack8_offset(uint32_t w) {
     uint32_t mask = 0x000F000Fu, c = Act<F16>::kOffsetBits;

@@ -121,7 +121,7 @@ hipError_t launch_dequant_expert(hipStream_t s, const uint8_t *arena_expert, Are
 // router.hip
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer, bool f16 = false);
+                         uint16_t *out_w, KernelTimer *timer, bool f16 = false);
 
 // skinny.hip
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
@@ -153,6 +153,14 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
                           const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
                           const ffmoe_pair *pairs, uint32_t n_pairs_in, uint16_t *y, uint16_t *partials_out,
                           PrefillScratch sc, KernelTimer *timer, bool f16 = false);
+
+// Test hook: the weight fragments of one expert's gate/up (or down) tiles as the grouped GEMM's matrix instructions
+// read them from LDS: [N-block][group][fragment 0..15][lane] x 16 bytes, `prefill_dump_fragments` fragments in all.
+// Fragment u = arena tile (u % 8) / 2 of the N-block, stream u % 2, k-half u / 8; lane l holds row l % 16 of the
+// stream and k = 32 * (k-half) + 8 * (l / 16) .. + 7 of the group.
+uint32_t prefill_dump_fragments(const ArenaGeom &g, bool gate_up);
+hipError_t launch_prefill_dump_tiles(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t expert, bool gate_up,
+                                     PrefillScratch sc, void *dump);
 
 // epilogue.hip: row-wise steps either side of the MoE stage
 hipError_t launch_post_attn_setup(hipStream_t s, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *attn,

@@ -194,10 +194,13 @@ struct GemmWave {
 
 // The k-loop and epilogue of one wave that owns NMB 16-row blocks (a compile-time count: the MFMA
 // sequence has no branches, so the scheduler can interleave it with the expansion of the next tile).
-template <bool GATE_UP, int NMB, bool OUT_F16>
+// DUMP: a test instantiation that also copies every weight fragment out of LDS, read exactly as the matrix
+// instructions read it, so that a test can hold the expanded tile itself against the reference's 16-bit weight.
+template <bool GATE_UP, int NMB, bool OUT_F16, bool DUMP = false>
 __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g, uint4 (*wb)[kTilesPerBlock][2][2][kWave],
                                           const uint32_t *__restrict__ sorted_token,
-                                          const uint32_t *__restrict__ sorted_out_row, uint16_t *__restrict__ out) {
+                                          const uint32_t *__restrict__ sorted_out_row, uint16_t *__restrict__ out,
+                                          uint4 *__restrict__ dump = nullptr) {
     constexpr int NA = NMB > 0 ? NMB : 1;
     const uint32_t lane = gw.lane, wave = gw.wave, j = lane & 15, jq = lane >> 4;
     const uint32_t n_groups = gw.n_groups;
@@ -291,6 +294,14 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
         load_b(min(grp + 2, n_groups - 1));
         uint4 bq[3];
         auto read_b = [&](int u) { bq[u % 3] = wb[buf][(u & 7) >> 1][u & 1][u >> 3][lane]; };
+        if (DUMP && wave == 0) {
+            // fragment u of group grp of this N-block, as unit u of the loop below receives it
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                read_b(u);
+                dump[(((size_t)gw.nb * n_groups + grp) * 16 + u) * kWave + lane] = bq[u % 3];
+            }
+        }
         if (NMB > 0) {
             read_b(0);
             read_b(1);
@@ -391,14 +402,15 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
 }
 
 // OUT_F16: the down projection's per-route rows leave as FP16 instead of bf16 (a context in FP16 mode)
-template <bool GATE_UP, bool OUT_F16 = false>
+template <bool GATE_UP, bool OUT_F16 = false, bool DUMP = false>
 __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                               const PrefillPlan *__restrict__ plan,
                                                               const PrefillTile *__restrict__ tiles,
                                                               const uint32_t *__restrict__ sorted_token,
                                                               const uint32_t *__restrict__ sorted_out_row,
                                                               const uint16_t *__restrict__ a, uint32_t a_stride,
-                                                              uint16_t *__restrict__ out, uint32_t n_nblocks) {
+                                                              uint16_t *__restrict__ out, uint32_t n_nblocks,
+                                                              uint4 *__restrict__ dump = nullptr) {
     __shared__ __align__(16) uint4 wb[2][kTilesPerBlock][2][2][kWave];   // [buffer][tile][stream][k-half][lane]
 
     const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
@@ -421,6 +433,12 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__r
 
     const uint32_t n_mb = (gw.tile.rows + 15) / 16;
     const uint32_t my_mb = n_mb > gw.wave ? (n_mb - gw.wave + 3) / 4 : 0;    // 16-row blocks of this wave
+    if (DUMP) {
+        // the test launch runs one pair: wave 0 owns its row block, the others only expand their tiles
+        if (my_mb) gemm_wave<GATE_UP, 1, OUT_F16, true>(gw, g, wb, sorted_token, sorted_out_row, out, dump);
+        else gemm_wave<GATE_UP, 0, OUT_F16, true>(gw, g, wb, sorted_token, sorted_out_row, out, dump);
+        return;
+    }
     switch (my_mb) {
         case 0: gemm_wave<GATE_UP, 0, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
         case 1: gemm_wave<GATE_UP, 1, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
@@ -478,7 +496,44 @@ __global__ __launch_bounds__(256) void rows_f16_to_bf16_kernel(const uint16_t *_
     *reinterpret_cast<uint4 *>(out + (size_t)blockIdx.y * d + c) = o;
 }
 
+// One pair of expert `expert` sent through the gate/up (or down) GEMM with the weight fragments copied out.
+__global__ void prefill_dump_plan_kernel(uint32_t expert, PrefillPlan *plan, PrefillTile *tiles, uint32_t *sorted_token,
+                                         uint32_t *sorted_out_row) {
+    plan->n_pairs = 1;
+    plan->n_tiles = 1;
+    PrefillTile tl;
+    tl.expert = expert;
+    tl.row_start = 0;
+    tl.rows = 1;
+    tl.pad = 0;
+    tiles[0] = tl;
+    sorted_token[0] = 0;
+    sorted_out_row[0] = 0;
+}
+
 }  // namespace
+
+uint32_t prefill_dump_fragments(const ArenaGeom &g, bool gate_up) {
+    const uint32_t tiles = gate_up ? g.gu_rb : g.dn_rbp, groups = gate_up ? g.gd : g.gf;
+    return (tiles + kTilesPerBlock - 1) / kTilesPerBlock * groups * 16;
+}
+
+hipError_t launch_prefill_dump_tiles(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t expert, bool gate_up,
+                                     PrefillScratch sc, void *dump) {
+    hipLaunchKernelGGL(prefill_dump_plan_kernel, dim3(1), dim3(1), 0, s, expert, sc.plan, sc.tiles, sc.sorted_token,
+                       sc.sorted_out_row);
+    // the pair's input row is whatever row 0 of the scratch holds: only the weight side is looked at
+    if (gate_up) {
+        const uint32_t nb = (g.gu_rb + kTilesPerBlock - 1) / kTilesPerBlock;
+        hipLaunchKernelGGL((prefill_gemm_kernel<true, false, true>), dim3(nb * 8), dim3(256), 0, s, arena_layer, g, sc.plan, sc.tiles,
+                           sc.sorted_token, sc.sorted_out_row, sc.partials, g.d, sc.acts, nb, static_cast<uint4 *>(dump));
+    } else {
+        const uint32_t nb = (g.dn_rbp + kTilesPerBlock - 1) / kTilesPerBlock;
+        hipLaunchKernelGGL((prefill_gemm_kernel<false, false, true>), dim3(nb * 8), dim3(256), 0, s, arena_layer, g, sc.plan, sc.tiles,
+                           sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, sc.partials, nb, static_cast<uint4 *>(dump));
+    }
+    return hipGetLastError();
+}
 
 hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
                           const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,

@@ -275,8 +275,7 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, co
 
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w, uint32_t *counters, KernelTimer *timer, bool f16) {
-    (void)counters;
+                         uint16_t *out_w, KernelTimer *timer, bool f16) {
     timer->begin(s);
     const bool x_aligned = (reinterpret_cast<uintptr_t>(x) % 8 == 0) && (x_stride % 4 == 0);
     if (f16 && !x_aligned) return hipErrorInvalidValue;     // FP16 rows come 8-byte aligned (checked at the boundary)

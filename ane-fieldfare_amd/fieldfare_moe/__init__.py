@@ -48,7 +48,7 @@ EXPORTS = [
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
     "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
     "ffmoe_layer_tail", "ffmoe_route_verify", "ffmoe_gemv_int4_listed",
-    "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype",
+    "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
 ]
 
 PROFILE_SLOTS = 16
@@ -150,6 +150,7 @@ def lib() -> C.CDLL:
     L.ffmoe_upload_router_bf16.argtypes = [vp, u32, vp, vp, vp, errp]
     L.ffmoe_upload_router_int8.argtypes = [vp, u32, vp, vp, vp, vp, vp, errp]
     L.ffmoe_dequant_expert.argtypes = [vp, vp, u32, u32, i32, vp, errp]
+    L.ffmoe_prefill_dump_tiles.argtypes = [vp, vp, u32, u32, i32, vp, sz, errp]
     L.ffmoe_router.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
     L.ffmoe_verify.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, vp, errp]
     L.ffmoe_verify_partials.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
@@ -323,6 +324,25 @@ class Context:
         err = C.c_char_p()
         _check(self.L.ffmoe_dequant_expert(self._h, _stream(), layer, expert, which, _ptr(out), C.byref(err)), err)
         return out
+
+    def prefill_tiles(self, layer: int, expert: int, which: int):
+        """The 16-bit weights of one sub-tensor as the grouped GEMM's matrix instructions read them from LDS, put
+        back into [rows][cols] order: bf16 CUDA tensor (ffmoe_prefill_dump_tiles)."""
+        import torch
+        d, f = self.shape.d, self.shape.f
+        gate_up = which != DOWN
+        tiles, groups = (f // 16, d // GROUP) if gate_up else (d // 32, f // GROUP)
+        nblocks = (tiles + 3) // 4
+        raw = torch.empty((nblocks, groups, 2, 4, 2, 4, 16, 8), dtype=torch.bfloat16, device=f"cuda:{self.device}")
+        err = C.c_char_p()
+        _check(self.L.ffmoe_prefill_dump_tiles(self._h, _stream(), layer, expert, int(gate_up), _ptr(raw),
+                                               raw.numel() * 2, C.byref(err)), err)
+        # raw[nb, g, khalf, tile, stream, kq, r, e]: fragment u = 8 khalf + 2 tile + stream, lane = 16 kq + r
+        t = raw.permute(0, 3, 4, 6, 1, 2, 5, 7)          # nb, tile, stream, r, g, khalf, kq, e
+        t = t.reshape(nblocks * 4, 2, 16, groups * GROUP)[:tiles]
+        if gate_up:
+            return t[:, 0 if which == GATE else 1].reshape(f, d).contiguous()
+        return t.reshape(d, f).contiguous()              # down rows 32 tile + 16 stream + r
 
     # -- router ----------------------------------------------------------------------------------
     def router(self, layer: int, router_x, want_logits: bool = False):

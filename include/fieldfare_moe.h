@@ -112,6 +112,17 @@ int ffmoe_upload_router_int8(ffmoe_ctx *ctx, uint32_t layer, const uint8_t *w, c
 int ffmoe_dequant_expert(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint32_t expert, int which,
                          uint16_t *out_bf16, char **err);
 
+/* Test hook for the grouped GEMM of ffmoe_prefill: runs one pair of `expert` through the gate/up (gate_up != 0) or
+ * the down GEMM and copies out every weight fragment exactly as the matrix instructions read it from LDS:
+ * out[N-block][group][fragment 0..15][lane 0..63] x 8 bf16, where an N-block is four 32-row arena tiles, fragment u is
+ * arena tile (u % 8) / 2 of the N-block, stream u % 2 (gate / up rows 16 * tile + r; down rows 32 * tile + 16 * stream + r),
+ * k-half u / 8, and lane l holds row r = l % 16 at k = 64 * group + 32 * (u / 8) + 8 * (l / 16) .. + 7. Tiles past the last
+ * arena tile repeat the last one. The 16-bit tile weight is what "bit-exact dequantized weights" is a property of
+ * (Tests/ANEFieldfareUpstreamTests/Kernels/TensorCore/MPPPrefillInt4QMMTests.swift:26-37,190-192 hold the Metal tile to
+ * bfloat(fma(q, s, b)) the same way). out_bytes >= ceil(tiles / 4) * groups * 16 KiB. */
+int ffmoe_prefill_dump_tiles(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint32_t expert, int gate_up, void *out,
+                             size_t out_bytes, char **err);
+
 /* ---- router ---------------------------------------------------------------------------------- */
 
 /* logits = W_router . (router_x * effective_scale); top-k by (score desc, index asc); weights =
@@ -223,11 +234,14 @@ typedef struct ffmoe_matrix ffmoe_matrix;
 /* Re-tiles one weight in the reference layout (W uint8 [m][n/2] with 2-byte alignment, S/B bf16
  * [m][n/64]; host or device memory) into HBM once, as LMHeadChainInt4 keeps the head's table and
  * scratch for its lifetime (Kernels/Fusions/LMHeadChainInt4.swift:57-88). n must be a multiple of 64,
- * at most FFMOE_MATRIX_MAX_N; m is free (the reference's head tests use 4,099 rows). with_greedy != 0
+ * at most FFMOE_MATRIX_MAX_N; m is any count whose re-tiled form, ceil(m / 32) * (n / 64) KiB, stays below 4 GiB
+ * (the reference's head tests use 4,099 rows; 262,144 x 2816 takes 352 MiB). with_greedy != 0
  * also allocates the scratch of ffmoe_matrix_greedy (a few KB of per-block winners). Blocking; not a
  * hot-path call. */
 int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                         uint32_t m, uint32_t n, int with_greedy, ffmoe_matrix **out, char **err);
+/* A matrix belongs to the context it was created on. Destroying that context first releases the matrix's
+ * device memory; the handle then only accepts ffmoe_matrix_destroy (compute calls return FFMOE_ERR_INVALID). */
 void ffmoe_matrix_destroy(ffmoe_matrix *mx);
 
 /* y[r][row] = sum_g [ s_g * sum_k q_k x_k + b_g * sum_k x_k ] for r < rows <= 16 with the matrix read

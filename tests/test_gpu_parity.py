@@ -86,6 +86,47 @@ def test_dequant_bit_exact_adversarial(oracle, ff, torch):
     ctx.close()
 
 
+def test_prefill_lds_tile_bit_exact_adversarial(oracle, ff, torch):
+    # The tile the grouped GEMM's matrix instructions read from LDS (copied out by the kernel itself, fragment
+    # by fragment, with the read indexing of the multiply loop) against bf16(fma(q, s, b)): every nibble value,
+    # the adversarial scale/bias set incl. bf16 subnormals and negative scales (MPPPrefillInt4QMMTests.swift:26-37,
+    # tile definition :190-192). Shapes: tiles that fill N-blocks exactly and ones that leave a ragged last block.
+    L = oracle.lib()
+    scales = [L.ffo_bf16_bits(0.001), L.ffo_bf16_bits(-0.0015), 0x0001, 0x8001, L.ffo_bf16_bits(0.0123)]
+    biases = [L.ffo_bf16_bits(-0.01), L.ffo_bf16_bits(0.006), 0x0001, 0x8001, L.ffo_bf16_bits(-0.0984)]
+    for d, f, e in ((128, 64, 2), (192, 320, 3)):
+        parts = []
+        for ex in range(e):
+            triple = []
+            for role, (rows, cols) in enumerate(((f, d), (f, d), (d, f))):
+                n = rows * cols // 2
+                W = ((np.arange(n) * 37 + 0x29 + 11 * role + 5 * ex) & 0xFF).astype(np.uint8).reshape(rows, cols // 2)
+                S = np.array([[scales[(r + g + ex) % 5] for g in range(cols // 64)] for r in range(rows)], np.uint16)
+                B = np.array([[biases[(r * 3 + g) % 5] for g in range(cols // 64)] for r in range(rows)], np.uint16)
+                triple.append((W, S, B))
+            parts.append(tuple(triple))
+        pool = oracle.pool_from_parts(parts, d, f, align=2)
+        ctx = ff.Context(d, f, e, 2, n_layers=1, max_tokens=16)
+        ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
+        for ex in range(e):
+            for which, name in ((ff.GATE, "gate"), (ff.UP, "up"), (ff.DOWN, "down")):
+                got = bits_of(ctx.prefill_tiles(0, ex, which))
+                want = oracle.dequantize_int4_bf16(*pool.sub(ex, name))
+                assert got.shape == want.shape
+                assert np.array_equal(got, want), (d, f, ex, name)
+        ctx.close()
+
+
+def test_prefill_lds_tile_bit_exact_real_shape(real, oracle, ff):
+    for ex in (0, 127):
+        for which, name in ((ff.GATE, "gate"), (ff.UP, "up"), (ff.DOWN, "down")):
+            got = bits_of(real["ctx"].prefill_tiles(0, ex, which))
+            want = oracle.dequantize_int4_bf16(*real["pool"].sub(ex, name))
+            assert np.array_equal(got, want), (ex, name)
+            # and the standalone expansion kernel holds the same bits
+            assert np.array_equal(got, bits_of(real["ctx"].dequant_expert(0, ex, which)))
+
+
 def test_dequant_bit_exact_real_shape(real, oracle, ff):
     # device-resident source blobs take the same re-tiling path as host blobs; spot-check experts
     for ex in (0, 63, 127):
