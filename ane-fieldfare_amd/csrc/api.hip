@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -55,7 +56,31 @@ struct ffmoe_ctx {
     std::vector<ffmoe_matrix *> matrices;   // resident matrices created on this context and not yet destroyed
 };
 
+// ---- scratch of ffmoe_verify_static: device memory that exists from the moment the library is loaded ----------
+// One array per GPU (every device holds its own copy of a __device__ variable), shared by every context and
+// every call on that GPU, never allocated and never freed. Layout: the route plan, then the activation rows
+// [16 * top_k][f] (16-bit), then the un-weighted fp32 down rows [16 * top_k][d].
+constexpr size_t kStaticPlanBytes = 32768;
+constexpr size_t kStaticScratchBytes = FFMOE_STATIC_SCRATCH_BYTES;
+static_assert(sizeof(VerifyPlan) <= kStaticPlanBytes, "the route plan outgrew its share of the static scratch");
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_addr[kMaxDevices] = {};     // device address of `scratch` per device (its host-side name is no address)
+std::mutex g_scratch_mutex;
+
+// With `device` current: look the array's address on that device up once.
+hipError_t resolve_static_scratch(int device) {
+    if (device < 0 || device >= kMaxDevices) return hipSuccess;      // such a device runs without the static entry point
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_addr[device]) return hipSuccess;
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e == hipSuccess) g_scratch_addr[device] = p;
+    return e;
+}
 
 int fail(char **err, int code, const char *fmt, ...) {
     if (err) {
@@ -121,6 +146,7 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     FF_HIP(hipGetDeviceCount(&count));
     if (device < 0 || device >= count) return fail(err, FFMOE_ERR_INVALID, "device %d not present (%d visible)", device, count);
     FF_HIP(hipSetDevice(device));
+    FF_HIP(resolve_static_scratch(device));
 
     ffmoe_ctx *ctx = new (std::nothrow) ffmoe_ctx();
     if (!ctx) return fail(err, FFMOE_ERR_ALLOC, "out of host memory");
@@ -405,6 +431,27 @@ int ffmoe_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x
                  const uint32_t *idx, const uint16_t *w, const uint16_t *residual, uint16_t *y, char **err) {
     if (!y) return fail(err, FFMOE_ERR_INVALID, "null output");
     return verify_common(ctx, stream, layer, x, x_stride, t, idx, w, residual, y, nullptr, err);
+}
+
+int ffmoe_verify_static(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride, uint32_t t,
+                        const uint32_t *idx, const uint16_t *w, const uint16_t *residual, uint16_t *y, char **err) {
+    if (!ctx) return fail(err, FFMOE_ERR_INVALID, "null context");
+    if (!y) return fail(err, FFMOE_ERR_INVALID, "null output");
+    void *base = ctx->device >= 0 && ctx->device < kMaxDevices ? g_scratch_addr[ctx->device] : nullptr;
+    if (!base) return fail(err, FFMOE_ERR_RUNTIME, "the static scratch has no address on device %d", ctx->device);
+    const size_t routes = (size_t)FFMOE_MAX_VERIFY_ROWS * ctx->shape.top_k;
+    const size_t acts_bytes = (routes * ctx->shape.f * sizeof(uint16_t) + 255) & ~(size_t)255;
+    const size_t rows_bytes = routes * ctx->shape.d * sizeof(float);
+    if (kStaticPlanBytes + acts_bytes + rows_bytes > kStaticScratchBytes)
+        return fail(err, FFMOE_ERR_INVALID,
+                    "d = %u, f = %u, top_k = %u need %zu bytes of scratch; the static array holds %zu (use ffmoe_verify)",
+                    ctx->shape.d, ctx->shape.f, ctx->shape.top_k, kStaticPlanBytes + acts_bytes + rows_bytes, kStaticScratchBytes);
+    uint8_t *p = static_cast<uint8_t *>(base);
+    const VerifyScratch sc{reinterpret_cast<VerifyPlan *>(p), reinterpret_cast<uint16_t *>(p + kStaticPlanBytes),
+                           reinterpret_cast<float *>(p + kStaticPlanBytes + acts_bytes)};
+    // Nothing in the array has to start at zero: every call rewrites the plan it reads (all slot counts, the live
+    // count and the live slots' route lists), and rows of the two buffers are read only where this call wrote them.
+    return verify_common(ctx, stream, layer, x, x_stride, t, idx, w, residual, y, nullptr, err, &sc);
 }
 
 int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *router_x, uint32_t router_x_stride,

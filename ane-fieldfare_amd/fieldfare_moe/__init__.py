@@ -49,6 +49,7 @@ EXPORTS = [
     "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
     "ffmoe_layer_tail", "ffmoe_route_verify", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
+    "ffmoe_verify_static",
 ]
 
 PROFILE_SLOTS = 16
@@ -153,6 +154,7 @@ def lib() -> C.CDLL:
     L.ffmoe_prefill_dump_tiles.argtypes = [vp, vp, u32, u32, i32, vp, sz, errp]
     L.ffmoe_router.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
     L.ffmoe_verify.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, vp, errp]
+    L.ffmoe_verify_static.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, vp, errp]
     L.ffmoe_verify_partials.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
     L.ffmoe_route_verify.argtypes = [vp, vp, u32, vp, u32, vp, u32, u32, vp, vp, vp, vp, errp]
     L.ffmoe_last_live_experts.argtypes = [vp, vp, C.POINTER(u32), errp]

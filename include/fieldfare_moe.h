@@ -149,6 +149,19 @@ int ffmoe_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x
                  uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual,
                  uint16_t *y, char **err);
 
+/* ffmoe_verify for callers that cannot allocate or free device memory around the call: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. Same
+ * arguments, same kernels and bit-identical results; its scratch (route plan, activation rows, un-weighted fp32
+ * rows) is a fixed array inside the library image instead of the context's allocations, and the call itself
+ * allocates nothing. Limit: 32 KiB + 16 * top_k * (2 f + 4 d) bytes must fit FFMOE_STATIC_SCRATCH_BYTES (3 MiB; the
+ * reference model takes 1.6 MiB); larger shapes are refused with FFMOE_ERR_INVALID. Every GPU holds one such array
+ * for the life of the process, shared by all contexts and calls on that GPU: calls that overlap on one GPU (two
+ * streams, two contexts, two threads) race on it, and ffmoe_last_live_experts does not see these calls. */
+#define FFMOE_STATIC_SCRATCH_BYTES (3u << 20)
+int ffmoe_verify_static(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
+                        uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual,
+                        uint16_t *y, char **err);
+
 /* Same expert pass, but writes the un-weighted per-route rows bf16 partials[(token*top_k+rank)*d ...]
  * the way the reference's verify and prefill kernels hand them to the reduce
  * (Metal/Prefill/prefill.metal:1372-1374, Runtime/Supervisor/DeviceSupervisor.swift:14-17). */
