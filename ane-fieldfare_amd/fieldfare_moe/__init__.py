@@ -119,10 +119,42 @@ class Matrix:
             pass
 
 
-def build() -> Path:
-    """Compile the library for gfx950 with the Makefile in csrc/ (hipcc cross-compiles without a GPU)."""
-    subprocess.run(["make", "-C", str(CSRC), "-B", "-j8"], check=True, stdout=subprocess.DEVNULL,
-                   stderr=subprocess.DEVNULL)
+HASH_PATH = LIB_PATH.with_suffix(".so.srchash")
+
+
+def source_hash() -> str:
+    """Digest of everything the library is compiled from (kernels, headers, Makefile, the C header)."""
+    import hashlib
+    h = hashlib.sha256()
+    files = sorted(p for p in CSRC.iterdir() if p.suffix in (".hip", ".hpp") or p.name == "Makefile")
+    for p in files + [_PKG.parent / "include" / "fieldfare_moe.h"]:
+        h.update(p.name.encode())
+        h.update(p.read_bytes())
+    return h.hexdigest()
+
+
+def is_stale() -> bool:
+    """True when no library is built or the sources changed since it was (file times do not survive a copy of the tree,
+    so the build leaves a digest of its sources beside the library)."""
+    return not (LIB_PATH.exists() and HASH_PATH.exists() and HASH_PATH.read_text().strip() == source_hash())
+
+
+def build(force: bool = True) -> Path:
+    """Compile the library for gfx950 with the Makefile in csrc/ (hipcc cross-compiles without a GPU). `force` recompiles
+    every source; otherwise make rebuilds what its dependencies say changed. A failed build raises with the compiler's
+    messages."""
+    cmd = ["make", "-C", str(CSRC), "-j8"] + (["-B"] if force else [])
+    run = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if run.returncode != 0:
+        raise RuntimeError(f"building {LIB_PATH.name} failed ({' '.join(cmd)}):\n{run.stdout[-6000:]}")
+    HASH_PATH.write_text(source_hash() + "\n")
+    return LIB_PATH
+
+
+def ensure_built() -> Path:
+    """Load what is built in-tree; compile only when nothing is, or when the sources are newer than the library."""
+    if is_stale():
+        build(force=not LIB_PATH.exists())
     return LIB_PATH
 
 
@@ -135,6 +167,9 @@ def lib() -> C.CDLL:
         return _lib
     if not LIB_PATH.exists():
         raise FileNotFoundError(f"{LIB_PATH} is not built; run __graft_entry__.build() (there is no fallback path)")
+    if is_stale():
+        raise RuntimeError(f"{LIB_PATH} was built from other sources than the ones in {CSRC}; run __graft_entry__.build() "
+                           "or fieldfare_moe.ensure_built()")
     # torch ships its own HIP runtime: it has to be in the process before this library resolves
     # libamdhip64, or two runtimes end up loaded and the second one finds no device
     import torch  # noqa: F401

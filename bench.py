@@ -34,33 +34,35 @@ GATE_UP_BYTES = 2_230_272                # the share the gate/up kernel streams 
 DOWN_BYTES = 1_115_136
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this same workload (seeded, so
-# the launches are the same ones), scaled by a plain 1 GiB copy: see profiles/hbm_traffic_verify16_prefill3072.txt
-TRAFFIC_GATE_UP_VERIFY16 = 113.3e6 + 0.3e6
-TRAFFIC_PREFILL_GEMMS_3072 = (447.7e6 + 34.6e6) + (179.7e6 + 138.4e6)
-TOKEN_CORRELATION = 0.45                 # shared component of the block's tokens -> 40-60 distinct experts
+TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic_verify16_prefill3072.txt"
 
 
-def synth_layer_gpu(torch, gen, offsets):
-    """One layer of experts in the reference blob layout, generated on the GPU: q ~ U{0..15},
-    scale = bf16(|N(0, 0.01)|), bias = bf16(-8 scale + N(0, 1e-3))."""
-    blob = torch.zeros((E, STRIDE), dtype=torch.uint8, device="cuda")
-    offs = offsets.as_tuple()
-    for i, (rows, cols) in enumerate(((F, D), (F, D), (D, F))):
-        wo, so, bo = offs[3 * i:3 * i + 3]
-        nw, ns = rows * cols // 2, rows * (cols // 64)
-        blob[:, wo:wo + nw] = torch.randint(0, 256, (E, nw), dtype=torch.uint8, device="cuda", generator=gen)
-        s = (torch.randn((E, ns), device="cuda", generator=gen) * 0.01).abs().to(torch.bfloat16)
-        b = (-8.0 * s.float() + torch.randn((E, ns), device="cuda", generator=gen) * 1e-3).to(torch.bfloat16)
-        blob[:, so:so + 2 * ns] = s.view(torch.uint8).view(E, 2 * ns)
-        blob[:, bo:bo + 2 * ns] = b.view(torch.uint8).view(E, 2 * ns)
-    return blob
+def measured_traffic():
+    """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this same seeded workload and
+    scaled by a plain 1 GiB copy: the lines `traffic <key> <bytes>` of the committed profile summary. {} when the
+    file is not there."""
+    out = {}
+    try:
+        for line in TRAFFIC_FILE.read_text().splitlines():
+            parts = line.split()
+            if len(parts) == 3 and parts[0] == "traffic":
+                out[parts[1]] = float(parts[2])
+    except OSError:
+        pass
+    return out
 
 
-def block_tokens(rng, t):
-    c = rng.normal(0, 1, D)
-    n = rng.normal(0, 1, (t, D))
-    return (np.sqrt(TOKEN_CORRELATION) * c + np.sqrt(1 - TOKEN_CORRELATION) * n).astype(np.float32)
+def host_cpu():
+    """(logical CPUs the OS shows, model string) of the host the CPU baseline runs on."""
+    model = None
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return os.cpu_count(), model
 
 
 def clocks_under_load(burst, torch):
@@ -113,10 +115,12 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy three times: the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE readings of a rocprofv3 --pmc run are scaled by")
-    ap.add_argument("--sweep", action="store_true",
-                    help="also run BASELINE.json config 5: 8,192-token Zipf prefill over all layers, then 256 decode "
-                         "steps as 16 verify blocks with the LM head once per block")
+    ap.add_argument("--no-sweep", action="store_true",
+                    help="skip BASELINE.json config 5 (8,192-token Zipf prefill over all layers, then 256 decode steps "
+                         "as 16 verify blocks with the LM head once per block)")
+    ap.add_argument("--sweep", action="store_true", help="accepted for older command lines: the sweep runs by default")
     args = ap.parse_args()
+    args.sweep = not args.no_sweep and not args.no_gemv
     if args.gpus != 1:
         print("bench.py measures the one-GPU hot path only; --gpus must be 1 "
               "(the path has no collective; it would shard by expert, each GPU running its own experts' share)", file=sys.stderr)
@@ -124,9 +128,11 @@ def main():
 
     import torch
     import fieldfare_moe as ff
-    if not ff.LIB_PATH.exists():          # nothing built in-tree: compile once, then load that
-        ff.build()
-    from oracle import oracle
+    from fieldfare_moe import synthetic as syn
+    ff.ensure_built()                     # loads what is built in-tree; compiles only if nothing (current) is
+    oracle = None
+    if not args.no_cpu:                   # the CPU oracle is the checker and the cpu_baseline leg, nothing else here
+        from oracle import oracle
 
     assert torch.cuda.is_available(), "bench.py needs a HIP device"
     torch.cuda.set_device(0)
@@ -134,25 +140,26 @@ def main():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0)
     rng = np.random.default_rng(0)
-    offsets, payload = oracle.layout_offsets(D, F, align=16)
-    assert payload == EXPERT_BYTES
-    ff_off = ff.Offsets(*offsets.as_tuple())
+    ff_off, payload = syn.layout_offsets(D, F, align=16)
+    assert payload == EXPERT_BYTES and (syn.D, syn.F, syn.E, syn.K, syn.STRIDE) == (D, F, E, K, STRIDE)
+    traffic = measured_traffic()
 
     ctx = ff.Context(D, F, E, K, n_layers=L, max_tokens=max(8192 if args.sweep else 4096, args.prefill_tokens))
+    config1 = None
     host_layer0 = None
     routers = []
     for layer in range(L):
-        blob = synth_layer_gpu(torch, gen, offsets)
+        blob = syn.synth_layer_gpu(torch, gen, ff_off)
         ctx.upload_layer(layer, blob.view(-1), STRIDE, ff_off)
-        if layer == 0:
+        if layer == 0 and not args.no_cpu:
             host_layer0 = blob.view(-1).cpu().numpy()
         del blob
-        r = oracle.bf16_bits(rng.normal(0, 0.02, (E, D)).astype(np.float32))
+        r = syn.router_weights(rng)
         routers.append(r)
         ctx.upload_router_bf16(layer, r)
     torch.cuda.empty_cache()
 
-    xb = oracle.bf16_bits(block_tokens(rng, T))
+    xb = syn.bf16_bits(syn.block_tokens(rng, T))
     x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
     idx = torch.empty((T, K), dtype=torch.int32, device="cuda")
     w = torch.empty((T, K), dtype=torch.bfloat16, device="cuda")
@@ -277,7 +284,8 @@ def main():
     TP = args.prefill_tokens
     prefill = None
     if TP > 0:
-        xp = torch.from_numpy(oracle.bf16_bits(rng.normal(0, 1, (TP, D)).astype(np.float32)).view(np.int16)).cuda().view(torch.bfloat16)
+        xp_bits = syn.bf16_bits(rng.normal(0, 1, (TP, D)).astype(np.float32))
+        xp = torch.from_numpy(xp_bits.view(np.int16)).cuda().view(torch.bfloat16)
         pidx_t = torch.empty((TP, K), dtype=torch.int32, device="cuda")
         pw_t = torch.empty((TP, K), dtype=torch.bfloat16, device="cuda")
         py_t = torch.empty((TP, D), dtype=torch.bfloat16, device="cuda")
@@ -314,19 +322,13 @@ def main():
                    "roofline": {"bound": "mfma", "kernel": "prefill_gemm_kernel (gate_up + down)",
                                 "achieved": round((flops_gu + flops_dn) / gemm_s / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                                 "unit": "TFLOP/s", "frac": round((flops_gu + flops_dn) / gemm_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-                                "traffic": TRAFFIC_PREFILL_GEMMS_3072 if TP == 3072 else None,
-                                "traffic_unit": "HBM bytes of the two launches (rocprofv3 --pmc, same profile file)"}}
+                                "traffic": traffic.get("prefill3072_gemms") if TP == 3072 else None,
+                                "traffic_unit": f"HBM bytes of the two launches (rocprofv3 --pmc, profiles/{TRAFFIC_FILE.name})"}}
         # BASELINE.json config 4 (ii): the same chunk with Zipf(1.1) routing imposed on the experts
         # (indices and weights given, no router): a few experts hold most pairs, many hold a handful
-        zr_ = np.random.default_rng(4)
-        pz_ = 1.0 / np.arange(1, E + 1) ** 1.1
-        pz_ /= pz_.sum()
-        perm_ = zr_.permutation(E)
-        zidx_ = np.stack([perm_[zr_.choice(E, K, replace=False, p=pz_)] for _ in range(TP)]).astype(np.int32)
-        zw_ = zr_.random((TP, K)).astype(np.float32)
-        zw_ = zw_ / zw_.sum(1, keepdims=True)
+        zidx_, zw_ = syn.zipf_routes(np.random.default_rng(4), TP)
         pidx_t.copy_(torch.from_numpy(zidx_))
-        pw_t.copy_(torch.from_numpy(oracle.bf16_bits(zw_).view(np.int16)).view(torch.bfloat16))
+        pw_t.copy_(torch.from_numpy(syn.bf16_bits(zw_).view(np.int16)).view(torch.bfloat16))
 
         def zstep(layer):
             if Lib.ffmoe_prefill(h, stream, layer, pxp, D, TP, ppi, ppw, ppy, C.byref(err)):
@@ -414,10 +416,7 @@ def main():
     head = None
     if not args.no_gemv:
         def synth_matrix(m):
-            W = torch.randint(0, 256, (m, D // 2), dtype=torch.uint8, device="cuda", generator=gen)
-            S = (torch.randn((m, D // 64), device="cuda", generator=gen) * 0.01).abs().to(torch.bfloat16)
-            Bq = (-8.0 * S.float() + torch.randn((m, D // 64), device="cuda", generator=gen) * 1e-3).to(torch.bfloat16)
-            return W, S, Bq
+            return syn.synth_matrix_gpu(torch, gen, m)
         gemv = {}
         W1, S1, B1 = synth_matrix(2 * F)
         m1 = ctx.matrix(W1, S1, B1)
@@ -425,9 +424,22 @@ def main():
         x1row = x[:1].contiguous()
         t_res = timed(lambda: m1.gemv(x1row), 200)
         t_raw = timed(lambda: ctx.gemv_int4(W1, S1, B1, x1row), 200)
+        # the kernels' own durations (HIP events on the launch stream, less one event record), beside the host-timed calls
+        ctx.set_profiling(True)
+        ctx.profile(reset=True)
+        for _ in range(50):
+            m1.gemv(x1row)
+        k_res = kernel_times(ctx.profile(reset=True)).get("gemv")
+        for _ in range(50):
+            ctx.gemv_int4(W1, S1, B1, x1row)
+        k_raw = kernel_times(ctx.profile(reset=True)).get("gemv")
+        ctx.set_profiling(False)
         gemv["config1_1408x2816"] = {"resident_us": round(t_res * 1e6, 2), "resident_GBs": round(bytes1 / t_res / 1e9, 1),
-                                     "reference_layout_us": round(t_raw * 1e6, 2), "bytes": bytes1,
-                                     "note": "host-timed back-to-back calls: launch latency, not bandwidth, bounds a 2.2 MB GEMV"}
+                                     "resident_kernel_us": k_res, "resident_kernel_GBs": round(bytes1 / (k_res * 1e-6) / 1e9, 1) if k_res else None,
+                                     "reference_layout_us": round(t_raw * 1e6, 2), "reference_layout_kernel_us": k_raw, "bytes": bytes1,
+                                     "note": "host-timed back-to-back calls next to the kernel's own duration: launch latency, "
+                                             "not bandwidth, bounds a 2.2 MB GEMV"}
+        config1 = (W1.cpu().numpy(), S1.view(torch.int16).cpu().numpy().view(np.uint16), B1.view(torch.int16).cpu().numpy().view(np.uint16))
         m1.close()
         V = 262144
         Wh, Sh, Bh = synth_matrix(V)
@@ -448,7 +460,7 @@ def main():
     # routed experts, as a context of one expert; 16 rows (verify block) and the prefill chunk
     if not args.no_shared:
         FS, LS = 2112, 8
-        s_off, s_payload = oracle.layout_offsets(D, FS, align=16)
+        s_off, s_payload = syn.layout_offsets(D, FS, align=16)
         dense = ff.Context(D, FS, 1, 1, n_layers=LS, max_tokens=max(args.prefill_tokens, 16))
         for layer in range(LS):
             blob = torch.empty(s_payload, dtype=torch.uint8, device="cuda")
@@ -461,7 +473,7 @@ def main():
                 bi = (-8.0 * sc.float() + torch.randn((rows, g_), device="cuda", generator=gen) * 1e-3).to(torch.bfloat16)
                 blob[s_o:s_o + rows * g_ * 2] = sc.view(torch.uint8).view(-1)
                 blob[b_o:b_o + rows * g_ * 2] = bi.view(torch.uint8).view(-1)
-            dense.upload_layer(layer, blob, s_payload, ff.Offsets(*s_off.as_tuple()))
+            dense.upload_layer(layer, blob, s_payload, s_off)
             del blob
         state = {"i": 0}
 
@@ -568,15 +580,10 @@ def main():
     if args.sweep:
         TS = 8192
         zr = np.random.default_rng(5)
-        pz = 1.0 / np.arange(1, E + 1) ** 1.1
-        pz /= pz.sum()
-        perm = zr.permutation(E)
-        zidx = np.stack([perm[zr.choice(E, K, replace=False, p=pz)] for _ in range(TS)]).astype(np.int32)
-        zw = zr.random((TS, K)).astype(np.float32)
-        zw = zw / zw.sum(1, keepdims=True)
-        xs_ = torch.from_numpy(oracle.bf16_bits(zr.normal(0, 1, (TS, D)).astype(np.float32)).view(np.int16)).cuda().view(torch.bfloat16)
+        zidx, zw = syn.zipf_routes(zr, TS)
+        xs_ = syn.bf16_cuda(torch, zr.normal(0, 1, (TS, D)).astype(np.float32))
         zi = torch.from_numpy(zidx).cuda()
-        zwt = torch.from_numpy(oracle.bf16_bits(zw).view(np.int16)).cuda().view(torch.bfloat16)
+        zwt = syn.bf16_cuda(torch, zw)
         ys_ = torch.empty((TS, D), dtype=torch.bfloat16, device="cuda")
         pzx, pzi, pzw, pzy = (C.c_void_p(t_.data_ptr()) for t_ in (xs_, zi, zwt, ys_))
 
@@ -624,23 +631,67 @@ def main():
 
     cpu = None
     if not args.no_cpu:
-        pool = oracle.ExpertPool(host_layer0, offsets, STRIDE, D, F)
+        # The CPU oracle (a C restatement of the reference's Swift test-support CPU path: dequantise, then multiply)
+        # on the box's host cores, bounded samples of the same workloads. Threads: the box's share of its host (16 for
+        # one GPU; OMP_NUM_THREADS says so), whatever the OS shows.
+        from concurrent.futures import ThreadPoolExecutor
+        o_off, _ = oracle.layout_offsets(D, F, align=16)
+        pool = oracle.ExpertPool(host_layer0, o_off, STRIDE, D, F)
         threads = min(16, oracle.max_threads())
+        nproc, cpu_model = host_cpu()
+
+        def best_of(fn, budget_s, min_reps=2):
+            reps, t_best, t_start = 0, float("inf"), time.perf_counter()
+            while reps < min_reps or time.perf_counter() - t_start < budget_s:
+                t0_ = time.perf_counter()
+                fn()
+                t_best = min(t_best, time.perf_counter() - t0_)
+                reps += 1
+            return t_best, reps
+
+        # config 3 (the headline): layer 0 of the same 16-token block
         t0 = time.perf_counter()
         ridx, rw, ry = oracle.moe_layer(pool, routers[0], xb, K, threads=1)
         single = time.perf_counter() - t0
-        reps = 0
-        t0 = time.perf_counter()
-        while reps < 3 or (time.perf_counter() - t0) * threads < 12.0:
-            oracle.moe_layer(pool, routers[0], xb, K, threads=threads)
-            reps += 1
-        multi = (time.perf_counter() - t0) / reps
+        multi, reps = best_of(lambda: oracle.moe_layer(pool, routers[0], xb, K, threads=threads), 1.5, 3)
         cpu_bytes = len(np.unique(ridx)) * EXPERT_BYTES
+        legs = {"config3_verify16": {"GBs_1_thread": round(cpu_bytes / single / 1e9, 3), f"GBs_{threads}_threads": round(cpu_bytes / multi / 1e9, 3),
+                                     "ms_1_thread": round(single * 1e3, 1), f"ms_{threads}_threads": round(multi * 1e3, 2)}}
+        # config 2: one token through the same layer (8 experts)
+        d1, _ = best_of(lambda: oracle.moe_layer(pool, routers[0], xb[:1], K, threads=1), 0.5)
+        dm, _ = best_of(lambda: oracle.moe_layer(pool, routers[0], xb[:1], K, threads=min(threads, K)), 0.5)
+        legs["config2_decode"] = {"ms_1_thread": round(d1 * 1e3, 2), f"ms_{min(threads, K)}_threads": round(dm * 1e3, 2),
+                                  "GBs_1_thread": round(K * EXPERT_BYTES / d1 / 1e9, 3),
+                                  f"GBs_{min(threads, K)}_threads": round(K * EXPERT_BYTES / dm / 1e9, 3),
+                                  "note": "8 routes: at most 8 threads have work"}
+        # config 1: the [1408 x 2816] GEMV (dequantise the row, then dot), one thread and rows split over the threads
+        if config1 is not None:
+            W1h, S1h, B1h = config1
+            x1f = oracle.bf16_to_float(xb[0])
+            g1, _ = best_of(lambda: oracle.gemv_int4_ref(W1h, S1h, B1h, x1f), 0.5, 5)
+            cuts = np.linspace(0, W1h.shape[0], threads + 1).astype(int)
+            with ThreadPoolExecutor(threads) as ex:
+                def split_gemv():
+                    list(ex.map(lambda i: oracle.gemv_int4_ref(W1h[cuts[i]:cuts[i + 1]], S1h[cuts[i]:cuts[i + 1]], B1h[cuts[i]:cuts[i + 1]], x1f),
+                                range(threads)))
+                gm, _ = best_of(split_gemv, 0.5, 5)
+            b1 = W1h.size + 2 * S1h.size * 2
+            legs["config1_gemv_1408x2816"] = {"us_1_thread": round(g1 * 1e6, 1), f"us_{threads}_threads": round(gm * 1e6, 1),
+                                              "GBs_1_thread": round(b1 / g1 / 1e9, 3), f"GBs_{threads}_threads": round(b1 / gm / 1e9, 3)}
+        # config 4: a sample of the 3,072-token chunk (the oracle's per-pair FFN is independent per token), extrapolated
+        if prefill is not None:
+            n_s = 4 * threads
+            ps, _ = best_of(lambda: oracle.moe_layer(pool, routers[0], xp_bits[:n_s], K, threads=threads), 2.0, 1)
+            legs["config4_prefill"] = {"sample_tokens": n_s, "sample_ms": round(ps * 1e3, 1), f"tok_per_s_{threads}_threads": round(n_s / ps, 1),
+                                       "ms_per_layer_extrapolated": round(ps / n_s * prefill["tokens"] * 1e3, 1),
+                                       "note": f"first {n_s} of the chunk's {prefill['tokens']} tokens; time scales with the token count"}
         cpu = {"value": round(cpu_bytes / multi / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-               "sample": f"layer 0 of the same 16-token block, {reps} reps on {threads} threads "
-                         f"({multi * 1e3:.1f} ms each); 1 thread: {single * 1e3:.0f} ms = "
-                         f"{cpu_bytes / single / 1e9:.3f} GB/s; C restatement of the reference's Swift CPU "
-                         f"dequant+matmul path, gcc -O3 -march=x86-64-v3"}
+               "nproc": nproc, "cpu_model": cpu_model, "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS"),
+               "compiler": "gcc -O3 -march=x86-64-v3 -ffp-contract=off -fopenmp",
+               "sample": f"config 3: layer 0 of the same 16-token block, best of {reps} reps on {threads} threads "
+                         f"({multi * 1e3:.1f} ms); 1 thread: {single * 1e3:.0f} ms = {cpu_bytes / single / 1e9:.3f} GB/s; "
+                         f"C restatement of the reference's Swift CPU dequant+matmul path; the other configurations' samples are in legs",
+               "legs": legs}
         # the GPU result of layer 0 against that CPU result: the bench measures a correct path
         step(0)
         torch.cuda.synchronize()
@@ -667,8 +718,8 @@ def main():
         "device": device_info,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": TRAFFIC_GATE_UP_VERIFY16 if (T == 16 and L == 30 and "down" in prof) else None,
-                     "traffic_unit": "bytes per launch (rocprofv3 --pmc, profiles/hbm_traffic_verify16_prefill3072.txt)",
+                     "traffic": traffic.get("verify16_gate_up") if (T == 16 and L == 30 and "down" in prof) else None,
+                     "traffic_unit": f"bytes per launch (rocprofv3 --pmc, profiles/{TRAFFIC_FILE.name})",
                      "algorithmic_bytes_per_launch": int(live_sum / args.steps * GATE_UP_BYTES),
                      "avg_kernel_us": kernel_us.get("gate_up")},
         "kernel_us": kernel_us,

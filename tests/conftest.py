@@ -22,8 +22,7 @@ def oracle():
 
 @pytest.fixture(scope="session", autouse=True)
 def built_library():
-    """The tests load the HIP library that is built in-tree; only when none is there (a fresh checkout) is it
-    compiled first - hipcc cross-compiles gfx950 without a GPU."""
+    """The tests load the HIP library that is built in-tree; it is compiled first only when none is there (a fresh
+    checkout) or when its sources changed since it was built - hipcc cross-compiles gfx950 without a GPU."""
     import fieldfare_moe
-    if not fieldfare_moe.LIB_PATH.exists():
-        fieldfare_moe.build()
+    fieldfare_moe.ensure_built()
