@@ -40,7 +40,9 @@ struct VerifyPlan {
     uint32_t n_live;
     uint32_t pad[3];
     PlanSlot slots[FFMOE_MAX_EXPERTS];
-    uint32_t route_valid[FFMOE_MAX_VERIFY_ROWS * 8];   // 1 when the route was planned (weight != 0, expert in range)
+    // 1 when the route takes part: weight != 0, expert in range, among its expert's first 16 routes (a row that names
+    // one expert several times can give an expert more than 16)
+    uint32_t route_valid[FFMOE_MAX_VERIFY_ROWS * 8];
 };
 
 // Per-kernel GPU timing with HIP events on the caller's stream, switched on by ffmoe_set_profiling.

@@ -56,9 +56,9 @@ __device__ __forceinline__ uint32_t build_plan_experts(PlanScratch &ps, uint32_t
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     e = tid < n_routes && (route_w & 0x7FFFu) != 0 && route_idx < n_experts ? route_idx : 0xFFFFFFFFu;
     ps.routes_of[tid] = uint4{0, 0, 0, 0};
-    __syncthreads();
+    lds_barrier();      // LDS only: the token rows requested before the plan stay in flight across it
     if (e != 0xFFFFFFFFu) atomicOr(reinterpret_cast<uint32_t *>(&ps.routes_of[e]) + (tid >> 5), 1u << (tid & 31));
-    __syncthreads();
+    lds_barrier();      // LDS only: the token rows requested before the plan stay in flight across it
     const uint4 mine = ps.routes_of[tid];
     const uint32_t count = tid < n_experts ? __popc(mine.x) + __popc(mine.y) + __popc(mine.z) + __popc(mine.w) : 0;
     ps.cnt[tid] = count;
@@ -66,7 +66,7 @@ __device__ __forceinline__ uint32_t build_plan_experts(PlanScratch &ps, uint32_t
     const unsigned long long mask = __ballot(live);
     const uint32_t before = __popcll(mask & ((1ull << lane) - 1ull));
     if (lane == 0) ps.wave_total[wave] = __popcll(mask);
-    __syncthreads();
+    lds_barrier();      // LDS only: the token rows requested before the plan stay in flight across it
     uint32_t base = 0, total = 0;
 #pragma unroll
     for (uint32_t v = 0; v < 4; ++v) {
@@ -90,7 +90,7 @@ __device__ __forceinline__ uint32_t build_plan_experts(PlanScratch &ps, uint32_t
     // row ranges, loop bounds, load offsets) is treated as per-lane data and computed in vector registers
     total = __builtin_amdgcn_readfirstlane(total);
     my_slot = slot_from_total(total);
-    __syncthreads();
+    lds_barrier();      // LDS only: the token rows requested before the plan stay in flight across it
     return total;
 }
 
@@ -104,6 +104,9 @@ __device__ __forceinline__ void build_plan_routes(PlanScratch &ps, uint32_t n_ro
                              (word >= 2 ? __popc(set.z & (word > 2 ? 0xFFFFFFFFu : below)) : 0) +
                              (word >= 3 ? __popc(set.w & below) : 0);
         if (pos < (uint32_t)kMaxRows) plan_out->slots[ps.slot_of[e]].routes[pos] = tid;
+        plan_out->route_valid[tid] = pos < (uint32_t)kMaxRows ? 1u : 0u;
+    } else if (tid < (uint32_t)kMaxRoutes) {
+        plan_out->route_valid[tid] = 0u;
     }
 }
 
@@ -410,87 +413,84 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     }
 }
 
-// down projection, persistent: the waves of the grid are dealt to the live experts; a wave keeps the
-// expert's (<= 16) activation rows in registers (all of K = F: at most kRing groups) and walks a range of
-// 32-row tile rows with the weight ring refilled across them. No K-split, so no LDS and no barrier.
+// down projection with the expert's activation rows in LDS: one block = four consecutive 32-row tile rows of one
+// expert, one per wave, the whole K = F (at most kRing groups) requested at the wave's first instruction. Without
+// the rows in registers a wave fits 128 registers, so a compute unit holds sixteen waves instead of four, and it
+// is the number of waves with requests in flight, not the depth of each wave's queue, that this 55 MB stream
+// responds to: measured on the same tiles, one wave per tile row reads them in 10 us, the persistent form's 1,024
+// waves of four to five tile rows each in 15 us. Slots past the last live expert hold n = 0 and leave at once.
+constexpr int kDownLdsRow = kRing * kGroup * 2 + 16;      // bytes per activation row in LDS, padded against bank conflicts
+
 template <bool OUT_BF16, bool F16>
-__global__ __launch_bounds__(256, 1) void skinny_down_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
-                                                                 const VerifyPlan *__restrict__ plan,
-                                                                 const uint16_t *__restrict__ acts,
-                                                                 float *__restrict__ partials_f32,
-                                                                 uint16_t *__restrict__ partials_bf16) {
-    const uint32_t n_live = __builtin_amdgcn_readfirstlane(plan->n_live);
-    if (n_live == 0) return;
-    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t gwave = blockIdx.x * 4 + wave;
-    const uint32_t waves_per_slot = max(1u, min(g.dn_rbp, gridDim.x * 4 / n_live));
-    const uint32_t slot_id = gwave / waves_per_slot;
-    if (slot_id >= n_live) return;
-    uint32_t rb0, rb1;
-    split_range(g.dn_rbp, waves_per_slot, gwave % waves_per_slot, rb0, rb1);
-    if (rb0 >= rb1) return;
+__global__ __launch_bounds__(256, 4) void skinny_down_lds(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                          const VerifyPlan *__restrict__ plan,
+                                                          const uint16_t *__restrict__ acts,
+                                                          float *__restrict__ partials_f32,
+                                                          uint16_t *__restrict__ partials_bf16, uint32_t parts) {
+    __shared__ __align__(16) uint8_t s_act[kMaxRows * kDownLdsRow];
+    __shared__ uint32_t s_route[kMaxRows];
+    const uint32_t slot_id = blockIdx.x / parts, part = blockIdx.x % parts;
     const PlanSlot &slot = plan->slots[slot_id];
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    // count, expert and the route list come back in one round trip (entries past the count are stale: unused)
     const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
     const uint32_t expert = __builtin_amdgcn_readfirstlane(slot.expert);
-    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint32_t route_t = threadIdx.x < (uint32_t)kMaxRows ? slot.routes[threadIdx.x] : 0u;
+    if (n == 0) return;
+    const uint32_t rb = part * 4 + wave;
+    const bool has_row = rb < g.dn_rbp;
     const uint8_t *expert_base = arena_layer + (size_t)expert * g.expert_bytes;
     const TileSource src = make_tile_source(expert_base + g.dn_tiles_off, (size_t)g.dn_rbp * g.gf * kTileBytes,
                                             expert_base + g.dn_scales_off, (size_t)g.dn_rbp * g.gf * kTileScaleBytes);
     const uint32_t ng = g.gf, g_last = g.gf - 1;
-
-    // the route list is read in the same round trip as the slot's count: every entry of the fixed-size
-    // list is addressable, entries past the count are stale and replaced by route 0 after the fact
-    const uint32_t route_j = slot.routes[j];
     WeightRing ring;
+    if (has_row) {
 #pragma unroll
-    for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb0 * ng + min((uint32_t)u, g_last), lane);
-    const uint32_t route_0 = __builtin_amdgcn_readfirstlane(route_j);
-    const uint32_t my_route = j < n ? route_j : route_0;
-    const uint16_t *arow = acts + (size_t)my_route * g.f + 8 * jq;
-    uint4 x0[kRing], x1[kRing];
+        for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb * ng + min((uint32_t)u, g_last), lane);
+    }
+    if (threadIdx.x < (uint32_t)kMaxRows) s_route[threadIdx.x] = threadIdx.x < n ? route_t : 0u;
+    __syncthreads();
+    // the n activation rows, 16 bytes per thread and turn, contiguous along a row
+    const uint32_t chunks = g.f / 8;                       // 16-byte pieces per row
+    for (uint32_t i = threadIdx.x; i < n * chunks; i += 256) {
+        const uint32_t r = i / chunks, c = i % chunks;
+        *reinterpret_cast<uint4 *>(s_act + r * kDownLdsRow + c * 16) =
+            *reinterpret_cast<const uint4 *>(acts + (size_t)s_route[r] * g.f + c * 8);
+    }
+    __syncthreads();
+    if (!has_row) return;
+    // token slot j of the operand: row j of the expert's list, row 0 again past the count (columns never stored)
+    const uint8_t *xrow = s_act + (j < n ? j : 0u) * kDownLdsRow + jq * 16;
+    TwoStreamAcc tot;
+    tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
+    tot.b = tot.a;
 #pragma unroll
     for (int u = 0; u < kRing; ++u) {
         const bool live = (uint32_t)u < ng;
         const uint32_t gg = min((uint32_t)u, g_last);
-        x0[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup) : uint4{0, 0, 0, 0};
-        x1[u] = live ? *reinterpret_cast<const uint4 *>(arow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
-    }
-    // per group: the sum of its inputs per token column, once for all the tile rows this wave walks
-    f32x4 sx[kRing];
+        const uint4 x0 = *reinterpret_cast<const uint4 *>(xrow + gg * (kGroup * 2));
+        const uint4 x1 = *reinterpret_cast<const uint4 *>(xrow + gg * (kGroup * 2) + 64);
+        const f32x4 sx = group_input_sum<F16>(x0, x1);
+        ring_step<F16, false>(ring, u, live, x0, x1, sx, tot, src, 0u, lane);
+        // The running sums are pinned here: left alone, the compiler sinks the scale-and-bias arithmetic of every
+        // group into the branches of the stores at the end and carries all eleven groups' matrix results there,
+        // which does not fit 128 registers.
 #pragma unroll
-    for (int u = 0; u < kRing; ++u) sx[u] = group_input_sum<F16>(x0[u], x1[u]);
-    uint32_t out_base[4];
+        for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(tot.a[r]), "+v"(tot.b[r]));
+    }
+    const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        // route of token slot 4 jq + r: lane 4 jq + r holds it (its j is that slot)
-        const uint32_t rt = (uint32_t)__shfl((int)route_j, (int)(4 * jq + r), 64);
-        out_base[r] = (4 * jq + r < n ? rt : route_0) * g.d;
-    }
-
-    for (uint32_t rb = rb0; rb < rb1; ++rb) {
-        const uint32_t next_row = min(rb + 1, rb1 - 1) * ng;
-        TwoStreamAcc tot;
-        tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
-        tot.b = tot.a;
-#pragma unroll
-        for (int u = 0; u < kRing; ++u)
-            ring_step<F16>(ring, u, (uint32_t)u < ng, x0[u], x1[u], sx[u], tot, src, next_row + min((uint32_t)u, g_last), lane);
-        // The compiler keeps every group's matrix results to the end of the tile row and applies scale and
-        // bias only inside the branch of a token slot that is stored: with the two or three slots an expert
-        // has on average most of those 16 fma per tile never run. That needs the 512 registers of one wave
-        // per SIMD; under the 256 of two it spills.
-        const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float va = tot.a[r], vb = tot.b[r];
-            if (4 * jq + r < n) {
-                if (OUT_BF16) {
-                    partials_bf16[(size_t)out_base[r] + row_a] = Act<F16>::round(va);
-                    partials_bf16[(size_t)out_base[r] + row_b] = Act<F16>::round(vb);
-                } else {
-                    partials_f32[(size_t)out_base[r] + row_a] = va;
-                    partials_f32[(size_t)out_base[r] + row_b] = vb;
-                }
+        const uint32_t ts = 4 * jq + r;
+        if (ts < n) {
+            const size_t base = (size_t)s_route[ts] * g.d;
+            if (OUT_BF16) {
+                partials_bf16[base + row_a] = Act<F16>::round(tot.a[r]);
+                partials_bf16[base + row_b] = Act<F16>::round(tot.b[r]);
+            } else {
+                partials_f32[base + row_a] = tot.a[r];
+                partials_f32[base + row_b] = tot.b[r];
             }
         }
     }
@@ -669,12 +669,12 @@ __global__ __launch_bounds__(512, 1) void decode_down_combine_kernel(const uint8
 }
 
 // y[t][c] = bf16(residual + sum_r w[t][r] * partial[t*k + r][c]) in rank order with fmaf, fp32 partials,
-// one rounding at the end (the decode form, moe.metal:627-636). Routes the plan skips (zero weight or
-// expert out of range) add nothing.
+// one rounding at the end (the decode form, moe.metal:627-636). Routes the plan skips (zero weight, expert
+// out of range, or beyond an expert's first 16 routes) add nothing: their rows were never written.
 template <bool F16>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ partials,
                                                       const uint16_t *__restrict__ w,
-                                                      const uint32_t *__restrict__ idx, uint32_t n_experts,
+                                                      const VerifyPlan *__restrict__ plan,
                                                       const uint16_t *__restrict__ residual, uint32_t top_k,
                                                       uint32_t d, uint16_t *__restrict__ y) {
     const uint32_t tok = blockIdx.y;
@@ -688,7 +688,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
     for (uint32_t r = 0; r < 8; ++r) {
         const uint32_t route = tok * top_k + min(r, top_k - 1);
         const uint16_t wb = w[route];
-        live[r] = r < top_k && (wb & 0x7FFFu) != 0 && idx[route] < n_experts;
+        live[r] = r < top_k && plan->route_valid[route] != 0;
         wv[r] = Act<F16>::widen(wb);
     }
     f32x4 p[8];
@@ -770,13 +770,14 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
         timer->finish();
         return hipGetLastError();
     }
-    const dim3 dn_grid = dn_whole    ? dim3(max((slots + 3) / 4, min(n_cus, (slots * g.dn_rbp + 3) / 4)))
+    const uint32_t dn_parts = (g.dn_rbp + 3) / 4;          // blocks per expert of the LDS form: four tile rows each
+    const dim3 dn_grid = dn_whole    ? dim3(slots * dn_parts)
                          : dn_ksplit ? dim3(max(slots, min(resident, slots * g.dn_rbp)))
                                      : dim3((g.dn_rbp + 3) / 4, slots);
 #define FFMOE_DOWN(BF)                                                                                                \
     if (dn_whole)                                                                                                     \
-        hipLaunchKernelGGL((skinny_down_persistent<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,   \
-                           partials_f32, partials_bf16);                                                              \
+        hipLaunchKernelGGL((skinny_down_lds<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,          \
+                           partials_f32, partials_bf16, dn_parts);                                                    \
     else if (dn_ksplit)                                                                                               \
         hipLaunchKernelGGL((skinny_down_ksplit_persistent<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan,  \
                            acts, partials_f32, partials_bf16);                                                        \
@@ -794,8 +795,8 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_DOWN);
-    hipLaunchKernelGGL(combine_kernel<F16>, dim3((g.d / 4 + 255) / 256, t), dim3(256), 0, s, partials_f32, w, idx, n_experts,
-                       residual, top_k, g.d, y);
+    hipLaunchKernelGGL(combine_kernel<F16>, dim3((g.d / 4 + 255) / 256, t), dim3(256), 0, s, partials_f32, w, plan, residual,
+                       top_k, g.d, y);
     timer->mark(s, FFMOE_K_COMBINE);
     timer->finish();
     return hipGetLastError();

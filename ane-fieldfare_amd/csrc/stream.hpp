@@ -62,8 +62,8 @@ __device__ __forceinline__ f32x4 group_input_sum(const uint4 &x0, const uint4 &x
 }
 
 // Consume ring slot u against the resident token operand (`sx` = its group_input_sum), then start the load
-// that refills the slot.
-template <bool F16 = false>
+// that refills the slot (REFILL = false: a wave that walks one tile row only has nothing to refill).
+template <bool F16 = false, bool REFILL = true>
 __device__ __forceinline__ void ring_step(WeightRing &ring, int u, bool live, const uint4 &x0, const uint4 &x1,
                                           const f32x4 &sx, TwoStreamAcc &tot, const TileSource &src,
                                           uint32_t next_tile_index, uint32_t lane) {
@@ -71,7 +71,7 @@ __device__ __forceinline__ void ring_step(WeightRing &ring, int u, bool live, co
     const uint4 tile = ring.t[u];
     uint2 sc = ring.s[u];
     if (!live) sc = make_uint2(0u, 0u);
-    ring_fill(ring, u, src, next_tile_index, lane);
+    if (REFILL) ring_fill(ring, u, src, next_tile_index, lane);
     f32x4 acc_a = Act<F16>::mfma(x0, unpack8_offset<F16>(tile.x), zero);
     acc_a = Act<F16>::mfma(x1, unpack8_offset<F16>(tile.y), acc_a);
     f32x4 acc_b = Act<F16>::mfma(x0, unpack8_offset<F16>(tile.z), zero);

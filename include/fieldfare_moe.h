@@ -144,7 +144,9 @@ int ffmoe_router(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *r
  * encodeGatherRoutedSlots / encodeRoutedPersistentGPUSlots (Kernels/MoE/MoE.swift:312-496); t <= 16
  * replaces PrefillGroupedRoutedMoE.encodeVerifyBound / encodeVerifyRows
  * (Kernels/Prefill/MoE/PrefillGroupedRoutedMoE.swift:331-448) followed by
- * PrefillMoE.encodeReduceTokenMajor. Routes whose weight is exactly zero are skipped. */
+ * PrefillMoE.encodeReduceTokenMajor. Routes whose weight is exactly zero are skipped. A row names an expert at most
+ * once in the reference (top-k selects distinct experts); should a table name one expert more than 16 times in all,
+ * its first 16 routes in [row][rank] order take part and the others add nothing. */
 int ffmoe_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
                  uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual,
                  uint16_t *y, char **err);

@@ -497,3 +497,30 @@ def test_gemv_int4_listed_rows(small, oracle, torch):
     for r in range(rows):
         ref = oracle.gemv_int4_ref(W[ids], S[ids], B[ids], oracle.bf16_to_float(xb[r]))
         assert rel_err(listed[r], ref) < 5e-3
+
+
+def test_expert_named_more_than_16_times_keeps_its_first_16_routes(small, oracle, torch):
+    # The router never names an expert twice in a row, but ffmoe_verify takes any table: an expert's route list holds
+    # 16 entries, further routes to it (in [row][rank] order) take no part - they add nothing, instead of whatever the
+    # scratch rows held.
+    ctx, d, t = small["ctx"], small["d"], 16
+    rng = np.random.default_rng(991)
+    xb = oracle.bf16_bits(rng.normal(0, 1, (t, d)).astype(np.float32))
+    x = bf16_tensor(torch, xb)
+    idx_np = np.stack([rng.permutation(np.arange(1, small["e"]))[:8] for _ in range(t)]).astype(np.uint32)
+    idx_np[idx_np == 5] = 6
+    idx_np[:, 0] = 5
+    idx_np[:, 3] = 5                      # expert 5: 32 routes, the first 16 are rows 0..7
+    w_np = rng.random((t, 8)).astype(np.float32)
+    w_np /= w_np.sum(1, keepdims=True)
+    wb = oracle.bf16_bits(w_np)
+    kept = oracle.bf16_to_float(wb).copy()
+    kept[8:, 0] = 0.0
+    kept[8:, 3] = 0.0
+    idx = torch.from_numpy(idx_np.astype(np.int32)).cuda()
+    w = bf16_tensor(torch, wb)
+    # poison the scratch rows first: a block whose every route is live fills them all
+    ctx.verify(1, x, *ctx.router(1, x))
+    got = oracle.bf16_to_float(bits_of(ctx.verify(1, x, idx, w)))
+    ref = oracle.moe_experts(small["pool"], xb, idx_np, kept)
+    assert rel_err(got, ref) <= 1e-2 and cosine(got, ref) >= 0.9999, (rel_err(got, ref), cosine(got, ref))
