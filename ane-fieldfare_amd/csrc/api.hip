@@ -184,7 +184,10 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.tiles), (size_t)ctx->pf.max_tiles * sizeof(PrefillTile));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.sorted_token), (size_t)ctx->max_pairs * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.sorted_out_row), (size_t)ctx->max_pairs * sizeof(uint32_t));
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.acts), (size_t)ctx->max_pairs * shape->f * sizeof(uint16_t));
+    // activations in 16-pair blocks: an M-tile's blocks start at a block of their own (see prefill.hip)
+    if (e == hipSuccess)
+        e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.acts),
+                      ((size_t)ctx->max_pairs / 16 + ctx->pf.max_tiles + 2) * 16 * shape->f * sizeof(uint16_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.partials), (size_t)ctx->max_pairs * shape->d * sizeof(uint16_t));
     if (e == hipSuccess && shape->n_experts == 1 && shape->top_k == 1) {
         e = hipMalloc(reinterpret_cast<void **>(&ctx->dense_idx), (size_t)router_rows * sizeof(uint32_t));

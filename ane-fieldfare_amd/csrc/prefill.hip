@@ -181,14 +181,21 @@ __global__ __launch_bounds__(kSortBlock) void prefill_scatter_kernel(ItemSource 
 //      64-wide group ahead, into registers - the rows are private to the wave, LDS would add nothing.
 //   B: wave w expands arena tile w of the next group to bf16(fma(q, scale, bias)) into the other half of
 //      a double-buffered LDS area while all waves multiply from the current half; one barrier per group.
-// GATE_UP: A rows are gathered token rows of x; streams are gate / up; out = acts[pair][F].
-// else:    A rows are acts[pair][F]; streams are two 16-row blocks; out = partials[out_row][D] (bf16).
+// GATE_UP: A rows are gathered token rows of x; streams are gate / up; out = the activations, stored in the order the
+//          down GEMM's matrix instructions want them (below).
+// else:    A = those activations, loaded straight into operand registers (1 KiB contiguous per wave and fragment, no
+//          cross-lane re-layout); streams are two 16-row blocks; out = partials[out_row][D] (16-bit).
+// Activation layout: [16-pair block][group of F][k-half][lane (j, jq)] x 8 values = pair j of the block at
+// k = 32 * (k-half) + 8 * jq .. + 7 of the group. The 16-pair blocks of M-tile ti start at block row_start / 16 + ti:
+// consecutive tiles never share a block (a tile adds at most one block of slack), so the buffer holds
+// max_pairs / 16 + max_tiles + 1 blocks.
 // ---------------------------------------------------------------------------------------------------
 
 struct GemmWave {
     const uint8_t *w_tiles, *w_scales;    // this wave's arena tile row
     const uint16_t *a;                    // A matrix
     uint32_t a_stride, n_groups, n_arena_tiles, nb, wave, lane;
+    uint32_t act_block0;                  // first 16-pair block of this M-tile in the activation layout
     PrefillTile tile;
 };
 
@@ -207,15 +214,23 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     const uint16_t *arow[NA];
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
+        if (!GATE_UP) {
+            // the activations are stored fragment by fragment: block, group, k-half, then 16 bytes per lane
+            arow[i] = gw.a + ((size_t)(gw.act_block0 + wave + 4 * i) * n_groups * 2) * (kWave * 8) + lane * 8;
+            continue;
+        }
         // load layout: four neighbouring lanes read 64 contiguous bytes of one row (row lane / 4, 8-element
         // chunk lane % 4), so a load touches 16 half-lines instead of 64 scattered 16-byte pieces
         const uint32_t prow = min((wave + 4 * i) * 16 + (lane >> 2), gw.tile.rows - 1);
-        const uint32_t src = GATE_UP ? sorted_token[gw.tile.row_start + prow] : gw.tile.row_start + prow;
-        arow[i] = gw.a + (size_t)src * gw.a_stride + 8 * (lane & 3);
+        const uint32_t src = sorted_token[gw.tile.row_start + prow];
+        // rows 8..15 take their four chunks rotated by two: the lanes a half-wave then pulls from in the re-layout
+        // below fall on 32 different LDS banks (in natural order rows r and r + 8 collide on every bank)
+        arow[i] = gw.a + (size_t)src * gw.a_stride + 8 * (((lane & 3) - 2 * (lane >> 5)) & 3);
     }
-    // MFMA layout: lane (j, jq) needs row j, chunk jq = what load-layout lane 4 j + jq holds
-    const int pull = (int)((4 * j + jq) * 4);
+    // MFMA layout: lane (j, jq) needs row j, chunk jq = what load-layout lane 4 j + ((jq + 2 (j / 8)) % 4) holds
+    const int pull = (int)((4 * j + ((jq + 2 * (j >> 3)) & 3)) * 4);
     auto to_frag = [&](const uint4 &v) {
+        if (!GATE_UP) return __builtin_bit_cast(bf16x8, v);      // already in operand order
         uint4 r;
         r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x);
         r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y);
@@ -268,7 +283,9 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     auto load_a = [&](uint32_t grp, int half) {
         if (NMB == 0) return;
 #pragma unroll
-        for (int i = 0; i < NA; ++i) araw[i][half] = *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup + 32 * half);
+        for (int i = 0; i < NA; ++i)
+            araw[i][half] = GATE_UP ? *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup + 32 * half)
+                                    : *reinterpret_cast<const uint4 *>(arow[i] + (size_t)(grp * 2 + half) * (kWave * 8));
     };
     auto frag_a = [&](int half) {
         if (NMB == 0) return;
@@ -348,15 +365,17 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
         for (int i = 0; i < NA; ++i) {
             const uint32_t prow = (wave + 4 * i) * 16 + j;
             if (prow >= gw.tile.rows) continue;
-            uint16_t *orow = out + (size_t)(gw.tile.row_start + prow) * g.f;
+            // this N-block is group nb of F (four arena tiles = 64 activations); arena tile tl holds k = 16 tl .. + 15
+            // of it, this lane the four values from k = 16 tl + 4 jq: k-half tl / 2, operand lane (j, 2 (tl % 2) + jq / 2),
+            // values 4 (jq % 2) .. + 3 of that lane's eight
+            uint16_t *oblk = out + ((size_t)(gw.act_block0 + wave + 4 * i) * g.gf + gw.nb) * 2 * (kWave * 8);
 #pragma unroll
             for (int tl = 0; tl < kTilesPerBlock; ++tl) {
-                const uint32_t atl = gw.nb * kTilesPerBlock + tl;
-                if (atl >= gw.n_arena_tiles) continue;
                 float h[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) h[r] = gelu_tanh_fast(acc[i][2 * tl][r]) * acc[i][2 * tl + 1][r];
-                *reinterpret_cast<uint2 *>(orow + atl * kTileRows + 4 * jq) = make_uint2(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]));
+                uint16_t *dst = oblk + (tl >> 1) * (kWave * 8) + (((tl & 1) * 2 + (jq >> 1)) * 16 + j) * 8 + (jq & 1) * 4;
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]));
             }
         }
         return;
@@ -425,6 +444,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__r
     gw.nb = nb;
     gw.a = a;
     gw.a_stride = a_stride;
+    gw.act_block0 = gw.tile.row_start / 16 + ti;
     // the arena tile row this wave expands; past the last one it expands the last again (never stored)
     const uint32_t at = min(nb * kTilesPerBlock + gw.wave, gw.n_arena_tiles - 1);
     const uint8_t *expert_base = arena_layer + (size_t)gw.tile.expert * g.expert_bytes;
