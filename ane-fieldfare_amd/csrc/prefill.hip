@@ -475,22 +475,39 @@ template <bool F16>
 __global__ __launch_bounds__(256) void prefill_combine_kernel(const uint16_t *__restrict__ partials,
                                                               const uint16_t *__restrict__ w,
                                                               const uint32_t *__restrict__ idx, uint32_t n_experts,
-                                                              uint32_t top_k, uint32_t d, uint16_t *__restrict__ y) {
-    const uint32_t tok = blockIdx.y;
-    const uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 8;
-    if (c >= d) return;
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (uint32_t r = 0; r < top_k; ++r) {
-        const uint32_t route = tok * top_k + r;
-        const uint16_t wbits = w[route];
-        if ((wbits & 0x7FFFu) == 0 || idx[route] >= n_experts) continue;
-        const float wv = Act<F16>::widen(wbits);
-        const uint4 p = *reinterpret_cast<const uint4 *>(partials + (size_t)route * d + c);
-        const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
+                                                              uint32_t top_k, uint32_t d, uint32_t t,
+                                                              uint16_t *__restrict__ y) {
+    // one thread per 16-byte piece of an output row, pieces numbered across rows so that every block is full
+    const uint32_t pieces = d / 8, piece = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t tok = piece / pieces, c = (piece % pieces) * 8;
+    if (tok >= t) return;
+    // every load of the thread is requested before the first is used: the routes' weights and experts, then the
+    // rows of the live ones (a dropped route's row was never written and is not touched)
+    float wv[8];
+    bool live[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            acc[2 * i] = __builtin_fmaf(wv, Act<F16>::lo(pw[i]), acc[2 * i]);
-            acc[2 * i + 1] = __builtin_fmaf(wv, Act<F16>::hi(pw[i]), acc[2 * i + 1]);
+    for (uint32_t r = 0; r < 8; ++r) {
+        const uint32_t route = tok * top_k + min(r, top_k - 1);
+        const uint16_t wbits = w[route];
+        live[r] = r < top_k && (wbits & 0x7FFFu) != 0 && idx[route] < n_experts;
+        wv[r] = Act<F16>::widen(wbits);
+    }
+    uint4 p[8];
+#pragma unroll
+    for (uint32_t r = 0; r < 8; ++r) {
+        const uint32_t route = tok * top_k + min(r, top_k - 1);
+        p[r] = live[r] ? *reinterpret_cast<const uint4 *>(partials + (size_t)route * d + c) : uint4{0, 0, 0, 0};
+    }
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (uint32_t r = 0; r < 8; ++r) {
+        if (live[r]) {
+            const uint32_t pw[4] = {p[r].x, p[r].y, p[r].z, p[r].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[2 * i] = __builtin_fmaf(wv[r], Act<F16>::lo(pw[i]), acc[2 * i]);
+                acc[2 * i + 1] = __builtin_fmaf(wv[r], Act<F16>::hi(pw[i]), acc[2 * i + 1]);
+            }
         }
     }
     uint4 o;
@@ -605,11 +622,11 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
     timer->mark(s, FFMOE_K_PREFILL_DOWN);
     if (y) {
         if (f16)
-            hipLaunchKernelGGL(prefill_combine_kernel<true>, dim3((g.d / 8 + 255) / 256, t), dim3(256), 0, s, partials, w, idx,
-                               n_experts, top_k, g.d, y);
+            hipLaunchKernelGGL(prefill_combine_kernel<true>, dim3((t * (g.d / 8) + 255) / 256), dim3(256), 0, s, partials, w, idx,
+                               n_experts, top_k, g.d, t, y);
         else
-            hipLaunchKernelGGL(prefill_combine_kernel<false>, dim3((g.d / 8 + 255) / 256, t), dim3(256), 0, s, partials, w, idx,
-                               n_experts, top_k, g.d, y);
+            hipLaunchKernelGGL(prefill_combine_kernel<false>, dim3((t * (g.d / 8) + 255) / 256), dim3(256), 0, s, partials, w, idx,
+                               n_experts, top_k, g.d, t, y);
         timer->mark(s, FFMOE_K_PREFILL_COMBINE);
     }
     timer->finish();
