@@ -46,6 +46,7 @@ struct ffmoe_ctx {
     VerifyPlan *plan = nullptr;
     uint16_t *acts = nullptr;        // [16*top_k][F]
     float *partials = nullptr;       // [16*top_k][D]
+    RouteMail *mail = nullptr;       // hand-over words of ffmoe_route_verify's one-launch router + gate/up
     PrefillScratch pf{};
     uint32_t max_pairs = 0;
     // dense FFN (n_experts == 1, top_k == 1): every row routes to expert 0 with weight 1
@@ -172,6 +173,12 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->logits), (size_t)router_rows * shape->n_experts * sizeof(float));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->plan), sizeof(VerifyPlan));
     if (e == hipSuccess) e = hipMemset(ctx->plan, 0, sizeof(VerifyPlan));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->mail), sizeof(RouteMail));
+    if (e == hipSuccess) e = hipMemset(ctx->mail, 0, sizeof(RouteMail));
+    if (e == hipSuccess) {
+        const uint32_t first_epoch = 1;      // zeroed words never carry it
+        e = hipMemcpy(&ctx->mail->epoch, &first_epoch, sizeof first_epoch, hipMemcpyHostToDevice);
+    }
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->acts), routes * shape->f * sizeof(uint16_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->partials), routes * shape->d * sizeof(float));
     // prefill scratch: sort tables, pair lists, activations and per-route rows for max_tokens tokens
@@ -217,6 +224,7 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (ctx->arena) (void)hipFree(ctx->arena);
     if (ctx->logits) (void)hipFree(ctx->logits);
     if (ctx->plan) (void)hipFree(ctx->plan);
+    if (ctx->mail) (void)hipFree(ctx->mail);
     if (ctx->acts) (void)hipFree(ctx->acts);
     if (ctx->partials) (void)hipFree(ctx->partials);
     if (ctx->pf.block_cnt) (void)hipFree(ctx->pf.block_cnt);
@@ -413,9 +421,10 @@ struct VerifyScratch {
 
 static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
                          uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual, uint16_t *y,
-                         uint16_t *partials_bf16, char **err, const VerifyScratch *use = nullptr) {
+                         uint16_t *partials_bf16, char **err, const VerifyScratch *use = nullptr,
+                         const RouteFusion *route = nullptr) {
     if (int rc = check_ctx(ctx, err)) return rc;
-    if (int rc = check_layer(ctx, layer, true, false, err)) return rc;
+    if (int rc = check_layer(ctx, layer, true, route != nullptr, err)) return rc;
     if (!x || !idx || !w || (!y && !partials_bf16)) return fail(err, FFMOE_ERR_INVALID, "null argument");
     if (t == 0 || t > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%d", t, FFMOE_MAX_VERIFY_ROWS);
     if (x_stride < ctx->shape.d || x_stride % 8 || reinterpret_cast<uintptr_t>(x) % 16)
@@ -426,7 +435,7 @@ static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uin
     const VerifyScratch &sc = use ? *use : own;
     FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                         sc.plan, sc.acts, sc.partials, ctx->n_cus, &ctx->timer, ctx->f16));
+                         sc.plan, sc.acts, sc.partials, ctx->n_cus, &ctx->timer, ctx->f16, route));
     return FFMOE_OK;
 }
 
@@ -461,9 +470,15 @@ int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint1
                        const uint16_t *x, uint32_t x_stride, uint32_t t, const uint16_t *residual, uint16_t *y,
                        uint32_t *out_idx, uint16_t *out_w, char **err) {
     if (int rc = check_ctx(ctx, err)) return rc;
-    if (!out_idx || !out_w || !y) return fail(err, FFMOE_ERR_INVALID, "null argument");
-    if (int rc = ffmoe_router(ctx, stream, layer, router_x, router_x_stride, t, out_idx, out_w, nullptr, err)) return rc;
-    return ffmoe_verify(ctx, stream, layer, x, x_stride, t, out_idx, out_w, residual, y, err);
+    if (!router_x || !out_idx || !out_w || !y) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (router_x_stride < ctx->shape.d) return fail(err, FFMOE_ERR_INVALID, "hidden stride is too small");
+    if (ctx->f16 && (reinterpret_cast<uintptr_t>(router_x) % 8 || router_x_stride % 4))
+        return fail(err, FFMOE_ERR_INVALID, "FP16 router rows must be 8-byte aligned with a stride that is a multiple of 4");
+    if (layer >= ctx->layers.size()) return fail(err, FFMOE_ERR_INVALID, "layer %u out of range", layer);
+    const ffmoe_layer &l = ctx->layers[layer];
+    const RouteFusion route{RouterWeights{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale}, router_x,
+                            router_x_stride, ctx->logits, ctx->mail};
+    return verify_common(ctx, stream, layer, x, x_stride, t, out_idx, out_w, residual, y, nullptr, err, nullptr, &route);
 }
 
 int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
@@ -477,6 +492,11 @@ int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char
     if (!n_live) return fail(err, FFMOE_ERR_INVALID, "null argument");
     FF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     FF_HIP(hipMemcpy(n_live, &ctx->plan->n_live, sizeof(uint32_t), hipMemcpyDeviceToHost));
+    uint32_t faults = 0;
+    FF_HIP(hipMemcpy(&faults, &ctx->mail->faults, sizeof(uint32_t), hipMemcpyDeviceToHost));
+    if (faults)
+        return fail(err, FFMOE_ERR_RUNTIME, "%u hand-over polls of ffmoe_route_verify gave up (the launch was not resident as a whole)",
+                    faults);
     return FFMOE_OK;
 }
 

@@ -45,6 +45,15 @@ struct VerifyPlan {
     uint32_t route_valid[FFMOE_MAX_VERIFY_ROWS * 8];
 };
 
+// Hand-over words of the launch that routes and runs gate/up in one go (skinny.hip): {epoch << 32 | payload},
+// written and polled with device-coherent accesses. `epoch` starts at 1 over zeroed words and is advanced by the
+// last launch of every call that used the words; `faults` counts polls that gave up.
+struct RouteMail {
+    uint32_t epoch, faults, pad[2];
+    unsigned long long routes[FFMOE_MAX_VERIFY_ROWS * 8];                    // weight bits << 16 | expert
+    unsigned long long logits[FFMOE_MAX_VERIFY_ROWS][FFMOE_MAX_EXPERTS];     // fp32 bits
+};
+
 // Per-kernel GPU timing with HIP events on the caller's stream, switched on by ffmoe_set_profiling.
 // The counterpart of the reference's traced compute encoders (Infrastructure/Metal/GPUTrace.swift:19-115).
 struct KernelTimer {
@@ -114,6 +123,15 @@ struct RouterWeights {
     const uint16_t *per_expert_scale;  // bf16 [E] or nullptr
 };
 
+// What launch_verify needs to make the routes itself (ffmoe_route_verify).
+struct RouteFusion {
+    RouterWeights rw;
+    const uint16_t *router_x;
+    uint32_t router_x_stride;
+    float *logits;          // scratch of the two-launch router (used when the one-launch form does not apply)
+    RouteMail *mail;
+};
+
 // repack.hip
 hipError_t launch_repack_layer(hipStream_t s, const uint8_t *blobs, size_t stride, ffmoe_offsets off,
                                uint32_t n_experts, ArenaGeom g, uint8_t *arena_layer);
@@ -130,7 +148,7 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
                          VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer,
-                         bool f16 = false);
+                         bool f16 = false, const RouteFusion *route = nullptr);
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,
                                      uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d, bool f16 = false);
 

@@ -17,7 +17,9 @@
 // wave has PD KiB of weights in flight from its first instruction.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "router_sum.hpp"
 #include "stream.hpp"
+#include "topk.hpp"
 
 namespace ffmoe {
 namespace {
@@ -289,45 +291,64 @@ __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restr
 // gate/up + GELU-tanh gating, persistent. grid = (blocks); the blocks are dealt to the live experts, each
 // block walks a range of 16-row blocks of its expert; its four waves split K and meet in LDS per row block
 // (partials added in wave order), each wave finishing a quarter of the token slots.
-template <bool F16>
-__global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
-                                                                    uint32_t top_k, uint32_t n_experts,
-                                                                    const uint32_t *__restrict__ idx,
-                                                                    const uint16_t *__restrict__ w, uint32_t n_routes,
-                                                                    VerifyPlan *__restrict__ plan,
-                                                                    const uint16_t *__restrict__ x, uint32_t x_stride,
-                                                                    uint16_t *__restrict__ acts) {
-    __shared__ float s_red[2][kKSplit][8][64];
-    __shared__ PlanScratch ps;
-    // The token operand is the block's rows themselves, row min(j, rows - 1) in token column j: which expert a
-    // block serves does not matter for fetching them, so they are requested first and are there when the plan
-    // is. An expert's routes only decide which columns of the result are stored.
-    const uint32_t rows = n_routes / top_k;
-    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t j = lane & 15, jq = lane >> 4;
-    const uint32_t per = (g.gd + kKSplit - 1) / kKSplit;
-    const uint32_t g0 = min(ks * per, g.gd), g1 = min(g.gd, g0 + per), ng = g1 - g0;
-    const uint32_t g_last = g1 > g0 ? g1 - 1 : g.gd - 1;
-    uint32_t route_idx = 0;
-    uint16_t route_w = 0;
-    if (threadIdx.x < n_routes) {
-        route_idx = idx[threadIdx.x];
-        route_w = w[threadIdx.x];
-    }
-    // Load layout: four neighbouring lanes read 64 contiguous bytes of one row (row lane / 4, 8-element chunk
-    // lane % 4), 16 requests of 64 bytes per instruction; with the matrix unit's own layout (row lane % 16)
-    // every lane would be a request of its own and the 22 loads of a wave would keep the address unit busy
-    // for microseconds. The rows are turned into the operand layout (lane (j, jq): row j, chunk jq) by
-    // cross-lane moves once the weight requests are out.
+struct KSlice {
+    uint32_t g0, ng, g_last;      // first group, number of groups, last valid group of this wave's share of K
+};
+__device__ __forceinline__ KSlice k_slice(uint32_t groups, uint32_t ks) {
+    const uint32_t per = (groups + kKSplit - 1) / kKSplit;
+    const uint32_t g0 = min(ks * per, groups), g1 = min(groups, g0 + per);
+    return KSlice{g0, g1 - g0, g1 > g0 ? g1 - 1 : groups - 1};
+}
+
+// The token operand is the block's rows themselves, row min(j, rows - 1) in token column j: which expert a
+// block serves does not matter for fetching them, so they can be requested before the routes are known. An
+// expert's routes only decide which columns of the result are stored.
+// Load layout: four neighbouring lanes read 64 contiguous bytes of one row (row lane / 4, 8-element chunk
+// lane % 4), 16 requests of 64 bytes per instruction; with the matrix unit's own layout (row lane % 16)
+// every lane would be a request of its own and the 22 loads of a wave would keep the address unit busy
+// for microseconds. turn_token_rows() re-lays them into the operand layout (lane (j, jq): row j, chunk jq).
+__device__ __forceinline__ void load_token_rows(const uint16_t *__restrict__ x, uint32_t x_stride, uint32_t rows,
+                                                uint32_t lane, const KSlice &k, uint4 (&x0)[kRing], uint4 (&x1)[kRing]) {
     const uint16_t *xrow = x + (size_t)min(lane >> 2, rows - 1) * x_stride + 8 * (lane & 3);
-    uint4 x0[kRing], x1[kRing];
 #pragma unroll
     for (int u = 0; u < kRing; ++u) {
-        const bool live = (uint32_t)u < ng;
-        const uint32_t gg = min(g0 + u, g_last);
+        const bool live = (uint32_t)u < k.ng;
+        const uint32_t gg = min(k.g0 + u, k.g_last);
         x0[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup) : uint4{0, 0, 0, 0};
         x1[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
     }
+}
+
+__device__ __forceinline__ void turn_token_rows(uint32_t lane, uint4 (&x0)[kRing], uint4 (&x1)[kRing]) {
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const int pull = (int)((4 * j + jq) * 4);       // operand lane (j, jq) takes what load lane 4 j + jq holds
+    auto turn = [&](uint4 &v) {
+        v.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x);
+        v.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y);
+        v.z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z);
+        v.w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w);
+    };
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) {
+        turn(x0[u]);
+        turn(x1[u]);
+    }
+}
+
+typedef float GateUpMerge[2][kKSplit][8][64];
+
+// From the routes (thread r < n_routes brings route r) to the stored activations: the plan, the block's share of
+// its expert's row blocks, the weight stream. x0 / x1: the wave's token rows as load_token_rows() left them.
+template <bool F16>
+__device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps, const uint8_t *__restrict__ arena_layer,
+                                             const ArenaGeom &g, uint32_t top_k, uint32_t n_experts, uint32_t route_idx,
+                                             uint16_t route_w, uint32_t n_routes, VerifyPlan *__restrict__ plan,
+                                             const KSlice &k, uint4 (&x0)[kRing], uint4 (&x1)[kRing],
+                                             uint16_t *__restrict__ acts) {
+    const uint32_t rows = n_routes / top_k;
+    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint32_t g0 = k.g0, ng = k.ng, g_last = k.g_last;
     // Every block derives the routing plan itself from the (at most 128) routes: a few dozen LDS
     // operations, against a separate launch plus two dependent global reads per block. Block 0 also
     // writes the plan out for the down kernel.
@@ -354,20 +375,7 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     }
     if (plan_out) build_plan_routes(ps, n_routes, plan_out, route_expert);
     if (!has_rows) return;
-    {
-        const int pull = (int)((4 * j + jq) * 4);       // operand lane (j, jq) takes what load lane 4 j + jq holds
-        auto turn = [&](uint4 &v) {
-            v.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x);
-            v.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y);
-            v.z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z);
-            v.w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w);
-        };
-#pragma unroll
-        for (int u = 0; u < kRing; ++u) {
-            turn(x0[u]);
-            turn(x1[u]);
-        }
-    }
+    turn_token_rows(lane, x0, x1);
     // per group: the sum of its inputs per token column, once for all the tile rows this wave walks
     f32x4 sx[kRing];
 #pragma unroll
@@ -413,16 +421,173 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     }
 }
 
+template <bool F16>
+__global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                                    uint32_t top_k, uint32_t n_experts,
+                                                                    const uint32_t *__restrict__ idx,
+                                                                    const uint16_t *__restrict__ w, uint32_t n_routes,
+                                                                    VerifyPlan *__restrict__ plan,
+                                                                    const uint16_t *__restrict__ x, uint32_t x_stride,
+                                                                    uint16_t *__restrict__ acts) {
+    __shared__ GateUpMerge s_red;
+    __shared__ PlanScratch ps;
+    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    uint32_t route_idx = 0;
+    uint16_t route_w = 0;
+    if (threadIdx.x < n_routes) {
+        route_idx = idx[threadIdx.x];
+        route_w = w[threadIdx.x];
+    }
+    // the rows are requested first and are there when the plan is; no gather waits for the routing
+    const KSlice k = k_slice(g.gd, ks);
+    uint4 x0[kRing], x1[kRing];
+    load_token_rows(x, x_stride, n_routes / top_k, lane, k, x0, x1);
+    gate_up_rows<F16>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, acts);
+}
+
+// Router and gate/up of a decode step or verify block in ONE launch: the logits, the top-k select and the routes'
+// way to every block, which otherwise are two launches in front of the kernel above, become hand-overs inside it.
+// A hand-over is a 64-bit word {epoch, payload} written and polled with device-coherent accesses (relaxed atomics
+// at agent scope: the store goes through to memory, the load does not stop at this chip's non-coherent L2): a word
+// is either the old one or the new one, so a consumer needs no flag, fence or counter beside the data, and the
+// producers wait for nobody. Measured on this part, such an edge costs 0.9 us against 2.4 us for a kernel boundary.
+//   1. logits: block b takes work items b, b + grid, ... = (expert, chunk of four rows) as router_small_kernel does,
+//      same pinned order, and writes the four logits as words mail->logits[row][expert].
+//   2. select: wave 1 of block r < rows polls row r's words, runs the select and writes the row's routes as words
+//      mail->routes[row * top_k + rank] = {epoch, weight bits << 16 | expert} (and as plain idx / w for the caller and
+//      the combine).
+//   3. every block polls the routes, then continues as the kernel above. The token rows of the expert pass are
+//      requested between 1 and 3, so they arrive while the block waits.
+// The epoch is read from mail->epoch by every block at its start and is advanced by a later launch of the same call
+// (the combine), which keeps a replayed HIP graph correct. Every block of the grid has to be resident at once (the
+// grid is at most two blocks per compute unit, the kernel's occupancy); a poll gives up after 0.2 s, counts a fault
+// in mail->faults and goes on with empty routes.
+constexpr unsigned long long kPollTicks = 20000000ull;      // wall_clock64() ticks at 100 MHz
+
+__device__ __forceinline__ unsigned long long mail_load(const unsigned long long *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void mail_store(unsigned long long *p, unsigned long long v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <bool W_F32, bool F16>
+__global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
+    const uint8_t *__restrict__ arena_layer, ArenaGeom g, uint32_t top_k, uint32_t n_experts, const void *__restrict__ router_w,
+    const uint16_t *__restrict__ effective_scale, const uint16_t *__restrict__ per_expert_scale,
+    const uint16_t *__restrict__ router_x, uint32_t router_x_stride, uint32_t rows, RouteMail *__restrict__ mail,
+    uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w, VerifyPlan *__restrict__ plan,
+    const uint16_t *__restrict__ x, uint32_t x_stride, uint16_t *__restrict__ acts) {
+    __shared__ GateUpMerge s_red;
+    __shared__ PlanScratch ps;
+    float(*s_part)[kChunkTokens][64] = reinterpret_cast<float(*)[kChunkTokens][64]>(&s_red[0][0][0][0]);   // 4 KiB of the 16
+    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t epoch = __builtin_amdgcn_readfirstlane(mail->epoch);
+    const unsigned long long stamp = (unsigned long long)epoch << 32;
+    const uint32_t n_routes = rows * top_k;
+
+    // 1. logits
+    const uint32_t chunks = (rows + kChunkTokens - 1) / kChunkTokens;
+    for (uint32_t item = blockIdx.x; item < n_experts * chunks; item += gridDim.x) {
+        const uint32_t e = item % n_experts, t0 = (item / n_experts) * kChunkTokens;
+        const uint32_t t_end = min(rows, t0 + kChunkTokens);
+        float acc[kChunkTokens] = {0.f, 0.f, 0.f, 0.f};
+        accumulate_sub<W_F32, F16 ? 2 : 1>(router_w, effective_scale, router_x, router_x_stride, e, g.d, ks, lane, t0, t_end - 1, acc);
+        if (item != blockIdx.x) __syncthreads();      // the previous item's partials have been read
+#pragma unroll
+        for (int r = 0; r < kChunkTokens; ++r) s_part[ks][r][lane] = acc[r];
+        __syncthreads();
+        if (ks == 0) {
+            float mine = 0.0f;
+#pragma unroll
+            for (int r = 0; r < kChunkTokens; ++r) {
+                const float v = router_finish(s_part, r, lane);
+                if (lane == (uint32_t)r) mine = v;
+            }
+            if (lane < t_end - t0)
+                mail_store(&mail->logits[t0 + lane][e], stamp | __float_as_uint(mine));
+        }
+    }
+    // the expert pass's token rows: in flight while the routes are made
+    const KSlice k = k_slice(g.gd, ks);
+    uint4 x0[kRing], x1[kRing];
+    load_token_rows(x, x_stride, rows, lane, k, x0, x1);
+
+    const unsigned long long t_start = wall_clock64();
+    // 2. select (one wave per row)
+    if (ks == 1 && blockIdx.x < rows) {
+        const uint32_t row = blockIdx.x;
+        TopkRow tr;
+        bool ok;
+        for (;;) {
+            ok = true;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t e = c * 64 + lane;
+                unsigned long long word = stamp;     // not a candidate: valid, and below every score
+                float v = -INFINITY;
+                if (e < n_experts) {
+                    word = mail_load(&mail->logits[row][e]);
+                    v = __uint_as_float((uint32_t)word);
+                }
+                ok = ok && (uint32_t)(word >> 32) == epoch;
+                tr.key[c] = v > -INFINITY ? orderable(v) : 0u;
+            }
+            if (__all(ok)) break;
+            if (wall_clock64() - t_start > kPollTicks) {
+                if (lane == 0) atomicAdd(&mail->faults, 1u);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) tr.key[c] = 0u;      // no candidates: weights 0, nothing is routed
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        topk_select(tr, top_k, lane);
+        topk_store(tr, per_expert_scale, top_k, out_idx + (size_t)row * top_k, out_w + (size_t)row * top_k, lane, F16);
+        if (lane < top_k) {
+            // the same weight bits topk_store wrote
+            const float gain = per_expert_scale ? bf16_to_f32(per_expert_scale[tr.idx]) : 1.0f;
+            const uint32_t wbits = Act<F16>::round(tr.ex / tr.sum * gain);
+            mail_store(&mail->routes[row * top_k + lane], stamp | (wbits << 16) | (tr.idx & 0xFFFFu));
+        }
+    }
+    // 3. the routes
+    uint32_t route_idx = 0;
+    uint16_t route_w = 0;
+    if (ks * 64 < n_routes) {
+        const bool mine = threadIdx.x < n_routes;
+        for (;;) {
+            const unsigned long long word = mine ? mail_load(&mail->routes[threadIdx.x]) : stamp;
+            if (__all((uint32_t)(word >> 32) == epoch)) {
+                route_idx = (uint32_t)word & 0xFFFFu;
+                route_w = (uint16_t)((uint32_t)word >> 16);
+                break;
+            }
+            if (wall_clock64() - t_start > kPollTicks) {
+                if (lane == 0) atomicAdd(&mail->faults, 1u);
+                break;          // empty routes: weight 0 takes no part
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+    }
+    gate_up_rows<F16>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, acts);
+}
+
 // down projection with the expert's activation rows in LDS: one block = four consecutive 32-row tile rows of one
-// expert, one per wave, the whole K = F (at most kRing groups) requested at the wave's first instruction. Without
-// the rows in registers a wave fits 128 registers, so a compute unit holds sixteen waves instead of four, and it
-// is the number of waves with requests in flight, not the depth of each wave's queue, that this 55 MB stream
-// responds to: measured on the same tiles, one wave per tile row reads them in 10 us, the persistent form's 1,024
-// waves of four to five tile rows each in 15 us. Slots past the last live expert hold n = 0 and leave at once.
+// expert, one per wave, the whole K = F (at most kRing groups) requested in one go. Without the rows in registers a
+// wave fits 96 registers, so a compute unit holds twenty waves, and it is the number of waves with requests in
+// flight, not the depth of each wave's queue, that this 55 MB stream responds to: measured on the same tiles, one
+// wave per tile row reads them in 10 us, a persistent form's 1,024 waves of four to five tile rows each in 15 us.
+// With five blocks per compute unit the blocks of up to 58 live experts are all resident from the start.
+// Order of the requests: the slot's count and expert (scalar loads; a slot past the last live expert holds n = 0
+// and its block leaves before it has issued anything else), the routes, then the activation rows and only then
+// the weights - vector loads return in order, so rows requested behind 11 KiB of weights arrive after them and
+// hold the first product back until the last tile is there; in front of them every tile is consumed as it lands.
 constexpr int kDownLdsRow = kRing * kGroup * 2 + 16;      // bytes per activation row in LDS, padded against bank conflicts
+constexpr int kDownEarly = 2;      // 16-byte pieces of the activation rows a thread requests ahead of the weights (covers 5 rows)
 
 template <bool OUT_BF16, bool F16>
-__global__ __launch_bounds__(256, 4) void skinny_down_lds(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+__global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                           const VerifyPlan *__restrict__ plan,
                                                           const uint16_t *__restrict__ acts,
                                                           float *__restrict__ partials_f32,
@@ -431,13 +596,20 @@ __global__ __launch_bounds__(256, 4) void skinny_down_lds(const uint8_t *__restr
     __shared__ uint32_t s_route[kMaxRows];
     const uint32_t slot_id = blockIdx.x / parts, part = blockIdx.x % parts;
     const PlanSlot &slot = plan->slots[slot_id];
-    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t j = lane & 15, jq = lane >> 4;
-    // count, expert and the route list come back in one round trip (entries past the count are stale: unused)
     const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
     const uint32_t expert = __builtin_amdgcn_readfirstlane(slot.expert);
-    const uint32_t route_t = threadIdx.x < (uint32_t)kMaxRows ? slot.routes[threadIdx.x] : 0u;
     if (n == 0) return;
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint32_t chunks = g.f / 8;                       // 16-byte pieces per row
+    const uint32_t route_t = threadIdx.x < (uint32_t)kMaxRows ? slot.routes[threadIdx.x] : 0u;
+    uint4 early[kDownEarly];
+#pragma unroll
+    for (int k = 0; k < kDownEarly; ++k) {
+        const uint32_t i = threadIdx.x + 256u * k, r = i / chunks, c = i % chunks;
+        // rows past the count re-read the last one (never stored): no load sits behind a branch
+        early[k] = *reinterpret_cast<const uint4 *>(acts + (size_t)slot.routes[min(r, n - 1)] * g.f + c * 8);
+    }
     const uint32_t rb = part * 4 + wave;
     const bool has_row = rb < g.dn_rbp;
     const uint8_t *expert_base = arena_layer + (size_t)expert * g.expert_bytes;
@@ -450,15 +622,21 @@ __global__ __launch_bounds__(256, 4) void skinny_down_lds(const uint8_t *__restr
         for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb * ng + min((uint32_t)u, g_last), lane);
     }
     if (threadIdx.x < (uint32_t)kMaxRows) s_route[threadIdx.x] = threadIdx.x < n ? route_t : 0u;
-    __syncthreads();
-    // the n activation rows, 16 bytes per thread and turn, contiguous along a row
-    const uint32_t chunks = g.f / 8;                       // 16-byte pieces per row
-    for (uint32_t i = threadIdx.x; i < n * chunks; i += 256) {
-        const uint32_t r = i / chunks, c = i % chunks;
-        *reinterpret_cast<uint4 *>(s_act + r * kDownLdsRow + c * 16) =
-            *reinterpret_cast<const uint4 *>(acts + (size_t)s_route[r] * g.f + c * 8);
+#pragma unroll
+    for (int k = 0; k < kDownEarly; ++k) {
+        const uint32_t i = threadIdx.x + 256u * k, r = i / chunks, c = i % chunks;
+        if (r < n) *reinterpret_cast<uint4 *>(s_act + r * kDownLdsRow + c * 16) = early[k];
     }
-    __syncthreads();
+    if (n * chunks > 256u * kDownEarly) {
+        // an expert with many rows: the remaining pieces, 16 bytes per thread and turn (these do queue behind the weights)
+        lds_barrier();
+        for (uint32_t i = threadIdx.x + 256u * kDownEarly; i < n * chunks; i += 256) {
+            const uint32_t r = i / chunks, c = i % chunks;
+            *reinterpret_cast<uint4 *>(s_act + r * kDownLdsRow + c * 16) =
+                *reinterpret_cast<const uint4 *>(acts + (size_t)s_route[r] * g.f + c * 8);
+        }
+    }
+    lds_barrier();      // LDS only: the weight tiles stay in flight across it
     if (!has_row) return;
     // token slot j of the operand: row j of the expert's list, row 0 again past the count (columns never stored)
     const uint8_t *xrow = s_act + (j < n ? j : 0u) * kDownLdsRow + jq * 16;
@@ -475,7 +653,7 @@ __global__ __launch_bounds__(256, 4) void skinny_down_lds(const uint8_t *__restr
         ring_step<F16, false>(ring, u, live, x0, x1, sx, tot, src, 0u, lane);
         // The running sums are pinned here: left alone, the compiler sinks the scale-and-bias arithmetic of every
         // group into the branches of the stores at the end and carries all eleven groups' matrix results there,
-        // which does not fit 128 registers.
+        // which does not fit the register budget.
 #pragma unroll
         for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(tot.a[r]), "+v"(tot.b[r]));
     }
@@ -611,8 +789,9 @@ __global__ __launch_bounds__(512, 1) void decode_down_combine_kernel(const uint8
                                                                      const uint16_t *__restrict__ w,
                                                                      const uint16_t *__restrict__ acts,
                                                                      const uint16_t *__restrict__ residual,
-                                                                     uint16_t *__restrict__ y) {
+                                                                     uint16_t *__restrict__ y, RouteMail *mail) {
     __shared__ float s_row[8][2 * kTileRows];
+    if (mail && blockIdx.x == 0 && threadIdx.x == 0) mail->epoch += 1;      // the routing launch of this call has read it
     __shared__ float s_w[8];
     const uint32_t lane = threadIdx.x & 63, r = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t rb = blockIdx.x, j = lane & 15, jq = lane >> 4;
@@ -676,8 +855,9 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                                                       const uint16_t *__restrict__ w,
                                                       const VerifyPlan *__restrict__ plan,
                                                       const uint16_t *__restrict__ residual, uint32_t top_k,
-                                                      uint32_t d, uint16_t *__restrict__ y) {
+                                                      uint32_t d, uint16_t *__restrict__ y, RouteMail *mail) {
     const uint32_t tok = blockIdx.y;
+    if (mail && blockIdx.x == 0 && tok == 0 && threadIdx.x == 0) mail->epoch += 1;      // the routing launch of this call has read it
     const uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (c >= d) return;
     // every load of the thread is requested before the first is used: the routes' weights and experts, then
@@ -740,7 +920,18 @@ template <bool F16>
 hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
                             const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
                             const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16, VerifyPlan *plan, uint16_t *acts,
-                            float *partials_f32, uint32_t n_cus, KernelTimer *timer) {
+                            float *partials_f32, uint32_t n_cus, KernelTimer *timer, const RouteFusion *route) {
+    // `route`: the routes are not there yet - idx / w are where this call has to write them. One launch does the
+    // router and gate/up when the expert fits the persistent kernel, the combine follows in this call (it advances
+    // the epoch) and the router rows are 8-byte aligned; otherwise the router's own two launches go first.
+    const bool fits_ring = (g.gd + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
+    const bool fuse = route && fits_ring && y && !partials_bf16 && top_k <= 8 && n_experts <= FFMOE_MAX_EXPERTS &&
+                      reinterpret_cast<uintptr_t>(route->router_x) % 8 == 0 && route->router_x_stride % 4 == 0;
+    if (route && !fuse) {
+        const hipError_t e = launch_router(s, route->rw, route->router_x, route->router_x_stride, t, n_experts, g.d, top_k,
+                                           route->logits, const_cast<uint32_t *>(idx), const_cast<uint16_t *>(w), timer, F16);
+        if (e != hipSuccess) return e;
+    }
     timer->begin(s);
     const uint32_t slots = min(n_experts, t * top_k);
     // the persistent kernels hold a K-slice of kRing groups per wave; larger experts take the one-shot grids
@@ -748,7 +939,17 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     const bool dn_whole = g.gf <= (uint32_t)kRing;                                     // a wave holds all of K
     const bool dn_ksplit = !dn_whole && (g.gf + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
     const uint32_t resident = 2 * n_cus;       // blocks the chip holds at once (__launch_bounds__(256, 2))
-    if (gu_persistent) {
+    if (fuse) {
+        // at least one block per row (its second wave selects the row's routes), at most what is resident at once
+        const uint32_t blocks = min(resident, max(max(slots, t), min(resident, slots * g.gu_rb)));
+#define FFMOE_ROUTE_GU(WF)                                                                                                  \
+    hipLaunchKernelGGL((route_gate_up_persistent<WF, F16>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, \
+                       route->rw.w, route->rw.effective_scale, route->rw.per_expert_scale, route->router_x,                  \
+                       route->router_x_stride, t, route->mail, const_cast<uint32_t *>(idx), const_cast<uint16_t *>(w), plan, \
+                       x, x_stride, acts)
+        if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true); else FFMOE_ROUTE_GU(false);
+#undef FFMOE_ROUTE_GU
+    } else if (gu_persistent) {
         // plan slot of the profile stays empty: the gate/up kernel builds the plan itself
         const uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
         hipLaunchKernelGGL(skinny_gate_up_persistent<F16>, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, idx,
@@ -761,11 +962,12 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    timer->mark(s, FFMOE_K_GATE_UP);
+    timer->mark(s, fuse ? FFMOE_K_ROUTE_GATE_UP : FFMOE_K_GATE_UP);
+    RouteMail *const mail = fuse ? route->mail : nullptr;
     if (t == 1 && dn_whole && !partials_bf16 && top_k <= 8) {
         // a decode step: down projection and combine in one launch (its time sits in the down slot)
         hipLaunchKernelGGL(decode_down_combine_kernel<F16>, dim3(g.dn_rbp), dim3(512), 0, s, arena_layer, g, n_experts, top_k, idx,
-                           w, acts, residual, y);
+                           w, acts, residual, y, mail);
         timer->mark(s, FFMOE_K_DOWN);
         timer->finish();
         return hipGetLastError();
@@ -796,7 +998,7 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_DOWN);
     hipLaunchKernelGGL(combine_kernel<F16>, dim3((g.d / 4 + 255) / 256, t), dim3(256), 0, s, partials_f32, w, plan, residual,
-                       top_k, g.d, y);
+                       top_k, g.d, y, mail);
     timer->mark(s, FFMOE_K_COMBINE);
     timer->finish();
     return hipGetLastError();
@@ -808,11 +1010,12 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
-                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer, bool f16) {
+                         VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer, bool f16,
+                         const RouteFusion *route) {
     return f16 ? launch_verify_as<true>(s, arena_layer, g, n_experts, top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                                        plan, acts, partials_f32, n_cus, timer)
+                                        plan, acts, partials_f32, n_cus, timer, route)
                : launch_verify_as<false>(s, arena_layer, g, n_experts, top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                                         plan, acts, partials_f32, n_cus, timer);
+                                         plan, acts, partials_f32, n_cus, timer, route);
 }
 
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,

@@ -54,7 +54,7 @@ EXPORTS = [
 
 PROFILE_SLOTS = 16
 KERNEL_NAMES = ["router_logits", "router_topk", "plan", "gate_up", "down", "combine", "prefill_sort",
-                "prefill_gate_up", "prefill_down", "prefill_combine", "gemv", "argmax", "event_gap", "reserved13",
+                "prefill_gate_up", "prefill_down", "prefill_combine", "gemv", "argmax", "event_gap", "route_gate_up",
                 "reserved14", "reserved15"]
 
 

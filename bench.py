@@ -171,11 +171,20 @@ def main():
     px, pidx, pw, py = (C.c_void_p(t_.data_ptr()) for t_ in (x, idx, w, y))
     err = C.c_char_p()
 
-    def step(layer):
+    def step_split(layer):
         rc = Lib.ffmoe_router(h, stream, layer, px, D, T, pidx, pw, None, C.byref(err))
         rc |= Lib.ffmoe_verify(h, stream, layer, px, D, T, pidx, pw, None, py, C.byref(err))
         if rc:
             raise RuntimeError(err.value)
+
+    def step(layer):
+        # router and expert pass of the block in one call (router logits, select and gate/up share a launch)
+        rc = Lib.ffmoe_route_verify(h, stream, layer, px, D, px, D, T, None, py, pidx, pw, C.byref(err))
+        if rc:
+            raise RuntimeError(err.value)
+
+    if os.environ.get("FFMOE_BENCH_SPLIT"):
+        step = step_split
 
     # distinct experts per layer for this block (decides the algorithmic bytes of each step)
     live = []
@@ -240,18 +249,18 @@ def main():
     def kernel_times(pr):
         return {k_: round((v[0] / v[1] - gap_ms) * 1e3, 2) for k_, v in pr.items() if k_ != "event_gap"}
     kernel_us = kernel_times(prof)
-    gu_ms = prof["gate_up"][0] - gap_ms * prof["gate_up"][1]
     live_sum = sum(live[i % L] for i in range(args.steps))
-    if "down" in prof:
-        # two launches: gate/up is the dominant kernel
-        dominant = "skinny_gate_up_persistent"
-        achieved = live_sum * GATE_UP_BYTES / (gu_ms * 1e-3) / 1e9
-        down_gbs = live_sum * DOWN_BYTES / ((prof["down"][0] - gap_ms * prof["down"][1]) * 1e-3) / 1e9
+    if "route_gate_up" in prof:
+        # router logits, select and gate/up share one launch: its bytes are the live experts' gate/up weights plus the
+        # router's [E][D] bf16 matrix, its time holds the routing chain as well
+        dominant = "route_gate_up_persistent (router logits + top-8 select + gate/up in one launch)"
+        gu_ms = prof["route_gate_up"][0] - gap_ms * prof["route_gate_up"][1]
+        achieved = (live_sum * GATE_UP_BYTES + args.steps * E * D * 2) / (gu_ms * 1e-3) / 1e9
     else:
-        # gate/up and down share one launch (its time sits in the gate_up slot): all expert bytes
-        dominant = "skinny_gate_up_persistent<1> (gate/up + down in one launch)"
-        achieved = live_sum * EXPERT_BYTES / (gu_ms * 1e-3) / 1e9
-        down_gbs = None
+        dominant = "skinny_gate_up_persistent"
+        gu_ms = prof["gate_up"][0] - gap_ms * prof["gate_up"][1]
+        achieved = live_sum * GATE_UP_BYTES / (gu_ms * 1e-3) / 1e9
+    down_gbs = live_sum * DOWN_BYTES / ((prof["down"][0] - gap_ms * prof["down"][1]) * 1e-3) / 1e9
 
     # secondary figures: decode step (T = 1) and config-1 GEMV
     extra = {"event_record_us": round(gap_ms * 1e3, 2)}
@@ -259,8 +268,8 @@ def main():
     px1 = C.c_void_p(x1.data_ptr())
 
     def decode(layer):
-        Lib.ffmoe_router(h, stream, layer, px1, D, 1, pidx, pw, None, C.byref(err))
-        Lib.ffmoe_verify(h, stream, layer, px1, D, 1, pidx, pw, None, py, C.byref(err))
+        # two launches: router + select + gate/up, then down + combine
+        Lib.ffmoe_route_verify(h, stream, layer, px1, D, px1, D, 1, None, py, pidx, pw, C.byref(err))
 
     if not args.no_decode:
         for name_, fn_ in (("decode_us_per_layer", decode),):
@@ -365,8 +374,7 @@ def main():
         pxh, pwh, pyh = (C.c_void_p(t_.data_ptr()) for t_ in (xh, wh, yh))
 
         def step16(layer, rows):
-            rc = Lib.ffmoe_router(h, stream, layer, pxh, D, rows, pidx, pwh, None, C.byref(err))
-            rc |= Lib.ffmoe_verify(h, stream, layer, pxh, D, rows, pidx, pwh, None, pyh, C.byref(err))
+            rc = Lib.ffmoe_route_verify(h, stream, layer, pxh, D, pxh, D, rows, None, pyh, pidx, pwh, C.byref(err))
             if rc:
                 raise RuntimeError(err.value)
         fp16 = {}
@@ -521,8 +529,7 @@ def main():
                     ev_join.record(side_s)
             else:
                 dense.dense_ffn(i % LS, outs_b[0], out=h1_b)
-            rc = Lib.ffmoe_router(h, stream, layer, pouts[2], D, T, pidx, pw, None, C.byref(err))
-            rc |= Lib.ffmoe_verify(h, stream, layer, pouts[1], D, T, pidx, pw, None, py, C.byref(err))
+            rc = Lib.ffmoe_route_verify(h, stream, layer, pouts[2], D, pouts[1], D, T, None, py, pidx, pw, C.byref(err))
             if rc:
                 raise RuntimeError(err.value)
             if concurrent:
@@ -718,10 +725,10 @@ def main():
         "device": device_info,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": traffic.get("verify16_gate_up") if (T == 16 and L == 30 and "down" in prof) else None,
+                     "traffic": traffic.get("verify16_route_gate_up" if "route_gate_up" in prof else "verify16_gate_up") if (T == 16 and L == 30) else None,
                      "traffic_unit": f"bytes per launch (rocprofv3 --pmc, profiles/{TRAFFIC_FILE.name})",
-                     "algorithmic_bytes_per_launch": int(live_sum / args.steps * GATE_UP_BYTES),
-                     "avg_kernel_us": kernel_us.get("gate_up")},
+                     "algorithmic_bytes_per_launch": int(achieved * 1e9 * gu_ms * 1e-3 / args.steps),
+                     "avg_kernel_us": round(gu_ms * 1e3 / args.steps, 2)},
         "kernel_us": kernel_us,
         "down_kernel_GBs": None if down_gbs is None else round(down_gbs, 1),
         "prefill_tok_s": prefill["tok_per_s"] if prefill else None,

@@ -172,16 +172,23 @@ int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const ui
                           uint16_t *partials, char **err);
 
 /* Router and expert pass of one block in one call, for the decode loop that never shows the routes to
- * the host: ffmoe_router followed by ffmoe_verify on the same stream, with the selected routes also
- * written to out_idx / out_w ([t][top_k], device). Replaces the pair MoE.encodeRouterGemma4 +
- * encodeRoutedPersistentGPUSlots (Kernels/MoE/MoE.swift:168-247,454-496), where the GPU routes the
- * persistent kernels without a host round trip. */
+ * the host: the results of ffmoe_router followed by ffmoe_verify on the same stream, bit for bit, with the
+ * selected routes also written to out_idx / out_w ([t][top_k], device). Replaces the pair
+ * MoE.encodeRouterGemma4 + encodeRoutedPersistentGPUSlots (Kernels/MoE/MoE.swift:168-247,454-496), where
+ * the GPU routes the persistent kernels without a host round trip.
+ * When the expert fits the persistent kernels and the router rows are 8-byte aligned, the router logits, the
+ * select and gate/up run as ONE launch (a decode step is two launches, a verify block three): the blocks
+ * hand logits and routes to each other through epoch-stamped words in device memory, which needs every
+ * block of that launch resident at once - the grid is sized for a GPU this stream has to itself. A block
+ * that waits 0.2 s for a word gives up, the call's output is then undefined and the next
+ * ffmoe_last_live_experts on the context reports FFMOE_ERR_RUNTIME. */
 int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *router_x,
                        uint32_t router_x_stride, const uint16_t *x, uint32_t x_stride, uint32_t t,
                        const uint16_t *residual, uint16_t *y, uint32_t *out_idx, uint16_t *out_w, char **err);
 
 /* Number of distinct experts the last ffmoe_verify* call on `stream` ran (reads back 4 bytes; waits
- * for the stream). For reporting only. */
+ * for the stream). For reporting only. FFMOE_ERR_RUNTIME if a launch of ffmoe_route_verify on this
+ * context ever gave up waiting for its own blocks (see there). */
 int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char **err);
 
 /* ---- routed experts, prefill chunk (t <= max_tokens) ------------------------------------------- */
@@ -378,6 +385,7 @@ enum {
     FFMOE_K_COMBINE, FFMOE_K_PREFILL_SORT, FFMOE_K_PREFILL_GATE_UP, FFMOE_K_PREFILL_DOWN,
     FFMOE_K_PREFILL_COMBINE, FFMOE_K_GEMV, FFMOE_K_ARGMAX,
     FFMOE_K_EVENT_GAP, /* two event records with nothing between them: what an event pair adds to every slot above */
+    FFMOE_K_ROUTE_GATE_UP, /* ffmoe_route_verify: router logits, select and gate/up in one launch */
     FFMOE_PROFILE_SLOTS = 16
 };
 typedef struct {

@@ -10,7 +10,12 @@ from helpers import bf16_tensor, bits_of, make_layer, to_ff_offsets
 pytestmark = pytest.mark.gpu
 
 
-def test_router_verify_and_dense_chain_in_a_graph(oracle):
+@pytest.mark.parametrize("one_call", [False, True], ids=["router_then_verify", "route_verify"])
+def test_router_verify_and_dense_chain_in_a_graph(oracle, one_call):
+    """`route_verify`: the router, the select and gate/up share one launch whose blocks hand the logits and routes
+    to each other through words stamped with an epoch that lives in device memory and is advanced by the call's
+    last launch - a replayed graph (same kernel arguments every time) and eager calls in between must still never
+    take a previous call's words for this call's."""
     import torch
     import fieldfare_moe as ff
     ff.lib()
@@ -39,10 +44,15 @@ def test_router_verify_and_dense_chain_in_a_graph(oracle):
         for layer in range(layers):
             ctx.post_attn_setup(hidden, x, ws[0], ws[1], ws[2], out=outs)
             dense.dense_ffn(layer, outs[0], out=h1)
-            i_, w_ = ctx.router(layer, outs[2])
-            idx.copy_(i_)
-            w.copy_(w_)
-            ctx.verify(layer, outs[1], idx, w, out=h2)
+            if one_call:
+                _, i_, w_ = ctx.route_verify(layer, outs[2], outs[1], out=h2)
+                idx.copy_(i_)
+                w.copy_(w_)
+            else:
+                i_, w_ = ctx.router(layer, outs[2])
+                idx.copy_(i_)
+                w.copy_(w_)
+                ctx.verify(layer, outs[1], idx, w, out=h2)
             ctx.layer_tail(h2, h1, hidden, ws[3], ws[4], 0.9)
 
     chain()
@@ -70,7 +80,11 @@ def test_router_verify_and_dense_chain_in_a_graph(oracle):
         assert np.array_equal(bits_of(hidden), eager), f"replay {replay}"
         # eager work of the same contexts between replays
         ctx.verify(replay % layers, x, idx, w)
+        if one_call:
+            for _ in range(replay + 1):     # moves the epoch by a different amount before every replay
+                ctx.route_verify(replay % layers, x, x)
         dense.dense_ffn(replay % layers, x)
         torch.cuda.synchronize()
+    assert ctx.last_live_experts() > 0      # also raises if a hand-over poll of route_verify ever gave up
     ctx.close()
     dense.close()
