@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -22,6 +23,8 @@ struct ffmoe_layer {
     int router_is_f32 = 0;
     uint16_t *effective_scale = nullptr;
     uint16_t *per_expert_scale = nullptr;
+    void *router_frag = nullptr;    // bf16 router weights in matrix-operand order (the prefill router's approximate pass)
+    float router_norm_max = 0.0f;   // upper bound of the largest 2-norm of an expert's router row
 };
 
 // A resident matrix: the re-tiled copy of one [m][n] INT4 weight plus the scratch of its greedy choice.
@@ -170,7 +173,7 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     const uint32_t router_rows = shape->max_tokens > FFMOE_MAX_VERIFY_ROWS ? shape->max_tokens : FFMOE_MAX_VERIFY_ROWS;
     const size_t routes = (size_t)FFMOE_MAX_VERIFY_ROWS * shape->top_k;
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&ctx->arena), ctx->layer_bytes * shape->n_layers);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->logits), (size_t)router_rows * shape->n_experts * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->logits), ((size_t)router_rows * shape->n_experts + router_rows + 64) * sizeof(float));      // logits, and the squared row norms in front of the approximate ones
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->plan), sizeof(VerifyPlan));
     if (e == hipSuccess) e = hipMemset(ctx->plan, 0, sizeof(VerifyPlan));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->mail), sizeof(RouteMail));
@@ -218,6 +221,7 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     (void)hipDeviceSynchronize();
     for (auto &l : ctx->layers) {
         if (l.router_w) (void)hipFree(l.router_w);
+        if (l.router_frag) (void)hipFree(l.router_frag);
         if (l.effective_scale) (void)hipFree(l.effective_scale);
         if (l.per_expert_scale) (void)hipFree(l.per_expert_scale);
     }
@@ -348,6 +352,26 @@ int ffmoe_upload_router_bf16(ffmoe_ctx *ctx, uint32_t layer, const uint16_t *w, 
     if (int rc = upload_vec(&dw, w, n, err)) return rc;
     l.router_w = dw;
     l.router_is_f32 = 0;
+    if (l.router_frag) { (void)hipFree(l.router_frag); l.router_frag = nullptr; }
+    if (ctx->shape.d % 32 == 0 && ctx->shape.n_experts % 16 == 0) {
+        // the prefill router's approximate pass reads the weights in matrix-operand order and bounds its error with
+        // the largest row norm (rounded up)
+        double worst = 0.0;
+        for (uint32_t e = 0; e < ctx->shape.n_experts; ++e) {
+            double sum = 0.0;
+            for (uint32_t k = 0; k < ctx->shape.d; ++k) {
+                const uint32_t bits = (uint32_t)w[(size_t)e * ctx->shape.d + k] << 16;
+                float v;
+                memcpy(&v, &bits, sizeof v);
+                sum += (double)v * (double)v;
+            }
+            if (!(sum <= worst)) worst = sum;       // a NaN or infinite row makes the bound non-finite: every expert becomes a candidate
+        }
+        l.router_norm_max = (float)(std::sqrt(worst) * (1.0 + 1e-6));
+        FF_HIP(hipMalloc(&l.router_frag, n * sizeof(uint16_t)));
+        FF_HIP(launch_router_fragments(nullptr, dw, ctx->shape.n_experts, ctx->shape.d, l.router_frag));
+        FF_HIP(hipDeviceSynchronize());
+    }
     if (int rc = upload_vec(&l.effective_scale, effective_scale, ctx->shape.d, err)) return rc;
     return upload_vec(&l.per_expert_scale, per_expert_scale, ctx->shape.n_experts, err);
 }
@@ -377,6 +401,7 @@ int ffmoe_upload_router_int8(ffmoe_ctx *ctx, uint32_t layer, const uint8_t *w, c
     if (int rc = upload_vec(&dw, deq.data(), deq.size(), err)) return rc;
     l.router_w = dw;
     l.router_is_f32 = 1;
+    if (l.router_frag) { (void)hipFree(l.router_frag); l.router_frag = nullptr; }
     if (int rc = upload_vec(&l.effective_scale, effective_scale, d, err)) return rc;
     return upload_vec(&l.per_expert_scale, per_expert_scale, e_count, err);
 }
@@ -405,10 +430,11 @@ int ffmoe_router(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *r
     const uint32_t cap = ctx->shape.max_tokens > FFMOE_MAX_VERIFY_ROWS ? ctx->shape.max_tokens : FFMOE_MAX_VERIFY_ROWS;
     if (!out_logits && t > cap) return fail(err, FFMOE_ERR_INVALID, "t = %u exceeds max_tokens = %u", t, cap);
     const ffmoe_layer &l = ctx->layers[layer];
-    RouterWeights rw{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale};
+    RouterWeights rw{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale,
+                     static_cast<const uint4 *>(l.router_frag), l.router_norm_max};
     FF_HIP(launch_router(static_cast<hipStream_t>(stream), rw, router_x, x_stride, t, ctx->shape.n_experts,
                          ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w, &ctx->timer,
-                         ctx->f16));
+                         ctx->f16, out_logits != nullptr, ctx->logits));
     return FFMOE_OK;
 }
 

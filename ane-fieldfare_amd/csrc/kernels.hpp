@@ -121,6 +121,8 @@ struct RouterWeights {
     int w_is_f32;
     const uint16_t *effective_scale;   // bf16 [D] or nullptr
     const uint16_t *per_expert_scale;  // bf16 [E] or nullptr
+    const uint4 *w_frag = nullptr;     // bf16 weights in matrix-operand order (router.hip), or nullptr
+    float w_norm_max = 0.0f;           // an upper bound of the largest 2-norm of an expert's row
 };
 
 // What launch_verify needs to make the routes itself (ffmoe_route_verify).
@@ -141,7 +143,10 @@ hipError_t launch_dequant_expert(hipStream_t s, const uint8_t *arena_expert, Are
 // router.hip
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w, KernelTimer *timer, bool f16 = false);
+                         uint16_t *out_w, KernelTimer *timer, bool f16 = false, bool want_logits = true,
+                         float *scratch = nullptr);
+// `frag`: E * d bf16 values, the weights in matrix-operand order (needs d % 32 == 0 and E % 16 == 0)
+hipError_t launch_router_fragments(hipStream_t s, const uint16_t *w, uint32_t n_experts, uint32_t d, void *frag);
 
 // skinny.hip
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,

@@ -191,11 +191,239 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, co
               out_w + (size_t)tok * top_k, threadIdx.x, w_f16);
 }
 
+
+// ---------------------------------------------------------------------------------------------------
+// Prefill router, fast form: the same routes and weights, bit for bit, without the pinned fp32 sums of all
+// E logits per token. The pinned order makes the logits a vector-ALU GEMM (2.2 GFLOP at 3,072 tokens: 31 us of
+// fma alone); only the selected experts' logits have to be the pinned ones.
+//   1. router_approx_kernel: every logit on the matrix unit (bf16 products are exact, the fp32 sum runs in
+//      whatever order the unit uses), plus the squared norm of every row.
+//   2. router_exact_topk_kernel, one wave per token: with a_e the approximate, p_e the pinned logit and
+//      B >= |a_e - L_e|, |p_e - L_e| for the real-number sum L_e (B = gamma * ||x|| * max_e ||w_e||, gamma = d * 2^-22:
+//      any summation order of d exact products with roundings of at most 2^-23 relative, twice over), an expert
+//      among the pinned top k has a_e >= v_k - 4 B, v_k the k-th largest approximate logit: were a_e below that,
+//      the k experts with a >= v_k would all have p >= a - 2 B > a_e + 2 B >= p_e. The wave computes the pinned logit
+//      of every expert above that threshold (a dozen at 128 experts) and selects among them with the same code as
+//      the other router kernels. A row with a non-finite value anywhere takes every expert as a candidate.
+// Needs: bf16 rows and weights, no per-input scale, d a multiple of 256 up to 4096, E a multiple of 16 up to 128
+// (the sixteen waves of the approximate pass hold two 16-expert fragments each).
+// ---------------------------------------------------------------------------------------------------
+constexpr int kApproxTok = 16;          // token rows per block of the approximate pass
+constexpr int kMaxFrags = FFMOE_MAX_EXPERTS / 16;
+
+// Router weights in matrix-operand order: frag[(h * E/16 + n) * 64 + lane] = the eight values
+// w[16 n + lane % 16][32 h + 8 (lane / 16) .. + 7], so that a wave's operand load is 1 KiB contiguous.
+__global__ __launch_bounds__(256) void router_frag_kernel(const uint16_t *__restrict__ w, uint32_t n_experts, uint32_t d,
+                                                          uint4 *__restrict__ frag) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x, lane = i & 63, piece = i >> 6;
+    const uint32_t nfrag = n_experts / 16, n = piece % nfrag, h = piece / nfrag;
+    if (h >= d / 32) return;
+    frag[i] = *reinterpret_cast<const uint4 *>(w + (size_t)(16 * n + (lane & 15)) * d + 32 * h + 8 * (lane >> 4));
+}
+
+// One block = 16 token rows x all experts, sixteen waves: wave (kq, nq) takes a quarter of K and a quarter of the
+// experts' 16-column fragments (NF of them), with four k-steps of operands in flight - the pass is a chain of
+// round trips to the weights (every block reads all of them once), so it is the number of loads in flight that
+// sets its time. The loop body has no branch: the compiler then counts the loads in flight exactly and waits for the
+// oldest step only (behind a branch it waits for all of them, and the pass is one round trip per step).
+constexpr int kApproxWaves = 16, kApproxDepth = 4;
+
+template <int NF>
+__global__ __launch_bounds__(64 * kApproxWaves) void router_approx_kernel(const uint4 *__restrict__ wfrag,
+                                                                           const uint16_t *__restrict__ x, uint32_t x_stride,
+                                                                           uint32_t t, uint32_t n_experts, uint32_t d,
+                                                                           float *__restrict__ approx, float *__restrict__ xnorm2) {
+    __shared__ float s_acc[4][4 * NF][4][64];       // [K quarter][fragment][value][lane]
+    __shared__ float s_x2[4][16];
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t kq = wave & 3, nq = wave >> 2;
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint32_t t0 = blockIdx.x * kApproxTok, nfrag = n_experts / 16, nh = d / 32;
+    const uint32_t h0 = kq * nh / 4, h1 = (kq + 1) * nh / 4, span = h1 - h0;
+    const uint32_t n0 = nq * NF;                       // this wave's fragments: n0 .. n0 + NF - 1 (those below nfrag)
+    // the rows are loaded four neighbouring lanes per 64 contiguous bytes (row lane / 4, chunk lane % 4: 16 requests per
+    // instruction instead of 64) and turned into the operand layout (lane (j, jq): row j, chunk jq) by cross-lane moves
+    const uint16_t *xr = x + (size_t)min(t0 + (lane >> 2), t - 1) * x_stride + 8 * (lane & 3);
+    const int pull = (int)((4 * j + jq) * 4);
+    const uint4 *wf = wfrag + lane;
+    f32x4 acc[NF];
+#pragma unroll
+    for (int n = 0; n < NF; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float x2 = 0.0f;
+    uint4 a_q[kApproxDepth], b_q[kApproxDepth][NF];
+    // step i of this wave = k-step h0 + i; past the end it repeats the last step and enters with a zero row
+    auto fetch = [&](int slot, uint32_t i) {
+        const uint32_t h = h0 + min(i, span - 1);
+        a_q[slot] = *reinterpret_cast<const uint4 *>(xr + 32 * h);
+#pragma unroll
+        for (int n = 0; n < NF; ++n) b_q[slot][n] = wf[((size_t)h * nfrag + min(n0 + n, nfrag - 1)) * 64];
+    };
+    if (span) {
+#pragma unroll
+        for (int u = 0; u < kApproxDepth; ++u) fetch(u, u);
+        for (uint32_t ib = 0; ib < span; ib += kApproxDepth) {
+#pragma unroll
+            for (int u = 0; u < kApproxDepth; ++u) {
+                uint4 a = a_q[u];
+                uint4 b[NF];
+#pragma unroll
+                for (int n = 0; n < NF; ++n) b[n] = b_q[u][n];
+                fetch(u, ib + u + kApproxDepth);
+                a.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a.x);
+                a.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a.y);
+                a.z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a.z);
+                a.w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a.w);
+                if (ib + u >= span) a = uint4{0, 0, 0, 0};
+                const uint32_t aw[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float lo = bf16lo_to_f32(aw[q]), hi = bf16hi_to_f32(aw[q]);
+                    x2 = __builtin_fmaf(lo, lo, x2);
+                    x2 = __builtin_fmaf(hi, hi, x2);
+                }
+#pragma unroll
+                for (int n = 0; n < NF; ++n) acc[n] = Act<false>::mfma(a, b[n], acc[n]);
+            }
+        }
+    }
+    // the row's squares: the four k-chunk lanes of a row, then the four K quarters
+    x2 += __shfl_xor(x2, 16, 64);
+    x2 += __shfl_xor(x2, 32, 64);
+    if (nq == 0 && jq == 0) s_x2[kq][j] = x2;
+#pragma unroll
+    for (int n = 0; n < NF; ++n)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s_acc[kq][n0 + n][r][lane] = acc[n][r];
+    __syncthreads();
+    if (wave == 0 && lane < 16 && t0 + lane < t)
+        xnorm2[t0 + lane] = (s_x2[0][lane] + s_x2[1][lane]) + (s_x2[2][lane] + s_x2[3][lane]);
+    // fragment n is finished by wave n (the lane holds tokens 4 jq .. + 3 of expert column j)
+    for (uint32_t n = wave; n < nfrag; n += kApproxWaves) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float v = (s_acc[0][n][r][lane] + s_acc[1][n][r][lane]) + (s_acc[2][n][r][lane] + s_acc[3][n][r][lane]);
+            const uint32_t tok = t0 + 4 * jq + r;
+            if (tok < t) approx[(size_t)tok * n_experts + 16 * n + j] = v;
+        }
+    }
+}
+
+constexpr int kExactSteps = 4;          // d <= 4096: k = 1024 i + 256 s + 4 lane + j, i < 4
+
+// STEPS: 1024-wide steps of the pinned order that d needs; CHUNK: candidates whose rows are requested together.
+template <int STEPS, int CHUNK>
+__global__ __launch_bounds__(256, 3) void router_exact_topk_kernel(const uint16_t *__restrict__ w, const uint16_t *__restrict__ x,
+                                                                   uint32_t x_stride, uint32_t t, uint32_t n_experts, uint32_t d,
+                                                                   uint32_t top_k, const float *__restrict__ approx,
+                                                                   const float *__restrict__ xnorm2, float w_norm_max,
+                                                                   const uint16_t *__restrict__ per_expert_scale,
+                                                                   uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w) {
+    const uint32_t lane = threadIdx.x & 63, tok = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tok >= t) return;
+    // the token's row, as the pinned order walks it: element j of (step i, sub-accumulator s) = x[1024 i + 256 s + 4 lane + j]
+    const uint16_t *xr = x + (size_t)tok * x_stride;
+    float xf[STEPS][4][4];
+    {
+        uint2 xraw[STEPS][4];
+#pragma unroll
+        for (int i = 0; i < STEPS; ++i)
+#pragma unroll
+            for (int s_ = 0; s_ < 4; ++s_) {
+                // d is a multiple of 256: a (step, sub-accumulator) pair is inside the row for every lane or for none
+                const uint32_t k = 1024 * i + 256 * s_;
+                xraw[i][s_] = k < d ? *reinterpret_cast<const uint2 *>(xr + k + 4 * lane) : make_uint2(0u, 0u);
+            }
+#pragma unroll
+        for (int i = 0; i < STEPS; ++i)
+#pragma unroll
+            for (int s_ = 0; s_ < 4; ++s_) {
+                xf[i][s_][0] = bf16lo_to_f32(xraw[i][s_].x), xf[i][s_][1] = bf16hi_to_f32(xraw[i][s_].x);
+                xf[i][s_][2] = bf16lo_to_f32(xraw[i][s_].y), xf[i][s_][3] = bf16hi_to_f32(xraw[i][s_].y);
+            }
+    }
+    // at most 128 experts: the lane's candidates are experts lane and 64 + lane
+    float a[2];
+    bool odd = false;       // a value that is not finite
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const uint32_t e = c * 64 + lane;
+        a[c] = e < n_experts ? approx[(size_t)tok * n_experts + e] : -INFINITY;
+        odd = odd || (e < n_experts && !(fabsf(a[c]) < INFINITY));
+    }
+    // 4 B: see the comment above; the absolute term covers products the matrix unit may flush to zero
+    const float gamma = (float)d * 0x1p-22f;
+    const float bound = 4.04f * gamma * sqrtf(xnorm2[tok]) * w_norm_max + 1e-30f;
+    const bool everyone = __any(odd) || !(bound < INFINITY);
+    // v_k, the k-th largest approximate logit (equal values leave together, which can only lower it)
+    uint32_t key0 = a[0] > -INFINITY ? orderable(a[0]) : 0u, key1 = a[1] > -INFINITY ? orderable(a[1]) : 0u;
+    uint32_t kth = 0;
+    for (uint32_t r = 0; r < top_k; ++r) {
+        kth = wave_max_u32(max(key0, key1));
+        if (key0 == kth) key0 = 0u;
+        if (key1 == kth) key1 = 0u;
+    }
+    const float v_k = kth ? __uint_as_float((kth & 0x80000000u) ? (kth & 0x7FFFFFFFu) : ~kth) : -INFINITY;
+    const float threshold = v_k - bound;        // -inf when fewer than k candidates exist: everyone is in
+    unsigned long long m0 = __ballot(lane < n_experts && (everyone || a[0] >= threshold));
+    unsigned long long m1 = __ballot(64 + lane < n_experts && (everyone || a[1] >= threshold));
+    uint32_t exact0 = 0u, exact1 = 0u;      // the pinned logits of this lane's two experts, as keys of the select
+    // The candidates CHUNK at a time: all rows of a chunk are requested before the first sum runs, so a token pays a
+    // few round trips to the weights instead of one per candidate.
+    while (m0 | m1) {
+        uint32_t e[CHUNK];
+        uint2 wq[CHUNK][STEPS][4];
+#pragma unroll
+        for (int q = 0; q < CHUNK; ++q) {
+            if (m0) {
+                e[q] = (uint32_t)__builtin_ctzll(m0);
+                m0 &= m0 - 1;
+            } else if (m1) {
+                e[q] = 64u + (uint32_t)__builtin_ctzll(m1);
+                m1 &= m1 - 1;
+            } else {
+                e[q] = 0xFFFFFFFFu;
+            }
+            const uint16_t *wr = w + (size_t)(e[q] == 0xFFFFFFFFu ? 0u : e[q]) * d;
+#pragma unroll
+            for (int i = 0; i < STEPS; ++i)
+#pragma unroll
+                for (int s_ = 0; s_ < 4; ++s_) {
+                    const uint32_t k = 1024 * i + 256 * s_;
+                    wq[q][i][s_] = k < d ? *reinterpret_cast<const uint2 *>(wr + k + 4 * lane) : make_uint2(0u, 0u);
+                }
+        }
+#pragma unroll
+        for (int q = 0; q < CHUNK; ++q) {
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < STEPS; ++i)
+#pragma unroll
+                for (int s_ = 0; s_ < 4; ++s_) {
+                    if (1024u * i + 256u * s_ < d) {
+                        const uint2 wv = wq[q][i][s_];
+                        acc[s_] = __builtin_fmaf(bf16lo_to_f32(wv.x), xf[i][s_][0], acc[s_]);
+                        acc[s_] = __builtin_fmaf(bf16hi_to_f32(wv.x), xf[i][s_][1], acc[s_]);
+                        acc[s_] = __builtin_fmaf(bf16lo_to_f32(wv.y), xf[i][s_][2], acc[s_]);
+                        acc[s_] = __builtin_fmaf(bf16hi_to_f32(wv.y), xf[i][s_][3], acc[s_]);
+                    }
+                }
+            const float v = wave_butterfly_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
+            const uint32_t k_ = v > -INFINITY ? orderable(v) : 0u;
+            if (e[q] == lane) exact0 = k_;
+            if (e[q] == 64u + lane) exact1 = k_;
+        }
+    }
+    TopkRow tr;
+    tr.key[0] = exact0, tr.key[1] = exact1, tr.key[2] = 0u, tr.key[3] = 0u;
+    topk_select<2>(tr, top_k, lane);
+    topk_store(tr, per_expert_scale, top_k, out_idx + (size_t)tok * top_k, out_w + (size_t)tok * top_k, lane, false);
+}
+
 }  // namespace
 
 hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uint32_t x_stride, uint32_t t,
                          uint32_t n_experts, uint32_t d, uint32_t top_k, float *logits, uint32_t *out_idx,
-                         uint16_t *out_w, KernelTimer *timer, bool f16) {
+                         uint16_t *out_w, KernelTimer *timer, bool f16, bool want_logits, float *scratch) {
     timer->begin(s);
     const bool x_aligned = (reinterpret_cast<uintptr_t>(x) % 8 == 0) && (x_stride % 4 == 0);
     if (f16 && !x_aligned) return hipErrorInvalidValue;     // FP16 rows come 8-byte aligned (checked at the boundary)
@@ -210,6 +438,28 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
         timer->mark(s, FFMOE_K_ROUTER_LOGITS);
         hipLaunchKernelGGL(router_topk_kernel, dim3(t), dim3(64), 0, s, logits, rw.per_expert_scale, n_experts, top_k, out_idx,
                            out_w, f16);
+        timer->mark(s, FFMOE_K_ROUTER_TOPK);
+        timer->finish();
+        return hipGetLastError();
+    }
+    if (rw.w_frag && !rw.w_is_f32 && !rw.effective_scale && !f16 && !want_logits && d % 256 == 0 && d <= 1024 * kExactSteps &&
+        n_experts % 16 == 0 && n_experts <= 128 && top_k <= 8 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && x_stride % 8 == 0 && scratch) {
+        // approximate logits of every expert on the matrix unit, the pinned ones only where the select can tell
+        float *xnorm2 = scratch, *approx = scratch + ((t + 63) & ~63u);
+        const dim3 agrid((t + kApproxTok - 1) / kApproxTok);
+        const uint32_t per_wave = (n_experts / 16 + 3) / 4;       // fragments per wave: the four N quarters cover all of them
+#define FFMOE_APPROX(NF)                                                                                               \
+    hipLaunchKernelGGL(router_approx_kernel<NF>, agrid, dim3(64 * kApproxWaves), 0, s, rw.w_frag, x, x_stride, t, n_experts, \
+                       d, approx, xnorm2)
+        if (per_wave <= 1) FFMOE_APPROX(1); else FFMOE_APPROX(2);
+#undef FFMOE_APPROX
+        timer->mark(s, FFMOE_K_ROUTER_LOGITS);
+#define FFMOE_EXACT(STEPS, CHUNK)                                                                                          \
+    hipLaunchKernelGGL((router_exact_topk_kernel<STEPS, CHUNK>), dim3((t + 3) / 4), dim3(256), 0, s,                         \
+                       static_cast<const uint16_t *>(rw.w), x, x_stride, t, n_experts, d, top_k, approx, xnorm2, rw.w_norm_max, \
+                       rw.per_expert_scale, out_idx, out_w)
+        if (d <= 1024) FFMOE_EXACT(1, 4); else if (d <= 2048) FFMOE_EXACT(2, 4); else if (d <= 3072) FFMOE_EXACT(3, 4); else FFMOE_EXACT(4, 3);
+#undef FFMOE_EXACT
         timer->mark(s, FFMOE_K_ROUTER_TOPK);
         timer->finish();
         return hipGetLastError();
@@ -238,4 +488,12 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
     return hipGetLastError();
 }
 
+}  // namespace ffmoe
+
+namespace ffmoe {
+hipError_t launch_router_fragments(hipStream_t s, const uint16_t *w, uint32_t n_experts, uint32_t d, void *frag) {
+    const uint32_t pieces = (d / 32) * (n_experts / 16);
+    hipLaunchKernelGGL(router_frag_kernel, dim3((pieces * 64 + 255) / 256), dim3(256), 0, s, w, n_experts, d, static_cast<uint4 *>(frag));
+    return hipGetLastError();
+}
 }  // namespace ffmoe

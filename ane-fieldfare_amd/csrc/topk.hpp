@@ -52,13 +52,18 @@ __device__ __forceinline__ void topk_load(TopkRow &t, const float *row, uint32_t
     }
 }
 
+// SLOTS: how many of the four key slots can hold a candidate (E <= 64 SLOTS).
+template <int SLOTS = 4>
 __device__ __forceinline__ void topk_select(TopkRow &t, uint32_t top_k, uint32_t lane) {
     float mine = -INFINITY, max_s = -INFINITY;      // lane i: score of rank i
     t.idx = 0;
 #pragma unroll
     for (uint32_t r = 0; r < 8; ++r) {
         if (r < top_k) {
-            const uint32_t best = wave_max_u32(max(max(t.key[0], t.key[1]), max(t.key[2], t.key[3])));
+            uint32_t mine_best = t.key[0];
+#pragma unroll
+            for (int c = 1; c < SLOTS; ++c) mine_best = max(mine_best, t.key[c]);
+            const uint32_t best = wave_max_u32(mine_best);
             uint32_t e = 0;
             float score = -INFINITY;
             if (best != 0u) {
@@ -66,7 +71,7 @@ __device__ __forceinline__ void topk_select(TopkRow &t, uint32_t top_k, uint32_t
                 score = __uint_as_float((best & 0x80000000u) ? (best & 0x7FFFFFFFu) : ~best);
                 bool found = false;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
+                for (int c = 0; c < SLOTS; ++c) {
                     const unsigned long long holders = __ballot(t.key[c] == best);
                     if (!found && holders != 0ull) {
                         const uint32_t l = (uint32_t)__builtin_ctzll(holders);

@@ -301,3 +301,63 @@ def test_prefill_real_shape_zipf_routing(real, oracle, torch):
     print(f"zipf: rel err {r:.2e} cosine {c:.6f}; tiles {n_tiles} per-expert min/max {counts.min()}/{counts.max()}")
     assert r <= 1e-2 and c >= 0.9999
     assert counts.max() > 1500 and np.array_equal(counts, np.bincount(idx_np.ravel(), minlength=e))
+
+
+def test_prefill_router_fast_form_equals_pinned_form(oracle, torch):
+    """More than 16 rows of a bf16 router without a per-input scale take the two-pass form: approximate logits of every
+    expert on the matrix unit, the pinned sums only for the experts within four error bounds of the k-th largest
+    approximate logit. Its routes and weights must be those of the pinned sums of ALL logits (`want_logits=True` runs
+    that form, which the tests above hold against the oracle), bit for bit, on rows chosen to sit on the select's
+    edges: experts with identical rows (exact ties: the lower index wins), rows one bf16 step apart, rows of huge,
+    tiny and zero norm, and rows with non-finite values (every expert becomes a candidate)."""
+    import fieldfare_moe as ff
+    ff.lib()
+    d, e, k, t = 2816, 128, 8, 96
+    rng = np.random.default_rng(77)
+    router = rng.normal(0, 0.02, (e, d)).astype(np.float32)
+    router[5] = router[3]                       # exact ties
+    router[64] = router[3]
+    router[100] = router[99]
+    router[101] = router[99]
+    bits = oracle.bf16_bits(router)
+    bits[7] = bits[6]
+    bits[7, 17] ^= 1                            # one bf16 step apart in one element
+    bits[120] = bits[119]
+    bits[120, 2000] ^= 1
+    x = rng.normal(0, 1, (t, d)).astype(np.float32)
+    x[1] *= 1e3
+    x[2] *= 1e-20
+    x[3] = 0.0
+    x[4] = np.abs(x[4])                         # all logits of one sign pattern of the weights: wide spread
+    x[5, :] = x[5, 0]                           # a constant row
+    x[6] *= 3e18                                # squares overflow fp32: the bound is not finite
+    x[7, 100] = np.inf
+    x[8, 5] = np.nan
+    x[9, 3] = -np.inf
+    # rows aligned with expert rows: one logit far above the rest, the duplicates tie at the top
+    x[10] = router[3] * 50
+    x[11] = router[99] * 50
+    x[12] = -router[6] * 50
+    xb = bf16_tensor(torch, oracle.bf16_bits(x))
+    ctx = ff.Context(d, 64, e, k, n_layers=1, max_tokens=128)
+    ctx.upload_router_bf16(0, bits)
+    idx_fast, w_fast = ctx.router(0, xb)
+    idx_ref, w_ref, logits = ctx.router(0, xb, want_logits=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(idx_fast.cpu().numpy(), idx_ref.cpu().numpy())
+    assert np.array_equal(bits_of(w_fast), bits_of(w_ref))
+    # and the pinned form is the oracle's on the finite rows
+    xbits = oracle.bf16_bits(x)
+    got_logits = logits.cpu().numpy()
+    got_idx = idx_fast.cpu().numpy()
+    for tok in range(t):
+        if not (np.isfinite(x[tok]).all() and np.abs(x[tok]).max() < 1e15):
+            continue
+        want = oracle.router_logits_pinned(bits, xbits[tok])
+        assert np.array_equal(got_logits[tok].view(np.uint32), want.view(np.uint32)), tok
+        o_idx, _ = oracle.topk_softmax(want, k)
+        assert np.array_equal(got_idx[tok], o_idx), tok
+    # the ties resolve to the lower index
+    got = got_idx
+    assert list(got[10][:3]) == [3, 5, 64] and list(got[11][:3]) == [99, 100, 101]
+    ctx.close()
