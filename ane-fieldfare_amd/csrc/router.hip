@@ -198,13 +198,18 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, co
 // fma alone); only the selected experts' logits have to be the pinned ones.
 //   1. router_approx_kernel: every logit on the matrix unit (bf16 products are exact, the fp32 sum runs in
 //      whatever order the unit uses), plus the squared norm of every row.
-//   2. router_exact_topk_kernel, one wave per token: with a_e the approximate, p_e the pinned logit and
-//      B >= |a_e - L_e|, |p_e - L_e| for the real-number sum L_e (B = gamma * ||x|| * max_e ||w_e||, gamma = d * 2^-22:
-//      any summation order of d exact products with roundings of at most 2^-23 relative, twice over), an expert
-//      among the pinned top k has a_e >= v_k - 4 B, v_k the k-th largest approximate logit: were a_e below that,
-//      the k experts with a >= v_k would all have p >= a - 2 B > a_e + 2 B >= p_e. The wave computes the pinned logit
-//      of every expert above that threshold (a dozen at 128 experts) and selects among them with the same code as
-//      the other router kernels. A row with a non-finite value anywhere takes every expert as a candidate.
+//   2. router_exact_topk_kernel, one wave per token. Let a_e be the approximate and p_e the pinned logit of expert e, and
+//      B >= |a_e - p_e|. An expert among the pinned top k has a_e >= v_k - 2 B, v_k the k-th largest approximate logit:
+//      were a_e below that, the k experts with a >= v_k would all have p >= a - B > a_e + B >= p_e. The wave computes
+//      the pinned logit of every expert above that threshold (eight or nine at 128 experts) and selects among them
+//      with the same code as the other router kernels. A row with a non-finite value anywhere takes every expert as
+//      a candidate.
+//      B: both sums add the same exact products (bf16 x bf16 fits fp32), so each differs from the real-number sum
+//      by at most (roundings on the longest path of its summation tree) x (relative size of one rounding) x
+//      sum_k |x_k w_ek| <= ... x ||x|| max_e ||w_e||. Approximate pass: d / 128 accumulations per wave, each adding 32
+//      products (counted as 33 roundings of 2^-23, whatever order the unit uses), and 2 to merge the four waves.
+//      Pinned order: 4 fmaf per 1024-wide step, 2 adds for the sub-accumulators, 6 for the butterfly, 2^-24 each.
+//      The launch takes four times both counts.
 // Needs: bf16 rows and weights, no per-input scale, d a multiple of 256 up to 4096, E a multiple of 16 up to 128
 // (the sixteen waves of the approximate pass hold two 16-expert fragments each).
 // ---------------------------------------------------------------------------------------------------
@@ -315,7 +320,7 @@ template <int STEPS, int CHUNK>
 __global__ __launch_bounds__(256, 3) void router_exact_topk_kernel(const uint16_t *__restrict__ w, const uint16_t *__restrict__ x,
                                                                    uint32_t x_stride, uint32_t t, uint32_t n_experts, uint32_t d,
                                                                    uint32_t top_k, const float *__restrict__ approx,
-                                                                   const float *__restrict__ xnorm2, float w_norm_max,
+                                                                   const float *__restrict__ xnorm2, float bound_per_norm,
                                                                    const uint16_t *__restrict__ per_expert_scale,
                                                                    uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w) {
     const uint32_t lane = threadIdx.x & 63, tok = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -350,9 +355,8 @@ __global__ __launch_bounds__(256, 3) void router_exact_topk_kernel(const uint16_
         a[c] = e < n_experts ? approx[(size_t)tok * n_experts + e] : -INFINITY;
         odd = odd || (e < n_experts && !(fabsf(a[c]) < INFINITY));
     }
-    // 4 B: see the comment above; the absolute term covers products the matrix unit may flush to zero
-    const float gamma = (float)d * 0x1p-22f;
-    const float bound = 4.04f * gamma * sqrtf(xnorm2[tok]) * w_norm_max + 1e-30f;
+    // 2 B: see the comment above; the absolute term covers products the matrix unit may flush to zero
+    const float bound = bound_per_norm * sqrtf(xnorm2[tok]) + 1e-30f;
     const bool everyone = __any(odd) || !(bound < INFINITY);
     // v_k, the k-th largest approximate logit (equal values leave together, which can only lower it)
     uint32_t key0 = a[0] > -INFINITY ? orderable(a[0]) : 0u, key1 = a[1] > -INFINITY ? orderable(a[1]) : 0u;
@@ -389,11 +393,12 @@ __global__ __launch_bounds__(256, 3) void router_exact_topk_kernel(const uint16_
 #pragma unroll
                 for (int s_ = 0; s_ < 4; ++s_) {
                     const uint32_t k = 1024 * i + 256 * s_;
-                    wq[q][i][s_] = k < d ? *reinterpret_cast<const uint2 *>(wr + k + 4 * lane) : make_uint2(0u, 0u);
+                    wq[q][i][s_] = k < d && e[q] != 0xFFFFFFFFu ? *reinterpret_cast<const uint2 *>(wr + k + 4 * lane) : make_uint2(0u, 0u);
                 }
         }
 #pragma unroll
         for (int q = 0; q < CHUNK; ++q) {
+            if (e[q] == 0xFFFFFFFFu) continue;
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < STEPS; ++i)
@@ -454,9 +459,12 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
         if (per_wave <= 1) FFMOE_APPROX(1); else FFMOE_APPROX(2);
 #undef FFMOE_APPROX
         timer->mark(s, FFMOE_K_ROUTER_LOGITS);
+        // 2 B per unit of ||x||: four times the rounding counts of the two sums (see above), 1 % on top for the norms' own rounding
+        const float approx_roundings = 4.0f * ((float)(d / 128 + 1) + 33.0f + 2.0f), pinned_roundings = 4.0f * (4.0f * ((d + 1023) / 1024) + 8.0f);
+        const float bound_per_norm = 2.02f * (approx_roundings * 0x1p-23f + pinned_roundings * 0x1p-24f) * rw.w_norm_max;
 #define FFMOE_EXACT(STEPS, CHUNK)                                                                                          \
     hipLaunchKernelGGL((router_exact_topk_kernel<STEPS, CHUNK>), dim3((t + 3) / 4), dim3(256), 0, s,                         \
-                       static_cast<const uint16_t *>(rw.w), x, x_stride, t, n_experts, d, top_k, approx, xnorm2, rw.w_norm_max, \
+                       static_cast<const uint16_t *>(rw.w), x, x_stride, t, n_experts, d, top_k, approx, xnorm2, bound_per_norm, \
                        rw.per_expert_scale, out_idx, out_w)
         if (d <= 1024) FFMOE_EXACT(1, 4); else if (d <= 2048) FFMOE_EXACT(2, 4); else if (d <= 3072) FFMOE_EXACT(3, 4); else FFMOE_EXACT(4, 3);
 #undef FFMOE_EXACT

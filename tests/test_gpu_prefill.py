@@ -305,7 +305,7 @@ def test_prefill_real_shape_zipf_routing(real, oracle, torch):
 
 def test_prefill_router_fast_form_equals_pinned_form(oracle, torch):
     """More than 16 rows of a bf16 router without a per-input scale take the two-pass form: approximate logits of every
-    expert on the matrix unit, the pinned sums only for the experts within four error bounds of the k-th largest
+    expert on the matrix unit, the pinned sums only for the experts within two error bounds of the k-th largest
     approximate logit. Its routes and weights must be those of the pinned sums of ALL logits (`want_logits=True` runs
     that form, which the tests above hold against the oracle), bit for bit, on rows chosen to sit on the select's
     edges: experts with identical rows (exact ties: the lower index wins), rows one bf16 step apart, rows of huge,
