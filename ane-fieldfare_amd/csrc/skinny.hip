@@ -542,7 +542,8 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
             }
             __builtin_amdgcn_s_sleep(1);
         }
-        topk_select(tr, top_k, lane);
+        if (n_experts <= 128) topk_select<2>(tr, top_k, lane);      // two key slots can hold a candidate: half the ballots per round
+        else topk_select<4>(tr, top_k, lane);
         topk_store(tr, per_expert_scale, top_k, out_idx + (size_t)row * top_k, out_w + (size_t)row * top_k, lane, F16);
         if (lane < top_k) {
             // the same weight bits topk_store wrote

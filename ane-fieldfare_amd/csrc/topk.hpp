@@ -111,7 +111,8 @@ __device__ __forceinline__ void wave_topk(const float *row, const uint16_t *__re
                                           uint16_t *__restrict__ out_w, uint32_t lane, bool w_f16) {
     TopkRow t;
     topk_load(t, row, n_experts, lane);
-    topk_select(t, top_k, lane);
+    if (n_experts <= 128) topk_select<2>(t, top_k, lane);
+    else topk_select<4>(t, top_k, lane);
     topk_store(t, per_expert_scale, top_k, out_idx, out_w, lane, w_f16);
 }
 
