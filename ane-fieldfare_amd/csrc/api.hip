@@ -50,6 +50,7 @@ struct ffmoe_ctx {
     uint16_t *acts = nullptr;        // [16*top_k][F]
     float *partials = nullptr;       // [16*top_k][D]
     RouteMail *mail = nullptr;       // hand-over words of ffmoe_route_verify's one-launch router + gate/up
+    unsigned long long handover_ticks = 20000000ull;      // 0.2 s at 100 MHz
     PrefillScratch pf{};
     uint32_t max_pairs = 0;
     // dense FFN (n_experts == 1, top_k == 1): every row routes to expert 0 with weight 1
@@ -503,8 +504,16 @@ int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint1
     if (layer >= ctx->layers.size()) return fail(err, FFMOE_ERR_INVALID, "layer %u out of range", layer);
     const ffmoe_layer &l = ctx->layers[layer];
     const RouteFusion route{RouterWeights{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale}, router_x,
-                            router_x_stride, ctx->logits, ctx->mail};
+                            router_x_stride, ctx->logits, ctx->mail, ctx->handover_ticks};
     return verify_common(ctx, stream, layer, x, x_stride, t, out_idx, out_w, residual, y, nullptr, err, nullptr, &route);
+}
+
+int ffmoe_set_handover_timeout(ffmoe_ctx *ctx, void *stream, uint64_t ticks, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    FF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    ctx->handover_ticks = ticks;
+    FF_HIP(hipMemset(&ctx->mail->faults, 0, sizeof(uint32_t)));
+    return FFMOE_OK;
 }
 
 int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,

@@ -132,6 +132,7 @@ struct RouteFusion {
     uint32_t router_x_stride;
     float *logits;          // scratch of the two-launch router (used when the one-launch form does not apply)
     RouteMail *mail;
+    unsigned long long poll_ticks;      // how long a block waits for a hand-over word (wall_clock64 ticks, 100 MHz)
 };
 
 // repack.hip

@@ -460,9 +460,8 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
 //      requested between 1 and 3, so they arrive while the block waits.
 // The epoch is read from mail->epoch by every block at its start and is advanced by a later launch of the same call
 // (the combine), which keeps a replayed HIP graph correct. Every block of the grid has to be resident at once (the
-// grid is at most two blocks per compute unit, the kernel's occupancy); a poll gives up after 0.2 s, counts a fault
-// in mail->faults and goes on with empty routes.
-constexpr unsigned long long kPollTicks = 20000000ull;      // wall_clock64() ticks at 100 MHz
+// grid is at most two blocks per compute unit, the kernel's occupancy); a poll gives up after `poll_ticks` (100 MHz ticks;
+// 0.2 s by default), counts a fault in mail->faults and goes on with empty routes.
 
 __device__ __forceinline__ unsigned long long mail_load(const unsigned long long *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -476,6 +475,7 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
     const uint8_t *__restrict__ arena_layer, ArenaGeom g, uint32_t top_k, uint32_t n_experts, const void *__restrict__ router_w,
     const uint16_t *__restrict__ effective_scale, const uint16_t *__restrict__ per_expert_scale,
     const uint16_t *__restrict__ router_x, uint32_t router_x_stride, uint32_t rows, RouteMail *__restrict__ mail,
+    unsigned long long poll_ticks,
     uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w, VerifyPlan *__restrict__ plan,
     const uint16_t *__restrict__ x, uint32_t x_stride, uint16_t *__restrict__ acts) {
     __shared__ GateUpMerge s_red;
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
                 tr.key[c] = v > -INFINITY ? orderable(v) : 0u;
             }
             if (__all(ok)) break;
-            if (wall_clock64() - t_start > kPollTicks) {
+            if (wall_clock64() - t_start > poll_ticks) {
                 if (lane == 0) atomicAdd(&mail->faults, 1u);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) tr.key[c] = 0u;      // no candidates: weights 0, nothing is routed
@@ -564,7 +564,7 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
                 route_w = (uint16_t)((uint32_t)word >> 16);
                 break;
             }
-            if (wall_clock64() - t_start > kPollTicks) {
+            if (wall_clock64() - t_start > poll_ticks) {
                 if (lane == 0) atomicAdd(&mail->faults, 1u);
                 break;          // empty routes: weight 0 takes no part
             }
@@ -861,23 +861,22 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
     if (mail && blockIdx.x == 0 && tok == 0 && threadIdx.x == 0) mail->epoch += 1;      // the routing launch of this call has read it
     const uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (c >= d) return;
-    // every load of the thread is requested before the first is used: the routes' weights and experts, then
-    // the rows of the live ones (a dead route's row may hold anything and is never touched)
+    // One round trip: the routes' weights and validity and all eight rows are requested together. A row the plan
+    // skipped was never written and may hold anything: it is loaded like the others and dropped by the select below
+    // (its address is inside the buffer either way), instead of being asked for only once its validity has arrived.
     float wv[8];
-    bool live[8];
-#pragma unroll
-    for (uint32_t r = 0; r < 8; ++r) {
-        const uint32_t route = tok * top_k + min(r, top_k - 1);
-        const uint16_t wb = w[route];
-        live[r] = r < top_k && plan->route_valid[route] != 0;
-        wv[r] = Act<F16>::widen(wb);
-    }
+    uint32_t valid[8];
     f32x4 p[8];
 #pragma unroll
     for (uint32_t r = 0; r < 8; ++r) {
         const uint32_t route = tok * top_k + min(r, top_k - 1);
-        p[r] = live[r] ? *reinterpret_cast<const f32x4 *>(partials + (size_t)route * d + c) : f32x4{0.f, 0.f, 0.f, 0.f};
+        wv[r] = Act<F16>::widen(w[route]);
+        valid[r] = plan->route_valid[route];
+        p[r] = *reinterpret_cast<const f32x4 *>(partials + (size_t)route * d + c);
     }
+    bool live[8];
+#pragma unroll
+    for (uint32_t r = 0; r < 8; ++r) live[r] = r < top_k && valid[r] != 0;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (residual) {
         const uint2 rv = *reinterpret_cast<const uint2 *>(residual + (size_t)tok * d + c);
@@ -946,7 +945,8 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
 #define FFMOE_ROUTE_GU(WF)                                                                                                  \
     hipLaunchKernelGGL((route_gate_up_persistent<WF, F16>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, \
                        route->rw.w, route->rw.effective_scale, route->rw.per_expert_scale, route->router_x,                  \
-                       route->router_x_stride, t, route->mail, const_cast<uint32_t *>(idx), const_cast<uint16_t *>(w), plan, \
+                       route->router_x_stride, t, route->mail, route->poll_ticks, const_cast<uint32_t *>(idx),                \
+                       const_cast<uint16_t *>(w), plan,                                                                     \
                        x, x_stride, acts)
         if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true); else FFMOE_ROUTE_GU(false);
 #undef FFMOE_ROUTE_GU

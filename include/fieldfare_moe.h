@@ -186,6 +186,12 @@ int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint1
                        uint32_t router_x_stride, const uint16_t *x, uint32_t x_stride, uint32_t t,
                        const uint16_t *residual, uint16_t *y, uint32_t *out_idx, uint16_t *out_w, char **err);
 
+/* How long a block of ffmoe_route_verify's one-launch form waits for a hand-over word before it gives up, in ticks of
+ * the GPU's constant 100 MHz clock (default 20,000,000 = 0.2 s); also clears the count of polls that gave up. Waits
+ * for the stream. No counterpart in the reference. A host that shares the GPU with other work may want a longer
+ * wait; the tests set 0 to see the give-up path end normally and be reported. */
+int ffmoe_set_handover_timeout(ffmoe_ctx *ctx, void *stream, uint64_t ticks, char **err);
+
 /* Number of distinct experts the last ffmoe_verify* call on `stream` ran (reads back 4 bytes; waits
  * for the stream). For reporting only. FFMOE_ERR_RUNTIME if a launch of ffmoe_route_verify on this
  * context ever gave up waiting for its own blocks (see there). */

@@ -454,6 +454,33 @@ def test_route_verify_equals_router_then_verify(small, real, oracle, torch, whic
         assert np.array_equal(got[r], ref_idx), f"row {r}"
 
 
+def test_route_verify_gives_up_on_a_missing_hand_over_and_says_so(real, oracle, torch):
+    """The blocks of route_verify's one-launch form wait for each other's words with a bounded poll. With the bound
+    set to zero from the host every poll that does not find its words at once gives up: the launch must still end
+    normally, the give-ups must be counted and reported by the next last_live_experts, and after the bound is set
+    back (which clears the count) the same call must again equal router + verify bit for bit."""
+    import fieldfare_moe as ff
+    ctx, d = real["ctx"], real["d"]
+    g = oracle.seed_tree_key(0x207E, "route-verify-timeout")
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, 16 * d)).reshape(16, d)
+    x = bf16_tensor(torch, xb)
+    try:
+        ctx.set_handover_timeout(0)
+        ctx.route_verify(0, x, x)
+        torch.cuda.synchronize()            # the launch ended
+        with pytest.raises(RuntimeError, match="gave up"):
+            ctx.last_live_experts()
+    finally:
+        ctx.set_handover_timeout(20_000_000)
+    assert ctx.last_live_experts() >= 0
+    idx2, w2 = ctx.router(0, x)
+    y2 = ctx.verify(0, x, idx2, w2)
+    y1, idx1, w1 = ctx.route_verify(0, x, x)
+    assert np.array_equal(idx1.cpu().numpy(), idx2.cpu().numpy())
+    assert np.array_equal(bits_of(y1), bits_of(y2))
+    assert ctx.last_live_experts() > 0
+
+
 @pytest.mark.parametrize("which", ["small", "real"])
 def test_decode_sized_blocks_equal_rows_of_a_larger_block(small, real, oracle, torch, which):
     # rows are independent of the block they arrive in: a block of two rows and a block of one row give the
