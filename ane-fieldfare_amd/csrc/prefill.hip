@@ -296,19 +296,22 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     // row blocks, and is followed by one piece of the next group's expansion, so the matrix pipe and the
     // VALU run side by side inside the wave (a scheduling fence after every unit keeps the order as
     // written). On entry: af[.][0] = k-half 0 of this group; araw[.][1] = its k-half 1 in load layout;
-    // araw[.][0] = k-half 0 of the next group in flight; wraw/sraw = packed tile of the next group in
-    // flight; wb[buf] = expanded tiles of this group. The k-half 1 fragments are made at the start of the
+    // araw[.][0] = k-half 0 of the next group in flight; wraw/sraw = packed tile of the group after next in
+    // flight (it is expanded during this step); wb[buf] = expanded tiles of this group, the next group's are
+    // there as well. The k-half 1 fragments are made at the start of the
     // step and the next k-half 0 fragments in its middle, each as soon as the registers they replace have
     // had their last use, with 8 units of MFMAs to cover the cross-lane latency; every register that a
     // conversion frees is reloaded at once for the following group. Past the last group the loads and the
     // expansion run once more on clamped indices and are never used: with no branch around them the
-    // compiler counts the loads in flight exactly.
+    // compiler counts the loads in flight exactly. The expanded tiles sit in four LDS buffers (group g in buffer
+    // g % 4) and the expansion runs two groups ahead of the products, so one barrier per PAIR of groups orders both
+    // the first read of a buffer behind its last write and its next write behind its last read.
     auto step = [&](uint32_t grp) {
-        const int buf = grp & 1;
+        const int buf = grp & 3;
         frag_a(1);
         load_a(min(grp + 1, n_groups - 1), 1);
         expand_begin();
-        load_b(min(grp + 2, n_groups - 1));
+        load_b(min(grp + 3, n_groups - 1));
         uint4 bq[3];
         auto read_b = [&](int u) { bq[u % 3] = wb[buf][(u & 7) >> 1][u & 1][u >> 3][lane]; };
         if (DUMP && wave == 0) {
@@ -335,7 +338,7 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
                     // one pair, which the epilogue packs into one 8-byte piece of that pair's output row
                     acc[i][u & 7] = mfma16(bfrag, af[i][u >> 3], acc[i][u & 7]);
             }
-            expand_piece(buf ^ 1, u);
+            expand_piece((buf + 2) & 3, u);
             __builtin_amdgcn_sched_barrier(0);
             if (u == 7) {
                 frag_a(0);
@@ -343,7 +346,7 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        lds_barrier();
+        if (grp & 1) lds_barrier();      // one barrier per pair of groups: the expansion runs two groups ahead
     };
 
     load_b(0);
@@ -353,10 +356,15 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     load_b(min(1u, n_groups - 1));
 #pragma unroll
     for (int piece = 0; piece < 16; ++piece) expand_piece(0, piece);
+    expand_begin();
+    load_b(min(2u, n_groups - 1));
+#pragma unroll
+    for (int piece = 0; piece < 16; ++piece) expand_piece(1, piece);
     frag_a(0);
     load_a(min(1u, n_groups - 1), 0);
     lds_barrier();
     for (uint32_t grp = 0; grp < n_groups; ++grp) step(grp);
+    if (n_groups & 1) lds_barrier();     // the last pair was half a pair
     if (NMB == 0) return;
 
     // epilogue: lane (j, jq) holds pair 16 (w + 4 i) + j, weight rows 4 jq .. 4 jq + 3 of every fragment
@@ -384,7 +392,7 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     // through a private LDS area (the weight buffers are free: the last step ended with a barrier) so that
     // 16 lanes store one row's 256 contiguous bytes, instead of 8-byte pieces 32 B apart per instruction.
     constexpr uint32_t kStageRow = 2 * kTilesPerBlock * kTileRows * 2 + 16;     // bytes: 128 columns + padding
-    static_assert(4 * 16 * kStageRow <= sizeof(uint4) * 2 * kTilesPerBlock * 2 * 2 * kWave, "staging fits the weight buffers");
+    static_assert(4 * 16 * kStageRow <= sizeof(uint4) * 4 * kTilesPerBlock * 2 * 2 * kWave, "staging fits the weight buffers");
     uint8_t *stage = reinterpret_cast<uint8_t *>(wb) + wave * 16 * kStageRow;
     const uint32_t rsub = lane >> 4, chunk = lane & 15;                         // read side: row 4 p + rsub, columns 8 chunk ..
     const bool col_ok = gw.nb * kTilesPerBlock + (chunk >> 2) < gw.n_arena_tiles;
@@ -430,7 +438,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__r
                                                               const uint16_t *__restrict__ a, uint32_t a_stride,
                                                               uint16_t *__restrict__ out, uint32_t n_nblocks,
                                                               uint4 *__restrict__ dump = nullptr) {
-    __shared__ __align__(16) uint4 wb[2][kTilesPerBlock][2][2][kWave];   // [buffer][tile][stream][k-half][lane]
+    __shared__ __align__(16) uint4 wb[4][kTilesPerBlock][2][2][kWave];   // [buffer][tile][stream][k-half][lane]: group g lives in buffer g % 4
 
     const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const uint32_t ti = (slot / n_nblocks) * 8 + xcd, nb = slot % n_nblocks;
