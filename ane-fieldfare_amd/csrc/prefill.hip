@@ -301,17 +301,20 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     // there as well. The k-half 1 fragments are made at the start of the
     // step and the next k-half 0 fragments in its middle, each as soon as the registers they replace have
     // had their last use, with 8 units of MFMAs to cover the cross-lane latency; every register that a
-    // conversion frees is reloaded at once for the following group. Past the last group the loads and the
-    // expansion run once more on clamped indices and are never used: with no branch around them the
-    // compiler counts the loads in flight exactly. The expanded tiles sit in four LDS buffers (group g in buffer
+    // conversion frees is reloaded at once for the following group. Loads past the last group run on clamped
+    // indices and are never used: with no branch around them the compiler counts the loads in flight exactly.
+    // The last two steps are a second instantiation without the expansion (their groups are in LDS already). The expanded tiles sit in four LDS buffers (group g in buffer
     // g % 4) and the expansion runs two groups ahead of the products, so one barrier per PAIR of groups orders both
     // the first read of a buffer behind its last write and its next write behind its last read.
-    auto step = [&](uint32_t grp) {
+    auto step = [&](uint32_t grp, auto expand_ahead) {
+        constexpr bool kExpand = decltype(expand_ahead)::value;     // false in the last two steps: nothing is left to expand
         const int buf = grp & 3;
         frag_a(1);
         load_a(min(grp + 1, n_groups - 1), 1);
-        expand_begin();
-        load_b(min(grp + 3, n_groups - 1));
+        if (kExpand) {
+            expand_begin();
+            load_b(min(grp + 3, n_groups - 1));
+        }
         uint4 bq[3];
         auto read_b = [&](int u) { bq[u % 3] = wb[buf][(u & 7) >> 1][u & 1][u >> 3][lane]; };
         if (DUMP && wave == 0) {
@@ -338,7 +341,7 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
                     // one pair, which the epilogue packs into one 8-byte piece of that pair's output row
                     acc[i][u & 7] = mfma16(bfrag, af[i][u >> 3], acc[i][u & 7]);
             }
-            expand_piece((buf + 2) & 3, u);
+            if (kExpand) expand_piece((buf + 2) & 3, u);
             __builtin_amdgcn_sched_barrier(0);
             if (u == 7) {
                 frag_a(0);
@@ -348,6 +351,8 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
         }
         if (grp & 1) lds_barrier();      // one barrier per pair of groups: the expansion runs two groups ahead
     };
+    using Ahead = std::integral_constant<bool, true>;
+    using Tail = std::integral_constant<bool, false>;
 
     load_b(0);
     load_a(0, 0);
@@ -363,7 +368,10 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     frag_a(0);
     load_a(min(1u, n_groups - 1), 0);
     lds_barrier();
-    for (uint32_t grp = 0; grp < n_groups; ++grp) step(grp);
+    // the last two steps multiply only: their groups were expanded two steps earlier
+    const uint32_t n_ahead = n_groups > 2 ? n_groups - 2 : 0;
+    for (uint32_t grp = 0; grp < n_ahead; ++grp) step(grp, Ahead{});
+    for (uint32_t grp = n_ahead; grp < n_groups; ++grp) step(grp, Tail{});
     if (n_groups & 1) lds_barrier();     // the last pair was half a pair
     if (NMB == 0) return;
 
