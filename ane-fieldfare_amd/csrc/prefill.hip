@@ -244,11 +244,14 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
 #pragma unroll
         for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) acc[i][nf] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    uint4 wraw = {0, 0, 0, 0};      // this wave's packed tile, in flight: the group after the one being expanded
-    uint2 sraw = {0, 0};
-    auto load_b = [&](uint32_t grp) {
-        wraw = reinterpret_cast<const uint4 *>(gw.w_tiles + (size_t)grp * kTileBytes)[lane];
-        sraw = reinterpret_cast<const uint2 *>(gw.w_scales + (size_t)grp * kTileScaleBytes)[j];
+    // this wave's packed tile of the next kSlots groups to expand, in flight: group g waits in slot g % kSlots
+    // (one slot where the row blocks leave no registers for a second: the steps are long enough there)
+    constexpr int kSlots = (GATE_UP && NMB >= 4) ? 1 : 2;
+    uint4 wraw[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+    uint2 sraw[2] = {{0, 0}, {0, 0}};
+    auto load_b = [&](uint32_t grp, int slot) {
+        wraw[slot] = reinterpret_cast<const uint4 *>(gw.w_tiles + (size_t)grp * kTileBytes)[lane];
+        sraw[slot] = reinterpret_cast<const uint2 *>(gw.w_scales + (size_t)grp * kTileScaleBytes)[j];
     };
     // Expansion of the packed tile in `wcur` into wb[buf], cut into 16 pieces of about five VALU
     // instructions (piece 4 c + q = output dword q of packed word c; the word's last piece stores it).
@@ -256,10 +259,10 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     float sc[2], bi[2];
     uint32_t lo = 0, hi = 0;
     uint4 ex = {0, 0, 0, 0};
-    auto expand_begin = [&]() {
-        wcur[0] = wraw.x, wcur[1] = wraw.y, wcur[2] = wraw.z, wcur[3] = wraw.w;
-        sc[0] = bf16lo_to_f32(sraw.x), bi[0] = bf16hi_to_f32(sraw.x);
-        sc[1] = bf16lo_to_f32(sraw.y), bi[1] = bf16hi_to_f32(sraw.y);
+    auto expand_begin = [&](int slot) {
+        wcur[0] = wraw[slot].x, wcur[1] = wraw[slot].y, wcur[2] = wraw[slot].z, wcur[3] = wraw[slot].w;
+        sc[0] = bf16lo_to_f32(sraw[slot].x), bi[0] = bf16hi_to_f32(sraw[slot].x);
+        sc[1] = bf16lo_to_f32(sraw[slot].y), bi[1] = bf16hi_to_f32(sraw[slot].y);
     };
     auto expand_piece = [&](int buf, int piece) {
         const int c = piece >> 2, q = piece & 3;
@@ -296,24 +299,26 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     // row blocks, and is followed by one piece of the next group's expansion, so the matrix pipe and the
     // VALU run side by side inside the wave (a scheduling fence after every unit keeps the order as
     // written). On entry: af[.][0] = k-half 0 of this group; araw[.][1] = its k-half 1 in load layout;
-    // araw[.][0] = k-half 0 of the next group in flight; wraw/sraw = packed tile of the group after next in
-    // flight (it is expanded during this step); wb[buf] = expanded tiles of this group, the next group's are
+    // araw[.][0] = k-half 0 of the next group in flight; wraw/sraw[grp % kSlots] = packed tile of the group after next
+    // (it is expanded during this step, and its slot is reloaded at once with the group kSlots further on: with
+    // two slots a packed tile has two steps to arrive); wb[buf] = expanded tiles of this group, the next group's are
     // there as well. The k-half 1 fragments are made at the start of the
     // step and the next k-half 0 fragments in its middle, each as soon as the registers they replace have
     // had their last use, with 8 units of MFMAs to cover the cross-lane latency; every register that a
     // conversion frees is reloaded at once for the following group. Loads past the last group run on clamped
     // indices and are never used: with no branch around them the compiler counts the loads in flight exactly.
-    // The last two steps are a second instantiation without the expansion (their groups are in LDS already). The expanded tiles sit in four LDS buffers (group g in buffer
-    // g % 4) and the expansion runs two groups ahead of the products, so one barrier per PAIR of groups orders both
+    // The last two steps are a second instantiation without the expansion (their groups are in LDS already).
+    // The expanded tiles sit in four LDS buffers (group g in buffer g % 4) and the expansion runs two groups ahead of the products, so one barrier per PAIR of groups orders both
     // the first read of a buffer behind its last write and its next write behind its last read.
-    auto step = [&](uint32_t grp, auto expand_ahead) {
+    auto step = [&](uint32_t grp, auto expand_ahead, auto parity) {
         constexpr bool kExpand = decltype(expand_ahead)::value;     // false in the last two steps: nothing is left to expand
+        constexpr int kSlot = decltype(parity)::value;              // grp % 2, known at compile time: the slots are registers
         const int buf = grp & 3;
         frag_a(1);
         load_a(min(grp + 1, n_groups - 1), 1);
         if (kExpand) {
-            expand_begin();
-            load_b(min(grp + 3, n_groups - 1));
+            expand_begin(kSlot % kSlots);                           // group grp + 2
+            load_b(min(grp + 2 + kSlots, n_groups - 1), kSlot % kSlots);
         }
         uint4 bq[3];
         auto read_b = [&](int u) { bq[u % 3] = wb[buf][(u & 7) >> 1][u & 1][u >> 3][lane]; };
@@ -349,29 +354,47 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if (grp & 1) lds_barrier();      // one barrier per pair of groups: the expansion runs two groups ahead
+        // one barrier per pair of groups: the expansion runs two groups ahead (the tail steps, which use no slot,
+        // are one instantiation and look at the group's parity itself)
+        if (kExpand && kSlots == 2 ? kSlot != 0 : (grp & 1) != 0) lds_barrier();
     };
     using Ahead = std::integral_constant<bool, true>;
     using Tail = std::integral_constant<bool, false>;
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
 
-    load_b(0);
+    load_b(0, 0);
+    if (kSlots == 2) load_b(min(1u, n_groups - 1), 1);
     load_a(0, 0);
     load_a(0, 1);
-    expand_begin();
-    load_b(min(1u, n_groups - 1));
+    expand_begin(0);
+    load_b(min((uint32_t)kSlots, n_groups - 1), 0);
 #pragma unroll
     for (int piece = 0; piece < 16; ++piece) expand_piece(0, piece);
-    expand_begin();
-    load_b(min(2u, n_groups - 1));
+    expand_begin(1 % kSlots);
+    load_b(min(1u + kSlots, n_groups - 1), 1 % kSlots);
 #pragma unroll
     for (int piece = 0; piece < 16; ++piece) expand_piece(1, piece);
     frag_a(0);
     load_a(min(1u, n_groups - 1), 0);
     lds_barrier();
-    // the last two steps multiply only: their groups were expanded two steps earlier
+    // steps in pairs (the slot of a group's packed tile and the barrier follow the group's parity); the last two
+    // steps multiply only: their groups were expanded two steps earlier
     const uint32_t n_ahead = n_groups > 2 ? n_groups - 2 : 0;
-    for (uint32_t grp = 0; grp < n_ahead; ++grp) step(grp, Ahead{});
-    for (uint32_t grp = n_ahead; grp < n_groups; ++grp) step(grp, Tail{});
+    uint32_t grp = 0;
+    if constexpr (kSlots == 2) {
+        for (; grp + 2 <= n_ahead; grp += 2) {
+            step(grp, Ahead{}, Even{});
+            step(grp + 1, Ahead{}, Odd{});
+        }
+        if (grp < n_ahead) {             // an odd number of groups: one more expanding step
+            step(grp, Ahead{}, Even{});
+            ++grp;
+        }
+    } else {
+        for (; grp < n_ahead; ++grp) step(grp, Ahead{}, Even{});
+    }
+    for (; grp < n_groups; ++grp) step(grp, Tail{}, Even{});
     if (n_groups & 1) lds_barrier();     // the last pair was half a pair
     if (NMB == 0) return;
 
