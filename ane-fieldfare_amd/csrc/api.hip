@@ -51,6 +51,7 @@ struct ffmoe_ctx {
     float *partials = nullptr;       // [16*top_k][D]
     RouteMail *mail = nullptr;       // hand-over words of ffmoe_route_verify's one-launch router + gate/up
     unsigned long long handover_ticks = 20000000ull;      // 0.2 s at 100 MHz
+    bool one_launch_routing = true;
     PrefillScratch pf{};
     uint32_t max_pairs = 0;
     // dense FFN (n_experts == 1, top_k == 1): every row routes to expert 0 with weight 1
@@ -504,7 +505,7 @@ int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint1
     if (layer >= ctx->layers.size()) return fail(err, FFMOE_ERR_INVALID, "layer %u out of range", layer);
     const ffmoe_layer &l = ctx->layers[layer];
     const RouteFusion route{RouterWeights{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale}, router_x,
-                            router_x_stride, ctx->logits, ctx->mail, ctx->handover_ticks};
+                            router_x_stride, ctx->logits, ctx->mail, ctx->handover_ticks, ctx->one_launch_routing};
     return verify_common(ctx, stream, layer, x, x_stride, t, out_idx, out_w, residual, y, nullptr, err, nullptr, &route);
 }
 
@@ -513,6 +514,12 @@ int ffmoe_set_handover_timeout(ffmoe_ctx *ctx, void *stream, uint64_t ticks, cha
     FF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     ctx->handover_ticks = ticks;
     FF_HIP(hipMemset(&ctx->mail->faults, 0, sizeof(uint32_t)));
+    return FFMOE_OK;
+}
+
+int ffmoe_set_one_launch_routing(ffmoe_ctx *ctx, int enabled, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    ctx->one_launch_routing = enabled != 0;      // host state only: takes effect with the next call
     return FFMOE_OK;
 }
 

@@ -133,6 +133,7 @@ struct RouteFusion {
     float *logits;          // scratch of the two-launch router (used when the one-launch form does not apply)
     RouteMail *mail;
     unsigned long long poll_ticks;      // how long a block waits for a hand-over word (wall_clock64 ticks, 100 MHz)
+    bool one_launch;                    // false: the router runs as launches of its own in front of the expert pass
 };
 
 // repack.hip

@@ -925,7 +925,7 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     // router and gate/up when the expert fits the persistent kernel, the combine follows in this call (it advances
     // the epoch) and the router rows are 8-byte aligned; otherwise the router's own two launches go first.
     const bool fits_ring = (g.gd + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
-    const bool fuse = route && fits_ring && y && !partials_bf16 && top_k <= 8 && n_experts <= FFMOE_MAX_EXPERTS &&
+    const bool fuse = route && route->one_launch && fits_ring && y && !partials_bf16 && top_k <= 8 && n_experts <= FFMOE_MAX_EXPERTS &&
                       reinterpret_cast<uintptr_t>(route->router_x) % 8 == 0 && route->router_x_stride % 4 == 0;
     if (route && !fuse) {
         const hipError_t e = launch_router(s, route->rw, route->router_x, route->router_x_stride, t, n_experts, g.d, top_k,

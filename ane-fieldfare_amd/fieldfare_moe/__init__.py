@@ -47,7 +47,7 @@ EXPORTS = [
     "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
     "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
-    "ffmoe_layer_tail", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_gemv_int4_listed",
+    "ffmoe_layer_tail", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
     "ffmoe_verify_static",
 ]
@@ -193,6 +193,7 @@ def lib() -> C.CDLL:
     L.ffmoe_verify_partials.argtypes = [vp, vp, u32, vp, u32, u32, vp, vp, vp, errp]
     L.ffmoe_route_verify.argtypes = [vp, vp, u32, vp, u32, vp, u32, u32, vp, vp, vp, vp, errp]
     L.ffmoe_set_handover_timeout.argtypes = [vp, vp, C.c_uint64, errp]
+    L.ffmoe_set_one_launch_routing.argtypes = [vp, C.c_int, errp]
     L.ffmoe_last_live_experts.argtypes = [vp, vp, C.POINTER(u32), errp]
     L.ffmoe_reduce_token_major.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, errp]
     L.ffmoe_gemv_int4.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, i32, errp]
@@ -434,6 +435,11 @@ class Context:
         """Ticks (100 MHz) a block of route_verify's one-launch form waits for a hand-over word; clears the fault count."""
         err = C.c_char_p()
         _check(self.L.ffmoe_set_handover_timeout(self._h, _stream(), ticks, C.byref(err)), err)
+
+    def set_one_launch_routing(self, enabled: bool):
+        """False: route_verify runs the router as launches of its own (no block waits for another)."""
+        err = C.c_char_p()
+        _check(self.L.ffmoe_set_one_launch_routing(self._h, int(bool(enabled)), C.byref(err)), err)
 
     def last_live_experts(self) -> int:
         n = C.c_uint32()

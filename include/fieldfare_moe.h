@@ -192,6 +192,13 @@ int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint1
  * wait; the tests set 0 to see the give-up path end normally and be reported. */
 int ffmoe_set_handover_timeout(ffmoe_ctx *ctx, void *stream, uint64_t ticks, char **err);
 
+/* enabled = 0: ffmoe_route_verify runs the router as launches of its own in front of the expert pass (five launches
+ * for a verify block, four for a decode step; same results bit for bit), which needs no block to wait for another:
+ * the form for a host whose other streams or processes keep compute units of this GPU busy, where the one-launch
+ * form's blocks cannot count on being resident together. enabled != 0 (the default) restores the one-launch form.
+ * Host state, takes effect with the next call. No counterpart in the reference. */
+int ffmoe_set_one_launch_routing(ffmoe_ctx *ctx, int enabled, char **err);
+
 /* Number of distinct experts the last ffmoe_verify* call on `stream` ran (reads back 4 bytes; waits
  * for the stream). For reporting only. FFMOE_ERR_RUNTIME if a launch of ffmoe_route_verify on this
  * context ever gave up waiting for its own blocks (see there). */

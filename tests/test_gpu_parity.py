@@ -481,6 +481,37 @@ def test_route_verify_gives_up_on_a_missing_hand_over_and_says_so(real, oracle, 
     assert ctx.last_live_experts() > 0
 
 
+@pytest.mark.parametrize("t", [1, 16])
+def test_route_verify_with_the_router_as_its_own_launches(real, oracle, torch, t):
+    """set_one_launch_routing(False): the same call runs the router in front of the expert pass (the timer's router
+    slots fill, the one-launch slot stays empty) and gives the bits of the one-launch form."""
+    ctx, d = real["ctx"], real["d"]
+    g = oracle.seed_tree_key(0x207E, f"route-verify-split-{t}")
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    x = bf16_tensor(torch, xb)
+    y1, idx1, w1 = ctx.route_verify(0, x, x)
+    try:
+        ctx.set_one_launch_routing(False)
+        ctx.set_profiling(True)
+        ctx.profile(reset=True)
+        y2, idx2, w2 = ctx.route_verify(0, x, x)
+        prof = ctx.profile(reset=True)
+    finally:
+        ctx.set_profiling(False)
+        ctx.set_one_launch_routing(True)
+    assert prof["router_logits"][1] == 1 and prof["router_topk"][1] == 1 and prof["gate_up"][1] == 1
+    assert prof.get("route_gate_up", (0.0, 0))[1] == 0
+    assert np.array_equal(idx1.cpu().numpy(), idx2.cpu().numpy())
+    assert np.array_equal(bits_of(w1), bits_of(w2))
+    assert np.array_equal(bits_of(y1), bits_of(y2))
+    ctx.set_profiling(True)
+    ctx.profile(reset=True)
+    ctx.route_verify(0, x, x)
+    prof = ctx.profile(reset=True)
+    ctx.set_profiling(False)
+    assert prof["route_gate_up"][1] == 1 and prof.get("router_logits", (0.0, 0))[1] == 0
+
+
 @pytest.mark.parametrize("which", ["small", "real"])
 def test_decode_sized_blocks_equal_rows_of_a_larger_block(small, real, oracle, torch, which):
     # rows are independent of the block they arrive in: a block of two rows and a block of one row give the
