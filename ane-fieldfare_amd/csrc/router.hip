@@ -214,7 +214,6 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, co
 // (the sixteen waves of the approximate pass hold two 16-expert fragments each).
 // ---------------------------------------------------------------------------------------------------
 constexpr int kApproxTok = 16;          // token rows per block of the approximate pass
-constexpr int kMaxFrags = FFMOE_MAX_EXPERTS / 16;
 
 // Router weights in matrix-operand order: frag[(h * E/16 + n) * 64 + lane] = the eight values
 // w[16 n + lane % 16][32 h + 8 (lane / 16) .. + 7], so that a wave's operand load is 1 KiB contiguous.
