@@ -110,15 +110,11 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
     WeightRing ring;
 #pragma unroll
     for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb0 * n_groups + min(g0 + u, g_last), lane);
-    const uint16_t *xrow = x + (size_t)min(j, rows - 1) * x_stride + 8 * jq;
+    // the input rows of this wave's K-slice: requested as 64-byte pieces (four lanes per row), then turned into the
+    // operand layout - with 16 rows the operand layout itself would make every lane of every load a request of its own
     uint4 x0[kRing], x1[kRing];
-#pragma unroll
-    for (int u = 0; u < kRing; ++u) {
-        const bool live = (uint32_t)u < ng;
-        const uint32_t gg = min(g0 + u, g_last);
-        x0[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup) : uint4{0, 0, 0, 0};
-        x1[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
-    }
+    load_token_rows(x, x_stride, rows, lane, KSlice{g0, ng, g_last}, x0, x1);
+    turn_token_rows(lane, x0, x1);
     // per group: the sum of its inputs per token column, once for all the tile rows this wave walks
     f32x4 sx[kRing];
 #pragma unroll

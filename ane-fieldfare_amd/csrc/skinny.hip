@@ -291,50 +291,6 @@ __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restr
 // gate/up + GELU-tanh gating, persistent. grid = (blocks); the blocks are dealt to the live experts, each
 // block walks a range of 16-row blocks of its expert; its four waves split K and meet in LDS per row block
 // (partials added in wave order), each wave finishing a quarter of the token slots.
-struct KSlice {
-    uint32_t g0, ng, g_last;      // first group, number of groups, last valid group of this wave's share of K
-};
-__device__ __forceinline__ KSlice k_slice(uint32_t groups, uint32_t ks) {
-    const uint32_t per = (groups + kKSplit - 1) / kKSplit;
-    const uint32_t g0 = min(ks * per, groups), g1 = min(groups, g0 + per);
-    return KSlice{g0, g1 - g0, g1 > g0 ? g1 - 1 : groups - 1};
-}
-
-// The token operand is the block's rows themselves, row min(j, rows - 1) in token column j: which expert a
-// block serves does not matter for fetching them, so they can be requested before the routes are known. An
-// expert's routes only decide which columns of the result are stored.
-// Load layout: four neighbouring lanes read 64 contiguous bytes of one row (row lane / 4, 8-element chunk
-// lane % 4), 16 requests of 64 bytes per instruction; with the matrix unit's own layout (row lane % 16)
-// every lane would be a request of its own and the 22 loads of a wave would keep the address unit busy
-// for microseconds. turn_token_rows() re-lays them into the operand layout (lane (j, jq): row j, chunk jq).
-__device__ __forceinline__ void load_token_rows(const uint16_t *__restrict__ x, uint32_t x_stride, uint32_t rows,
-                                                uint32_t lane, const KSlice &k, uint4 (&x0)[kRing], uint4 (&x1)[kRing]) {
-    const uint16_t *xrow = x + (size_t)min(lane >> 2, rows - 1) * x_stride + 8 * (lane & 3);
-#pragma unroll
-    for (int u = 0; u < kRing; ++u) {
-        const bool live = (uint32_t)u < k.ng;
-        const uint32_t gg = min(k.g0 + u, k.g_last);
-        x0[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup) : uint4{0, 0, 0, 0};
-        x1[u] = live ? *reinterpret_cast<const uint4 *>(xrow + gg * kGroup + 32) : uint4{0, 0, 0, 0};
-    }
-}
-
-__device__ __forceinline__ void turn_token_rows(uint32_t lane, uint4 (&x0)[kRing], uint4 (&x1)[kRing]) {
-    const uint32_t j = lane & 15, jq = lane >> 4;
-    const int pull = (int)((4 * j + jq) * 4);       // operand lane (j, jq) takes what load lane 4 j + jq holds
-    auto turn = [&](uint4 &v) {
-        v.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x);
-        v.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y);
-        v.z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z);
-        v.w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w);
-    };
-#pragma unroll
-    for (int u = 0; u < kRing; ++u) {
-        turn(x0[u]);
-        turn(x1[u]);
-    }
-}
-
 typedef float GateUpMerge[2][kKSplit][8][64];
 
 // From the routes (thread r < n_routes brings route r) to the stored activations: the plan, the block's share of
