@@ -468,11 +468,23 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__r
                                                               const uint32_t *__restrict__ sorted_out_row,
                                                               const uint16_t *__restrict__ a, uint32_t a_stride,
                                                               uint16_t *__restrict__ out, uint32_t n_nblocks,
-                                                              uint4 *__restrict__ dump = nullptr) {
+                                                              bool nb_major, uint4 *__restrict__ dump = nullptr) {
     __shared__ __align__(16) uint4 wb[4][kTilesPerBlock][2][2][kWave];   // [buffer][tile][stream][k-half][lane]: group g lives in buffer g % 4
 
+    // Consecutive block ids go to consecutive XCDs. Many experts: all N-blocks of an M-tile share an XCD (its L2 holds
+    // the tile's A rows). One expert (the dense FFN: few M-tiles, every one against the same weights): all M-tiles of
+    // an N-block share an XCD instead, so each XCD reads its eighth of the weights once and every XCD is equally full.
     const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const uint32_t ti = (slot / n_nblocks) * 8 + xcd, nb = slot % n_nblocks;
+    uint32_t ti, nb;
+    if (nb_major) {
+        const uint32_t per_xcd = (n_nblocks + 7) / 8;
+        ti = slot / per_xcd;
+        nb = (slot % per_xcd) * 8 + xcd;
+        if (nb >= n_nblocks) return;
+    } else {
+        ti = (slot / n_nblocks) * 8 + xcd;
+        nb = slot % n_nblocks;
+    }
     if (ti >= plan->n_tiles) return;
     GemmWave gw;
     gw.tile = tiles[ti];
@@ -602,11 +614,11 @@ hipError_t launch_prefill_dump_tiles(hipStream_t s, const uint8_t *arena_layer, 
     if (gate_up) {
         const uint32_t nb = (g.gu_rb + kTilesPerBlock - 1) / kTilesPerBlock;
         hipLaunchKernelGGL((prefill_gemm_kernel<true, false, true>), dim3(nb * 8), dim3(256), 0, s, arena_layer, g, sc.plan, sc.tiles,
-                           sc.sorted_token, sc.sorted_out_row, sc.partials, g.d, sc.acts, nb, static_cast<uint4 *>(dump));
+                           sc.sorted_token, sc.sorted_out_row, sc.partials, g.d, sc.acts, nb, false, static_cast<uint4 *>(dump));
     } else {
         const uint32_t nb = (g.dn_rbp + kTilesPerBlock - 1) / kTilesPerBlock;
         hipLaunchKernelGGL((prefill_gemm_kernel<false, false, true>), dim3(nb * 8), dim3(256), 0, s, arena_layer, g, sc.plan, sc.tiles,
-                           sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, sc.partials, nb, static_cast<uint4 *>(dump));
+                           sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, sc.partials, nb, false, static_cast<uint4 *>(dump));
     }
     return hipGetLastError();
 }
@@ -646,16 +658,19 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
         x = sc.x16;
         x_stride = g.d;
     }
-    hipLaunchKernelGGL(prefill_gemm_kernel<true>, dim3(nb_gu * tile_slots), dim3(256), 0, s, arena_layer, g, sc.plan,
-                       sc.tiles, sc.sorted_token, sc.sorted_out_row, x, x_stride, sc.acts, nb_gu);
+    // grid: (N-blocks x tile slots) in either order of the kernel's block map
+    const bool nb_major = n_experts == 1;
+    auto grid_of = [&](uint32_t n_nblocks) { return nb_major ? 8 * ((n_nblocks + 7) / 8) * tile_cap : n_nblocks * tile_slots; };
+    hipLaunchKernelGGL(prefill_gemm_kernel<true>, dim3(grid_of(nb_gu)), dim3(256), 0, s, arena_layer, g, sc.plan,
+                       sc.tiles, sc.sorted_token, sc.sorted_out_row, x, x_stride, sc.acts, nb_gu, nb_major);
     timer->mark(s, FFMOE_K_PREFILL_GATE_UP);
     uint16_t *partials = partials_out ? partials_out : sc.partials;
     if (f16)
-        hipLaunchKernelGGL((prefill_gemm_kernel<false, true>), dim3(nb_dn * tile_slots), dim3(256), 0, s, arena_layer, g, sc.plan,
-                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn);
+        hipLaunchKernelGGL((prefill_gemm_kernel<false, true>), dim3(grid_of(nb_dn)), dim3(256), 0, s, arena_layer, g, sc.plan,
+                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn, nb_major);
     else
-        hipLaunchKernelGGL((prefill_gemm_kernel<false, false>), dim3(nb_dn * tile_slots), dim3(256), 0, s, arena_layer, g, sc.plan,
-                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn);
+        hipLaunchKernelGGL((prefill_gemm_kernel<false, false>), dim3(grid_of(nb_dn)), dim3(256), 0, s, arena_layer, g, sc.plan,
+                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn, nb_major);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_PREFILL_DOWN);
