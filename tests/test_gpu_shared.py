@@ -84,9 +84,10 @@ def test_shared_expert_rows(ff, oracle, torch, d, f, t):
     ctx.close()
 
 
-@pytest.mark.parametrize("d,f,t", [(128, 64, 40), (256, 192, 300), (2816, 2112, 64)])
+@pytest.mark.parametrize("d,f,t", [(128, 64, 40), (256, 192, 300), (2816, 2112, 64), (512, 640, 700)])
 def test_shared_expert_batched(ff, oracle, torch, d, f, t):
-    # more than 16 rows: the grouped GEMMs. 64 rows of U(-2, 2) at the model's shape restate
+    # more than 16 rows: the grouped GEMMs ((512, 640, 700): three M-tiles against ten and four N-blocks, so that the
+    # one-expert block map has tiles, N-blocks past the first eight and empty block slots all at once). 64 rows of U(-2, 2) at the model's shape restate
     # batchedIsNoLessAccurateThanPerToken (PrefillSharedExpertBatchedTests.swift:47-101), whose reference is
     # MoeRef.runFFN per token and whose bound is a relative L2 error below 5e-3 on FP16 outputs.
     g = oracle.seed_tree_key(0x5EED, f"shared-ffn-batched-d{d}-f{f}-t{t}")
