@@ -77,6 +77,7 @@ __global__ __launch_bounds__(kScanThreads) void prefill_scan_kernel(uint32_t n_b
     __shared__ uint32_t offset[FFMOE_MAX_EXPERTS + 1];
     __shared__ uint32_t tile_off[FFMOE_MAX_EXPERTS + 1];
     __shared__ uint32_t part[kScanThreads];                 // [chunk][e_pad]: chunk sums, then chunk bases
+    __shared__ unsigned long long scan_own[FFMOE_MAX_EXPERTS], wave_sum[FFMOE_MAX_EXPERTS / 64];
     const uint32_t e = threadIdx.x % e_pad, ch = threadIdx.x / e_pad, chunks = kScanThreads / e_pad;
     const uint32_t per = (n_blocks + chunks - 1) / chunks;
     const uint32_t b_lo = min(n_blocks, ch * per), b_hi = min(n_blocks, b_lo + per);
@@ -103,19 +104,45 @@ __global__ __launch_bounds__(kScanThreads) void prefill_scan_kernel(uint32_t n_b
         total[e] = run;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t run = 0, trun = 0;
-        for (uint32_t i = 0; i < n_experts; ++i) {
-            offset[i] = run;
-            tile_off[i] = trun;
-            run += total[i];
-            trun += (total[i] + kBM - 1) / kBM;
+    // exclusive prefix sums over the experts of (pairs, tiles), packed into one 64-bit value: four waves scan 64
+    // experts each, then add the waves in front of them
+    if (threadIdx.x < FFMOE_MAX_EXPERTS) {
+        const uint32_t i = threadIdx.x, lane = i & 63, wv = i >> 6;
+        const uint32_t n = i < n_experts ? total[i] : 0;
+        const unsigned long long own = ((unsigned long long)((n + kBM - 1) / kBM) << 32) | n;
+        unsigned long long inc = own;
+#pragma unroll
+        for (int sh = 1; sh < 64; sh <<= 1) {
+            const unsigned long long up = __shfl_up(inc, sh, 64);
+            if (lane >= (uint32_t)sh) inc += up;
         }
-        offset[n_experts] = run;
-        tile_off[n_experts] = trun;
-        plan->n_pairs = run;
-        plan->n_tiles = min(trun, max_tiles);
-        plan->expert_offset[n_experts] = run;
+        if (lane == 63) wave_sum[wv] = inc;
+        scan_own[i] = inc - own;
+    }
+    __syncthreads();
+    if (threadIdx.x < FFMOE_MAX_EXPERTS) {
+        const uint32_t i = threadIdx.x, wv = i >> 6;
+        unsigned long long base = 0;
+        for (uint32_t v = 0; v < wv; ++v) base += wave_sum[v];
+        const unsigned long long ex = base + scan_own[i];
+        if (i <= n_experts) {
+            offset[i] = (uint32_t)ex;
+            tile_off[i] = (uint32_t)(ex >> 32);
+        }
+        if (i == n_experts || (i == FFMOE_MAX_EXPERTS - 1 && n_experts == FFMOE_MAX_EXPERTS)) {
+            // the totals: the prefix in front of the first expert past the end (or, with every slot in use, the last
+            // expert's prefix plus its own share)
+            unsigned long long all = ex;
+            if (i != n_experts) {
+                const uint32_t n = total[i];
+                all += ((unsigned long long)((n + kBM - 1) / kBM) << 32) | n;
+                offset[n_experts] = (uint32_t)all;
+                tile_off[n_experts] = (uint32_t)(all >> 32);
+            }
+            plan->n_pairs = (uint32_t)all;
+            plan->n_tiles = min((uint32_t)(all >> 32), max_tiles);
+            plan->expert_offset[n_experts] = (uint32_t)all;
+        }
     }
     __syncthreads();
     if (!live) return;
@@ -150,14 +177,29 @@ __global__ __launch_bounds__(kScanThreads) void prefill_scan_kernel(uint32_t n_b
 __global__ __launch_bounds__(kSortBlock) void prefill_scatter_kernel(ItemSource src, const uint32_t *__restrict__ block_base,
                                                                      uint32_t *__restrict__ sorted_token,
                                                                      uint32_t *__restrict__ sorted_out_row) {
-    __shared__ uint32_t ex[kSortBlock];
-    const uint32_t i = blockIdx.x * kSortBlock + threadIdx.x;
+    // an item's place inside its block's share of its expert = the items of the same expert in front of it: those in
+    // the waves in front (per-wave counts in LDS) plus those in lower lanes of its own wave (a mask built from one
+    // ballot per bit of the expert number)
+    __shared__ uint32_t wave_cnt[kSortBlock / 64][FFMOE_MAX_EXPERTS];
+    static_assert(FFMOE_MAX_EXPERTS <= 256, "eight ballots tell the experts apart");
+    const uint32_t i = blockIdx.x * kSortBlock + threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (uint32_t c = threadIdx.x; c < (kSortBlock / 64) * FFMOE_MAX_EXPERTS; c += kSortBlock) (&wave_cnt[0][0])[c] = 0;
     const uint32_t e = item_expert(src, i);
-    ex[threadIdx.x] = e;
+    const bool valid = e != 0xFFFFFFFFu;
+    unsigned long long same = __ballot(valid);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const bool bit = (e >> b) & 1u;
+        const unsigned long long with = __ballot(bit);
+        same &= bit ? with : ~with;
+    }
+    const uint32_t in_front = __popcll(same & ((1ull << lane) - 1ull));
     __syncthreads();
-    if (e == 0xFFFFFFFFu) return;
-    uint32_t rank = 0;
-    for (uint32_t j = 0; j < threadIdx.x; ++j) rank += ex[j] == e ? 1u : 0u;
+    if (valid && in_front == 0) wave_cnt[wave][e] = __popcll(same);
+    __syncthreads();
+    if (!valid) return;
+    uint32_t rank = in_front;
+    for (uint32_t v = 0; v < wave; ++v) rank += wave_cnt[v][e];
     const uint32_t pos = block_base[(size_t)blockIdx.x * src.n_experts + e] + rank;
     uint32_t token, out_row;
     if (src.pairs) {
