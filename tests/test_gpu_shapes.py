@@ -19,7 +19,9 @@ SHAPES = [(64, 64, 1, 1, 1, 19),
           (128, 704, 128, 8, 16, 64),
           (448, 448, 128, 1, 16, 300),
           (2816, 64, 8, 8, 1, 17),
-          (1088, 1088, 3, 3, 5, 23)]
+          (1088, 1088, 3, 3, 5, 23),
+          (256, 128, 256, 8, 16, 300),      # the most experts a context takes: selects over four key slots per lane
+          (128, 64, 200, 4, 9, 100)]
 
 
 @pytest.mark.parametrize("d,f,e,k,t,tp", SHAPES)
