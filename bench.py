@@ -3,13 +3,15 @@
 
 Workload (BASELINE.json config 3, the one the metric is quoted on): a 16-token DFlash verify block
 through one Gemma-4-26B-A4B-shaped MoE layer (hidden 2816, 128 experts of intermediate 704, top-8
-softmax router, MLX-affine INT4 g64 experts), synthetic seeded weights and inputs. A step is one pass
-of the hot path over one block: router logits + top-8, GPU-side route planning, gate/up + GELU-tanh
-gating, down projection, router-weighted combine. Steps cycle over `--layers` distinct resident layers
-(default 30 = 12.85 GB of experts) so that no step finds its experts in the 256 MB Infinity Cache.
+softmax router, MLX-affine INT4 g64 experts), synthetic seeded weights and inputs. A layer pass is one
+pass of the hot path over the block: router logits + top-8, GPU-side route planning, gate/up +
+GELU-tanh gating, down projection, router-weighted combine. A step takes the block through the
+`--layers` distinct resident layers once (default 30 = 12.85 GB of experts), as a decode loop does, so
+that no pass finds its experts in the 256 MB Infinity Cache and the timed region of even a few steps
+is tens of milliseconds long.
 
-Prints ONE JSON line. `value` = INT4 expert bytes the step streams (distinct experts x 3,345,408 B)
-divided by the whole step time, inputs resident in HBM. `roofline` prices the dominant kernel
+Prints ONE JSON line. `value` = INT4 expert bytes the timed steps stream (distinct experts x
+3,345,408 B per layer pass) divided by their whole time, inputs resident in HBM. `roofline` prices the dominant kernel
 (gate/up) against the 8 TB/s HBM peak from HIP-event timings; `cpu_baseline` times the CPU oracle
 (a C restatement of the reference's Swift test-support CPU path) on the same block.
 """
@@ -102,8 +104,9 @@ def clocks_under_load(burst, torch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=120)
-    ap.add_argument("--warmup", type=int, default=300)
+    ap.add_argument("--steps", type=int, default=8,
+                    help="timed steps; a step = the verify block through every resident layer once (--layers layer passes)")
+    ap.add_argument("--warmup", type=int, default=2, help="untimed steps in front of the timed ones (after the settling passes)")
     ap.add_argument("--layers", type=int, default=30)
     ap.add_argument("--tokens", type=int, default=16)
     ap.add_argument("--prefill-tokens", type=int, default=3072, help="0 skips the prefill leg")
@@ -195,30 +198,38 @@ def main():
         per_expert = np.bincount(idx.cpu().numpy().astype(np.int64).ravel(), minlength=E)
         assert int((per_expert > 0).sum()) == live[-1], "plan and routes disagree on the live experts"
         tokens_per_expert += np.bincount(per_expert[per_expert > 0], minlength=T * K + 1)
-    for i in range(args.warmup):
+    # A step = the block through all L resident layers, one after the other, as a decode loop runs them (L layer
+    # passes; every pass streams its own layer's experts from HBM). The clocks and the address translation caches
+    # settle over the first ~15 ms of back-to-back passes (with 30 passes in front the timed ones still ran 5 % below
+    # the settled rate), so kSettlePasses untimed passes come first, whatever --warmup says; then the warm-up steps,
+    # then exactly --steps timed steps between two device synchronisations.
+    kSettlePasses = 300
+    n_warm, n_timed = args.warmup * L, args.steps * L
+    for i in range(kSettlePasses + n_warm):
         step(i % L)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(n_timed):
         step(i % L)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
-    bytes_total = sum(live[i % L] for i in range(args.steps)) * EXPERT_BYTES
+    bytes_total = args.steps * sum(live) * EXPERT_BYTES
     value = bytes_total / elapsed / 1e9
 
     # spread of the step time: one event after every step (a record costs the stream a few microseconds, so
     # these intervals sit above ms_per_step by about one record; the spread is what they are for)
-    evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    n_spread = min(n_timed, 240)
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(n_spread + 1)]
     evs[0].record()
-    for i in range(args.steps):
+    for i in range(n_spread):
         step(i % L)
         evs[i + 1].record()
     torch.cuda.synchronize()
-    per_step = np.array([evs[i].elapsed_time(evs[i + 1]) * 1e3 for i in range(args.steps)])
+    per_step = np.array([evs[i].elapsed_time(evs[i + 1]) * 1e3 for i in range(n_spread)])
     step_spread = {"median": round(float(np.median(per_step)), 2), "p10": round(float(np.percentile(per_step, 10)), 2),
-                   "p90": round(float(np.percentile(per_step, 90)), 2), "n": int(args.steps),
-                   "note": "per-step HIP-event intervals, each including one event record"}
+                   "p90": round(float(np.percentile(per_step, 90)), 2), "n": int(n_spread),
+                   "note": "per-layer-pass HIP-event intervals, each including one event record"}
     props = torch.cuda.get_device_properties(0)
     device_info = {"name": props.name, "compute_units": props.multi_processor_count,
                    "hbm_GiB": round(props.total_memory / 2 ** 30, 1), "torch": torch.__version__, "hip": torch.version.hip,
@@ -236,7 +247,7 @@ def main():
     # per-kernel times (HIP events on the launch stream) for the same steps
     ctx.set_profiling(True)
     ctx.profile(reset=True)
-    for i in range(args.steps):
+    for i in range(n_timed):
         step(i % L)
     prof = ctx.profile(reset=True)
     ctx.set_profiling(False)
@@ -249,13 +260,13 @@ def main():
     def kernel_times(pr):
         return {k_: round((v[0] / v[1] - gap_ms) * 1e3, 2) for k_, v in pr.items() if k_ != "event_gap"}
     kernel_us = kernel_times(prof)
-    live_sum = sum(live[i % L] for i in range(args.steps))
+    live_sum = args.steps * sum(live)
     if "route_gate_up" in prof:
         # router logits, select and gate/up share one launch: its bytes are the live experts' gate/up weights plus the
         # router's [E][D] bf16 matrix, its time holds the routing chain as well
         dominant = "route_gate_up_persistent (router logits + top-8 select + gate/up in one launch)"
         gu_ms = prof["route_gate_up"][0] - gap_ms * prof["route_gate_up"][1]
-        achieved = (live_sum * GATE_UP_BYTES + args.steps * E * D * 2) / (gu_ms * 1e-3) / 1e9
+        achieved = (live_sum * GATE_UP_BYTES + n_timed * E * D * 2) / (gu_ms * 1e-3) / 1e9
     else:
         dominant = "skinny_gate_up_persistent"
         gu_ms = prof["gate_up"][0] - gap_ms * prof["gate_up"][1]
@@ -265,24 +276,24 @@ def main():
     # without the routing chain in front of it, and what the one-call form gains on the whole step
     split = None
     if "route_gate_up" in prof:
-        for i in range(args.warmup):
+        for i in range(max(n_warm, 2 * L)):
             step_split(i % L)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(args.steps):
+        for i in range(n_timed):
             step_split(i % L)
         torch.cuda.synchronize()
-        split_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        split_ms = (time.perf_counter() - t0) * 1e3 / n_timed
         ctx.set_profiling(True)
         ctx.profile(reset=True)
-        for i in range(args.steps):
+        for i in range(n_timed):
             step_split(i % L)
         sprof = ctx.profile(reset=True)
         ctx.set_profiling(False)
         sgu_ms = sprof["gate_up"][0] - gap_ms * sprof["gate_up"][1]
         sgbs = live_sum * GATE_UP_BYTES / (sgu_ms * 1e-3) / 1e9
         split = {"calls": "ffmoe_router + ffmoe_verify (router logits, select, gate/up, down, combine: five launches)",
-                 "us_per_step": round(split_ms * 1e3, 2), "kernel_us": kernel_times(sprof),
+                 "us_per_layer_pass": round(split_ms * 1e3, 2), "kernel_us": kernel_times(sprof),
                  "gate_up_kernel": "skinny_gate_up_persistent", "gate_up_GBs": round(sgbs, 1),
                  "gate_up_frac_hbm_peak": round(sgbs / HBM_PEAK_GBS, 4)}
 
@@ -329,9 +340,9 @@ def main():
             rc |= Lib.ffmoe_prefill(h, stream, layer, pxp, D, TP, ppi, ppw, ppy, C.byref(err))
             if rc:
                 raise RuntimeError(err.value)
-        psteps = max(4, min(args.steps, 2 * L))
-        for i in range(L):              # one pass over the layers (14 ms): clocks and address translation settled
-            pstep(i)
+        psteps = 2 * L                 # two passes over the layers (25 ms), whatever --steps says
+        for i in range(2 * L):          # and two in front of them: clocks and address translation settled
+            pstep(i % L)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(psteps):
@@ -735,24 +746,28 @@ def main():
     out = {
         "metric": "MoE-layer INT4 weight GB/s (% HBM peak) @16-tok verify; prefill MoE tok/s",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 5), "us_per_layer_pass": round(ms_per_step * 1e3 / L, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"config 3: {T}-token DFlash verify block through one MoE layer, hidden {D}, "
-                               f"{E} experts x intermediate {F}, top-{K}, INT4 g64; steps cycle {L} resident layers",
-                   "tokens": T, "layers_resident": L, "distinct_experts_mean": round(float(np.mean(live)), 1),
+        "config": {"workload": f"config 3: {T}-token DFlash verify block through the MoE layer, hidden {D}, "
+                               f"{E} experts x intermediate {F}, top-{K}, INT4 g64; a step takes the block through "
+                               f"the {L} resident layers once ({L} layer passes, each streaming its own layer's experts)",
+                   "tokens": T, "layers_resident": L, "layer_passes_per_step": L,
+                   "settle_layer_passes_before_warmup": kSettlePasses,
+                   "distinct_experts_mean": round(float(np.mean(live)), 1),
                    "distinct_experts_min": int(min(live)), "distinct_experts_max": int(max(live)),
-                   "expert_bytes_per_step_mean": int(np.mean(live) * EXPERT_BYTES),
+                   "expert_bytes_per_step": int(sum(live) * EXPERT_BYTES),
+                   "expert_bytes_per_layer_pass_mean": int(np.mean(live) * EXPERT_BYTES),
                    "routes_per_live_expert_hist": {str(n): int(c) for n, c in enumerate(tokens_per_expert) if c},
                    "routes_per_live_expert_note": f"over the {L} layers: how many live experts receive n of the block's {T * K} routes"},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
-        "step_us": step_spread,
+        "layer_pass_us": step_spread,
         "device": device_info,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": traffic.get("verify16_route_gate_up" if "route_gate_up" in prof else "verify16_gate_up") if (T == 16 and L == 30) else None,
                      "traffic_unit": f"bytes per launch (rocprofv3 --pmc, profiles/{TRAFFIC_FILE.name})",
-                     "algorithmic_bytes_per_launch": int(achieved * 1e9 * gu_ms * 1e-3 / args.steps),
-                     "avg_kernel_us": round(gu_ms * 1e3 / args.steps, 2),
+                     "algorithmic_bytes_per_launch": int(achieved * 1e9 * gu_ms * 1e-3 / n_timed),
+                     "avg_kernel_us": round(gu_ms * 1e3 / n_timed, 2),
                      "note": ("the launch also holds the routing chain (logits, select, routes: about 6 us before the first weight is "
                               "requested); five_launch_form.gate_up_* is the same stream as a launch of its own") if split else None},
         "five_launch_form": split,
