@@ -50,8 +50,9 @@ struct ffmoe_ctx {
     uint16_t *acts = nullptr;        // [16*top_k][F]
     float *partials = nullptr;       // [16*top_k][D]
     RouteMail *mail = nullptr;       // hand-over words of ffmoe_route_verify's one-launch router + gate/up
-    unsigned long long handover_ticks = 20000000ull;      // 0.2 s at 100 MHz
+    unsigned long long handover_ticks = FFMOE_DEFAULT_HANDOVER_TICKS;
     bool one_launch_routing = true;
+    uint32_t route_resident_blocks = 0;     // occupancy of the one-launch routing kernel x compute units
     PrefillScratch pf{};
     uint32_t max_pairs = 0;
     // dense FFN (n_experts == 1, top_k == 1): every row routes to expert 0 with weight 1
@@ -152,7 +153,8 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     FF_HIP(hipGetDeviceCount(&count));
     if (device < 0 || device >= count) return fail(err, FFMOE_ERR_INVALID, "device %d not present (%d visible)", device, count);
     FF_HIP(hipSetDevice(device));
-    FF_HIP(resolve_static_scratch(device));
+    // a device on which the array has no address runs everything but ffmoe_verify_static, which then says so
+    if (resolve_static_scratch(device) != hipSuccess) (void)hipGetLastError();
 
     ffmoe_ctx *ctx = new (std::nothrow) ffmoe_ctx();
     if (!ctx) return fail(err, FFMOE_ERR_ALLOC, "out of host memory");
@@ -162,6 +164,7 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
         ctx->n_cus = (uint32_t)cus;
     }
+    ctx->route_resident_blocks = route_launch_resident_blocks(ctx->n_cus);
     ctx->shape = *shape;
     ctx->geom = make_geom(shape->d, shape->f);
     // an expert's tile regions are addressed through buffer descriptors with 32-bit sizes and offsets
@@ -505,7 +508,8 @@ int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint1
     if (layer >= ctx->layers.size()) return fail(err, FFMOE_ERR_INVALID, "layer %u out of range", layer);
     const ffmoe_layer &l = ctx->layers[layer];
     const RouteFusion route{RouterWeights{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale}, router_x,
-                            router_x_stride, ctx->logits, ctx->mail, ctx->handover_ticks, ctx->one_launch_routing};
+                            router_x_stride, ctx->logits, ctx->mail, ctx->handover_ticks, ctx->one_launch_routing,
+                            ctx->route_resident_blocks};
     return verify_common(ctx, stream, layer, x, x_stride, t, out_idx, out_w, residual, y, nullptr, err, nullptr, &route);
 }
 
@@ -534,11 +538,28 @@ int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char
     if (!n_live) return fail(err, FFMOE_ERR_INVALID, "null argument");
     FF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     FF_HIP(hipMemcpy(n_live, &ctx->plan->n_live, sizeof(uint32_t), hipMemcpyDeviceToHost));
-    uint32_t faults = 0;
-    FF_HIP(hipMemcpy(&faults, &ctx->mail->faults, sizeof(uint32_t), hipMemcpyDeviceToHost));
-    if (faults)
-        return fail(err, FFMOE_ERR_RUNTIME, "%u hand-over polls of ffmoe_route_verify gave up (the launch was not resident as a whole)",
-                    faults);
+    return FFMOE_OK;
+}
+
+int ffmoe_probe_stream(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint32_t n_live, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, true, false, err)) return rc;
+    if (n_live == 0 || n_live > ctx->shape.n_experts)
+        return fail(err, FFMOE_ERR_INVALID, "n_live = %u outside 1...%u", n_live, ctx->shape.n_experts);
+    if ((ctx->geom.gd + 3) / 4 > 11 || ctx->geom.gf > 11)
+        return fail(err, FFMOE_ERR_INVALID, "the stream probe covers the persistent kernels' shapes (d <= 2816, f <= 704)");
+    // the sink: the first words of the un-weighted rows' scratch (never written on real data, see the launch)
+    FF_HIP(launch_probe_stream(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
+                               ctx->shape.n_experts, n_live, ctx->n_cus, reinterpret_cast<uint32_t *>(ctx->partials),
+                               &ctx->timer));
+    return FFMOE_OK;
+}
+
+int ffmoe_handover_giveups(ffmoe_ctx *ctx, void *stream, uint32_t *count, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!count) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    FF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    FF_HIP(hipMemcpy(count, &ctx->mail->faults, sizeof(uint32_t), hipMemcpyDeviceToHost));
     return FFMOE_OK;
 }
 

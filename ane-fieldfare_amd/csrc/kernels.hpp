@@ -132,8 +132,9 @@ struct RouteFusion {
     uint32_t router_x_stride;
     float *logits;          // scratch of the two-launch router (used when the one-launch form does not apply)
     RouteMail *mail;
-    unsigned long long poll_ticks;      // how long a block waits for a hand-over word (wall_clock64 ticks, 100 MHz)
+    unsigned long long poll_ticks;      // how long a wave waits for a hand-over word (wall_clock64 ticks, 100 MHz)
     bool one_launch;                    // false: the router runs as launches of its own in front of the expert pass
+    uint32_t resident_blocks;           // blocks of the one-launch form the GPU holds at once (0: unknown, use the launches)
 };
 
 // repack.hip
@@ -156,6 +157,10 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
                          VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer,
                          bool f16 = false, const RouteFusion *route = nullptr);
+uint32_t route_launch_resident_blocks(uint32_t n_cus);
+// the two expert kernels' weight loads for n_live experts and nothing else (`sink`: 256 words nobody reads)
+hipError_t launch_probe_stream(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t n_live,
+                               uint32_t n_cus, uint32_t *sink, KernelTimer *timer);
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,
                                      uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d, bool f16 = false);
 

@@ -292,6 +292,18 @@ __global__ __launch_bounds__(256) void skinny_down_kernel(const uint8_t *__restr
 // block walks a range of 16-row blocks of its expert; its four waves split K and meet in LDS per row block
 // (partials added in wave order), each wave finishing a quarter of the token slots.
 typedef float GateUpMerge[2][kKSplit][8][64];
+constexpr unsigned long long kFirstPollTicks = 100;      // 1 us (100 MHz ticks) between a block's own logits and its first look at the routes
+
+// The token rows into the operand layout and, per group, the sum of its inputs per token column (once for all the
+// tile rows a wave walks). Depends on the rows only: the launch that waits for its routes does this while it waits
+// (`prepared` in gate_up_rows; measured at 1 / 8 / 16 rows: 1.0 / 1.3 / 1.5 us per call less than behind the first
+// weight request), the launch that is handed its routes does it behind that request.
+template <bool F16>
+__device__ __forceinline__ void prepare_token_rows(uint32_t lane, uint4 (&x0)[kRing], uint4 (&x1)[kRing], f32x4 (&sx)[kRing]) {
+    turn_token_rows(lane, x0, x1);
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) sx[u] = group_input_sum<F16>(x0[u], x1[u]);
+}
 
 // From the routes (thread r < n_routes brings route r) to the stored activations: the plan, the block's share of
 // its expert's row blocks, the weight stream. x0 / x1: the wave's token rows as load_token_rows() left them.
@@ -299,8 +311,8 @@ template <bool F16>
 __device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps, const uint8_t *__restrict__ arena_layer,
                                              const ArenaGeom &g, uint32_t top_k, uint32_t n_experts, uint32_t route_idx,
                                              uint16_t route_w, uint32_t n_routes, VerifyPlan *__restrict__ plan,
-                                             const KSlice &k, uint4 (&x0)[kRing], uint4 (&x1)[kRing],
-                                             uint16_t *__restrict__ acts) {
+                                             const KSlice &k, uint4 (&x0)[kRing], uint4 (&x1)[kRing], f32x4 (&sx)[kRing],
+                                             bool prepared, uint16_t *__restrict__ acts) {
     const uint32_t rows = n_routes / top_k;
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15, jq = lane >> 4;
@@ -331,11 +343,7 @@ __device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps
     }
     if (plan_out) build_plan_routes(ps, n_routes, plan_out, route_expert);
     if (!has_rows) return;
-    turn_token_rows(lane, x0, x1);
-    // per group: the sum of its inputs per token column, once for all the tile rows this wave walks
-    f32x4 sx[kRing];
-#pragma unroll
-    for (int u = 0; u < kRing; ++u) sx[u] = group_input_sum<F16>(x0[u], x1[u]);
+    if (!prepared) prepare_token_rows<F16>(lane, x0, x1, sx);
     // this lane finishes token column 4 jq + ks; `stores` = which of that row's top_k routes go to the expert
     // (one bit at most unless a row names an expert twice)
     const uint32_t col = 4 * jq + ks;
@@ -398,7 +406,8 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     const KSlice k = k_slice(g.gd, ks);
     uint4 x0[kRing], x1[kRing];
     load_token_rows(x, x_stride, n_routes / top_k, lane, k, x0, x1);
-    gate_up_rows<F16>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, acts);
+    f32x4 sx[kRing];
+    gate_up_rows<F16>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, sx, false, acts);
 }
 
 // Router and gate/up of a decode step or verify block in ONE launch: the logits, the top-k select and the routes'
@@ -409,21 +418,71 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
 // producers wait for nobody. Measured on this part, such an edge costs 0.9 us against 2.4 us for a kernel boundary.
 //   1. logits: block b takes work items b, b + grid, ... = (expert, chunk of four rows) as router_small_kernel does,
 //      same pinned order, and writes the four logits as words mail->logits[row][expert].
-//   2. select: wave 1 of block r < rows polls row r's words, runs the select and writes the row's routes as words
+//   2. select: the four waves of block r < rows poll row r's words and rank its candidates together
+//      (block_topk_select); wave 1 writes the row's routes as words
 //      mail->routes[row * top_k + rank] = {epoch, weight bits << 16 | expert} (and as plain idx / w for the caller and
 //      the combine).
 //   3. every block polls the routes, then continues as the kernel above. The token rows of the expert pass are
 //      requested between 1 and 3, so they arrive while the block waits.
 // The epoch is read from mail->epoch by every block at its start and is advanced by a later launch of the same call
-// (the combine), which keeps a replayed HIP graph correct. Every block of the grid has to be resident at once (the
-// grid is at most two blocks per compute unit, the kernel's occupancy); a poll gives up after `poll_ticks` (100 MHz ticks;
-// 0.2 s by default), counts a fault in mail->faults and goes on with empty routes.
+// (the combine), which keeps a replayed HIP graph correct. The hand-overs are fast when every block of the grid is
+// resident at once (the grid is at most the kernel's occupancy on a GPU the stream has to itself), and the results
+// do not depend on it: a wave whose poll has waited `poll_ticks` (100 MHz ticks) stops waiting and makes what it
+// waited for itself - the row's logits in step 2, the rows' logits, select and weights in step 3 - with the same
+// arithmetic in the same order, so the call returns the same bits, later. mail->faults counts such waves.
+
+// The next epoch, never 0: words that were never written are zero and must not look current after a wrap.
+__device__ __forceinline__ void advance_epoch(RouteMail *mail) {
+    const uint32_t next = mail->epoch + 1u;
+    mail->epoch = next ? next : 1u;
+}
+// A call that cannot launch what follows its routing launch still has to retire the words that launch wrote.
+__global__ void advance_epoch_kernel(RouteMail *mail) { advance_epoch(mail); }
 
 __device__ __forceinline__ unsigned long long mail_load(const unsigned long long *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void mail_store(unsigned long long *p, unsigned long long v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The weight bits topk_store writes for the rank a lane holds (lane < top_k).
+template <bool F16>
+__device__ __forceinline__ uint16_t route_weight_bits(const TopkRow &tr, const uint16_t *__restrict__ per_expert_scale) {
+    const float gain = per_expert_scale ? bf16_to_f32(per_expert_scale[tr.idx]) : 1.0f;
+    return Act<F16>::round(tr.ex / tr.sum * gain);
+}
+
+// What a wave does when a hand-over never arrives: the logits of rows t0 .. t_last (at most kChunkTokens of them)
+// against every expert by this wave alone, in the pinned order - the four sub-accumulators one after the other
+// instead of one per wave, merged as router_finish merges them - as select keys (slot c, lane l: expert 64 c + l).
+// Slow (hundreds of dependent memory round trips) and exact: the bits of the block-wide form.
+template <bool W_F32, bool F16>
+__device__ __forceinline__ void lone_wave_keys(const void *__restrict__ router_w, const uint16_t *__restrict__ effective_scale,
+                                               const uint16_t *__restrict__ router_x, uint32_t router_x_stride,
+                                               uint32_t n_experts, uint32_t d, uint32_t t0, uint32_t t_last, uint32_t lane,
+                                               uint32_t (&keys)[kChunkTokens][4]) {
+#pragma unroll
+    for (int r = 0; r < kChunkTokens; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) keys[r][c] = 0u;
+    for (uint32_t e = 0; e < n_experts; ++e) {
+        float p0[kChunkTokens] = {0.f, 0.f, 0.f, 0.f}, p1[kChunkTokens] = {0.f, 0.f, 0.f, 0.f};
+        float p2[kChunkTokens] = {0.f, 0.f, 0.f, 0.f}, p3[kChunkTokens] = {0.f, 0.f, 0.f, 0.f};
+        accumulate_sub<W_F32, F16 ? 2 : 1>(router_w, effective_scale, router_x, router_x_stride, e, d, 0, lane, t0, t_last, p0);
+        accumulate_sub<W_F32, F16 ? 2 : 1>(router_w, effective_scale, router_x, router_x_stride, e, d, 1, lane, t0, t_last, p1);
+        accumulate_sub<W_F32, F16 ? 2 : 1>(router_w, effective_scale, router_x, router_x_stride, e, d, 2, lane, t0, t_last, p2);
+        accumulate_sub<W_F32, F16 ? 2 : 1>(router_w, effective_scale, router_x, router_x_stride, e, d, 3, lane, t0, t_last, p3);
+        const bool holder = lane == (e & 63u);
+#pragma unroll
+        for (int r = 0; r < kChunkTokens; ++r) {
+            const float v = wave_butterfly_sum((p0[r] + p1[r]) + (p2[r] + p3[r]));
+            const uint32_t key = v > -INFINITY ? orderable(v) : 0u;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (holder && (e >> 6) == (uint32_t)c) keys[r][c] = key;
+        }
+    }
 }
 
 template <bool W_F32, bool F16>
@@ -470,13 +529,12 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
     load_token_rows(x, x_stride, rows, lane, k, x0, x1);
 
     const unsigned long long t_start = wall_clock64();
-    // 2. select (one wave per row)
-    if (ks == 1 && blockIdx.x < rows) {
+    // 2. select: the four waves of block r < rows rank row r's candidates together, wave 1 publishes the routes
+    if (blockIdx.x < rows) {
         const uint32_t row = blockIdx.x;
         TopkRow tr;
-        bool ok;
         for (;;) {
-            ok = true;
+            bool ok = true;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint32_t e = c * 64 + lane;
@@ -491,28 +549,37 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
             }
             if (__all(ok)) break;
             if (wall_clock64() - t_start > poll_ticks) {
-                if (lane == 0) atomicAdd(&mail->faults, 1u);
+                // the row's logits are not coming (a block that makes them is not running): this wave makes them itself
+                if (lane == 0 && ks == 1) atomicAdd(&mail->faults, 1u);
+                uint32_t keys[kChunkTokens][4];
+                lone_wave_keys<W_F32, F16>(router_w, effective_scale, router_x, router_x_stride, n_experts, g.d, row, row, lane, keys);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) tr.key[c] = 0u;      // no candidates: weights 0, nothing is routed
+                for (int c = 0; c < 4; ++c) tr.key[c] = keys[0][c];
                 break;
             }
             __builtin_amdgcn_s_sleep(1);
         }
-        if (n_experts <= 128) topk_select<2>(tr, top_k, lane);      // two key slots can hold a candidate: half the ballots per round
-        else topk_select<4>(tr, top_k, lane);
-        topk_store(tr, per_expert_scale, top_k, out_idx + (size_t)row * top_k, out_w + (size_t)row * top_k, lane, F16);
-        if (lane < top_k) {
-            // the same weight bits topk_store wrote
-            const float gain = per_expert_scale ? bf16_to_f32(per_expert_scale[tr.idx]) : 1.0f;
-            const uint32_t wbits = Act<F16>::round(tr.ex / tr.sum * gain);
-            mail_store(&mail->routes[row * top_k + lane], stamp | (wbits << 16) | (tr.idx & 0xFFFFu));
+        uint32_t(*s_cnt)[4][64] = reinterpret_cast<uint32_t(*)[4][64]>(&s_red[0][2][0][0]);    // the 4 KiB behind the logits' partial sums
+        if (n_experts <= 128) block_topk_select<2>(tr, top_k, lane, ks, 1, s_cnt);
+        else block_topk_select<4>(tr, top_k, lane, ks, 1, s_cnt);
+        if (ks == 1) {
+            topk_store(tr, per_expert_scale, top_k, out_idx + (size_t)row * top_k, out_w + (size_t)row * top_k, lane, F16);
+            if (lane < top_k)
+                mail_store(&mail->routes[row * top_k + lane], stamp | ((unsigned long long)route_weight_bits<F16>(tr, per_expert_scale) << 16) | (tr.idx & 0xFFFFu));
         }
     }
+    // the rows into operand order while the routes are on their way
+    f32x4 sx[kRing];
+    prepare_token_rows<F16>(lane, x0, x1, sx);
     // 3. the routes
     uint32_t route_idx = 0;
     uint16_t route_w = 0;
     if (ks * 64 < n_routes) {
         const bool mine = threadIdx.x < n_routes;
+        // the routes cannot be there yet: the logits' hand-over and the select come first (3 us at least). Every read
+        // of the words that is spared until then is one request less for the few lines that all blocks ask for
+        // (measured: 0.35 us per call; three reads in flight per wave instead of one cost 0.7 to 1.5 us)
+        while (wall_clock64() - t_start < kFirstPollTicks) __builtin_amdgcn_s_sleep(8);
         for (;;) {
             const unsigned long long word = mine ? mail_load(&mail->routes[threadIdx.x]) : stamp;
             if (__all((uint32_t)(word >> 32) == epoch)) {
@@ -521,13 +588,36 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
                 break;
             }
             if (wall_clock64() - t_start > poll_ticks) {
+                // the routes are not coming (a block that selects is not running): this wave routes the rows of its
+                // 64 routes itself - the same logits, select and weights, so the same bits
                 if (lane == 0) atomicAdd(&mail->faults, 1u);
-                break;          // empty routes: weight 0 takes no part
+                const uint32_t r_first = (ks * 64) / top_k, r_last = min(rows - 1, (ks * 64 + 63) / top_k);
+                const uint32_t my_row = threadIdx.x / top_k, my_rank = threadIdx.x % top_k;
+                for (uint32_t t0 = r_first; t0 <= r_last; t0 += kChunkTokens) {
+                    uint32_t keys[kChunkTokens][4];
+                    lone_wave_keys<W_F32, F16>(router_w, effective_scale, router_x, router_x_stride, n_experts, g.d, t0,
+                                               min(t0 + kChunkTokens - 1, rows - 1), lane, keys);
+#pragma unroll
+                    for (int i = 0; i < kChunkTokens; ++i) {
+                        TopkRow tr;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) tr.key[c] = keys[i][c];
+                        if (n_experts <= 128) topk_select<2>(tr, top_k, lane);
+                        else topk_select<4>(tr, top_k, lane);
+                        const uint32_t packed = ((uint32_t)route_weight_bits<F16>(tr, per_expert_scale) << 16) | (tr.idx & 0xFFFFu);
+                        const uint32_t got = (uint32_t)__shfl((int)packed, (int)my_rank, 64);
+                        if (mine && my_row == t0 + i) {
+                            route_idx = got & 0xFFFFu;
+                            route_w = (uint16_t)(got >> 16);
+                        }
+                    }
+                }
+                break;
             }
             __builtin_amdgcn_s_sleep(1);
         }
     }
-    gate_up_rows<F16>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, acts);
+    gate_up_rows<F16>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, sx, true, acts);
 }
 
 // down projection with the expert's activation rows in LDS: one block = four consecutive 32-row tile rows of one
@@ -537,10 +627,18 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
 // wave per tile row reads them in 10 us, a persistent form's 1,024 waves of four to five tile rows each in 15 us.
 // With five blocks per compute unit the blocks of up to 58 live experts are all resident from the start.
 // Order of the requests: the slot's count and expert (scalar loads; a slot past the last live expert holds n = 0
-// and its block leaves before it has issued anything else), the routes, then the activation rows and only then
-// the weights - vector loads return in order, so rows requested behind 11 KiB of weights arrive after them and
-// hold the first product back until the last tile is there; in front of them every tile is consumed as it lands.
+// and its block leaves before it has issued anything else), the routes, then the first pieces of the activation rows
+// and only then the weights. (The rows sit two dependent round trips behind the slot; a form that found them from
+// the slot alone - the gate/up kernel storing them per expert - ran at the same speed: they are not what the first
+// product waits for.)
 constexpr int kDownLdsRow = kRing * kGroup * 2 + 16;      // bytes per activation row in LDS, padded against bank conflicts
+// Weight tiles a wave has in flight. With all eleven requested at once the compute unit's twenty waves are served one
+// after the other - a wave's tiles arrive in a burst, the last wave's burst at the very end of the stream, and its
+// eleven products (3 us) run after everything else has finished. With four in flight and a refill per product the
+// waves advance together and the stream ends with about one product per wave: 15.8 -> 13.5 us per launch
+// (3 / 4 / 6 / 11 in flight: 13.8 / 13.5 / 14.2 / 15.8 us; four tiles x twenty waves = 80 KiB per compute unit in
+// flight still covers the memory latency).
+constexpr int kDownDepth = 4;
 constexpr int kDownEarly = 2;      // 16-byte pieces of the activation rows a thread requests ahead of the weights (covers 5 rows)
 
 template <bool OUT_BF16, bool F16>
@@ -576,7 +674,7 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
     WeightRing ring;
     if (has_row) {
 #pragma unroll
-        for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb * ng + min((uint32_t)u, g_last), lane);
+        for (int u = 0; u < kDownDepth; ++u) ring_fill(ring, u, src, rb * ng + min((uint32_t)u, g_last), lane);
     }
     if (threadIdx.x < (uint32_t)kMaxRows) s_route[threadIdx.x] = threadIdx.x < n ? route_t : 0u;
 #pragma unroll
@@ -607,7 +705,11 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
         const uint4 x0 = *reinterpret_cast<const uint4 *>(xrow + gg * (kGroup * 2));
         const uint4 x1 = *reinterpret_cast<const uint4 *>(xrow + gg * (kGroup * 2) + 64);
         const f32x4 sx = group_input_sum<F16>(x0, x1);
-        ring_step<F16, false>(ring, u, live, x0, x1, sx, tot, src, 0u, lane);
+        // consume slot u % kDownDepth; the load that refills it (group u + kDownDepth) starts inside the step
+        if (u + kDownDepth < kRing)
+            ring_step<F16, true>(ring, u % kDownDepth, live, x0, x1, sx, tot, src, rb * ng + min((uint32_t)(u + kDownDepth), g_last), lane);
+        else
+            ring_step<F16, false>(ring, u % kDownDepth, live, x0, x1, sx, tot, src, 0u, lane);
         // The running sums are pinned here: left alone, the compiler sinks the scale-and-bias arithmetic of every
         // group into the branches of the stores at the end and carries all eleven groups' matrix results there,
         // which does not fit the register budget.
@@ -748,7 +850,7 @@ __global__ __launch_bounds__(512, 1) void decode_down_combine_kernel(const uint8
                                                                      const uint16_t *__restrict__ residual,
                                                                      uint16_t *__restrict__ y, RouteMail *mail) {
     __shared__ float s_row[8][2 * kTileRows];
-    if (mail && blockIdx.x == 0 && threadIdx.x == 0) mail->epoch += 1;      // the routing launch of this call has read it
+    if (mail && blockIdx.x == 0 && threadIdx.x == 0) advance_epoch(mail);      // the routing launch of this call has read it
     __shared__ float s_w[8];
     const uint32_t lane = threadIdx.x & 63, r = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t rb = blockIdx.x, j = lane & 15, jq = lane >> 4;
@@ -814,7 +916,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                                                       const uint16_t *__restrict__ residual, uint32_t top_k,
                                                       uint32_t d, uint16_t *__restrict__ y, RouteMail *mail) {
     const uint32_t tok = blockIdx.y;
-    if (mail && blockIdx.x == 0 && tok == 0 && threadIdx.x == 0) mail->epoch += 1;      // the routing launch of this call has read it
+    if (mail && blockIdx.x == 0 && tok == 0 && threadIdx.x == 0) advance_epoch(mail);      // the routing launch of this call has read it
     const uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (c >= d) return;
     // One round trip: the routes' weights and validity and all eight rows are requested together. A row the plan
@@ -881,8 +983,9 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     // router and gate/up when the expert fits the persistent kernel, the combine follows in this call (it advances
     // the epoch) and the router rows are 8-byte aligned; otherwise the router's own two launches go first.
     const bool fits_ring = (g.gd + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
-    const bool fuse = route && route->one_launch && fits_ring && y && !partials_bf16 && top_k <= 8 && n_experts <= FFMOE_MAX_EXPERTS &&
-                      reinterpret_cast<uintptr_t>(route->router_x) % 8 == 0 && route->router_x_stride % 4 == 0;
+    const bool fuse = route && route->one_launch && route->resident_blocks >= t && fits_ring && y && !partials_bf16 && top_k <= 8 &&
+                      n_experts <= FFMOE_MAX_EXPERTS && reinterpret_cast<uintptr_t>(route->router_x) % 8 == 0 &&
+                      route->router_x_stride % 4 == 0;
     if (route && !fuse) {
         const hipError_t e = launch_router(s, route->rw, route->router_x, route->router_x_stride, t, n_experts, g.d, top_k,
                                            route->logits, const_cast<uint32_t *>(idx), const_cast<uint16_t *>(w), timer, F16);
@@ -895,9 +998,10 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     const bool dn_whole = g.gf <= (uint32_t)kRing;                                     // a wave holds all of K
     const bool dn_ksplit = !dn_whole && (g.gf + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
     const uint32_t resident = 2 * n_cus;       // blocks the chip holds at once (__launch_bounds__(256, 2))
+    const bool decode_form = t == 1 && dn_whole && !partials_bf16 && top_k <= 8;
     if (fuse) {
-        // at least one block per row (its second wave selects the row's routes), at most what is resident at once
-        const uint32_t blocks = min(resident, max(max(slots, t), min(resident, slots * g.gu_rb)));
+        // at least one block per row (it selects the row's routes), at most what is resident at once
+        const uint32_t blocks = min(route->resident_blocks, max(max(slots, t), min(route->resident_blocks, slots * g.gu_rb)));
 #define FFMOE_ROUTE_GU(WF)                                                                                                  \
     hipLaunchKernelGGL((route_gate_up_persistent<WF, F16>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, \
                        route->rw.w, route->rw.effective_scale, route->rw.per_expert_scale, route->router_x,                  \
@@ -921,13 +1025,23 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     if (e != hipSuccess) return e;
     timer->mark(s, fuse ? FFMOE_K_ROUTE_GATE_UP : FFMOE_K_GATE_UP);
     RouteMail *const mail = fuse ? route->mail : nullptr;
-    if (t == 1 && dn_whole && !partials_bf16 && top_k <= 8) {
+    // from here on the routing launch's words are out: whatever else fails, the epoch moves on, or the next call
+    // would take this call's words for its own
+    auto give_up = [&](hipError_t why) {
+        if (mail) hipLaunchKernelGGL(advance_epoch_kernel, dim3(1), dim3(1), 0, s, mail);
+        (void)hipGetLastError();
+        timer->finish();
+        return why;
+    };
+    if (decode_form) {
         // a decode step: down projection and combine in one launch (its time sits in the down slot)
         hipLaunchKernelGGL(decode_down_combine_kernel<F16>, dim3(g.dn_rbp), dim3(512), 0, s, arena_layer, g, n_experts, top_k, idx,
                            w, acts, residual, y, mail);
+        e = hipGetLastError();
+        if (e != hipSuccess) return give_up(e);
         timer->mark(s, FFMOE_K_DOWN);
         timer->finish();
-        return hipGetLastError();
+        return hipSuccess;
     }
     const uint32_t dn_parts = (g.dn_rbp + 3) / 4;          // blocks per expert of the LDS form: four tile rows each
     const dim3 dn_grid = dn_whole    ? dim3(slots * dn_parts)
@@ -952,16 +1066,121 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     FFMOE_DOWN(false);
 #undef FFMOE_DOWN
     e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess) return give_up(e);
     timer->mark(s, FFMOE_K_DOWN);
     hipLaunchKernelGGL(combine_kernel<F16>, dim3((g.d / 4 + 255) / 256, t), dim3(256), 0, s, partials_f32, w, plan, residual,
                        top_k, g.d, y, mail);
+    e = hipGetLastError();
+    if (e != hipSuccess) return give_up(e);
     timer->mark(s, FFMOE_K_COMBINE);
+    timer->finish();
+    return hipSuccess;
+}
+
+}  // namespace
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------------
+// Stream probe: the tile and scale loads of the two expert kernels for `n_live` experts, in their grids, with their
+// ring and their refill order - and nothing else: no routes, no token rows, no matrix products, no stores (a word
+// leaves only if the or of everything a wave read equals a value the caller picks). What these two launches take is
+// what this memory system gives the access pattern: the ceiling the expert pass is held against.
+// ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t ring_or(const WeightRing &ring, int u) {
+    return ring.t[u].x | ring.t[u].y | ring.t[u].z | ring.t[u].w | ring.s[u].x | ring.s[u].y;
+}
+
+__global__ __launch_bounds__(256, 2) void probe_gate_up_stream_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                                      uint32_t n_experts, uint32_t n_live, uint32_t never,
+                                                                      uint32_t *__restrict__ sink) {
+    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const KSlice k = k_slice(g.gd, ks);
+    const uint32_t blocks_per_slot = max(1u, min(g.gu_rb, gridDim.x / n_live));
+    const uint32_t slot_id = blockIdx.x / blocks_per_slot;
+    if (slot_id >= n_live) return;
+    uint32_t rb0, rb1;
+    split_range(g.gu_rb, blocks_per_slot, blockIdx.x % blocks_per_slot, rb0, rb1);
+    if (rb0 >= rb1) return;
+    const uint32_t expert = (uint32_t)((uint64_t)slot_id * n_experts / n_live);      // spread over the layer
+    const uint8_t *expert_base = arena_layer + (size_t)expert * g.expert_bytes;
+    const TileSource src = make_tile_source(expert_base + g.gu_tiles_off, (size_t)g.gu_rb * g.gd * kTileBytes,
+                                            expert_base + g.gu_scales_off, (size_t)g.gu_rb * g.gd * kTileScaleBytes);
+    WeightRing ring;
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb0 * g.gd + min(k.g0 + u, k.g_last), lane);
+    uint32_t seen = 0;
+    for (uint32_t rb = rb0; rb < rb1; ++rb) {
+        const uint32_t next_row = min(rb + 1, rb1 - 1) * g.gd;
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) {
+            seen |= ring_or(ring, u);
+            ring_fill(ring, u, src, next_row + min(k.g0 + u, k.g_last), lane);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) seen |= ring_or(ring, u);
+    if (seen == never) sink[threadIdx.x] = seen;
+}
+
+__global__ __launch_bounds__(256, 5) void probe_down_stream_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
+                                                                   uint32_t n_experts, uint32_t n_live, uint32_t parts,
+                                                                   uint32_t never, uint32_t *__restrict__ sink) {
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t slot_id = blockIdx.x / parts, part = blockIdx.x % parts;
+    if (slot_id >= n_live) return;
+    const uint32_t rb = part * 4 + wave;
+    if (rb >= g.dn_rbp) return;
+    const uint32_t expert = (uint32_t)((uint64_t)slot_id * n_experts / n_live);
+    const uint8_t *expert_base = arena_layer + (size_t)expert * g.expert_bytes;
+    const TileSource src = make_tile_source(expert_base + g.dn_tiles_off, (size_t)g.dn_rbp * g.gf * kTileBytes,
+                                            expert_base + g.dn_scales_off, (size_t)g.dn_rbp * g.gf * kTileScaleBytes);
+    WeightRing ring;
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb * g.gf + min((uint32_t)u, g.gf - 1), lane);
+    uint32_t seen = 0;
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) seen |= ring_or(ring, u);
+    if (seen == never) sink[threadIdx.x] = seen;
+}
+
+}  // namespace
+
+hipError_t launch_probe_stream(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t n_live,
+                               uint32_t n_cus, uint32_t *sink, KernelTimer *timer) {
+    timer->begin(s);
+    const uint32_t resident = 2 * n_cus;
+    const uint32_t gu_blocks = max(n_live, min(resident, n_live * g.gu_rb));
+    // the value that is never seen: the or of everything a lane read, with bit 0 clear and every other bit set.
+    // Should a layer's data ever produce it, a lane writes one word into the 256-word sink: harmless.
+    hipLaunchKernelGGL(probe_gate_up_stream_kernel, dim3(gu_blocks), dim3(256), 0, s, arena_layer, g, n_experts, n_live,
+                       0xFFFFFFFEu, sink);
+    timer->mark(s, FFMOE_K_PROBE_GATE_UP);
+    const uint32_t dn_parts = (g.dn_rbp + 3) / 4;
+    hipLaunchKernelGGL(probe_down_stream_kernel, dim3(n_live * dn_parts), dim3(256), 0, s, arena_layer, g, n_experts, n_live,
+                       dn_parts, 0xFFFFFFFEu, sink);
+    timer->mark(s, FFMOE_K_PROBE_DOWN);
     timer->finish();
     return hipGetLastError();
 }
 
-}  // namespace
+// Blocks of the routing launch that one GPU holds at once: the kernel's own occupancy (registers, LDS) as the runtime
+// reports it for every instantiation, times the compute units. 0 when the query fails: the call then routes with
+// launches of its own.
+uint32_t route_launch_resident_blocks(uint32_t n_cus) {
+    int least = 1 << 30;
+    auto ask = [&](auto kernel) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess) n = 0;
+        least = n < least ? n : least;
+    };
+    ask(route_gate_up_persistent<false, false>);
+    ask(route_gate_up_persistent<true, false>);
+    ask(route_gate_up_persistent<false, true>);
+    ask(route_gate_up_persistent<true, true>);
+    (void)hipGetLastError();
+    return least > 0 ? (uint32_t)least * n_cus : 0u;
+}
 
 // x, w, residual, y and the 16-bit partial rows are FP16 when `f16`, bf16 otherwise
 hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts,

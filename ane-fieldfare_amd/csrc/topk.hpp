@@ -52,6 +52,16 @@ __device__ __forceinline__ void topk_load(TopkRow &t, const float *row, uint32_t
     }
 }
 
+// The weights' part of a select, shared by its two forms: lane i < top_k holds the score of rank i (`mine`; -inf
+// for an empty rank), `max_s` is rank 0's score in every lane.
+__device__ __forceinline__ void topk_weights(TopkRow &t, float mine, float max_s, uint32_t top_k) {
+    t.ex = expf(mine - max_s);
+    t.sum = 0.0f;
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i)
+        if (i < top_k) t.sum += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(t.ex), (int)i));
+}
+
 // SLOTS: how many of the four key slots can hold a candidate (E <= 64 SLOTS).
 template <int SLOTS = 4>
 __device__ __forceinline__ void topk_select(TopkRow &t, uint32_t top_k, uint32_t lane) {
@@ -88,11 +98,65 @@ __device__ __forceinline__ void topk_select(TopkRow &t, uint32_t top_k, uint32_t
             }
         }
     }
-    t.ex = expf(mine - max_s);
-    t.sum = 0.0f;
+    topk_weights(t, mine, max_s, top_k);
+}
+
+// The same select by the four waves of a block together (moe.metal:186-237 ranks with a SIMD-wide pass as well):
+// instead of top_k dependent rounds of a wave-wide maximum, every candidate's rank is COUNTED - how many candidates
+// have a larger key - and the candidates of rank < top_k go to their places. Every wave holds the row's keys (t.key,
+// identical in the four waves); wave v counts over a quarter of the candidates (two vector instructions per pair of
+// keys: compare, add with carry), the partial counts meet in `cnt` ([wave][slot][lane], LDS) behind one barrier, and
+// wave `finisher` adds them, moves the winners to lanes 0 .. top_k - 1 by cross-lane writes and computes the weights.
+// Equal keys (two experts with the same logit bits) get equal counts; the total order breaks such a tie by index,
+// so when two candidates land on one rank - seen as fewer filled ranks than placed candidates - the finisher runs
+// topk_select instead. Same routes and weights as topk_select bit for bit either way: without a tie the ranks are
+// those of the total order, and the weights come from the same code. Returns in `t` for the finisher wave only.
+// Every wave of the block has to call it.
+template <int SLOTS>
+__device__ __forceinline__ void block_topk_select(TopkRow &t, uint32_t top_k, uint32_t lane, uint32_t wave, uint32_t finisher,
+                                                  uint32_t (*cnt)[4][64]) {
+    constexpr uint32_t kPerWave = 16 * SLOTS;                 // candidates a wave counts over
+    const uint32_t first = wave * kPerWave, c_other = __builtin_amdgcn_readfirstlane(first >> 6);
+    const uint32_t l0 = __builtin_amdgcn_readfirstlane(first & 63);
+    uint32_t theirs = t.key[0];
 #pragma unroll
-    for (uint32_t i = 0; i < 8; ++i)
-        if (i < top_k) t.sum += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(t.ex), (int)i));
+    for (int c = 1; c < SLOTS; ++c) theirs = c_other == (uint32_t)c ? t.key[c] : theirs;
+    // a non-candidate's key is 0 and is larger than nothing; what is counted for a lane's own empty slot is never used
+    uint32_t count[SLOTS];
+#pragma unroll
+    for (int c = 0; c < SLOTS; ++c) count[c] = 0;
+#pragma unroll 8
+    for (uint32_t i = 0; i < kPerWave; ++i) {
+        const uint32_t ko = (uint32_t)__builtin_amdgcn_readlane((int)theirs, (int)(l0 + i));
+#pragma unroll
+        for (int c = 0; c < SLOTS; ++c) count[c] += ko > t.key[c] ? 1u : 0u;
+    }
+#pragma unroll
+    for (int c = 0; c < SLOTS; ++c) cnt[wave][c][lane] = count[c];
+    lds_barrier();
+    if (wave != finisher) return;
+    uint32_t got_key = 0, got_idx = 0, placed_n = 0;
+#pragma unroll
+    for (int c = 0; c < SLOTS; ++c) {
+        const uint32_t rank = cnt[0][c][lane] + cnt[1][c][lane] + cnt[2][c][lane] + cnt[3][c][lane];
+        const bool placed = t.key[c] != 0u && rank < top_k;
+        placed_n += (uint32_t)__popcll(__ballot(placed));
+        // a cross-lane write: lane `rank` receives the value, lanes nobody writes to receive 0; the others aim at
+        // lane 63, which holds no rank (top_k <= 8)
+        const int to = (int)((placed ? rank : 63u) * 4u);
+        got_key |= (uint32_t)__builtin_amdgcn_ds_permute(to, (int)(placed ? t.key[c] : 0u));
+        got_idx |= (uint32_t)__builtin_amdgcn_ds_permute(to, (int)(placed ? (uint32_t)c * 64u + lane : 0u));
+    }
+    const bool have = lane < top_k && got_key != 0u;
+    if ((uint32_t)__popcll(__ballot(have)) != placed_n) {      // two candidates on one rank: equal keys
+        topk_select<SLOTS>(t, top_k, lane);
+        return;
+    }
+    // recover the score from the key: orderable() is a bijection
+    const float mine = have ? __uint_as_float((got_key & 0x80000000u) ? (got_key & 0x7FFFFFFFu) : ~got_key) : -INFINITY;
+    t.idx = have ? got_idx : 0u;
+    const float max_s = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(mine), 0));
+    topk_weights(t, mine, max_s, top_k);
 }
 
 __device__ __forceinline__ void topk_store(const TopkRow &t, const uint16_t *__restrict__ per_expert_scale, uint32_t top_k,

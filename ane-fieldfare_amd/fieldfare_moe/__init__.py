@@ -43,7 +43,7 @@ BF16, FP16 = 0, 1     # FFMOE_BF16, FFMOE_FP16
 EXPORTS = [
     "ffmoe_version", "ffmoe_create", "ffmoe_destroy", "ffmoe_layer_arena_bytes", "ffmoe_upload_layer",
     "ffmoe_upload_router_bf16", "ffmoe_upload_router_int8", "ffmoe_dequant_expert", "ffmoe_router",
-    "ffmoe_verify", "ffmoe_verify_partials", "ffmoe_last_live_experts", "ffmoe_reduce_token_major",
+    "ffmoe_verify", "ffmoe_verify_partials", "ffmoe_last_live_experts", "ffmoe_handover_giveups", "ffmoe_probe_stream", "ffmoe_reduce_token_major",
     "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
     "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
@@ -55,7 +55,7 @@ EXPORTS = [
 PROFILE_SLOTS = 16
 KERNEL_NAMES = ["router_logits", "router_topk", "plan", "gate_up", "down", "combine", "prefill_sort",
                 "prefill_gate_up", "prefill_down", "prefill_combine", "gemv", "argmax", "event_gap", "route_gate_up",
-                "reserved14", "reserved15"]
+                "probe_gate_up", "probe_down"]
 
 
 class Projection(C.Structure):
@@ -195,6 +195,8 @@ def lib() -> C.CDLL:
     L.ffmoe_set_handover_timeout.argtypes = [vp, vp, C.c_uint64, errp]
     L.ffmoe_set_one_launch_routing.argtypes = [vp, C.c_int, errp]
     L.ffmoe_last_live_experts.argtypes = [vp, vp, C.POINTER(u32), errp]
+    L.ffmoe_handover_giveups.argtypes = [vp, vp, C.POINTER(u32), errp]
+    L.ffmoe_probe_stream.argtypes = [vp, vp, u32, u32, errp]
     L.ffmoe_reduce_token_major.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, errp]
     L.ffmoe_gemv_int4.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, i32, errp]
     L.ffmoe_layer_tail_norms.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, vp, vp, vp, vp, u32, u32, u32, C.c_float,
@@ -432,7 +434,8 @@ class Context:
         return partials
 
     def set_handover_timeout(self, ticks: int):
-        """Ticks (100 MHz) a block of route_verify's one-launch form waits for a hand-over word; clears the fault count."""
+        """Ticks (100 MHz) a wave of route_verify's one-launch form waits for a hand-over word before it computes the
+        word's content itself; clears the count handover_giveups() reports."""
         err = C.c_char_p()
         _check(self.L.ffmoe_set_handover_timeout(self._h, _stream(), ticks, C.byref(err)), err)
 
@@ -445,6 +448,18 @@ class Context:
         n = C.c_uint32()
         err = C.c_char_p()
         _check(self.L.ffmoe_last_live_experts(self._h, _stream(), C.byref(n), C.byref(err)), err)
+        return int(n.value)
+
+    def probe_stream(self, layer: int, n_live: int):
+        """The weight loads of the decode / verify expert kernels for n_live experts and nothing else (a timing probe)."""
+        err = C.c_char_p()
+        _check(self.L.ffmoe_probe_stream(self._h, _stream(), layer, n_live, C.byref(err)), err)
+
+    def handover_giveups(self) -> int:
+        """Waves of route_verify's one-launch form that stopped waiting for another block and helped themselves."""
+        n = C.c_uint32()
+        err = C.c_char_p()
+        _check(self.L.ffmoe_handover_giveups(self._h, _stream(), C.byref(n), C.byref(err)), err)
         return int(n.value)
 
     def reduce_token_major(self, partials, weights):

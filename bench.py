@@ -205,6 +205,18 @@ def main():
     # then exactly --steps timed steps between two device synchronisations.
     kSettlePasses = 300
     n_warm, n_timed = args.warmup * L, args.steps * L
+    # What a short run without the settling passes reads (the method of this benchmark's first form: a step = one layer
+    # pass, 5 warm-up passes, 20 timed ones, a timed region of about 1 ms between two synchronisations), for comparison.
+    time.sleep(0.5)
+    for i in range(5):
+        step(i % L)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(20):
+        step((5 + i) % L)
+    torch.cuda.synchronize()
+    cold_el = time.perf_counter() - t0
+    cold_value = sum(live[(5 + i) % L] for i in range(20)) * EXPERT_BYTES / cold_el / 1e9
     for i in range(kSettlePasses + n_warm):
         step(i % L)
     torch.cuda.synchronize()
@@ -216,6 +228,24 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     bytes_total = args.steps * sum(live) * EXPERT_BYTES
     value = bytes_total / elapsed / 1e9
+    giveups = ctx.handover_giveups()     # waves of the one-launch routing that stopped waiting for another block: 0 on a GPU of its own
+
+    # The ceiling of the expert stream on this box, measured in this run: ffmoe_probe_stream issues exactly the weight
+    # loads of the gate/up and the down kernel for as many experts as the block touches in each layer - no routing, no
+    # rows, no arithmetic, no output - as two launches per layer pass over the same cycled layers.
+    def probe(layer):
+        rc = Lib.ffmoe_probe_stream(h, stream, layer, live[layer], C.byref(err))
+        if rc:
+            raise RuntimeError(err.value)
+    for i in range(2 * L):
+        probe(i % L)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(n_timed):
+        probe(i % L)
+    torch.cuda.synchronize()
+    probe_el = time.perf_counter() - t0
+    ceiling_value = bytes_total / probe_el / 1e9
 
     # spread of the step time: one event after every step (a record costs the stream a few microseconds, so
     # these intervals sit above ms_per_step by about one record; the spread is what they are for)
@@ -250,6 +280,9 @@ def main():
     for i in range(n_timed):
         step(i % L)
     prof = ctx.profile(reset=True)
+    for i in range(n_timed):
+        probe(i % L)
+    probe_prof = ctx.profile(reset=True)
     ctx.set_profiling(False)
     # An event record costs the stream a few microseconds. The library measures an empty interval (two
     # records with nothing between them, once per call); a kernel's interval carries half of that - one
@@ -272,6 +305,20 @@ def main():
         gu_ms = prof["gate_up"][0] - gap_ms * prof["gate_up"][1]
         achieved = live_sum * GATE_UP_BYTES / (gu_ms * 1e-3) / 1e9
     down_gbs = live_sum * DOWN_BYTES / ((prof["down"][0] - gap_ms * prof["down"][1]) * 1e-3) / 1e9
+    probe_us = kernel_times(probe_prof)
+    pg_ms = probe_prof["probe_gate_up"][0] - gap_ms * probe_prof["probe_gate_up"][1]
+    pd_ms = probe_prof["probe_down"][0] - gap_ms * probe_prof["probe_down"][1]
+    ceiling_gu = live_sum * GATE_UP_BYTES / (pg_ms * 1e-3) / 1e9
+    ceiling_dn = live_sum * DOWN_BYTES / (pd_ms * 1e-3) / 1e9
+    stream_ceiling = {
+        "what": "ffmoe_probe_stream: the tile and scale loads of the gate/up and the down kernel for the same number of "
+                "experts per layer, in those kernels' grids and order, and nothing else; two launches per layer pass, same cycled layers",
+        "us_per_layer_pass": round(probe_el * 1e6 / n_timed, 2), "GBs": round(ceiling_value, 1),
+        "frac_hbm_peak": round(ceiling_value / HBM_PEAK_GBS, 4),
+        "value_frac_of_ceiling": round(value / ceiling_value, 4),
+        "kernel_us": {"probe_gate_up": probe_us.get("probe_gate_up"), "probe_down": probe_us.get("probe_down")},
+        "gate_up_stream_GBs": round(ceiling_gu, 1), "down_stream_GBs": round(ceiling_dn, 1),
+        "down_kernel_frac_of_ceiling": round(down_gbs / ceiling_dn, 4)}
     # the same steps as ffmoe_router + ffmoe_verify (five launches): what the gate/up stream does as a launch of its own,
     # without the routing chain in front of it, and what the one-call form gains on the whole step
     split = None
@@ -368,6 +415,36 @@ def main():
                                 "unit": "TFLOP/s", "frac": round((flops_gu + flops_dn) / gemm_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                                 "traffic": traffic.get("prefill3072_gemms") if TP == 3072 else None,
                                 "traffic_unit": f"HBM bytes of the two launches (rocprofv3 --pmc, profiles/{TRAFFIC_FILE.name})"}}
+        # The dense bf16 GEMM ceiling of this box in the same run: the two products of the chunk's n_pairs rows as plain
+        # library GEMMs (torch.matmul -> hipBLASLt / rocBLAS) on bf16 operands - no INT4 expansion, no gather, one
+        # weight matrix instead of 128, a shape the library is tuned for.
+        mrows = int(n_pairs)
+        a_gu = torch.randn((mrows, D), device="cuda", generator=gen).to(torch.bfloat16)
+        b_gu = torch.randn((D, 2 * F), device="cuda", generator=gen).to(torch.bfloat16)
+        a_dn = torch.randn((mrows, F), device="cuda", generator=gen).to(torch.bfloat16)
+        b_dn = torch.randn((F, D), device="cuda", generator=gen).to(torch.bfloat16)
+        o_gu = torch.empty((mrows, 2 * F), dtype=torch.bfloat16, device="cuda")
+        o_dn = torch.empty((mrows, D), dtype=torch.bfloat16, device="cuda")
+
+        def dense_time(a_, b_, o_):
+            for _ in range(5):
+                torch.matmul(a_, b_, out=o_)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                torch.matmul(a_, b_, out=o_)
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e-3 / 20
+        t_dgu, t_ddn = dense_time(a_gu, b_gu, o_gu), dense_time(a_dn, b_dn, o_dn)
+        dense_tf = (flops_gu + flops_dn) / (t_dgu + t_ddn) / 1e12
+        prefill["dense_bf16_ceiling_TFLOPs"] = round(dense_tf, 1)
+        prefill["dense_bf16_ceiling"] = {
+            "gate_up_us": round(t_dgu * 1e6, 1), "down_us": round(t_ddn * 1e6, 1),
+            "shapes": f"[{mrows} x {D}] . [{D} x {2 * F}] and [{mrows} x {F}] . [{F} x {D}], bf16, torch.matmul",
+            "frac_mfma_peak": round(dense_tf / MFMA_BF16_PEAK_TFLOPS, 4),
+            "gemm_frac_of_dense_ceiling": round((flops_gu + flops_dn) / gemm_s / 1e12 / dense_tf, 4)}
+        del a_gu, b_gu, a_dn, b_dn, o_gu, o_dn
         # BASELINE.json config 4 (ii): the same chunk with Zipf(1.1) routing imposed on the experts
         # (indices and weights given, no router): a few experts hold most pairs, many hold a handful
         zidx_, zw_ = syn.zipf_routes(np.random.default_rng(4), TP)
@@ -760,6 +837,12 @@ def main():
                    "routes_per_live_expert_hist": {str(n): int(c) for n, c in enumerate(tokens_per_expert) if c},
                    "routes_per_live_expert_note": f"over the {L} layers: how many live experts receive n of the block's {T * K} routes"},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "stream_ceiling": stream_ceiling,
+        "handover_giveups_in_timed_region": giveups,
+        "value_first_20_passes_after_5": {"GBs": round(cold_value, 1), "us_per_layer_pass": round(cold_el * 1e6 / 20, 2),
+                                          "note": "25 layer passes straight after a pause, no settling passes: a 1 ms timed region "
+                                                  "between two synchronisations, which the launch latency in front and the "
+                                                  "wake-up behind it weigh on"},
         "layer_pass_us": step_spread,
         "device": device_info,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1),
@@ -768,6 +851,8 @@ def main():
                      "traffic_unit": f"bytes per launch (rocprofv3 --pmc, profiles/{TRAFFIC_FILE.name})",
                      "algorithmic_bytes_per_launch": int(achieved * 1e9 * gu_ms * 1e-3 / n_timed),
                      "avg_kernel_us": round(gu_ms * 1e3 / n_timed, 2),
+                     "measured_ceiling_GBs": round(ceiling_gu, 1), "frac_of_ceiling": round(achieved / ceiling_gu, 4),
+                     "ceiling_note": "measured_ceiling_GBs: the same launch's weight loads alone (stream_ceiling.kernel_us.probe_gate_up), this run, this box",
                      "note": ("the launch also holds the routing chain (logits, select, routes: about 6 us before the first weight is "
                               "requested); five_launch_form.gate_up_* is the same stream as a launch of its own") if split else None},
         "five_launch_form": split,

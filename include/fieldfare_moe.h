@@ -178,31 +178,47 @@ int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const ui
  * the GPU routes the persistent kernels without a host round trip.
  * When the expert fits the persistent kernels and the router rows are 8-byte aligned, the router logits, the
  * select and gate/up run as ONE launch (a decode step is two launches, a verify block three): the blocks
- * hand logits and routes to each other through epoch-stamped words in device memory, which needs every
- * block of that launch resident at once - the grid is sized for a GPU this stream has to itself. A block
- * that waits 0.2 s for a word gives up, the call's output is then undefined and the next
- * ffmoe_last_live_experts on the context reports FFMOE_ERR_RUNTIME. */
+ * hand logits and routes to each other through epoch-stamped words in device memory. That is fast when every
+ * block of the launch is resident at once - the grid is sized from the kernel's occupancy on a GPU this stream has
+ * to itself - and correct either way: a wave that has waited FFMOE_DEFAULT_HANDOVER_TICKS for a word (other work
+ * on the GPU keeps the block that makes it from running) stops waiting and computes what it waited for itself,
+ * with the same arithmetic in the same order, so the call returns the same routes and rows, only later.
+ * ffmoe_handover_giveups counts such waves. */
 int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *router_x,
                        uint32_t router_x_stride, const uint16_t *x, uint32_t x_stride, uint32_t t,
                        const uint16_t *residual, uint16_t *y, uint32_t *out_idx, uint16_t *out_w, char **err);
 
-/* How long a block of ffmoe_route_verify's one-launch form waits for a hand-over word before it gives up, in ticks of
- * the GPU's constant 100 MHz clock (default 20,000,000 = 0.2 s); also clears the count of polls that gave up. Waits
- * for the stream. No counterpart in the reference. A host that shares the GPU with other work may want a longer
- * wait; the tests set 0 to see the give-up path end normally and be reported. */
+/* How long a wave of ffmoe_route_verify's one-launch form waits for a hand-over word before it computes the word's
+ * content itself, in ticks of the GPU's constant 100 MHz clock (default FFMOE_DEFAULT_HANDOVER_TICKS = 1 ms); also
+ * clears the count of waves that stopped waiting. Waits for the stream. No counterpart in the reference. The tests
+ * set 0, which sends every wave that does not find its words at once down the self-sufficient path. */
+#define FFMOE_DEFAULT_HANDOVER_TICKS 100000ull
 int ffmoe_set_handover_timeout(ffmoe_ctx *ctx, void *stream, uint64_t ticks, char **err);
 
 /* enabled = 0: ffmoe_route_verify runs the router as launches of its own in front of the expert pass (five launches
- * for a verify block, four for a decode step; same results bit for bit), which needs no block to wait for another:
- * the form for a host whose other streams or processes keep compute units of this GPU busy, where the one-launch
- * form's blocks cannot count on being resident together. enabled != 0 (the default) restores the one-launch form.
- * Host state, takes effect with the next call. No counterpart in the reference. */
+ * for a verify block, four for a decode step; same results bit for bit), in which no block waits for another: the
+ * faster form for a host whose other streams or processes keep compute units of this GPU busy, where the one-launch
+ * form's waves would wait out their bound before they help themselves. enabled != 0 (the default) restores the
+ * one-launch form. Host state, takes effect with the next call. No counterpart in the reference. */
 int ffmoe_set_one_launch_routing(ffmoe_ctx *ctx, int enabled, char **err);
 
+/* Measurement hook, no counterpart in the reference: issues exactly the weight loads (tiles and scales) of the
+ * decode / verify gate/up and down kernels for `n_live` experts of `layer` (spread over the layer's experts), in
+ * those kernels' grids and order, with no routing, no token rows, no arithmetic and no output. Two launches; what
+ * they take is what the memory system gives this access pattern, i.e. the ceiling the expert pass can be held
+ * against (with ffmoe_set_profiling: slots FFMOE_K_PROBE_GATE_UP / FFMOE_K_PROBE_DOWN). 1 <= n_live <= n_experts;
+ * needs a shape that fits the persistent kernels (d <= 2816, f <= 704). */
+int ffmoe_probe_stream(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint32_t n_live, char **err);
+
 /* Number of distinct experts the last ffmoe_verify* call on `stream` ran (reads back 4 bytes; waits
- * for the stream). For reporting only. FFMOE_ERR_RUNTIME if a launch of ffmoe_route_verify on this
- * context ever gave up waiting for its own blocks (see there). */
+ * for the stream). For reporting only. */
 int ffmoe_last_live_experts(ffmoe_ctx *ctx, void *stream, uint32_t *n_live, char **err);
+
+/* Waves of ffmoe_route_verify's one-launch form that stopped waiting for a hand-over word and computed it themselves,
+ * since the context was created or ffmoe_set_handover_timeout was last called (reads back 4 bytes; waits for the
+ * stream). The results of such calls are correct; a count that keeps growing says the GPU is shared and
+ * ffmoe_set_one_launch_routing(ctx, 0) would serve this host better. No counterpart in the reference. */
+int ffmoe_handover_giveups(ffmoe_ctx *ctx, void *stream, uint32_t *count, char **err);
 
 /* ---- routed experts, prefill chunk (t <= max_tokens) ------------------------------------------- */
 
@@ -399,6 +415,7 @@ enum {
     FFMOE_K_PREFILL_COMBINE, FFMOE_K_GEMV, FFMOE_K_ARGMAX,
     FFMOE_K_EVENT_GAP, /* two event records with nothing between them: what an event pair adds to every slot above */
     FFMOE_K_ROUTE_GATE_UP, /* ffmoe_route_verify: router logits, select and gate/up in one launch */
+    FFMOE_K_PROBE_GATE_UP, FFMOE_K_PROBE_DOWN, /* ffmoe_probe_stream: the weight loads of gate/up and of down alone */
     FFMOE_PROFILE_SLOTS = 16
 };
 typedef struct {

@@ -85,6 +85,7 @@ def test_router_verify_and_dense_chain_in_a_graph(oracle, one_call):
                 ctx.route_verify(replay % layers, x, x)
         dense.dense_ffn(replay % layers, x)
         torch.cuda.synchronize()
-    assert ctx.last_live_experts() > 0      # also raises if a hand-over poll of route_verify ever gave up
+    assert ctx.last_live_experts() > 0
+    assert ctx.handover_giveups() == 0      # on a GPU of its own no wave of the one-launch form had to help itself
     ctx.close()
     dense.close()

@@ -76,6 +76,20 @@ def test_verify_block_on_deep_layers(model, oracle, torch, layer):
     ref = oracle.moe_experts(model["pools"][layer], xb, idx_np, oracle.bf16_to_float(bits_of(w)))
     got = oracle.bf16_to_float(bits_of(y))
     assert rel_err(got, ref) <= 1e-2 and cosine(got, ref) >= 0.9999, (layer, rel_err(got, ref), cosine(got, ref))
+    # the call the benchmark times - router, select and gate/up in one launch - on the same block: routes, weights and
+    # rows equal the two calls' bit for bit (so they are the oracle's routes and rows as well), and no wave of the
+    # one-launch form had to help itself
+    y1, idx1, w1 = ctx.route_verify(layer, x, x)
+    assert np.array_equal(idx1.cpu().numpy(), idx.cpu().numpy())
+    assert np.array_equal(bits_of(w1), bits_of(w))
+    assert np.array_equal(bits_of(y1), bits_of(y))
+    assert ctx.last_live_experts() == distinct and ctx.handover_giveups() == 0
+    # a decode step (one row) of the same block through the same call
+    y_one, idx_one, w_one = ctx.route_verify(layer, x[:1], x[:1])
+    assert np.array_equal(idx_one.cpu().numpy(), idx.cpu().numpy()[:1]) and np.array_equal(bits_of(w_one), bits_of(w)[:1])
+    ref_one = oracle.moe_experts(model["pools"][layer], xb[:1], idx_np[:1], oracle.bf16_to_float(bits_of(w))[:1])
+    got_one = oracle.bf16_to_float(bits_of(y_one))
+    assert rel_err(got_one, ref_one) <= 1e-2 and cosine(got_one, ref_one) >= 0.9999
 
 
 @pytest.mark.parametrize("layer", DEEP)
@@ -124,9 +138,9 @@ def test_lm_head_262144_greedy(model, oracle, torch):
     logits = head.gemv(x, f32_out=True).cpu().numpy()
     # every row's choice is the first maximum of the GEMV's own fp32 logits
     assert np.array_equal(tokens, logits.argmax(1))
-    # two rows against the CPU reference (dequantise the row, then dot: DequantInt4GemvRef); the gap between the best
+    # every row against the CPU reference (dequantise the row, then dot: DequantInt4GemvRef); the gap between the best
     # and the second-best logit says how much room the comparison had
-    for row in (0, 15):
+    for row in range(16):
         ref = oracle.gemv_int4_ref(Wh, Sh, Bh, oracle.bf16_to_float(xb[row]))
         order = np.argsort(-ref, kind="stable")
         gap = float(ref[order[0]] - ref[order[1]])

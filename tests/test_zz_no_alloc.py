@@ -34,6 +34,15 @@ def test_static_scratch_verify_equals_verify(oracle, shape):
     ctx = ff.Context(d, f, e, 8, n_layers=1, max_tokens=64)
     ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
     ctx.upload_router_bf16(0, router)
+    # a second context of the same shape: the call under test runs on `ctx`, whose own scratch a verify on a
+    # throw-away block has filled with unrelated rows just before (so a static call that read or wrote the context's
+    # allocations instead of the array would give other bits)
+    junk = bf16_tensor(torch, oracle.bf16_bits(rng.normal(0, 3, (16, d)).astype(np.float32)))
+
+    def sentinel(c):
+        ji, jw = c.router(0, junk)
+        c.verify(0, junk, ji, jw)
+        torch.cuda.synchronize()
     for t, with_residual in ((16, True), (5, False), (1, True)):     # in a row; each smaller than the one before
         xb = oracle.bf16_bits(rng.normal(0, 1, (t, d)).astype(np.float32))
         x = bf16_tensor(torch, xb)
@@ -42,8 +51,13 @@ def test_static_scratch_verify_equals_verify(oracle, shape):
         y_ref = torch.full((t, d), float("nan"), dtype=torch.bfloat16, device="cuda")
         y_new = torch.full((t, d), float("nan"), dtype=torch.bfloat16, device="cuda")
         _call(L.ffmoe_verify, ctx, torch, 0, x, idx, w, residual, y_ref)
+        torch.cuda.synchronize()
+        # the context's own scratch must play no part in the static call: fill it with a pattern that would show
+        sentinel(ctx)
+        free_before = torch.cuda.mem_get_info()[0]
         _call(L.ffmoe_verify_static, ctx, torch, 0, x, idx, w, residual, y_new)
         torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before, "the static call changed the free device memory"
         assert np.array_equal(bits_of(y_new), bits_of(y_ref)), (shape, t)
         # and the pair is right, not merely equal: the oracle's fp32 layer on the same routes
         w_np = oracle.bf16_to_float(bits_of(w))
@@ -59,13 +73,14 @@ def test_static_scratch_rejects_shapes_beyond_its_size(oracle):
     import torch
     import fieldfare_moe as ff
     L = ff.lib()
-    ctx = ff.Context(6144, 2048, 8, 8, n_layers=1, max_tokens=16)
-    x = torch.zeros((1, 6144), dtype=torch.bfloat16, device="cuda")
+    d = 6144           # 16 * 8 un-weighted fp32 rows of this width alone take 3 MiB
+    ctx = ff.Context(d, 2048, 8, 8, n_layers=1, max_tokens=16)
+    x = torch.zeros((1, d), dtype=torch.bfloat16, device="cuda")
     idx = torch.zeros((1, 8), dtype=torch.int32, device="cuda")
     w = torch.zeros((1, 8), dtype=torch.bfloat16, device="cuda")
-    y = torch.zeros((1, 6144), dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros((1, d), dtype=torch.bfloat16, device="cuda")
     err = C.c_char_p()
-    rc = L.ffmoe_verify_static(ctx._h, None, 0, C.c_void_p(x.data_ptr()), 6144, 1, C.c_void_p(idx.data_ptr()),
+    rc = L.ffmoe_verify_static(ctx._h, None, 0, C.c_void_p(x.data_ptr()), d, 1, C.c_void_p(idx.data_ptr()),
                                C.c_void_p(w.data_ptr()), None, C.c_void_p(y.data_ptr()), C.byref(err))
     assert rc == -1 and b"static array holds" in err.value, (rc, err.value)
     ctx.close()
