@@ -453,10 +453,10 @@ struct VerifyScratch {
 static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
                          uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual, uint16_t *y,
                          uint16_t *partials_bf16, char **err, const VerifyScratch *use = nullptr,
-                         const RouteFusion *route = nullptr) {
+                         const RouteFusion *route = nullptr, bool dense = false) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (int rc = check_layer(ctx, layer, true, route != nullptr, err)) return rc;
-    if (!x || !idx || !w || (!y && !partials_bf16)) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (!x || !idx || !w || (!y && !partials_bf16 && !route)) return fail(err, FFMOE_ERR_INVALID, "null argument");
     if (t == 0 || t > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%d", t, FFMOE_MAX_VERIFY_ROWS);
     if (x_stride < ctx->shape.d || x_stride % 8 || reinterpret_cast<uintptr_t>(x) % 16)
         return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
@@ -466,7 +466,7 @@ static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uin
     const VerifyScratch &sc = use ? *use : own;
     FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                         sc.plan, sc.acts, sc.partials, ctx->n_cus, &ctx->timer, ctx->f16, route));
+                         sc.plan, sc.acts, sc.partials, ctx->n_cus, &ctx->timer, ctx->f16, route, dense));
     return FFMOE_OK;
 }
 
@@ -501,7 +501,8 @@ int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint1
                        const uint16_t *x, uint32_t x_stride, uint32_t t, const uint16_t *residual, uint16_t *y,
                        uint32_t *out_idx, uint16_t *out_w, char **err) {
     if (int rc = check_ctx(ctx, err)) return rc;
-    if (!router_x || !out_idx || !out_w || !y) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (!router_x || !out_idx || !out_w) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (!y && residual) return fail(err, FFMOE_ERR_INVALID, "a residual needs y: without y the rows stay un-combined");
     if (router_x_stride < ctx->shape.d) return fail(err, FFMOE_ERR_INVALID, "hidden stride is too small");
     if (ctx->f16 && (reinterpret_cast<uintptr_t>(router_x) % 8 || router_x_stride % 4))
         return fail(err, FFMOE_ERR_INVALID, "FP16 router rows must be 8-byte aligned with a stride that is a multiple of 4");
@@ -621,7 +622,8 @@ int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t
     // With one route per row at weight 1, the un-weighted bf16 row of route t is the output row t: the
     // down projection writes y itself and the combine pass has nothing to add.
     if (t <= FFMOE_MAX_VERIFY_ROWS)
-        return verify_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, nullptr, y, err);
+        return verify_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, nullptr, y, err, nullptr,
+                             nullptr, true);
     return prefill_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, 0, nullptr, y, err);
 }
 
@@ -670,6 +672,20 @@ int ffmoe_layer_tail(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uint32_t 
     if (int rc = check_rows(t, d, strides, 3, err)) return rc;
     FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), h2, h2_stride, h1, h1_stride, hidden, hidden_stride,
                              w_postffn2, w_postffn, t, d, eps, layer_scalar, nullptr, nullptr, nullptr, 0, ctx->f16));
+    return FFMOE_OK;
+}
+
+int ffmoe_layer_tail_routed(ffmoe_ctx *ctx, void *stream, const uint16_t *route_w, const uint16_t *h1, uint32_t h1_stride,
+                            uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
+                            uint32_t t, float eps, float layer_scalar, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!route_w || !h1 || !hidden || !w_postffn2 || !w_postffn) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (t == 0 || t > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%d", t, FFMOE_MAX_VERIFY_ROWS);
+    const uint32_t strides[2] = {h1_stride, hidden_stride};
+    if (int rc = check_rows(t, ctx->shape.d, strides, 2, err)) return rc;
+    FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), nullptr, 0, h1, h1_stride, hidden, hidden_stride, w_postffn2,
+                             w_postffn, t, ctx->shape.d, eps, layer_scalar, nullptr, nullptr, nullptr, 0, ctx->f16, ctx->partials,
+                             route_w, ctx->plan->route_valid, ctx->shape.top_k));
     return FFMOE_OK;
 }
 

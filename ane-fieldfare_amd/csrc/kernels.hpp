@@ -156,7 +156,7 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
                          VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer,
-                         bool f16 = false, const RouteFusion *route = nullptr);
+                         bool f16 = false, const RouteFusion *route = nullptr, bool dense = false);
 uint32_t route_launch_resident_blocks(uint32_t n_cus);
 // the two expert kernels' weight loads for n_live experts and nothing else (`sink`: 256 words nobody reads)
 hipError_t launch_probe_stream(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t n_live,
@@ -204,7 +204,8 @@ hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stri
                              uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
                              uint32_t t, uint32_t d, float eps, float layer_scalar, const uint16_t *w_postffn1 = nullptr,
                              const uint16_t *w_next = nullptr, uint16_t *normed = nullptr, uint32_t normed_stride = 0,
-                             bool f16 = false);
+                             bool f16 = false, const float *routed_partials = nullptr, const uint16_t *routed_w = nullptr,
+                             const uint32_t *route_valid = nullptr, uint32_t top_k = 0);
 hipError_t launch_rmsnorm(hipStream_t s, const uint16_t *x, uint32_t x_stride, const uint16_t *w, uint16_t *out,
                           uint32_t out_stride, uint32_t t, uint32_t d, float eps, bool f16 = false);
 

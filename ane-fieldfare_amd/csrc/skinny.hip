@@ -307,7 +307,10 @@ __device__ __forceinline__ void prepare_token_rows(uint32_t lane, uint4 (&x0)[kR
 
 // From the routes (thread r < n_routes brings route r) to the stored activations: the plan, the block's share of
 // its expert's row blocks, the weight stream. x0 / x1: the wave's token rows as load_token_rows() left them.
-template <bool F16>
+// DENSE: the one expert of a dense FFN takes every row at weight 1 (route r = row r): nothing to plan, the first
+// weight request goes out with the kernel's first instructions, and block 0 writes the plan the down kernel's
+// general forms and ffmoe_last_live_experts read without any block waiting for it.
+template <bool F16, bool DENSE = false>
 __device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps, const uint8_t *__restrict__ arena_layer,
                                              const ArenaGeom &g, uint32_t top_k, uint32_t n_experts, uint32_t route_idx,
                                              uint16_t route_w, uint32_t n_routes, VerifyPlan *__restrict__ plan,
@@ -321,18 +324,34 @@ __device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps
     // operations, against a separate launch plus two dependent global reads per block. Block 0 also
     // writes the plan out for the down kernel.
     const uint32_t gu_rb = g.gu_rb, n_blocks = gridDim.x, bid = blockIdx.x;
-    uint32_t slot_id, route_expert;
+    uint32_t slot_id = 0, route_expert = 0, n_live = 1;
     VerifyPlan *plan_out = bid == 0 ? plan : nullptr;
-    const uint32_t n_live = build_plan_experts(
-        ps, route_idx, route_w, n_routes, n_experts, plan_out,
-        [=](uint32_t total) { return total ? bid / max(1u, min(gu_rb, n_blocks / total)) : 0xFFFFFFFFu; }, slot_id,
-        route_expert);
+    if constexpr (DENSE) {
+        slot_id = bid / max(1u, min(gu_rb, n_blocks));
+        if (plan_out) {
+            const uint32_t tid = threadIdx.x;
+            if (tid == 0) {
+                plan_out->n_live = 1;
+                plan_out->slots[0].expert = 0;
+                plan_out->slots[0].n = rows;
+            } else if (tid < (uint32_t)FFMOE_MAX_EXPERTS) {
+                plan_out->slots[tid].n = 0;
+            }
+            if (tid < (uint32_t)kMaxRows) plan_out->slots[0].routes[tid] = tid;
+            if (tid < (uint32_t)kMaxRoutes) plan_out->route_valid[tid] = tid < rows ? 1u : 0u;
+        }
+    } else {
+        n_live = build_plan_experts(
+            ps, route_idx, route_w, n_routes, n_experts, plan_out,
+            [=](uint32_t total) { return total ? bid / max(1u, min(gu_rb, n_blocks / total)) : 0xFFFFFFFFu; }, slot_id,
+            route_expert);
+    }
     const bool has_slot = n_live != 0 && slot_id < n_live;
     const uint32_t blocks_per_slot = max(1u, min(gu_rb, n_blocks / max(1u, n_live)));
     uint32_t rb0 = 0, rb1 = 0;
     if (has_slot) split_range(gu_rb, blocks_per_slot, bid % blocks_per_slot, rb0, rb1);
     const bool has_rows = has_slot && rb0 < rb1;
-    const uint32_t slot_expert = has_slot ? __builtin_amdgcn_readfirstlane(ps.expert_of[slot_id]) : 0;
+    const uint32_t slot_expert = DENSE ? 0u : has_slot ? __builtin_amdgcn_readfirstlane(ps.expert_of[slot_id]) : 0;
     const uint8_t *expert_base = arena_layer + (size_t)slot_expert * g.expert_bytes;
     const TileSource gu_src = make_tile_source(expert_base + g.gu_tiles_off, (size_t)g.gu_rb * g.gd * kTileBytes,
                                                expert_base + g.gu_scales_off, (size_t)g.gu_rb * g.gd * kTileScaleBytes);
@@ -341,14 +360,16 @@ __device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps
 #pragma unroll
         for (int u = 0; u < kRing; ++u) ring_fill(ring, u, gu_src, rb0 * g.gd + min(g0 + u, g_last), lane);
     }
-    if (plan_out) build_plan_routes(ps, n_routes, plan_out, route_expert);
+    if (!DENSE && plan_out) build_plan_routes(ps, n_routes, plan_out, route_expert);
     if (!has_rows) return;
     if (!prepared) prepare_token_rows<F16>(lane, x0, x1, sx);
     // this lane finishes token column 4 jq + ks; `stores` = which of that row's top_k routes go to the expert
     // (one bit at most unless a row names an expert twice)
     const uint32_t col = 4 * jq + ks;
     uint32_t stores = 0;
-    if (col < rows) {
+    if (DENSE) {
+        stores = col < rows ? 1u : 0u;
+    } else if (col < rows) {
         const uint32_t *set = reinterpret_cast<const uint32_t *>(&ps.routes_of[slot_expert]);
         const uint32_t first = col * top_k, word = first >> 5;
         const uint64_t pair = (uint64_t)set[word] | ((uint64_t)(word < 3 ? set[word + 1] : 0u) << 32);
@@ -385,7 +406,7 @@ __device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps
     }
 }
 
-template <bool F16>
+template <bool F16, bool DENSE = false>
 __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                                     uint32_t top_k, uint32_t n_experts,
                                                                     const uint32_t *__restrict__ idx,
@@ -398,7 +419,7 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     uint32_t route_idx = 0;
     uint16_t route_w = 0;
-    if (threadIdx.x < n_routes) {
+    if (!DENSE && threadIdx.x < n_routes) {
         route_idx = idx[threadIdx.x];
         route_w = w[threadIdx.x];
     }
@@ -407,7 +428,7 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     uint4 x0[kRing], x1[kRing];
     load_token_rows(x, x_stride, n_routes / top_k, lane, k, x0, x1);
     f32x4 sx[kRing];
-    gate_up_rows<F16>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, sx, false, acts);
+    gate_up_rows<F16, DENSE>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, sx, false, acts);
 }
 
 // Router and gate/up of a decode step or verify block in ONE launch: the logits, the top-k select and the routes'
@@ -646,9 +667,11 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
                                                           const VerifyPlan *__restrict__ plan,
                                                           const uint16_t *__restrict__ acts,
                                                           float *__restrict__ partials_f32,
-                                                          uint16_t *__restrict__ partials_bf16, uint32_t parts) {
+                                                          uint16_t *__restrict__ partials_bf16, uint32_t parts, RouteMail *mail) {
     __shared__ __align__(16) uint8_t s_act[kMaxRows * kDownLdsRow];
     __shared__ uint32_t s_route[kMaxRows];
+    // the last launch of a call that leaves its rows un-combined: the routing launch of this call has read the epoch
+    if (mail && blockIdx.x == 0 && threadIdx.x == 0) advance_epoch(mail);
     const uint32_t slot_id = blockIdx.x / parts, part = blockIdx.x % parts;
     const PlanSlot &slot = plan->slots[slot_id];
     const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
@@ -737,14 +760,17 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
 // grid are dealt to the live experts and the four waves of a block split K as in the gate/up kernel, each
 // with its slice of the activation rows in registers; the partial sums meet in LDS and wave ks finishes
 // token slots 4 * (lane / 16) + ks.
-template <bool OUT_BF16, bool F16>
+// DENSE (dense_rows > 0 rows of a dense FFN: expert 0, route r = row r): nothing is read from the plan, so the weights
+// and the activation rows are requested with the kernel's first instructions instead of two and three dependent
+// round trips in.
+template <bool OUT_BF16, bool F16, bool DENSE = false>
 __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                                         const VerifyPlan *__restrict__ plan,
                                                                         const uint16_t *__restrict__ acts,
                                                                         float *__restrict__ partials_f32,
-                                                                        uint16_t *__restrict__ partials_bf16) {
+                                                                        uint16_t *__restrict__ partials_bf16, uint32_t dense_rows) {
     __shared__ float s_red[2][kKSplit][8][64];
-    const uint32_t n_live = __builtin_amdgcn_readfirstlane(plan->n_live);
+    const uint32_t n_live = DENSE ? 1u : __builtin_amdgcn_readfirstlane(plan->n_live);
     if (n_live == 0) return;
     const uint32_t bid = blockIdx.x;
     const uint32_t blocks_per_slot = max(1u, min(g.dn_rbp, gridDim.x / n_live));
@@ -754,10 +780,11 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
     split_range(g.dn_rbp, blocks_per_slot, bid % blocks_per_slot, rb0, rb1);
     if (rb0 >= rb1) return;
     const PlanSlot &slot = plan->slots[slot_id];
-    const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
-    const uint32_t expert = __builtin_amdgcn_readfirstlane(slot.expert);
+    const uint32_t n = DENSE ? dense_rows : __builtin_amdgcn_readfirstlane(slot.n);
+    const uint32_t expert = DENSE ? 0u : __builtin_amdgcn_readfirstlane(slot.expert);
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15, jq = lane >> 4;
+    auto route_of = [&](uint32_t i) { return DENSE ? i : slot.routes[i]; };
     const uint8_t *expert_base = arena_layer + (size_t)expert * g.expert_bytes;
     const uint32_t per = (g.gf + kKSplit - 1) / kKSplit;
     const uint32_t g0 = min(ks * per, g.gf), g1 = min(g.gf, g0 + per), ng = g1 - g0;
@@ -771,8 +798,8 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
     // bytes (slot lane / 4, chunk lane % 4) and turned into the operand layout by cross-lane moves
     // (with one or two rows the operand layout itself is as cheap to load, and needs no moves)
     const bool gather4 = n > 2;
-    const uint16_t *arow = gather4 ? acts + (size_t)slot.routes[min(lane >> 2, n - 1)] * g.f + 8 * (lane & 3)
-                                   : acts + (size_t)slot.routes[min(j, n - 1)] * g.f + 8 * jq;
+    const uint16_t *arow = gather4 ? acts + (size_t)route_of(min(lane >> 2, n - 1)) * g.f + 8 * (lane & 3)
+                                   : acts + (size_t)route_of(min(j, n - 1)) * g.f + 8 * jq;
     uint4 x0[kRing], x1[kRing];
 #pragma unroll
     for (int u = 0; u < kRing; ++u) {
@@ -800,7 +827,7 @@ __global__ __launch_bounds__(256, 2) void skinny_down_ksplit_persistent(const ui
 #pragma unroll
     for (int u = 0; u < kRing; ++u) sx[u] = group_input_sum<F16>(x0[u], x1[u]);
     const uint32_t my_ts = 4 * jq + ks;     // the token slot this lane finishes
-    const size_t out_base = (size_t)slot.routes[min(my_ts, n - 1)] * g.d;
+    const size_t out_base = (size_t)route_of(min(my_ts, n - 1)) * g.d;
 
     for (uint32_t rb = rb0; rb < rb1; ++rb) {
         const uint32_t next_row = min(rb + 1, rb1 - 1) * g.gf;
@@ -978,12 +1005,15 @@ template <bool F16>
 hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
                             const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
                             const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16, VerifyPlan *plan, uint16_t *acts,
-                            float *partials_f32, uint32_t n_cus, KernelTimer *timer, const RouteFusion *route) {
+                            float *partials_f32, uint32_t n_cus, KernelTimer *timer, const RouteFusion *route, bool dense) {
     // `route`: the routes are not there yet - idx / w are where this call has to write them. One launch does the
     // router and gate/up when the expert fits the persistent kernel, the combine follows in this call (it advances
     // the epoch) and the router rows are 8-byte aligned; otherwise the router's own two launches go first.
     const bool fits_ring = (g.gd + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
-    const bool fuse = route && route->one_launch && route->resident_blocks >= t && fits_ring && y && !partials_bf16 && top_k <= 8 &&
+    // y == nullptr (and no 16-bit rows wanted): the call ends with the down projection and leaves the un-weighted fp32
+    // rows, the plan's route_valid and the routes' weights to a later launch that combines them (the layer tail)
+    const bool rows_only = !y && !partials_bf16;
+    const bool fuse = route && route->one_launch && route->resident_blocks >= t && fits_ring && !partials_bf16 && top_k <= 8 &&
                       n_experts <= FFMOE_MAX_EXPERTS && reinterpret_cast<uintptr_t>(route->router_x) % 8 == 0 &&
                       route->router_x_stride % 4 == 0;
     if (route && !fuse) {
@@ -998,7 +1028,7 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     const bool dn_whole = g.gf <= (uint32_t)kRing;                                     // a wave holds all of K
     const bool dn_ksplit = !dn_whole && (g.gf + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
     const uint32_t resident = 2 * n_cus;       // blocks the chip holds at once (__launch_bounds__(256, 2))
-    const bool decode_form = t == 1 && dn_whole && !partials_bf16 && top_k <= 8;
+    const bool decode_form = t == 1 && dn_whole && !partials_bf16 && !rows_only && top_k <= 8;
     if (fuse) {
         // at least one block per row (it selects the row's routes), at most what is resident at once
         const uint32_t blocks = min(route->resident_blocks, max(max(slots, t), min(route->resident_blocks, slots * g.gu_rb)));
@@ -1013,8 +1043,12 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     } else if (gu_persistent) {
         // plan slot of the profile stays empty: the gate/up kernel builds the plan itself
         const uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
-        hipLaunchKernelGGL(skinny_gate_up_persistent<F16>, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, idx,
-                           w, t * top_k, plan, x, x_stride, acts);
+        if (dense)
+            hipLaunchKernelGGL((skinny_gate_up_persistent<F16, true>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k,
+                               n_experts, idx, w, t * top_k, plan, x, x_stride, acts);
+        else
+            hipLaunchKernelGGL(skinny_gate_up_persistent<F16>, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, idx,
+                               w, t * top_k, plan, x, x_stride, acts);
     } else {
         hipLaunchKernelGGL(verify_plan_kernel, dim3(1), dim3(256), 0, s, idx, w, t * top_k, n_experts, plan);
         timer->mark(s, FFMOE_K_PLAN);
@@ -1044,16 +1078,20 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
         return hipSuccess;
     }
     const uint32_t dn_parts = (g.dn_rbp + 3) / 4;          // blocks per expert of the LDS form: four tile rows each
+    const bool dense_ksplit = dense && gu_persistent;      // the plan-free forms go together
     const dim3 dn_grid = dn_whole    ? dim3(slots * dn_parts)
                          : dn_ksplit ? dim3(max(slots, min(resident, slots * g.dn_rbp)))
                                      : dim3((g.dn_rbp + 3) / 4, slots);
 #define FFMOE_DOWN(BF)                                                                                                \
     if (dn_whole)                                                                                                     \
         hipLaunchKernelGGL((skinny_down_lds<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,          \
-                           partials_f32, partials_bf16, dn_parts);                                                    \
+                           partials_f32, partials_bf16, dn_parts, rows_only ? mail : nullptr);                         \
+    else if (dn_ksplit && dense_ksplit)                                                                               \
+        hipLaunchKernelGGL((skinny_down_ksplit_persistent<BF, F16, true>), dn_grid, dim3(256), 0, s, arena_layer, g,  \
+                           plan, acts, partials_f32, partials_bf16, t);                                               \
     else if (dn_ksplit)                                                                                               \
         hipLaunchKernelGGL((skinny_down_ksplit_persistent<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan,  \
-                           acts, partials_f32, partials_bf16);                                                        \
+                           acts, partials_f32, partials_bf16, 0u);                                                    \
     else                                                                                                              \
         hipLaunchKernelGGL((skinny_down_kernel<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,       \
                            partials_f32, partials_bf16)
@@ -1068,6 +1106,12 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     e = hipGetLastError();
     if (e != hipSuccess) return give_up(e);
     timer->mark(s, FFMOE_K_DOWN);
+    if (rows_only) {
+        // the epoch went on with the down launch; a down kernel that takes no mail gets a launch of its own for it
+        if (mail && !dn_whole) hipLaunchKernelGGL(advance_epoch_kernel, dim3(1), dim3(1), 0, s, mail);
+        timer->finish();
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(combine_kernel<F16>, dim3((g.d / 4 + 255) / 256, t), dim3(256), 0, s, partials_f32, w, plan, residual,
                        top_k, g.d, y, mail);
     e = hipGetLastError();
@@ -1187,11 +1231,13 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
                          VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer, bool f16,
-                         const RouteFusion *route) {
+                         const RouteFusion *route, bool dense) {
+    // dense: the caller vouches that this is a dense FFN - one expert, top_k = 1, every row at weight 1
+    dense = dense && n_experts == 1 && top_k == 1 && !route;
     return f16 ? launch_verify_as<true>(s, arena_layer, g, n_experts, top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                                        plan, acts, partials_f32, n_cus, timer, route)
+                                        plan, acts, partials_f32, n_cus, timer, route, dense)
                : launch_verify_as<false>(s, arena_layer, g, n_experts, top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                                         plan, acts, partials_f32, n_cus, timer, route);
+                                         plan, acts, partials_f32, n_cus, timer, route, dense);
 }
 
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,

@@ -47,7 +47,7 @@ EXPORTS = [
     "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
     "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
-    "ffmoe_layer_tail", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
+    "ffmoe_layer_tail", "ffmoe_layer_tail_routed", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
     "ffmoe_verify_static",
 ]
@@ -220,6 +220,7 @@ def lib() -> C.CDLL:
     L.ffmoe_post_attn_setup.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, u32, vp, u32, vp, vp, vp, u32, u32,
                                         C.c_float, errp]
     L.ffmoe_layer_tail.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, vp, u32, u32, C.c_float, C.c_float, errp]
+    L.ffmoe_layer_tail_routed.argtypes = [vp, vp, vp, vp, u32, vp, u32, vp, vp, u32, C.c_float, C.c_float, errp]
     _lib = L
     return L
 
@@ -411,11 +412,12 @@ class Context:
                                    _ptr(y), C.byref(err)), err)
         return y
 
-    def route_verify(self, layer: int, router_x, x, residual=None, out=None):
-        """Router + expert pass of a block of <= 16 rows in one call. Returns (y, idx, w)."""
+    def route_verify(self, layer: int, router_x, x, residual=None, out=None, combine: bool = True):
+        """Router + expert pass of a block of <= 16 rows in one call. Returns (y, idx, w); combine=False leaves the
+        routes' rows un-combined in the context (y is None) for layer_tail_routed."""
         import torch
         t, k = x.shape[0], self.shape.top_k
-        y = out if out is not None else torch.empty((t, self.shape.d), dtype=self.act, device=x.device)
+        y = None if not combine else out if out is not None else torch.empty((t, self.shape.d), dtype=self.act, device=x.device)
         idx = torch.empty((t, k), dtype=torch.int32, device=x.device)
         w = torch.empty((t, k), dtype=self.act, device=x.device)
         err = C.c_char_p()
@@ -531,6 +533,15 @@ class Context:
         _check(self.L.ffmoe_layer_tail(self._h, _stream(), _ptr(h2), _row_stride(h2), _ptr(h1), _row_stride(h1), _ptr(hidden),
                                        _row_stride(hidden), _ptr(w_postffn2), _ptr(w_postffn), t, d, eps, layer_scalar,
                                        C.byref(err)), err)
+        return hidden
+
+    def layer_tail_routed(self, route_w, h1, hidden, w_postffn2, w_postffn, layer_scalar: float, eps: float = 1e-6):
+        """layer_tail on the rows the last route_verify(..., combine=False) left un-combined (weights: that call's w)."""
+        t = hidden.shape[0]
+        err = C.c_char_p()
+        _check(self.L.ffmoe_layer_tail_routed(self._h, _stream(), _ptr(route_w), _ptr(h1), _row_stride(h1), _ptr(hidden),
+                                              _row_stride(hidden), _ptr(w_postffn2), _ptr(w_postffn), t, eps, layer_scalar,
+                                              C.byref(err)), err)
         return hidden
 
     def layer_tail_norms(self, h2, h1, hidden, w_postffn1, w_postffn2, w_postffn, layer_scalar: float, w_next=None,

@@ -652,12 +652,26 @@ def main():
         def run_block(concurrent):
             layer_block(counter["i"], concurrent)
             counter["i"] += 1
+        def layer_block_fused(i):
+            # the same block with the routed experts' combine folded into the layer tail: six launches
+            layer = i % L
+            ctx.post_attn_setup(hid_b, att_b, wn_b[0], wn_b[1], wn_b[2], out=outs_b)
+            dense.dense_ffn(i % LS, outs_b[0], out=h1_b)
+            rc = Lib.ffmoe_route_verify(h, stream, layer, pouts[2], D, pouts[1], D, T, None, None, pidx, pw, C.byref(err))
+            if rc:
+                raise RuntimeError(err.value)
+            ctx.layer_tail_routed(w, h1_b, hid_b, wn_b[3], wn_b[4], 1.0)
+
+        def run_fused():
+            layer_block_fused(counter["i"])
+            counter["i"] += 1
         t_seq = timed(lambda: run_block(False), 120, warm=30)
         t_con = timed(lambda: run_block(True), 120, warm=30)
+        t_fus = timed(run_fused, 120, warm=30)
         # the same chain of L layers as a HIP graph: nine launches per layer from Python are host-bound,
         # a replay shows the device time (the library only enqueues kernels, so the chain captures as it is)
         graph_us = {}
-        for label, conc in (("one_stream", False), ("shared_expert_on_second_stream", True)):
+        for label, conc in (("one_stream", False), ("shared_expert_on_second_stream", True), ("combine_in_layer_tail", None)):
             gph = torch.cuda.CUDAGraph()
             cap = torch.cuda.Stream()
             cap.wait_stream(main_s)
@@ -665,12 +679,16 @@ def main():
                 main_s = torch.cuda.current_stream()
                 stream = C.c_void_p(main_s.cuda_stream)
                 for i in range(L):
-                    layer_block(i, conc)
+                    if conc is None:
+                        layer_block_fused(i)
+                    else:
+                        layer_block(i, conc)
             main_s = torch.cuda.current_stream()
             stream = C.c_void_p(main_s.cuda_stream)
             graph_us[label] = round(timed(gph.replay, 8, warm=2) / L * 1e6, 2)
             del gph
         extra["layer_block_rows16"] = {"one_stream_us": round(t_seq * 1e6, 2), "shared_expert_on_second_stream_us": round(t_con * 1e6, 2),
+                                       "combine_in_layer_tail_us": round(t_fus * 1e6, 2),
                                        "hip_graph_replay_us": graph_us,
                                        "steps": "post-attention setup, shared expert, router, routed experts, layer tail"}
         dense.close()

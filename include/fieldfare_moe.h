@@ -183,7 +183,10 @@ int ffmoe_verify_partials(ffmoe_ctx *ctx, void *stream, uint32_t layer, const ui
  * to itself - and correct either way: a wave that has waited FFMOE_DEFAULT_HANDOVER_TICKS for a word (other work
  * on the GPU keeps the block that makes it from running) stops waiting and computes what it waited for itself,
  * with the same arithmetic in the same order, so the call returns the same routes and rows, only later.
- * ffmoe_handover_giveups counts such waves. */
+ * ffmoe_handover_giveups counts such waves.
+ * y may be NULL (residual then too): the call ends with the down projection and leaves the routes' un-weighted fp32
+ * rows in the context, for ffmoe_layer_tail_routed to combine in its load stage (one launch and one pass over the
+ * rows less per layer); out_idx / out_w are written as usual. */
 int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *router_x,
                        uint32_t router_x_stride, const uint16_t *x, uint32_t x_stride, uint32_t t,
                        const uint16_t *residual, uint16_t *y, uint32_t *out_idx, uint16_t *out_w, char **err);
@@ -372,6 +375,16 @@ int ffmoe_post_attn_setup(ffmoe_ctx *ctx, void *stream, uint16_t *hidden, uint32
 int ffmoe_layer_tail(ffmoe_ctx *ctx, void *stream, const uint16_t *h2, uint32_t h2_stride, const uint16_t *h1,
                      uint32_t h1_stride, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2,
                      const uint16_t *w_postffn, uint32_t t, uint32_t d, float eps, float layer_scalar, char **err);
+
+/* ffmoe_layer_tail on the rows the last ffmoe_route_verify(..., y = NULL, ...) call on this context and stream left
+ * un-combined: h2 = the router-weighted combine of those rows under `route_w` (that call's out_w, [t][top_k]), made
+ * while the tail loads its inputs instead of by a launch of its own, then the tail as above with d = the context's
+ * hidden size. Bit for bit ffmoe_route_verify with y followed by ffmoe_layer_tail. This is the fusion of the routed
+ * experts' weighted combine (Metal/Prefill/prefill.metal:544-565) into the layer tail (:320-399) for the decode /
+ * verify block (t <= 16). */
+int ffmoe_layer_tail_routed(ffmoe_ctx *ctx, void *stream, const uint16_t *route_w, const uint16_t *h1, uint32_t h1_stride,
+                            uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
+                            uint32_t t, float eps, float layer_scalar, char **err);
 
 /* The layer tail with the two decode norms either side of it folded in: h1 arrives BEFORE its own norm
  * (w_postffn1, the shared expert's post-FFN-1 norm; h1 is left as found), and when w_next / normed are

@@ -591,3 +591,42 @@ def test_expert_named_more_than_16_times_keeps_its_first_16_routes(small, oracle
     got = oracle.bf16_to_float(bits_of(ctx.verify(1, x, idx, w)))
     ref = oracle.moe_experts(small["pool"], xb, idx_np, kept)
     assert rel_err(got, ref) <= 1e-2 and cosine(got, ref) >= 0.9999, (rel_err(got, ref), cosine(got, ref))
+
+
+@pytest.mark.parametrize("which,t,stride_pad", [("small", 1, 0), ("small", 7, 5), ("real", 1, 0), ("real", 16, 0), ("real", 16, 13)])
+def test_layer_tail_routed_equals_route_verify_then_layer_tail(small, real, oracle, torch, which, t, stride_pad):
+    """The routed experts' weighted combine folded into the layer tail (ffmoe_route_verify without y, then
+    ffmoe_layer_tail_routed) against the separate calls: the new hidden rows bit for bit, padding untouched; and the
+    separate calls' hidden rows are the oracle's layer tail on the combined rows."""
+    fx = small if which == "small" else real
+    ctx, d, layer = fx["ctx"], fx["d"], 1 if which == "small" else 0
+    g = oracle.seed_tree_key(0x7A11, f"tail-routed-{which}-{t}-{stride_pad}")
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    x = bf16_tensor(torch, xb)
+    h1 = np.full((t, d + stride_pad), oracle.bf16_bits(np.float32(-23.0)), np.uint16)
+    hid = np.full((t, d + stride_pad), oracle.bf16_bits(np.float32(-25.0)), np.uint16)
+    h1[:, :d] = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    hid[:, :d] = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    w2 = oracle.bf16_bits(g.uniform(0.5, 1.5, d))
+    w1 = oracle.bf16_bits(g.uniform(0.5, 1.5, d))
+    tw2, tw1 = bf16_tensor(torch, w2), bf16_tensor(torch, w1)
+    th1 = bf16_tensor(torch, h1)
+    # separate calls
+    y, idx_a, w_a = ctx.route_verify(layer, x, x)
+    hid_a = bf16_tensor(torch, hid)
+    ctx.layer_tail(y, th1, hid_a, tw2, tw1, 0.875, 1e-6, d=d)
+    want = hid.copy()
+    want[:, :d] = oracle.layer_tail(bits_of(y), h1[:, :d], hid[:, :d], w2, w1, 0.875, 1e-6)
+    assert np.array_equal(bits_of(hid_a), want)
+    # the fused pair
+    none, idx_b, w_b = ctx.route_verify(layer, x, x, combine=False)
+    assert none is None
+    hid_b = bf16_tensor(torch, hid)
+    ctx.layer_tail_routed(w_b, th1, hid_b, tw2, tw1, 0.875, 1e-6)
+    assert np.array_equal(idx_a.cpu().numpy(), idx_b.cpu().numpy()) and np.array_equal(bits_of(w_a), bits_of(w_b))
+    assert np.array_equal(bits_of(hid_b), bits_of(hid_a))
+    assert np.array_equal(bits_of(th1), h1)
+    # the next call on the context is an ordinary one again (the epoch moved on with the un-combined call)
+    y2, idx_c, _ = ctx.route_verify(layer, x, x)
+    assert np.array_equal(bits_of(y2), bits_of(y)) and np.array_equal(idx_c.cpu().numpy(), idx_a.cpu().numpy())
+    assert ctx.handover_giveups() == 0
