@@ -837,7 +837,8 @@ int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales
     FF_MX(hipMalloc(&mx->tiles, matrix_tiles_bytes(m, n)));
     FF_MX(hipMalloc(&mx->scales, matrix_scales_bytes(m, n)));
     if (with_greedy) {
-        FF_MX(hipMalloc(&mx->partials, (size_t)FFMOE_MAX_VERIFY_ROWS * greedy_segments(m, ctx->n_cus) * sizeof(unsigned long long)));
+        // per input row and block of the GEMV grid: the winner's key, then its softmax pair (8 bytes each)
+        FF_MX(hipMalloc(&mx->partials, 2 * (size_t)FFMOE_MAX_VERIFY_ROWS * greedy_segments(m, ctx->n_cus) * sizeof(unsigned long long)));
     }
     // the source may live on the host (an mmap of the checkpoint) or on the device
     const uint8_t *dw = w;
@@ -908,16 +909,43 @@ int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_
     return FFMOE_OK;
 }
 
-int ffmoe_matrix_greedy(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
-                        uint32_t *out_tokens, char **err) {
+static int matrix_greedy_common(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
+                                float softcap, uint32_t *out_tokens, float *out_conf, char **err) {
     if (int rc = check_matrix_call(mx, x, x_stride, rows, err)) return rc;
     if (!out_tokens) return fail(err, FFMOE_ERR_INVALID, "null argument");
     if (!mx->partials) return fail(err, FFMOE_ERR_INVALID, "matrix was created without the greedy scratch");
+    if (!(softcap >= 0.0f) || std::isinf(softcap)) return fail(err, FFMOE_ERR_INVALID, "softcap must be finite and >= 0 (0 disables it)");
     ffmoe_ctx *ctx = mx->ctx;
     hipStream_t s = static_cast<hipStream_t>(stream);
     ctx->timer.begin(s);
     FF_HIP(launch_matrix_greedy(s, mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows, mx->partials, out_tokens,
-                                ctx->n_cus, ctx->f16, &ctx->timer));
+                                ctx->n_cus, ctx->f16, &ctx->timer, softcap, out_conf));
+    ctx->timer.finish();
+    return FFMOE_OK;
+}
+
+int ffmoe_matrix_greedy(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
+                        uint32_t *out_tokens, char **err) {
+    return matrix_greedy_common(mx, stream, x, x_stride, rows, 0.0f, out_tokens, nullptr, err);
+}
+
+int ffmoe_matrix_greedy_conf(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
+                             float softcap, uint32_t *out_tokens, float *out_conf, char **err) {
+    if (!out_conf) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    return matrix_greedy_common(mx, stream, x, x_stride, rows, softcap, out_tokens, out_conf, err);
+}
+
+int ffmoe_argmax_rows(ffmoe_ctx *ctx, void *stream, const float *logits, uint32_t stride, uint32_t rows, uint32_t count,
+                      float softcap, uint32_t *out_index, float *out_conf, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!logits || !out_index) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (rows == 0 || count == 0) return fail(err, FFMOE_ERR_INVALID, "rows and count must be positive");
+    if (stride < count) return fail(err, FFMOE_ERR_INVALID, "stride smaller than the row");
+    if (!(softcap >= 0.0f) || std::isinf(softcap)) return fail(err, FFMOE_ERR_INVALID, "softcap must be finite and >= 0 (0 disables it)");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    ctx->timer.begin(s);
+    FF_HIP(launch_argmax_rows(s, logits, stride, rows, count, softcap, out_index, out_conf));
+    ctx->timer.mark(s, FFMOE_K_ARGMAX);
     ctx->timer.finish();
     return FFMOE_OK;
 }

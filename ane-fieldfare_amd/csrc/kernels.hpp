@@ -177,7 +177,11 @@ uint32_t greedy_segments(uint32_t m, uint32_t n_cus);
 // the GEMV with the greedy choice as its epilogue: per-block winners, then one block per input row
 hipError_t launch_matrix_greedy(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                                 const uint16_t *x, uint32_t x_stride, uint32_t rows, unsigned long long *partials,
-                                uint32_t *out, uint32_t n_cus, bool f16, KernelTimer *timer);
+                                uint32_t *out, uint32_t n_cus, bool f16, KernelTimer *timer, float softcap = 0.0f,
+                                float *out_conf = nullptr);
+// greedy choice (and the winner's softmax probability under the softcap) over rows of fp32 logits in memory
+hipError_t launch_argmax_rows(hipStream_t s, const float *logits, uint32_t stride, uint32_t rows, uint32_t count, float softcap,
+                              uint32_t *out, float *out_conf);
 
 // prefill.hip: routes come from (idx, w) [t][top_k], or from an explicit pair list when `pairs` != nullptr.
 // Writes y [t][d] (combined) when y != nullptr; un-weighted bf16 rows go to partials_out or to scratch.

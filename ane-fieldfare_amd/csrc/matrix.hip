@@ -78,25 +78,59 @@ __device__ __forceinline__ unsigned long long argmax_key(float v, uint32_t i) {
     return ((unsigned long long)ord << 32) | (0xFFFFFFFFu - i);
 }
 
+// The winner's probability under the final logit softcap, as argmax_rows_f32 leaves it for a drafter
+// (Metal/Sampling/logit.metal:946-1010): softmax over the finite logits, each capped to softcap * tanh(v / softcap)
+// when softcap > 0, kept as an online (maximum, sum of exp(c - maximum)) pair that merges associatively.
+struct SoftmaxAcc {
+    float m, s;      // m = -inf: nothing seen yet
+};
+__device__ __forceinline__ float capped(float v, float softcap) {
+    if (!(softcap > 0.0f)) return v;
+    // tanh z = 1 - 2 / (exp(2 z) + 1); exp saturates to inf / 0 cleanly, so large |z| give +-1
+    const float z = v / softcap;
+    return softcap * (1.0f - 2.0f / (__expf(2.0f * z) + 1.0f));
+}
+__device__ __forceinline__ void softmax_take(SoftmaxAcc &a, float v, float softcap) {
+    if (!(__builtin_fabsf(v) < INFINITY)) return;          // non-finite logits take no part (they never win either)
+    const float c = capped(v, softcap);
+    if (c > a.m) {
+        a.s = a.s * __expf(a.m - c) + 1.0f;                 // exp(-inf) = 0 covers the first value
+        a.m = c;
+    } else {
+        a.s += __expf(c - a.m);
+    }
+}
+__device__ __forceinline__ SoftmaxAcc softmax_merge(const SoftmaxAcc &a, const SoftmaxAcc &b) {
+    const float m = fmaxf(a.m, b.m);
+    if (m == -INFINITY) return SoftmaxAcc{-INFINITY, 0.0f};
+    return SoftmaxAcc{m, a.s * __expf(a.m - m) + b.s * __expf(b.m - m)};
+}
+__device__ __forceinline__ SoftmaxAcc softmax_shuffle(const SoftmaxAcc &a, int mask) {
+    return SoftmaxAcc{__shfl_xor(a.m, mask, 64), __shfl_xor(a.s, mask, 64)};
+}
+
 // y[r][m] = sum_g [ s_g * sum_k q_k x_k + b_g * sum_k x_k ] (moe.metal:323-378, logit.metal:614-667) for all
 // input rows at once. grid = (blocks): every block walks a range of 32-row tiles; its four waves split K
 // (at most kRing groups each), keep their slice of the input rows in registers and refill the weight
 // ring across tiles; per tile the partial sums meet in LDS, are added in wave order, and each wave
 // stores a quarter of the input rows. GREEDY: nothing is stored per weight row; every lane keeps the best
 // (value, index) key of the sums it finishes and the block leaves one key per input row in
-// y_[row * gridDim.x + block], so the [rows][m] fp32 logits never travel to memory and back.
-template <bool Y_F32, bool F16, bool GREEDY = false>
+// y_[row * gridDim.x + block], so the [rows][m] fp32 logits never travel to memory and back. CONF: the block also
+// leaves the softmax pair of the sums it finished in conf_part[row * gridDim.x + block].
+template <bool Y_F32, bool F16, bool GREEDY = false, bool CONF = false>
 __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__restrict__ tiles,
                                                              const uint8_t *__restrict__ scales, uint32_t m,
                                                              uint32_t n_groups, const uint16_t *__restrict__ x,
                                                              uint32_t x_stride, uint32_t rows, void *__restrict__ y_,
-                                                             uint32_t y_stride) {
+                                                             uint32_t y_stride, float2 *__restrict__ conf_part = nullptr,
+                                                             float softcap = 0.0f) {
     __shared__ float s_red[2][kKSplit][8][64];
     const uint32_t n_tiles = (m + 31) / 32;
     uint32_t rb0, rb1;
     split_range(n_tiles, gridDim.x, blockIdx.x, rb0, rb1);
     if (rb0 >= rb1) {
         if (GREEDY && threadIdx.x < rows) reinterpret_cast<unsigned long long *>(y_)[(size_t)threadIdx.x * gridDim.x + blockIdx.x] = 0ull;
+        if (CONF && threadIdx.x < rows) conf_part[(size_t)threadIdx.x * gridDim.x + blockIdx.x] = make_float2(-INFINITY, 0.0f);
         return;
     }
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -123,6 +157,7 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
     float *y32 = reinterpret_cast<float *>(y_);
     uint16_t *y16 = reinterpret_cast<uint16_t *>(y_);
     unsigned long long best = 0ull;
+    SoftmaxAcc soft{-INFINITY, 0.0f};
 
     for (uint32_t rb = rb0; rb < rb1; ++rb) {
         const uint32_t next_row = min(rb + 1, rb1 - 1) * n_groups;
@@ -152,6 +187,10 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
                 const unsigned long long ka = row_a < m ? argmax_key(va, row_a) : 0ull;
                 const unsigned long long kb = row_b < m ? argmax_key(vb, row_b) : 0ull;
                 best = max(best, max(ka, kb));
+                if (CONF) {
+                    if (row_a < m) softmax_take(soft, va, softcap);
+                    if (row_b < m) softmax_take(soft, vb, softcap);
+                }
             } else if (Y_F32) {
                 if (row_a < m) y32[base + row_a] = va;
                 if (row_b < m) y32[base + row_b] = vb;
@@ -167,6 +206,11 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
         for (int mk = 8; mk >= 1; mk >>= 1) best = max(best, (unsigned long long)__shfl_xor(best, mk, 64));
         if (j == 0 && my_row < rows)
             reinterpret_cast<unsigned long long *>(y_)[(size_t)my_row * gridDim.x + blockIdx.x] = best;
+        if (CONF) {
+#pragma unroll
+            for (int mk = 8; mk >= 1; mk >>= 1) soft = softmax_merge(soft, softmax_shuffle(soft, mk));
+            if (j == 0 && my_row < rows) conf_part[(size_t)my_row * gridDim.x + blockIdx.x] = make_float2(soft.m, soft.s);
+        }
     }
 }
 
@@ -183,17 +227,75 @@ __device__ __forceinline__ unsigned long long block_max_key(unsigned long long k
     return k;
 }
 
+// The block's softmax pair, the same in every thread.
+__device__ __forceinline__ SoftmaxAcc block_softmax(SoftmaxAcc a, float2 *s_p) {
+#pragma unroll
+    for (int mk = 32; mk >= 1; mk >>= 1) a = softmax_merge(a, softmax_shuffle(a, mk));
+    if ((threadIdx.x & 63) == 0) s_p[threadIdx.x >> 6] = make_float2(a.m, a.s);
+    __syncthreads();
+    a = SoftmaxAcc{s_p[0].x, s_p[0].y};
+    for (uint32_t v = 1; v < blockDim.x / 64; ++v) a = softmax_merge(a, SoftmaxAcc{s_p[v].x, s_p[v].y});
+    return a;
+}
+
+// The winner's value from its key (argmax_key is a bijection on the finite values).
+__device__ __forceinline__ float key_value(unsigned long long k) {
+    const uint32_t ord = (uint32_t)(k >> 32);
+    return __uint_as_float((ord & 0x80000000u) ? (ord & 0x7FFFFFFFu) : ~ord);
+}
+
+__device__ __forceinline__ float winner_confidence(unsigned long long best, const SoftmaxAcc &all, float softcap) {
+    if (best == 0ull || !(all.s > 0.0f)) return 0.0f;
+    return __expf(capped(key_value(best), softcap) - all.m) / all.s;
+}
+
 __global__ __launch_bounds__(256) void argmax_final_kernel(const unsigned long long *__restrict__ part, uint32_t n_seg,
-                                                           uint32_t *__restrict__ out) {
+                                                           uint32_t *__restrict__ out, const float2 *__restrict__ conf_part,
+                                                           float softcap, float *__restrict__ out_conf) {
     __shared__ unsigned long long s_k[4];
+    __shared__ float2 s_p[4];
     const uint32_t row = blockIdx.x;
     unsigned long long best = 0ull;
+    SoftmaxAcc soft{-INFINITY, 0.0f};
     for (uint32_t i = threadIdx.x; i < n_seg; i += 256) {
         const unsigned long long k = part[(size_t)row * n_seg + i];
         best = k > best ? k : best;
+        if (out_conf) {
+            const float2 q = conf_part[(size_t)row * n_seg + i];
+            soft = softmax_merge(soft, SoftmaxAcc{q.x, q.y});
+        }
     }
     best = block_max_key(best, s_k);
     if (threadIdx.x == 0) out[row] = best ? 0xFFFFFFFFu - (uint32_t)best : 0u;
+    if (out_conf) {
+        soft = block_softmax(soft, s_p);
+        if (threadIdx.x == 0) out_conf[row] = winner_confidence(best, soft, softcap);
+    }
+}
+
+// argmax_rows_f32 (Metal/Sampling/logit.metal:946-1010): the greedy choice over rows of fp32 logits that are in
+// memory already (the listed GEMV's output: a drafter's hot vocabulary), one block per row: the largest finite value,
+// ties to the lowest position, 0xFFFFFFFF and confidence 0 when no value is finite; and the winner's probability
+// under the softcap.
+__global__ __launch_bounds__(256) void argmax_rows_kernel(const float *__restrict__ logits, uint32_t stride, uint32_t count,
+                                                          float softcap, uint32_t *__restrict__ out, float *__restrict__ out_conf) {
+    __shared__ unsigned long long s_k[4];
+    __shared__ float2 s_p[4];
+    const float *row = logits + (size_t)blockIdx.x * stride;
+    unsigned long long best = 0ull;
+    SoftmaxAcc soft{-INFINITY, 0.0f};
+    for (uint32_t i = threadIdx.x; i < count; i += 256) {
+        const float v = row[i];
+        const unsigned long long k = argmax_key(v, i);
+        best = k > best ? k : best;
+        if (out_conf) softmax_take(soft, v, softcap);
+    }
+    best = block_max_key(best, s_k);
+    if (threadIdx.x == 0) out[blockIdx.x] = best ? 0xFFFFFFFFu - (uint32_t)best : 0xFFFFFFFFu;
+    if (out_conf) {
+        soft = block_softmax(soft, s_p);
+        if (threadIdx.x == 0) out_conf[blockIdx.x] = winner_confidence(best, soft, softcap);
+    }
 }
 
 }  // namespace
@@ -227,21 +329,29 @@ hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t
 // keys per input row that launch_matrix_greedy leaves between its two kernels
 uint32_t greedy_segments(uint32_t m, uint32_t n_cus) { return min(2 * n_cus, (m + 31) / 32); }
 
+// `partials`: [16][segments] keys, then (when out_conf is wanted) [16][segments] softmax pairs
 hipError_t launch_matrix_greedy(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                                 const uint16_t *x, uint32_t x_stride, uint32_t rows, unsigned long long *partials,
-                                uint32_t *out, uint32_t n_cus, bool f16, KernelTimer *timer) {
+                                uint32_t *out, uint32_t n_cus, bool f16, KernelTimer *timer, float softcap, float *out_conf) {
     const dim3 grid(greedy_segments(m, n_cus));
-    if (f16)
-        hipLaunchKernelGGL((matrix_gemv_kernel<true, true, true>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride,
-                           rows, partials, 0u);
-    else
-        hipLaunchKernelGGL((matrix_gemv_kernel<true, false, true>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride,
-                           rows, partials, 0u);
+    float2 *conf_part = reinterpret_cast<float2 *>(partials + (size_t)FFMOE_MAX_VERIFY_ROWS * grid.x);
+#define FFMOE_GREEDY(H, C)                                                                                                  \
+    hipLaunchKernelGGL((matrix_gemv_kernel<true, H, true, C>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, \
+                       rows, partials, 0u, conf_part, softcap)
+    if (f16) { if (out_conf) FFMOE_GREEDY(true, true); else FFMOE_GREEDY(true, false); }
+    else { if (out_conf) FFMOE_GREEDY(false, true); else FFMOE_GREEDY(false, false); }
+#undef FFMOE_GREEDY
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_GEMV);
-    hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, partials, grid.x, out);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, partials, grid.x, out, conf_part, softcap, out_conf);
     timer->mark(s, FFMOE_K_ARGMAX);
+    return hipGetLastError();
+}
+
+hipError_t launch_argmax_rows(hipStream_t s, const float *logits, uint32_t stride, uint32_t rows, uint32_t count, float softcap,
+                              uint32_t *out, float *out_conf) {
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(256), 0, s, logits, stride, count, softcap, out, out_conf);
     return hipGetLastError();
 }
 

@@ -46,7 +46,7 @@ EXPORTS = [
     "ffmoe_verify", "ffmoe_verify_partials", "ffmoe_last_live_experts", "ffmoe_handover_giveups", "ffmoe_probe_stream", "ffmoe_reduce_token_major",
     "ffmoe_gemv_int4", "ffmoe_set_profiling", "ffmoe_get_profile", "ffmoe_prefill", "ffmoe_prefill_pairs",
     "ffmoe_prefill_plan_stats", "ffmoe_matrix_create", "ffmoe_matrix_destroy", "ffmoe_matrix_gemv",
-    "ffmoe_matrix_greedy", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
+    "ffmoe_matrix_greedy", "ffmoe_matrix_greedy_conf", "ffmoe_argmax_rows", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
     "ffmoe_layer_tail", "ffmoe_layer_tail_routed", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
     "ffmoe_verify_static",
@@ -106,6 +106,17 @@ class Matrix:
         _check(self.L.ffmoe_matrix_greedy(self._h, _stream(), _ptr(x), _row_stride(x), rows, _ptr(out), C.byref(err)),
                err)
         return out
+
+    def greedy_conf(self, x, softcap: float = 0.0):
+        """(tokens int32 [rows], confidence fp32 [rows]): the greedy choice and its softmax probability under the softcap."""
+        import torch
+        rows = x.shape[0]
+        out = torch.empty((rows,), dtype=torch.int32, device=x.device)
+        conf = torch.empty((rows,), dtype=torch.float32, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_matrix_greedy_conf(self._h, _stream(), _ptr(x), _row_stride(x), rows, softcap, _ptr(out), _ptr(conf),
+                                               C.byref(err)), err)
+        return out, conf
 
     def close(self):
         if self._h:
@@ -214,6 +225,8 @@ def lib() -> C.CDLL:
     L.ffmoe_matrix_destroy.restype = None
     L.ffmoe_matrix_gemv.argtypes = [vp, vp, vp, u32, u32, vp, u32, i32, errp]
     L.ffmoe_matrix_greedy.argtypes = [vp, vp, vp, u32, u32, vp, errp]
+    L.ffmoe_matrix_greedy_conf.argtypes = [vp, vp, vp, u32, u32, C.c_float, vp, vp, errp]
+    L.ffmoe_argmax_rows.argtypes = [vp, vp, vp, u32, u32, u32, C.c_float, vp, vp, errp]
     L.ffmoe_upload_expert_parts.argtypes = [vp, u32, u32, C.POINTER(Projection), C.POINTER(Projection),
                                             C.POINTER(Projection), i32, errp]
     L.ffmoe_dense_ffn.argtypes = [vp, vp, u32, vp, u32, u32, vp, errp]
@@ -571,6 +584,19 @@ class Context:
     def matrix(self, W, S, B, greedy: bool = False, w_byte_offset: int = 0):
         """Resident re-tiled copy of W uint8 [M, N/2], S/B bf16 bits [M, N/64] (numpy arrays or tensors)."""
         return Matrix(self, W, S, B, greedy, w_byte_offset)
+
+    def argmax_rows(self, logits, count: int | None = None, softcap: float = 0.0, want_conf: bool = True):
+        """Greedy position per row of fp32 logits [rows, >= count] (int32, -1 when no value is finite) and, with
+        want_conf, the winner's softmax probability under the softcap."""
+        import torch
+        rows = logits.shape[0]
+        count = count or logits.shape[1]
+        out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+        conf = torch.empty((rows,), dtype=torch.float32, device=logits.device) if want_conf else None
+        err = C.c_char_p()
+        _check(self.L.ffmoe_argmax_rows(self._h, _stream(), _ptr(logits), _row_stride(logits), rows, count, softcap, _ptr(out),
+                                        _ptr(conf), C.byref(err)), err)
+        return (out, conf) if want_conf else out
 
     def gemv_int4_listed(self, W, S, B, ids, x):
         """GEMV over the weight rows listed in `ids` (int32 CUDA tensor [m]): y fp32 [R, m], y[:, o] = row ids[o]."""

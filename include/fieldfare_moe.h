@@ -290,7 +290,7 @@ typedef struct ffmoe_matrix ffmoe_matrix;
  * scratch for its lifetime (Kernels/Fusions/LMHeadChainInt4.swift:57-88). n must be a multiple of 64,
  * at most FFMOE_MATRIX_MAX_N; m is any count whose re-tiled form, ceil(m / 32) * (n / 64) KiB, stays below 4 GiB
  * (the reference's head tests use 4,099 rows; 262,144 x 2816 takes 352 MiB). with_greedy != 0
- * also allocates the scratch of ffmoe_matrix_greedy (a few KB of per-block winners). Blocking; not a
+ * also allocates the scratch of ffmoe_matrix_greedy / _conf (per-block winners and softmax pairs, 128 KiB). Blocking; not a
  * hot-path call. */
 int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                         uint32_t m, uint32_t n, int with_greedy, ffmoe_matrix **out, char **err);
@@ -312,6 +312,23 @@ int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_
  * input rows are the already normalised hidden rows (the reference runs its RMSNorm operator first). */
 int ffmoe_matrix_greedy(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
                         uint32_t *out_tokens, char **err);
+
+/* ffmoe_matrix_greedy that also leaves each row's confidence: the chosen token's softmax probability over the finite
+ * logits, each capped to softcap * tanh(logit / softcap) when softcap > 0 (0 disables the cap) - what
+ * argmax_rows_f32 writes to rowsConfidence for the DFlash drafter (Metal/Sampling/logit.metal:946-1010,
+ * LMHeadChainInt4.encodeGreedyRows with softcap, LMHeadChainInt4.swift:94-139,209-223). The token is chosen on the
+ * uncapped logits, as there. out_conf fp32 [rows] (0 for a row without a finite logit). The softmax sums run in
+ * this build's order (the reference's simd_sum leaves it open): a probability is comparable to 1e-5, not to the bit. */
+int ffmoe_matrix_greedy_conf(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
+                             float softcap, uint32_t *out_tokens, float *out_conf, char **err);
+
+/* The greedy choice over rows of fp32 logits that are in memory already - the output of ffmoe_gemv_int4_listed for a
+ * drafter's hot vocabulary: out_index[r] = position of the largest finite value of logits[r][0..count), ties to the
+ * lowest position, 0xFFFFFFFF when none is finite; out_conf (may be NULL) as above. The caller maps a position
+ * through its id list. Replaces argmax_rows_f32 as LMHeadChainInt4.encodeHotGreedyRows dispatches it
+ * (LMHeadChainInt4.swift:144-186,209-223). */
+int ffmoe_argmax_rows(ffmoe_ctx *ctx, void *stream, const float *logits, uint32_t stride, uint32_t rows, uint32_t count,
+                      float softcap, uint32_t *out_index, float *out_conf, char **err);
 
 /* ---- dense (shared-expert) FFN ------------------------------------------------------------------ */
 
@@ -411,10 +428,15 @@ int ffmoe_rmsnorm(ffmoe_ctx *ctx, void *stream, const uint16_t *x, uint32_t x_st
  * quantized tensors, per-expert scales and effective scales are bf16 in both (as in the reference's
  * checkpoints). FFMOE_FP16 reproduces the reference's text path: the router reads FP16 rows exactly, the
  * decode / verify kernels multiply FP16 rows with the INT4 weights on the FP16 matrix instruction and
- * round where the reference rounds to FP16 (activations, per-route rows, outputs); the prefill GEMMs
- * keep their bf16 tiles - input rows are rounded to bf16 once, which also makes the reference's
- * power-of-two block scaling (Metal/Prefill/prefill.metal:593-598,685-702, an FP16 range fix)
- * unnecessary - and write FP16 rows. In FFMOE_FP16 input rows must be 16-byte aligned with strides
+ * round where the reference rounds to FP16 (activations, per-route rows, outputs). The prefill GEMMs
+ * (ffmoe_prefill, ffmoe_prefill_pairs, ffmoe_dense_ffn beyond 16 rows) are the exception: in FFMOE_FP16 they
+ * COMPUTE ON BF16-ROUNDED INPUTS - the chunk's FP16 rows are rounded to bf16 once (8 significant bits instead of
+ * FP16's 11), the tiles, the gating product and the activations stay bf16, and only the per-route rows and the
+ * combined rows leave as FP16. That keeps the reference's range (no overflow where its FP16 tiles need the
+ * power-of-two block scaling of Metal/Prefill/prefill.metal:593-598,685-702) and stays inside the 1e-2 /
+ * cosine 0.9999 bar against the FP16 reference, but it is three mantissa bits narrower per input value than the
+ * reference's own FP16 operand in that mode: a caller that needs the reference's FP16 prefill precision bit for
+ * bit does not get it here. In FFMOE_FP16 input rows must be 16-byte aligned with strides
  * that are multiples of 8 wherever a call accepts less otherwise (router, GEMV). Set it before the
  * first compute call; switching waits for the device. May allocate (once). */
 int ffmoe_set_activation_dtype(ffmoe_ctx *ctx, int dtype, char **err);

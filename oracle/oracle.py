@@ -394,6 +394,29 @@ def topk_softmax(logits, top_k: int = 8, per_expert_scale_bits=None):
     return idx, w
 
 
+def greedy_choice_rows(logits, softcap: float = 0.0):
+    """argmax_rows_f32 (Metal/Sampling/logit.metal:946-1010) on rows of fp32 logits [R][V]: per row the position of the
+    largest finite value (ties to the lowest position; 0xFFFFFFFF when no value is finite) and that value's softmax
+    probability over the finite values, each capped to softcap * tanh(v / softcap) when softcap > 0 (:978,1001-1002;
+    0 when there is no winner). The sums run in float64 here; the kernel's float32 order is its own, so probabilities
+    are compared to a tolerance."""
+    logits = np.atleast_2d(np.asarray(logits, np.float32))
+    tokens = np.empty(logits.shape[0], np.uint32)
+    conf = np.zeros(logits.shape[0], np.float64)
+    for r, row in enumerate(logits):
+        finite = np.isfinite(row)
+        if not finite.any():
+            tokens[r] = 0xFFFFFFFF
+            continue
+        best = int(np.flatnonzero(finite & (row == row[finite].max()))[0])
+        tokens[r] = best
+        v = row[finite].astype(np.float64)
+        c = softcap * np.tanh(v / softcap) if softcap > 0 else v
+        cb = softcap * np.tanh(np.float64(row[best]) / softcap) if softcap > 0 else np.float64(row[best])
+        conf[r] = np.exp(cb - c.max()) / np.exp(c - c.max()).sum()
+    return tokens, conf
+
+
 def moe_layer(pool: ExpertPool, router_w_bits, x_bits, top_k: int = 8, dtype: int = BF16, threads: int = 0):
     """Router + top-k + experts + combine in fp32-reference mode. Returns (idx [T][K], w f32 [T][K], y f32 [T][D])."""
     x_bits = np.ascontiguousarray(x_bits, np.uint16)

@@ -159,3 +159,57 @@ def test_matrix_argument_errors(ctx, ff, oracle, torch):
     with pytest.raises(ff.FieldfareError, match="outside 1...16"):
         mx.gemv(torch.zeros((17, 64), dtype=torch.bfloat16, device="cuda"))
     mx.close()
+
+
+@pytest.mark.parametrize("softcap", [0.0, 30.0, 1.5])
+def test_argmax_rows_choice_and_confidence(ctx, oracle, torch, softcap):
+    # argmax_rows_f32 (logit.metal:946-1010): first maximum among the finite values, 0xFFFFFFFF without one; the
+    # winner's probability under the softcap against the float64 restatement (the sums' order is the kernel's own)
+    rng = np.random.default_rng(41)
+    rows = rng.normal(0, 4, (7, 4099)).astype(np.float32)
+    rows[1, 17] = rows[1, 311] = rows[1].max() + 1.0
+    rows[2, :5] = [np.inf, -np.inf, np.nan, 1e30, -1e30]
+    rows[3, :] = np.nan
+    rows[4, :] = -7.25
+    rows[5, 4098] = 99.0                                       # the winner in the last position
+    padded = np.full((7, 4099 + 5), 1e9, np.float32)           # a row stride beyond the count: the padding is not looked at
+    padded[:, :4099] = rows
+    want_tok, want_conf = oracle.greedy_choice_rows(rows, softcap)
+    tok, conf = ctx.argmax_rows(torch.from_numpy(padded).cuda()[:, :4099], softcap=softcap)
+    assert np.array_equal(tok.cpu().numpy().astype(np.uint32), want_tok)
+    assert np.abs(conf.cpu().numpy() - want_conf).max() <= 1e-5 + 1e-4 * want_conf.max()
+    only = ctx.argmax_rows(torch.from_numpy(padded).cuda()[:, :4099], softcap=softcap, want_conf=False)
+    assert np.array_equal(only.cpu().numpy().astype(np.uint32), want_tok)
+
+
+def test_greedy_conf_and_hot_vocabulary_choice(ctx, oracle, torch):
+    # LMHeadChainInt4.encodeGreedyRows with its confidence output, and encodeHotGreedyRows (LMHeadChainInt4.swift:
+    # 94-186): the choice over the listed rows of the head, mapped back through the list, equals the full head's
+    # whenever the list holds the full head's winner; positions follow the list's order
+    m, n, rows = 4099, 2816, 5
+    g = oracle.seed_tree_key(0x1A4E, "head-conf")
+    W, S, B = oracle.quantize_int4(g.uniform(-0.5, 0.5, m * n).reshape(m, n))
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, rows * n)).reshape(rows, n)
+    x = bf16_tensor(torch, xb)
+    Wd, Sd, Bd = torch.from_numpy(W).cuda(), _i16(torch, S), _i16(torch, B)
+    head = ctx.matrix(Wd, Sd, Bd, greedy=True)
+    logits = head.gemv(x, f32_out=True).cpu().numpy()
+    plain = head.greedy(x).cpu().numpy()
+    for cap in (0.0, 30.0):
+        tok, conf = head.greedy_conf(x, softcap=cap)
+        want_tok, want_conf = oracle.greedy_choice_rows(logits, cap)
+        assert np.array_equal(tok.cpu().numpy().astype(np.uint32), want_tok) and np.array_equal(tok.cpu().numpy(), plain)
+        assert np.abs(conf.cpu().numpy() - want_conf).max() <= 1e-5 + 1e-4 * want_conf.max()
+    # hot vocabulary: 512 listed rows in a shuffled order that hold every row's winner
+    rng = np.random.default_rng(5)
+    ids = np.unique(np.concatenate([plain.astype(np.int64), rng.choice(m, 512, replace=False)]))
+    rng.shuffle(ids)
+    ids_d = torch.from_numpy(ids.astype(np.int32)).cuda()
+    listed = ctx.gemv_int4_listed(Wd, Sd, Bd, ids_d, x)
+    pos, conf = ctx.argmax_rows(listed)
+    pos = pos.cpu().numpy()
+    assert np.array_equal(ids[pos], plain)
+    want_pos, want_conf = oracle.greedy_choice_rows(listed.cpu().numpy(), 0.0)
+    assert np.array_equal(pos.astype(np.uint32), want_pos)
+    assert np.abs(conf.cpu().numpy() - want_conf).max() <= 1e-5 + 1e-4 * want_conf.max()
+    head.close()

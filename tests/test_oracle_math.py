@@ -442,3 +442,31 @@ def test_layer_tail_invariants(oracle):
     blk = oracle.layer_tail(np.stack([h2, h1]), np.stack([h1, h2]), np.stack([hidden, hidden]), w2, w1, 0.9, eps)
     assert np.array_equal(blk[0], oracle.layer_tail(h2, h1, hidden, w2, w1, 0.9, eps)[0])
     assert np.array_equal(blk[1], oracle.layer_tail(h1, h2, hidden, w2, w1, 0.9, eps)[0])
+
+
+def test_greedy_choice_rows_against_closed_forms(oracle):
+    # the choice: first maximum among the finite values; the confidence: scipy's softmax of the (capped) finite values
+    from scipy.special import softmax
+    rng = np.random.default_rng(31)
+    rows = rng.normal(0, 4, (6, 513)).astype(np.float32)
+    rows[1, 17] = rows[1, 311] = rows[1].max() + 1.0           # a tie: the lower position wins (LMHeadChainInt4Tests.swift:100-116)
+    rows[2, :5] = [np.inf, -np.inf, np.nan, 1e30, -1e30]        # non-finite values never win and carry no probability
+    rows[3, :] = np.nan                                        # no candidate at all
+    rows[4, :] = -7.25                                         # all equal: position 0, probability 1 / V
+    for cap in (0.0, 30.0, 2.0):
+        tok, conf = oracle.greedy_choice_rows(rows, cap)
+        for r in range(6):
+            finite = np.isfinite(rows[r])
+            if not finite.any():
+                assert tok[r] == 0xFFFFFFFF and conf[r] == 0.0
+                continue
+            want = int(np.argmax(np.where(finite, rows[r], -np.inf)))      # numpy's argmax returns the first maximum
+            assert tok[r] == want
+            v = rows[r][finite].astype(np.float64)
+            p = softmax(cap * np.tanh(v / cap) if cap > 0 else v)
+            assert abs(conf[r] - p[np.flatnonzero(finite).tolist().index(want)]) <= 1e-12
+        assert tok[1] == 17 and tok[4] == 0 and abs(conf[4] - 1 / 513) < 1e-12
+    # a cap far below the spread flattens the distribution: the winner's probability falls towards 1 / V
+    _, c0 = oracle.greedy_choice_rows(rows[:1], 0.0)
+    _, c2 = oracle.greedy_choice_rows(rows[:1], 0.5)
+    assert c2[0] < c0[0]
