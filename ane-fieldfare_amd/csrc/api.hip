@@ -566,7 +566,7 @@ int ffmoe_handover_giveups(ffmoe_ctx *ctx, void *stream, uint32_t *count, char *
 
 static int prefill_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride, uint32_t t,
                           const uint32_t *idx, const uint16_t *w, const ffmoe_pair *pairs, uint32_t n_pairs, uint16_t *y,
-                          uint16_t *partials, char **err) {
+                          uint16_t *partials, char **err, bool dense = false) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (int rc = check_layer(ctx, layer, true, false, err)) return rc;
     if (!x) return fail(err, FFMOE_ERR_INVALID, "null argument");
@@ -581,7 +581,7 @@ static int prefill_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const ui
         return fail(err, FFMOE_ERR_INVALID, "outputs must be 16-byte aligned");
     FF_HIP(launch_prefill(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                           ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, pairs, n_pairs, y, partials,
-                          ctx->pf, &ctx->timer, ctx->f16));
+                          ctx->pf, &ctx->timer, ctx->f16, dense));
     return FFMOE_OK;
 }
 
@@ -624,7 +624,7 @@ int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t
     if (t <= FFMOE_MAX_VERIFY_ROWS)
         return verify_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, nullptr, y, err, nullptr,
                              nullptr, true);
-    return prefill_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, 0, nullptr, y, err);
+    return prefill_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, 0, nullptr, y, err, true);
 }
 
 int ffmoe_prefill_plan_stats(ffmoe_ctx *ctx, void *stream, uint32_t *n_pairs, uint32_t *n_tiles, uint32_t *counts,

@@ -188,7 +188,7 @@ hipError_t launch_argmax_rows(hipStream_t s, const float *logits, uint32_t strid
 hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
                           const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
                           const ffmoe_pair *pairs, uint32_t n_pairs_in, uint16_t *y, uint16_t *partials_out,
-                          PrefillScratch sc, KernelTimer *timer, bool f16 = false);
+                          PrefillScratch sc, KernelTimer *timer, bool f16 = false, bool dense = false);
 
 // Test hook: the weight fragments of one expert's gate/up (or down) tiles as the grouped GEMM's matrix instructions
 // read them from LDS: [N-block][group][fragment 0..15][lane] x 16 bytes, `prefill_dump_fragments` fragments in all.

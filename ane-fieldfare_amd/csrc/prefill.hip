@@ -214,6 +214,35 @@ __global__ __launch_bounds__(kSortBlock) void prefill_scatter_kernel(ItemSource 
     sorted_out_row[pos] = out_row;
 }
 
+// A dense FFN's chunk needs no sort: one expert, route r = row r. One launch writes what the three above would: the
+// identity tables and the chunk cut into M-tiles.
+__global__ __launch_bounds__(kSortBlock) void prefill_dense_plan_kernel(uint32_t t, PrefillPlan *__restrict__ plan,
+                                                                       PrefillTile *__restrict__ tiles,
+                                                                       uint32_t *__restrict__ sorted_token,
+                                                                       uint32_t *__restrict__ sorted_out_row) {
+    const uint32_t i = blockIdx.x * kSortBlock + threadIdx.x;
+    if (i < t) {
+        sorted_token[i] = i;
+        sorted_out_row[i] = i;
+    }
+    const uint32_t n_tiles = (t + kBM - 1) / kBM;
+    if (i < n_tiles) {
+        PrefillTile tl;
+        tl.expert = 0;
+        tl.row_start = i * kBM;
+        tl.rows = min((uint32_t)kBM, t - i * kBM);
+        tl.pad = 0;
+        tiles[i] = tl;
+    }
+    if (i == 0) {
+        plan->n_pairs = t;
+        plan->n_tiles = n_tiles;
+        plan->expert_count[0] = t;
+        plan->expert_offset[0] = 0;
+        plan->expert_offset[1] = t;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Grouped GEMM. One block = one M-tile (up to 256 pairs of one expert) x one N-block (4 arena tiles =
 // 128 weight rows); block ids are laid out so that all N-blocks of an M-tile run on one XCD and find the
@@ -668,7 +697,9 @@ hipError_t launch_prefill_dump_tiles(hipStream_t s, const uint8_t *arena_layer, 
 hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
                           const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
                           const ffmoe_pair *pairs, uint32_t n_pairs_in, uint16_t *y, uint16_t *partials_out,
-                          PrefillScratch sc, KernelTimer *timer, bool f16) {
+                          PrefillScratch sc, KernelTimer *timer, bool f16, bool dense) {
+    // dense: the caller vouches for a dense FFN's chunk - one expert, top_k = 1, every row routed to it at weight 1
+    dense = dense && n_experts == 1 && top_k == 1 && !pairs && !y;
     timer->begin(s);
     ItemSource src{};
     src.idx = pairs ? nullptr : idx;
@@ -680,13 +711,18 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
     src.t = t;
     if (src.n_items == 0) return hipSuccess;
     const uint32_t n_blocks = (src.n_items + kSortBlock - 1) / kSortBlock;
-    hipLaunchKernelGGL(prefill_hist_kernel, dim3(n_blocks), dim3(kSortBlock), 0, s, src, sc.block_cnt);
-    uint32_t e_pad = 1;
-    while (e_pad < n_experts) e_pad <<= 1;          // n_experts <= FFMOE_MAX_EXPERTS = 256 <= kScanThreads
-    hipLaunchKernelGGL(prefill_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, n_blocks, n_experts, e_pad, sc.block_cnt, sc.plan,
-                       sc.tiles, sc.max_tiles);
-    hipLaunchKernelGGL(prefill_scatter_kernel, dim3(n_blocks), dim3(kSortBlock), 0, s, src, sc.block_cnt, sc.sorted_token,
-                       sc.sorted_out_row);
+    if (dense) {
+        hipLaunchKernelGGL(prefill_dense_plan_kernel, dim3(n_blocks), dim3(kSortBlock), 0, s, t, sc.plan, sc.tiles, sc.sorted_token,
+                           sc.sorted_out_row);
+    } else {
+        hipLaunchKernelGGL(prefill_hist_kernel, dim3(n_blocks), dim3(kSortBlock), 0, s, src, sc.block_cnt);
+        uint32_t e_pad = 1;
+        while (e_pad < n_experts) e_pad <<= 1;          // n_experts <= FFMOE_MAX_EXPERTS = 256 <= kScanThreads
+        hipLaunchKernelGGL(prefill_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, n_blocks, n_experts, e_pad, sc.block_cnt,
+                           sc.plan, sc.tiles, sc.max_tiles);
+        hipLaunchKernelGGL(prefill_scatter_kernel, dim3(n_blocks), dim3(kSortBlock), 0, s, src, sc.block_cnt, sc.sorted_token,
+                           sc.sorted_out_row);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_PREFILL_SORT);
