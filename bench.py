@@ -121,6 +121,9 @@ def main():
     ap.add_argument("--no-sweep", action="store_true",
                     help="skip BASELINE.json config 5 (8,192-token Zipf prefill over all layers, then 256 decode steps "
                          "as 16 verify blocks with the LM head once per block)")
+    ap.add_argument("--no-zipf", action="store_true",
+                    help="skip the Zipf(1.1) half of the prefill leg (so that a profiler's per-kernel averages of the prefill "
+                         "kernels cover the router-made, near-uniform routes alone)")
     ap.add_argument("--sweep", action="store_true", help="accepted for older command lines: the sweep runs by default")
     args = ap.parse_args()
     args.sweep = not args.no_sweep and not args.no_gemv
@@ -134,8 +137,13 @@ def main():
     from fieldfare_moe import synthetic as syn
     ff.ensure_built()                     # loads what is built in-tree; compiles only if nothing (current) is
     oracle = None
+    cpu_flags = "gcc -O3 -march=x86-64-v3 -ffp-contract=off -fno-fast-math -fopenmp (the in-tree build)"
     if not args.no_cpu:                   # the CPU oracle is the checker and the cpu_baseline leg, nothing else here
         from oracle import oracle
+        import tempfile
+        native = oracle.use_native_build(tempfile.mkdtemp(prefix="ffmoe_oracle_"))      # this host's own instruction set
+        if native:
+            cpu_flags = "gcc " + native + " (compiled on this host for the baseline)"
 
     assert torch.cuda.is_available(), "bench.py needs a HIP device"
     torch.cuda.set_device(0)
@@ -436,36 +444,41 @@ def main():
             e1.record()
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) * 1e-3 / 20
-        t_dgu, t_ddn = dense_time(a_gu, b_gu, o_gu), dense_time(a_dn, b_dn, o_dn)
+        # both operand layouts of the weight ([K x N] and the transposed view of [N x K]); the faster one counts
+        bt_gu, bt_dn = b_gu.t().contiguous(), b_dn.t().contiguous()
+        t_dgu = min(dense_time(a_gu, b_gu, o_gu), dense_time(a_gu, bt_gu.t(), o_gu))
+        t_ddn = min(dense_time(a_dn, b_dn, o_dn), dense_time(a_dn, bt_dn.t(), o_dn))
+        del bt_gu, bt_dn
         dense_tf = (flops_gu + flops_dn) / (t_dgu + t_ddn) / 1e12
         prefill["dense_bf16_ceiling_TFLOPs"] = round(dense_tf, 1)
         prefill["dense_bf16_ceiling"] = {
             "gate_up_us": round(t_dgu * 1e6, 1), "down_us": round(t_ddn * 1e6, 1),
-            "shapes": f"[{mrows} x {D}] . [{D} x {2 * F}] and [{mrows} x {F}] . [{F} x {D}], bf16, torch.matmul",
+            "shapes": f"[{mrows} x {D}] . [{D} x {2 * F}] and [{mrows} x {F}] . [{F} x {D}], bf16, torch.matmul, the faster of the weight as [K x N] and as [N x K] transposed",
             "frac_mfma_peak": round(dense_tf / MFMA_BF16_PEAK_TFLOPS, 4),
             "gemm_frac_of_dense_ceiling": round((flops_gu + flops_dn) / gemm_s / 1e12 / dense_tf, 4)}
         del a_gu, b_gu, a_dn, b_dn, o_gu, o_dn
         # BASELINE.json config 4 (ii): the same chunk with Zipf(1.1) routing imposed on the experts
         # (indices and weights given, no router): a few experts hold most pairs, many hold a handful
-        zidx_, zw_ = syn.zipf_routes(np.random.default_rng(4), TP)
-        pidx_t.copy_(torch.from_numpy(zidx_))
-        pw_t.copy_(torch.from_numpy(syn.bf16_bits(zw_).view(np.int16)).view(torch.bfloat16))
+        if not args.no_zipf:
+            zidx_, zw_ = syn.zipf_routes(np.random.default_rng(4), TP)
+            pidx_t.copy_(torch.from_numpy(zidx_))
+            pw_t.copy_(torch.from_numpy(syn.bf16_bits(zw_).view(np.int16)).view(torch.bfloat16))
 
-        def zstep(layer):
-            if Lib.ffmoe_prefill(h, stream, layer, pxp, D, TP, ppi, ppw, ppy, C.byref(err)):
-                raise RuntimeError(err.value)
-        for i in range(4):
-            zstep(i % L)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(psteps):
-            zstep(i % L)
-        torch.cuda.synchronize()
-        zel = (time.perf_counter() - t0) / psteps
-        _, z_tiles, zcounts = ctx.prefill_stats()
-        prefill["zipf_1p1"] = {"tok_per_s": round(TP / zel, 1), "ms_per_layer": round(zel * 1e3, 4), "m_tiles": z_tiles,
-                               "pairs_per_expert_min": int(zcounts.min()), "pairs_per_expert_max": int(zcounts.max()),
-                               "pairs_per_expert_median": int(np.median(zcounts)), "router": "not run (routes imposed)"}
+            def zstep(layer):
+                if Lib.ffmoe_prefill(h, stream, layer, pxp, D, TP, ppi, ppw, ppy, C.byref(err)):
+                    raise RuntimeError(err.value)
+            for i in range(4):
+                zstep(i % L)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(psteps):
+                zstep(i % L)
+            torch.cuda.synchronize()
+            zel = (time.perf_counter() - t0) / psteps
+            _, z_tiles, zcounts = ctx.prefill_stats()
+            prefill["zipf_1p1"] = {"tok_per_s": round(TP / zel, 1), "ms_per_layer": round(zel * 1e3, 4), "m_tiles": z_tiles,
+                                   "pairs_per_expert_min": int(zcounts.min()), "pairs_per_expert_max": int(zcounts.max()),
+                                   "pairs_per_expert_median": int(np.median(zcounts)), "router": "not run (routes imposed)"}
 
     def timed(fn, reps, warm=3):
         for _ in range(warm):
@@ -534,6 +547,7 @@ def main():
     # INT4 GEMV: BASELINE.json config 1 ([1408 x 2816], one input row) and the LM head of config 5
     # ([262144 x 2816]) as resident matrices; synthetic weights as in synth_layer_gpu
     head = None
+    head_sample = None
     if not args.no_gemv:
         def synth_matrix(m):
             return syn.synth_matrix_gpu(torch, gen, m)
@@ -563,6 +577,9 @@ def main():
         m1.close()
         V = 262144
         Wh, Sh, Bh = synth_matrix(V)
+        if not args.no_cpu:             # the first 16,384 rows on the host, for the CPU baseline's head leg
+            head_sample = (Wh[:16384].cpu().numpy(), Sh[:16384].view(torch.int16).cpu().numpy().view(np.uint16),
+                           Bh[:16384].view(torch.int16).cpu().numpy().view(np.uint16))
         head = ctx.matrix(Wh, Sh, Bh, greedy=True)
         del Wh, Sh, Bh
         torch.cuda.empty_cache()
@@ -822,9 +839,25 @@ def main():
             legs["config4_prefill"] = {"sample_tokens": n_s, "sample_ms": round(ps * 1e3, 1), f"tok_per_s_{threads}_threads": round(n_s / ps, 1),
                                        "ms_per_layer_extrapolated": round(ps / n_s * prefill["tokens"] * 1e3, 1),
                                        "note": f"first {n_s} of the chunk's {prefill['tokens']} tokens; time scales with the token count"}
+        # config 5: the LM head GEMV [262144 x 2816] (dequantise the row, then dot), on a sample of its rows split over
+        # the threads, extrapolated to the whole head (the rows are independent)
+        if head_sample is not None:
+            Wq, Sq, Bq = head_sample
+            xh = oracle.bf16_to_float(xb[0])
+            cuts_h = np.linspace(0, Wq.shape[0], threads + 1).astype(int)
+            with ThreadPoolExecutor(threads) as ex:
+                def split_head():
+                    list(ex.map(lambda i: oracle.gemv_int4_ref(Wq[cuts_h[i]:cuts_h[i + 1]], Sq[cuts_h[i]:cuts_h[i + 1]],
+                                                               Bq[cuts_h[i]:cuts_h[i + 1]], xh), range(threads)))
+                hm, _ = best_of(split_head, 1.0, 2)
+            hb = Wq.size + 2 * Sq.size * 2
+            legs["config5_lm_head_262144x2816"] = {
+                "sample_rows": int(Wq.shape[0]), "sample_ms": round(hm * 1e3, 2), f"GBs_{threads}_threads": round(hb / hm / 1e9, 3),
+                "ms_per_row_of_x_extrapolated": round(hm * 262144 / Wq.shape[0] * 1e3, 1),
+                "note": f"first {Wq.shape[0]} of the head's 262,144 rows, one input row; time scales with the row count"}
         cpu = {"value": round(cpu_bytes / multi / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
                "nproc": nproc, "cpu_model": cpu_model, "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS"),
-               "compiler": "gcc -O3 -march=x86-64-v3 -ffp-contract=off -fopenmp",
+               "compiler": cpu_flags,
                "sample": f"config 3: layer 0 of the same 16-token block, best of {reps} reps on {threads} threads "
                          f"({multi * 1e3:.1f} ms); 1 thread: {single * 1e3:.0f} ms = {cpu_bytes / single / 1e9:.3f} GB/s; "
                          f"C restatement of the reference's Swift CPU dequant+matmul path; the other configurations' samples are in legs",

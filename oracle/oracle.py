@@ -22,12 +22,31 @@ BF16, FP16, F32 = 0, 1, 2
 GROUP = 64
 
 
+NATIVE_FLAGS = "-O3 -march=native -ffp-contract=off -fno-fast-math -fopenmp -fPIC -std=c11"
+
+
 def build(force: bool = False) -> Path:
     """Compile the C oracle with the Makefile beside it."""
     if force or not _LIB_PATH.exists():
         subprocess.run(["make", "-C", str(_DIR), "-B", "libffmoe_oracle.so"], check=True,
                        stdout=subprocess.DEVNULL)
     return _LIB_PATH
+
+
+def use_native_build(out_dir) -> str | None:
+    """For the CPU baseline on the machine that runs it: compile the same source with -march=native into `out_dir`
+    and make it the library this module calls (the in-tree build targets x86-64-v3 so that one file runs on every
+    host it is carried to). Returns the flags used, or None when no compiler is there and the in-tree build stays.
+    Same arithmetic either way: contraction and fast-math stay off."""
+    global _lib, _LIB_PATH
+    out = Path(out_dir) / "libffmoe_oracle_native.so"
+    try:
+        subprocess.run(["gcc", *NATIVE_FLAGS.split(), "-shared", "-o", str(out), str(_DIR / "ffmoe_oracle.c"), "-lm"],
+                       check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=120)
+    except (OSError, subprocess.SubprocessError):
+        return None
+    _LIB_PATH, _lib = out, None
+    return NATIVE_FLAGS
 
 
 class Offsets(C.Structure):
