@@ -188,7 +188,9 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
         e = hipMemcpy(&ctx->mail->epoch, &first_epoch, sizeof first_epoch, hipMemcpyHostToDevice);
     }
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->acts), routes * shape->f * sizeof(uint16_t));
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->partials), routes * shape->d * sizeof(float));
+    // the un-weighted fp32 rows; a dense expert whose K exceeds a wave's ring leaves one set per chunk of K when it rides
+    // along in another context's launches (ffmoe_route_verify_shared)
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->partials), routes * shape->d * sizeof(float) * std::max(1u, shared_chunks(ctx->geom)));
     // prefill scratch: sort tables, pair lists, activations and per-route rows for max_tokens tokens
     ctx->max_pairs = (shape->max_tokens > FFMOE_MAX_VERIFY_ROWS ? shape->max_tokens : FFMOE_MAX_VERIFY_ROWS) * shape->top_k;
     const size_t sort_blocks = (ctx->max_pairs + 255) / 256;
@@ -453,7 +455,7 @@ struct VerifyScratch {
 static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
                          uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual, uint16_t *y,
                          uint16_t *partials_bf16, char **err, const VerifyScratch *use = nullptr,
-                         const RouteFusion *route = nullptr, bool dense = false) {
+                         const RouteFusion *route = nullptr, bool dense = false, const SharedExpert *shared = nullptr) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (int rc = check_layer(ctx, layer, true, route != nullptr, err)) return rc;
     if (!x || !idx || !w || (!y && !partials_bf16 && !route)) return fail(err, FFMOE_ERR_INVALID, "null argument");
@@ -466,7 +468,7 @@ static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uin
     const VerifyScratch &sc = use ? *use : own;
     FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                         sc.plan, sc.acts, sc.partials, ctx->n_cus, &ctx->timer, ctx->f16, route, dense));
+                         sc.plan, sc.acts, sc.partials, ctx->n_cus, &ctx->timer, ctx->f16, route, dense, shared));
     return FFMOE_OK;
 }
 
@@ -512,6 +514,41 @@ int ffmoe_route_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint1
                             router_x_stride, ctx->logits, ctx->mail, ctx->handover_ticks, ctx->one_launch_routing,
                             ctx->route_resident_blocks};
     return verify_common(ctx, stream, layer, x, x_stride, t, out_idx, out_w, residual, y, nullptr, err, nullptr, &route);
+}
+
+int ffmoe_route_verify_shared(ffmoe_ctx *ctx, ffmoe_ctx *shared, void *stream, uint32_t layer, uint32_t shared_layer,
+                              const uint16_t *router_x, uint32_t router_x_stride, const uint16_t *x, uint32_t x_stride,
+                              const uint16_t *shared_x, uint32_t shared_x_stride, uint32_t t, uint32_t *out_idx,
+                              uint16_t *out_w, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_ctx(shared, err)) return rc;
+    if (!router_x || !out_idx || !out_w || !shared_x) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (!shared->dense_idx)
+        return fail(err, FFMOE_ERR_INVALID, "the shared expert needs a context with n_experts = 1 and top_k = 1");
+    if (shared == ctx) return fail(err, FFMOE_ERR_INVALID, "the shared expert lives in a context of its own");
+    if (shared->device != ctx->device || shared->f16 != ctx->f16)
+        return fail(err, FFMOE_ERR_INVALID, "the two contexts must share the device and the activation type");
+    if (int rc = check_layer(shared, shared_layer, true, false, err)) return rc;
+    const ArenaGeom &sg = shared->geom;
+    if (sg.d != ctx->geom.d || ctx->geom.gf > kSharedChunkGroups || (ctx->geom.gd + 3) / 4 > kSharedChunkGroups ||
+        shared_chunks(sg) > 4 || ctx->shape.top_k > 8)
+        return fail(err, FFMOE_ERR_INVALID,
+                    "the shared expert rides along when both have the same d <= 2816 and the routed experts' f <= 704 "
+                    "(run ffmoe_dense_ffn and ffmoe_route_verify otherwise)");
+    if (shared_x_stride < sg.d || shared_x_stride % 8 || reinterpret_cast<uintptr_t>(shared_x) % 16)
+        return fail(err, FFMOE_ERR_INVALID, "shared_x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
+    if (router_x_stride < ctx->shape.d) return fail(err, FFMOE_ERR_INVALID, "hidden stride is too small");
+    if (ctx->f16 && (reinterpret_cast<uintptr_t>(router_x) % 8 || router_x_stride % 4))
+        return fail(err, FFMOE_ERR_INVALID, "FP16 router rows must be 8-byte aligned with a stride that is a multiple of 4");
+    if (layer >= ctx->layers.size()) return fail(err, FFMOE_ERR_INVALID, "layer %u out of range", layer);
+    const ffmoe_layer &l = ctx->layers[layer];
+    const RouteFusion route{RouterWeights{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale}, router_x,
+                            router_x_stride, ctx->logits, ctx->mail, ctx->handover_ticks, ctx->one_launch_routing,
+                            ctx->route_resident_blocks};
+    const SharedExpert sh{shared->arena + (size_t)shared_layer * shared->layer_bytes, sg, shared_x, shared_x_stride, shared->acts,
+                          shared->partials};
+    return verify_common(ctx, stream, layer, x, x_stride, t, out_idx, out_w, nullptr, nullptr, nullptr, err, nullptr, &route,
+                         false, &sh);
 }
 
 int ffmoe_set_handover_timeout(ffmoe_ctx *ctx, void *stream, uint64_t ticks, char **err) {
@@ -686,6 +723,23 @@ int ffmoe_layer_tail_routed(ffmoe_ctx *ctx, void *stream, const uint16_t *route_
     FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), nullptr, 0, h1, h1_stride, hidden, hidden_stride, w_postffn2,
                              w_postffn, t, ctx->shape.d, eps, layer_scalar, nullptr, nullptr, nullptr, 0, ctx->f16, ctx->partials,
                              route_w, ctx->plan->route_valid, ctx->shape.top_k));
+    return FFMOE_OK;
+}
+
+int ffmoe_layer_tail_routed_shared(ffmoe_ctx *ctx, ffmoe_ctx *shared, void *stream, const uint16_t *route_w, uint16_t *hidden,
+                                   uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn, uint32_t t,
+                                   float eps, float layer_scalar, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_ctx(shared, err)) return rc;
+    if (!route_w || !hidden || !w_postffn2 || !w_postffn) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (!shared->dense_idx || shared == ctx || shared->geom.d != ctx->geom.d || shared->f16 != ctx->f16)
+        return fail(err, FFMOE_ERR_INVALID, "the shared expert's context does not match (one expert, top_k = 1, same d and type)");
+    if (t == 0 || t > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%d", t, FFMOE_MAX_VERIFY_ROWS);
+    const uint32_t strides[1] = {hidden_stride};
+    if (int rc = check_rows(t, ctx->shape.d, strides, 1, err)) return rc;
+    FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), nullptr, 0, nullptr, 0, hidden, hidden_stride, w_postffn2,
+                             w_postffn, t, ctx->shape.d, eps, layer_scalar, nullptr, nullptr, nullptr, 0, ctx->f16, ctx->partials,
+                             route_w, ctx->plan->route_valid, ctx->shape.top_k, shared->partials, shared_chunks(shared->geom)));
     return FFMOE_OK;
 }
 

@@ -141,7 +141,39 @@ struct RoutedRows {
     const uint16_t *w;               // [t][top_k]
     const uint32_t *route_valid;     // [t * top_k]
     uint32_t top_k;
+    // h1 likewise, when the shared expert's down projection rode along in the routed experts' launch and left its K in
+    // chunks: h1 = the chunks' fp32 rows added in chunk order, one rounding to 16 bits (what the dense FFN's own down
+    // launch rounds once too). Null: h1 is read as a 16-bit row.
+    const float *shared_partials;    // [shared_chunks][t][d]
+    uint32_t shared_chunks, t;
 };
+
+template <bool F16>
+__device__ __forceinline__ Row8 shared_row8(const RoutedRows &rr, uint32_t row, uint32_t d, uint32_t chunk) {
+    Row8 out;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out.v[i] = 0.0f;
+    f32x4 lo[4], hi[4];
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        const float *src = rr.shared_partials + ((size_t)min(c, rr.shared_chunks - 1) * rr.t + row) * d + 8 * chunk;
+        lo[c] = *reinterpret_cast<const f32x4 *>(src);
+        hi[c] = *reinterpret_cast<const f32x4 *>(src + 4);
+    }
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        if (c < rr.shared_chunks) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                out.v[i] += lo[c][i];
+                out.v[4 + i] += hi[c][i];
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out.v[i] = round16<F16>(out.v[i]);
+    return out;
+}
 
 template <bool F16>
 __device__ __forceinline__ Row8 combine8(const RoutedRows &rr, uint32_t row, uint32_t d, uint32_t chunk) {
@@ -199,7 +231,7 @@ __global__ __launch_bounds__(kRowThreads) void layer_tail_kernel(const uint16_t 
         if ((uint32_t)c < n_mine) {
             const uint32_t chunk = t + c * kRowThreads;
             if (!COMBINE) a[c] = load8<VEC, F16>(h2 + (size_t)row * h2_stride, chunk);
-            h12[c] = load8<VEC, F16>(h1 + (size_t)row * h1_stride, chunk);
+            if (!COMBINE || !routed.shared_partials) h12[c] = load8<VEC, F16>(h1 + (size_t)row * h1_stride, chunk);
             hv[c] = load8<VEC, F16>(hrow, chunk);
             wf2[c] = loadw8<VEC>(w_postffn2, chunk);
             wf[c] = loadw8<VEC>(w_postffn, chunk);
@@ -209,7 +241,10 @@ __global__ __launch_bounds__(kRowThreads) void layer_tail_kernel(const uint16_t 
     if (COMBINE) {
 #pragma unroll
         for (int c = 0; c < kMaxChunks; ++c)
-            if ((uint32_t)c < n_mine) a[c] = combine8<F16>(routed, row, d, t + c * kRowThreads);
+            if ((uint32_t)c < n_mine) {
+                a[c] = combine8<F16>(routed, row, d, t + c * kRowThreads);
+                if (routed.shared_partials) h12[c] = shared_row8<F16>(routed, row, d, t + c * kRowThreads);
+            }
     }
     if (NORMS) {
         const float inv_h1 = block_rms_inv(h12, n_mine, d, eps, s_sum[2]);
@@ -307,12 +342,14 @@ hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stri
                              uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
                              uint32_t t, uint32_t d, float eps, float layer_scalar, const uint16_t *w_postffn1,
                              const uint16_t *w_next, uint16_t *normed, uint32_t normed_stride, bool f16,
-                             const float *routed_partials, const uint16_t *routed_w, const uint32_t *route_valid, uint32_t top_k) {
+                             const float *routed_partials, const uint16_t *routed_w, const uint32_t *route_valid, uint32_t top_k,
+                             const float *shared_partials, uint32_t shared_chunks) {
     const bool norms = w_postffn1 != nullptr;
-    const RoutedRows routed{routed_partials, routed_w, route_valid, top_k};
+    if (shared_partials && (!routed_partials || shared_chunks == 0 || shared_chunks > 4)) return hipErrorInvalidValue;
+    const RoutedRows routed{routed_partials, routed_w, route_valid, top_k, shared_partials, shared_chunks, t};
     if (routed_partials) {
         // h2 is made from the un-combined rows (16-byte aligned fp32 rows: d % 8 == 0); the plain tail only
-        const bool vec = aligned16(h1, h1_stride) && aligned16(hidden, hidden_stride) && aligned16(w_postffn2, 8) && aligned16(w_postffn, 8);
+        const bool vec = (shared_partials || aligned16(h1, h1_stride)) && aligned16(hidden, hidden_stride) && aligned16(w_postffn2, 8) && aligned16(w_postffn, 8);
 #define FFMOE_TAILC(V, H)                                                                                             \
     hipLaunchKernelGGL((layer_tail_kernel<V, false, H, true>), dim3(t), dim3(kRowThreads), 0, s, nullptr, 0u, h1, h1_stride, \
                        hidden, hidden_stride, w_postffn2, w_postffn, d, eps, layer_scalar, nullptr, nullptr, nullptr, 0u, routed)

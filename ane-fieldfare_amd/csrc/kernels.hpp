@@ -137,6 +137,22 @@ struct RouteFusion {
     uint32_t resident_blocks;           // blocks of the one-launch form the GPU holds at once (0: unknown, use the launches)
 };
 
+// The shared expert of the same MoE block (a dense FFN with its own input rows; SharedExpertInt4.swift:23-89), served by
+// blocks of the routed experts' launches instead of launches of its own (ffmoe_route_verify_shared): some blocks of the
+// gate/up launch walk its gate/up row blocks - they need no routes and start while the others wait for theirs -, and
+// the down launch takes its K = f in chunks of kRing groups, one extra "expert" per chunk, whose un-weighted fp32 rows
+// the layer tail adds up.
+struct SharedExpert {
+    const uint8_t *arena_layer;     // the one expert of the dense context's layer
+    ArenaGeom g;                    // d as the routed experts'; f = 64 * gf
+    const uint16_t *x;              // [t][x_stride]
+    uint32_t x_stride;
+    uint16_t *acts;                 // [t][g.f]
+    float *partials;                // [chunks][t][g.d], chunk c = groups [kRing c, kRing c + kRing) of K
+};
+constexpr uint32_t kSharedChunkGroups = 11;      // = kRing of the streaming kernels
+inline uint32_t shared_chunks(const ArenaGeom &g) { return (g.gf + kSharedChunkGroups - 1) / kSharedChunkGroups; }
+
 // repack.hip
 hipError_t launch_repack_layer(hipStream_t s, const uint8_t *blobs, size_t stride, ffmoe_offsets off,
                                uint32_t n_experts, ArenaGeom g, uint8_t *arena_layer);
@@ -156,7 +172,8 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
                          VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer,
-                         bool f16 = false, const RouteFusion *route = nullptr, bool dense = false);
+                         bool f16 = false, const RouteFusion *route = nullptr, bool dense = false,
+                         const SharedExpert *shared = nullptr);
 uint32_t route_launch_resident_blocks(uint32_t n_cus);
 // the two expert kernels' weight loads for n_live experts and nothing else (`sink`: 256 words nobody reads)
 hipError_t launch_probe_stream(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t n_live,
@@ -209,7 +226,8 @@ hipError_t launch_layer_tail(hipStream_t s, const uint16_t *h2, uint32_t h2_stri
                              uint32_t t, uint32_t d, float eps, float layer_scalar, const uint16_t *w_postffn1 = nullptr,
                              const uint16_t *w_next = nullptr, uint16_t *normed = nullptr, uint32_t normed_stride = 0,
                              bool f16 = false, const float *routed_partials = nullptr, const uint16_t *routed_w = nullptr,
-                             const uint32_t *route_valid = nullptr, uint32_t top_k = 0);
+                             const uint32_t *route_valid = nullptr, uint32_t top_k = 0, const float *shared_partials = nullptr,
+                             uint32_t shared_chunks = 0);
 hipError_t launch_rmsnorm(hipStream_t s, const uint16_t *x, uint32_t x_stride, const uint16_t *w, uint16_t *out,
                           uint32_t out_stride, uint32_t t, uint32_t d, float eps, bool f16 = false);
 

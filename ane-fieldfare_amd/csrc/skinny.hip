@@ -309,13 +309,13 @@ __device__ __forceinline__ void prepare_token_rows(uint32_t lane, uint4 (&x0)[kR
 // its expert's row blocks, the weight stream. x0 / x1: the wave's token rows as load_token_rows() left them.
 // DENSE: the one expert of a dense FFN takes every row at weight 1 (route r = row r): nothing to plan, the first
 // weight request goes out with the kernel's first instructions, and block 0 writes the plan the down kernel's
-// general forms and ffmoe_last_live_experts read without any block waiting for it.
+// general forms and ffmoe_last_live_experts read without any block waiting for it (no plan given: none written).
 template <bool F16, bool DENSE = false>
 __device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps, const uint8_t *__restrict__ arena_layer,
                                              const ArenaGeom &g, uint32_t top_k, uint32_t n_experts, uint32_t route_idx,
                                              uint16_t route_w, uint32_t n_routes, VerifyPlan *__restrict__ plan,
                                              const KSlice &k, uint4 (&x0)[kRing], uint4 (&x1)[kRing], f32x4 (&sx)[kRing],
-                                             bool prepared, uint16_t *__restrict__ acts) {
+                                             bool prepared, uint16_t *__restrict__ acts, uint32_t bid, uint32_t n_blocks) {
     const uint32_t rows = n_routes / top_k;
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15, jq = lane >> 4;
@@ -323,7 +323,7 @@ __device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps
     // Every block derives the routing plan itself from the (at most 128) routes: a few dozen LDS
     // operations, against a separate launch plus two dependent global reads per block. Block 0 also
     // writes the plan out for the down kernel.
-    const uint32_t gu_rb = g.gu_rb, n_blocks = gridDim.x, bid = blockIdx.x;
+    const uint32_t gu_rb = g.gu_rb;       // bid of n_blocks: this block among those that share the work
     uint32_t slot_id = 0, route_expert = 0, n_live = 1;
     VerifyPlan *plan_out = bid == 0 ? plan : nullptr;
     if constexpr (DENSE) {
@@ -406,16 +406,58 @@ __device__ __forceinline__ void gate_up_rows(GateUpMerge &s_red, PlanScratch &ps
     }
 }
 
-template <bool F16, bool DENSE = false>
+// The shared expert's gate/up as the last `blocks` blocks of a routed gate/up launch (blocks == 0: none).
+struct SharedGateUp {
+    const uint8_t *arena_layer;
+    ArenaGeom g;
+    const uint16_t *x;
+    uint32_t x_stride;
+    uint16_t *acts;
+    uint32_t blocks;
+};
+
+// What a kernel instantiated without the shared expert's role takes in its place: nothing to pass, nothing to load.
+struct NoSharedExpert {};
+template <bool SHARED, typename T>
+using SharedArg = std::conditional_t<SHARED, T, NoSharedExpert>;
+template <bool SHARED, typename T>
+SharedArg<SHARED, T> shared_arg(const T &v) {
+    if constexpr (SHARED) return v;
+    else return NoSharedExpert{};
+}
+
+// A block in that role: block `bid` of sh.blocks walks its share of the dense expert's row blocks for all `rows` rows.
+template <bool F16>
+__device__ __forceinline__ void shared_gate_up_role(GateUpMerge &s_red, PlanScratch &ps, const SharedGateUp &sh, uint32_t rows,
+                                                    uint32_t bid) {
+    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const KSlice k = k_slice(sh.g.gd, ks);
+    uint4 x0[kRing], x1[kRing];
+    f32x4 sx[kRing];
+    load_token_rows(sh.x, sh.x_stride, rows, lane, k, x0, x1);
+    gate_up_rows<F16, true>(s_red, ps, sh.arena_layer, sh.g, 1u, 1u, 0u, (uint16_t)0, rows, nullptr, k, x0, x1, sx, false, sh.acts,
+                            bid, sh.blocks);
+}
+
+template <bool F16, bool DENSE = false, bool SHARED = false>
 __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                                     uint32_t top_k, uint32_t n_experts,
                                                                     const uint32_t *__restrict__ idx,
                                                                     const uint16_t *__restrict__ w, uint32_t n_routes,
                                                                     VerifyPlan *__restrict__ plan,
                                                                     const uint16_t *__restrict__ x, uint32_t x_stride,
-                                                                    uint16_t *__restrict__ acts) {
+                                                                    uint16_t *__restrict__ acts,
+                                                                    SharedArg<SHARED, SharedGateUp> sh) {
     __shared__ GateUpMerge s_red;
     __shared__ PlanScratch ps;
+    uint32_t routed_blocks = gridDim.x;
+    if constexpr (SHARED) {
+        routed_blocks -= sh.blocks;
+        if (blockIdx.x >= routed_blocks) {
+            shared_gate_up_role<F16>(s_red, ps, sh, n_routes / top_k, blockIdx.x - routed_blocks);
+            return;
+        }
+    }
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     uint32_t route_idx = 0;
     uint16_t route_w = 0;
@@ -428,7 +470,8 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     uint4 x0[kRing], x1[kRing];
     load_token_rows(x, x_stride, n_routes / top_k, lane, k, x0, x1);
     f32x4 sx[kRing];
-    gate_up_rows<F16, DENSE>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, sx, false, acts);
+    gate_up_rows<F16, DENSE>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, sx, false, acts,
+                             blockIdx.x, routed_blocks);
 }
 
 // Router and gate/up of a decode step or verify block in ONE launch: the logits, the top-k select and the routes'
@@ -506,14 +549,14 @@ __device__ __forceinline__ void lone_wave_keys(const void *__restrict__ router_w
     }
 }
 
-template <bool W_F32, bool F16>
+template <bool W_F32, bool F16, bool SHARED>
 __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
     const uint8_t *__restrict__ arena_layer, ArenaGeom g, uint32_t top_k, uint32_t n_experts, const void *__restrict__ router_w,
     const uint16_t *__restrict__ effective_scale, const uint16_t *__restrict__ per_expert_scale,
     const uint16_t *__restrict__ router_x, uint32_t router_x_stride, uint32_t rows, RouteMail *__restrict__ mail,
     unsigned long long poll_ticks,
     uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w, VerifyPlan *__restrict__ plan,
-    const uint16_t *__restrict__ x, uint32_t x_stride, uint16_t *__restrict__ acts) {
+    const uint16_t *__restrict__ x, uint32_t x_stride, uint16_t *__restrict__ acts, SharedArg<SHARED, SharedGateUp> sh) {
     __shared__ GateUpMerge s_red;
     __shared__ PlanScratch ps;
     float(*s_part)[kChunkTokens][64] = reinterpret_cast<float(*)[kChunkTokens][64]>(&s_red[0][0][0][0]);   // 4 KiB of the 16
@@ -542,6 +585,16 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
             }
             if (lane < t_end - t0)
                 mail_store(&mail->logits[t0 + lane][e], stamp | __float_as_uint(mine));
+        }
+    }
+    // the blocks that serve the shared expert need no routes: they start on its rows now
+    uint32_t routed_blocks = gridDim.x;
+    if constexpr (SHARED) {
+        routed_blocks -= sh.blocks;
+        if (blockIdx.x >= routed_blocks) {
+            __syncthreads();      // the logits' partial sums (in s_red) have been read
+            shared_gate_up_role<F16>(s_red, ps, sh, rows, blockIdx.x - routed_blocks);
+            return;
         }
     }
     // the expert pass's token rows: in flight while the routes are made
@@ -638,7 +691,8 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
             __builtin_amdgcn_s_sleep(1);
         }
     }
-    gate_up_rows<F16>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, sx, true, acts);
+    gate_up_rows<F16>(s_red, ps, arena_layer, g, top_k, n_experts, route_idx, route_w, n_routes, plan, k, x0, x1, sx, true, acts,
+                      blockIdx.x, routed_blocks);
 }
 
 // down projection with the expert's activation rows in LDS: one block = four consecutive 32-row tile rows of one
@@ -662,42 +716,66 @@ constexpr int kDownLdsRow = kRing * kGroup * 2 + 16;      // bytes per activatio
 constexpr int kDownDepth = 4;
 constexpr int kDownEarly = 2;      // 16-byte pieces of the activation rows a thread requests ahead of the weights (covers 5 rows)
 
-template <bool OUT_BF16, bool F16>
+// The shared expert's down projection as extra slots of the launch (first_slot = the routed slots' count; ~0u: none):
+// slot first_slot + c takes groups [kRing c, kRing c + kRing) of the dense expert's K for all `rows` rows (route r = row r)
+// and leaves its un-weighted fp32 rows in partials[c].
+struct SharedDown {
+    const uint8_t *arena_layer;
+    ArenaGeom g;
+    const uint16_t *acts;       // [rows][g.f]
+    float *partials;            // [chunks][rows][g.d]
+    uint32_t first_slot, rows;
+};
+
+template <bool OUT_BF16, bool F16, bool SHARED>
 __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                           const VerifyPlan *__restrict__ plan,
                                                           const uint16_t *__restrict__ acts,
                                                           float *__restrict__ partials_f32,
-                                                          uint16_t *__restrict__ partials_bf16, uint32_t parts, RouteMail *mail) {
+                                                          uint16_t *__restrict__ partials_bf16, uint32_t parts, RouteMail *mail,
+                                                          SharedArg<SHARED, SharedDown> sh_arg) {
+    SharedDown sh{nullptr, g, nullptr, nullptr, 0xFFFFFFFFu, 0u};
+    if constexpr (SHARED) sh = sh_arg;
     __shared__ __align__(16) uint8_t s_act[kMaxRows * kDownLdsRow];
     __shared__ uint32_t s_route[kMaxRows];
     // the last launch of a call that leaves its rows un-combined: the routing launch of this call has read the epoch
     if (mail && blockIdx.x == 0 && threadIdx.x == 0) advance_epoch(mail);
     const uint32_t slot_id = blockIdx.x / parts, part = blockIdx.x % parts;
-    const PlanSlot &slot = plan->slots[slot_id];
-    const uint32_t n = __builtin_amdgcn_readfirstlane(slot.n);
-    const uint32_t expert = __builtin_amdgcn_readfirstlane(slot.expert);
+    const bool shared = SHARED && slot_id >= sh.first_slot;
+    const uint32_t chunk = shared ? slot_id - sh.first_slot : 0u;
+    const PlanSlot &slot = plan->slots[shared ? 0u : slot_id];
+    const uint32_t n = shared ? sh.rows : __builtin_amdgcn_readfirstlane(slot.n);
+    const uint32_t expert = shared ? 0u : __builtin_amdgcn_readfirstlane(slot.expert);
     if (n == 0) return;
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15, jq = lane >> 4;
-    const uint32_t chunks = g.f / 8;                       // 16-byte pieces per row
-    const uint32_t route_t = threadIdx.x < (uint32_t)kMaxRows ? slot.routes[threadIdx.x] : 0u;
+    // the slot's share of K: all of a routed expert's f, one chunk of the shared expert's
+    const uint32_t row_groups = shared ? sh.g.gf : g.gf;                                           // groups per tile row
+    const uint32_t g_first = shared ? chunk * (uint32_t)kRing : 0u;
+    const uint32_t ng = shared ? min((uint32_t)kRing, sh.g.gf - g_first) : g.gf, g_last = ng - 1;
+    const uint32_t act_stride = shared ? sh.g.f : g.f;
+    const uint16_t *act_rows = shared ? sh.acts + g_first * kGroup : acts;
+    const uint32_t chunks = ng * (kGroup / 8);            // 16-byte pieces per row
+    auto route_of = [&](uint32_t i) { return shared ? i : slot.routes[i]; };
+    const uint32_t route_t = threadIdx.x < (uint32_t)kMaxRows ? route_of(threadIdx.x) : 0u;
     uint4 early[kDownEarly];
 #pragma unroll
     for (int k = 0; k < kDownEarly; ++k) {
         const uint32_t i = threadIdx.x + 256u * k, r = i / chunks, c = i % chunks;
         // rows past the count re-read the last one (never stored): no load sits behind a branch
-        early[k] = *reinterpret_cast<const uint4 *>(acts + (size_t)slot.routes[min(r, n - 1)] * g.f + c * 8);
+        early[k] = *reinterpret_cast<const uint4 *>(act_rows + (size_t)route_of(min(r, n - 1)) * act_stride + c * 8);
     }
     const uint32_t rb = part * 4 + wave;
     const bool has_row = rb < g.dn_rbp;
-    const uint8_t *expert_base = arena_layer + (size_t)expert * g.expert_bytes;
-    const TileSource src = make_tile_source(expert_base + g.dn_tiles_off, (size_t)g.dn_rbp * g.gf * kTileBytes,
-                                            expert_base + g.dn_scales_off, (size_t)g.dn_rbp * g.gf * kTileScaleBytes);
-    const uint32_t ng = g.gf, g_last = g.gf - 1;
+    const ArenaGeom &eg = shared ? sh.g : g;
+    const uint8_t *expert_base = shared ? sh.arena_layer : arena_layer + (size_t)expert * g.expert_bytes;
+    const TileSource src = make_tile_source(expert_base + eg.dn_tiles_off, (size_t)eg.dn_rbp * eg.gf * kTileBytes,
+                                            expert_base + eg.dn_scales_off, (size_t)eg.dn_rbp * eg.gf * kTileScaleBytes);
+    const uint32_t tile0 = rb * row_groups + g_first;      // the wave's first tile
     WeightRing ring;
     if (has_row) {
 #pragma unroll
-        for (int u = 0; u < kDownDepth; ++u) ring_fill(ring, u, src, rb * ng + min((uint32_t)u, g_last), lane);
+        for (int u = 0; u < kDownDepth; ++u) ring_fill(ring, u, src, tile0 + min((uint32_t)u, g_last), lane);
     }
     if (threadIdx.x < (uint32_t)kMaxRows) s_route[threadIdx.x] = threadIdx.x < n ? route_t : 0u;
 #pragma unroll
@@ -711,7 +789,7 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
         for (uint32_t i = threadIdx.x + 256u * kDownEarly; i < n * chunks; i += 256) {
             const uint32_t r = i / chunks, c = i % chunks;
             *reinterpret_cast<uint4 *>(s_act + r * kDownLdsRow + c * 16) =
-                *reinterpret_cast<const uint4 *>(acts + (size_t)s_route[r] * g.f + c * 8);
+                *reinterpret_cast<const uint4 *>(act_rows + (size_t)s_route[r] * act_stride + c * 8);
         }
     }
     lds_barrier();      // LDS only: the weight tiles stay in flight across it
@@ -730,7 +808,7 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
         const f32x4 sx = group_input_sum<F16>(x0, x1);
         // consume slot u % kDownDepth; the load that refills it (group u + kDownDepth) starts inside the step
         if (u + kDownDepth < kRing)
-            ring_step<F16, true>(ring, u % kDownDepth, live, x0, x1, sx, tot, src, rb * ng + min((uint32_t)(u + kDownDepth), g_last), lane);
+            ring_step<F16, true>(ring, u % kDownDepth, live, x0, x1, sx, tot, src, tile0 + min((uint32_t)(u + kDownDepth), g_last), lane);
         else
             ring_step<F16, false>(ring, u % kDownDepth, live, x0, x1, sx, tot, src, 0u, lane);
         // The running sums are pinned here: left alone, the compiler sinks the scale-and-bias arithmetic of every
@@ -740,17 +818,18 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
         for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(tot.a[r]), "+v"(tot.b[r]));
     }
     const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
+    float *rows_f32 = shared ? sh.partials + (size_t)chunk * sh.rows * g.d : partials_f32;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const uint32_t ts = 4 * jq + r;
         if (ts < n) {
             const size_t base = (size_t)s_route[ts] * g.d;
-            if (OUT_BF16) {
+            if (OUT_BF16 && !shared) {
                 partials_bf16[base + row_a] = Act<F16>::round(tot.a[r]);
                 partials_bf16[base + row_b] = Act<F16>::round(tot.b[r]);
             } else {
-                partials_f32[base + row_a] = tot.a[r];
-                partials_f32[base + row_b] = tot.b[r];
+                rows_f32[base + row_a] = tot.a[r];
+                rows_f32[base + row_b] = tot.b[r];
             }
         }
     }
@@ -1005,7 +1084,8 @@ template <bool F16>
 hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t top_k,
                             const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx, const uint16_t *w,
                             const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16, VerifyPlan *plan, uint16_t *acts,
-                            float *partials_f32, uint32_t n_cus, KernelTimer *timer, const RouteFusion *route, bool dense) {
+                            float *partials_f32, uint32_t n_cus, KernelTimer *timer, const RouteFusion *route, bool dense,
+                            const SharedExpert *shared) {
     // `route`: the routes are not there yet - idx / w are where this call has to write them. One launch does the
     // router and gate/up when the expert fits the persistent kernel, the combine follows in this call (it advances
     // the epoch) and the router rows are 8-byte aligned; otherwise the router's own two launches go first.
@@ -1029,26 +1109,58 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     const bool dn_ksplit = !dn_whole && (g.gf + kKSplit - 1) / kKSplit <= (uint32_t)kRing;
     const uint32_t resident = 2 * n_cus;       // blocks the chip holds at once (__launch_bounds__(256, 2))
     const bool decode_form = t == 1 && dn_whole && !partials_bf16 && !rows_only && top_k <= 8;
+    // The shared expert rides along in the persistent gate/up launch and the LDS form of the down launch.
+    if (shared && !(gu_persistent && dn_whole && rows_only && shared->g.d == g.d && shared->g.gd == g.gd))
+        return hipErrorInvalidValue;
+    SharedGateUp sh_gu{nullptr, g, nullptr, 0u, nullptr, 0u};
+    SharedDown sh_dn{nullptr, g, nullptr, nullptr, 0xFFFFFFFFu, 0u};
+    auto shared_blocks = [&](uint32_t cap, uint32_t routed_wanted) -> uint32_t {
+        // Blocks for the shared expert's row blocks: one each when the grid has room (a decode step); else its share of
+        // the resident blocks by row blocks, the routed experts counted at the number of live ones a block of t rows
+        // typically has (three per row). They start while the routed blocks wait for their routes, so a block of
+        // theirs may walk a row block or two more than a routed one: a fifth fewer than the fair share. Measured per
+        // layer block of 16 / 8 / 4 rows with 12 ... 132 such blocks: flat within 0.5 us from 19 / 27 / 33 blocks up
+        // (70.0 / 55.8 / 44.4 us; this rule picks 23 / 42 / 72), 6 to 12 us worse at 12 blocks.
+        const uint32_t rb = shared->g.gu_rb;
+        if (routed_wanted + rb <= cap) return rb;
+        const uint32_t live = min(slots, 3 * t + 2);
+        const uint32_t fair = (uint32_t)(((uint64_t)cap * rb) / ((uint64_t)live * g.gu_rb + rb));
+        return max(1u, min(rb, min(cap / 2, fair - fair / 5)));
+    };
     if (fuse) {
         // at least one block per row (it selects the row's routes), at most what is resident at once
-        const uint32_t blocks = min(route->resident_blocks, max(max(slots, t), min(route->resident_blocks, slots * g.gu_rb)));
-#define FFMOE_ROUTE_GU(WF)                                                                                                  \
-    hipLaunchKernelGGL((route_gate_up_persistent<WF, F16>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, \
+        uint32_t blocks = min(route->resident_blocks, max(max(slots, t), min(route->resident_blocks, slots * g.gu_rb)));
+        if (shared) {
+            const uint32_t sb = shared_blocks(route->resident_blocks, blocks);
+            sh_gu = SharedGateUp{shared->arena_layer, shared->g, shared->x, shared->x_stride, shared->acts, sb};
+            blocks = max(t, min(blocks, route->resident_blocks - sb)) + sb;
+        }
+#define FFMOE_ROUTE_GU(WF, SH)                                                                                              \
+    hipLaunchKernelGGL((route_gate_up_persistent<WF, F16, SH>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, \
                        route->rw.w, route->rw.effective_scale, route->rw.per_expert_scale, route->router_x,                  \
                        route->router_x_stride, t, route->mail, route->poll_ticks, const_cast<uint32_t *>(idx),                \
                        const_cast<uint16_t *>(w), plan,                                                                     \
-                       x, x_stride, acts)
-        if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true); else FFMOE_ROUTE_GU(false);
+                       x, x_stride, acts, shared_arg<SH>(sh_gu))
+        if (shared) { if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true, true); else FFMOE_ROUTE_GU(false, true); }
+        else { if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true, false); else FFMOE_ROUTE_GU(false, false); }
 #undef FFMOE_ROUTE_GU
     } else if (gu_persistent) {
         // plan slot of the profile stays empty: the gate/up kernel builds the plan itself
-        const uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
+        uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
+        if (shared) {
+            const uint32_t sb = shared_blocks(max(resident, blocks), blocks);
+            sh_gu = SharedGateUp{shared->arena_layer, shared->g, shared->x, shared->x_stride, shared->acts, sb};
+            blocks = max(1u, min(blocks, max(resident, blocks) - sb)) + sb;
+        }
         if (dense)
             hipLaunchKernelGGL((skinny_gate_up_persistent<F16, true>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k,
-                               n_experts, idx, w, t * top_k, plan, x, x_stride, acts);
+                               n_experts, idx, w, t * top_k, plan, x, x_stride, acts, NoSharedExpert{});
+        else if (shared)
+            hipLaunchKernelGGL((skinny_gate_up_persistent<F16, false, true>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k,
+                               n_experts, idx, w, t * top_k, plan, x, x_stride, acts, sh_gu);
         else
             hipLaunchKernelGGL(skinny_gate_up_persistent<F16>, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, idx,
-                               w, t * top_k, plan, x, x_stride, acts);
+                               w, t * top_k, plan, x, x_stride, acts, NoSharedExpert{});
     } else {
         hipLaunchKernelGGL(verify_plan_kernel, dim3(1), dim3(256), 0, s, idx, w, t * top_k, n_experts, plan);
         timer->mark(s, FFMOE_K_PLAN);
@@ -1079,13 +1191,17 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     }
     const uint32_t dn_parts = (g.dn_rbp + 3) / 4;          // blocks per expert of the LDS form: four tile rows each
     const bool dense_ksplit = dense && gu_persistent;      // the plan-free forms go together
-    const dim3 dn_grid = dn_whole    ? dim3(slots * dn_parts)
+    if (shared) sh_dn = SharedDown{shared->arena_layer, shared->g, shared->acts, shared->partials, slots, t};
+    const dim3 dn_grid = dn_whole    ? dim3((slots + (shared ? shared_chunks(shared->g) : 0u)) * dn_parts)
                          : dn_ksplit ? dim3(max(slots, min(resident, slots * g.dn_rbp)))
                                      : dim3((g.dn_rbp + 3) / 4, slots);
 #define FFMOE_DOWN(BF)                                                                                                \
-    if (dn_whole)                                                                                                     \
-        hipLaunchKernelGGL((skinny_down_lds<BF, F16>), dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,          \
-                           partials_f32, partials_bf16, dn_parts, rows_only ? mail : nullptr);                         \
+    if (dn_whole && shared)                                                                                           \
+        hipLaunchKernelGGL((skinny_down_lds<BF, F16, true>), dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,    \
+                           partials_f32, partials_bf16, dn_parts, rows_only ? mail : nullptr, sh_dn);                  \
+    else if (dn_whole)                                                                                                \
+        hipLaunchKernelGGL((skinny_down_lds<BF, F16, false>), dn_grid, dim3(256), 0, s, arena_layer, g, plan, acts,   \
+                           partials_f32, partials_bf16, dn_parts, rows_only ? mail : nullptr, NoSharedExpert{});       \
     else if (dn_ksplit && dense_ksplit)                                                                               \
         hipLaunchKernelGGL((skinny_down_ksplit_persistent<BF, F16, true>), dn_grid, dim3(256), 0, s, arena_layer, g,  \
                            plan, acts, partials_f32, partials_bf16, t);                                               \
@@ -1218,10 +1334,14 @@ uint32_t route_launch_resident_blocks(uint32_t n_cus) {
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess) n = 0;
         least = n < least ? n : least;
     };
-    ask(route_gate_up_persistent<false, false>);
-    ask(route_gate_up_persistent<true, false>);
-    ask(route_gate_up_persistent<false, true>);
-    ask(route_gate_up_persistent<true, true>);
+    ask(route_gate_up_persistent<false, false, false>);
+    ask(route_gate_up_persistent<true, false, false>);
+    ask(route_gate_up_persistent<false, true, false>);
+    ask(route_gate_up_persistent<true, true, false>);
+    ask(route_gate_up_persistent<false, false, true>);
+    ask(route_gate_up_persistent<true, false, true>);
+    ask(route_gate_up_persistent<false, true, true>);
+    ask(route_gate_up_persistent<true, true, true>);
     (void)hipGetLastError();
     return least > 0 ? (uint32_t)least * n_cus : 0u;
 }
@@ -1231,13 +1351,13 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
                          uint32_t top_k, const uint16_t *x, uint32_t x_stride, uint32_t t, const uint32_t *idx,
                          const uint16_t *w, const uint16_t *residual, uint16_t *y, uint16_t *partials_bf16,
                          VerifyPlan *plan, uint16_t *acts, float *partials_f32, uint32_t n_cus, KernelTimer *timer, bool f16,
-                         const RouteFusion *route, bool dense) {
+                         const RouteFusion *route, bool dense, const SharedExpert *shared) {
     // dense: the caller vouches that this is a dense FFN - one expert, top_k = 1, every row at weight 1
     dense = dense && n_experts == 1 && top_k == 1 && !route;
     return f16 ? launch_verify_as<true>(s, arena_layer, g, n_experts, top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                                        plan, acts, partials_f32, n_cus, timer, route, dense)
+                                        plan, acts, partials_f32, n_cus, timer, route, dense, shared)
                : launch_verify_as<false>(s, arena_layer, g, n_experts, top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
-                                         plan, acts, partials_f32, n_cus, timer, route, dense);
+                                         plan, acts, partials_f32, n_cus, timer, route, dense, shared);
 }
 
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,

@@ -49,7 +49,7 @@ EXPORTS = [
     "ffmoe_matrix_greedy", "ffmoe_matrix_greedy_conf", "ffmoe_argmax_rows", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
     "ffmoe_layer_tail", "ffmoe_layer_tail_routed", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
-    "ffmoe_verify_static",
+    "ffmoe_verify_static", "ffmoe_route_verify_shared", "ffmoe_layer_tail_routed_shared",
 ]
 
 PROFILE_SLOTS = 16
@@ -234,6 +234,8 @@ def lib() -> C.CDLL:
                                         C.c_float, errp]
     L.ffmoe_layer_tail.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, vp, u32, u32, C.c_float, C.c_float, errp]
     L.ffmoe_layer_tail_routed.argtypes = [vp, vp, vp, vp, u32, vp, u32, vp, vp, u32, C.c_float, C.c_float, errp]
+    L.ffmoe_route_verify_shared.argtypes = [vp, vp, vp, u32, u32, vp, u32, vp, u32, vp, u32, u32, vp, vp, errp]
+    L.ffmoe_layer_tail_routed_shared.argtypes = [vp, vp, vp, vp, vp, u32, vp, vp, u32, C.c_float, C.c_float, errp]
     _lib = L
     return L
 
@@ -438,6 +440,19 @@ class Context:
                                          t, _ptr(residual), _ptr(y), _ptr(idx), _ptr(w), C.byref(err)), err)
         return y, idx, w
 
+    def route_verify_shared(self, shared: "Context", layer: int, shared_layer: int, router_x, x, shared_x):
+        """route_verify(..., combine=False) with the shared expert (the dense context `shared`, on shared_x) inside the
+        same two launches. Returns (idx, w); the rows stay in the two contexts for layer_tail_routed_shared."""
+        import torch
+        t, k = x.shape[0], self.shape.top_k
+        idx = torch.empty((t, k), dtype=torch.int32, device=x.device)
+        w = torch.empty((t, k), dtype=self.act, device=x.device)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_route_verify_shared(self._h, shared._h, _stream(), layer, shared_layer, _ptr(router_x),
+                                                _row_stride(router_x), _ptr(x), _row_stride(x), _ptr(shared_x),
+                                                _row_stride(shared_x), t, _ptr(idx), _ptr(w), C.byref(err)), err)
+        return idx, w
+
     def verify_partials(self, layer: int, x, idx, w, partials=None):
         import torch
         t = x.shape[0]
@@ -555,6 +570,16 @@ class Context:
         _check(self.L.ffmoe_layer_tail_routed(self._h, _stream(), _ptr(route_w), _ptr(h1), _row_stride(h1), _ptr(hidden),
                                               _row_stride(hidden), _ptr(w_postffn2), _ptr(w_postffn), t, eps, layer_scalar,
                                               C.byref(err)), err)
+        return hidden
+
+    def layer_tail_routed_shared(self, shared: "Context", route_w, hidden, w_postffn2, w_postffn, layer_scalar: float,
+                                 eps: float = 1e-6):
+        """layer_tail on the rows the last route_verify_shared left in this context (routed) and in `shared` (h1)."""
+        t = hidden.shape[0]
+        err = C.c_char_p()
+        _check(self.L.ffmoe_layer_tail_routed_shared(self._h, shared._h, _stream(), _ptr(route_w), _ptr(hidden),
+                                                     _row_stride(hidden), _ptr(w_postffn2), _ptr(w_postffn), t, eps,
+                                                     layer_scalar, C.byref(err)), err)
         return hidden
 
     def layer_tail_norms(self, h2, h1, hidden, w_postffn1, w_postffn2, w_postffn, layer_scalar: float, w_next=None,

@@ -682,13 +682,28 @@ def main():
         def run_fused():
             layer_block_fused(counter["i"])
             counter["i"] += 1
+
+        def layer_block_inside(i):
+            # the shared expert inside the routed experts' two launches as well: three launches
+            ctx.post_attn_setup(hid_b, att_b, wn_b[0], wn_b[1], wn_b[2], out=outs_b)
+            rc = Lib.ffmoe_route_verify_shared(h, dense._h, stream, i % L, i % LS, pouts[2], D, pouts[1], D, pouts[0], D, T,
+                                               pidx, pw, C.byref(err))
+            if rc:
+                raise RuntimeError(err.value)
+            ctx.layer_tail_routed_shared(dense, w, hid_b, wn_b[3], wn_b[4], 1.0)
+
+        def run_inside():
+            layer_block_inside(counter["i"])
+            counter["i"] += 1
         t_seq = timed(lambda: run_block(False), 120, warm=30)
         t_con = timed(lambda: run_block(True), 120, warm=30)
         t_fus = timed(run_fused, 120, warm=30)
+        t_ins = timed(run_inside, 120, warm=30)
         # the same chain of L layers as a HIP graph: nine launches per layer from Python are host-bound,
         # a replay shows the device time (the library only enqueues kernels, so the chain captures as it is)
         graph_us = {}
-        for label, conc in (("one_stream", False), ("shared_expert_on_second_stream", True), ("combine_in_layer_tail", None)):
+        for label, conc in (("one_stream", False), ("shared_expert_on_second_stream", True), ("combine_in_layer_tail", None),
+                            ("shared_expert_inside_routed_launches", "inside")):
             gph = torch.cuda.CUDAGraph()
             cap = torch.cuda.Stream()
             cap.wait_stream(main_s)
@@ -696,7 +711,9 @@ def main():
                 main_s = torch.cuda.current_stream()
                 stream = C.c_void_p(main_s.cuda_stream)
                 for i in range(L):
-                    if conc is None:
+                    if conc == "inside":
+                        layer_block_inside(i)
+                    elif conc is None:
                         layer_block_fused(i)
                     else:
                         layer_block(i, conc)
@@ -706,6 +723,7 @@ def main():
             del gph
         extra["layer_block_rows16"] = {"one_stream_us": round(t_seq * 1e6, 2), "shared_expert_on_second_stream_us": round(t_con * 1e6, 2),
                                        "combine_in_layer_tail_us": round(t_fus * 1e6, 2),
+                                       "shared_expert_inside_routed_launches_us": round(t_ins * 1e6, 2),
                                        "hip_graph_replay_us": graph_us,
                                        "steps": "post-attention setup, shared expert, router, routed experts, layer tail"}
         dense.close()

@@ -403,6 +403,31 @@ int ffmoe_layer_tail_routed(ffmoe_ctx *ctx, void *stream, const uint16_t *route_
                             uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
                             uint32_t t, float eps, float layer_scalar, char **err);
 
+/* The expert work of one MoE block for a decode step / verify block (t <= 16) with the shared expert inside the
+ * routed experts' two launches: ffmoe_route_verify(ctx, ..., y = NULL) on (router_x, x) and ffmoe_dense_ffn(shared, ...)
+ * on shared_x in one call. `shared` is a context with n_experts = 1 and top_k = 1 (ffmoe_upload_expert_parts /
+ * ffmoe_upload_layer) on the same device with the same hidden size and activation type. Some blocks of the gate/up
+ * launch walk the shared expert's rows - they need no routes, so they stream while the others wait for theirs - and the
+ * down launch takes the shared expert's K = f in chunks of 704 as extra experts (f <= 2816). Nothing is combined: the
+ * routed rows stay un-weighted in `ctx`, the shared expert's chunk rows in `shared`, for
+ * ffmoe_layer_tail_routed_shared. out_idx / out_w as in ffmoe_route_verify (same routes, bit for bit). The routed part
+ * equals ffmoe_route_verify bit for bit; the shared expert's row is the same sum in another order (K in three
+ * chunks instead of four interleaved slices), inside the 1e-2 / 0.9999 bar of the dense FFN. Shapes outside
+ * (routed f > 704, d > 2816) are refused: run the two calls. This is the reference's schedule - shared expert beside
+ * router + routed experts (Runtime/Inference/RealForwardRunner.swift:454-756; Kernels/MoE/SharedExpertInt4.swift:23-89
+ * beside Kernels/MoE/MoE.swift:454-496) - as one pair of launches. */
+int ffmoe_route_verify_shared(ffmoe_ctx *ctx, ffmoe_ctx *shared, void *stream, uint32_t layer, uint32_t shared_layer,
+                              const uint16_t *router_x, uint32_t router_x_stride, const uint16_t *x, uint32_t x_stride,
+                              const uint16_t *shared_x, uint32_t shared_x_stride, uint32_t t, uint32_t *out_idx,
+                              uint16_t *out_w, char **err);
+
+/* ffmoe_layer_tail_routed with h1 taken from the rows the last ffmoe_route_verify_shared(ctx, shared, ...) left in
+ * `shared`: h1 = the chunk rows added in chunk order, rounded once to 16 bits (the dense FFN's output row); h2 and
+ * the tail as in ffmoe_layer_tail_routed. */
+int ffmoe_layer_tail_routed_shared(ffmoe_ctx *ctx, ffmoe_ctx *shared, void *stream, const uint16_t *route_w,
+                                   uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2,
+                                   const uint16_t *w_postffn, uint32_t t, float eps, float layer_scalar, char **err);
+
 /* The layer tail with the two decode norms either side of it folded in: h1 arrives BEFORE its own norm
  * (w_postffn1, the shared expert's post-FFN-1 norm; h1 is left as found), and when w_next / normed are
  * given the norm of the new hidden row under w_next (the next layer's input norm) is written to normed.

@@ -154,3 +154,97 @@ def test_dense_ffn_argument_errors(ff, oracle, torch):
         dense.dense_ffn(0, torch.zeros((33, 128), dtype=torch.bfloat16, device="cuda"))
     assert float(dense.dense_ffn(0, x).abs().max()) == 0.0
     dense.close()
+
+
+@pytest.mark.parametrize("d,f,e,fs,t,mode", [
+    (128, 64, 16, 192, 5, "one_launch"),          # shared K in one short chunk
+    (128, 64, 16, 1472, 16, "one_launch"),        # 23 groups: chunks of 11, 11 and 1
+    (128, 64, 16, 1472, 3, "router_launches"),    # the router as launches of its own: the plain gate/up kernel hosts the blocks
+    (128, 64, 16, 1472, 7, "no_hand_over"),       # every wave gives up waiting at once and routes for itself
+    (2816, 704, 128, 2112, 1, "one_launch"),      # the model's shapes: decode step
+    (2816, 704, 128, 2112, 16, "one_launch"),     # verify block
+    (2816, 704, 128, 2112, 6, "router_launches"),
+])
+def test_shared_expert_inside_the_routed_launches(ff, oracle, torch, d, f, e, fs, t, mode):
+    """ffmoe_route_verify_shared + ffmoe_layer_tail_routed_shared against the separate calls (ffmoe_route_verify,
+    ffmoe_dense_ffn, ffmoe_layer_tail): same routes bit for bit; the new hidden rows agree to the rounding of the
+    shared expert's row (its K is summed in chunks instead of interleaved slices), and with the shared expert's rows
+    zeroed out of the comparison - a shared expert of zero weights - bit for bit. Padding stays untouched."""
+    from helpers import make_layer, to_ff_offsets
+    rng, pool, router = make_layer(oracle, 5, d, f, e, align=16)
+    ctx = ff.Context(d, f, e, 8, n_layers=1, max_tokens=16)
+    ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
+    ctx.upload_router_bf16(0, router)
+    g = oracle.seed_tree_key(0x5A4E, f"shared-inside-d{d}-fs{fs}-t{t}-{mode}")
+    scale = 0.4 if d < 1024 else 0.08
+    parts = tuple(oracle.quantize_int4(g.uniform(-scale, scale, r * c).reshape(r, c)) for r, c in ((fs, d), (fs, d), (d, fs)))
+    zero_parts = tuple(oracle.quantize_int4(np.zeros((r, c), np.float32)) for r, c in ((fs, d), (fs, d), (d, fs)))
+    shared = ff.Context(d, fs, 1, 1, n_layers=2, max_tokens=16)
+    shared.upload_expert_parts(0, 0, *zero_parts)
+    shared.upload_expert_parts(1, 0, *parts)
+    pad = 8
+    xb, rxb, sxb = (oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d) for _ in range(3))
+    x, rx, sx = bf16_tensor(torch, xb), bf16_tensor(torch, rxb), bf16_tensor(torch, sxb)
+    hid = np.full((t, d + pad), oracle.bf16_bits(np.float32(-25.0)), np.uint16)
+    hid[:, :d] = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    tw2, tw1 = (bf16_tensor(torch, oracle.bf16_bits(g.uniform(0.5, 1.5, d))) for _ in range(2))
+    if mode == "router_launches":
+        ctx.set_one_launch_routing(False)
+    if mode == "no_hand_over":
+        ctx.set_handover_timeout(0)
+    for layer_s in (0, 1):
+        y, idx_a, w_a = ctx.route_verify(0, rx, x)
+        h1 = shared.dense_ffn(layer_s, sx)
+        hid_a = bf16_tensor(torch, hid)
+        ctx.layer_tail(y, h1, hid_a, tw2, tw1, 0.875, 1e-6, d=d)
+        idx_b, w_b = ctx.route_verify_shared(shared, 0, layer_s, rx, x, sx)
+        hid_b = bf16_tensor(torch, hid)
+        ctx.layer_tail_routed_shared(shared, w_b, hid_b, tw2, tw1, 0.875, 1e-6)
+        assert np.array_equal(idx_a.cpu().numpy(), idx_b.cpu().numpy()) and np.array_equal(bits_of(w_a), bits_of(w_b))
+        got, want = bits_of(hid_b), bits_of(hid_a)[:, :d]
+        assert np.array_equal(got[:, d:], hid[:, d:])
+        if layer_s == 0:
+            assert float(h1.abs().max()) == 0.0
+            assert np.array_equal(got[:, :d], want)
+        else:
+            gf, wf = oracle.bf16_to_float(got[:, :d]), oracle.bf16_to_float(want)
+            assert rel_err(gf, wf) < 1e-2 and cosine(gf, wf) > 0.9999, (rel_err(gf, wf), cosine(gf, wf))
+            assert np.mean(got[:, :d] == want) > 0.8
+    # the shared expert's row itself: with the routed rows' norm weight at zero the tail is hidden + norm(h1) scaled
+    zero = torch.zeros_like(tw2)
+    one = torch.ones_like(tw1)
+    hid0 = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    ctx.route_verify_shared(shared, 0, 1, rx, x, sx)
+    ctx.layer_tail_routed_shared(shared, w_b, hid0, zero, one, 1.0, 1e-6)
+    ref = _reference_rows(oracle, parts, sxb)
+    ref_bits = oracle.bf16_bits(ref.astype(np.float32))
+    want0 = oracle.layer_tail(np.zeros((t, d), np.uint16), ref_bits, np.zeros((t, d), np.uint16), bits_of(zero), bits_of(one), 1.0, 1e-6)
+    g0, w0 = oracle.bf16_to_float(bits_of(hid0)), oracle.bf16_to_float(want0)
+    assert rel_err(g0, w0) < 1e-2 and cosine(g0, w0) > 0.9999, (rel_err(g0, w0), cosine(g0, w0))
+    if mode == "no_hand_over":
+        assert ctx.handover_giveups() > 0
+    elif mode == "one_launch":
+        assert ctx.handover_giveups() == 0
+    # ordinary calls on both contexts afterwards
+    y2, idx_c, _ = ctx.route_verify(0, rx, x)
+    assert np.array_equal(bits_of(y2), bits_of(y)) and np.array_equal(idx_c.cpu().numpy(), idx_a.cpu().numpy())
+    assert np.array_equal(bits_of(shared.dense_ffn(1, sx)), bits_of(h1))
+    ctx.close()
+    shared.close()
+
+
+def test_route_verify_shared_argument_errors(ff, oracle, torch):
+    ctx = ff.Context(128, 64, 4, 2, n_layers=1, max_tokens=16)
+    other = ff.Context(128, 64, 4, 2, n_layers=1, max_tokens=16)
+    wide = ff.Context(256, 64, 1, 1, n_layers=1, max_tokens=16)
+    x = torch.zeros((2, 128), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ff.FieldfareError, match="n_experts = 1"):
+        ctx.route_verify_shared(other, 0, 0, x, x, x)
+    with pytest.raises(ff.FieldfareError, match="not uploaded"):
+        ctx.route_verify_shared(wide, 0, 0, x, x, x)
+    parts = tuple(oracle.quantize_int4(np.zeros((r, c), np.float32)) for r, c in ((64, 256), (64, 256), (256, 64)))
+    wide.upload_expert_parts(0, 0, *parts)
+    with pytest.raises(ff.FieldfareError, match="same d"):
+        ctx.route_verify_shared(wide, 0, 0, x, x, x)
+    for c in (ctx, other, wide):
+        c.close()
