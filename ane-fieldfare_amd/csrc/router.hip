@@ -206,10 +206,11 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, co
 //      a candidate.
 //      B: both sums add the same exact products (bf16 x bf16 fits fp32), so each differs from the real-number sum
 //      by at most (roundings on the longest path of its summation tree) x (relative size of one rounding) x
-//      sum_k |x_k w_ek| <= ... x ||x|| max_e ||w_e||. Approximate pass: d / 128 accumulations per wave, each adding 32
-//      products (counted as 33 roundings of 2^-23, whatever order the unit uses), and 2 to merge the four waves.
-//      Pinned order: 4 fmaf per 1024-wide step, 2 adds for the sub-accumulators, 6 for the butterfly, 2^-24 each.
-//      The launch takes four times both counts.
+//      sum_k |x_k w_ek| <= ... x ||x|| max_e ||w_e||. Approximate pass: d / 128 matrix instructions per wave, each
+//      adding 32 products to the running sum in an order the unit does not document; the count assumes the worst one,
+//      the running sum carried through all 33 additions of every instruction: 33 d / 128 roundings of 2^-23, and 2 to
+//      merge the four waves. Pinned order: 4 fmaf per 1024-wide step, 2 adds for the sub-accumulators, 6 for the
+//      butterfly, 2^-24 each (the order is this build's own, so the count is exact).
 // Needs: bf16 rows and weights, no per-input scale, d a multiple of 256 up to 4096, E a multiple of 16 up to 128
 // (the sixteen waves of the approximate pass hold two 16-expert fragments each).
 // ---------------------------------------------------------------------------------------------------
@@ -458,8 +459,8 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
         if (per_wave <= 1) FFMOE_APPROX(1); else FFMOE_APPROX(2);
 #undef FFMOE_APPROX
         timer->mark(s, FFMOE_K_ROUTER_LOGITS);
-        // 2 B per unit of ||x||: four times the rounding counts of the two sums (see above), 1 % on top for the norms' own rounding
-        const float approx_roundings = 4.0f * ((float)(d / 128 + 1) + 33.0f + 2.0f), pinned_roundings = 4.0f * (4.0f * ((d + 1023) / 1024) + 8.0f);
+        // 2 B per unit of ||x||: the rounding counts of the two sums (see above), 1 % on top for the norms' own rounding
+        const float approx_roundings = 33.0f * (float)(d / 128) + 2.0f, pinned_roundings = 4.0f * ((d + 1023) / 1024) + 8.0f;
         const float bound_per_norm = 2.02f * (approx_roundings * 0x1p-23f + pinned_roundings * 0x1p-24f) * rw.w_norm_max;
 #define FFMOE_EXACT(STEPS, CHUNK)                                                                                          \
     hipLaunchKernelGGL((router_exact_topk_kernel<STEPS, CHUNK>), dim3((t + 3) / 4), dim3(256), 0, s,                         \

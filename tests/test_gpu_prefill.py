@@ -338,6 +338,13 @@ def test_prefill_router_fast_form_equals_pinned_form(oracle, torch):
     x[10] = router[3] * 50
     x[11] = router[99] * 50
     x[12] = -router[6] * 50
+    # a near-tie exactly at the select's edge, under a large norm: seven experts far in front, then experts 6 and 7,
+    # whose rows differ by one bf16 step in one element, as eighth and ninth - their pinned logits are a few fp32
+    # steps apart, far less than the approximate pass's error at that norm, so only the pinned sums can order them
+    wf = oracle.bf16_to_float(bits)
+    front = [20, 30, 40, 50, 60, 70, 80]
+    for row, scale in ((13, 50.0), (14, 2000.0)):
+        x[row] = scale * (1.5 * wf[front].sum(axis=0) + wf[6])
     xb = bf16_tensor(torch, oracle.bf16_bits(x))
     ctx = ff.Context(d, 64, e, k, n_layers=1, max_tokens=128)
     ctx.upload_router_bf16(0, bits)
@@ -360,4 +367,10 @@ def test_prefill_router_fast_form_equals_pinned_form(oracle, torch):
     # the ties resolve to the lower index
     got = got_idx
     assert list(got[10][:3]) == [3, 5, 64] and list(got[11][:3]) == [99, 100, 101]
+    for row in (13, 14):
+        want = oracle.router_logits_pinned(bits, xbits[row])
+        order = np.argsort(-want, kind="stable")
+        assert set(order[:7]) == set(front) and set(order[7:9]) == {6, 7}, (row, order[:10])
+        assert want[6] != want[7] and abs(want[6] - want[7]) < 1e-4 * abs(want[6])
+        assert sorted(got[row]) == sorted(order[:8])
     ctx.close()
