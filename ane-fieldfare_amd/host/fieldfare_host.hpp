@@ -265,6 +265,27 @@ public:
         check(ffmoe_route_verify(c_.raw(), stream, layer, routerHidden, routerStrideElements, x, xStrideElements, (uint32_t)rows,
                                  residual, y, outIndices, outWeights, &err), err);
     }
+    // The same pair with the shared expert of the block (SharedExpertInt4.encode on `sharedX`, which the runner issues
+    // beside the routed experts: RealForwardRunner.swift:454-756) inside its two launches. Nothing is combined: the rows
+    // stay on the device for FusedLayerTail::encodeRoutedShared, which needs `outWeights`.
+    void encodeRouterRoutedAndSharedExperts(void *stream, Context &shared, uint32_t layer, uint32_t sharedLayer,
+                                            const uint16_t *routerHidden, uint32_t routerStrideElements, const uint16_t *x,
+                                            uint32_t xStrideElements, const uint16_t *sharedX, uint32_t sharedStrideElements,
+                                            int rows, uint32_t *outIndices, uint16_t *outWeights) {
+        if (rows < 1 || rows > maxRouterRows) throw std::invalid_argument("rows outside 1...16");
+        char *err = nullptr;
+        check(ffmoe_route_verify_shared(c_.raw(), shared.raw(), stream, layer, sharedLayer, routerHidden, routerStrideElements, x,
+                                        xStrideElements, sharedX, sharedStrideElements, (uint32_t)rows, outIndices, outWeights, &err),
+              err);
+    }
+    // Waves of the one-launch form that stopped waiting for another block and computed its part themselves (the results
+    // are the same; a count above zero says the GPU is shared and the routing should run as launches of its own).
+    uint32_t handoverGiveups(void *stream) {
+        uint32_t n = 0;
+        char *err = nullptr;
+        check(ffmoe_handover_giveups(c_.raw(), stream, &n, &err), err);
+        return n;
+    }
 
 private:
     Context &c_;
@@ -386,6 +407,29 @@ public:
         if (rowCount <= 0 || rowCount > maxGreedyRows) throw std::invalid_argument("rowCount outside 1...16");
         char *err = nullptr;
         check(ffmoe_matrix_gemv(mx_, stream, normedHidden, hiddenStrideElements, (uint32_t)rowCount, logits, logitsStrideElements, 1,
+                                &err), err);
+    }
+    // encodeGreedyRows with the chain's softcap and rowsConfidence (LMHeadChainInt4.swift:94-139 with `softcap`, the
+    // probability of the chosen token that argmax_rows_f32 leaves for the drafter: logit.metal:946-1010)
+    void encodeGreedyRowsWithConfidence(void *stream, const uint16_t *normedHidden, uint32_t hiddenStrideElements, int rowCount,
+                                        float softcap, uint32_t *outTokens, float *rowsConfidence) {
+        if (rowCount <= 0 || rowCount > maxGreedyRows) throw std::invalid_argument("rowCount outside 1...16");
+        char *err = nullptr;
+        check(ffmoe_matrix_greedy_conf(mx_, stream, normedHidden, hiddenStrideElements, (uint32_t)rowCount, softcap, outTokens,
+                                       rowsConfidence, &err), err);
+    }
+    // encodeHotGreedyRows (LMHeadChainInt4.swift:143-178): the greedy choice among the `count` listed rows of the head
+    // in the reference layout (weights / scales / biases / ids in DEVICE memory, as DequantInt4GEMV.encodeRowsListed takes them). outIndices
+    // are positions in `ids`, as the reference's argmax leaves them; rowsLogits is the chain's [rowCount][count] scratch.
+    static void encodeHotGreedyRows(Context &c, void *stream, const uint16_t *normedHidden, uint32_t hiddenStrideElements,
+                                    int rowCount, const uint32_t *ids, uint32_t count, const uint8_t *weights,
+                                    const uint16_t *scales, const uint16_t *biases, uint32_t d, float softcap, float *rowsLogits,
+                                    uint32_t *outIndices, float *rowsConfidence) {
+        if (rowCount <= 0 || rowCount > maxGreedyRows || count == 0) throw std::invalid_argument("rowCount outside 1...16 or an empty table");
+        char *err = nullptr;
+        check(ffmoe_gemv_int4_listed(c.raw(), stream, weights, scales, biases, ids, normedHidden, rowsLogits, count, d,
+                                     (uint32_t)rowCount, hiddenStrideElements, count, &err), err);
+        check(ffmoe_argmax_rows(c.raw(), stream, rowsLogits, count, (uint32_t)rowCount, count, softcap, outIndices, rowsConfidence,
                                 &err), err);
     }
     uint32_t vocab() const { return vocab_; }
@@ -542,6 +586,22 @@ public:
     void encode(void *stream, const uint16_t *h2, const uint16_t *h1, uint16_t *hidden, const uint16_t *postFFN2Weight,
                 const uint16_t *postFFNWeight, uint32_t d, float eps, float layerScalar) {
         PrefillLayerTail::encode(stream, h2, h1, hidden, postFFN2Weight, postFFNWeight, 1, d, d, d, d, eps, layerScalar);
+    }
+    // The tail on the rows MoE::encodeRouterAndRoutedExperts left un-combined (y = nullptr there): the routed experts'
+    // weighted combine (prefill.metal:544-565) happens while this launch loads its inputs
+    void encodeRouted(void *stream, const uint16_t *routeWeights, const uint16_t *h1, uint16_t *hidden, const uint16_t *postFFN2Weight,
+                      const uint16_t *postFFNWeight, int rows, float eps, float layerScalar) {
+        char *err = nullptr;
+        const uint32_t d = c_.shape().d;
+        check(ffmoe_layer_tail_routed(c_.raw(), stream, routeWeights, h1, d, hidden, d, postFFN2Weight, postFFNWeight, (uint32_t)rows,
+                                      eps, layerScalar, &err), err);
+    }
+    // ... and on the rows MoE::encodeRouterRoutedAndSharedExperts left in the two contexts (h1 = the shared expert's row)
+    void encodeRoutedShared(void *stream, Context &shared, const uint16_t *routeWeights, uint16_t *hidden,
+                            const uint16_t *postFFN2Weight, const uint16_t *postFFNWeight, int rows, float eps, float layerScalar) {
+        char *err = nullptr;
+        check(ffmoe_layer_tail_routed_shared(c_.raw(), shared.raw(), stream, routeWeights, hidden, c_.shape().d, postFFN2Weight,
+                                             postFFNWeight, (uint32_t)rows, eps, layerScalar, &err), err);
     }
     // encodeWithNorms (FusedLayerTail.swift:74-117): h1 before its post-FFN-1 norm; nextInputNorm / nextNormed
     // may both be null (no next layer)

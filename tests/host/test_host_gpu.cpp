@@ -219,6 +219,43 @@ int main() {
         bool threwRows = false;
         try { head.encodeGreedyRows(stream, dx, d, 17, dTok); } catch (const std::invalid_argument &) { threwRows = true; }
         EXPECT(threwRows);
+        // the same choice with the winner's probability (softmax of the row's logits, no softcap): same tokens, and
+        // the probability the fp64 softmax of the CPU logits gives
+        float *dConf = nullptr, *dLogits = nullptr;
+        uint32_t *dTok2 = nullptr, *dIds = nullptr;
+        HIP(hipMalloc(reinterpret_cast<void **>(&dConf), 4 * sizeof(float)));
+        HIP(hipMalloc(reinterpret_cast<void **>(&dTok2), 4 * sizeof(uint32_t)));
+        head.encodeGreedyRowsWithConfidence(stream, dx, d, 3, 0.0f, dTok2, dConf);
+        HIP(hipStreamSynchronize(stream));
+        EXPECT(toHost(dTok2, 3) == tok);
+        auto conf = toHost(dConf, 3);
+        // the hot-vocabulary form over eight listed rows of the table: position of the best listed row
+        const std::vector<uint32_t> ids = {60, 5, 33, 9, 17, 41, 2, 50};
+        dIds = toDevice(ids);
+        HIP(hipMalloc(reinterpret_cast<void **>(&dLogits), 3 * ids.size() * sizeof(float)));
+        // (the listed projection reads the table where it lies: the device copy of the blob)
+        LMHeadChainInt4::encodeHotGreedyRows(ctx, stream, dx, d, 3, dIds, (uint32_t)ids.size(), dPool + off.gate_w,
+                                             reinterpret_cast<uint16_t *>(dPool + off.gate_s),
+                                             reinterpret_cast<uint16_t *>(dPool + off.gate_b), d, 0.0f, dLogits, dTok2, dConf);
+        HIP(hipStreamSynchronize(stream));
+        auto hot = toHost(dTok2, 3);
+        for (int r = 0; r < 3; ++r) {
+            std::vector<float> xr(d), ref(f);
+            for (int i = 0; i < d; ++i) xr[i] = ffo_bf16_to_float(x[(size_t)r * d + i]);
+            ffo_gemv_int4_ref(pool.data() + off.gate_w, reinterpret_cast<uint16_t *>(pool.data() + off.gate_s),
+                              reinterpret_cast<uint16_t *>(pool.data() + off.gate_b), f, d, xr.data(), ref.data());
+            double sum = 0;
+            for (int i = 0; i < f; ++i) sum += std::exp((double)ref[i] - (double)ref[tok[r]]);
+            EXPECT(std::fabs(conf[r] - 1.0 / sum) <= 2e-3 * (1.0 / sum) + 1e-6);
+            uint32_t best = 0;
+            for (size_t i = 1; i < ids.size(); ++i)
+                if (ref[ids[i]] > ref[ids[best]]) best = (uint32_t)i;
+            EXPECT(hot[r] == best);
+        }
+        HIP(hipFree(dConf));
+        HIP(hipFree(dTok2));
+        HIP(hipFree(dIds));
+        HIP(hipFree(dLogits));
         HIP(hipFree(dTok));
     }
 
@@ -437,6 +474,55 @@ int main() {
         HIP(hipFree(dA));
         HIP(hipFree(dB));
         EXPECT(std::system(("rm -rf " + root).c_str()) == 0);
+    }
+
+    // --- the MoE block of a 5-row verify step three ways: the separate operators (router + routed experts, shared
+    // expert, tail); the routed rows left un-combined for the tail; the shared expert inside the routed experts'
+    // launches as well. Same routes; the same hidden rows bit for bit (first two) and to the shared row's rounding ---
+    {
+        const int R = 5;
+        ffmoe_shape denseShape{(uint32_t)d, (uint32_t)f, 1, 1, 1, 16};
+        Context dense(0, denseShape);
+        const uint8_t *blob = pool.data() + 3 * stride;
+        auto u16 = [&](uint32_t o) { return reinterpret_cast<const uint16_t *>(blob + o); };
+        PrefillSharedExpert shared(dense);
+        shared.load(0, SharedExpertProjection{blob + off.gate_w, u16(off.gate_s), u16(off.gate_b), (uint32_t)f, (uint32_t)d},
+                    SharedExpertProjection{blob + off.up_w, u16(off.up_s), u16(off.up_b), (uint32_t)f, (uint32_t)d},
+                    SharedExpertProjection{blob + off.down_w, u16(off.down_s), u16(off.down_b), (uint32_t)d, (uint32_t)f});
+        std::vector<uint16_t> hid((size_t)R * d), w3(d), w4(d);
+        for (auto &b : hid) b = ffo_bf16_bits(ffo_splitmix64_uniform(&rng, -2.f, 2.f));
+        for (auto &b : w3) b = ffo_bf16_bits(ffo_splitmix64_uniform(&rng, 0.5f, 1.5f));
+        for (auto &b : w4) b = ffo_bf16_bits(ffo_splitmix64_uniform(&rng, 0.5f, 1.5f));
+        uint16_t *dHidA = toDevice(hid), *dHidB = toDevice(hid), *dHidC = toDevice(hid), *dW3 = toDevice(w3), *dW4 = toDevice(w4);
+        uint16_t *dY = nullptr, *dH1 = nullptr, *dWA = nullptr, *dWB = nullptr, *dWC = nullptr;
+        uint32_t *dIA = nullptr, *dIB = nullptr, *dIC = nullptr;
+        for (auto p : {&dY, &dH1}) HIP(hipMalloc(reinterpret_cast<void **>(p), (size_t)R * d * 2));
+        for (auto p : {&dWA, &dWB, &dWC}) HIP(hipMalloc(reinterpret_cast<void **>(p), (size_t)R * K * 2));
+        for (auto p : {&dIA, &dIB, &dIC}) HIP(hipMalloc(reinterpret_cast<void **>(p), (size_t)R * K * 4));
+        MoE block(ctx);
+        PrefillLayerTail tail(ctx);
+        FusedLayerTail fused(ctx);
+        block.encodeRouterAndRoutedExperts(stream, 0, dx, d, dx, d, R, nullptr, dY, dIA, dWA);
+        shared.encodeBlock(stream, 0, dx, dH1, R, d, f, d, d);
+        tail.encode(stream, dY, dH1, dHidA, dW3, dW4, R, d, d, d, d, 1e-6f, 0.875f);
+        block.encodeRouterAndRoutedExperts(stream, 0, dx, d, dx, d, R, nullptr, nullptr, dIB, dWB);
+        fused.encodeRouted(stream, dWB, dH1, dHidB, dW3, dW4, R, 1e-6f, 0.875f);
+        block.encodeRouterRoutedAndSharedExperts(stream, dense, 0, 0, dx, d, dx, d, dx, d, R, dIC, dWC);
+        fused.encodeRoutedShared(stream, dense, dWC, dHidC, dW3, dW4, R, 1e-6f, 0.875f);
+        HIP(hipStreamSynchronize(stream));
+        EXPECT(toHost(dIA, (size_t)R * K) == toHost(dIB, (size_t)R * K) && toHost(dIA, (size_t)R * K) == toHost(dIC, (size_t)R * K));
+        EXPECT(toHost(dWA, (size_t)R * K) == toHost(dWB, (size_t)R * K) && toHost(dWA, (size_t)R * K) == toHost(dWC, (size_t)R * K));
+        const auto hA = toHost(dHidA, (size_t)R * d), hB = toHost(dHidB, (size_t)R * d), hC = toHost(dHidC, (size_t)R * d);
+        EXPECT(hA == hB);
+        std::vector<float> refA(hA.size());
+        for (size_t i = 0; i < hA.size(); ++i) refA[i] = ffo_bf16_to_float(hA[i]);
+        double relC, cosC;
+        errorStats(hC, refA, relC, cosC);
+        EXPECT(relC <= 1e-2 && cosC >= 0.9999);
+        EXPECT(hA != hid);
+        EXPECT(block.handoverGiveups(stream) == 0);
+        for (auto p : {dHidA, dHidB, dHidC, dW3, dW4, dY, dH1, dWA, dWB, dWC}) HIP(hipFree(p));
+        for (auto p : {dIA, dIB, dIC}) HIP(hipFree(p));
     }
 
     std::printf(failures ? "%d FAILURES\n" : "host gpu ok\n", failures);
