@@ -205,6 +205,7 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     if (e == hipSuccess)
         e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.acts),
                       ((size_t)ctx->max_pairs / 16 + ctx->pf.max_tiles + 2) * 16 * shape->f * sizeof(uint16_t));
+    ctx->pf.act_blocks = ctx->max_pairs / 16 + ctx->pf.max_tiles + 2;
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.partials), (size_t)ctx->max_pairs * shape->d * sizeof(uint16_t));
     if (e == hipSuccess && shape->n_experts == 1 && shape->top_k == 1) {
         e = hipMalloc(reinterpret_cast<void **>(&ctx->dense_idx), (size_t)router_rows * sizeof(uint32_t));
@@ -245,7 +246,7 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (ctx->pf.sorted_out_row) (void)hipFree(ctx->pf.sorted_out_row);
     if (ctx->pf.acts) (void)hipFree(ctx->pf.acts);
     if (ctx->pf.partials) (void)hipFree(ctx->pf.partials);
-    if (ctx->pf.x16) (void)hipFree(ctx->pf.x16);
+    if (ctx->pf.act_scale) (void)hipFree(ctx->pf.act_scale);
     if (ctx->dense_idx) (void)hipFree(ctx->dense_idx);
     if (ctx->dense_w) (void)hipFree(ctx->dense_w);
     // matrices that outlive their context lose their device memory here; the handles stay valid to destroy
@@ -645,7 +646,7 @@ int ffmoe_prefill_dump_tiles(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint3
     const size_t need = (size_t)prefill_dump_fragments(ctx->geom, gate_up != 0) * 64 * sizeof(uint4);
     if (out_bytes < need) return fail(err, FFMOE_ERR_INVALID, "output holds %zu bytes, the fragments take %zu", out_bytes, need);
     FF_HIP(launch_prefill_dump_tiles(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
-                                     expert, gate_up != 0, ctx->pf, out));
+                                     expert, gate_up != 0, ctx->pf, out, ctx->f16));
     return FFMOE_OK;
 }
 
@@ -772,11 +773,10 @@ int ffmoe_set_activation_dtype(ffmoe_ctx *ctx, int dtype, char **err) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (dtype != FFMOE_BF16 && dtype != FFMOE_FP16) return fail(err, FFMOE_ERR_INVALID, "activation dtype %d is neither FFMOE_BF16 nor FFMOE_FP16", dtype);
     const bool f16 = dtype == FFMOE_FP16;
-    if (f16 && !ctx->pf.x16) {
-        // the prefill GEMMs run on bf16 tiles: room for the converted input rows of the largest chunk
-        const uint32_t cap = ctx->shape.max_tokens > FFMOE_MAX_VERIFY_ROWS ? ctx->shape.max_tokens : FFMOE_MAX_VERIFY_ROWS;
-        hipError_t e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.x16), (size_t)cap * ctx->shape.d * sizeof(uint16_t));
-        if (e != hipSuccess) return fail(err, FFMOE_ERR_ALLOC, "hipMalloc of the FP16 conversion rows: %s", hipGetErrorString(e));
+    if (f16 && !ctx->pf.act_scale) {
+        // the FP16 prefill keeps its activations FP16 with a power-of-two scale per pair and 64-wide block of F
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&ctx->pf.act_scale), (size_t)ctx->pf.act_blocks * 16 * (ctx->geom.gf + 1) * sizeof(float));
+        if (e != hipSuccess) return fail(err, FFMOE_ERR_ALLOC, "hipMalloc of the FP16 activation scales: %s", hipGetErrorString(e));
     }
     if (ctx->dense_w) {
         // the dense FFN's unit route weights follow the type

@@ -113,7 +113,8 @@ struct PrefillScratch {
     uint32_t *sorted_out_row;   // [max pairs]: token * top_k + rank
     uint16_t *acts;             // [max pairs][F] bf16
     uint16_t *partials;         // [max pairs][D] 16-bit (used when the caller wants the combined output)
-    uint16_t *x16;              // [max tokens][D] bf16: the input rows of a context in FP16 mode, converted (else null)
+    float *act_scale;           // FP16 prefill: [act_blocks][F / 64][16] block scales of the activations, then [act_blocks][16] the pairs' largest (a context in FP16 mode; else null)
+    uint32_t act_blocks;        // 16-pair blocks `acts` holds
 };
 
 struct RouterWeights {
@@ -213,7 +214,7 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
 // stream and k = 32 * (k-half) + 8 * (l / 16) .. + 7 of the group.
 uint32_t prefill_dump_fragments(const ArenaGeom &g, bool gate_up);
 hipError_t launch_prefill_dump_tiles(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t expert, bool gate_up,
-                                     PrefillScratch sc, void *dump);
+                                     PrefillScratch sc, void *dump, bool f16 = false);
 
 // epilogue.hip: row-wise steps either side of the MoE stage
 hipError_t launch_post_attn_setup(hipStream_t s, uint16_t *hidden, uint32_t hidden_stride, const uint16_t *attn,

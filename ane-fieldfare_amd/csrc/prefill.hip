@@ -266,6 +266,7 @@ struct GemmWave {
     const uint8_t *w_tiles, *w_scales;    // this wave's arena tile row
     const uint16_t *a;                    // A matrix
     uint32_t a_stride, n_groups, n_arena_tiles, nb, wave, lane;
+    uint32_t act_blocks;                  // 16-pair blocks the activation buffer holds (the scale tables' extent)
     uint32_t act_block0;                  // first 16-pair block of this M-tile in the activation layout
     PrefillTile tile;
 };
@@ -274,11 +275,17 @@ struct GemmWave {
 // sequence has no branches, so the scheduler can interleave it with the expansion of the next tile).
 // DUMP: a test instantiation that also copies every weight fragment out of LDS, read exactly as the matrix
 // instructions read it, so that a test can hold the expanded tile itself against the reference's 16-bit weight.
-template <bool GATE_UP, int NMB, bool OUT_F16, bool DUMP = false>
+// F16: the reference's FP16 prefill (prefill.metal:581-598,685-702,723-777): FP16 rows against FP16 tile weights
+// half(fma(q, scale, bias)), fp32 sums; the activations between the two GEMMs are FP16 with a power-of-two scale per
+// pair and 64-wide block of F (`act_scale[pair][block]`; the block's largest magnitude lands below 2^14), so values
+// past FP16's range keep FP16's relative precision; the down GEMM brings every block of a pair to the pair's largest
+// scale as it takes it in (exact unless a value falls below FP16's normal range relative to that largest) and
+// applies that scale to the pair's sums.
+template <bool GATE_UP, int NMB, bool F16, bool DUMP = false>
 __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g, uint4 (*wb)[kTilesPerBlock][2][2][kWave],
                                           const uint32_t *__restrict__ sorted_token,
                                           const uint32_t *__restrict__ sorted_out_row, uint16_t *__restrict__ out,
-                                          uint4 *__restrict__ dump = nullptr) {
+                                          float *__restrict__ act_scale, uint4 *__restrict__ dump = nullptr) {
     constexpr int NA = NMB > 0 ? NMB : 1;
     const uint32_t lane = gw.lane, wave = gw.wave, j = lane & 15, jq = lane >> 4;
     const uint32_t n_groups = gw.n_groups;
@@ -300,14 +307,31 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     }
     // MFMA layout: lane (j, jq) needs row j, chunk jq = what load-layout lane 4 j + ((jq + 2 (j / 8)) % 4) holds
     const int pull = (int)((4 * j + ((jq + 2 * (j >> 3)) & 3)) * 4);
-    auto to_frag = [&](const uint4 &v) {
-        if (!GATE_UP) return __builtin_bit_cast(bf16x8, v);      // already in operand order
+    // FP16 down GEMM: the pair a lane holds in row block i (operand lane (j, jq) = pair j of the block), its largest
+    // block scale and the reciprocal (powers of two: exact)
+    // FP16: the block scales are laid out like the activations - act_scale[(16-pair block * groups of F + group) * 16 + j],
+    // pair j of the block - so a lane's address is a wave-uniform base plus 4 j. The down GEMM finds them already
+    // divided by the pair's largest (prefill_pair_scale_kernel ran in between: powers of two <= 1), and the largest
+    // itself in a second table behind the first, [block * 16 + j].
+    auto scale_at = [&](int i, uint32_t grp) { return ((size_t)(gw.act_block0 + wave + 4 * i) * g.gf + grp) * 16 + j; };
+    auto to_frag = [&](const uint4 &v, float rel) {
+        if (!GATE_UP) {                                           // already in operand order
+            if constexpr (!F16) return v;
+            const _Float16 r = (_Float16)rel;
+            const f16x2 r2 = {r, r};
+            uint4 o;
+            o.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, v.x) * r2);
+            o.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, v.y) * r2);
+            o.z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, v.z) * r2);
+            o.w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, v.w) * r2);
+            return o;
+        }
         uint4 r;
         r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x);
         r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y);
         r.z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z);
         r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w);
-        return __builtin_bit_cast(bf16x8, r);
+        return r;
     };
     f32x4 acc[NA][2 * kTilesPerBlock];
 #pragma unroll
@@ -317,7 +341,7 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
 
     // this wave's packed tile of the next kSlots groups to expand, in flight: group g waits in slot g % kSlots
     // (one slot where the row blocks leave no registers for a second: the steps are long enough there)
-    constexpr int kSlots = (GATE_UP && NMB >= 4) ? 1 : 2;
+    constexpr int kSlots = ((GATE_UP || F16) && NMB >= 4) ? 1 : 2;      // (the FP16 down GEMM carries the pairs' block scales besides)
     uint4 wraw[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
     uint2 sraw[2] = {{0, 0}, {0, 0}};
     auto load_b = [&](uint32_t grp, int slot) {
@@ -342,29 +366,36 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
             // even / odd nibbles as bytes; the empty asm keeps the masks as written (one v_cvt_f32_ubyteN per byte)
             lo = wcur[c] & 0x0F0F0F0Fu, hi = (wcur[c] >> 4) & 0x0F0F0F0Fu;
             asm("" : "+v"(lo), "+v"(hi));
-            ex.x = pack_bf16x2(__builtin_fmaf((float)(lo & 0xFFu), s_, b_), __builtin_fmaf((float)((lo >> 16) & 0xFFu), s_, b_));
+            ex.x = Act<F16>::pack(__builtin_fmaf((float)(lo & 0xFFu), s_, b_), __builtin_fmaf((float)((lo >> 16) & 0xFFu), s_, b_));
         } else if (q == 1) {
-            ex.y = pack_bf16x2(__builtin_fmaf((float)(hi & 0xFFu), s_, b_), __builtin_fmaf((float)((hi >> 16) & 0xFFu), s_, b_));
+            ex.y = Act<F16>::pack(__builtin_fmaf((float)(hi & 0xFFu), s_, b_), __builtin_fmaf((float)((hi >> 16) & 0xFFu), s_, b_));
         } else if (q == 2) {
-            ex.z = pack_bf16x2(__builtin_fmaf((float)((lo >> 8) & 0xFFu), s_, b_), __builtin_fmaf((float)(lo >> 24), s_, b_));
+            ex.z = Act<F16>::pack(__builtin_fmaf((float)((lo >> 8) & 0xFFu), s_, b_), __builtin_fmaf((float)(lo >> 24), s_, b_));
         } else {
-            ex.w = pack_bf16x2(__builtin_fmaf((float)((hi >> 8) & 0xFFu), s_, b_), __builtin_fmaf((float)(hi >> 24), s_, b_));
+            ex.w = Act<F16>::pack(__builtin_fmaf((float)((hi >> 8) & 0xFFu), s_, b_), __builtin_fmaf((float)(hi >> 24), s_, b_));
             wb[buf][wave][c >> 1][c & 1][lane] = ex;
         }
     };
     uint4 araw[NA][2];      // A in load layout, in flight: [.][0] k-half 0, [.][1] k-half 1
-    bf16x8 af[NA][2];       // A as MFMA fragments
+    uint4 af[NA][2];        // A as MFMA fragments
+    float ablock[NA][2];    // FP16 down GEMM: the block scale of the group araw[.][half] belongs to
     auto load_a = [&](uint32_t grp, int half) {
         if (NMB == 0) return;
 #pragma unroll
-        for (int i = 0; i < NA; ++i)
+        for (int i = 0; i < NA; ++i) {
             araw[i][half] = GATE_UP ? *reinterpret_cast<const uint4 *>(arow[i] + grp * kGroup + 32 * half)
                                     : *reinterpret_cast<const uint4 *>(arow[i] + (size_t)(grp * 2 + half) * (kWave * 8));
+            if constexpr (F16 && !GATE_UP) ablock[i][half] = act_scale[scale_at(i, grp)];
+        }
     };
     auto frag_a = [&](int half) {
         if (NMB == 0) return;
 #pragma unroll
-        for (int i = 0; i < NA; ++i) af[i][half] = to_frag(araw[i][half]);
+        for (int i = 0; i < NA; ++i) {
+            float rel = 1.0f;
+            if constexpr (F16 && !GATE_UP) rel = ablock[i][half];
+            af[i][half] = to_frag(araw[i][half], rel);
+        }
     };
     // One 64-wide group = 16 units; unit u multiplies weight fragment (nf = u % 8, k-half u / 8) with the NA
     // row blocks, and is followed by one piece of the next group's expansion, so the matrix pipe and the
@@ -410,12 +441,11 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
         for (int u = 0; u < 16; ++u) {
             if (NMB > 0) {
                 if (u + 2 < 16) read_b(u + 2);
-                const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bq[u % 3]);
 #pragma unroll
                 for (int i = 0; i < NA; ++i)
                     // weights as the first operand: the lane ends up with four consecutive weight rows of
                     // one pair, which the epilogue packs into one 8-byte piece of that pair's output row
-                    acc[i][u & 7] = mfma16(bfrag, af[i][u >> 3], acc[i][u & 7]);
+                    acc[i][u & 7] = Act<F16>::mfma(bq[u % 3], af[i][u >> 3], acc[i][u & 7]);
             }
             if (kExpand) expand_piece((buf + 2) & 3, u);
             __builtin_amdgcn_sched_barrier(0);
@@ -479,13 +509,35 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
             // of it, this lane the four values from k = 16 tl + 4 jq: k-half tl / 2, operand lane (j, 2 (tl % 2) + jq / 2),
             // values 4 (jq % 2) .. + 3 of that lane's eight
             uint16_t *oblk = out + ((size_t)(gw.act_block0 + wave + 4 * i) * g.gf + gw.nb) * 2 * (kWave * 8);
+            float h[kTilesPerBlock][4];
+#pragma unroll
+            for (int tl = 0; tl < kTilesPerBlock; ++tl)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) h[tl][r] = gelu_tanh_fast(acc[i][2 * tl][r]) * acc[i][2 * tl + 1][r];
+            if constexpr (F16) {
+                // the pair's 64 activations of this block sit in the four lanes (j, 0..3), sixteen each: their
+                // largest magnitude peak < 2^e goes to 2^14 (frexp / ldexp as prefill.metal:689-702)
+                float peak = 0.0f;
+#pragma unroll
+                for (int tl = 0; tl < kTilesPerBlock; ++tl)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) peak = fmaxf(peak, fabsf(h[tl][r]));
+                peak = fmaxf(peak, __shfl_xor(peak, 16, 64));
+                peak = fmaxf(peak, __shfl_xor(peak, 32, 64));
+                int e = 0;
+                (void)frexpf(peak, &e);
+                e = max(e, -100);                                   // 2^(14 - e) stays finite for a block of denormal size
+                const float to_half = ldexpf(1.0f, 14 - e);
+#pragma unroll
+                for (int tl = 0; tl < kTilesPerBlock; ++tl)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) h[tl][r] *= to_half;
+                if (jq == 0) act_scale[scale_at(i, gw.nb)] = ldexpf(1.0f, e - 14);
+            }
 #pragma unroll
             for (int tl = 0; tl < kTilesPerBlock; ++tl) {
-                float h[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) h[r] = gelu_tanh_fast(acc[i][2 * tl][r]) * acc[i][2 * tl + 1][r];
                 uint16_t *dst = oblk + (tl >> 1) * (kWave * 8) + (((tl & 1) * 2 + (jq >> 1)) * 16 + j) * 8 + (jq & 1) * 4;
-                *reinterpret_cast<uint2 *>(dst) = make_uint2(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]));
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(Act<F16>::pack(h[tl][0], h[tl][1]), Act<F16>::pack(h[tl][2], h[tl][3]));
             }
         }
         return;
@@ -498,6 +550,11 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     uint8_t *stage = reinterpret_cast<uint8_t *>(wb) + wave * 16 * kStageRow;
     const uint32_t rsub = lane >> 4, chunk = lane & 15;                         // read side: row 4 p + rsub, columns 8 chunk ..
     const bool col_ok = gw.nb * kTilesPerBlock + (chunk >> 2) < gw.n_arena_tiles;
+    float pair_largest[NA];
+    if constexpr (F16) {
+#pragma unroll
+        for (int i = 0; i < NA; ++i) pair_largest[i] = act_scale[(size_t)gw.act_blocks * g.gf * 16 + (gw.act_block0 + wave + 4 * i) * 16 + j];
+    }
     uint32_t orow_idx[NA][4];
 #pragma unroll
     for (int i = 0; i < NA; ++i)
@@ -510,9 +567,13 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     for (int i = 0; i < NA; ++i) {
 #pragma unroll
         for (int nf = 0; nf < 2 * kTilesPerBlock; ++nf) {
-            const f32x4 v = acc[i][nf];
+            f32x4 v = acc[i][nf];
+            if constexpr (F16) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] *= pair_largest[i];      // the pair's sums back to their scale
+            }
             *reinterpret_cast<uint2 *>(stage + j * kStageRow + nf * 32 + 8 * jq) =
-                make_uint2(Act<OUT_F16>::pack(v[0], v[1]), Act<OUT_F16>::pack(v[2], v[3]));
+                make_uint2(Act<F16>::pack(v[0], v[1]), Act<F16>::pack(v[2], v[3]));
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -530,8 +591,8 @@ __device__ __forceinline__ void gemm_wave(const GemmWave &gw, const ArenaGeom &g
     }
 }
 
-// OUT_F16: the down projection's per-route rows leave as FP16 instead of bf16 (a context in FP16 mode)
-template <bool GATE_UP, bool OUT_F16 = false, bool DUMP = false>
+// F16: a context in FP16 mode - FP16 rows in, FP16 tiles, block-scaled FP16 activations, FP16 per-route rows out
+template <bool GATE_UP, bool F16 = false, bool DUMP = false>
 __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                               const PrefillPlan *__restrict__ plan,
                                                               const PrefillTile *__restrict__ tiles,
@@ -539,7 +600,8 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__r
                                                               const uint32_t *__restrict__ sorted_out_row,
                                                               const uint16_t *__restrict__ a, uint32_t a_stride,
                                                               uint16_t *__restrict__ out, uint32_t n_nblocks,
-                                                              bool nb_major, uint4 *__restrict__ dump = nullptr) {
+                                                              bool nb_major, float *__restrict__ act_scale, uint32_t act_blocks,
+                                                              uint4 *__restrict__ dump = nullptr) {
     __shared__ __align__(16) uint4 wb[4][kTilesPerBlock][2][2][kWave];   // [buffer][tile][stream][k-half][lane]: group g lives in buffer g % 4
 
     // Consecutive block ids go to consecutive XCDs. Many experts: all N-blocks of an M-tile share an XCD (its L2 holds
@@ -567,6 +629,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__r
     gw.a = a;
     gw.a_stride = a_stride;
     gw.act_block0 = gw.tile.row_start / 16 + ti;
+    gw.act_blocks = act_blocks;
     // the arena tile row this wave expands; past the last one it expands the last again (never stored)
     const uint32_t at = min(nb * kTilesPerBlock + gw.wave, gw.n_arena_tiles - 1);
     const uint8_t *expert_base = arena_layer + (size_t)gw.tile.expert * g.expert_bytes;
@@ -577,17 +640,37 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__r
     const uint32_t my_mb = n_mb > gw.wave ? (n_mb - gw.wave + 3) / 4 : 0;    // 16-row blocks of this wave
     if (DUMP) {
         // the test launch runs one pair: wave 0 owns its row block, the others only expand their tiles
-        if (my_mb) gemm_wave<GATE_UP, 1, OUT_F16, true>(gw, g, wb, sorted_token, sorted_out_row, out, dump);
-        else gemm_wave<GATE_UP, 0, OUT_F16, true>(gw, g, wb, sorted_token, sorted_out_row, out, dump);
+        if (my_mb) gemm_wave<GATE_UP, 1, F16, true>(gw, g, wb, sorted_token, sorted_out_row, out, act_scale, dump);
+        else gemm_wave<GATE_UP, 0, F16, true>(gw, g, wb, sorted_token, sorted_out_row, out, act_scale, dump);
         return;
     }
     switch (my_mb) {
-        case 0: gemm_wave<GATE_UP, 0, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
-        case 1: gemm_wave<GATE_UP, 1, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
-        case 2: gemm_wave<GATE_UP, 2, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
-        case 3: gemm_wave<GATE_UP, 3, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
-        default: gemm_wave<GATE_UP, 4, OUT_F16>(gw, g, wb, sorted_token, sorted_out_row, out); break;
+        case 0: gemm_wave<GATE_UP, 0, F16>(gw, g, wb, sorted_token, sorted_out_row, out, act_scale); break;
+        case 1: gemm_wave<GATE_UP, 1, F16>(gw, g, wb, sorted_token, sorted_out_row, out, act_scale); break;
+        case 2: gemm_wave<GATE_UP, 2, F16>(gw, g, wb, sorted_token, sorted_out_row, out, act_scale); break;
+        case 3: gemm_wave<GATE_UP, 3, F16>(gw, g, wb, sorted_token, sorted_out_row, out, act_scale); break;
+        default: gemm_wave<GATE_UP, 4, F16>(gw, g, wb, sorted_token, sorted_out_row, out, act_scale); break;
     }
+}
+
+// Between the two GEMMs of the FP16 prefill: a pair's block scales divided by its largest (powers of two: exact), the
+// largest itself stored behind the table at [n_pairs * blocks + pair] - what prefill_routed_down_tensorops computes per
+// threadgroup into `relative` and `pair_scale` (prefill.metal:731-741), done once per pair here.
+// One block per M-tile, one thread per pair of it.
+__global__ __launch_bounds__(kBM) void prefill_pair_scale_kernel(const PrefillPlan *__restrict__ plan,
+                                                                 const PrefillTile *__restrict__ tiles, uint32_t groups,
+                                                                 uint32_t act_blocks, float *__restrict__ act_scale) {
+    const uint32_t ti = blockIdx.x;
+    if (ti >= plan->n_tiles) return;
+    const PrefillTile tile = tiles[ti];
+    if (threadIdx.x >= tile.rows) return;
+    const uint32_t block = tile.row_start / 16 + ti + threadIdx.x / 16, j = threadIdx.x % 16;
+    float *s = act_scale + (size_t)block * groups * 16 + j;
+    float largest = 0.0f;
+    for (uint32_t b = 0; b < groups; ++b) largest = fmaxf(largest, s[b * 16]);
+    const float inv = 1.0f / largest;          // a scale is 2^(e - 14) with e >= -100: never zero
+    for (uint32_t b = 0; b < groups; ++b) s[b * 16] *= inv;
+    act_scale[(size_t)act_blocks * groups * 16 + block * 16 + j] = largest;
 }
 
 // h2[t][c] = bf16(sum_r w[t][r] * partial[t][r][c]) over the routes the sort kept, fma in rank order
@@ -640,21 +723,6 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(const uint16_t *__
     *reinterpret_cast<uint4 *>(y + (size_t)tok * d + c) = o;
 }
 
-// FP16 rows -> bf16 rows (round to nearest even), 8 elements per thread: a context in FP16 mode feeds the
-// gate/up GEMM, whose tiles are bf16, through this pass.
-__global__ __launch_bounds__(256) void rows_f16_to_bf16_kernel(const uint16_t *__restrict__ x, uint32_t x_stride, uint32_t d,
-                                                               uint16_t *__restrict__ out) {
-    const uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 8;
-    if (c >= d) return;
-    const uint4 q = *reinterpret_cast<const uint4 *>(x + (size_t)blockIdx.y * x_stride + c);
-    uint4 o;
-    o.x = pack_bf16x2(Act<true>::lo(q.x), Act<true>::hi(q.x));
-    o.y = pack_bf16x2(Act<true>::lo(q.y), Act<true>::hi(q.y));
-    o.z = pack_bf16x2(Act<true>::lo(q.z), Act<true>::hi(q.z));
-    o.w = pack_bf16x2(Act<true>::lo(q.w), Act<true>::hi(q.w));
-    *reinterpret_cast<uint4 *>(out + (size_t)blockIdx.y * d + c) = o;
-}
-
 // One pair of expert `expert` sent through the gate/up (or down) GEMM with the weight fragments copied out.
 __global__ void prefill_dump_plan_kernel(uint32_t expert, PrefillPlan *plan, PrefillTile *tiles, uint32_t *sorted_token,
                                          uint32_t *sorted_out_row) {
@@ -678,19 +746,22 @@ uint32_t prefill_dump_fragments(const ArenaGeom &g, bool gate_up) {
 }
 
 hipError_t launch_prefill_dump_tiles(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t expert, bool gate_up,
-                                     PrefillScratch sc, void *dump) {
+                                     PrefillScratch sc, void *dump, bool f16) {
+    if (f16 && !sc.act_scale) return hipErrorInvalidValue;
     hipLaunchKernelGGL(prefill_dump_plan_kernel, dim3(1), dim3(1), 0, s, expert, sc.plan, sc.tiles, sc.sorted_token,
                        sc.sorted_out_row);
     // the pair's input row is whatever row 0 of the scratch holds: only the weight side is looked at
+#define FFMOE_DUMP(GU, H, A, STRIDE, OUT, NB)                                                                              \
+    hipLaunchKernelGGL((prefill_gemm_kernel<GU, H, true>), dim3((NB) * 8), dim3(256), 0, s, arena_layer, g, sc.plan, sc.tiles,  \
+                       sc.sorted_token, sc.sorted_out_row, A, STRIDE, OUT, NB, false, sc.act_scale, sc.act_blocks, static_cast<uint4 *>(dump))
     if (gate_up) {
         const uint32_t nb = (g.gu_rb + kTilesPerBlock - 1) / kTilesPerBlock;
-        hipLaunchKernelGGL((prefill_gemm_kernel<true, false, true>), dim3(nb * 8), dim3(256), 0, s, arena_layer, g, sc.plan, sc.tiles,
-                           sc.sorted_token, sc.sorted_out_row, sc.partials, g.d, sc.acts, nb, false, static_cast<uint4 *>(dump));
+        if (f16) FFMOE_DUMP(true, true, sc.partials, g.d, sc.acts, nb); else FFMOE_DUMP(true, false, sc.partials, g.d, sc.acts, nb);
     } else {
         const uint32_t nb = (g.dn_rbp + kTilesPerBlock - 1) / kTilesPerBlock;
-        hipLaunchKernelGGL((prefill_gemm_kernel<false, false, true>), dim3(nb * 8), dim3(256), 0, s, arena_layer, g, sc.plan, sc.tiles,
-                           sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, sc.partials, nb, false, static_cast<uint4 *>(dump));
+        if (f16) FFMOE_DUMP(false, true, sc.acts, g.f, sc.partials, nb); else FFMOE_DUMP(false, false, sc.acts, g.f, sc.partials, nb);
     }
+#undef FFMOE_DUMP
     return hipGetLastError();
 }
 
@@ -729,26 +800,26 @@ hipError_t launch_prefill(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g
     const uint32_t tile_cap = min(sc.max_tiles, (src.n_items + kBM - 1) / kBM + n_experts);
     const uint32_t tile_slots = (tile_cap + 7) / 8 * 8;
     const uint32_t nb_gu = (g.gu_rb + kTilesPerBlock - 1) / kTilesPerBlock, nb_dn = (g.dn_rbp + kTilesPerBlock - 1) / kTilesPerBlock;
-    if (f16) {
-        // the GEMMs compute on bf16 tiles: FP16 inputs are rounded to bf16 once, outputs leave as FP16
-        if (!sc.x16) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(rows_f16_to_bf16_kernel, dim3((g.d / 8 + 255) / 256, t), dim3(256), 0, s, x, x_stride, g.d, sc.x16);
-        x = sc.x16;
-        x_stride = g.d;
-    }
+    if (f16 && !sc.act_scale) return hipErrorInvalidValue;      // allocated when the context was switched to FP16
     // grid: (N-blocks x tile slots) in either order of the kernel's block map
     const bool nb_major = n_experts == 1;
     auto grid_of = [&](uint32_t n_nblocks) { return nb_major ? 8 * ((n_nblocks + 7) / 8) * tile_cap : n_nblocks * tile_slots; };
-    hipLaunchKernelGGL(prefill_gemm_kernel<true>, dim3(grid_of(nb_gu)), dim3(256), 0, s, arena_layer, g, sc.plan,
-                       sc.tiles, sc.sorted_token, sc.sorted_out_row, x, x_stride, sc.acts, nb_gu, nb_major);
+    if (f16)
+        hipLaunchKernelGGL((prefill_gemm_kernel<true, true>), dim3(grid_of(nb_gu)), dim3(256), 0, s, arena_layer, g, sc.plan,
+                           sc.tiles, sc.sorted_token, sc.sorted_out_row, x, x_stride, sc.acts, nb_gu, nb_major, sc.act_scale, sc.act_blocks);
+    else
+        hipLaunchKernelGGL((prefill_gemm_kernel<true, false>), dim3(grid_of(nb_gu)), dim3(256), 0, s, arena_layer, g, sc.plan,
+                           sc.tiles, sc.sorted_token, sc.sorted_out_row, x, x_stride, sc.acts, nb_gu, nb_major, nullptr, 0u);
     timer->mark(s, FFMOE_K_PREFILL_GATE_UP);
     uint16_t *partials = partials_out ? partials_out : sc.partials;
     if (f16)
+        hipLaunchKernelGGL(prefill_pair_scale_kernel, dim3(tile_cap), dim3(kBM), 0, s, sc.plan, sc.tiles, g.gf, sc.act_blocks, sc.act_scale);
+    if (f16)
         hipLaunchKernelGGL((prefill_gemm_kernel<false, true>), dim3(grid_of(nb_dn)), dim3(256), 0, s, arena_layer, g, sc.plan,
-                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn, nb_major);
+                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn, nb_major, sc.act_scale, sc.act_blocks);
     else
         hipLaunchKernelGGL((prefill_gemm_kernel<false, false>), dim3(grid_of(nb_dn)), dim3(256), 0, s, arena_layer, g, sc.plan,
-                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn, nb_major);
+                           sc.tiles, sc.sorted_token, sc.sorted_out_row, sc.acts, g.f, partials, nb_dn, nb_major, nullptr, 0u);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     timer->mark(s, FFMOE_K_PREFILL_DOWN);

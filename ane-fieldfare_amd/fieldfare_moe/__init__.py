@@ -384,13 +384,14 @@ class Context:
 
     def prefill_tiles(self, layer: int, expert: int, which: int):
         """The 16-bit weights of one sub-tensor as the grouped GEMM's matrix instructions read them from LDS, put
-        back into [rows][cols] order: bf16 CUDA tensor (ffmoe_prefill_dump_tiles)."""
+        back into [rows][cols] order: a CUDA tensor of the context's activation type - bf16(fma(q, s, b)), or
+        half(fma(q, s, b)) for a context in FP16 mode (ffmoe_prefill_dump_tiles)."""
         import torch
         d, f = self.shape.d, self.shape.f
         gate_up = which != DOWN
         tiles, groups = (f // 16, d // GROUP) if gate_up else (d // 32, f // GROUP)
         nblocks = (tiles + 3) // 4
-        raw = torch.empty((nblocks, groups, 2, 4, 2, 4, 16, 8), dtype=torch.bfloat16, device=f"cuda:{self.device}")
+        raw = torch.empty((nblocks, groups, 2, 4, 2, 4, 16, 8), dtype=self.act, device=f"cuda:{self.device}")
         err = C.c_char_p()
         _check(self.L.ffmoe_prefill_dump_tiles(self._h, _stream(), layer, expert, int(gate_up), _ptr(raw),
                                                raw.numel() * 2, C.byref(err)), err)

@@ -540,7 +540,7 @@ def main():
             fp16["prefill_kernel_us"] = kernel_times(ctx.profile(reset=True))
             ctx.set_profiling(False)
             del xph, ih, wph, yph
-        fp16["note"] = "FFMOE_FP16: router, experts and combine on FP16 rows; the prefill converts its input rows to bf16 once"
+        fp16["note"] = "FFMOE_FP16: router, experts and combine on FP16 rows; the prefill multiplies FP16 rows by FP16 tiles and keeps block-scaled FP16 activations (the reference's FP16 prefill arithmetic)"
         extra["fp16_mode"] = fp16
         ctx.set_act_dtype("bf16")
 

@@ -454,14 +454,11 @@ int ffmoe_rmsnorm(ffmoe_ctx *ctx, void *stream, const uint16_t *x, uint32_t x_st
  * checkpoints). FFMOE_FP16 reproduces the reference's text path: the router reads FP16 rows exactly, the
  * decode / verify kernels multiply FP16 rows with the INT4 weights on the FP16 matrix instruction and
  * round where the reference rounds to FP16 (activations, per-route rows, outputs). The prefill GEMMs
- * (ffmoe_prefill, ffmoe_prefill_pairs, ffmoe_dense_ffn beyond 16 rows) are the exception: in FFMOE_FP16 they
- * COMPUTE ON BF16-ROUNDED INPUTS - the chunk's FP16 rows are rounded to bf16 once (8 significant bits instead of
- * FP16's 11), the tiles, the gating product and the activations stay bf16, and only the per-route rows and the
- * combined rows leave as FP16. That keeps the reference's range (no overflow where its FP16 tiles need the
- * power-of-two block scaling of Metal/Prefill/prefill.metal:593-598,685-702) and stays inside the 1e-2 /
- * cosine 0.9999 bar against the FP16 reference, but it is three mantissa bits narrower per input value than the
- * reference's own FP16 operand in that mode: a caller that needs the reference's FP16 prefill precision bit for
- * bit does not get it here. In FFMOE_FP16 input rows must be 16-byte aligned with strides
+ * (ffmoe_prefill, ffmoe_prefill_pairs, ffmoe_dense_ffn beyond 16 rows) follow the reference's FP16 tiles
+ * (Metal/Prefill/prefill.metal:581-598,685-702,723-777): FP16 rows against tile weights half(fma(q, scale, bias)), fp32
+ * sums, and the activations between the two GEMMs FP16 with a power-of-two scale per pair and 64-wide block of the
+ * intermediate size, so that values past FP16's range keep FP16's relative precision; the down GEMM brings a
+ * pair's blocks to the pair's largest scale as it reads them and applies that scale to the pair's sums. In FFMOE_FP16 input rows must be 16-byte aligned with strides
  * that are multiples of 8 wherever a call accepts less otherwise (router, GEMV). Set it before the
  * first compute call; switching waits for the device. May allocate (once). */
 int ffmoe_set_activation_dtype(ffmoe_ctx *ctx, int dtype, char **err);

@@ -126,7 +126,7 @@ def test_verify_fp16_against_oracle(small, real, oracle, torch, which, t):
 
 @pytest.mark.parametrize("which,t", [("small", 40), ("small", 300), ("real", 64)])
 def test_prefill_fp16_against_oracle(small, real, oracle, torch, which, t):
-    # prefill chunk in FP16 mode: rows rounded to bf16 once for the GEMMs, FP16 rows out
+    # prefill chunk in FP16 mode: FP16 rows against FP16 tiles, block-scaled FP16 activations, FP16 rows out
     fx = small if which == "small" else real
     rng = np.random.default_rng(1300 + t)
     xb = f16_bits(rng.uniform(-0.5, 0.5, (t, fx["d"])))
@@ -140,6 +140,61 @@ def test_prefill_fp16_against_oracle(small, real, oracle, torch, which, t):
     head = f16_float(bits_of(fx["ctx"].verify(0, f16_tensor(torch, xb[:8]), torch.from_numpy(idx[:8].astype(np.int32)).cuda(),
                                              f16_tensor(torch, wb[:8]))))
     assert rel_err(head, yf[:8]) < 1e-2
+
+
+def test_prefill_fp16_tiles_are_half_of_fma(small, real, oracle, ff, torch):
+    """The tile weights the FP16 prefill's matrix instructions read from LDS (copied out by the kernel itself) are the
+    reference's FP16 tile weights half(fma(q, scale, bias)) (prefill_mma_dequant32, prefill.metal:581-590), bit for bit:
+    q * scale is exact in fp32, so numpy's float32 product-and-sum rounded to float16 is that value."""
+    for fx, experts in ((small, (0, 15)), (real, (3,))):
+        for ex in experts:
+            for which, name in ((ff.GATE, "gate"), (ff.UP, "up"), (ff.DOWN, "down")):
+                got = fx["ctx"].prefill_tiles(0, ex, which)
+                assert got.dtype == torch.float16
+                W, S, B = fx["pool"].sub(ex, name)
+                rows, half_cols = W.shape
+                q = np.empty((rows, half_cols * 2), np.float32)
+                q[:, 0::2] = W & 0xF
+                q[:, 1::2] = W >> 4
+                sc = np.repeat(oracle.bf16_to_float(S), 64, axis=1)
+                bi = np.repeat(oracle.bf16_to_float(B), 64, axis=1)
+                want = (q * sc + bi).astype(np.float32).astype(np.float16).view(np.uint16)
+                assert np.array_equal(bits_of(got), want), (ex, name)
+
+
+def test_prefill_fp16_keeps_activations_past_half_range(oracle, ff, torch):
+    """Inputs large enough that gelu(gate) * up passes FP16's largest value (65,504) while the layer's outputs stay
+    inside it: the block-scaled FP16 activations (prefill.metal:593-598,685-702) carry them, so the rows are finite and
+    within the usual bar of the fp32 reference; stored as plain FP16 the activations would be infinite."""
+    d, f, e, t = 128, 64, 4, 48
+    g = oracle.seed_tree_key(0xF16, "prefill-fp16-range")
+    gates = [g.uniform(-0.5, 0.5, f * d).reshape(f, d) for _ in range(e)]
+    ups = [g.uniform(-0.5, 0.5, f * d).reshape(f, d) for _ in range(e)]
+    downs = [g.uniform(-0.004, 0.004, d * f).reshape(d, f) for _ in range(e)]
+    pool = oracle.pool_from_float(gates, ups, downs, align=16)
+    ctx = ff.Context(d, f, e, 2, n_layers=1, max_tokens=64, act_dtype="fp16")
+    ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
+    xb = f16_bits(g.uniform(-1.0, 1.0, t * d).reshape(t, d) * 160.0)
+    idx = np.stack([np.array([r % e, (r + 1) % e], np.uint32) for r in range(t)])
+    w = np.full((t, 2), 0.5, np.float32)
+    # the reference in float64 (the oracle's FP16 mode stores the activations as plain FP16: infinite here)
+    x = f16_float(xb)
+    ref = np.zeros((t, d), np.float64)
+    peak = 0.0
+    for r in range(t):
+        for k in range(2):
+            ex = int(idx[r, k])
+            gw_, uw_, dw_ = (oracle.dequantize_int4(*pool.sub(ex, name)).astype(np.float64) for name in ("gate", "up", "down"))
+            act = oracle.gelu_tanh((gw_ @ x[r]).astype(np.float32)).astype(np.float64) * (uw_ @ x[r])
+            peak = max(peak, float(np.abs(act).max()))
+            ref[r] += 0.5 * (dw_ @ act)
+    ref = ref.astype(np.float32)
+    assert peak > 2 * 65504.0 and np.abs(ref).max() < 3e4, (peak, np.abs(ref).max())
+    y = ctx.prefill(0, f16_tensor(torch, xb), torch.from_numpy(idx.astype(np.int32)).cuda(), f16_tensor(torch, f16_bits(w)))
+    yf = f16_float(bits_of(y))
+    assert np.isfinite(yf).all()
+    assert rel_err(yf, ref) < 1e-2 and cosine(yf, ref) > 0.9999, (rel_err(yf, ref), cosine(yf, ref))
+    ctx.close()
 
 
 def test_gemv_and_resident_matrix_fp16(ff, oracle, torch):
