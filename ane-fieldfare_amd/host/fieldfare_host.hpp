@@ -125,7 +125,11 @@ struct PrefillMoEGroupingError : std::runtime_error {
 };
 
 struct PrefillMoEGrouping {
-    // PrefillMoEGrouping.swift:49-110. Sort key: (expertSortKeys[expert] if given, expert, token, rank).
+    // The contract of PrefillMoEGrouping.groupTokenExpertPairs (PrefillMoEGrouping.swift:49-110): the pairs ordered by
+    // (expertSortKeys[expert] if given, expert, token, rank), one group per expert that has pairs, tiles of up to
+    // tileExpertCount consecutive groups. Built as a bucket pass rather than one comparison sort over all pairs: the
+    // experts are put in order once, every pair drops into its expert's bucket (two linear passes), and only the
+    // inside of a bucket is sorted - a no-op for pairs that arrive token-major, as makeTokenExpertPairs emits them.
     static PrefillMoEGroupedRoutes groupTokenExpertPairs(const std::vector<PrefillTokenExpertPair> &pairs, int queryCount,
                                                          int topK, int numExperts, int tileExpertCount,
                                                          const std::vector<uint64_t> *expertSortKeys = nullptr) {
@@ -133,35 +137,38 @@ struct PrefillMoEGrouping {
             throw std::invalid_argument("groupTokenExpertPairs: bad arguments");
         if (pairs.size() > (size_t)queryCount * (size_t)topK) throw std::invalid_argument("more pairs than queryCount * topK");
         if (expertSortKeys && expertSortKeys->size() != (size_t)numExperts) throw std::invalid_argument("expertSortKeys count mismatch");
-        for (const auto &p : pairs)
+        std::vector<uint32_t> bucketSize((size_t)numExperts, 0);
+        for (const auto &p : pairs) {
             if (p.expert >= (uint32_t)numExperts) throw PrefillMoEGroupingError(p.expert);
-        PrefillMoEGroupedRoutes out;
-        out.sortedPairs = pairs;
-        std::sort(out.sortedPairs.begin(), out.sortedPairs.end(),
-                  [&](const PrefillTokenExpertPair &a, const PrefillTokenExpertPair &b) {
-                      if (expertSortKeys) {
-                          const uint64_t ka = (*expertSortKeys)[a.expert], kb = (*expertSortKeys)[b.expert];
-                          if (ka != kb) return ka < kb;
-                      }
-                      if (a.expert != b.expert) return a.expert < b.expert;
-                      if (a.token != b.token) return a.token < b.token;
-                      return a.rank < b.rank;
-                  });
-        size_t i = 0;
-        while (i < out.sortedPairs.size()) {
-            const uint32_t expert = out.sortedPairs[i].expert;
-            const size_t start = i;
-            while (i < out.sortedPairs.size() && out.sortedPairs[i].expert == expert) ++i;
-            out.groups.push_back({expert, (uint32_t)start, (uint32_t)(i - start)});
+            ++bucketSize[p.expert];
         }
-        size_t groupStart = 0;
-        while (groupStart < out.groups.size()) {
-            const size_t groupEnd = std::min(out.groups.size(), groupStart + (size_t)tileExpertCount);
-            const auto &first = out.groups[groupStart];
-            const auto &last = out.groups[groupEnd - 1];
-            out.tiles.push_back({(uint32_t)groupStart, (uint32_t)(groupEnd - groupStart), first.pairStart,
-                                 last.pairStart + last.pairCount - first.pairStart});
-            groupStart = groupEnd;
+        // the experts in output order
+        std::vector<uint32_t> order((size_t)numExperts);
+        for (uint32_t e = 0; e < (uint32_t)numExperts; ++e) order[e] = e;
+        if (expertSortKeys)
+            std::stable_sort(order.begin(), order.end(),
+                             [&](uint32_t x, uint32_t y) { return (*expertSortKeys)[x] < (*expertSortKeys)[y]; });
+        // where each expert's bucket starts; a group per non-empty bucket
+        PrefillMoEGroupedRoutes out;
+        std::vector<uint32_t> cursor((size_t)numExperts, 0);
+        uint32_t filled = 0;
+        for (uint32_t e : order) {
+            cursor[e] = filled;
+            if (bucketSize[e]) out.groups.push_back({e, filled, bucketSize[e]});
+            filled += bucketSize[e];
+        }
+        out.sortedPairs.resize(pairs.size());
+        for (const auto &p : pairs) out.sortedPairs[cursor[p.expert]++] = p;
+        auto position = [](const PrefillTokenExpertPair &p) { return ((uint64_t)p.token << 32) | p.rank; };
+        for (const auto &g : out.groups) {
+            auto first = out.sortedPairs.begin() + g.pairStart, last = first + g.pairCount;
+            if (!std::is_sorted(first, last, [&](const auto &x, const auto &y) { return position(x) < position(y); }))
+                std::sort(first, last, [&](const auto &x, const auto &y) { return position(x) < position(y); });
+        }
+        for (size_t at = 0; at < out.groups.size(); at += (size_t)tileExpertCount) {
+            const size_t n = std::min((size_t)tileExpertCount, out.groups.size() - at);
+            const PrefillMoEGroup &head = out.groups[at], &tail = out.groups[at + n - 1];
+            out.tiles.push_back({(uint32_t)at, (uint32_t)n, head.pairStart, tail.pairStart + tail.pairCount - head.pairStart});
         }
         return out;
     }
