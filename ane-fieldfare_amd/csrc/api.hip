@@ -61,6 +61,10 @@ struct ffmoe_ctx {
     bool f16 = false;                // activations are FP16 (ffmoe_set_activation_dtype)
     KernelTimer timer;
     std::vector<ffmoe_matrix *> matrices;   // resident matrices created on this context and not yet destroyed
+    // the stream the scratch was last used on, and the event a call on another stream waits for (claim_scratch)
+    hipStream_t scratch_stream = nullptr;
+    bool scratch_claimed = false;
+    hipEvent_t scratch_event = nullptr;
 };
 
 // ---- scratch of ffmoe_verify_static: device memory that exists from the moment the library is loaded ----------
@@ -77,6 +81,10 @@ namespace {
 constexpr int kMaxDevices = 64;
 void *g_scratch_addr[kMaxDevices] = {};     // device address of `scratch` per device (its host-side name is no address)
 std::mutex g_scratch_mutex;
+// the stream that used a device's array last and the event a call on another stream waits for (claim_static_scratch)
+hipStream_t g_scratch_stream[kMaxDevices] = {};
+bool g_scratch_claimed[kMaxDevices] = {};
+hipEvent_t g_scratch_event[kMaxDevices] = {};
 
 // With `device` current: look the array's address on that device up once.
 hipError_t resolve_static_scratch(int device) {
@@ -85,8 +93,45 @@ hipError_t resolve_static_scratch(int device) {
     if (g_scratch_addr[device]) return hipSuccess;
     void *p = nullptr;
     const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e == hipSuccess) g_scratch_addr[device] = p;
+    if (e == hipSuccess) {
+        g_scratch_addr[device] = p;
+        if (hipEventCreateWithFlags(&g_scratch_event[device], hipEventDisableTiming) != hipSuccess) {
+            g_scratch_event[device] = nullptr;
+            (void)hipGetLastError();
+        }
+    }
     return e;
+}
+
+// Stream hand-over of one piece of scratch: `last` used it, `s` wants it. With `s` or `last` under graph capture, or
+// `last` gone, nothing is done. Returns whether `s` now owns it.
+bool hand_over(hipStream_t last, bool claimed, hipEvent_t event, hipStream_t s) {
+    hipStreamCaptureStatus now = hipStreamCaptureStatusNone, before = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &now) != hipSuccess || now != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (claimed && event) {
+        // the previous stream may be gone by now (its owner destroyed it): then there is nothing left to wait for
+        if (hipStreamIsCapturing(last, &before) == hipSuccess && before == hipStreamCaptureStatusNone &&
+            hipEventRecord(event, last) == hipSuccess)
+            (void)hipStreamWaitEvent(s, event, 0);
+        (void)hipGetLastError();
+    }
+    return true;
+}
+
+// The static array serves every context on its GPU: the same stream-to-stream ordering as a context's own scratch
+// (claim_scratch below), kept per device. Allocates nothing: the event exists since the address was looked up.
+void claim_static_scratch(int device, void *stream) {
+    if (device < 0 || device >= kMaxDevices) return;
+    const hipStream_t s = static_cast<hipStream_t>(stream);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_claimed[device] && g_scratch_stream[device] == s) return;
+    if (hand_over(g_scratch_stream[device], g_scratch_claimed[device], g_scratch_event[device], s)) {
+        g_scratch_stream[device] = s;
+        g_scratch_claimed[device] = true;
+    }
 }
 
 int fail(char **err, int code, const char *fmt, ...) {
@@ -111,6 +156,21 @@ int check_ctx(ffmoe_ctx *ctx, char **err) {
     if (!ctx) return fail(err, FFMOE_ERR_INVALID, "null context");
     FF_HIP(hipSetDevice(ctx->device));
     return FFMOE_OK;
+}
+
+// The context's scratch (plan, activation rows, un-weighted rows, hand-over words, sort tables) serves one stream at a
+// time. Calls on the stream that used it last cost nothing here; a call that arrives on ANOTHER stream first makes that
+// stream wait, on the device, for everything the previous stream has been given, so that two streams sharing a
+// context run one call after the other instead of racing for the scratch. (Streams under graph capture are left
+// alone: a capture orders its own nodes, and an event from outside may not enter it.) Host threads are a different
+// matter: a context is for one host thread at a time.
+void claim_scratch(ffmoe_ctx *ctx, void *stream) {
+    const hipStream_t s = static_cast<hipStream_t>(stream);
+    if (ctx->scratch_claimed && ctx->scratch_stream == s) return;
+    if (hand_over(ctx->scratch_stream, ctx->scratch_claimed, ctx->scratch_event, s)) {
+        ctx->scratch_stream = s;
+        ctx->scratch_claimed = true;
+    }
 }
 
 int check_layer(ffmoe_ctx *ctx, uint32_t layer, bool need_experts, bool need_router, char **err) {
@@ -165,6 +225,10 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
         ctx->n_cus = (uint32_t)cus;
     }
     ctx->route_resident_blocks = route_launch_resident_blocks(ctx->n_cus);
+    if (hipEventCreateWithFlags(&ctx->scratch_event, hipEventDisableTiming) != hipSuccess) {
+        ctx->scratch_event = nullptr;      // without it calls on different streams are the caller's to order, as documented
+        (void)hipGetLastError();
+    }
     ctx->shape = *shape;
     ctx->geom = make_geom(shape->d, shape->f);
     // an expert's tile regions are addressed through buffer descriptors with 32-bit sizes and offsets
@@ -258,6 +322,7 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
         mx->partials = nullptr;
         mx->ctx = nullptr;
     }
+    if (ctx->scratch_event) (void)hipEventDestroy(ctx->scratch_event);
     for (auto &ev : ctx->timer.ev)
         if (ev) (void)hipEventDestroy(ev);
     delete ctx;
@@ -440,6 +505,7 @@ int ffmoe_router(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *r
     const ffmoe_layer &l = ctx->layers[layer];
     RouterWeights rw{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale,
                      static_cast<const uint4 *>(l.router_frag), l.router_norm_max};
+    claim_scratch(ctx, stream);
     FF_HIP(launch_router(static_cast<hipStream_t>(stream), rw, router_x, x_stride, t, ctx->shape.n_experts,
                          ctx->shape.d, ctx->shape.top_k, out_logits ? out_logits : ctx->logits, out_idx, out_w, &ctx->timer,
                          ctx->f16, out_logits != nullptr, ctx->logits));
@@ -456,7 +522,8 @@ struct VerifyScratch {
 static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
                          uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual, uint16_t *y,
                          uint16_t *partials_bf16, char **err, const VerifyScratch *use = nullptr,
-                         const RouteFusion *route = nullptr, bool dense = false, const SharedExpert *shared = nullptr) {
+                         const RouteFusion *route = nullptr, bool dense = false, const SharedExpert *shared = nullptr,
+                         ffmoe_ctx *shared_ctx = nullptr) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (int rc = check_layer(ctx, layer, true, route != nullptr, err)) return rc;
     if (!x || !idx || !w || (!y && !partials_bf16 && !route)) return fail(err, FFMOE_ERR_INVALID, "null argument");
@@ -467,6 +534,8 @@ static int verify_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uin
         return fail(err, FFMOE_ERR_INVALID, "y and residual must be 8-byte aligned");
     const VerifyScratch own{ctx->plan, ctx->acts, ctx->partials};
     const VerifyScratch &sc = use ? *use : own;
+    if (use) claim_static_scratch(ctx->device, stream); else claim_scratch(ctx, stream);
+    if (shared_ctx) claim_scratch(shared_ctx, stream);
     FF_HIP(launch_verify(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                          ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, residual, y, partials_bf16,
                          sc.plan, sc.acts, sc.partials, ctx->n_cus, &ctx->timer, ctx->f16, route, dense, shared));
@@ -549,7 +618,7 @@ int ffmoe_route_verify_shared(ffmoe_ctx *ctx, ffmoe_ctx *shared, void *stream, u
     const SharedExpert sh{shared->arena + (size_t)shared_layer * shared->layer_bytes, sg, shared_x, shared_x_stride, shared->acts,
                           shared->partials};
     return verify_common(ctx, stream, layer, x, x_stride, t, out_idx, out_w, nullptr, nullptr, nullptr, err, nullptr, &route,
-                         false, &sh);
+                         false, &sh, shared);
 }
 
 int ffmoe_set_handover_timeout(ffmoe_ctx *ctx, void *stream, uint64_t ticks, char **err) {
@@ -588,6 +657,7 @@ int ffmoe_probe_stream(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint32_t n_
     if ((ctx->geom.gd + 3) / 4 > 11 || ctx->geom.gf > 11)
         return fail(err, FFMOE_ERR_INVALID, "the stream probe covers the persistent kernels' shapes (d <= 2816, f <= 704)");
     // the sink: the first words of the un-weighted rows' scratch (never written on real data, see the launch)
+    claim_scratch(ctx, stream);
     FF_HIP(launch_probe_stream(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                                ctx->shape.n_experts, n_live, ctx->n_cus, reinterpret_cast<uint32_t *>(ctx->partials),
                                &ctx->timer));
@@ -617,6 +687,7 @@ static int prefill_common(ffmoe_ctx *ctx, void *stream, uint32_t layer, const ui
         return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
     if ((y && reinterpret_cast<uintptr_t>(y) % 16) || (partials && reinterpret_cast<uintptr_t>(partials) % 16))
         return fail(err, FFMOE_ERR_INVALID, "outputs must be 16-byte aligned");
+    claim_scratch(ctx, stream);
     FF_HIP(launch_prefill(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                           ctx->shape.n_experts, ctx->shape.top_k, x, x_stride, t, idx, w, pairs, n_pairs, y, partials,
                           ctx->pf, &ctx->timer, ctx->f16, dense));
@@ -645,6 +716,7 @@ int ffmoe_prefill_dump_tiles(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint3
     if (!out || reinterpret_cast<uintptr_t>(out) % 16) return fail(err, FFMOE_ERR_INVALID, "output must be a 16-byte aligned device pointer");
     const size_t need = (size_t)prefill_dump_fragments(ctx->geom, gate_up != 0) * 64 * sizeof(uint4);
     if (out_bytes < need) return fail(err, FFMOE_ERR_INVALID, "output holds %zu bytes, the fragments take %zu", out_bytes, need);
+    claim_scratch(ctx, stream);
     FF_HIP(launch_prefill_dump_tiles(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
                                      expert, gate_up != 0, ctx->pf, out, ctx->f16));
     return FFMOE_OK;
@@ -721,6 +793,7 @@ int ffmoe_layer_tail_routed(ffmoe_ctx *ctx, void *stream, const uint16_t *route_
     if (t == 0 || t > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%d", t, FFMOE_MAX_VERIFY_ROWS);
     const uint32_t strides[2] = {h1_stride, hidden_stride};
     if (int rc = check_rows(t, ctx->shape.d, strides, 2, err)) return rc;
+    claim_scratch(ctx, stream);      // the rows it combines are the context's
     FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), nullptr, 0, h1, h1_stride, hidden, hidden_stride, w_postffn2,
                              w_postffn, t, ctx->shape.d, eps, layer_scalar, nullptr, nullptr, nullptr, 0, ctx->f16, ctx->partials,
                              route_w, ctx->plan->route_valid, ctx->shape.top_k));
@@ -738,6 +811,8 @@ int ffmoe_layer_tail_routed_shared(ffmoe_ctx *ctx, ffmoe_ctx *shared, void *stre
     if (t == 0 || t > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%d", t, FFMOE_MAX_VERIFY_ROWS);
     const uint32_t strides[1] = {hidden_stride};
     if (int rc = check_rows(t, ctx->shape.d, strides, 1, err)) return rc;
+    claim_scratch(ctx, stream);
+    claim_scratch(shared, stream);
     FF_HIP(launch_layer_tail(static_cast<hipStream_t>(stream), nullptr, 0, nullptr, 0, hidden, hidden_stride, w_postffn2,
                              w_postffn, t, ctx->shape.d, eps, layer_scalar, nullptr, nullptr, nullptr, 0, ctx->f16, ctx->partials,
                              route_w, ctx->plan->route_valid, ctx->shape.top_k, shared->partials, shared_chunks(shared->geom)));
@@ -971,6 +1046,7 @@ static int matrix_greedy_common(ffmoe_matrix *mx, void *stream, const uint16_t *
     if (!(softcap >= 0.0f) || std::isinf(softcap)) return fail(err, FFMOE_ERR_INVALID, "softcap must be finite and >= 0 (0 disables it)");
     ffmoe_ctx *ctx = mx->ctx;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    claim_scratch(ctx, stream);      // the per-block winners go through the matrix's scratch
     ctx->timer.begin(s);
     FF_HIP(launch_matrix_greedy(s, mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows, mx->partials, out_tokens,
                                 ctx->n_cus, ctx->f16, &ctx->timer, softcap, out_conf));

@@ -8,7 +8,11 @@
  *   - every compute call ENQUEUES work on the caller's HIP stream (`stream` is a hipStream_t passed
  *     as void*, NULL = the default stream), returns without waiting, and allocates nothing; the
  *     stream plays the part of the reference's MTLCommandBuffer;
- *   - device buffers are caller-owned raw device pointers; scratch lives in the context;
+ *   - device buffers are caller-owned raw device pointers; scratch lives in the context and serves one stream at
+ *     a time: a call that arrives on another stream than the context's previous call first makes its stream wait
+ *     (on the device, hipStreamWaitEvent) for what the previous stream was given, so two streams that share a
+ *     context run its calls one after the other instead of racing for the scratch; streams under graph capture
+ *     are left alone (a capture orders its own nodes). The caller's own buffers are the caller's to order;
  *   - return value: FFMOE_OK (0) or a negative status; when `err` is non-NULL and the call fails,
  *     `*err` receives a strdup'd message the caller releases with free();
  *   - a context belongs to one host thread at a time (the reference's operators are not Sendable).
@@ -157,8 +161,10 @@ int ffmoe_verify(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x
  * rows) is a fixed array inside the library image instead of the context's allocations, and the call itself
  * allocates nothing. Limit: 32 KiB + 16 * top_k * (2 f + 4 d) bytes must fit FFMOE_STATIC_SCRATCH_BYTES (3 MiB; the
  * reference model takes 1.6 MiB); larger shapes are refused with FFMOE_ERR_INVALID. Every GPU holds one such array
- * for the life of the process, shared by all contexts and calls on that GPU: calls that overlap on one GPU (two
- * streams, two contexts, two threads) race on it, and ffmoe_last_live_experts does not see these calls. */
+ * for the life of the process, shared by all contexts and calls on that GPU. Calls from one host thread on different
+ * streams are ordered like a context's own (the stream of a later call waits, on the device, for the stream of the
+ * earlier one; no allocation: the event exists since the library looked the array's address up); calls that overlap
+ * from two host threads, or under graph capture, race on it. ffmoe_last_live_experts does not see these calls. */
 #define FFMOE_STATIC_SCRATCH_BYTES (3u << 20)
 int ffmoe_verify_static(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t *x, uint32_t x_stride,
                         uint32_t t, const uint32_t *idx, const uint16_t *w, const uint16_t *residual,

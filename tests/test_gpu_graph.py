@@ -89,3 +89,54 @@ def test_router_verify_and_dense_chain_in_a_graph(oracle, one_call):
     assert ctx.handover_giveups() == 0      # on a GPU of its own no wave of the one-launch form had to help itself
     ctx.close()
     dense.close()
+
+
+def test_two_streams_on_one_context_run_one_after_the_other(oracle):
+    """Calls on a context from two streams, no synchronisation between them on the caller's side: the later call's
+    stream waits on the device for the earlier one's, so the context's scratch (plan, activation rows, hand-over
+    words) is never used by two calls at once. Each result equals the same call made alone. The static-scratch entry
+    point, whose array every context on the GPU shares, is held to the same."""
+    import ctypes as C
+    import torch
+    import fieldfare_moe as ff
+    L = ff.lib()
+    d, f, e, k, t = 2816, 704, 128, 8, 16
+    ctx = ff.Context(d, f, e, k, n_layers=1, max_tokens=16)
+    _, pool, router = make_layer(oracle, 3, d, f, e)
+    ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
+    ctx.upload_router_bf16(0, router)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(77)
+    xs = [torch.randn((t, d), device="cuda", generator=g).to(torch.bfloat16) for _ in range(6)]
+    alone = []
+    for x in xs:
+        y, idx, w = ctx.route_verify(0, x, x)
+        alone.append((y.clone(), idx.clone(), w.clone()))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = []
+    for i, x in enumerate(xs):
+        with torch.cuda.stream(streams[i % 2]):
+            outs.append(ctx.route_verify(0, x, x))
+    torch.cuda.synchronize()
+    for (y, idx, w), (y0, idx0, w0) in zip(outs, alone):
+        assert torch.equal(idx, idx0) and torch.equal(w.view(torch.int16), w0.view(torch.int16))
+        assert torch.equal(y.view(torch.int16), y0.view(torch.int16))
+    assert ctx.handover_giveups() == 0
+    # the static array, from a second context on the same GPU as well
+    other = ff.Context(d, f, e, k, n_layers=1, max_tokens=16)
+    other.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
+    ys = [torch.empty((t, d), dtype=torch.bfloat16, device="cuda") for _ in xs]
+    for i, x in enumerate(xs):
+        with torch.cuda.stream(streams[i % 2]):
+            err = C.c_char_p()
+            stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            rc = L.ffmoe_verify_static((ctx if i % 3 else other)._h, stream, 0, C.c_void_p(x.data_ptr()), d, t,
+                                       C.c_void_p(alone[i][1].data_ptr()), C.c_void_p(alone[i][2].data_ptr()), None,
+                                       C.c_void_p(ys[i].data_ptr()), C.byref(err))
+            assert rc == 0, err.value
+    torch.cuda.synchronize()
+    for y, (y0, _, _) in zip(ys, alone):
+        assert torch.equal(y.view(torch.int16), y0.view(torch.int16))
+    ctx.close()
+    other.close()
