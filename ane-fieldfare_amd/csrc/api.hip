@@ -369,6 +369,24 @@ int ffmoe_upload_layer(ffmoe_ctx *ctx, uint32_t layer, const void *blobs, size_t
     return FFMOE_OK;
 }
 
+int ffmoe_sample_rows(ffmoe_ctx *ctx, void *stream, const float *logits, uint32_t stride, uint32_t rows, uint32_t count,
+                      const uint32_t *ids, const ffmoe_sampling *rule, const uint32_t *key_offset, uint32_t *out_tokens,
+                      float *out_prob, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!logits || !rule || !out_tokens || !out_prob) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (rows == 0 || rows > FFMOE_MAX_VERIFY_ROWS) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%d", rows, FFMOE_MAX_VERIFY_ROWS);
+    if (count == 0 || stride < count) return fail(err, FFMOE_ERR_INVALID, "count must be positive and the stride at least the count");
+    if (!(rule->temperature > 0.0f) || std::isinf(rule->temperature))
+        return fail(err, FFMOE_ERR_INVALID, "temperature must be positive and finite (temperature 0 is the greedy choice: ffmoe_argmax_rows)");
+    if (!(rule->softcap > 0.0f) || std::isinf(rule->softcap))
+        return fail(err, FFMOE_ERR_INVALID, "the sampled choice caps its logits: softcap must be positive and finite");
+    if (rule->top_k > 256) return fail(err, FFMOE_ERR_INVALID, "top_k = %u outside 0...256", rule->top_k);
+    if (rule->top_k && !(rule->top_p > 0.0f && rule->top_p <= 1.0f)) return fail(err, FFMOE_ERR_INVALID, "top_p outside (0, 1]");
+    FF_HIP(launch_sample_rows(static_cast<hipStream_t>(stream), logits, stride, rows, count, ids, rule->temperature, rule->top_p,
+                              rule->top_k, rule->key_base, rule->softcap, rule->seed, key_offset, out_tokens, out_prob));
+    return FFMOE_OK;
+}
+
 int ffmoe_upload_expert_parts(ffmoe_ctx *ctx, uint32_t layer, uint32_t expert, const ffmoe_projection *gate,
                               const ffmoe_projection *up, const ffmoe_projection *down, int src_is_device,
                               char **err) {

@@ -237,4 +237,10 @@ hipError_t launch_gemv_int4(hipStream_t s, const uint8_t *w, const uint16_t *sca
                             const uint16_t *x, void *y, uint32_t m, uint32_t n, uint32_t rows,
                             uint32_t x_stride, uint32_t y_stride, int y_f32, const uint32_t *ids = nullptr, bool f16 = false);
 
+// sample.hip: the sampled choice over rows of fp32 logits (Gumbel-max draw, exact top-k, top-p prefix)
+hipError_t launch_sample_rows(hipStream_t s, const float *logits, uint32_t stride, uint32_t rows, uint32_t count,
+                              const uint32_t *ids, float temperature, float top_p, uint32_t top_k, uint32_t key_base,
+                              float softcap, unsigned long long seed, const uint32_t *key_offset, uint32_t *out_tokens,
+                              float *out_prob);
+
 }  // namespace ffmoe

@@ -49,7 +49,7 @@ EXPORTS = [
     "ffmoe_matrix_greedy", "ffmoe_matrix_greedy_conf", "ffmoe_argmax_rows", "ffmoe_upload_expert_parts", "ffmoe_dense_ffn", "ffmoe_post_attn_setup",
     "ffmoe_layer_tail", "ffmoe_layer_tail_routed", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
-    "ffmoe_verify_static", "ffmoe_route_verify_shared", "ffmoe_layer_tail_routed_shared",
+    "ffmoe_verify_static", "ffmoe_route_verify_shared", "ffmoe_layer_tail_routed_shared", "ffmoe_sample_rows",
 ]
 
 PROFILE_SLOTS = 16
@@ -61,6 +61,12 @@ KERNEL_NAMES = ["router_logits", "router_topk", "plan", "gate_up", "down", "comb
 class Projection(C.Structure):
     """SharedExpertProjection: W uint8 [rows][cols/2], S/B bf16 [rows][cols/64] (Kernels/MoE/SharedExpertInt4.swift:32-40)."""
     _fields_ = [("w", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p)]
+
+
+class Sampling(C.Structure):
+    """ffmoe_sampling: TokenSampling + the position key of LMHeadChainInt4.RowSampling (LMHeadChainInt4.swift:183-190)."""
+    _fields_ = [("temperature", C.c_float), ("top_p", C.c_float), ("top_k", C.c_uint32), ("key_base", C.c_uint32),
+                ("softcap", C.c_float), ("seed", C.c_uint64)]
 
 
 class Profile(C.Structure):
@@ -234,6 +240,7 @@ def lib() -> C.CDLL:
                                         C.c_float, errp]
     L.ffmoe_layer_tail.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, vp, u32, u32, C.c_float, C.c_float, errp]
     L.ffmoe_layer_tail_routed.argtypes = [vp, vp, vp, vp, u32, vp, u32, vp, vp, u32, C.c_float, C.c_float, errp]
+    L.ffmoe_sample_rows.argtypes = [vp, vp, vp, u32, u32, u32, vp, C.POINTER(Sampling), vp, vp, vp, errp]
     L.ffmoe_route_verify_shared.argtypes = [vp, vp, vp, u32, u32, vp, u32, vp, u32, vp, u32, u32, vp, vp, errp]
     L.ffmoe_layer_tail_routed_shared.argtypes = [vp, vp, vp, vp, vp, u32, vp, vp, u32, C.c_float, C.c_float, errp]
     _lib = L
@@ -623,6 +630,20 @@ class Context:
         _check(self.L.ffmoe_argmax_rows(self._h, _stream(), _ptr(logits), _row_stride(logits), rows, count, softcap, _ptr(out),
                                         _ptr(conf), C.byref(err)), err)
         return (out, conf) if want_conf else out
+
+    def sample_rows(self, logits, temperature: float, softcap: float, seed: int, key_base: int = 0, top_k: int = 0,
+                    top_p: float = 1.0, ids=None, key_offset=None, count: int | None = None):
+        """The sampled choice per row of fp32 logits [rows, >= count]: (position int32 [-1: nothing finite], probability)."""
+        import torch
+        rows = logits.shape[0]
+        count = count or logits.shape[1]
+        out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+        prob = torch.empty((rows,), dtype=torch.float32, device=logits.device)
+        rule = Sampling(temperature, top_p, top_k, key_base, softcap, seed)
+        err = C.c_char_p()
+        _check(self.L.ffmoe_sample_rows(self._h, _stream(), _ptr(logits), _row_stride(logits), rows, count, _ptr(ids),
+                                        C.byref(rule), _ptr(key_offset), _ptr(out), _ptr(prob), C.byref(err)), err)
+        return out, prob
 
     def gemv_int4_listed(self, W, S, B, ids, x):
         """GEMV over the weight rows listed in `ids` (int32 CUDA tensor [m]): y fp32 [R, m], y[:, o] = row ids[o]."""

@@ -439,6 +439,25 @@ public:
         check(ffmoe_argmax_rows(c.raw(), stream, rowsLogits, count, (uint32_t)rowCount, count, softcap, outIndices, rowsConfidence,
                                 &err), err);
     }
+    // TokenSampling + RowSampling (LMHeadChainInt4.swift:183-190): how a row picks its token when it is not the argmax
+    struct RowSampling {
+        float temperature = 1.0f, topP = 1.0f;
+        uint32_t topK = 0;            // 0: no truncation
+        uint64_t seed = 0;
+        uint32_t keyBase = 0;         // position of row 0's token
+        const uint32_t *keyOffset = nullptr;   // device: one uint32 added to keyBase, or null
+    };
+    // encodeChoice with a sampling rule (LMHeadChainInt4.swift:192-216): the draw over `count` fp32 logits per row that
+    // are in device memory (encodeLogitsRows' output, or the listed projection's with `ids`); outIndices are positions
+    static void encodeSampledChoice(Context &c, void *stream, const float *rowsLogits, uint32_t logitsStrideElements, int rowCount,
+                                    uint32_t count, const uint32_t *ids, float softcap, const RowSampling &sampling,
+                                    uint32_t *outIndices, float *rowsConfidence) {
+        if (rowCount <= 0 || rowCount > maxGreedyRows) throw std::invalid_argument("rowCount outside 1...16");
+        const ffmoe_sampling rule{sampling.temperature, sampling.topP, sampling.topK, sampling.keyBase, softcap, sampling.seed};
+        char *err = nullptr;
+        check(ffmoe_sample_rows(c.raw(), stream, rowsLogits, logitsStrideElements, (uint32_t)rowCount, count, ids, &rule,
+                                sampling.keyOffset, outIndices, rowsConfidence, &err), err);
+    }
     uint32_t vocab() const { return vocab_; }
 
 private:

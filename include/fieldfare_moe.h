@@ -336,6 +336,34 @@ int ffmoe_matrix_greedy_conf(ffmoe_matrix *mx, void *stream, const uint16_t *x, 
 int ffmoe_argmax_rows(ffmoe_ctx *ctx, void *stream, const float *logits, uint32_t stride, uint32_t rows, uint32_t count,
                       float softcap, uint32_t *out_index, float *out_conf, char **err);
 
+/* How a row of fp32 logits picks its token when it is not the argmax: TokenSampling + the position key of
+ * LMHeadChainInt4.RowSampling (Kernels/Fusions/LMHeadChainInt4.swift:183-190; SampleRowsParams,
+ * Metal/Sampling/logit.metal:1025-1035). */
+typedef struct ffmoe_sampling {
+    float temperature;   /* > 0 */
+    float top_p;         /* (0, 1]; applies only with top_k */
+    uint32_t top_k;      /* 0 = no truncation, else 1...256 */
+    uint32_t key_base;   /* position of row 0's token (row r draws for position key_base + key_offset[0] + r) */
+    float softcap;       /* > 0: logits are capped to (-softcap, softcap) */
+    uint64_t seed;
+} ffmoe_sampling;
+
+/* The sampled choice over rows of fp32 logits that are in memory (ffmoe_matrix_gemv's output, or the listed
+ * projection's): per row one draw from the tempered softmax of the capped logits by the Gumbel-max rule,
+ * argmax_i capped(logit_i) / T + G(seed, key, token_i), over the entries the truncation keeps - the top_k largest
+ * capped logits (ties to the lower position), of those the shortest prefix whose T = 1 probability reaches top_p.
+ * The noise G is a hash of (seed, the drawn token's position, token id) alone, so every producer that draws a
+ * position draws the same noise. out_tokens[r] = the POSITION drawn (0xFFFFFFFF when no logit is finite), out_prob[r]
+ * its probability among the survivors at temperature T. ids (device, may be NULL): entry i is token ids[i] (the
+ * noise follows the token id; the position is returned, as in the reference). key_offset (device, may be NULL): one
+ * uint32 added to key_base, for a base that lives on the GPU. Replaces sample_rows_f32 as
+ * LMHeadChainInt4.encodeChoice dispatches it (Metal/Sampling/logit.metal:1010-1259,
+ * Kernels/Fusions/LMHeadChainInt4.swift:192-223). The top_k set is found exactly (a radix select), where the
+ * reference gathers the histogram's edge bin into at most 1,024 candidates. rows <= 16. */
+int ffmoe_sample_rows(ffmoe_ctx *ctx, void *stream, const float *logits, uint32_t stride, uint32_t rows, uint32_t count,
+                      const uint32_t *ids, const ffmoe_sampling *rule, const uint32_t *key_offset, uint32_t *out_tokens,
+                      float *out_prob, char **err);
+
 /* ---- dense (shared-expert) FFN ------------------------------------------------------------------ */
 
 /* One projection in the reference layout: W uint8 [rows][cols/2], S/B bf16 [rows][cols/64]

@@ -436,6 +436,69 @@ def greedy_choice_rows(logits, softcap: float = 0.0):
     return tokens, conf
 
 
+def sample_gumbel(seed: int, key: int, tokens) -> np.ndarray:
+    """sample_gumbel (Metal/Sampling/logit.metal:1042-1051): standard Gumbel noise per token from one SplitMix64 step of
+    the state seed ^ key * 0x9E3779B97F4A7C15 ^ token * 0xD1B54A32D192ED03; the output's top 24 bits (+ 0.5) / 2^24 are
+    the uniform. float32 throughout, as the kernel computes it."""
+    mask = (1 << 64) - 1
+    out = np.empty(len(tokens), np.float32)
+    for n, tok in enumerate(np.asarray(tokens, np.uint64)):
+        z = (seed ^ ((key * 0x9E3779B97F4A7C15) & mask) ^ ((int(tok) * 0xD1B54A32D192ED03) & mask)) & mask
+        z = (z + 0x9E3779B97F4A7C15) & mask
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
+        z ^= z >> 31
+        u = np.float32((np.float32(z >> 40) + np.float32(0.5)) * np.float32(1.0 / 16777216.0))
+        out[n] = -np.log(-np.log(u, dtype=np.float32), dtype=np.float32)
+    return out
+
+
+def sample_rows(logits, temperature: float, top_p: float, top_k: int, key_base: int, softcap: float, seed: int,
+                ids=None, key_offset: int = 0):
+    """sample_rows_f32 (Metal/Sampling/logit.metal:1010-1259) on rows of fp32 logits [R][V]: per row the position drawn by
+    the Gumbel-max rule over the entries the truncation keeps, its probability among them, and - for tests - the gap
+    between the winning and the second perturbed score (a draw whose gap is within float rounding may fall either
+    way on another machine's log / tanh). Truncation as the kernel's: the top_k largest capped logits by (value
+    descending, index ascending) when 0 < top_k < V, of those the shortest prefix whose T = 1 mass (relative to ALL
+    finite entries) reaches top_p, the draw at temperature T over the survivors. The noise key of row r is key_base +
+    key_offset + r; entry i's token is ids[i] when ids are given. Normalisers are summed in float64 here."""
+    logits = np.atleast_2d(np.asarray(logits, np.float32))
+    rows, count = logits.shape
+    tokens = np.full(rows, 0xFFFFFFFF, np.uint32)
+    prob = np.zeros(rows, np.float64)
+    gap = np.full(rows, np.inf, np.float64)
+    cap, inv_t = np.float32(softcap), np.float32(1.0) / np.float32(temperature)
+    for r in range(rows):
+        row = logits[r]
+        finite = np.isfinite(row)
+        if not finite.any():
+            continue
+        pos = np.flatnonzero(finite)
+        c = (cap * np.tanh(row[pos] / cap, dtype=np.float32)).astype(np.float32)
+        key = (key_base + key_offset + r) & 0xFFFFFFFF
+        if 0 < top_k < count:
+            order = np.lexsort((pos, -c.astype(np.float64)))[:top_k]          # value descending, then index ascending
+            total1 = np.exp(c.astype(np.float64) - float(cap)).sum()
+            cum, keep = 0.0, 0
+            while keep < len(order):
+                cum += float(np.exp(np.float32(c[order[keep]] - cap), dtype=np.float32)) / total1
+                keep += 1
+                if np.float32(cum) >= np.float32(top_p):
+                    break
+            order = order[:max(keep, 1)]
+            pos, c = pos[order], c[order]
+        tok = pos if ids is None else np.asarray(ids, np.uint32)[pos]
+        g = (c * inv_t).astype(np.float32) + sample_gumbel(seed, key, tok)
+        best = int(np.flatnonzero(g == g.max())[0])                           # ties: the first in (rank or index) order
+        tokens[r] = pos[best]
+        e = np.exp((c.astype(np.float64) - float(c.max())) * float(inv_t))
+        prob[r] = e[best] / e.sum()
+        if len(g) > 1:
+            rest = np.delete(g, best)
+            gap[r] = float(g[best]) - float(rest.max())
+    return tokens, prob, gap
+
+
 def moe_layer(pool: ExpertPool, router_w_bits, x_bits, top_k: int = 8, dtype: int = BF16, threads: int = 0):
     """Router + top-k + experts + combine in fp32-reference mode. Returns (idx [T][K], w f32 [T][K], y f32 [T][D])."""
     x_bits = np.ascontiguousarray(x_bits, np.uint16)

@@ -252,6 +252,16 @@ int main() {
                 if (ref[ids[i]] > ref[ids[best]]) best = (uint32_t)i;
             EXPECT(hot[r] == best);
         }
+        // the sampled choice over the same listed logits: top_k = 1 keeps the best listed row alone, whatever the noise
+        LMHeadChainInt4::RowSampling sampling;
+        sampling.topK = 1;
+        sampling.seed = 0x5EED;
+        sampling.keyBase = 40;
+        LMHeadChainInt4::encodeSampledChoice(ctx, stream, dLogits, (uint32_t)ids.size(), 3, (uint32_t)ids.size(), dIds, 30.0f,
+                                             sampling, dTok2, dConf);
+        HIP(hipStreamSynchronize(stream));
+        EXPECT(toHost(dTok2, 3) == hot);
+        EXPECT(toHost(dConf, 3) == std::vector<float>(3, 1.0f));
         HIP(hipFree(dConf));
         HIP(hipFree(dTok2));
         HIP(hipFree(dIds));

@@ -213,3 +213,81 @@ def test_greedy_conf_and_hot_vocabulary_choice(ctx, oracle, torch):
     assert np.array_equal(pos.astype(np.uint32), want_pos)
     assert np.abs(conf.cpu().numpy() - want_conf).max() <= 1e-5 + 1e-4 * want_conf.max()
     head.close()
+
+
+def _assert_draws(tok, prob, want_tok, want_prob, gap, what):
+    """Positions equal wherever the oracle's winning margin is beyond float rounding of the log / tanh the two machines
+    evaluate (a closer call may fall either way); nearly all rows must be of the first kind."""
+    tok = tok.cpu().numpy().astype(np.uint32)
+    clear = gap > 1e-4
+    assert clear.mean() >= 0.9, (what, gap)
+    assert np.array_equal(tok[clear], want_tok[clear]), (what, tok, want_tok, gap)
+    p = prob.cpu().numpy().astype(np.float64)
+    same = tok == want_tok
+    assert (np.abs(p[same] - want_prob[same]) <= 1e-5 + 2e-3 * want_prob[same]).all(), (what, p, want_prob)
+
+
+@pytest.mark.parametrize("count,temperature,top_k,top_p", [(4099, 1.0, 0, 1.0), (4099, 0.7, 0, 1.0), (300, 1.3, 0, 1.0),
+                                                           (4099, 1.0, 64, 1.0), (4099, 0.8, 40, 0.9), (4099, 1.0, 256, 0.95),
+                                                           (300, 1.0, 256, 0.5), (200, 1.0, 256, 0.9), (70000, 0.9, 50, 0.9)])
+def test_sample_rows_draw_and_probability(ctx, oracle, torch, count, temperature, top_k, top_p):
+    """ffmoe_sample_rows against the restated sample_rows_f32 (logit.metal:1010-1259): same drawn position and
+    probability per row, without truncation and with top_k / top_p; rows with ties at the top_k edge (equal values:
+    the lower positions survive), non-finite entries, fewer finite entries than top_k, nothing finite at all; a
+    row stride beyond the count."""
+    rng = np.random.default_rng(count + top_k)
+    rows = rng.normal(0, 4, (16, count)).astype(np.float32)
+    rows[1] = np.round(rows[1])                               # many equal values: the edge of the top_k set is a tie
+    rows[2, :5] = [np.inf, -np.inf, np.nan, 1e30, -1e30]
+    rows[3, :] = np.nan
+    rows[4, 30:] = -np.inf                                     # 30 finite entries
+    rows[5, :] = 2.5                                           # all equal: the lowest top_k positions survive
+    padded = np.full((16, count + 3), 1e9, np.float32)
+    padded[:, :count] = rows
+    logits = torch.from_numpy(padded).cuda()[:, :count]
+    want_tok, want_prob, gap = oracle.sample_rows(rows, temperature, top_p, top_k, key_base=100, softcap=30.0, seed=0xFEED_F00D)
+    tok, prob = ctx.sample_rows(logits, temperature, 30.0, 0xFEED_F00D, key_base=100, top_k=top_k, top_p=top_p)
+    assert tok.cpu().numpy()[3] == -1 and float(prob[3]) == 0.0
+    _assert_draws(tok, prob, want_tok, want_prob, gap, (count, temperature, top_k, top_p))
+
+
+def test_sample_rows_ids_key_offset_and_position_keys(ctx, oracle, torch):
+    # the noise follows the token id (ids) and the position (key_base + key_offset[0] + row)
+    rng = np.random.default_rng(77)
+    count = 1000
+    rows = rng.normal(0, 3, (8, count)).astype(np.float32)
+    ids = rng.permutation(50000)[:count].astype(np.uint32)
+    logits = torch.from_numpy(rows).cuda()
+    tids = torch.from_numpy(ids.astype(np.int32)).cuda()
+    koff = torch.tensor([12345], dtype=torch.int32, device="cuda")
+    for top_k, top_p in ((0, 1.0), (32, 0.9)):
+        want_tok, want_prob, gap = oracle.sample_rows(rows, 0.9, top_p, top_k, key_base=7, softcap=30.0, seed=3, ids=ids, key_offset=12345)
+        tok, prob = ctx.sample_rows(logits, 0.9, 30.0, 3, key_base=7, top_k=top_k, top_p=top_p, ids=tids, key_offset=koff)
+        _assert_draws(tok, prob, want_tok, want_prob, gap, ("ids", top_k))
+        # without the ids the draws differ (other noise), with the offset folded into the base they are the same
+        tok2, _ = ctx.sample_rows(logits, 0.9, 30.0, 3, key_base=7 + 12345, top_k=top_k, top_p=top_p, ids=tids)
+        assert np.array_equal(tok2.cpu().numpy(), tok.cpu().numpy())
+    # the same position drawn as row 3 of a block and as row 0 of a later call: the same token
+    blk, _ = ctx.sample_rows(logits[:4], 1.0, 30.0, 9, key_base=50)
+    one, _ = ctx.sample_rows(logits[3:4], 1.0, 30.0, 9, key_base=53)
+    assert int(blk[3]) == int(one[0])
+
+
+def test_sample_rows_full_vocabulary_row(ctx, oracle, torch):
+    # a 262,144-entry row (the LM head's), top-64 / top-p 0.9 and the plain draw
+    rng = np.random.default_rng(5)
+    rows = rng.normal(0, 3, (2, 262144)).astype(np.float32)
+    logits = torch.from_numpy(rows).cuda()
+    for top_k, top_p in ((64, 0.9), (0, 1.0)):
+        want_tok, want_prob, gap = oracle.sample_rows(rows, 0.8, top_p, top_k, key_base=1, softcap=30.0, seed=17)
+        tok, prob = ctx.sample_rows(logits, 0.8, 30.0, 17, key_base=1, top_k=top_k, top_p=top_p)
+        _assert_draws(tok, prob, want_tok, want_prob, gap, ("vocab", top_k))
+
+
+def test_sample_rows_argument_errors(ctx, ff, torch):
+    logits = torch.zeros((2, 64), dtype=torch.float32, device="cuda")
+    for kwargs, match in ((dict(temperature=0.0, softcap=30.0), "temperature"), (dict(temperature=1.0, softcap=0.0), "softcap"),
+                          (dict(temperature=1.0, softcap=30.0, top_k=257), "top_k"),
+                          (dict(temperature=1.0, softcap=30.0, top_k=8, top_p=0.0), "top_p")):
+        with pytest.raises(ff.FieldfareError, match=match):
+            ctx.sample_rows(logits, kwargs["temperature"], kwargs["softcap"], 1, top_k=kwargs.get("top_k", 0), top_p=kwargs.get("top_p", 1.0))

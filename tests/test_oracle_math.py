@@ -470,3 +470,77 @@ def test_greedy_choice_rows_against_closed_forms(oracle):
     _, c0 = oracle.greedy_choice_rows(rows[:1], 0.0)
     _, c2 = oracle.greedy_choice_rows(rows[:1], 0.5)
     assert c2[0] < c0[0]
+
+
+def test_sample_gumbel_is_one_splitmix64_step(oracle):
+    """The noise hash is SplitMix64 (pinned to its published vectors in test_oracle_codecs.py) stepped once from the
+    state seed ^ key * 0x9E3779B97F4A7C15 ^ token * 0xD1B54A32D192ED03; its top 24 bits make the uniform."""
+    mask = (1 << 64) - 1
+    for seed, key, tok in ((0, 0, 0), (0x1234_5678_9ABC_DEF0, 7, 262143), (mask, 0xFFFFFFFF, 0xFFFFFFFF), (42, 1000, 17)):
+        state = (seed ^ ((key * 0x9E3779B97F4A7C15) & mask) ^ ((tok * 0xD1B54A32D192ED03) & mask)) & mask
+        z = oracle.SplitMix64(state).next()
+        u = (np.float64(z >> 40) + 0.5) / 16777216.0
+        want = -np.log(-np.log(u))
+        got = float(oracle.sample_gumbel(seed, key, [tok])[0])
+        assert 0.0 < u < 1.0 and abs(got - want) <= 4e-6 * max(1.0, abs(want)), (seed, key, tok, got, want)
+
+
+def test_sample_rows_draws_from_the_truncated_tempered_softmax(oracle):
+    """The draw's law, by counting: over 30,000 positions the frequencies of the drawn entries match the softmax of
+    capped(logit) / T over the survivors (chi-square well inside its 99.9 % bound), and nothing outside the
+    survivors is ever drawn. Survivors by brute force: sort by (value descending, index ascending), first top_k, then
+    the shortest prefix whose T = 1 mass over ALL entries reaches top_p."""
+    logits = np.array([2.0, -1.0, 0.5, 2.0, 1.5, -3.0, 0.0, 1.9], np.float32)
+    cap = 30.0
+    capped = cap * np.tanh(logits.astype(np.float64) / cap)
+    n = 30000
+    rows = np.tile(logits, (n, 1))
+    for temperature, top_k, top_p in ((1.0, 0, 1.0), (0.7, 0, 1.0), (1.3, 5, 1.0), (0.9, 6, 0.8)):
+        tokens, prob, _ = oracle.sample_rows(rows, temperature, top_p, top_k, key_base=1000, softcap=cap, seed=0xC0FFEE)
+        order = sorted(range(len(logits)), key=lambda i: (-capped[i], i))
+        if 0 < top_k < len(logits):
+            p1 = np.exp(capped) / np.exp(capped).sum()
+            kept, cum = [], 0.0
+            for i in order[:top_k]:
+                kept.append(i)
+                cum += p1[i]
+                if cum >= top_p:
+                    break
+        else:
+            kept = order
+        law = np.zeros(len(logits))
+        law[kept] = np.exp(capped[kept] / temperature)
+        law /= law.sum()
+        seen = np.bincount(tokens, minlength=len(logits)).astype(np.float64)
+        assert seen[law == 0].sum() == 0
+        chi2 = (((seen - n * law) ** 2)[law > 0] / (n * law[law > 0])).sum()
+        assert chi2 < 30.0, (temperature, top_k, top_p, chi2)        # 99.9 % point of chi-square with 7 degrees: 24.3
+        # the reported probability is the law's value at the drawn entry
+        assert np.allclose(prob, law[tokens], rtol=1e-5)
+
+
+def test_sample_rows_special_cases(oracle):
+    rng = np.random.default_rng(8)
+    rows = rng.normal(0, 3, (5, 300)).astype(np.float32)
+    rows[1, 40] = rows[1, 200] = rows[1].max() + 2.0
+    rows[2, :4] = [np.inf, np.nan, -np.inf, 1e30]
+    rows[3, :] = -np.inf
+    greedy, _ = oracle.greedy_choice_rows(rows, 25.0)
+    # top_k = 1 keeps the largest capped logit alone (ties: the lower position); a vanishing temperature does the same
+    # (an exact tie survives a vanishing temperature: the noise, not the position, breaks it)
+    for kwargs in (dict(temperature=1.0, top_k=1, top_p=1.0), dict(temperature=1e-4, top_k=0, top_p=1.0)):
+        tokens, prob, _ = oracle.sample_rows(rows, key_base=3, softcap=25.0, seed=99, **kwargs)
+        untied = [0, 2, 3, 4]
+        assert np.array_equal(tokens[untied], greedy[untied]), kwargs
+        assert tokens[1] == 40 if kwargs["top_k"] == 1 else tokens[1] in (40, 200)
+        assert prob[3] == 0.0 and np.all(prob[[0, 1, 2, 4]] > 0.0)
+    # the noise follows the token id, not the position: a permuted table with ids draws the same TOKEN
+    perm = rng.permutation(300).astype(np.uint32)
+    base, _, _ = oracle.sample_rows(rows[:1], 0.8, 1.0, 0, key_base=11, softcap=25.0, seed=5)
+    listed, _, _ = oracle.sample_rows(rows[:1, perm], 0.8, 1.0, 0, key_base=11, softcap=25.0, seed=5, ids=perm)
+    assert perm[listed[0]] == base[0]
+    # and the key is the row's position: row r with base b draws what row 0 draws with base b + r
+    two, _, _ = oracle.sample_rows(np.stack([rows[0], rows[0]]), 0.8, 1.0, 0, key_base=20, softcap=25.0, seed=5)
+    one, _, _ = oracle.sample_rows(rows[:1], 0.8, 1.0, 0, key_base=21, softcap=25.0, seed=5)
+    off, _, _ = oracle.sample_rows(rows[:1], 0.8, 1.0, 0, key_base=20, softcap=25.0, seed=5, key_offset=1)
+    assert two[1] == one[0] == off[0]
