@@ -724,6 +724,8 @@ def main():
         extra["layer_block_rows16"] = {"one_stream_us": round(t_seq * 1e6, 2), "shared_expert_on_second_stream_us": round(t_con * 1e6, 2),
                                        "combine_in_layer_tail_us": round(t_fus * 1e6, 2),
                                        "shared_expert_inside_routed_launches_us": round(t_ins * 1e6, 2),
+                                       "best_one_stream_us": round(min(t_seq, t_fus, t_ins) * 1e6, 2),
+                                       "launches": {"one_stream": 7, "combine_in_layer_tail": 6, "shared_expert_inside_routed_launches": 4},
                                        "hip_graph_replay_us": graph_us,
                                        "steps": "post-attention setup, shared expert, router, routed experts, layer tail"}
         dense.close()
