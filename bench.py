@@ -728,6 +728,32 @@ def main():
                                        "launches": {"one_stream": 7, "combine_in_layer_tail": 6, "shared_expert_inside_routed_launches": 4},
                                        "hip_graph_replay_us": graph_us,
                                        "steps": "post-attention setup, shared expert, router, routed experts, layer tail"}
+        # the same block for a decode step (one row), separate calls against the shared expert inside the routed launches
+        hid1, att1 = hid_b[:1].contiguous(), att_b[:1].contiguous()
+        outs1 = tuple(torch.empty((1, D), dtype=torch.bfloat16, device="cuda") for _ in range(3))
+        h11 = torch.empty((1, D), dtype=torch.bfloat16, device="cuda")
+
+        def block1_separate():
+            i = counter["i"]
+            counter["i"] += 1
+            ctx.post_attn_setup(hid1, att1, wn_b[0], wn_b[1], wn_b[2], out=outs1)
+            dense.dense_ffn(i % LS, outs1[0], out=h11)
+            _, _, w1 = ctx.route_verify(i % L, outs1[2], outs1[1], combine=False)
+            ctx.layer_tail_routed(w1, h11, hid1, wn_b[3], wn_b[4], 1.0)
+
+        def block1_inside():
+            i = counter["i"]
+            counter["i"] += 1
+            ctx.post_attn_setup(hid1, att1, wn_b[0], wn_b[1], wn_b[2], out=outs1)
+            _, w1 = ctx.route_verify_shared(dense, i % L, i % LS, outs1[2], outs1[1], outs1[0])
+            ctx.layer_tail_routed_shared(dense, w1, hid1, wn_b[3], wn_b[4], 1.0)
+        t1_sep = timed(block1_separate, 120, warm=30)
+        t1_ins = timed(block1_inside, 120, warm=30)
+        extra["layer_block_rows1"] = {"separate_calls_us": round(t1_sep * 1e6, 2),
+                                      "shared_expert_inside_routed_launches_us": round(t1_ins * 1e6, 2),
+                                      "launches": {"separate_calls": 6, "shared_expert_inside_routed_launches": 4},
+                                      "moe_blocks_of_30_layers_ms": round(30 * t1_ins * 1e3, 3),
+                                      "steps": "post-attention setup, shared expert, router, routed experts, layer tail (combine in the tail)"}
         dense.close()
 
     # The row-wise steps either side of the MoE stage at the prefill chunk and at a verify block:
