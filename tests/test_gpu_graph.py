@@ -10,7 +10,7 @@ from helpers import bf16_tensor, bits_of, make_layer, to_ff_offsets
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("one_call", [False, True], ids=["router_then_verify", "route_verify"])
+@pytest.mark.parametrize("one_call", [False, True, "shared_inside"], ids=["router_then_verify", "route_verify", "shared_expert_inside"])
 def test_router_verify_and_dense_chain_in_a_graph(oracle, one_call):
     """`route_verify`: the router, the select and gate/up share one launch whose blocks hand the logits and routes
     to each other through words stamped with an epoch that lives in device memory and is advanced by the call's
@@ -43,6 +43,14 @@ def test_router_verify_and_dense_chain_in_a_graph(oracle, one_call):
         # one decoder-layer MoE block per layer: setup -> (shared expert, router -> routed experts) -> tail
         for layer in range(layers):
             ctx.post_attn_setup(hidden, x, ws[0], ws[1], ws[2], out=outs)
+            if one_call == "shared_inside":
+                # the shared expert inside the routed experts' launches, both combined in the tail: the call's last launch
+                # (the down projection) moves the epoch on
+                i_, w_ = ctx.route_verify_shared(dense, layer, layer, outs[2], outs[1], outs[0])
+                idx.copy_(i_)
+                w.copy_(w_)
+                ctx.layer_tail_routed_shared(dense, w, hidden, ws[3], ws[4], 0.9)
+                continue
             dense.dense_ffn(layer, outs[0], out=h1)
             if one_call:
                 _, i_, w_ = ctx.route_verify(layer, outs[2], outs[1], out=h2)
