@@ -466,7 +466,7 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
     hipLaunchKernelGGL((router_exact_topk_kernel<STEPS, CHUNK>), dim3((t + 3) / 4), dim3(256), 0, s,                         \
                        static_cast<const uint16_t *>(rw.w), x, x_stride, t, n_experts, d, top_k, approx, xnorm2, bound_per_norm, \
                        rw.per_expert_scale, out_idx, out_w)
-        if (d <= 1024) FFMOE_EXACT(1, 4); else if (d <= 2048) FFMOE_EXACT(2, 4); else if (d <= 3072) FFMOE_EXACT(3, 4); else FFMOE_EXACT(4, 3);
+        if (d <= 1024) FFMOE_EXACT(1, 4); else if (d <= 2048) FFMOE_EXACT(2, 4); else if (d <= 3072) FFMOE_EXACT(3, 4); else FFMOE_EXACT(4, 2);
 #undef FFMOE_EXACT
         timer->mark(s, FFMOE_K_ROUTER_TOPK);
         timer->finish();

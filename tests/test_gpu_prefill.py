@@ -374,3 +374,32 @@ def test_prefill_router_fast_form_equals_pinned_form(oracle, torch):
         assert want[6] != want[7] and abs(want[6] - want[7]) < 1e-4 * abs(want[6])
         assert sorted(got[row]) == sorted(order[:8])
     ctx.close()
+
+
+@pytest.mark.parametrize("d,e", [(1024, 16), (2048, 64), (3584, 32), (4096, 128)])
+def test_prefill_router_fast_form_other_widths(oracle, torch, d, e):
+    """The two-pass prefill router at the other hidden sizes its instantiations cover (one to four 1,024-wide steps of
+    the pinned order): routes and weights bit for bit those of the form that computes every pinned logit, which is
+    held against the oracle row by row."""
+    import fieldfare_moe as ff
+    ff.lib()
+    k, t = 8, 48
+    rng = np.random.default_rng(d + e)
+    bits = oracle.bf16_bits(rng.normal(0, 0.02, (e, d)).astype(np.float32))
+    bits[1] = bits[0]                                             # an exact tie
+    x = rng.normal(0, 1, (t, d)).astype(np.float32)
+    x[3] *= 200.0
+    xbits = oracle.bf16_bits(x)
+    ctx = ff.Context(d, 64, e, k, n_layers=1, max_tokens=64)
+    ctx.upload_router_bf16(0, bits)
+    xb = bf16_tensor(torch, xbits)
+    idx_fast, w_fast = ctx.router(0, xb)
+    idx_ref, w_ref, logits = ctx.router(0, xb, want_logits=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(idx_fast.cpu().numpy(), idx_ref.cpu().numpy())
+    assert np.array_equal(bits_of(w_fast), bits_of(w_ref))
+    got = logits.cpu().numpy()
+    for tok in (0, 3, t - 1):
+        want = oracle.router_logits_pinned(bits, xbits[tok])
+        assert np.array_equal(got[tok].view(np.uint32), want.view(np.uint32)), tok
+    ctx.close()
