@@ -206,15 +206,17 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, co
 //      a candidate.
 //      B: both sums add the same exact products (bf16 x bf16 fits fp32), so each differs from the real-number sum
 //      by at most (roundings on the longest path of its summation tree) x (relative size of one rounding) x
-//      sum_k |x_k w_ek| <= ... x ||x|| max_e ||w_e||. Approximate pass: d / 128 matrix instructions per wave, each
-//      adding 32 products to the running sum in an order the unit does not document; the count assumes the worst one,
-//      the running sum carried through all 33 additions of every instruction: 33 d / 128 roundings of 2^-23, and 2 to
-//      merge the four waves. Pinned order: 4 fmaf per 1024-wide step, 2 adds for the sub-accumulators, 6 for the
-//      butterfly, 2^-24 each (the order is this build's own, so the count is exact).
+//      sum_k |x_k w_ek| <= ... x ||x|| max_e ||w_e||. Approximate pass: a block sums one part of K (a quarter) with
+//      d / 128 matrix instructions, each adding 32 products to the running sum in an order the unit does not document;
+//      the count assumes the worst one, the running sum carried through all 33 additions of every instruction:
+//      33 d / 128 roundings of 2^-23, and 2 to add the four parts in a tree. Pinned order: 4 fmaf per 1024-wide step, 2 adds for the sub-accumulators, 6 for the butterfly,
+//      2^-24 each (the order is this build's own, so the count is exact).
 // Needs: bf16 rows and weights, no per-input scale, d a multiple of 256 up to 4096, E a multiple of 16 up to 128
-// (the sixteen waves of the approximate pass hold two 16-expert fragments each).
+// (the four waves of a block of the approximate pass hold two 16-expert fragments each).
 // ---------------------------------------------------------------------------------------------------
-constexpr int kApproxTok = 16;          // token rows per block of the approximate pass
+constexpr int kApproxFrags = 2;                      // 16-row operand fragments of token rows per block of the approximate pass
+constexpr int kApproxTok = 16 * kApproxFrags;
+constexpr int kApproxKParts = 4;        // K is cut into parts, one block each; the pass that follows adds the parts' sums
 
 // Router weights in matrix-operand order: frag[(h * E/16 + n) * 64 + lane] = the eight values
 // w[16 n + lane % 16][32 h + 8 (lane / 16) .. + 7], so that a wave's operand load is 1 KiB contiguous.
@@ -226,40 +228,48 @@ __global__ __launch_bounds__(256) void router_frag_kernel(const uint16_t *__rest
     frag[i] = *reinterpret_cast<const uint4 *>(w + (size_t)(16 * n + (lane & 15)) * d + 32 * h + 8 * (lane >> 4));
 }
 
-// One block = 16 token rows x all experts, sixteen waves: wave (kq, nq) takes a quarter of K and a quarter of the
-// experts' 16-column fragments (NF of them), with four k-steps of operands in flight - the pass is a chain of
-// round trips to the weights (every block reads all of them once), so it is the number of loads in flight that
-// sets its time. The loop body has no branch: the compiler then counts the loads in flight exactly and waits for the
-// oldest step only (behind a branch it waits for all of them, and the pass is one round trip per step).
-constexpr int kApproxWaves = 16, kApproxDepth = 4;
+// One block = 32 token rows x one quarter of K x all experts, four waves: wave nq takes a quarter of the experts'
+// 16-column fragments (NF of them) against both 16-row fragments of the block's rows, with four k-steps of operands in
+// flight. Every block reads its quarter of the weights once, so what the pass moves through the second-level cache is
+// (rows / 32) x the weights - the time of this pass is that traffic and the round trips it is made of, not its
+// arithmetic; 16 rows per block with K inside the block moved twice as much on three quarters of the compute units.
+// Block 4 b + q leaves the sums of K quarter q for rows 32 b .. 32 b + 31 in approx[q] and the rows' squares in
+// xnorm2[q]; the reader adds them as (q0 + q1) + (q2 + q3). The loop body has no branch: the compiler then counts the
+// loads in flight exactly and waits for the oldest step only (behind a branch it waits for all of them, and the pass is
+// one round trip per step).
+constexpr int kApproxDepth = 4;
 
 template <int NF>
-__global__ __launch_bounds__(64 * kApproxWaves) void router_approx_kernel(const uint4 *__restrict__ wfrag,
-                                                                           const uint16_t *__restrict__ x, uint32_t x_stride,
-                                                                           uint32_t t, uint32_t n_experts, uint32_t d,
-                                                                           float *__restrict__ approx, float *__restrict__ xnorm2) {
-    __shared__ float s_acc[4][4 * NF][4][64];       // [K quarter][fragment][value][lane]
-    __shared__ float s_x2[4][16];
-    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t kq = wave & 3, nq = wave >> 2;
+__global__ __launch_bounds__(256) void router_approx_kernel(const uint4 *__restrict__ wfrag, const uint16_t *__restrict__ x,
+                                                            uint32_t x_stride, uint32_t t, uint32_t t_pad, uint32_t n_experts,
+                                                            uint32_t d, float *__restrict__ approx, float *__restrict__ xnorm2) {
+    const uint32_t lane = threadIdx.x & 63, nq = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t kq = blockIdx.x % kApproxKParts, t0 = (blockIdx.x / kApproxKParts) * kApproxTok;
     const uint32_t j = lane & 15, jq = lane >> 4;
-    const uint32_t t0 = blockIdx.x * kApproxTok, nfrag = n_experts / 16, nh = d / 32;
-    const uint32_t h0 = kq * nh / 4, h1 = (kq + 1) * nh / 4, span = h1 - h0;
+    const uint32_t nfrag = n_experts / 16, nh = d / 32;
+    const uint32_t h0 = kq * nh / kApproxKParts, h1 = (kq + 1) * nh / kApproxKParts, span = h1 - h0;
     const uint32_t n0 = nq * NF;                       // this wave's fragments: n0 .. n0 + NF - 1 (those below nfrag)
     // the rows are loaded four neighbouring lanes per 64 contiguous bytes (row lane / 4, chunk lane % 4: 16 requests per
     // instruction instead of 64) and turned into the operand layout (lane (j, jq): row j, chunk jq) by cross-lane moves
-    const uint16_t *xr = x + (size_t)min(t0 + (lane >> 2), t - 1) * x_stride + 8 * (lane & 3);
+    const uint16_t *xr[kApproxFrags];
+#pragma unroll
+    for (int f = 0; f < kApproxFrags; ++f) xr[f] = x + (size_t)min(t0 + 16 * f + (lane >> 2), t - 1) * x_stride + 8 * (lane & 3);
     const int pull = (int)((4 * j + jq) * 4);
     const uint4 *wf = wfrag + lane;
-    f32x4 acc[NF];
+    f32x4 acc[kApproxFrags][NF];
+    float x2[kApproxFrags];
 #pragma unroll
-    for (int n = 0; n < NF; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float x2 = 0.0f;
-    uint4 a_q[kApproxDepth], b_q[kApproxDepth][NF];
-    // step i of this wave = k-step h0 + i; past the end it repeats the last step and enters with a zero row
+    for (int f = 0; f < kApproxFrags; ++f) {
+        x2[f] = 0.0f;
+#pragma unroll
+        for (int n = 0; n < NF; ++n) acc[f][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    uint4 a_q[kApproxDepth][kApproxFrags], b_q[kApproxDepth][NF];
+    // step i of this block = k-step h0 + i; past the end it repeats the last step and enters with zero rows
     auto fetch = [&](int slot, uint32_t i) {
         const uint32_t h = h0 + min(i, span - 1);
-        a_q[slot] = *reinterpret_cast<const uint4 *>(xr + 32 * h);
+#pragma unroll
+        for (int f = 0; f < kApproxFrags; ++f) a_q[slot][f] = *reinterpret_cast<const uint4 *>(xr[f] + 32 * h);
 #pragma unroll
         for (int n = 0; n < NF; ++n) b_q[slot][n] = wf[((size_t)h * nfrag + min(n0 + n, nfrag - 1)) * 64];
     };
@@ -269,48 +279,63 @@ __global__ __launch_bounds__(64 * kApproxWaves) void router_approx_kernel(const 
         for (uint32_t ib = 0; ib < span; ib += kApproxDepth) {
 #pragma unroll
             for (int u = 0; u < kApproxDepth; ++u) {
-                uint4 a = a_q[u];
-                uint4 b[NF];
+                uint4 a[kApproxFrags], b[NF];
+#pragma unroll
+                for (int f = 0; f < kApproxFrags; ++f) a[f] = a_q[u][f];
 #pragma unroll
                 for (int n = 0; n < NF; ++n) b[n] = b_q[u][n];
                 fetch(u, ib + u + kApproxDepth);
-                a.x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a.x);
-                a.y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a.y);
-                a.z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a.z);
-                a.w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a.w);
-                if (ib + u >= span) a = uint4{0, 0, 0, 0};
-                const uint32_t aw[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float lo = bf16lo_to_f32(aw[q]), hi = bf16hi_to_f32(aw[q]);
-                    x2 = __builtin_fmaf(lo, lo, x2);
-                    x2 = __builtin_fmaf(hi, hi, x2);
+                for (int f = 0; f < kApproxFrags; ++f) {
+                    a[f].x = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a[f].x);
+                    a[f].y = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a[f].y);
+                    a[f].z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a[f].z);
+                    a[f].w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a[f].w);
+                    if (ib + u >= span) a[f] = uint4{0, 0, 0, 0};
+                    const uint32_t aw[4] = {a[f].x, a[f].y, a[f].z, a[f].w};
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float lo = bf16lo_to_f32(aw[q]), hi = bf16hi_to_f32(aw[q]);
+                        x2[f] = __builtin_fmaf(lo, lo, x2[f]);
+                        x2[f] = __builtin_fmaf(hi, hi, x2[f]);
+                    }
+#pragma unroll
+                    for (int n = 0; n < NF; ++n) acc[f][n] = Act<false>::mfma(a[f], b[n], acc[f][n]);
                 }
-#pragma unroll
-                for (int n = 0; n < NF; ++n) acc[n] = Act<false>::mfma(a, b[n], acc[n]);
             }
         }
     }
-    // the row's squares: the four k-chunk lanes of a row, then the four K quarters
-    x2 += __shfl_xor(x2, 16, 64);
-    x2 += __shfl_xor(x2, 32, 64);
-    if (nq == 0 && jq == 0) s_x2[kq][j] = x2;
 #pragma unroll
-    for (int n = 0; n < NF; ++n)
+    for (int f = 0; f < kApproxFrags; ++f) {
+        // the row's squares over this part of K: the four k-chunk lanes of a row
+        x2[f] += __shfl_xor(x2[f], 16, 64);
+        x2[f] += __shfl_xor(x2[f], 32, 64);
+        const uint32_t row = t0 + 16 * f + j;
+        if (nq == 0 && jq == 0 && row < t) xnorm2[(size_t)kq * t_pad + row] = x2[f];
+        // the lane holds tokens 4 jq .. + 3 of expert column j of each of its fragments
 #pragma unroll
-        for (int r = 0; r < 4; ++r) s_acc[kq][n0 + n][r][lane] = acc[n][r];
-    __syncthreads();
-    if (wave == 0 && lane < 16 && t0 + lane < t)
-        xnorm2[t0 + lane] = (s_x2[0][lane] + s_x2[1][lane]) + (s_x2[2][lane] + s_x2[3][lane]);
-    // fragment n is finished by wave n (the lane holds tokens 4 jq .. + 3 of expert column j)
-    for (uint32_t n = wave; n < nfrag; n += kApproxWaves) {
+        for (int n = 0; n < NF; ++n) {
+            if (n0 + n < nfrag) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float v = (s_acc[0][n][r][lane] + s_acc[1][n][r][lane]) + (s_acc[2][n][r][lane] + s_acc[3][n][r][lane]);
-            const uint32_t tok = t0 + 4 * jq + r;
-            if (tok < t) approx[(size_t)tok * n_experts + 16 * n + j] = v;
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t tok = t0 + 16 * f + 4 * jq + r;
+                    if (tok < t) approx[((size_t)kq * t_pad + tok) * n_experts + 16 * (n0 + n) + j] = acc[f][n][r];
+                }
+            }
         }
     }
+}
+
+// What the approximate pass left per part of K, added pairwise (a tree of log2(parts) levels; all loads first).
+__device__ __forceinline__ float sum_k_parts(const float *__restrict__ p, size_t part_stride) {
+    float v[kApproxKParts];
+#pragma unroll
+    for (int q = 0; q < kApproxKParts; ++q) v[q] = p[q * part_stride];
+#pragma unroll
+    for (int w = 1; w < kApproxKParts; w *= 2)
+#pragma unroll
+        for (int q = 0; q + w < kApproxKParts; q += 2 * w) v[q] += v[q + w];
+    return v[0];
 }
 
 constexpr int kExactSteps = 4;          // d <= 4096: k = 1024 i + 256 s + 4 lane + j, i < 4
@@ -320,7 +345,8 @@ template <int STEPS, int CHUNK>
 __global__ __launch_bounds__(256, 3) void router_exact_topk_kernel(const uint16_t *__restrict__ w, const uint16_t *__restrict__ x,
                                                                    uint32_t x_stride, uint32_t t, uint32_t n_experts, uint32_t d,
                                                                    uint32_t top_k, const float *__restrict__ approx,
-                                                                   const float *__restrict__ xnorm2, float bound_per_norm,
+                                                                   const float *__restrict__ xnorm2, uint32_t t_pad,
+                                                                   float bound_per_norm,
                                                                    const uint16_t *__restrict__ per_expert_scale,
                                                                    uint32_t *__restrict__ out_idx, uint16_t *__restrict__ out_w) {
     const uint32_t lane = threadIdx.x & 63, tok = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -352,11 +378,12 @@ __global__ __launch_bounds__(256, 3) void router_exact_topk_kernel(const uint16_
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
         const uint32_t e = c * 64 + lane;
-        a[c] = e < n_experts ? approx[(size_t)tok * n_experts + e] : -INFINITY;
+        a[c] = e < n_experts ? sum_k_parts(approx + (size_t)tok * n_experts + e, (size_t)t_pad * n_experts) : -INFINITY;
         odd = odd || (e < n_experts && !(fabsf(a[c]) < INFINITY));
     }
     // 2 B: see the comment above; the absolute term covers products the matrix unit may flush to zero
-    const float bound = bound_per_norm * sqrtf(xnorm2[tok]) + 1e-30f;
+    const float norm2 = sum_k_parts(xnorm2 + tok, t_pad);
+    const float bound = bound_per_norm * sqrtf(norm2) + 1e-30f;
     const bool everyone = __any(odd) || !(bound < INFINITY);
     // v_k, the k-th largest approximate logit (equal values leave together, which can only lower it)
     uint32_t key0 = a[0] > -INFINITY ? orderable(a[0]) : 0u, key1 = a[1] > -INFINITY ? orderable(a[1]) : 0u;
@@ -450,21 +477,24 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
     if (rw.w_frag && !rw.w_is_f32 && !rw.effective_scale && !f16 && !want_logits && d % 256 == 0 && d <= 1024 * kExactSteps &&
         n_experts % 16 == 0 && n_experts <= 128 && top_k <= 8 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && x_stride % 8 == 0 && scratch) {
         // approximate logits of every expert on the matrix unit, the pinned ones only where the select can tell
-        float *xnorm2 = scratch, *approx = scratch + ((t + 63) & ~63u);
-        const dim3 agrid((t + kApproxTok - 1) / kApproxTok);
+        const uint32_t t_pad = (t + 63) & ~63u;
+        float *xnorm2 = scratch, *approx = scratch + (size_t)kApproxKParts * t_pad;
+        const dim3 agrid((t + kApproxTok - 1) / kApproxTok * kApproxKParts);
         const uint32_t per_wave = (n_experts / 16 + 3) / 4;       // fragments per wave: the four N quarters cover all of them
 #define FFMOE_APPROX(NF)                                                                                               \
-    hipLaunchKernelGGL(router_approx_kernel<NF>, agrid, dim3(64 * kApproxWaves), 0, s, rw.w_frag, x, x_stride, t, n_experts, \
-                       d, approx, xnorm2)
+    hipLaunchKernelGGL(router_approx_kernel<NF>, agrid, dim3(256), 0, s, rw.w_frag, x, x_stride, t, t_pad, n_experts, d, approx, \
+                       xnorm2)
         if (per_wave <= 1) FFMOE_APPROX(1); else FFMOE_APPROX(2);
 #undef FFMOE_APPROX
         timer->mark(s, FFMOE_K_ROUTER_LOGITS);
         // 2 B per unit of ||x||: the rounding counts of the two sums (see above), 1 % on top for the norms' own rounding
+        static_assert(kApproxKParts == 4, "the rounding count below is that of four parts of K added in a tree of two levels");
         const float approx_roundings = 33.0f * (float)(d / 128) + 2.0f, pinned_roundings = 4.0f * ((d + 1023) / 1024) + 8.0f;
         const float bound_per_norm = 2.02f * (approx_roundings * 0x1p-23f + pinned_roundings * 0x1p-24f) * rw.w_norm_max;
 #define FFMOE_EXACT(STEPS, CHUNK)                                                                                          \
     hipLaunchKernelGGL((router_exact_topk_kernel<STEPS, CHUNK>), dim3((t + 3) / 4), dim3(256), 0, s,                         \
-                       static_cast<const uint16_t *>(rw.w), x, x_stride, t, n_experts, d, top_k, approx, xnorm2, bound_per_norm, \
+                       static_cast<const uint16_t *>(rw.w), x, x_stride, t, n_experts, d, top_k, approx, xnorm2, t_pad,        \
+                       bound_per_norm,                                                                                      \
                        rw.per_expert_scale, out_idx, out_w)
         if (d <= 1024) FFMOE_EXACT(1, 4); else if (d <= 2048) FFMOE_EXACT(2, 4); else if (d <= 3072) FFMOE_EXACT(3, 4); else FFMOE_EXACT(4, 2);
 #undef FFMOE_EXACT
