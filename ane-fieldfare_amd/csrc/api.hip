@@ -674,11 +674,9 @@ int ffmoe_probe_stream(ffmoe_ctx *ctx, void *stream, uint32_t layer, uint32_t n_
         return fail(err, FFMOE_ERR_INVALID, "n_live = %u outside 1...%u", n_live, ctx->shape.n_experts);
     if ((ctx->geom.gd + 3) / 4 > 11 || ctx->geom.gf > 11)
         return fail(err, FFMOE_ERR_INVALID, "the stream probe covers the persistent kernels' shapes (d <= 2816, f <= 704)");
-    // the sink: the first words of the un-weighted rows' scratch (never written on real data, see the launch)
-    claim_scratch(ctx, stream);
+    // reads the arena only: no scratch of the context is touched
     FF_HIP(launch_probe_stream(static_cast<hipStream_t>(stream), ctx->arena + (size_t)layer * ctx->layer_bytes, ctx->geom,
-                               ctx->shape.n_experts, n_live, ctx->n_cus, reinterpret_cast<uint32_t *>(ctx->partials),
-                               &ctx->timer));
+                               ctx->shape.n_experts, n_live, ctx->n_cus, &ctx->timer));
     return FFMOE_OK;
 }
 

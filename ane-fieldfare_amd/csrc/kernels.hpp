@@ -176,9 +176,9 @@ hipError_t launch_verify(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g,
                          bool f16 = false, const RouteFusion *route = nullptr, bool dense = false,
                          const SharedExpert *shared = nullptr);
 uint32_t route_launch_resident_blocks(uint32_t n_cus);
-// the two expert kernels' weight loads for n_live experts and nothing else (`sink`: 256 words nobody reads)
+// the two expert kernels' weight loads for n_live experts and nothing else (nothing is stored)
 hipError_t launch_probe_stream(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t n_live,
-                               uint32_t n_cus, uint32_t *sink, KernelTimer *timer);
+                               uint32_t n_cus, KernelTimer *timer);
 hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, const uint16_t *weights,
                                      uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d, bool f16 = false);
 

@@ -1301,8 +1301,7 @@ __device__ __forceinline__ uint32_t ring_or(const WeightRing &ring, int u) {
 }
 
 __global__ __launch_bounds__(256, 2) void probe_gate_up_stream_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
-                                                                      uint32_t n_experts, uint32_t n_live, uint32_t never,
-                                                                      uint32_t *__restrict__ sink) {
+                                                                      uint32_t n_experts, uint32_t n_live) {
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const KSlice k = k_slice(g.gd, ks);
     const uint32_t blocks_per_slot = max(1u, min(g.gu_rb, gridDim.x / n_live));
@@ -1330,13 +1329,10 @@ __global__ __launch_bounds__(256, 2) void probe_gate_up_stream_kernel(const uint
 #pragma unroll
     for (int u = 0; u < kRing; ++u) seen |= ring_or(ring, u);
     asm volatile("" ::"v"(seen));      // names the value: the loads stay, nothing is stored
-    (void)never;
-    (void)sink;
 }
 
 __global__ __launch_bounds__(256, 5) void probe_down_stream_kernel(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
-                                                                   uint32_t n_experts, uint32_t n_live, uint32_t parts,
-                                                                   uint32_t never, uint32_t *__restrict__ sink) {
+                                                                   uint32_t n_experts, uint32_t n_live, uint32_t parts) {
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t slot_id = blockIdx.x / parts, part = blockIdx.x % parts;
     if (slot_id >= n_live) return;
@@ -1353,24 +1349,20 @@ __global__ __launch_bounds__(256, 5) void probe_down_stream_kernel(const uint8_t
 #pragma unroll
     for (int u = 0; u < kRing; ++u) seen |= ring_or(ring, u);
     asm volatile("" ::"v"(seen));      // names the value: the loads stay, nothing is stored
-    (void)never;
-    (void)sink;
 }
 
 }  // namespace
 
 hipError_t launch_probe_stream(hipStream_t s, const uint8_t *arena_layer, ArenaGeom g, uint32_t n_experts, uint32_t n_live,
-                               uint32_t n_cus, uint32_t *sink, KernelTimer *timer) {
+                               uint32_t n_cus, KernelTimer *timer) {
     timer->begin(s);
     const uint32_t resident = 2 * n_cus;
     const uint32_t gu_blocks = max(n_live, min(resident, n_live * g.gu_rb));
-    // (`sink` and the value passed beside it are no longer used: the kernels store nothing)
-    hipLaunchKernelGGL(probe_gate_up_stream_kernel, dim3(gu_blocks), dim3(256), 0, s, arena_layer, g, n_experts, n_live,
-                       0xFFFFFFFEu, sink);
+    hipLaunchKernelGGL(probe_gate_up_stream_kernel, dim3(gu_blocks), dim3(256), 0, s, arena_layer, g, n_experts, n_live);
     timer->mark(s, FFMOE_K_PROBE_GATE_UP);
     const uint32_t dn_parts = (g.dn_rbp + 3) / 4;
     hipLaunchKernelGGL(probe_down_stream_kernel, dim3(n_live * dn_parts), dim3(256), 0, s, arena_layer, g, n_experts, n_live,
-                       dn_parts, 0xFFFFFFFEu, sink);
+                       dn_parts);
     timer->mark(s, FFMOE_K_PROBE_DOWN);
     timer->finish();
     return hipGetLastError();
