@@ -211,7 +211,9 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *logits, co
 //      the count assumes the worst one, the running sum carried through all 33 additions of every instruction:
 //      33 d / 128 roundings of 2^-23, and 2 to add the four parts in a tree. Pinned order: 4 fmaf per 1024-wide step, 2 adds for the sub-accumulators, 6 for the butterfly,
 //      2^-24 each (the order is this build's own, so the count is exact).
-// Needs: bf16 rows and weights, no per-input scale, d a multiple of 256 up to 4096, E a multiple of 16 up to 128
+// FP16 rows enter the approximate pass as two bf16 halves per value (split_f16x8: exact), which doubles its
+// instructions and its rounding count; the pinned sums widen them to fp32 as every other kernel does.
+// Needs: bf16 weights, no per-input scale, d a multiple of 256 up to 4096, E a multiple of 16 up to 128
 // (the four waves of a block of the approximate pass hold two 16-expert fragments each).
 // ---------------------------------------------------------------------------------------------------
 constexpr int kApproxFrags = 2;                      // 16-row operand fragments of token rows per block of the approximate pass
@@ -239,7 +241,27 @@ __global__ __launch_bounds__(256) void router_frag_kernel(const uint16_t *__rest
 // one round trip per step).
 constexpr int kApproxDepth = 4;
 
-template <int NF>
+// Eight FP16 values as two sets of eight bf16 values whose sums are the FP16 values exactly (eleven significant bits =
+// the leading eight + the remaining three), so that FP16 rows meet the bf16 weights on the bf16 matrix instruction with
+// exact products. A value that is not finite leaves a NaN in one of the halves, and the row takes every expert.
+__device__ __forceinline__ void split_f16x8(const uint4 &v, uint4 &lead, uint4 &rest, float &x2) {
+    const uint32_t in[4] = {v.x, v.y, v.z, v.w};
+    uint32_t a[4], b[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const float f0 = Act<true>::lo(in[q]), f1 = Act<true>::hi(in[q]);
+        x2 = __builtin_fmaf(f0, f0, x2);
+        x2 = __builtin_fmaf(f1, f1, x2);
+        const uint32_t l0 = __float_as_uint(f0) & 0xFFFF0000u, l1 = __float_as_uint(f1) & 0xFFFF0000u;
+        const uint32_t r0 = __float_as_uint(f0 - __uint_as_float(l0)), r1 = __float_as_uint(f1 - __uint_as_float(l1));
+        a[q] = (l0 >> 16) | l1;
+        b[q] = (r0 >> 16) | (r1 & 0xFFFF0000u);
+    }
+    lead = uint4{a[0], a[1], a[2], a[3]};
+    rest = uint4{b[0], b[1], b[2], b[3]};
+}
+
+template <int NF, bool F16>
 __global__ __launch_bounds__(256) void router_approx_kernel(const uint4 *__restrict__ wfrag, const uint16_t *__restrict__ x,
                                                             uint32_t x_stride, uint32_t t, uint32_t t_pad, uint32_t n_experts,
                                                             uint32_t d, float *__restrict__ approx, float *__restrict__ xnorm2) {
@@ -292,15 +314,25 @@ __global__ __launch_bounds__(256) void router_approx_kernel(const uint4 *__restr
                     a[f].z = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a[f].z);
                     a[f].w = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)a[f].w);
                     if (ib + u >= span) a[f] = uint4{0, 0, 0, 0};
-                    const uint32_t aw[4] = {a[f].x, a[f].y, a[f].z, a[f].w};
+                    if constexpr (F16) {
+                        uint4 lead, rest;
+                        split_f16x8(a[f], lead, rest, x2[f]);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const float lo = bf16lo_to_f32(aw[q]), hi = bf16hi_to_f32(aw[q]);
-                        x2[f] = __builtin_fmaf(lo, lo, x2[f]);
-                        x2[f] = __builtin_fmaf(hi, hi, x2[f]);
+                        for (int n = 0; n < NF; ++n) {
+                            acc[f][n] = Act<false>::mfma(lead, b[n], acc[f][n]);
+                            acc[f][n] = Act<false>::mfma(rest, b[n], acc[f][n]);
+                        }
+                    } else {
+                        const uint32_t aw[4] = {a[f].x, a[f].y, a[f].z, a[f].w};
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const float lo = bf16lo_to_f32(aw[q]), hi = bf16hi_to_f32(aw[q]);
+                            x2[f] = __builtin_fmaf(lo, lo, x2[f]);
+                            x2[f] = __builtin_fmaf(hi, hi, x2[f]);
+                        }
+#pragma unroll
+                        for (int n = 0; n < NF; ++n) acc[f][n] = Act<false>::mfma(a[f], b[n], acc[f][n]);
                     }
-#pragma unroll
-                    for (int n = 0; n < NF; ++n) acc[f][n] = Act<false>::mfma(a[f], b[n], acc[f][n]);
                 }
             }
         }
@@ -341,7 +373,7 @@ __device__ __forceinline__ float sum_k_parts(const float *__restrict__ p, size_t
 constexpr int kExactSteps = 4;          // d <= 4096: k = 1024 i + 256 s + 4 lane + j, i < 4
 
 // STEPS: 1024-wide steps of the pinned order that d needs; CHUNK: candidates whose rows are requested together.
-template <int STEPS, int CHUNK>
+template <int STEPS, int CHUNK, bool F16>
 __global__ __launch_bounds__(256, 3) void router_exact_topk_kernel(const uint16_t *__restrict__ w, const uint16_t *__restrict__ x,
                                                                    uint32_t x_stride, uint32_t t, uint32_t n_experts, uint32_t d,
                                                                    uint32_t top_k, const float *__restrict__ approx,
@@ -368,8 +400,8 @@ __global__ __launch_bounds__(256, 3) void router_exact_topk_kernel(const uint16_
         for (int i = 0; i < STEPS; ++i)
 #pragma unroll
             for (int s_ = 0; s_ < 4; ++s_) {
-                xf[i][s_][0] = bf16lo_to_f32(xraw[i][s_].x), xf[i][s_][1] = bf16hi_to_f32(xraw[i][s_].x);
-                xf[i][s_][2] = bf16lo_to_f32(xraw[i][s_].y), xf[i][s_][3] = bf16hi_to_f32(xraw[i][s_].y);
+                xf[i][s_][0] = Act<F16>::lo(xraw[i][s_].x), xf[i][s_][1] = Act<F16>::hi(xraw[i][s_].x);
+                xf[i][s_][2] = Act<F16>::lo(xraw[i][s_].y), xf[i][s_][3] = Act<F16>::hi(xraw[i][s_].y);
             }
     }
     // at most 128 experts: the lane's candidates are experts lane and 64 + lane
@@ -448,7 +480,7 @@ __global__ __launch_bounds__(256, 3) void router_exact_topk_kernel(const uint16_
     TopkRow tr;
     tr.key[0] = exact0, tr.key[1] = exact1, tr.key[2] = 0u, tr.key[3] = 0u;
     topk_select<2>(tr, top_k, lane);
-    topk_store(tr, per_expert_scale, top_k, out_idx + (size_t)tok * top_k, out_w + (size_t)tok * top_k, lane, false);
+    topk_store(tr, per_expert_scale, top_k, out_idx + (size_t)tok * top_k, out_w + (size_t)tok * top_k, lane, F16);
 }
 
 }  // namespace
@@ -474,30 +506,38 @@ hipError_t launch_router(hipStream_t s, RouterWeights rw, const uint16_t *x, uin
         timer->finish();
         return hipGetLastError();
     }
-    if (rw.w_frag && !rw.w_is_f32 && !rw.effective_scale && !f16 && !want_logits && d % 256 == 0 && d <= 1024 * kExactSteps &&
+    if (rw.w_frag && !rw.w_is_f32 && !rw.effective_scale && !want_logits && d % 256 == 0 && d <= 1024 * kExactSteps &&
         n_experts % 16 == 0 && n_experts <= 128 && top_k <= 8 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && x_stride % 8 == 0 && scratch) {
         // approximate logits of every expert on the matrix unit, the pinned ones only where the select can tell
         const uint32_t t_pad = (t + 63) & ~63u;
         float *xnorm2 = scratch, *approx = scratch + (size_t)kApproxKParts * t_pad;
         const dim3 agrid((t + kApproxTok - 1) / kApproxTok * kApproxKParts);
         const uint32_t per_wave = (n_experts / 16 + 3) / 4;       // fragments per wave: the four N quarters cover all of them
-#define FFMOE_APPROX(NF)                                                                                               \
-    hipLaunchKernelGGL(router_approx_kernel<NF>, agrid, dim3(256), 0, s, rw.w_frag, x, x_stride, t, t_pad, n_experts, d, approx, \
-                       xnorm2)
-        if (per_wave <= 1) FFMOE_APPROX(1); else FFMOE_APPROX(2);
+#define FFMOE_APPROX(NF, H)                                                                                            \
+    hipLaunchKernelGGL((router_approx_kernel<NF, H>), agrid, dim3(256), 0, s, rw.w_frag, x, x_stride, t, t_pad, n_experts, d,  \
+                       approx, xnorm2)
+        if (f16) { if (per_wave <= 1) FFMOE_APPROX(1, true); else FFMOE_APPROX(2, true); }
+        else { if (per_wave <= 1) FFMOE_APPROX(1, false); else FFMOE_APPROX(2, false); }
 #undef FFMOE_APPROX
         timer->mark(s, FFMOE_K_ROUTER_LOGITS);
         // 2 B per unit of ||x||: the rounding counts of the two sums (see above), 1 % on top for the norms' own rounding
         static_assert(kApproxKParts == 4, "the rounding count below is that of four parts of K added in a tree of two levels");
-        const float approx_roundings = 33.0f * (float)(d / 128) + 2.0f, pinned_roundings = 4.0f * ((d + 1023) / 1024) + 8.0f;
+        // (FP16 rows enter as two bf16 halves: two instructions, 66 additions, per 32 elements)
+        const float approx_roundings = (f16 ? 66.0f : 33.0f) * (float)(d / 128) + 2.0f, pinned_roundings = 4.0f * ((d + 1023) / 1024) + 8.0f;
         const float bound_per_norm = 2.02f * (approx_roundings * 0x1p-23f + pinned_roundings * 0x1p-24f) * rw.w_norm_max;
-#define FFMOE_EXACT(STEPS, CHUNK)                                                                                          \
-    hipLaunchKernelGGL((router_exact_topk_kernel<STEPS, CHUNK>), dim3((t + 3) / 4), dim3(256), 0, s,                         \
+#define FFMOE_EXACT_AS(STEPS, CHUNK, H)                                                                                    \
+    hipLaunchKernelGGL((router_exact_topk_kernel<STEPS, CHUNK, H>), dim3((t + 3) / 4), dim3(256), 0, s,                      \
                        static_cast<const uint16_t *>(rw.w), x, x_stride, t, n_experts, d, top_k, approx, xnorm2, t_pad,        \
                        bound_per_norm,                                                                                      \
                        rw.per_expert_scale, out_idx, out_w)
+#define FFMOE_EXACT(STEPS, CHUNK)                                     \
+    do {                                                              \
+        if (f16) FFMOE_EXACT_AS(STEPS, CHUNK, true);                  \
+        else FFMOE_EXACT_AS(STEPS, CHUNK, false);                     \
+    } while (0)
         if (d <= 1024) FFMOE_EXACT(1, 4); else if (d <= 2048) FFMOE_EXACT(2, 4); else if (d <= 3072) FFMOE_EXACT(3, 4); else FFMOE_EXACT(4, 2);
 #undef FFMOE_EXACT
+#undef FFMOE_EXACT_AS
         timer->mark(s, FFMOE_K_ROUTER_TOPK);
         timer->finish();
         return hipGetLastError();

@@ -294,3 +294,47 @@ def test_guest_pairs_and_reduce_fp16(small, oracle, torch):
     h2 = bits_of(ctx.reduce_token_major(partials, w))
     assert np.array_equal(h2, oracle.reduce_token_major(bits_of(partials), oracle.FP16, bits_of(w), oracle.FP16))
     assert np.array_equal(h2, bits_of(ctx.prefill(0, x, idx, w)))
+
+
+def test_prefill_router_fp16_fast_form_equals_pinned_form(oracle, ff, torch):
+    """FP16 rows through the two-pass prefill router (every value enters the approximate pass as two bf16 halves):
+    routes and weights bit for bit those of the form that computes every pinned logit, which is held against the oracle
+    - on rows with exact ties between experts, rows one bf16 step of a weight apart, rows at both ends of the FP16
+    range, FP16 subnormals, zero and constant rows, and rows with non-finite values."""
+    d, e, k, t = 2816, 128, 8, 80
+    rng = np.random.default_rng(91)
+    router = rng.normal(0, 0.02, (e, d)).astype(np.float32)
+    router[5] = router[3]
+    router[64] = router[3]
+    bits = oracle.bf16_bits(router)
+    bits[7] = bits[6]
+    bits[7, 17] ^= 1
+    x = rng.normal(0, 1, (t, d)).astype(np.float32)
+    x[1] *= 2e3                                 # near the top of the FP16 range
+    x[2] *= 1e-6                                # FP16 subnormals
+    x[3] = 0.0
+    x[4, :] = x[4, 0]
+    x[5, 100] = np.inf
+    x[6, 5] = np.nan
+    x[7] = 60000.0                              # squares overflow fp32 sums nowhere near, the norm is large
+    wf = oracle.bf16_to_float(bits)
+    x[8] = wf[3] * 50
+    front = [20, 30, 40, 50, 60, 70, 80]
+    x[9] = 50.0 * (1.5 * wf[front].sum(axis=0) + wf[6])      # experts 6 and 7 as eighth and ninth, a few fp32 steps apart
+    xb = f16_bits(x)
+    ctx = ff.Context(d, 64, e, k, n_layers=1, max_tokens=128, act_dtype="fp16")
+    ctx.upload_router_bf16(0, bits)
+    xt = f16_tensor(torch, xb)
+    idx_fast, w_fast = ctx.router(0, xt)
+    idx_ref, w_ref, logits = ctx.router(0, xt, want_logits=True)
+    torch.cuda.synchronize()
+    assert w_fast.dtype == torch.float16
+    assert np.array_equal(idx_fast.cpu().numpy(), idx_ref.cpu().numpy())
+    assert np.array_equal(bits_of(w_fast), bits_of(w_ref))
+    got = logits.cpu().numpy()
+    for tok in (0, 1, 2, 3, 4, 8, 9, t - 1):
+        want = oracle.router_logits_pinned(bits, xb[tok], oracle.FP16)
+        assert np.array_equal(got[tok].view(np.uint32), want.view(np.uint32)), tok
+        o_idx, _ = oracle.topk_softmax(want, k)
+        assert np.array_equal(idx_fast.cpu().numpy()[tok].astype(np.uint32), o_idx), tok
+    ctx.close()
