@@ -586,10 +586,10 @@ def main():
         head_bytes = V * D // 2 + 2 * V * (D // 64) * 2
         for rows in (1, 16):
             xr = x[:rows].contiguous()
-            tg = timed(lambda: head.gemv(xr, f32_out=True), 20)
+            tg = timed(lambda: head.gemv(xr, f32_out=True), 40, warm=20)
             gemv[f"lm_head_262144x2816_rows{rows}"] = {"us": round(tg * 1e6, 1), "GBs": round(head_bytes / tg / 1e9, 1),
                                                         "pct_hbm_peak": round(100 * head_bytes / tg / 1e9 / HBM_PEAK_GBS, 1)}
-        tg = timed(lambda: head.greedy(x), 20)
+        tg = timed(lambda: head.greedy(x), 40, warm=20)
         gemv["lm_head_greedy_rows16_us"] = round(tg * 1e6, 1)
         extra["gemv"] = gemv
 
@@ -628,7 +628,7 @@ def main():
             TPs = args.prefill_tokens
             xps = torch.randn((TPs, D), device="cuda", generator=gen).to(torch.bfloat16)
             yps = torch.empty((TPs, D), dtype=torch.bfloat16, device="cuda")
-            tp_ = timed(lambda: dense_step(xps, yps), 20)
+            tp_ = timed(lambda: dense_step(xps, yps), 60, warm=60)      # timed like the routed prefill: after as many steps in front
             fl = 2.0 * 3 * D * FS * TPs
             shared[f"rows{TPs}"] = {"us": round(tp_ * 1e6, 1), "TFLOPs": round(fl / tp_ / 1e12, 1),
                                     "frac_mfma_peak": round(fl / tp_ / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
