@@ -242,7 +242,9 @@ int ffmoe_create(int device, const ffmoe_shape *shape, ffmoe_ctx **out, char **e
     const uint32_t router_rows = shape->max_tokens > FFMOE_MAX_VERIFY_ROWS ? shape->max_tokens : FFMOE_MAX_VERIFY_ROWS;
     const size_t routes = (size_t)FFMOE_MAX_VERIFY_ROWS * shape->top_k;
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&ctx->arena), ctx->layer_bytes * shape->n_layers);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->logits), 4 * ((size_t)router_rows * shape->n_experts + router_rows + 64) * sizeof(float));      // logits; or, for the two-pass prefill router, the four K parts' squared row norms and approximate logits
+    // (the two-pass router lays its four parts out with the row count rounded up to 64)
+    const size_t router_rows_padded = ((size_t)router_rows + 63) & ~(size_t)63;
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->logits), 4 * router_rows_padded * ((size_t)shape->n_experts + 1) * sizeof(float));      // logits; or, for the two-pass prefill router, the four K parts' squared row norms and approximate logits
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->plan), sizeof(VerifyPlan));
     if (e == hipSuccess) e = hipMemset(ctx->plan, 0, sizeof(VerifyPlan));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->mail), sizeof(RouteMail));

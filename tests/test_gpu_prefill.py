@@ -403,3 +403,32 @@ def test_prefill_router_fast_form_other_widths(oracle, torch, d, e):
         want = oracle.router_logits_pinned(bits, xbits[tok])
         assert np.array_equal(got[tok].view(np.uint32), want.view(np.uint32)), tok
     ctx.close()
+
+
+@pytest.mark.parametrize("act", ["bf16", "fp16"])
+@pytest.mark.parametrize("d,e,t", [(512, 96, 359), (256, 128, 65), (2816, 128, 1000)])
+def test_prefill_router_fast_form_at_the_context_row_limit(oracle, torch, act, d, e, t):
+    """The two-pass router keeps its intermediate sums per quarter of K with the row count rounded up to 64; a context
+    made for exactly t rows (t no multiple of 64) must hold them. Routes and weights equal the one-pass form's, and a
+    verify call on the same context afterwards still works (the scratch behind the router's is intact)."""
+    import fieldfare_moe as ff
+    ff.lib()
+    k = 8
+    rng = np.random.default_rng(t)
+    bits = oracle.bf16_bits(rng.normal(0, 0.02, (e, d)).astype(np.float32))
+    ctx = ff.Context(d, 64, e, k, n_layers=1, max_tokens=t, act_dtype=act)
+    ctx.upload_router_bf16(0, bits)
+    x = rng.normal(0, 1, (t, d)).astype(np.float32)
+    if act == "fp16":
+        xt = torch.from_numpy(x.astype(np.float16).view(np.int16)).cuda().view(torch.float16)
+    else:
+        xt = bf16_tensor(torch, oracle.bf16_bits(x))
+    idx_fast, w_fast = ctx.router(0, xt)
+    idx_ref, w_ref, _ = ctx.router(0, xt, want_logits=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(idx_fast.cpu().numpy(), idx_ref.cpu().numpy())
+    assert np.array_equal(bits_of(w_fast), bits_of(w_ref))
+    idx16, w16 = ctx.router(0, xt[:16])
+    torch.cuda.synchronize()
+    assert np.array_equal(idx16.cpu().numpy(), idx_ref.cpu().numpy()[:16])
+    ctx.close()
