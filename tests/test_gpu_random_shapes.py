@@ -21,6 +21,10 @@ def _draw(seed, n_cases, dense):
         t, tp = int(rng.integers(1, 17)), int(rng.integers(17, 700))
         if d * f * e > 24_000_000 or (dense and d * f > 1_500_000):
             continue
+        if not dense and len(cases) % 3 == 0:
+            # a shape the prefill router's two-pass form takes (d a multiple of 256, 16 ... 128 experts in sixteens)
+            d, e = 256 * max(1, d // 256), 16 * max(1, min(8, e // 16))
+            k = min(k, e)
         cases.append((len(cases), d, f, e, k, t, tp))
     return cases
 
