@@ -338,3 +338,36 @@ def test_prefill_router_fp16_fast_form_equals_pinned_form(oracle, ff, torch):
         o_idx, _ = oracle.topk_softmax(want, k)
         assert np.array_equal(idx_fast.cpu().numpy()[tok].astype(np.uint32), o_idx), tok
     ctx.close()
+
+
+@pytest.mark.parametrize("d,f,e,fs,t", [(128, 64, 16, 1472, 5), (2816, 704, 128, 2112, 16), (2816, 704, 128, 2112, 1)])
+def test_shared_expert_inside_the_routed_launches_fp16(oracle, ff, torch, d, f, e, fs, t):
+    """FP16 rows through ffmoe_route_verify_shared + ffmoe_layer_tail_routed_shared against the separate FP16 calls
+    (ffmoe_route_verify, ffmoe_dense_ffn, ffmoe_layer_tail): the same routes bit for bit, the new hidden rows to the
+    rounding of the shared expert's row (its K is summed in chunks)."""
+    _, pool, router = make_layer(oracle, 5, d, f, e, align=16)
+    ctx = ff.Context(d, f, e, 8, n_layers=1, max_tokens=16, act_dtype="fp16")
+    ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
+    ctx.upload_router_bf16(0, router)
+    g = np.random.default_rng(d + fs + t)
+    scale = 0.4 if d < 1024 else 0.08
+    parts = tuple(oracle.quantize_int4(g.uniform(-scale, scale, (r, c)).astype(np.float32)) for r, c in ((fs, d), (fs, d), (d, fs)))
+    shared = ff.Context(d, fs, 1, 1, n_layers=1, max_tokens=16, act_dtype="fp16")
+    shared.upload_expert_parts(0, 0, *parts)
+    x, rx, sx = (f16_tensor(torch, f16_bits(g.uniform(-1.0, 1.0, (t, d)))) for _ in range(3))
+    hid = f16_bits(g.uniform(-1.0, 1.0, (t, d)))
+    tw2, tw1 = (bf16_tensor(torch, oracle.bf16_bits(g.uniform(0.5, 1.5, d).astype(np.float32))) for _ in range(2))
+    y, idx_a, w_a = ctx.route_verify(0, rx, x)
+    h1 = shared.dense_ffn(0, sx)
+    hid_a = f16_tensor(torch, hid)
+    ctx.layer_tail(y, h1, hid_a, tw2, tw1, 0.875, 1e-6, d=d)
+    idx_b, w_b = ctx.route_verify_shared(shared, 0, 0, rx, x, sx)
+    hid_b = f16_tensor(torch, hid)
+    ctx.layer_tail_routed_shared(shared, w_b, hid_b, tw2, tw1, 0.875, 1e-6)
+    assert hid_b.dtype == torch.float16 and w_b.dtype == torch.float16
+    assert np.array_equal(idx_a.cpu().numpy(), idx_b.cpu().numpy()) and np.array_equal(bits_of(w_a), bits_of(w_b))
+    got, want = f16_float(bits_of(hid_b)), f16_float(bits_of(hid_a))
+    assert rel_err(got, want) < 1e-2 and cosine(got, want) > 0.9999, (rel_err(got, want), cosine(got, want))
+    assert ctx.handover_giveups() == 0
+    ctx.close()
+    shared.close()
