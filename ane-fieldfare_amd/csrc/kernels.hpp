@@ -97,7 +97,8 @@ struct KernelTimer {
 
 // Prefill: expert-sorted pairs and their M-tiles, built on the GPU.
 struct PrefillTile {
-    uint32_t expert, row_start, rows, pad;     // rows [row_start, row_start + rows) of the sorted pair list
+    uint32_t expert, row_start, rows;     // rows [row_start, row_start + rows) of the sorted pair list
+    uint32_t order;                       // the tile's number in row order (the tile list itself runs from the largest tile down)
 };
 struct PrefillPlan {
     uint32_t n_pairs, n_tiles, pad[2];

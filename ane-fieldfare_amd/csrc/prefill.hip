@@ -78,6 +78,7 @@ __global__ __launch_bounds__(kScanThreads) void prefill_scan_kernel(uint32_t n_b
     __shared__ uint32_t tile_off[FFMOE_MAX_EXPERTS + 1];
     __shared__ uint32_t part[kScanThreads];                 // [chunk][e_pad]: chunk sums, then chunk bases
     __shared__ unsigned long long scan_own[FFMOE_MAX_EXPERTS], wave_sum[FFMOE_MAX_EXPERTS / 64];
+    __shared__ uint32_t shorter[3][FFMOE_MAX_EXPERTS];      // per expert: shorter tiles in all, in front of it, ranked above its own
     const uint32_t e = threadIdx.x % e_pad, ch = threadIdx.x / e_pad, chunks = kScanThreads / e_pad;
     const uint32_t per = (n_blocks + chunks - 1) / chunks;
     const uint32_t b_lo = min(n_blocks, ch * per), b_hi = min(n_blocks, b_lo + per);
@@ -92,7 +93,10 @@ __global__ __launch_bounds__(kScanThreads) void prefill_scan_kernel(uint32_t n_b
     if (live)
         for (uint32_t b = b_lo + kScanKeep; b < b_hi; ++b) sum += block_cnt[(size_t)b * n_experts + e];
     part[threadIdx.x] = sum;
-    if (threadIdx.x < FFMOE_MAX_EXPERTS) total[threadIdx.x] = 0;
+    if (threadIdx.x < FFMOE_MAX_EXPERTS) {
+        total[threadIdx.x] = 0;
+        shorter[0][threadIdx.x] = shorter[1][threadIdx.x] = shorter[2][threadIdx.x] = 0;
+    }
     __syncthreads();
     if (ch == 0 && live) {
         uint32_t run = 0;
@@ -145,6 +149,29 @@ __global__ __launch_bounds__(kScanThreads) void prefill_scan_kernel(uint32_t n_b
         }
     }
     __syncthreads();
+    // The tile list runs from the largest tile down: the full tiles in expert order, then every expert's last, shorter
+    // tile by its rows (ties in expert order). The GEMM grids walk the list eight tiles at a time, so the launches end
+    // with their shortest blocks instead of with whatever the last experts hold (a Zipf chunk's heavy experts sit
+    // anywhere in the expert order). Where an expert's shorter tile goes takes a look at every other expert's: the
+    // threads of an expert share that out (one thread alone is a chain of two thousand instructions).
+    if (live) {
+        const uint32_t rest = total[e] % kBM, per_o = (e_pad + chunks - 1) / chunks;
+        const uint32_t o_lo = min(e_pad, ch * per_o), o_hi = min(e_pad, o_lo + per_o);
+        uint32_t all = 0, in_front = 0, above = 0;
+        for (uint32_t o = o_lo; o < o_hi; ++o) {
+            const uint32_t r = total[o] % kBM;          // experts past n_experts hold zero
+            const uint32_t has = r != 0 ? 1u : 0u;
+            all += has;
+            in_front += has & (o < e ? 1u : 0u);
+            above += has & ((r > rest || (r == rest && o < e)) ? 1u : 0u);
+        }
+        if (all) {
+            atomicAdd(&shorter[0][e], all);
+            atomicAdd(&shorter[1][e], in_front);
+            atomicAdd(&shorter[2][e], above);
+        }
+    }
+    __syncthreads();
     if (!live) return;
     uint32_t run = offset[e] + part[threadIdx.x];
 #pragma unroll
@@ -160,15 +187,18 @@ __global__ __launch_bounds__(kScanThreads) void prefill_scan_kernel(uint32_t n_b
     if (ch != 0) return;
     plan->expert_offset[e] = offset[e];
     plan->expert_count[e] = total[e];
-    const uint32_t nt = (total[e] + kBM - 1) / kBM;
+    // a tile keeps its number in row order, which places its activation blocks
+    const uint32_t nt = (total[e] + kBM - 1) / kBM, n_full = total[e] / kBM;
+    const uint32_t shorter_tiles = shorter[0][e], shorter_in_front = shorter[1][e], ranked_above = shorter[2][e];
+    const uint32_t full_in_front = tile_off[e] - shorter_in_front, full_tiles = tile_off[n_experts] - shorter_tiles;
     for (uint32_t i = 0; i < nt; ++i) {
-        const uint32_t ti = tile_off[e] + i;
+        const uint32_t ti = i < n_full ? full_in_front + i : full_tiles + ranked_above;
         if (ti < max_tiles) {
             PrefillTile tl;
             tl.expert = e;
             tl.row_start = offset[e] + i * kBM;
             tl.rows = min((uint32_t)kBM, total[e] - i * kBM);
-            tl.pad = 0;
+            tl.order = tile_off[e] + i;
             tiles[ti] = tl;
         }
     }
@@ -231,7 +261,7 @@ __global__ __launch_bounds__(kSortBlock) void prefill_dense_plan_kernel(uint32_t
         tl.expert = 0;
         tl.row_start = i * kBM;
         tl.rows = min((uint32_t)kBM, t - i * kBM);
-        tl.pad = 0;
+        tl.order = i;
         tiles[i] = tl;
     }
     if (i == 0) {
@@ -257,8 +287,8 @@ __global__ __launch_bounds__(kSortBlock) void prefill_dense_plan_kernel(uint32_t
 // else:    A = those activations, loaded straight into operand registers (1 KiB contiguous per wave and fragment, no
 //          cross-lane re-layout); streams are two 16-row blocks; out = partials[out_row][D] (16-bit).
 // Activation layout: [16-pair block][group of F][k-half][lane (j, jq)] x 8 values = pair j of the block at
-// k = 32 * (k-half) + 8 * jq .. + 7 of the group. The 16-pair blocks of M-tile ti start at block row_start / 16 + ti:
-// consecutive tiles never share a block (a tile adds at most one block of slack), so the buffer holds
+// k = 32 * (k-half) + 8 * jq .. + 7 of the group. The 16-pair blocks of an M-tile start at block row_start / 16 + its number
+// in row order: consecutive tiles never share a block (a tile adds at most one block of slack), so the buffer holds
 // max_pairs / 16 + max_tiles + 1 blocks.
 // ---------------------------------------------------------------------------------------------------
 
@@ -628,7 +658,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(const uint8_t *__r
     gw.nb = nb;
     gw.a = a;
     gw.a_stride = a_stride;
-    gw.act_block0 = gw.tile.row_start / 16 + ti;
+    gw.act_block0 = gw.tile.row_start / 16 + gw.tile.order;
     gw.act_blocks = act_blocks;
     // the arena tile row this wave expands; past the last one it expands the last again (never stored)
     const uint32_t at = min(nb * kTilesPerBlock + gw.wave, gw.n_arena_tiles - 1);
@@ -664,7 +694,7 @@ __global__ __launch_bounds__(kBM) void prefill_pair_scale_kernel(const PrefillPl
     if (ti >= plan->n_tiles) return;
     const PrefillTile tile = tiles[ti];
     if (threadIdx.x >= tile.rows) return;
-    const uint32_t block = tile.row_start / 16 + ti + threadIdx.x / 16, j = threadIdx.x % 16;
+    const uint32_t block = tile.row_start / 16 + tile.order + threadIdx.x / 16, j = threadIdx.x % 16;
     float *s = act_scale + (size_t)block * groups * 16 + j;
     float largest = 0.0f;
     for (uint32_t b = 0; b < groups; ++b) largest = fmaxf(largest, s[b * 16]);
@@ -732,7 +762,7 @@ __global__ void prefill_dump_plan_kernel(uint32_t expert, PrefillPlan *plan, Pre
     tl.expert = expert;
     tl.row_start = 0;
     tl.rows = 1;
-    tl.pad = 0;
+    tl.order = 0;
     tiles[0] = tl;
     sorted_token[0] = 0;
     sorted_out_row[0] = 0;
