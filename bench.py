@@ -121,6 +121,8 @@ def main():
     ap.add_argument("--no-sweep", action="store_true",
                     help="skip BASELINE.json config 5 (8,192-token Zipf prefill over all layers, then 256 decode steps "
                          "as 16 verify blocks with the LM head once per block)")
+    ap.add_argument("--tune-dense", action="store_true",
+                    help="also time the dense bf16 ceiling after the library tuned itself for the two shapes (TunableOp)")
     ap.add_argument("--no-zipf", action="store_true",
                     help="skip the Zipf(1.1) half of the prefill leg (so that a profiler's per-kernel averages of the prefill "
                          "kernels cover the router-made, near-uniform routes alone)")
@@ -448,6 +450,25 @@ def main():
         bt_gu, bt_dn = b_gu.t().contiguous(), b_dn.t().contiguous()
         t_dgu = min(dense_time(a_gu, b_gu, o_gu), dense_time(a_gu, bt_gu.t(), o_gu))
         t_ddn = min(dense_time(a_dn, b_dn, o_dn), dense_time(a_dn, bt_dn.t(), o_dn))
+        tuned = None
+        if args.tune_dense:
+            # the same products after the library searched its own solutions for them (torch's TunableOp: a few seconds
+            # per shape and layout); its result file goes to the temporary directory
+            try:
+                torch.cuda.tunable.enable(True)
+                torch.cuda.tunable.tuning_enable(True)
+                import tempfile
+                torch.cuda.tunable.set_filename(os.path.join(tempfile.gettempdir(), "ffmoe_bench_tunableop.csv"))
+                torch.cuda.tunable.set_max_tuning_duration(30)
+                t_tgu = min(dense_time(a_gu, b_gu, o_gu), dense_time(a_gu, bt_gu.t(), o_gu))
+                t_tdn = min(dense_time(a_dn, b_dn, o_dn), dense_time(a_dn, bt_dn.t(), o_dn))
+                tuned_tf = (flops_gu + flops_dn) / (t_tgu + t_tdn) / 1e12
+                tuned = {"gate_up_us": round(t_tgu * 1e6, 1), "down_us": round(t_tdn * 1e6, 1),
+                         "frac_mfma_peak": round(tuned_tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                         "gemm_frac_of_tuned_dense": round((flops_gu + flops_dn) / gemm_s / 1e12 / tuned_tf, 4)}
+            finally:
+                torch.cuda.tunable.tuning_enable(False)
+                torch.cuda.tunable.enable(False)
         del bt_gu, bt_dn
         dense_tf = (flops_gu + flops_dn) / (t_dgu + t_ddn) / 1e12
         prefill["dense_bf16_ceiling_TFLOPs"] = round(dense_tf, 1)
@@ -456,6 +477,8 @@ def main():
             "shapes": f"[{mrows} x {D}] . [{D} x {2 * F}] and [{mrows} x {F}] . [{F} x {D}], bf16, torch.matmul, the faster of the weight as [K x N] and as [N x K] transposed",
             "frac_mfma_peak": round(dense_tf / MFMA_BF16_PEAK_TFLOPS, 4),
             "gemm_frac_of_dense_ceiling": round((flops_gu + flops_dn) / gemm_s / 1e12 / dense_tf, 4)}
+        if tuned:
+            prefill["dense_bf16_ceiling"]["tuned_by_the_library"] = tuned
         del a_gu, b_gu, a_dn, b_dn, o_gu, o_dn
         # BASELINE.json config 4 (ii): the same chunk with Zipf(1.1) routing imposed on the experts
         # (indices and weights given, no router): a few experts hold most pairs, many hold a handful
