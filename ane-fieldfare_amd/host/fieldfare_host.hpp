@@ -17,6 +17,7 @@
 //   PrefillGroupedRoutedMoE       PrefillGroupedRoutedMoE.swift:183-448 -> PrefillGroupedRoutedMoE
 //   PrefillMoE.encodeReduceTokenMajor             PrefillMoE.swift:11-32       -> PrefillMoE::encodeReduceTokenMajor
 //   DequantInt4GEMV               Kernels/Quant/DequantInt4GEMV.swift   -> DequantInt4GEMV
+//   activeRoutedExperts, prefillExpertUnionCap    Runtime/Inference/RealForwardRunner.swift:818-847,1952-1961 -> RouteTrimming
 //   RoutedPrefillGuest, DeviceSupervisor, RuntimeFaultPolicy, GuestFault
 //                                 Runtime/Supervisor/DeviceSupervisor.swift:5-125 -> same names
 #pragma once
@@ -24,6 +25,7 @@
 #include <algorithm>
 #include <cstdint>
 #include <cstdlib>
+#include <cstring>
 #include <functional>
 #include <memory>
 #include <optional>
@@ -171,6 +173,121 @@ struct PrefillMoEGrouping {
             out.tiles.push_back({(uint32_t)at, (uint32_t)n, head.pairStart, tail.pairStart + tail.pairCount - head.pairStart});
         }
         return out;
+    }
+};
+
+// The reference's two lossy routing options, applied on the host to a block's routes between the router and the
+// expert pass, as the reference does on its shared-memory route buffers (both are off by default there):
+//   activeRoutedExperts < topK   RealForwardRunner.swift:1952-1961: only the first `active` ranks of a row run, their
+//                                weights rescaled so that the row keeps the total of all topK weights;
+//   prefillExpertUnionCap        RealForwardRunner.swift:818-847 (capExpertUnion): a block keeps the `cap` experts with
+//                                the most routed weight (ties to the lower expert), each row's kept weights rescaled to
+//                                the row's original total, the others set to zero.
+// Weights are 16-bit patterns in the context's activation type: bf16 (the default) or FP16. A route whose weight is
+// zero takes no part in ffmoe_verify / ffmoe_prefill, which is how the trimmed routes drop out of the expert pass.
+struct RouteTrimming {
+    enum class WeightType { bf16, fp16 };
+
+    static float widen(uint16_t bits, WeightType type) {
+        if (type == WeightType::fp16) {
+            const uint32_t sign = (uint32_t)(bits & 0x8000u) << 16, exp = (bits >> 10) & 0x1Fu, man = bits & 0x3FFu;
+            uint32_t u;
+            if (exp == 0x1Fu) {
+                u = sign | 0x7F800000u | (man << 13);                       // infinity, NaN
+            } else if (exp != 0) {
+                u = sign | ((exp + 112u) << 23) | (man << 13);
+            } else if (man == 0) {
+                u = sign;
+            } else {                                                        // subnormal: man * 2^-24, exact in fp32
+                float f = (float)man * 0x1p-24f;
+                std::memcpy(&u, &f, sizeof u);
+                u |= sign;
+            }
+            float f;
+            std::memcpy(&f, &u, sizeof f);
+            return f;
+        }
+        const uint32_t u = (uint32_t)bits << 16;
+        float f;
+        std::memcpy(&f, &u, sizeof f);
+        return f;
+    }
+    static uint16_t narrow(float value, WeightType type) {
+        uint32_t u;
+        std::memcpy(&u, &value, sizeof u);
+        if (type == WeightType::fp16) {
+            // round to nearest even, as a conversion instruction does
+            const uint32_t sign = (u >> 16) & 0x8000u, mag = u & 0x7FFFFFFFu;
+            if (mag > 0x7F800000u) return (uint16_t)(sign | 0x7E00u);                     // NaN
+            if (mag >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u);                    // rounds to 65520 or more: infinity
+            if (mag < 0x33000001u) return (uint16_t)sign;                                 // at most half the smallest subnormal: zero
+            if (mag < 0x38800000u) {                                                      // subnormal result: whole multiples of 2^-24
+                float f;
+                std::memcpy(&f, &mag, sizeof f);
+                const float scaled = f * 0x1p24f;                                         // exact
+                uint32_t q = (uint32_t)scaled;
+                const float rest = scaled - (float)q;
+                if (rest > 0.5f || (rest == 0.5f && (q & 1u))) ++q;
+                return (uint16_t)(sign | q);
+            }
+            const uint32_t rounded = mag + 0xFFFu + ((mag >> 13) & 1u);
+            return (uint16_t)(sign | ((rounded - 0x38000000u) >> 13));
+        }
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);      // NaN stays NaN
+        return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);                            // round to nearest even
+    }
+
+    // weights [rows][topK], in place: ranks >= active become zero, the others are rescaled by full / kept (left alone
+    // when the kept weights add up to zero)
+    static void keepActiveRanks(uint16_t *weights, int rows, int topK, int active, WeightType type = WeightType::bf16) {
+        if (!(rows >= 0 && topK > 0 && active >= 1 && active <= topK)) throw std::invalid_argument("keepActiveRanks: bad arguments");
+        if (active == topK) return;
+        for (int row = 0; row < rows; ++row) {
+            uint16_t *w = weights + (size_t)row * topK;
+            float full = 0.0f, kept = 0.0f;
+            for (int r = 0; r < topK; ++r) full += widen(w[r], type);
+            for (int r = 0; r < active; ++r) kept += widen(w[r], type);
+            if (kept != 0.0f)
+                for (int r = 0; r < active; ++r) w[r] = narrow(widen(w[r], type) * full / kept, type);
+            for (int r = active; r < topK; ++r) w[r] = 0;
+        }
+    }
+
+    // ids, weights [rows][topK]; weights are changed in place. Returns the number of distinct experts before the cap.
+    static int capExpertUnion(const uint32_t *ids, uint16_t *weights, int rows, int topK, int numExperts, int cap,
+                              WeightType type = WeightType::bf16) {
+        if (!(rows >= 0 && topK > 0 && numExperts > 0 && cap >= 1)) throw std::invalid_argument("capExpertUnion: bad arguments");
+        const size_t count = (size_t)rows * topK;
+        std::vector<float> mass((size_t)numExperts, 0.0f);
+        std::vector<char> seen((size_t)numExperts, 0);
+        int distinct = 0;
+        for (size_t i = 0; i < count; ++i) {
+            if (ids[i] >= (uint32_t)numExperts) throw std::invalid_argument("router wrote an expert past the expert count");
+            if (!seen[ids[i]]) {
+                seen[ids[i]] = 1;
+                ++distinct;
+            }
+            const float w = widen(weights[i], type);
+            mass[ids[i]] += w < 0.0f ? -w : w;
+        }
+        if (distinct <= cap) return distinct;
+        std::vector<uint32_t> order;
+        for (uint32_t e = 0; e < (uint32_t)numExperts; ++e)
+            if (mass[e] > 0.0f) order.push_back(e);
+        std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) { return mass[x] > mass[y]; });
+        std::vector<char> retained((size_t)numExperts, 0);
+        for (size_t i = 0; i < order.size() && i < (size_t)cap; ++i) retained[order[i]] = 1;
+        for (int row = 0; row < rows; ++row) {
+            uint16_t *w = weights + (size_t)row * topK;
+            const uint32_t *id = ids + (size_t)row * topK;
+            float original = 0.0f, kept = 0.0f;
+            for (int r = 0; r < topK; ++r) original += widen(w[r], type);
+            for (int r = 0; r < topK; ++r)
+                if (retained[id[r]]) kept += widen(w[r], type);
+            const float scale = kept != 0.0f ? original / kept : 0.0f;
+            for (int r = 0; r < topK; ++r) w[r] = retained[id[r]] ? narrow(widen(w[r], type) * scale, type) : (uint16_t)0;
+        }
+        return distinct;
     }
 };
 

@@ -1,7 +1,8 @@
 // Host-logic tests of the C++ operator mirror (no GPU): exact expected arrays restated from the reference's
 // PrefillMoEGroupingTests.swift, PrefillRouterTests.swift:12-22, PrefillGroupedRoutedMoETests+Binding.swift and
 // the fault policy of DeviceSupervisorFailoverTests.swift:19-81, and the packed-experts layout cases of
-// GTurboFormatCodecTests.swift:47-66,136-183 and ModelLoaderTests.swift:56-90,204-241.
+// GTurboFormatCodecTests.swift:47-66,136-183 and ModelLoaderTests.swift:56-90,204-241; the two route-trimming options of
+// RealForwardRunner.swift:818-847,1952-1961 on hand-computed rows (the reference has no test of its own for them).
 #include <cstdio>
 #include <cstring>
 
@@ -243,7 +244,73 @@ static void packedExpertsLayoutCodec() {
     }
 }
 
+static uint16_t bf(float v) { return RouteTrimming::narrow(v, RouteTrimming::WeightType::bf16); }
+static float fl(uint16_t b) { return RouteTrimming::widen(b, RouteTrimming::WeightType::bf16); }
+
+static void routeTrimming() {
+    // activeRoutedExperts (RealForwardRunner.swift:1952-1961): the first two ranks carry the row's whole weight
+    {
+        uint16_t w[8] = {bf(0.5f), bf(0.25f), bf(0.125f), bf(0.125f), bf(0.25f), bf(0.25f), bf(0.25f), bf(0.25f)};
+        RouteTrimming::keepActiveRanks(w, 2, 4, 2);
+        // row 0: full 1.0, kept 0.75: 0.5 / 0.75 and 0.25 / 0.75, rounded to bf16; row 1: kept 0.5 of 1.0
+        EXPECT(w[0] == bf(0.5f * 1.0f / 0.75f) && w[1] == bf(0.25f * 1.0f / 0.75f) && w[2] == 0 && w[3] == 0);
+        EXPECT(w[4] == bf(0.5f) && w[5] == bf(0.5f) && w[6] == 0 && w[7] == 0);
+        uint16_t same[4] = {bf(0.4f), bf(0.3f), bf(0.2f), bf(0.1f)}, keep[4];
+        std::memcpy(keep, same, sizeof keep);
+        RouteTrimming::keepActiveRanks(same, 1, 4, 4);                 // all ranks active: nothing changes
+        EXPECT(std::memcmp(same, keep, sizeof keep) == 0);
+        uint16_t zero[2] = {0, bf(1.0f)};
+        RouteTrimming::keepActiveRanks(zero, 1, 2, 1);                 // the kept weights add up to zero: left alone, the rest dropped
+        EXPECT(zero[0] == 0 && zero[1] == 0);
+        bool threw = false;
+        try { RouteTrimming::keepActiveRanks(zero, 1, 2, 3); } catch (const std::invalid_argument &) { threw = true; }
+        EXPECT(threw);
+    }
+    // prefillExpertUnionCap (capExpertUnion, RealForwardRunner.swift:828-847): three rows, top 2, five experts in use
+    {
+        const uint32_t ids[6] = {0, 1, 2, 1, 3, 4};
+        uint16_t w[6] = {bf(0.75f), bf(0.25f), bf(0.5f), bf(0.5f), bf(0.5f), bf(0.5f)};
+        // routed weight per expert: 0: 0.75, 1: 0.75, 2: 0.5, 3: 0.5, 4: 0.5 -> cap 3 keeps 0, 1 (tie: both in) and 2 (the lowest of the tie)
+        const int before = RouteTrimming::capExpertUnion(ids, w, 3, 2, 8, 3);
+        EXPECT(before == 5);
+        EXPECT(w[0] == bf(0.75f) && w[1] == bf(0.25f));               // row 0 keeps both: scale 1
+        EXPECT(w[2] == bf(0.5f) && w[3] == bf(0.5f));                 // row 1 keeps both
+        EXPECT(w[4] == 0 && w[5] == 0);                               // row 2 lost both: nothing kept, scale 0
+        uint16_t w2[4] = {bf(0.75f), bf(0.25f), bf(0.25f), bf(0.75f)};
+        const uint32_t ids2[4] = {5, 6, 6, 7};
+        // 5: 0.75, 6: 0.5, 7: 0.75 -> cap 2 keeps 5 and 7; each row's kept weight is rescaled to the row's total
+        EXPECT(RouteTrimming::capExpertUnion(ids2, w2, 2, 2, 8, 2) == 3);
+        EXPECT(w2[0] == bf(1.0f) && w2[1] == 0 && w2[2] == 0 && w2[3] == bf(1.0f));
+        uint16_t w3[2] = {bf(0.5f), bf(0.5f)};
+        const uint32_t ids3[2] = {1, 2};
+        EXPECT(RouteTrimming::capExpertUnion(ids3, w3, 1, 2, 4, 2) == 2 && w3[0] == bf(0.5f) && w3[1] == bf(0.5f));   // within the cap: untouched
+        bool threw = false;
+        const uint32_t bad[2] = {1, 9};
+        try { RouteTrimming::capExpertUnion(bad, w3, 1, 2, 4, 1); } catch (const std::invalid_argument &) { threw = true; }
+        EXPECT(threw);
+    }
+    // FP16 patterns go through the same arithmetic
+    {
+        const auto h = RouteTrimming::WeightType::fp16;
+        uint16_t w[2] = {RouteTrimming::narrow(0.75f, h), RouteTrimming::narrow(0.25f, h)};
+        RouteTrimming::keepActiveRanks(w, 1, 2, 1, h);
+        EXPECT(RouteTrimming::widen(w[0], h) == 1.0f && w[1] == 0);
+        EXPECT(fl(bf(1.0f)) == 1.0f && bf(1.0f) == 0x3F80 && RouteTrimming::narrow(1.0f, h) == 0x3C00);
+        // every FP16 pattern that is a number survives widen -> narrow; midpoints go to the even neighbour
+        int bad = 0;
+        for (uint32_t b = 0; b < 0x10000u; ++b) {
+            if ((b & 0x7C00u) == 0x7C00u && (b & 0x3FFu)) continue;      // NaN
+            bad += RouteTrimming::narrow(RouteTrimming::widen((uint16_t)b, h), h) != b;
+        }
+        EXPECT(bad == 0);
+        EXPECT(RouteTrimming::narrow(65520.0f, h) == 0x7C00 && RouteTrimming::narrow(65519.0f, h) == 0x7BFF);
+        EXPECT(RouteTrimming::narrow(1.0f + 0x1p-11f, h) == 0x3C00 && RouteTrimming::narrow(1.0f + 3 * 0x1p-11f, h) == 0x3C02);
+        EXPECT(RouteTrimming::narrow(0x1p-25f, h) == 0 && RouteTrimming::narrow(0x1.8p-24f, h) == 2 && RouteTrimming::narrow(0x1p-24f, h) == 1);
+    }
+}
+
 int main() {
+    routeTrimming();
     groupingSortsPairsAndBuildsOffsetsCountsAndTiles();
     groupingCanOrderTilesByExpertSortKeys();
     groupingRejectsInvalidMetadataBeforeKernelUse();
