@@ -32,6 +32,7 @@ struct ffmoe_matrix {
     ffmoe_ctx *ctx = nullptr;     // null once the owning context was destroyed (the device memory went with it)
     int device = 0;
     uint32_t m = 0, n = 0;
+    bool planes8 = false;         // an 8-bit weight kept as two nibble planes (ffmoe_matrix_create_int8)
     uint8_t *tiles = nullptr, *scales = nullptr;
     unsigned long long *partials = nullptr;   // [16][blocks of the GEMV grid]: per-block winners of the greedy choice
 };
@@ -943,8 +944,8 @@ int ffmoe_gemv_int4_listed(ffmoe_ctx *ctx, void *stream, const uint8_t *w, const
     return gemv_common(ctx, stream, w, scales, biases, ids, x, y, m, n, rows, x_stride, y_stride, 1, err);
 }
 
-int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases, uint32_t m,
-                        uint32_t n, int with_greedy, ffmoe_matrix **out, char **err) {
+static int matrix_create_common(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases, uint32_t m,
+                                uint32_t n, int with_greedy, bool planes8, ffmoe_matrix **out, char **err) {
     if (int rc = check_ctx(ctx, err)) return rc;
     if (!w || !scales || !biases || !out) return fail(err, FFMOE_ERR_INVALID, "null argument");
     *out = nullptr;
@@ -952,18 +953,19 @@ int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales
     if (n == 0 || !matrix_shape_ok(n))
         return fail(err, FFMOE_ERR_INVALID, "N = %u must be a multiple of %d and at most %d", n, FFMOE_GROUP,
                     FFMOE_MATRIX_MAX_N);
-    if (reinterpret_cast<uintptr_t>(w) % 2) return fail(err, FFMOE_ERR_INVALID, "weights need a 2-aligned offset");
+    if (!planes8 && reinterpret_cast<uintptr_t>(w) % 2) return fail(err, FFMOE_ERR_INVALID, "weights need a 2-aligned offset");
     // the kernels address the tile region through a buffer descriptor with 32-bit sizes and offsets
-    if (matrix_tiles_bytes(m, n) >= ((size_t)1 << 32))
+    if (matrix_tiles_bytes(m, n, planes8) >= ((size_t)1 << 32))
         return fail(err, FFMOE_ERR_INVALID, "M = %u x N = %u needs a tile region of %zu bytes; the limit is 4 GiB", m, n,
-                    matrix_tiles_bytes(m, n));
+                    matrix_tiles_bytes(m, n, planes8));
     ffmoe_matrix *mx = new (std::nothrow) ffmoe_matrix();
     if (!mx) return fail(err, FFMOE_ERR_ALLOC, "out of host memory");
     mx->ctx = ctx;
     mx->device = ctx->device;
     mx->m = m;
     mx->n = n;
-    const size_t w_bytes = (size_t)m * n / 2, s_bytes = (size_t)m * (n / FFMOE_GROUP) * 2;
+    mx->planes8 = planes8;
+    const size_t w_bytes = planes8 ? (size_t)m * n : (size_t)m * n / 2, s_bytes = (size_t)m * (n / FFMOE_GROUP) * 2;
     uint8_t *stage = nullptr;
     auto cleanup = [&]() {
         if (stage) (void)hipFree(stage);
@@ -981,8 +983,8 @@ int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales
                         "%s: %s", #call, hipGetErrorString(e_));                                      \
         }                                                                                             \
     } while (0)
-    FF_MX(hipMalloc(&mx->tiles, matrix_tiles_bytes(m, n)));
-    FF_MX(hipMalloc(&mx->scales, matrix_scales_bytes(m, n)));
+    FF_MX(hipMalloc(&mx->tiles, matrix_tiles_bytes(m, n, planes8)));
+    FF_MX(hipMalloc(&mx->scales, matrix_scales_bytes(m, n, planes8)));
     if (with_greedy) {
         // per input row and block of the GEMV grid: the winner's key, then its softmax pair (8 bytes each)
         FF_MX(hipMalloc(&mx->partials, 2 * (size_t)FFMOE_MAX_VERIFY_ROWS * greedy_segments(m, ctx->n_cus) * sizeof(unsigned long long)));
@@ -1003,12 +1005,33 @@ int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales
         ds = reinterpret_cast<const uint16_t *>(stage + w_pad);
         db = reinterpret_cast<const uint16_t *>(stage + w_pad + s_pad);
     }
-    FF_MX(launch_matrix_repack(nullptr, dw, ds, db, m, n, mx->tiles, mx->scales));
+    FF_MX(launch_matrix_repack(nullptr, dw, ds, db, m, n, mx->tiles, mx->scales, planes8));
     FF_MX(hipDeviceSynchronize());
 #undef FF_MX
     if (stage) (void)hipFree(stage);
     ctx->matrices.push_back(mx);
     *out = mx;
+    return FFMOE_OK;
+}
+
+int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases, uint32_t m,
+                        uint32_t n, int with_greedy, ffmoe_matrix **out, char **err) {
+    return matrix_create_common(ctx, w, scales, biases, m, n, with_greedy, false, out, err);
+}
+
+int ffmoe_matrix_create_int8(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases, uint32_t m,
+                             uint32_t n, ffmoe_matrix **out, char **err) {
+    return matrix_create_common(ctx, w, scales, biases, m, n, 0, true, out, err);
+}
+
+int ffmoe_gelu_mul(ffmoe_ctx *ctx, void *stream, const uint16_t *gate, uint32_t gate_stride, const uint16_t *up,
+                   uint32_t up_stride, uint16_t *out, uint32_t out_stride, uint32_t rows, uint32_t count, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!gate || !up || !out) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (rows == 0 || count == 0) return fail(err, FFMOE_ERR_INVALID, "rows and count must be positive");
+    if (gate_stride < count || up_stride < count || out_stride < count) return fail(err, FFMOE_ERR_INVALID, "stride smaller than the row");
+    if (rows > 65535u) return fail(err, FFMOE_ERR_INVALID, "rows = %u: at most 65535 per call", rows);
+    FF_HIP(launch_gelu_mul(static_cast<hipStream_t>(stream), gate, gate_stride, up, up_stride, out, out_stride, rows, count, ctx->f16));
     return FFMOE_OK;
 }
 
@@ -1050,7 +1073,7 @@ int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_
     ffmoe_ctx *ctx = mx->ctx;
     ctx->timer.begin(static_cast<hipStream_t>(stream));
     FF_HIP(launch_matrix_gemv(static_cast<hipStream_t>(stream), mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows,
-                              y, y_stride, y_f32 != 0, ctx->n_cus, ctx->f16));
+                              y, y_stride, y_f32 != 0, ctx->n_cus, ctx->f16, mx->planes8));
     ctx->timer.mark(static_cast<hipStream_t>(stream), FFMOE_K_GEMV);
     ctx->timer.finish();
     return FFMOE_OK;
@@ -1060,7 +1083,7 @@ static int matrix_greedy_common(ffmoe_matrix *mx, void *stream, const uint16_t *
                                 float softcap, uint32_t *out_tokens, float *out_conf, char **err) {
     if (int rc = check_matrix_call(mx, x, x_stride, rows, err)) return rc;
     if (!out_tokens) return fail(err, FFMOE_ERR_INVALID, "null argument");
-    if (!mx->partials) return fail(err, FFMOE_ERR_INVALID, "matrix was created without the greedy scratch");
+    if (!mx->partials || mx->planes8) return fail(err, FFMOE_ERR_INVALID, "matrix was created without the greedy scratch");
     if (!(softcap >= 0.0f) || std::isinf(softcap)) return fail(err, FFMOE_ERR_INVALID, "softcap must be finite and >= 0 (0 disables it)");
     ffmoe_ctx *ctx = mx->ctx;
     hipStream_t s = static_cast<hipStream_t>(stream);

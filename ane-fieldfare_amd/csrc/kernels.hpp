@@ -184,14 +184,17 @@ hipError_t launch_reduce_token_major(hipStream_t s, const uint16_t *partials, co
                                      uint16_t *h2, uint32_t t, uint32_t top_k, uint32_t d, bool f16 = false);
 
 // matrix.hip: resident two-stream tiling of a [M][N] INT4 matrix, its multi-row GEMV and the greedy choice.
-size_t matrix_tiles_bytes(uint32_t m, uint32_t n);
-size_t matrix_scales_bytes(uint32_t m, uint32_t n);
+// planes8: the weight is an 8-bit affine one, kept as two nibble planes per 16-row tile (csrc/matrix.hip)
+size_t matrix_tiles_bytes(uint32_t m, uint32_t n, bool planes8 = false);
+size_t matrix_scales_bytes(uint32_t m, uint32_t n, bool planes8 = false);
 bool matrix_shape_ok(uint32_t n);
 hipError_t launch_matrix_repack(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
-                                uint32_t m, uint32_t n, uint8_t *tiles_out, uint8_t *scales_out);
+                                uint32_t m, uint32_t n, uint8_t *tiles_out, uint8_t *scales_out, bool planes8 = false);
 hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                               const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
-                              bool y_f32, uint32_t n_cus, bool f16 = false);
+                              bool y_f32, uint32_t n_cus, bool f16 = false, bool planes8 = false);
+hipError_t launch_gelu_mul(hipStream_t s, const uint16_t *gate, uint32_t gate_stride, const uint16_t *up, uint32_t up_stride,
+                           uint16_t *out, uint32_t out_stride, uint32_t rows, uint32_t count, bool f16);
 uint32_t greedy_segments(uint32_t m, uint32_t n_cus);
 // the GEMV with the greedy choice as its epilogue: per-block winners, then one block per input row
 hipError_t launch_matrix_greedy(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,

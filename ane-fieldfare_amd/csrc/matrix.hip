@@ -7,6 +7,11 @@
 // static-weight uses of DequantInt4GEMV.encodeRows (Kernels/Quant/DequantInt4GEMV.swift:72-182).
 // A tile holds rows a = 32 p + l % 16 (stream A) and a + 16 (stream B) of one 64-wide group, in the
 // same lane order as the expert arena, so the kernels share the expert path's register-ring code.
+//
+// An 8-bit affine weight (Metal/Quant/dequant_int8.metal:5-12: w = q s + b, q = 0 .. 255) rides the same kernels as two
+// 4-bit ones: q = 16 h + l, so w = (16 s) h + b + s l. A tile then holds rows 16 p + l % 16 twice - stream A their
+// high nibbles with scale 16 s (exact: a power of two) and bias b, stream B their low nibbles with scale s and bias
+// 0 - and an output is the sum of its two streams. Same bytes as the 8-bit matrix, same stream, same speed.
 #include "common.hpp"
 #include "kernels.hpp"
 #include "stream.hpp"
@@ -67,6 +72,49 @@ __global__ __launch_bounds__(256) void repack_matrix_kernel(const uint8_t *__res
     }
 }
 
+// The 8-bit form: w uint8 [m][n]. One thread per (tile, lane); a tile = 16 rows x one group, both nibble planes.
+__device__ __forceinline__ void nibble_planes8(const uint8_t *p, uint32_t &high, uint32_t &low) {
+    high = low = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        high |= (uint32_t)(p[i] >> 4) << (4 * i);
+        low |= (uint32_t)(p[i] & 15u) << (4 * i);
+    }
+}
+
+__global__ __launch_bounds__(256) void repack_matrix8_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ s,
+                                                             const uint8_t *__restrict__ b, uint32_t m, uint32_t n,
+                                                             uint8_t *__restrict__ tiles, uint8_t *__restrict__ scales) {
+    const uint32_t n_groups = n / kGroup;
+    const size_t n_tiles = (size_t)((m + 15) / 16) * n_groups;
+    const size_t total = n_tiles * kWave;
+    for (size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x; gid < total;
+         gid += (size_t)gridDim.x * blockDim.x) {
+        const uint32_t lane = gid & 63, i = lane & 15, jq = lane >> 4;
+        const size_t tile = gid >> 6;
+        const uint32_t rb = tile / n_groups, grp = tile % n_groups;
+        const uint32_t row = rb * kTileRows + i, k0 = grp * kGroup + 8 * jq;
+        uint4 chunk = {0, 0, 0, 0};
+        if (row < m) {
+            uint32_t h0, l0, h1, l1;
+            nibble_planes8(w + (size_t)row * n + k0, h0, l0);
+            nibble_planes8(w + (size_t)row * n + k0 + 32, h1, l1);
+            chunk = uint4{to_arena_order(h0), to_arena_order(h1), to_arena_order(l0), to_arena_order(l1)};
+        }
+        reinterpret_cast<uint4 *>(tiles + tile * kTileBytes)[lane] = chunk;
+        if (jq == 0) {
+            uint2 sc = {0, 0};
+            if (row < m) {
+                const size_t at = ((size_t)row * n_groups + grp) * 2;
+                const uint16_t scale = load_u16(s + at), bias = load_u16(b + at);
+                sc.x = (uint32_t)f32_to_bf16(bf16_to_f32(scale) * 16.0f) | ((uint32_t)bias << 16);
+                sc.y = (uint32_t)scale;
+            }
+            reinterpret_cast<uint2 *>(scales + tile * kTileScaleBytes)[i] = sc;
+        }
+    }
+}
+
 // Greedy choice per row: the largest finite value wins, ties go to the lowest index, NaN and +-inf never
 // win; a row with no candidate yields index 0 (Metal/Sampling/logit.metal:689-720, 916-921). Two stages: the
 // GEMV's blocks each leave the winner of the weight rows they walked, then one block per input row picks
@@ -117,7 +165,9 @@ __device__ __forceinline__ SoftmaxAcc softmax_shuffle(const SoftmaxAcc &a, int m
 // (value, index) key of the sums it finishes and the block leaves one key per input row in
 // y_[row * gridDim.x + block], so the [rows][m] fp32 logits never travel to memory and back. CONF: the block also
 // leaves the softmax pair of the sums it finished in conf_part[row * gridDim.x + block].
-template <bool Y_F32, bool F16, bool GREEDY = false, bool CONF = false>
+// PLANES8: the matrix is an 8-bit one stored as two nibble planes (above): a tile is 16 rows, an output the sum of its
+// two streams.
+template <bool Y_F32, bool F16, bool GREEDY = false, bool CONF = false, bool PLANES8 = false>
 __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__restrict__ tiles,
                                                              const uint8_t *__restrict__ scales, uint32_t m,
                                                              uint32_t n_groups, const uint16_t *__restrict__ x,
@@ -125,7 +175,8 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
                                                              uint32_t y_stride, float2 *__restrict__ conf_part = nullptr,
                                                              float softcap = 0.0f) {
     __shared__ float s_red[2][kKSplit][8][64];
-    const uint32_t n_tiles = (m + 31) / 32;
+    static_assert(!(PLANES8 && GREEDY), "the greedy choice is built for the 4-bit head only");
+    const uint32_t n_tiles = PLANES8 ? (m + 15) / 16 : (m + 31) / 32;
     uint32_t rb0, rb1;
     split_range(n_tiles, gridDim.x, blockIdx.x, rb0, rb1);
     if (rb0 >= rb1) {
@@ -180,7 +231,14 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
             va += s_red[buf][o][ks][lane];
             vb += s_red[buf][o][4 + ks][lane];
         }
-        if (my_row < rows) {
+        if (PLANES8) {
+            const uint32_t row = rb * kTileRows + j;
+            if (my_row < rows && row < m) {
+                const float v = va + vb;
+                if (Y_F32) y32[(size_t)my_row * y_stride + row] = v;
+                else y16[(size_t)my_row * y_stride + row] = Act<F16>::round(v);
+            }
+        } else if (my_row < rows) {
             const uint32_t row_a = rb * 2 * kTileRows + j, row_b = row_a + kTileRows;
             const size_t base = (size_t)my_row * y_stride;
             if (GREEDY) {
@@ -300,29 +358,65 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const float *__restric
 
 }  // namespace
 
-size_t matrix_tiles_bytes(uint32_t m, uint32_t n) { return (size_t)((m + 31) / 32) * (n / kGroup) * kTileBytes; }
-size_t matrix_scales_bytes(uint32_t m, uint32_t n) { return (size_t)((m + 31) / 32) * (n / kGroup) * kTileScaleBytes; }
+size_t matrix_tiles_bytes(uint32_t m, uint32_t n, bool planes8) {
+    return (size_t)(planes8 ? (m + 15) / 16 : (m + 31) / 32) * (n / kGroup) * kTileBytes;
+}
+size_t matrix_scales_bytes(uint32_t m, uint32_t n, bool planes8) {
+    return (size_t)(planes8 ? (m + 15) / 16 : (m + 31) / 32) * (n / kGroup) * kTileScaleBytes;
+}
 bool matrix_shape_ok(uint32_t n) { return n % kGroup == 0 && (n / kGroup + kKSplit - 1) / kKSplit <= (uint32_t)kRing; }
 
 hipError_t launch_matrix_repack(hipStream_t s, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
-                                uint32_t m, uint32_t n, uint8_t *tiles_out, uint8_t *scales_out) {
-    const size_t total = matrix_tiles_bytes(m, n) / kTileBytes * kWave;
+                                uint32_t m, uint32_t n, uint8_t *tiles_out, uint8_t *scales_out, bool planes8) {
+    const size_t total = matrix_tiles_bytes(m, n, planes8) / kTileBytes * kWave;
     const uint32_t blocks = (uint32_t)min((size_t)65535 * 16, (total + 255) / 256);
-    hipLaunchKernelGGL(repack_matrix_kernel, dim3(blocks), dim3(256), 0, s, w, reinterpret_cast<const uint8_t *>(scales),
-                       reinterpret_cast<const uint8_t *>(biases), m, n, tiles_out, scales_out);
+    if (planes8)
+        hipLaunchKernelGGL(repack_matrix8_kernel, dim3(blocks), dim3(256), 0, s, w, reinterpret_cast<const uint8_t *>(scales),
+                           reinterpret_cast<const uint8_t *>(biases), m, n, tiles_out, scales_out);
+    else
+        hipLaunchKernelGGL(repack_matrix_kernel, dim3(blocks), dim3(256), 0, s, w, reinterpret_cast<const uint8_t *>(scales),
+                           reinterpret_cast<const uint8_t *>(biases), m, n, tiles_out, scales_out);
     return hipGetLastError();
 }
 
 hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                               const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
-                              bool y_f32, uint32_t n_cus, bool f16) {
-    const uint32_t n_tiles = (m + 31) / 32;
+                              bool y_f32, uint32_t n_cus, bool f16, bool planes8) {
+    const uint32_t n_tiles = planes8 ? (m + 15) / 16 : (m + 31) / 32;
     const dim3 grid(min(2 * n_cus, n_tiles));
-#define FFMOE_MGEMV(Y, H) \
-    hipLaunchKernelGGL((matrix_gemv_kernel<Y, H>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, rows, y, y_stride)
-    if (f16) { if (y_f32) FFMOE_MGEMV(true, true); else FFMOE_MGEMV(false, true); }
-    else { if (y_f32) FFMOE_MGEMV(true, false); else FFMOE_MGEMV(false, false); }
+#define FFMOE_MGEMV(Y, H, P)                                                                                                \
+    hipLaunchKernelGGL((matrix_gemv_kernel<Y, H, false, false, P>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, \
+                       rows, y, y_stride)
+    if (planes8) {
+        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, true); else FFMOE_MGEMV(false, true, true); }
+        else { if (y_f32) FFMOE_MGEMV(true, false, true); else FFMOE_MGEMV(false, false, true); }
+    } else {
+        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, false); else FFMOE_MGEMV(false, true, false); }
+        else { if (y_f32) FFMOE_MGEMV(true, false, false); else FFMOE_MGEMV(false, false, false); }
+    }
 #undef FFMOE_MGEMV
+    return hipGetLastError();
+}
+
+// out = round16(gelu_tanh(gate) * up) per element of `rows` rows of `count` values: gelu_mul_fp16
+// (Metal/Primitives/utility.metal:4-17), the step between the projections of the 8-bit shared expert
+// (shared_int8_gate_up_act_simd rounds gate and up to 16 bits in front of it: Metal/Quant/dequant_int8.metal:131-136).
+template <bool F16>
+__global__ __launch_bounds__(256) void gelu_mul_kernel(const uint16_t *gate, uint32_t gate_stride, const uint16_t *up,
+                                                       uint32_t up_stride, uint16_t *out, uint32_t out_stride, uint32_t count) {
+    // no __restrict__: `out` may be `gate` or `up` itself (each element is read before it is written, by the same lane)
+    const uint32_t row = blockIdx.y;
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < count; i += gridDim.x * 256) {
+        const float g = Act<F16>::widen(gate[(size_t)row * gate_stride + i]), u = Act<F16>::widen(up[(size_t)row * up_stride + i]);
+        out[(size_t)row * out_stride + i] = Act<F16>::round(gelu_tanh_fast(g) * u);
+    }
+}
+
+hipError_t launch_gelu_mul(hipStream_t s, const uint16_t *gate, uint32_t gate_stride, const uint16_t *up, uint32_t up_stride,
+                           uint16_t *out, uint32_t out_stride, uint32_t rows, uint32_t count, bool f16) {
+    const dim3 grid(min(64u, (count + 255) / 256), rows);
+    if (f16) hipLaunchKernelGGL(gelu_mul_kernel<true>, grid, dim3(256), 0, s, gate, gate_stride, up, up_stride, out, out_stride, count);
+    else hipLaunchKernelGGL(gelu_mul_kernel<false>, grid, dim3(256), 0, s, gate, gate_stride, up, up_stride, out, out_stride, count);
     return hipGetLastError();
 }
 

@@ -50,6 +50,7 @@ EXPORTS = [
     "ffmoe_layer_tail", "ffmoe_layer_tail_routed", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
     "ffmoe_verify_static", "ffmoe_route_verify_shared", "ffmoe_layer_tail_routed_shared", "ffmoe_sample_rows",
+    "ffmoe_matrix_create_int8", "ffmoe_gelu_mul",
 ]
 
 PROFILE_SLOTS = 16
@@ -76,10 +77,11 @@ class Profile(C.Structure):
 class Matrix:
     """ffmoe_matrix: the LM head (or any static INT4 weight) kept re-tiled in HBM."""
 
-    def __init__(self, ctx, W, S, B, greedy: bool, w_byte_offset: int = 0):
+    def __init__(self, ctx, W, S, B, greedy: bool, w_byte_offset: int = 0, int8: bool = False):
         import numpy as np
         self.ctx, self.L = ctx, ctx.L
         self.m, self.n = int(S.shape[0]), int(S.shape[1]) * GROUP
+        self.int8 = int8
         keep = []
 
         def raw(a, off=0):
@@ -91,16 +93,20 @@ class Matrix:
             return C.c_void_p(a.data_ptr() + off)
 
         h, err = C.c_void_p(), C.c_char_p()
-        _check(self.L.ffmoe_matrix_create(ctx._h, raw(W, w_byte_offset), raw(S), raw(B), self.m, self.n, int(greedy),
-                                          C.byref(h), C.byref(err)), err)
+        if int8:
+            _check(self.L.ffmoe_matrix_create_int8(ctx._h, raw(W, w_byte_offset), raw(S), raw(B), self.m, self.n,
+                                                   C.byref(h), C.byref(err)), err)
+        else:
+            _check(self.L.ffmoe_matrix_create(ctx._h, raw(W, w_byte_offset), raw(S), raw(B), self.m, self.n, int(greedy),
+                                              C.byref(h), C.byref(err)), err)
         self._h = h
 
-    def gemv(self, x, f32_out: bool = False):
+    def gemv(self, x, f32_out: bool = False, out=None):
         import torch
         rows = x.shape[0]
-        y = torch.empty((rows, self.m), dtype=torch.float32 if f32_out else self.ctx.act, device=x.device)
+        y = torch.empty((rows, self.m), dtype=torch.float32 if f32_out else self.ctx.act, device=x.device) if out is None else out
         err = C.c_char_p()
-        _check(self.L.ffmoe_matrix_gemv(self._h, _stream(), _ptr(x), _row_stride(x), rows, _ptr(y), self.m,
+        _check(self.L.ffmoe_matrix_gemv(self._h, _stream(), _ptr(x), _row_stride(x), rows, _ptr(y), _row_stride(y),
                                         int(f32_out), C.byref(err)), err)
         return y
 
@@ -227,6 +233,8 @@ def lib() -> C.CDLL:
     L.ffmoe_prefill_pairs.argtypes = [vp, vp, u32, vp, u32, vp, u32, u32, vp, errp]
     L.ffmoe_prefill_plan_stats.argtypes = [vp, vp, C.POINTER(u32), C.POINTER(u32), vp, errp]
     L.ffmoe_matrix_create.argtypes = [vp, vp, vp, vp, u32, u32, i32, C.POINTER(vp), errp]
+    L.ffmoe_matrix_create_int8.argtypes = [vp, vp, vp, vp, u32, u32, C.POINTER(vp), errp]
+    L.ffmoe_gelu_mul.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, u32, u32, errp]
     L.ffmoe_matrix_destroy.argtypes = [vp]
     L.ffmoe_matrix_destroy.restype = None
     L.ffmoe_matrix_gemv.argtypes = [vp, vp, vp, u32, u32, vp, u32, i32, errp]
@@ -617,6 +625,20 @@ class Context:
     def matrix(self, W, S, B, greedy: bool = False, w_byte_offset: int = 0):
         """Resident re-tiled copy of W uint8 [M, N/2], S/B bf16 bits [M, N/64] (numpy arrays or tensors)."""
         return Matrix(self, W, S, B, greedy, w_byte_offset)
+
+    def matrix_int8(self, W, S, B):
+        """Resident copy of an 8-bit affine weight: W uint8 [M, N], S/B bf16 bits [M, N/64] (numpy arrays or tensors)."""
+        return Matrix(self, W, S, B, False, 0, int8=True)
+
+    def gelu_mul(self, gate, up, out=None):
+        """out = round16(gelu_tanh(gate) * up), rows of the activation type (2-D tensors of one shape)."""
+        import torch
+        rows, count = gate.shape
+        out = torch.empty((rows, count), dtype=gate.dtype, device=gate.device) if out is None else out
+        err = C.c_char_p()
+        _check(self.L.ffmoe_gelu_mul(self._h, _stream(), _ptr(gate), _row_stride(gate), _ptr(up), _row_stride(up), _ptr(out),
+                                     _row_stride(out), rows, count, C.byref(err)), err)
+        return out
 
     def argmax_rows(self, logits, count: int | None = None, softcap: float = 0.0, want_conf: bool = True):
         """Greedy position per row of fp32 logits [rows, >= count] (int32, -1 when no value is finite) and, with

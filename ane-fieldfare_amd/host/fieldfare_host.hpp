@@ -631,15 +631,122 @@ protected:
     Context &c_;
 };
 
-// SharedExpertRuntime (SharedExpertInt4.swift:92-130): picks the implementation by weight width; only the
-// 4-bit one is part of this library.
-class SharedExpertRuntime : public SharedExpertInt4 {
+// DequantInt8GEMV (Kernels/Quant/DequantInt8GEMV.swift:7-56): y = W x with W 8-bit affine (uint8 [m][n], scales / biases
+// bf16 [m][n/64]). The Swift operator binds the weight on every call; here the weight is re-tiled once and owned, and a
+// call takes 1...16 rows of x with one pass over it.
+class DequantInt8GEMV {
 public:
-    SharedExpertRuntime(Context &dense, int weightBits) : SharedExpertInt4(dense) {
-        if (weightBits != 4)
+    static constexpr int maxBatchRows = 16;
+    DequantInt8GEMV(Context &c, const uint8_t *weights, const uint16_t *scales, const uint16_t *biases, uint32_t m, uint32_t n)
+        : m_(m), n_(n) {
+        if (n % FFMOE_GROUP) throw std::invalid_argument("N must be a multiple of 64");
+        char *err = nullptr;
+        check(ffmoe_matrix_create_int8(c.raw(), weights, scales, biases, m, n, &mx_, &err), err);
+    }
+    ~DequantInt8GEMV() { ffmoe_matrix_destroy(mx_); }
+    DequantInt8GEMV(const DequantInt8GEMV &) = delete;
+    DequantInt8GEMV &operator=(const DequantInt8GEMV &) = delete;
+    // encode (DequantInt8GEMV.swift:25-56): one row
+    void encode(void *stream, const uint16_t *x, uint16_t *y) { encodeRows(stream, x, y, 1, n_, m_); }
+    void encodeRows(void *stream, const uint16_t *x, uint16_t *y, int rows, uint32_t xStrideElements, uint32_t yStrideElements) {
+        if (rows <= 0 || rows > maxBatchRows) throw std::invalid_argument("rows outside 1...16");
+        char *err = nullptr;
+        check(ffmoe_matrix_gemv(mx_, stream, x, xStrideElements, (uint32_t)rows, y, yStrideElements, 0, &err), err);
+    }
+    uint32_t m() const { return m_; }
+    uint32_t n() const { return n_; }
+
+private:
+    ffmoe_matrix *mx_ = nullptr;
+    uint32_t m_, n_;
+};
+
+// SharedExpertInt8 (Kernels/MoE/SharedExpertInt8.swift:40-97): y = down(gelu_tanh(gate(x)) * up(x)) with the three
+// projections 8-bit affine, the form in which the packs hold the shared expert by default. The Swift class binds
+// the projections on every call; here load() re-tiles one layer's three once and the object keeps them. The caller's
+// activation scratch holds gate(x) and up(x) side by side - 2 * F values per row where the Swift kernel, which fuses the
+// two projections with the activation, needs F - and may be reused across layers, as there.
+class SharedExpertInt8 {
+public:
+    static constexpr int maxBatchRows = DequantInt8GEMV::maxBatchRows;
+    explicit SharedExpertInt8(Context &c) : c_(c) {}
+    // the guards of SharedExpertInt8.encode (SharedExpertInt8.swift:63-70), then the three uploads
+    void load(const SharedExpertProjection &gate, const SharedExpertProjection &up, const SharedExpertProjection &down) {
+        if (gate.rows != up.rows || gate.cols != up.cols)
+            throw SharedExpertError(SharedExpertError::dimensionMismatch,
+                                    "gate/up shapes differ: gate=(" + std::to_string(gate.rows) + "," + std::to_string(gate.cols) +
+                                        ") up=(" + std::to_string(up.rows) + "," + std::to_string(up.cols) + ")");
+        if (down.rows != gate.cols || down.cols != gate.rows)
+            throw SharedExpertError(SharedExpertError::dimensionMismatch,
+                                    "down expected (" + std::to_string(gate.cols) + "," + std::to_string(gate.rows) + "), got (" +
+                                        std::to_string(down.rows) + "," + std::to_string(down.cols) + ")");
+        gate_.reset(new DequantInt8GEMV(c_, gate.weights, gate.scales, gate.biases, gate.rows, gate.cols));
+        up_.reset(new DequantInt8GEMV(c_, up.weights, up.scales, up.biases, up.rows, up.cols));
+        down_.reset(new DequantInt8GEMV(c_, down.weights, down.scales, down.biases, down.rows, down.cols));
+    }
+    // encode (SharedExpertInt8.swift:56-97): one row; scratchActElements is the room behind scratchAct in 16-bit values
+    void encode(void *stream, const uint16_t *x, uint16_t *y, uint16_t *scratchAct, size_t scratchActElements) {
+        encodeBlock(stream, x, y, 1, (int)d(), (int)d(), scratchAct, scratchActElements);
+    }
+    // a block of rows, each as encode does it; more than 16 rows go through in parts of 16 that reuse the scratch
+    void encodeBlock(void *stream, const uint16_t *x, uint16_t *y, int queryCount, int xStrideElements, int yStrideElements,
+                     uint16_t *scratchAct, size_t scratchActElements) {
+        if (!gate_) throw std::logic_error("SharedExpertInt8: load() first");
+        if (queryCount < 0) throw std::invalid_argument("queryCount must be non-negative");
+        if (xStrideElements < (int)d()) throw std::invalid_argument("x stride is too small");
+        if (yStrideElements < (int)d()) throw std::invalid_argument("y stride is too small");
+        const uint32_t f = gate_->m(), pitch = (f + 7u) & ~7u;      // rows of the scratch stay 16-byte aligned
+        const int part = queryCount < maxBatchRows ? queryCount : maxBatchRows;
+        if (scratchActElements < (size_t)2 * part * pitch)
+            throw SharedExpertError(SharedExpertError::scratchTooSmall,
+                                    "scratchAct needs " + std::to_string((size_t)2 * part * pitch) + " values, has " +
+                                        std::to_string(scratchActElements));
+        uint16_t *g = scratchAct, *u = scratchAct + (size_t)part * pitch;
+        for (int r0 = 0; r0 < queryCount; r0 += maxBatchRows) {
+            const int rows = queryCount - r0 < maxBatchRows ? queryCount - r0 : maxBatchRows;
+            const uint16_t *xr = x + (size_t)r0 * xStrideElements;
+            gate_->encodeRows(stream, xr, g, rows, (uint32_t)xStrideElements, pitch);
+            up_->encodeRows(stream, xr, u, rows, (uint32_t)xStrideElements, pitch);
+            char *err = nullptr;
+            check(ffmoe_gelu_mul(c_.raw(), stream, g, pitch, u, pitch, g, pitch, (uint32_t)rows, f, &err), err);
+            down_->encodeRows(stream, g, y + (size_t)r0 * yStrideElements, rows, pitch, (uint32_t)yStrideElements);
+        }
+    }
+    uint32_t d() const { return gate_ ? gate_->n() : 0; }
+    uint32_t intermediate() const { return gate_ ? gate_->m() : 0; }
+
+private:
+    Context &c_;
+    std::unique_ptr<DequantInt8GEMV> gate_, up_, down_;
+};
+
+// SharedExpertRuntime (SharedExpertInt4.swift:92-130): picks the implementation by weight width. For 4 bits `c` is the
+// one-expert context SharedExpertInt4 takes and the calls name the layer; for 8 bits `c` is any context, one object
+// serves one layer (the `layer` arguments are ignored) and encode needs the activation scratch.
+class SharedExpertRuntime {
+public:
+    SharedExpertRuntime(Context &c, int weightBits) {
+        if (weightBits == 4) int4_.reset(new SharedExpertInt4(c));
+        else if (weightBits == 8) int8_.reset(new SharedExpertInt8(c));
+        else
             throw SharedExpertError(SharedExpertError::unsupportedWeightBits,
                                     "SharedExpert unsupported weight bits: " + std::to_string(weightBits));
     }
+    int weightBits() const { return int4_ ? 4 : 8; }
+    void load(uint32_t layer, const SharedExpertProjection &gate, const SharedExpertProjection &up,
+              const SharedExpertProjection &down) {
+        if (int4_) int4_->load(layer, gate, up, down);
+        else int8_->load(gate, up, down);
+    }
+    void encode(void *stream, uint32_t layer, const uint16_t *x, uint16_t *y, uint16_t *scratchAct = nullptr,
+                size_t scratchActElements = 0) {
+        if (int4_) int4_->encode(stream, layer, x, y);
+        else int8_->encode(stream, x, y, scratchAct, scratchActElements);
+    }
+
+private:
+    std::unique_ptr<SharedExpertInt4> int4_;
+    std::unique_ptr<SharedExpertInt8> int8_;
 };
 
 // PrefillSharedExpert.encodeBlock (PrefillSharedExpert.swift:94-137): a block of rows. The Swift class loops

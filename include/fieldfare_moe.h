@@ -300,6 +300,16 @@ typedef struct ffmoe_matrix ffmoe_matrix;
  * hot-path call. */
 int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                         uint32_t m, uint32_t n, int with_greedy, ffmoe_matrix **out, char **err);
+/* The same for an 8-bit affine weight (W uint8 [m][n], one value per byte, S/B bf16 [m][n/64]: w = q s + b with
+ * q = 0 .. 255, Metal/Quant/dequant_int8.metal:5-12): the form in which the reference's packs hold the shared expert
+ * by default (Model.sharedExpertWeightBits, Runtime/Inference/Model.swift:13). The matrix then serves
+ * ffmoe_matrix_gemv (not the greedy calls) and replaces DequantInt8GEMV.encode
+ * (Kernels/Quant/DequantInt8GEMV.swift:26-56, kernel dequant_int8_gemv_simd, dequant_int8.metal:41-83) for 1 to 16
+ * rows per call. Held as two 4-bit planes per 16-row tile (q = 16 h + l: the high nibbles with scale 16 s and the
+ * bias, the low ones with scale s), so it takes m x n bytes + scales like the source and streams at the 4-bit
+ * matrix's rate. */
+int ffmoe_matrix_create_int8(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                             uint32_t m, uint32_t n, ffmoe_matrix **out, char **err);
 /* A matrix belongs to the context it was created on. Destroying that context first releases the matrix's
  * device memory; the handle then only accepts ffmoe_matrix_destroy (compute calls return FFMOE_ERR_INVALID). */
 void ffmoe_matrix_destroy(ffmoe_matrix *mx);
@@ -310,6 +320,16 @@ void ffmoe_matrix_destroy(ffmoe_matrix *mx);
  * [rows][x_stride], 16-byte aligned, stride a multiple of 8; y bf16 or (y_f32 != 0) fp32 [rows][y_stride]. */
 int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
                       void *y, uint32_t y_stride, int y_f32, char **err);
+
+/* out[r][i] = round16(gelu_tanh(gate[r][i]) * up[r][i]) for `rows` rows of `count` values in the context's activation
+ * type: gelu_mul_fp16 (Metal/Primitives/utility.metal:4-17, run by PrefillSharedExpert.encodeBatched,
+ * Kernels/Prefill/MoE/PrefillSharedExpert.swift:78-91), and with two ffmoe_matrix_gemv calls in front and one behind
+ * the 8-bit shared expert: SharedExpertInt8.encode (Kernels/MoE/SharedExpertInt8.swift:56-97; its fused kernel
+ * shared_int8_gate_up_act_simd rounds gate and up to 16 bits before the activation just as the separate calls do,
+ * dequant_int8.metal:131-136). Strides in elements, each at least `count`; `out` may be `gate` or `up` itself (same
+ * pointer and stride), and no other overlap is allowed. */
+int ffmoe_gelu_mul(ffmoe_ctx *ctx, void *stream, const uint16_t *gate, uint32_t gate_stride, const uint16_t *up,
+                   uint32_t up_stride, uint16_t *out, uint32_t out_stride, uint32_t rows, uint32_t count, char **err);
 
 /* Greedy token per row: the fp32 logits of the GEMV above and, as that kernel's epilogue (the logits are
  * never written out), the index of the largest finite logit,

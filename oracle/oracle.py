@@ -253,6 +253,14 @@ def gemv_int4_ref(W, S, B, x) -> np.ndarray:
     return y
 
 
+def gemv_int8_ref(W, S, B, x) -> np.ndarray:
+    """DequantInt8GemvRef.apply (Tests/Support/Validation/Reference/Quant/DequantInt8Gemv.swift:8-37) for one input
+    vector: every row dequantised (Quantization.dequantizeInt8Affine), then a dot product - in float64 here, where the
+    reference's vDSP_dotpr sums in fp32 (it is a tolerance reference there as well)."""
+    rows = dequantize_int8(W, S, B).astype(np.float64)
+    return (rows @ np.ascontiguousarray(x, np.float64)).astype(np.float32)
+
+
 def gelu_tanh(x) -> np.ndarray:
     x = np.atleast_1d(np.asarray(x, np.float32))
     return np.array([lib().ffo_gelu_tanh(float(v)) for v in x.ravel()], np.float32).reshape(x.shape)

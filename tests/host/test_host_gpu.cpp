@@ -283,7 +283,7 @@ int main() {
         try { shared.load(0, gate, down, down); } catch (const SharedExpertError &e) { threwDims = e.kind == SharedExpertError::dimensionMismatch; }
         EXPECT(threwDims);
         bool threwBits = false;
-        try { SharedExpertRuntime bad(dense, 8); } catch (const SharedExpertError &e) { threwBits = e.kind == SharedExpertError::unsupportedWeightBits; }
+        try { SharedExpertRuntime bad(dense, 6); } catch (const SharedExpertError &e) { threwBits = e.kind == SharedExpertError::unsupportedWeightBits; }
         EXPECT(threwBits);
         shared.load(0, gate, up, down);
         ffo_offsets fo{off.gate_w, off.gate_s, off.gate_b, off.up_w, off.up_s, off.up_b, off.down_w, off.down_s, off.down_b};
@@ -337,6 +337,77 @@ int main() {
         asBf16Ref(toHost(dH2, (size_t)d), std::vector<float>(refAll.begin(), refAll.begin() + d), relS, cosS);
         EXPECT(relS <= 1e-2 && cosS >= 0.9999);
         HIP(hipFree(dxh));
+    }
+
+    // --- the 8-bit shared expert (SharedExpertInt8, the packs' default form): 1 row and a 40-row block against the
+    // dequantised rows in double with the operator's 16-bit roundings (gate, up, activation), and its guards ---
+    {
+        struct Proj8 { std::vector<uint8_t> w; std::vector<uint16_t> s, b; std::vector<float> deq; };
+        auto make8 = [&](int rows, int cols) {
+            Proj8 p;
+            p.w.resize((size_t)rows * cols); p.s.resize((size_t)rows * cols / 64); p.b.resize(p.s.size()); p.deq.resize(p.w.size());
+            std::vector<float> row(cols);
+            for (int r = 0; r < rows; ++r) {
+                ffo_splitmix64_fill_uniform(&rng, -0.08f, 0.08f, row.data(), (size_t)cols);
+                ffo_quantize_int8_affine(row.data(), cols, &p.w[(size_t)r * cols], &p.s[(size_t)r * cols / 64], &p.b[(size_t)r * cols / 64]);
+                ffo_dequantize_int8_affine(&p.w[(size_t)r * cols], &p.s[(size_t)r * cols / 64], &p.b[(size_t)r * cols / 64], cols,
+                                           &p.deq[(size_t)r * cols]);
+            }
+            return p;
+        };
+        const Proj8 g8 = make8(f, d), u8 = make8(f, d), d8 = make8(d, f);
+        const SharedExpertProjection gate{g8.w.data(), g8.s.data(), g8.b.data(), (uint32_t)f, (uint32_t)d};
+        const SharedExpertProjection up{u8.w.data(), u8.s.data(), u8.b.data(), (uint32_t)f, (uint32_t)d};
+        const SharedExpertProjection down{d8.w.data(), d8.s.data(), d8.b.data(), (uint32_t)d, (uint32_t)f};
+        std::vector<float> ref8((size_t)T * d), act(f);
+        for (int r = 0; r < T; ++r) {
+            for (int j = 0; j < f; ++j) {
+                double ga = 0, ua = 0;
+                for (int i = 0; i < d; ++i) {
+                    const double xi = ffo_bf16_to_float(x[(size_t)r * d + i]);
+                    ga += (double)g8.deq[(size_t)j * d + i] * xi;
+                    ua += (double)u8.deq[(size_t)j * d + i] * xi;
+                }
+                const float gr = ffo_bf16_to_float(ffo_bf16_bits((float)ga)), ur = ffo_bf16_to_float(ffo_bf16_bits((float)ua));
+                act[j] = ffo_bf16_to_float(ffo_bf16_bits(ffo_gelu_tanh(gr) * ur));
+            }
+            for (int i = 0; i < d; ++i) {
+                double ya = 0;
+                for (int j = 0; j < f; ++j) ya += (double)d8.deq[(size_t)i * f + j] * act[j];
+                ref8[(size_t)r * d + i] = (float)ya;
+            }
+        }
+        SharedExpertInt8 shared8(ctx);
+        bool threwDims = false, threwScratch = false, threwUnloaded = false;
+        try { shared8.encode(stream, dx, dH2, nullptr, 0); } catch (const std::logic_error &) { threwUnloaded = true; }
+        EXPECT(threwUnloaded);
+        try { shared8.load(gate, up, up); } catch (const SharedExpertError &e) { threwDims = e.kind == SharedExpertError::dimensionMismatch; }
+        EXPECT(threwDims);
+        shared8.load(gate, up, down);
+        EXPECT(shared8.d() == (uint32_t)d && shared8.intermediate() == (uint32_t)f);
+        const size_t scratchValues = (size_t)2 * 16 * ((f + 7) & ~7);
+        uint16_t *dScratch = nullptr;
+        HIP(hipMalloc(&dScratch, scratchValues * 2));
+        try { shared8.encodeBlock(stream, dx, dH2b, T, d, d, dScratch, scratchValues - 1); }
+        catch (const SharedExpertError &e) { threwScratch = e.kind == SharedExpertError::scratchTooSmall; }
+        EXPECT(threwScratch);
+        shared8.encode(stream, dx, dH2, dScratch, scratchValues);
+        shared8.encodeBlock(stream, dx, dH2b, T, d, d, dScratch, scratchValues);
+        HIP(hipStreamSynchronize(stream));
+        double rel8 = 0, cos8 = 0;
+        errorStats(toHost(dH2, (size_t)d), std::vector<float>(ref8.begin(), ref8.begin() + d), rel8, cos8);
+        EXPECT(rel8 <= 1e-2 && cos8 >= 0.9999);
+        errorStats(toHost(dH2b, (size_t)T * d), ref8, rel8, cos8);
+        EXPECT(rel8 <= 1e-2 && cos8 >= 0.9999);
+        // the runtime that picks by weight width, on the same weights: the same row, bit for bit
+        const std::vector<uint16_t> row0 = toHost(dH2, (size_t)d);
+        SharedExpertRuntime runtime8(ctx, 8);
+        EXPECT(runtime8.weightBits() == 8);
+        runtime8.load(0, gate, up, down);
+        runtime8.encode(stream, 0, dx, dH2, dScratch, scratchValues);
+        HIP(hipStreamSynchronize(stream));
+        EXPECT(toHost(dH2, (size_t)d) == row0);
+        HIP(hipFree(dScratch));
     }
 
     // --- post-attention setup and layer tail through the mirrored classes: a 5-row block against the oracle's

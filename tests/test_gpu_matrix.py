@@ -291,3 +291,139 @@ def test_sample_rows_argument_errors(ctx, ff, torch):
                           (dict(temperature=1.0, softcap=30.0, top_k=8, top_p=0.0), "top_p")):
         with pytest.raises(ff.FieldfareError, match=match):
             ctx.sample_rows(logits, kwargs["temperature"], kwargs["softcap"], 1, top_k=kwargs.get("top_k", 0), top_p=kwargs.get("top_p", 1.0))
+
+
+# ---- the 8-bit affine matrix and the 8-bit shared expert built from it ------------------------------------------
+
+def _shared_int8(ctx, parts):
+    (gW, gS, gB), (uW, uS, uB), (dW, dS, dB) = parts
+    return ctx.matrix_int8(gW, gS, gB), ctx.matrix_int8(uW, uS, uB), ctx.matrix_int8(dW, dS, dB)
+
+
+def _shared_int8_rows(ctx, mats, x):
+    gate, up, down = mats
+    return down.gemv(ctx.gelu_mul(gate.gemv(x), up.gemv(x)))
+
+
+def _shared_int8_reference(oracle, parts, x_rows, widen, narrow):
+    """SharedExpertInt8Tests.swift:33-41: DequantInt8GemvRef for gate and up, gelu_pytorch_tanh(gate) * up rounded to 16
+    bits once, DequantInt8GemvRef for down."""
+    (gW, gS, gB), (uW, uS, uB), (dW, dS, dB) = parts
+    out = []
+    for row in x_rows:
+        x = widen(row)
+        g, u = oracle.gemv_int8_ref(gW, gS, gB, x), oracle.gemv_int8_ref(uW, uS, uB, x)
+        g64 = g.astype(np.float64)
+        act = (0.5 * g64 * (1.0 + np.tanh(0.7978845608028654 * (g64 + 0.044715 * g64 ** 3)))).astype(np.float32) * u
+        out.append(oracle.gemv_int8_ref(dW, dS, dB, widen(narrow(act))))
+    return np.stack(out)
+
+
+@pytest.mark.parametrize("act", ["bf16", "fp16"])
+def test_shared_expert_int8_matches_reference(ff, oracle, torch, act):
+    # sharedExpertInt8_matchesReference (SharedExpertInt8Tests.swift:19-72): same seed, draw order, shapes and reference;
+    # the reference's bound is Tolerance.quantInt8 * 4 = 4e-3 on FP16 outputs, bf16 outputs carry 2^-9 on top
+    d, f = 128, 64
+    rng = oracle.seed_tree_key(0x601, "shared-expert-int8")
+    x = rng.uniform(-0.4, 0.4, d)
+    gate = np.stack([rng.uniform(-0.4, 0.4, d) for _ in range(f)])
+    up = np.stack([rng.uniform(-0.4, 0.4, d) for _ in range(f)])
+    down = np.stack([rng.uniform(-0.4, 0.4, f) for _ in range(d)])
+    parts = (oracle.quantize_int8(gate), oracle.quantize_int8(up), oracle.quantize_int8(down))
+    c = ff.Context(128, 64, 16, 8, n_layers=1, max_tokens=16, act_dtype=act)
+    if act == "fp16":
+        widen = lambda b: np.ascontiguousarray(b, np.uint16).view(np.float16).astype(np.float32)
+        narrow = lambda v: np.ascontiguousarray(v, np.float32).astype(np.float16).view(np.uint16)
+        xt = torch.from_numpy(narrow(x)[None, :].view(np.int16)).cuda().view(torch.float16)
+    else:
+        widen, narrow = oracle.bf16_to_float, oracle.bf16_bits
+        xt = bf16_tensor(torch, narrow(x)[None, :])
+    ref = _shared_int8_reference(oracle, parts, narrow(x)[None, :], widen, narrow)
+    mats = _shared_int8(c, parts)
+    y = widen(bits_of(_shared_int8_rows(c, mats, xt)))
+    assert rel_err(y, ref) < (4e-3 if act == "fp16" else 1e-2), rel_err(y, ref)
+    for m_ in mats:
+        m_.close()
+    c.close()
+
+
+def test_int8_matrix_block_equals_repeated_single_rows(ctx, oracle, torch):
+    # blockSharedExpertMatchesRepeatedScalarRows (PrefillSharedExpertTests.swift:15-82): four rows with an input stride of
+    # 144 and an output stride of 137 over sentinels - the block call equals the four single-row calls bit for bit,
+    # padding included (here per projection: every stage of the expert is such a call)
+    import ctypes as C
+    rows, d, f, xs, ys = 4, 128, 64, 144, 137
+    rng = oracle.seed_tree_key(0xC0FFEE, "prefill-shared-expert")
+    sentinel = oracle.bf16_bits(np.float32(-7.25))
+    xb = np.full((rows, xs), sentinel, np.uint16)
+    for r in range(rows):
+        xb[r, :d] = oracle.bf16_bits(rng.uniform(-0.35, 0.35, d))
+    W, S, B = oracle.quantize_int8(np.stack([rng.uniform(-0.4, 0.4, d) for _ in range(f)]))
+    mx = ctx.matrix_int8(W, S, B)
+    x = bf16_tensor(torch, xb)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def run(first, count):
+        y = bf16_tensor(torch, np.full((rows, ys), sentinel, np.uint16))
+        err = C.c_char_p()
+        for r in (range(first, first + count) if count == 1 else [first]):
+            n = 1 if count == 1 else count
+            rc = ctx.L.ffmoe_matrix_gemv(mx._h, stream, C.c_void_p(x.data_ptr() + r * xs * 2), xs, n,
+                                         C.c_void_p(y.data_ptr() + r * ys * 2), ys, 0, C.byref(err))
+            assert rc == 0, err.value
+        return y
+
+    block = run(0, rows)
+    single = bf16_tensor(torch, np.full((rows, ys), sentinel, np.uint16))
+    for r in range(rows):
+        single[r] = run(r, 1)[r]
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(block), bits_of(single))
+    assert np.array_equal(bits_of(block)[:, f:], np.full((rows, ys - f), sentinel, np.uint16))
+    ref = np.stack([oracle.gemv_int8_ref(W, S, B, oracle.bf16_to_float(xb[r, :d])) for r in range(rows)])
+    assert rel_err(oracle.bf16_to_float(bits_of(block)[:, :f]), ref) < 1e-2
+    mx.close()
+
+
+@pytest.mark.parametrize("m,n,rows", [(2112, 2816, 1), (2112, 2816, 16), (2816, 2112, 16), (300, 2112, 3), (17, 64, 5)])
+def test_int8_matrix_gemv_shapes(ctx, ff, oracle, torch, m, n, rows):
+    # the 26B-A4B shared expert's projections (gate / up 2112 x 2816, down 2816 x 2112: DequantInt8GEMV.swift:12-19) and
+    # ragged row counts; fp32 outputs against the float64 reference, 16-bit outputs = their rounding, row r of a block
+    # = the single-row call bit for bit; q = 0 and q = 255 in every group exercise both nibble planes' ends
+    g = oracle.seed_tree_key(0xE8 + rows, f"matrix8-m{m}-n{n}-r{rows}")
+    W, S, B = oracle.quantize_int8(g.uniform(-0.5, 0.5, m * n).reshape(m, n))
+    assert W.min() == 0 and W.max() == 255
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, rows * n)).reshape(rows, n)
+    mx = ctx.matrix_int8(torch.from_numpy(W).cuda(), _i16(torch, S), _i16(torch, B)) if rows % 2 else ctx.matrix_int8(W, S, B)
+    x = bf16_tensor(torch, xb)
+    y32 = mx.gemv(x, f32_out=True).cpu().numpy()
+    y16 = bits_of(mx.gemv(x))
+    for r in range(rows):
+        ref = oracle.gemv_int8_ref(W, S, B, oracle.bf16_to_float(xb[r]))
+        assert rel_err(y32[r], ref) < 1e-3, (r, rel_err(y32[r], ref))        # Tolerance.quantInt8
+        assert np.array_equal(y16[r], oracle.bf16_bits(y32[r]))
+        single = mx.gemv(x[r:r + 1], f32_out=True).cpu().numpy()[0]
+        assert np.array_equal(single.view(np.uint32), y32[r].view(np.uint32)), f"row {r}"
+    with pytest.raises(ff.FieldfareError, match="greedy"):
+        mx.greedy(x)
+    mx.close()
+
+
+def test_gelu_mul_and_int8_argument_errors(ctx, ff, oracle, torch):
+    g = np.random.default_rng(3)
+    a, b = (oracle.bf16_bits(g.normal(0, 2, (5, 200)).astype(np.float32)) for _ in range(2))
+    a[0, :4] = oracle.bf16_bits(np.array([0.0, -0.0, 30.0, -30.0], np.float32))
+    out = bits_of(ctx.gelu_mul(bf16_tensor(torch, a), bf16_tensor(torch, b)))
+    x = oracle.bf16_to_float(a).astype(np.float64)
+    want = 0.5 * x * (1.0 + np.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3))) * oracle.bf16_to_float(b)
+    # the tanh form in float64 (utility.metal:4-17 states it in single precision, where 1 + tanh cancels for inputs
+    # below about -4): the kernels' form, x / (1 + exp(-2 * inner)), has no cancellation and follows it to a bf16 step
+    assert (np.abs(oracle.bf16_to_float(out) - want) <= 2.0 ** -7 * np.abs(want) + 1e-7).all()
+    near = np.abs(x) <= 3.0                            # and the single-precision oracle where that one is accurate
+    want32 = oracle.gelu_tanh(oracle.bf16_to_float(a)) * oracle.bf16_to_float(b)
+    assert (np.abs(oracle.bf16_to_float(out) - want32)[near] <= 2.0 ** -7 * np.abs(want32)[near] + 1e-7).all()
+    ga = bf16_tensor(torch, a)
+    assert ctx.gelu_mul(ga, bf16_tensor(torch, b), out=ga) is ga and (bits_of(ga) == out).all()   # in place, over the gate
+    W, S, B = oracle.quantize_int8(g.uniform(-1, 1, (8, 100 * 64)).astype(np.float32))
+    with pytest.raises(ff.FieldfareError, match="at most"):
+        ctx.matrix_int8(W, S, B)                       # N beyond what a wave's register ring holds
