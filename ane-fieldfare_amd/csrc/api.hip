@@ -33,6 +33,7 @@ struct ffmoe_matrix {
     int device = 0;
     uint32_t m = 0, n = 0;
     bool planes8 = false;         // an 8-bit weight kept as two nibble planes (ffmoe_matrix_create_int8)
+    bool glu = false;             // gate and up projections interleaved 16 rows at a time; m = the outputs of the gated product
     uint8_t *tiles = nullptr, *scales = nullptr;
     unsigned long long *partials = nullptr;   // [16][blocks of the GEMV grid]: per-block winners of the greedy choice
 };
@@ -1024,6 +1025,57 @@ int ffmoe_matrix_create_int8(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *s
     return matrix_create_common(ctx, w, scales, biases, m, n, 0, true, out, err);
 }
 
+int ffmoe_matrix_create_int8_glu(ffmoe_ctx *ctx, const uint8_t *gate_w, const uint16_t *gate_scales, const uint16_t *gate_biases,
+                                 const uint8_t *up_w, const uint16_t *up_scales, const uint16_t *up_biases, uint32_t f, uint32_t n,
+                                 ffmoe_matrix **out, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (!gate_w || !gate_scales || !gate_biases || !up_w || !up_scales || !up_biases || !out)
+        return fail(err, FFMOE_ERR_INVALID, "null argument");
+    *out = nullptr;
+    if (f == 0 || f > (1u << 24)) return fail(err, FFMOE_ERR_INVALID, "F = %u outside 1...2^24", f);
+    if (n == 0 || !matrix_shape_ok(n))
+        return fail(err, FFMOE_ERR_INVALID, "N = %u must be a multiple of %d and at most %d", n, FFMOE_GROUP, FFMOE_MATRIX_MAX_N);
+    // one source matrix on the device with the two projections' rows interleaved 16 at a time (rows past F stay zero)
+    const uint32_t full = f / 16, rest = f % 16, rows2 = 32 * ((f + 15) / 16), groups = n / FFMOE_GROUP;
+    const size_t w_bytes = (size_t)rows2 * n, s_bytes = (size_t)rows2 * groups * 2;
+    const size_t w_pad = (w_bytes + 15) / 16 * 16, s_pad = (s_bytes + 15) / 16 * 16;
+    uint8_t *stage = nullptr;
+    hipPointerAttribute_t attr{};
+    const bool on_device = hipPointerGetAttributes(&attr, gate_w) == hipSuccess && attr.type == hipMemoryTypeDevice;
+    (void)hipGetLastError();
+    const hipMemcpyKind kind = on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice;
+    auto place = [&](uint8_t *dst, const void *src, size_t row_bytes, uint32_t half) -> hipError_t {
+        hipError_t e = hipSuccess;
+        if (full)
+            e = hipMemcpy2D(dst + (size_t)half * 16 * row_bytes, 32 * row_bytes, src, 16 * row_bytes, 16 * row_bytes, full, kind);
+        if (e == hipSuccess && rest)
+            e = hipMemcpy(dst + ((size_t)32 * full + 16 * half) * row_bytes, static_cast<const uint8_t *>(src) + (size_t)full * 16 * row_bytes,
+                          (size_t)rest * row_bytes, kind);
+        return e;
+    };
+    hipError_t e = hipMalloc(&stage, w_pad + 2 * s_pad);
+    if (e == hipSuccess) e = hipMemset(stage, 0, w_pad + 2 * s_pad);
+    if (e == hipSuccess) e = place(stage, gate_w, n, 0);
+    if (e == hipSuccess) e = place(stage, up_w, n, 1);
+    if (e == hipSuccess) e = place(stage + w_pad, gate_scales, (size_t)groups * 2, 0);
+    if (e == hipSuccess) e = place(stage + w_pad, up_scales, (size_t)groups * 2, 1);
+    if (e == hipSuccess) e = place(stage + w_pad + s_pad, gate_biases, (size_t)groups * 2, 0);
+    if (e == hipSuccess) e = place(stage + w_pad + s_pad, up_biases, (size_t)groups * 2, 1);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e != hipSuccess) {
+        if (stage) (void)hipFree(stage);
+        return fail(err, e == hipErrorOutOfMemory ? FFMOE_ERR_ALLOC : FFMOE_ERR_RUNTIME, "staging the gate and up projections: %s",
+                    hipGetErrorString(e));
+    }
+    const int rc = matrix_create_common(ctx, stage, reinterpret_cast<const uint16_t *>(stage + w_pad),
+                                        reinterpret_cast<const uint16_t *>(stage + w_pad + s_pad), rows2, n, 0, true, out, err);
+    (void)hipFree(stage);
+    if (rc != FFMOE_OK) return rc;
+    (*out)->glu = true;
+    (*out)->m = f;
+    return FFMOE_OK;
+}
+
 int ffmoe_gelu_mul(ffmoe_ctx *ctx, void *stream, const uint16_t *gate, uint32_t gate_stride, const uint16_t *up,
                    uint32_t up_stride, uint16_t *out, uint32_t out_stride, uint32_t rows, uint32_t count, char **err) {
     if (int rc = check_ctx(ctx, err)) return rc;
@@ -1073,7 +1125,7 @@ int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_
     ffmoe_ctx *ctx = mx->ctx;
     ctx->timer.begin(static_cast<hipStream_t>(stream));
     FF_HIP(launch_matrix_gemv(static_cast<hipStream_t>(stream), mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows,
-                              y, y_stride, y_f32 != 0, ctx->n_cus, ctx->f16, mx->planes8));
+                              y, y_stride, y_f32 != 0, ctx->n_cus, ctx->f16, mx->planes8, mx->glu));
     ctx->timer.mark(static_cast<hipStream_t>(stream), FFMOE_K_GEMV);
     ctx->timer.finish();
     return FFMOE_OK;

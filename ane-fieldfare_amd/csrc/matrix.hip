@@ -167,7 +167,7 @@ __device__ __forceinline__ SoftmaxAcc softmax_shuffle(const SoftmaxAcc &a, int m
 // leaves the softmax pair of the sums it finished in conf_part[row * gridDim.x + block].
 // PLANES8: the matrix is an 8-bit one stored as two nibble planes (above): a tile is 16 rows, an output the sum of its
 // two streams.
-template <bool Y_F32, bool F16, bool GREEDY = false, bool CONF = false, bool PLANES8 = false>
+template <bool Y_F32, bool F16, bool GREEDY = false, bool CONF = false, bool PLANES8 = false, bool GLU = false>
 __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__restrict__ tiles,
                                                              const uint8_t *__restrict__ scales, uint32_t m,
                                                              uint32_t n_groups, const uint16_t *__restrict__ x,
@@ -176,9 +176,16 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
                                                              float softcap = 0.0f) {
     __shared__ float s_red[2][kKSplit][8][64];
     static_assert(!(PLANES8 && GREEDY), "the greedy choice is built for the 4-bit head only");
-    const uint32_t n_tiles = PLANES8 ? (m + 15) / 16 : (m + 31) / 32;
+    static_assert(PLANES8 || !GLU, "the gated form is built for the 8-bit planes only");
+    // GLU: tiles 2 p and 2 p + 1 hold rows 16 p ... 16 p + 15 of a gate and of an up projection; a block takes whole
+    // pairs, and `m` counts the outputs gelu_tanh(gate . x) * (up . x)
+    const uint32_t n_tiles = GLU ? 2 * ((m + 15) / 16) : PLANES8 ? (m + 15) / 16 : (m + 31) / 32;
     uint32_t rb0, rb1;
-    split_range(n_tiles, gridDim.x, blockIdx.x, rb0, rb1);
+    split_range(GLU ? n_tiles / 2 : n_tiles, gridDim.x, blockIdx.x, rb0, rb1);
+    if (GLU) {
+        rb0 *= 2;
+        rb1 *= 2;
+    }
     if (rb0 >= rb1) {
         if (GREEDY && threadIdx.x < rows) reinterpret_cast<unsigned long long *>(y_)[(size_t)threadIdx.x * gridDim.x + blockIdx.x] = 0ull;
         if (CONF && threadIdx.x < rows) conf_part[(size_t)threadIdx.x * gridDim.x + blockIdx.x] = make_float2(-INFINITY, 0.0f);
@@ -209,6 +216,7 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
     uint16_t *y16 = reinterpret_cast<uint16_t *>(y_);
     unsigned long long best = 0ull;
     SoftmaxAcc soft{-INFINITY, 0.0f};
+    float gate_kept = 0.0f;
 
     for (uint32_t rb = rb0; rb < rb1; ++rb) {
         const uint32_t next_row = min(rb + 1, rb1 - 1) * n_groups;
@@ -231,7 +239,19 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
             va += s_red[buf][o][ks][lane];
             vb += s_red[buf][o][4 + ks][lane];
         }
-        if (PLANES8) {
+        if (GLU) {
+            // both projections are rounded to 16 bits in front of the activation, as shared_int8_gate_up_act_simd does
+            // (Metal/Quant/dequant_int8.metal:131-136) and as two separate calls with the activation between them would
+            const float v = Act<F16>::widen(Act<F16>::round(va + vb));
+            const uint32_t col = (rb >> 1) * kTileRows + j;
+            if (!(rb & 1u)) {
+                gate_kept = v;
+            } else if (my_row < rows && col < m) {
+                const float act = gelu_tanh_fast(gate_kept) * v;
+                if (Y_F32) y32[(size_t)my_row * y_stride + col] = act;
+                else y16[(size_t)my_row * y_stride + col] = Act<F16>::round(act);
+            }
+        } else if (PLANES8) {
             const uint32_t row = rb * kTileRows + j;
             if (my_row < rows && row < m) {
                 const float v = va + vb;
@@ -381,18 +401,21 @@ hipError_t launch_matrix_repack(hipStream_t s, const uint8_t *w, const uint16_t 
 
 hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                               const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
-                              bool y_f32, uint32_t n_cus, bool f16, bool planes8) {
-    const uint32_t n_tiles = planes8 ? (m + 15) / 16 : (m + 31) / 32;
+                              bool y_f32, uint32_t n_cus, bool f16, bool planes8, bool glu) {
+    const uint32_t n_tiles = planes8 ? (m + 15) / 16 : (m + 31) / 32;      // gated: pairs of tiles
     const dim3 grid(min(2 * n_cus, n_tiles));
-#define FFMOE_MGEMV(Y, H, P)                                                                                                \
-    hipLaunchKernelGGL((matrix_gemv_kernel<Y, H, false, false, P>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, \
+#define FFMOE_MGEMV(Y, H, P, G)                                                                                             \
+    hipLaunchKernelGGL((matrix_gemv_kernel<Y, H, false, false, P, G>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, \
                        rows, y, y_stride)
-    if (planes8) {
-        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, true); else FFMOE_MGEMV(false, true, true); }
-        else { if (y_f32) FFMOE_MGEMV(true, false, true); else FFMOE_MGEMV(false, false, true); }
+    if (glu) {
+        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, true, true); else FFMOE_MGEMV(false, true, true, true); }
+        else { if (y_f32) FFMOE_MGEMV(true, false, true, true); else FFMOE_MGEMV(false, false, true, true); }
+    } else if (planes8) {
+        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, true, false); else FFMOE_MGEMV(false, true, true, false); }
+        else { if (y_f32) FFMOE_MGEMV(true, false, true, false); else FFMOE_MGEMV(false, false, true, false); }
     } else {
-        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, false); else FFMOE_MGEMV(false, true, false); }
-        else { if (y_f32) FFMOE_MGEMV(true, false, false); else FFMOE_MGEMV(false, false, false); }
+        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, false, false); else FFMOE_MGEMV(false, true, false, false); }
+        else { if (y_f32) FFMOE_MGEMV(true, false, false, false); else FFMOE_MGEMV(false, false, false, false); }
     }
 #undef FFMOE_MGEMV
     return hipGetLastError();

@@ -50,7 +50,7 @@ EXPORTS = [
     "ffmoe_layer_tail", "ffmoe_layer_tail_routed", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
     "ffmoe_verify_static", "ffmoe_route_verify_shared", "ffmoe_layer_tail_routed_shared", "ffmoe_sample_rows",
-    "ffmoe_matrix_create_int8", "ffmoe_gelu_mul",
+    "ffmoe_matrix_create_int8", "ffmoe_matrix_create_int8_glu", "ffmoe_gelu_mul",
 ]
 
 PROFILE_SLOTS = 16
@@ -77,11 +77,13 @@ class Profile(C.Structure):
 class Matrix:
     """ffmoe_matrix: the LM head (or any static INT4 weight) kept re-tiled in HBM."""
 
-    def __init__(self, ctx, W, S, B, greedy: bool, w_byte_offset: int = 0, int8: bool = False):
+    def __init__(self, ctx, W, S, B, greedy: bool, w_byte_offset: int = 0, int8: bool = False, up=None):
+        """`up` = (W, S, B) of an up projection makes W, S, B the gate of a gated 8-bit pair: gemv then returns
+        round16(gelu_tanh(gate x) * up x)."""
         import numpy as np
         self.ctx, self.L = ctx, ctx.L
         self.m, self.n = int(S.shape[0]), int(S.shape[1]) * GROUP
-        self.int8 = int8
+        self.int8 = int8 or up is not None
         keep = []
 
         def raw(a, off=0):
@@ -93,7 +95,10 @@ class Matrix:
             return C.c_void_p(a.data_ptr() + off)
 
         h, err = C.c_void_p(), C.c_char_p()
-        if int8:
+        if up is not None:
+            _check(self.L.ffmoe_matrix_create_int8_glu(ctx._h, raw(W), raw(S), raw(B), raw(up[0]), raw(up[1]), raw(up[2]), self.m,
+                                                       self.n, C.byref(h), C.byref(err)), err)
+        elif int8:
             _check(self.L.ffmoe_matrix_create_int8(ctx._h, raw(W, w_byte_offset), raw(S), raw(B), self.m, self.n,
                                                    C.byref(h), C.byref(err)), err)
         else:
@@ -234,6 +239,7 @@ def lib() -> C.CDLL:
     L.ffmoe_prefill_plan_stats.argtypes = [vp, vp, C.POINTER(u32), C.POINTER(u32), vp, errp]
     L.ffmoe_matrix_create.argtypes = [vp, vp, vp, vp, u32, u32, i32, C.POINTER(vp), errp]
     L.ffmoe_matrix_create_int8.argtypes = [vp, vp, vp, vp, u32, u32, C.POINTER(vp), errp]
+    L.ffmoe_matrix_create_int8_glu.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, C.POINTER(vp), errp]
     L.ffmoe_gelu_mul.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, u32, u32, errp]
     L.ffmoe_matrix_destroy.argtypes = [vp]
     L.ffmoe_matrix_destroy.restype = None
@@ -629,6 +635,10 @@ class Context:
     def matrix_int8(self, W, S, B):
         """Resident copy of an 8-bit affine weight: W uint8 [M, N], S/B bf16 bits [M, N/64] (numpy arrays or tensors)."""
         return Matrix(self, W, S, B, False, 0, int8=True)
+
+    def matrix_int8_glu(self, gate, up):
+        """Gate and up projections (each a (W, S, B) triple as matrix_int8 takes them) as one gated matrix."""
+        return Matrix(self, gate[0], gate[1], gate[2], False, 0, up=up)
 
     def gelu_mul(self, gate, up, out=None):
         """out = round16(gelu_tanh(gate) * up), rows of the activation type (2-D tensors of one shape)."""

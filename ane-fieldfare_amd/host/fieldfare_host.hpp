@@ -661,16 +661,19 @@ private:
     uint32_t m_, n_;
 };
 
-// SharedExpertInt8 (Kernels/MoE/SharedExpertInt8.swift:40-97): y = down(gelu_tanh(gate(x)) * up(x)) with the three
+// SharedExpertInt8 (Kernels/MoE/SharedExpertInt8.swift:40-135): y = down(gelu_tanh(gate(x)) * up(x)) with the three
 // projections 8-bit affine, the form in which the packs hold the shared expert by default. The Swift class binds
-// the projections on every call; here load() re-tiles one layer's three once and the object keeps them. The caller's
-// activation scratch holds gate(x) and up(x) side by side - 2 * F values per row where the Swift kernel, which fuses the
-// two projections with the activation, needs F - and may be reused across layers, as there.
+// the projections on every call; here load() re-tiles one layer's three once (gate and up into one gated matrix, as
+// the Swift class's fused kernel reads them) and the object keeps them. The caller's activation scratch holds
+// F values per row, as there, and may be reused across layers.
 class SharedExpertInt8 {
 public:
     static constexpr int maxBatchRows = DequantInt8GEMV::maxBatchRows;
     explicit SharedExpertInt8(Context &c) : c_(c) {}
-    // the guards of SharedExpertInt8.encode (SharedExpertInt8.swift:63-70), then the three uploads
+    ~SharedExpertInt8() { ffmoe_matrix_destroy(gateUp_); }
+    SharedExpertInt8(const SharedExpertInt8 &) = delete;
+    SharedExpertInt8 &operator=(const SharedExpertInt8 &) = delete;
+    // the guards of SharedExpertInt8.encode (SharedExpertInt8.swift:63-70), then the uploads
     void load(const SharedExpertProjection &gate, const SharedExpertProjection &up, const SharedExpertProjection &down) {
         if (gate.rows != up.rows || gate.cols != up.cols)
             throw SharedExpertError(SharedExpertError::dimensionMismatch,
@@ -680,44 +683,49 @@ public:
             throw SharedExpertError(SharedExpertError::dimensionMismatch,
                                     "down expected (" + std::to_string(gate.cols) + "," + std::to_string(gate.rows) + "), got (" +
                                         std::to_string(down.rows) + "," + std::to_string(down.cols) + ")");
-        gate_.reset(new DequantInt8GEMV(c_, gate.weights, gate.scales, gate.biases, gate.rows, gate.cols));
-        up_.reset(new DequantInt8GEMV(c_, up.weights, up.scales, up.biases, up.rows, up.cols));
+        if (gate.cols % FFMOE_GROUP || gate.rows % FFMOE_GROUP) throw std::invalid_argument("N must be a multiple of 64");
+        ffmoe_matrix *gu = nullptr;
+        char *err = nullptr;
+        check(ffmoe_matrix_create_int8_glu(c_.raw(), gate.weights, gate.scales, gate.biases, up.weights, up.scales, up.biases,
+                                           gate.rows, gate.cols, &gu, &err), err);
+        ffmoe_matrix_destroy(gateUp_);
+        gateUp_ = gu;
+        f_ = gate.rows;
+        d_ = gate.cols;
         down_.reset(new DequantInt8GEMV(c_, down.weights, down.scales, down.biases, down.rows, down.cols));
     }
     // encode (SharedExpertInt8.swift:56-97): one row; scratchActElements is the room behind scratchAct in 16-bit values
     void encode(void *stream, const uint16_t *x, uint16_t *y, uint16_t *scratchAct, size_t scratchActElements) {
-        encodeBlock(stream, x, y, 1, (int)d(), (int)d(), scratchAct, scratchActElements);
+        encodeBlock(stream, x, y, 1, (int)d_, (int)d_, scratchAct, scratchActElements);
     }
     // a block of rows, each as encode does it; more than 16 rows go through in parts of 16 that reuse the scratch
     void encodeBlock(void *stream, const uint16_t *x, uint16_t *y, int queryCount, int xStrideElements, int yStrideElements,
                      uint16_t *scratchAct, size_t scratchActElements) {
-        if (!gate_) throw std::logic_error("SharedExpertInt8: load() first");
+        if (!gateUp_) throw std::logic_error("SharedExpertInt8: load() first");
         if (queryCount < 0) throw std::invalid_argument("queryCount must be non-negative");
-        if (xStrideElements < (int)d()) throw std::invalid_argument("x stride is too small");
-        if (yStrideElements < (int)d()) throw std::invalid_argument("y stride is too small");
-        const uint32_t f = gate_->m(), pitch = (f + 7u) & ~7u;      // rows of the scratch stay 16-byte aligned
+        if (xStrideElements < (int)d_) throw std::invalid_argument("x stride is too small");
+        if (yStrideElements < (int)d_) throw std::invalid_argument("y stride is too small");
         const int part = queryCount < maxBatchRows ? queryCount : maxBatchRows;
-        if (scratchActElements < (size_t)2 * part * pitch)
+        if (scratchActElements < (size_t)part * f_)
             throw SharedExpertError(SharedExpertError::scratchTooSmall,
-                                    "scratchAct needs " + std::to_string((size_t)2 * part * pitch) + " values, has " +
+                                    "scratchAct needs " + std::to_string((size_t)part * f_) + " values, has " +
                                         std::to_string(scratchActElements));
-        uint16_t *g = scratchAct, *u = scratchAct + (size_t)part * pitch;
         for (int r0 = 0; r0 < queryCount; r0 += maxBatchRows) {
             const int rows = queryCount - r0 < maxBatchRows ? queryCount - r0 : maxBatchRows;
-            const uint16_t *xr = x + (size_t)r0 * xStrideElements;
-            gate_->encodeRows(stream, xr, g, rows, (uint32_t)xStrideElements, pitch);
-            up_->encodeRows(stream, xr, u, rows, (uint32_t)xStrideElements, pitch);
             char *err = nullptr;
-            check(ffmoe_gelu_mul(c_.raw(), stream, g, pitch, u, pitch, g, pitch, (uint32_t)rows, f, &err), err);
-            down_->encodeRows(stream, g, y + (size_t)r0 * yStrideElements, rows, pitch, (uint32_t)yStrideElements);
+            check(ffmoe_matrix_gemv(gateUp_, stream, x + (size_t)r0 * xStrideElements, (uint32_t)xStrideElements, (uint32_t)rows,
+                                    scratchAct, f_, 0, &err), err);
+            down_->encodeRows(stream, scratchAct, y + (size_t)r0 * yStrideElements, rows, f_, (uint32_t)yStrideElements);
         }
     }
-    uint32_t d() const { return gate_ ? gate_->n() : 0; }
-    uint32_t intermediate() const { return gate_ ? gate_->m() : 0; }
+    uint32_t d() const { return d_; }
+    uint32_t intermediate() const { return f_; }
 
 private:
     Context &c_;
-    std::unique_ptr<DequantInt8GEMV> gate_, up_, down_;
+    ffmoe_matrix *gateUp_ = nullptr;
+    std::unique_ptr<DequantInt8GEMV> down_;
+    uint32_t f_ = 0, d_ = 0;
 };
 
 // SharedExpertRuntime (SharedExpertInt4.swift:92-130): picks the implementation by weight width. For 4 bits `c` is the

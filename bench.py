@@ -647,33 +647,32 @@ def main():
         x1s, y1s = x[:1].contiguous(), torch.empty((1, D), dtype=torch.bfloat16, device="cuda")
         t1 = timed(lambda: dense_step(x1s, y1s), 200, warm=10)
         shared["rows1"] = {"us": round(t1 * 1e6, 2), "GBs": round(s_payload / t1 / 1e9, 1)}
-        # the same FFN in the 8-bit form the reference's packs hold by default (SharedExpertInt8.swift:56-97): three
-        # matrices of two nibble planes each on the 4-bit streaming kernel, and the activation between them
+        # the same FFN in the 8-bit form the reference's packs hold by default (SharedExpertInt8.swift:56-135): two nibble
+        # planes per weight on the 4-bit streaming kernel; gate and up as one gated matrix (the activation is that pass's
+        # epilogue), then the down projection: two launches
         m8, bytes8 = [], 0
         for layer in range(LS):
-            trio = []
+            parts8 = []
             for rows, cols in ((FS, D), (FS, D), (D, FS)):
                 g_ = cols // 64
                 w8 = torch.randint(0, 256, (rows, cols), dtype=torch.uint8, device="cuda", generator=gen)
                 sc = (torch.randn((rows, g_), device="cuda", generator=gen) * 0.001).abs().to(torch.bfloat16)
                 bi = (-128.0 * sc.float() + torch.randn((rows, g_), device="cuda", generator=gen) * 1e-3).to(torch.bfloat16)
-                trio.append(ctx.matrix_int8(w8, sc, bi))
+                parts8.append((w8, sc, bi))
                 bytes8 += (rows * cols + 4 * rows * g_) if layer == 0 else 0
-                del w8, sc, bi
-            m8.append(trio)
-        act8 = torch.empty((2, T, FS), dtype=torch.bfloat16, device="cuda")
+            m8.append((ctx.matrix_int8_glu(parts8[0], parts8[1]), ctx.matrix_int8(*parts8[2])))
+            del parts8
+        act8 = torch.empty((T, FS), dtype=torch.bfloat16, device="cuda")
 
         def int8_step(xin, yout):
-            gate8, up8, down8 = m8[state["i"] % LS]
-            rows_ = xin.shape[0]
-            gate8.gemv(xin, out=act8[0, :rows_])
-            up8.gemv(xin, out=act8[1, :rows_])
-            ctx.gelu_mul(act8[0, :rows_], act8[1, :rows_], out=act8[0, :rows_])
-            down8.gemv(act8[0, :rows_], out=yout)
+            gate_up8, down8 = m8[state["i"] % LS]
+            a8 = act8[:xin.shape[0]]
+            gate_up8.gemv(xin, out=a8)
+            down8.gemv(a8, out=yout)
             state["i"] += 1
         t8_16 = timed(lambda: int8_step(x, y16), 200, warm=10)
         t8_1 = timed(lambda: int8_step(x1s, y1s), 200, warm=10)
-        shared["int8"] = {"bytes_per_layer": bytes8, "launches": 4,
+        shared["int8"] = {"bytes_per_layer": bytes8, "launches": 2,
                           "rows16": {"us": round(t8_16 * 1e6, 2), "GBs": round(bytes8 / t8_16 / 1e9, 1)},
                           "rows1": {"us": round(t8_1 * 1e6, 2), "GBs": round(bytes8 / t8_1 / 1e9, 1)}}
         if args.prefill_tokens:

@@ -310,6 +310,16 @@ int ffmoe_matrix_create(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales
  * matrix's rate. */
 int ffmoe_matrix_create_int8(ffmoe_ctx *ctx, const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
                              uint32_t m, uint32_t n, ffmoe_matrix **out, char **err);
+/* The gate and up projections of an 8-bit gated FFN as ONE matrix (each W uint8 [f][n], S/B bf16 [f][n/64], host or
+ * device memory, all six of the same kind), their rows interleaved 16 at a time: ffmoe_matrix_gemv on it then writes
+ * y[r][i] = round16(gelu_tanh(round16(gate_i . x_r)) * round16(up_i . x_r)) for i < f - the activation row of the
+ * shared expert in one pass over both projections, as the reference's fused kernel shared_int8_gate_up_act_simd makes it
+ * (Metal/Quant/dequant_int8.metal:84-140, run by SharedExpertInt8.encodeFusedGateUpAct,
+ * Kernels/MoE/SharedExpertInt8.swift:99-135), and bit for bit what two ffmoe_matrix_gemv calls on separate matrices
+ * and ffmoe_gelu_mul leave. A ffmoe_matrix_create_int8 matrix of the down projection finishes the expert. */
+int ffmoe_matrix_create_int8_glu(ffmoe_ctx *ctx, const uint8_t *gate_w, const uint16_t *gate_scales,
+                                 const uint16_t *gate_biases, const uint8_t *up_w, const uint16_t *up_scales,
+                                 const uint16_t *up_biases, uint32_t f, uint32_t n, ffmoe_matrix **out, char **err);
 /* A matrix belongs to the context it was created on. Destroying that context first releases the matrix's
  * device memory; the handle then only accepts ffmoe_matrix_destroy (compute calls return FFMOE_ERR_INVALID). */
 void ffmoe_matrix_destroy(ffmoe_matrix *mx);

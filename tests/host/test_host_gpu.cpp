@@ -385,7 +385,7 @@ int main() {
         EXPECT(threwDims);
         shared8.load(gate, up, down);
         EXPECT(shared8.d() == (uint32_t)d && shared8.intermediate() == (uint32_t)f);
-        const size_t scratchValues = (size_t)2 * 16 * ((f + 7) & ~7);
+        const size_t scratchValues = (size_t)16 * f;
         uint16_t *dScratch = nullptr;
         HIP(hipMalloc(&dScratch, scratchValues * 2));
         try { shared8.encodeBlock(stream, dx, dH2b, T, d, d, dScratch, scratchValues - 1); }

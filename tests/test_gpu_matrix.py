@@ -347,6 +347,37 @@ def test_shared_expert_int8_matches_reference(ff, oracle, torch, act):
     c.close()
 
 
+@pytest.mark.parametrize("act", ["bf16", "fp16"])
+@pytest.mark.parametrize("f,d,rows", [(64, 128, 1), (2112, 2816, 16), (100, 192, 5), (8, 64, 16), (33, 704, 3)])
+def test_int8_gated_matrix_equals_separate_calls(ff, oracle, torch, act, f, d, rows):
+    # the fused gate / up / activation pass (shared_int8_gate_up_act_simd, dequant_int8.metal:84-140) against the three
+    # separate calls, bit for bit: F a multiple of 16 and not, one row to sixteen, sources on the host and on the device
+    g = np.random.default_rng(f * 131 + d + rows)
+    gate = oracle.quantize_int8(g.uniform(-0.4, 0.4, (f, d)).astype(np.float32))
+    up = oracle.quantize_int8(g.uniform(-0.4, 0.4, (f, d)).astype(np.float32))
+    c = ff.Context(128, 64, 16, 8, n_layers=1, max_tokens=16, act_dtype=act)
+    xv = g.uniform(-0.5, 0.5, (rows, d)).astype(np.float32)
+    x = (torch.from_numpy(xv.astype(np.float16)).cuda() if act == "fp16" else bf16_tensor(torch, oracle.bf16_bits(xv)))
+    mg, mu = c.matrix_int8(*gate), c.matrix_int8(*up)
+    want = c.gelu_mul(mg.gemv(x), mu.gemv(x))
+    fused = c.matrix_int8_glu(gate, up)
+    assert fused.m == f
+    got = fused.gemv(x)
+    assert got.shape == (rows, f) and torch.equal(got.view(torch.int16), want.view(torch.int16))
+    on_device = lambda t: tuple(torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in t)
+    fused_dev = c.matrix_int8_glu(on_device(gate), on_device(up))
+    assert torch.equal(fused_dev.gemv(x).view(torch.int16), want.view(torch.int16))
+    # fp32 out: the un-rounded product of the two rounded projections
+    g32 = fused.gemv(x, f32_out=True)
+    step = 2.0 ** -11 if act == "fp16" else 2.0 ** -8
+    assert g32.dtype == torch.float32 and ((g32 - want.float()).abs() <= step * g32.abs() + 1e-6).all()
+    with pytest.raises(ff.FieldfareError):
+        fused.greedy(x)
+    for m_ in (mg, mu, fused, fused_dev):
+        m_.close()
+    c.close()
+
+
 def test_int8_matrix_block_equals_repeated_single_rows(ctx, oracle, torch):
     # blockSharedExpertMatchesRepeatedScalarRows (PrefillSharedExpertTests.swift:15-82): four rows with an input stride of
     # 144 and an output stride of 137 over sentinels - the block call equals the four single-row calls bit for bit,
