@@ -582,6 +582,41 @@ private:
     uint32_t d_, vocab_;
 };
 
+// PrefillFinalRowHeadInt4 (Kernels/Prefill/Epilogues/PrefillFinalRowHead.swift:4-66): the head's logits for ONE row of
+// a prefill block - the last prompt token's -, the final norm applied to that row where it lies. The Swift class binds
+// the head's table on every call and owns the normed row's buffer; here the table is the resident copy a
+// LMHeadChainInt4-style constructor makes, and the caller passes the normed row's scratch (d values, 16-byte aligned).
+class PrefillFinalRowHeadInt4 {
+public:
+    PrefillFinalRowHeadInt4(Context &c, int maxD, const uint8_t *weights, const uint16_t *scales, const uint16_t *biases, uint32_t d,
+                            uint32_t vocab)
+        : c_(c), d_(d), vocab_(vocab) {
+        if (maxD <= 0) throw std::invalid_argument("maxD must be positive");
+        if ((int)d > maxD) throw std::invalid_argument("d=" + std::to_string(d) + " exceeds maxD=" + std::to_string(maxD));
+        if (d % FFMOE_GROUP) throw std::invalid_argument("d must be a multiple of 64");
+        char *err = nullptr;
+        check(ffmoe_matrix_create(c.raw(), weights, scales, biases, vocab, d, 0, &mx_, &err), err);
+    }
+    ~PrefillFinalRowHeadInt4() { ffmoe_matrix_destroy(mx_); }
+    PrefillFinalRowHeadInt4(const PrefillFinalRowHeadInt4 &) = delete;
+    PrefillFinalRowHeadInt4 &operator=(const PrefillFinalRowHeadInt4 &) = delete;
+    // encodeLogits (PrefillFinalRowHead.swift:19-65): logits [vocab] in the activation type
+    void encodeLogits(void *stream, const uint16_t *hiddenBlock, int row, int rowStrideElements, const uint16_t *normWeight,
+                      uint16_t *normed, uint16_t *logits, float rmsEps) {
+        if (row < 0) throw std::invalid_argument("row must be non-negative");
+        if (rowStrideElements < (int)d_) throw std::invalid_argument("row stride must cover d");
+        char *err = nullptr;
+        check(ffmoe_rmsnorm(c_.raw(), stream, hiddenBlock + (size_t)row * rowStrideElements, (uint32_t)rowStrideElements, normWeight,
+                            normed, d_, 1, d_, rmsEps, &err), err);
+        check(ffmoe_matrix_gemv(mx_, stream, normed, d_, 1, logits, vocab_, 0, &err), err);
+    }
+
+private:
+    Context &c_;
+    ffmoe_matrix *mx_ = nullptr;
+    uint32_t d_, vocab_;
+};
+
 // ---------------------------------------------------------------------------------------------------
 // Shared expert (Kernels/MoE/SharedExpertInt4.swift, Kernels/Prefill/MoE/PrefillSharedExpert.swift): the dense
 // INT4 FFN every token passes through. The Swift operators bind the three projections on every call; here

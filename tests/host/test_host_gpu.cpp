@@ -197,6 +197,40 @@ int main() {
     errorStats(yg, refg, rel, cosine);
     EXPECT(rel <= 1e-2);
 
+    // --- PrefillFinalRowHeadInt4: row 2 of the block through a norm and the same 64-row "head": the oracle's normed row
+    // bit for bit, and logits of its dequantised rows ---
+    {
+        std::vector<uint16_t> normW(d);
+        for (auto &v : normW) v = ffo_bf16_bits(ffo_splitmix64_uniform(&rng, 0.5f, 1.5f));
+        uint16_t *dNormW = toDevice(normW), *dNormed = nullptr, *dLogits16 = nullptr;
+        HIP(hipMalloc(reinterpret_cast<void **>(&dNormed), (size_t)d * 2));
+        HIP(hipMalloc(reinterpret_cast<void **>(&dLogits16), (size_t)f * 2));
+        PrefillFinalRowHeadInt4 finalRow(ctx, 256, pool.data() + off.gate_w, reinterpret_cast<uint16_t *>(pool.data() + off.gate_s),
+                                         reinterpret_cast<uint16_t *>(pool.data() + off.gate_b), d, f);
+        bool threwStride = false, threwMaxD = false;
+        try { finalRow.encodeLogits(stream, dx, 2, d - 1, dNormW, dNormed, dLogits16, 1e-6f); }
+        catch (const std::invalid_argument &) { threwStride = true; }
+        EXPECT(threwStride);
+        try {
+            PrefillFinalRowHeadInt4 small(ctx, 64, pool.data() + off.gate_w, reinterpret_cast<uint16_t *>(pool.data() + off.gate_s),
+                                          reinterpret_cast<uint16_t *>(pool.data() + off.gate_b), d, f);
+        } catch (const std::invalid_argument &) { threwMaxD = true; }
+        EXPECT(threwMaxD);
+        finalRow.encodeLogits(stream, dx, 2, d, dNormW, dNormed, dLogits16, 1e-6f);
+        HIP(hipStreamSynchronize(stream));
+        std::vector<uint16_t> refNormed(d);
+        ffo_rmsnorm(x.data() + (size_t)2 * d, normW.data(), refNormed.data(), d, 1e-6f, FFO_BF16);
+        EXPECT(toHost(dNormed, (size_t)d) == refNormed);
+        std::vector<float> xr(d), refLogits(f);
+        for (int i = 0; i < d; ++i) xr[i] = ffo_bf16_to_float(refNormed[i]);
+        ffo_gemv_int4_ref(pool.data() + off.gate_w, reinterpret_cast<uint16_t *>(pool.data() + off.gate_s),
+                          reinterpret_cast<uint16_t *>(pool.data() + off.gate_b), f, d, xr.data(), refLogits.data());
+        double relF = 0, cosF = 0;
+        errorStats(toHost(dLogits16, (size_t)f), refLogits, relF, cosF);
+        EXPECT(relF <= 1e-2 && cosF >= 0.9999);
+        HIP(hipFree(dNormW)); HIP(hipFree(dNormed)); HIP(hipFree(dLogits16));
+    }
+
     // --- LMHeadChainInt4 over the same matrix as a 64-token "vocabulary": greedy token == CPU argmax ---
     {
         LMHeadChainInt4 head(ctx, pool.data() + off.gate_w, reinterpret_cast<uint16_t *>(pool.data() + off.gate_s),

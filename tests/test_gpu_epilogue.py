@@ -183,3 +183,27 @@ def test_rmsnorm_rows_in_place_and_unit_rms(ctx, oracle, torch):
         assert np.array_equal(bits_of(x), ref)
         unit = oracle.bf16_to_float(bits_of(ctx.rmsnorm(bf16_tensor(torch, xb), bf16_tensor(torch, oracle.bf16_bits(np.ones(d, np.float32))), 0.0, d=d)))
         assert np.allclose(np.sqrt((unit.astype(np.float64) ** 2).mean(axis=1)), 1.0, atol=3e-3)
+
+
+@pytest.mark.parametrize("act", ["fp16", "bf16"])
+def test_rmsnorm_reference_case_hidden_size(oracle, torch, act):
+    import fieldfare_moe as ff
+    # rmsNorm_matchesReference_hiddenSize (RMSNormTests.swift:19-45): same seed, label and draw order (x, then the bf16
+    # weight), FP16 rows as there (and bf16 rows), against the un-rounded norm within Tolerance.fp16Reduction = 5e-3
+    d = 2816
+    rng = oracle.seed_tree_key(0xD4, f"rmsnorm-d{d}-weighted=true")
+    xv = rng.uniform(-1.0, 1.0, d).astype(np.float32)
+    wb = oracle.bf16_bits(rng.uniform(0.5, 1.5, d))
+    c = ff.Context(128, 64, 16, 8, n_layers=1, max_tokens=16, act_dtype=act)
+    if act == "fp16":
+        x = torch.from_numpy(xv.astype(np.float16)[None, :]).cuda()
+        x64 = xv.astype(np.float16).astype(np.float64)
+    else:
+        x = bf16_tensor(torch, oracle.bf16_bits(xv)[None, :])
+        x64 = oracle.bf16_to_float(oracle.bf16_bits(xv)).astype(np.float64)
+    out = c.rmsnorm(x, bf16_tensor(torch, wb), 1e-6, d=d)
+    got = out.float().cpu().numpy()[0].astype(np.float64)
+    ref = x64 / np.sqrt((x64 ** 2).mean() + 1e-6) * oracle.bf16_to_float(wb).astype(np.float64)
+    rel = np.abs(got - ref).max() / np.abs(ref).max()
+    assert rel < 5e-3, rel
+    c.close()

@@ -458,3 +458,38 @@ def test_gelu_mul_and_int8_argument_errors(ctx, ff, oracle, torch):
     W, S, B = oracle.quantize_int8(g.uniform(-1, 1, (8, 100 * 64)).astype(np.float32))
     with pytest.raises(ff.FieldfareError, match="at most"):
         ctx.matrix_int8(W, S, B)                       # N beyond what a wave's register ring holds
+
+
+def test_final_row_head_matches_scalar_offset_path(ctx, oracle, torch):
+    # finalRowHeadLogitsMatchesScalarOffsetPath (PrefillFinalRowHeadTests.swift:31-127): row 3 of a five-row block with a
+    # row stride of d + 17 values, norm then head. Same seed, label, draw order and shapes. The block path norms the row
+    # where it lies (the 2-byte aligned offset the stride gives) and projects through the resident head; the scalar path
+    # norms a copy of the row and projects through the reference-layout GEMV. The reference allows 1e-3 / 1e-4 between
+    # them (held here on the fp32 logits); the normed row is the oracle's bit for bit and the logits those of its
+    # dequantised rows.
+    rows, sel, d, vocab = 5, 3, 128, 96
+    stride = d + 17
+    rng = oracle.seed_tree_key(0xB501, "prefill-final-row-head")
+    hid = np.zeros((rows, stride), np.float32)
+    for r in range(rows):
+        hid[r, :d] = rng.uniform(-1.0, 1.0, d)
+    hb = oracle.bf16_bits(hid)
+    nb = oracle.bf16_bits(rng.uniform(0.5, 1.5, d))
+    W, S, B = oracle.quantize_int4(np.stack([rng.uniform(-0.5, 0.5, d) for _ in range(vocab)]))
+    block = bf16_tensor(torch, hb)
+    norm_w = bf16_tensor(torch, nb)
+    head = ctx.matrix(W, S, B)
+    normed = ctx.rmsnorm(block[sel:sel + 1], norm_w, 1e-6, d=d)                 # read at offset 3 * 145 values
+    logits_block = head.gemv(normed, f32_out=True)
+    row_copy = block[sel, :d].clone()[None, :]
+    Wt, St, Bt = (torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (W, S.view(np.int16), B.view(np.int16)))
+    normed_copy = ctx.rmsnorm(row_copy, norm_w, 1e-6, d=d)
+    assert torch.equal(normed.view(torch.int16), normed_copy.view(torch.int16))
+    logits_scalar = ctx.gemv_int4(Wt, St, Bt, normed_copy, f32_out=True)
+    a, b = logits_block.cpu().numpy()[0], logits_scalar.cpu().numpy()[0]
+    assert np.abs(a - b).max() <= 1e-3 and rel_err(a, b) <= 1e-4            # the reference's two bounds
+    ref_normed = oracle.rmsnorm(hb[sel:sel + 1, :d], nb, 1e-6)
+    assert np.array_equal(bits_of(normed), ref_normed)
+    ref = oracle.gemv_int4_ref(W, S, B, oracle.bf16_to_float(ref_normed[0]))
+    assert rel_err(a, ref) < 5e-3                                           # Tolerance.fp16Reduction
+    head.close()
