@@ -25,6 +25,8 @@ struct ffmoe_layer {
     uint16_t *per_expert_scale = nullptr;
     void *router_frag = nullptr;    // bf16 router weights in matrix-operand order (the prefill router's approximate pass)
     float router_norm_max = 0.0f;   // upper bound of the largest 2-norm of an expert's router row
+    // a dense context's layer held 8-bit (ffmoe_upload_expert_parts_int8): the gated gate/up matrix and the down matrix
+    struct ffmoe_matrix *gate_up8 = nullptr, *down8 = nullptr;
 };
 
 // A resident matrix: the re-tiled copy of one [m][n] INT4 weight plus the scratch of its greedy choice.
@@ -296,6 +298,10 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipDeviceSynchronize();
     for (auto &l : ctx->layers) {
+        // the layer's own 8-bit matrices: nobody else holds their handles
+        ffmoe_matrix_destroy(l.gate_up8);
+        ffmoe_matrix_destroy(l.down8);
+        l.gate_up8 = l.down8 = nullptr;
         if (l.router_w) (void)hipFree(l.router_w);
         if (l.router_frag) (void)hipFree(l.router_frag);
         if (l.effective_scale) (void)hipFree(l.effective_scale);
@@ -620,7 +626,10 @@ int ffmoe_route_verify_shared(ffmoe_ctx *ctx, ffmoe_ctx *shared, void *stream, u
     if (shared == ctx) return fail(err, FFMOE_ERR_INVALID, "the shared expert lives in a context of its own");
     if (shared->device != ctx->device || shared->f16 != ctx->f16)
         return fail(err, FFMOE_ERR_INVALID, "the two contexts must share the device and the activation type");
-    if (int rc = check_layer(shared, shared_layer, true, false, err)) return rc;
+    if (int rc = check_layer(shared, shared_layer, false, false, err)) return rc;
+    const ffmoe_layer &shared_l = shared->layers[shared_layer];
+    if (!shared_l.gate_up8)
+        if (int rc = check_layer(shared, shared_layer, true, false, err)) return rc;
     const ArenaGeom &sg = shared->geom;
     if (sg.d != ctx->geom.d || ctx->geom.gf > kSharedChunkGroups || (ctx->geom.gd + 3) / 4 > kSharedChunkGroups ||
         shared_chunks(sg) > 4 || ctx->shape.top_k > 8)
@@ -637,8 +646,14 @@ int ffmoe_route_verify_shared(ffmoe_ctx *ctx, ffmoe_ctx *shared, void *stream, u
     const RouteFusion route{RouterWeights{l.router_w, l.router_is_f32, l.effective_scale, l.per_expert_scale}, router_x,
                             router_x_stride, ctx->logits, ctx->mail, ctx->handover_ticks, ctx->one_launch_routing,
                             ctx->route_resident_blocks};
-    const SharedExpert sh{shared->arena + (size_t)shared_layer * shared->layer_bytes, sg, shared_x, shared_x_stride, shared->acts,
-                          shared->partials};
+    SharedExpert sh{shared->arena + (size_t)shared_layer * shared->layer_bytes, sg, shared_x, shared_x_stride, shared->acts,
+                    shared->partials};
+    if (shared_l.gate_up8) {
+        sh.gu_tiles8 = shared_l.gate_up8->tiles;
+        sh.gu_scales8 = shared_l.gate_up8->scales;
+        sh.dn_tiles8 = shared_l.down8->tiles;
+        sh.dn_scales8 = shared_l.down8->scales;
+    }
     return verify_common(ctx, stream, layer, x, x_stride, t, out_idx, out_w, nullptr, nullptr, nullptr, err, nullptr, &route,
                          false, &sh, shared);
 }
@@ -749,6 +764,29 @@ int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t
         return fail(err, FFMOE_ERR_INVALID, "the dense FFN needs a context with n_experts = 1 and top_k = 1");
     if (!y) return fail(err, FFMOE_ERR_INVALID, "null output");
     if (reinterpret_cast<uintptr_t>(y) % 16) return fail(err, FFMOE_ERR_INVALID, "y must be 16-byte aligned");
+    if (int rc = check_layer(ctx, layer, false, false, err)) return rc;
+    if (ctx->layers[layer].gate_up8) {
+        // an 8-bit layer: the gated gate/up pass into the activation scratch, then the down pass, 16 rows at a time
+        const ffmoe_layer &l = ctx->layers[layer];
+        const uint32_t cap = std::max<uint32_t>(ctx->shape.max_tokens, FFMOE_MAX_VERIFY_ROWS);
+        if (!x || t == 0 || t > cap) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%u", t, cap);
+        if (x_stride < ctx->shape.d || x_stride % 8 || reinterpret_cast<uintptr_t>(x) % 16)
+            return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        claim_scratch(ctx, stream);
+        ctx->timer.begin(s);
+        for (uint32_t r0 = 0; r0 < t; r0 += FFMOE_MAX_VERIFY_ROWS) {
+            const uint32_t rows = std::min<uint32_t>(FFMOE_MAX_VERIFY_ROWS, t - r0);
+            FF_HIP(launch_matrix_gemv(s, l.gate_up8->tiles, l.gate_up8->scales, ctx->shape.f, ctx->shape.d, x + (size_t)r0 * x_stride,
+                                      x_stride, rows, ctx->acts, ctx->shape.f, false, ctx->n_cus, ctx->f16, true, true));
+            ctx->timer.mark(s, FFMOE_K_GATE_UP);
+            FF_HIP(launch_matrix_gemv(s, l.down8->tiles, l.down8->scales, ctx->shape.d, ctx->shape.f, ctx->acts, ctx->shape.f, rows,
+                                      y + (size_t)r0 * ctx->shape.d, ctx->shape.d, false, ctx->n_cus, ctx->f16, true, false));
+            ctx->timer.mark(s, FFMOE_K_DOWN);
+        }
+        ctx->timer.finish();
+        return FFMOE_OK;
+    }
     // With one route per row at weight 1, the un-weighted bf16 row of route t is the output row t: the
     // down projection writes y itself and the combine pass has nothing to add.
     if (t <= FFMOE_MAX_VERIFY_ROWS)
@@ -1073,6 +1111,35 @@ int ffmoe_matrix_create_int8_glu(ffmoe_ctx *ctx, const uint8_t *gate_w, const ui
     if (rc != FFMOE_OK) return rc;
     (*out)->glu = true;
     (*out)->m = f;
+    return FFMOE_OK;
+}
+
+int ffmoe_upload_expert_parts_int8(ffmoe_ctx *ctx, uint32_t layer, const ffmoe_projection *gate, const ffmoe_projection *up,
+                                   const ffmoe_projection *down, char **err) {
+    if (int rc = check_ctx(ctx, err)) return rc;
+    if (int rc = check_layer(ctx, layer, false, false, err)) return rc;
+    if (!ctx->dense_idx)
+        return fail(err, FFMOE_ERR_INVALID, "an 8-bit expert needs a context with n_experts = 1 and top_k = 1 (the shared expert's)");
+    const ffmoe_projection *proj[3] = {gate, up, down};
+    for (const ffmoe_projection *p : proj)
+        if (!p || !p->w || !p->scales || !p->biases) return fail(err, FFMOE_ERR_INVALID, "null projection");
+    const ffmoe_shape &sh = ctx->shape;
+    if (!matrix_shape_ok(sh.d) || !matrix_shape_ok(sh.f))
+        return fail(err, FFMOE_ERR_INVALID, "an 8-bit expert needs d and f that are multiples of %d and at most %d", FFMOE_GROUP,
+                    FFMOE_MATRIX_MAX_N);
+    ffmoe_matrix *gu = nullptr, *dn = nullptr;
+    if (int rc = ffmoe_matrix_create_int8_glu(ctx, gate->w, gate->scales, gate->biases, up->w, up->scales, up->biases, sh.f, sh.d,
+                                              &gu, err))
+        return rc;
+    if (int rc = ffmoe_matrix_create_int8(ctx, down->w, down->scales, down->biases, sh.d, sh.f, &dn, err)) {
+        ffmoe_matrix_destroy(gu);
+        return rc;
+    }
+    ffmoe_layer &l = ctx->layers[layer];
+    ffmoe_matrix_destroy(l.gate_up8);
+    ffmoe_matrix_destroy(l.down8);
+    l.gate_up8 = gu;
+    l.down8 = dn;
     return FFMOE_OK;
 }
 

@@ -151,6 +151,9 @@ struct SharedExpert {
     uint32_t x_stride;
     uint16_t *acts;                 // [t][g.f]
     float *partials;                // [chunks][t][g.d], chunk c = groups [kRing c, kRing c + kRing) of K
+    // an 8-bit shared expert (all four set; arena_layer unused): the nibble-plane tiles and scales of its gated gate/up
+    // matrix and of its down matrix as launch_matrix_repack lays them out (matrix.hip)
+    const uint8_t *gu_tiles8 = nullptr, *gu_scales8 = nullptr, *dn_tiles8 = nullptr, *dn_scales8 = nullptr;
 };
 constexpr uint32_t kSharedChunkGroups = 11;      // = kRing of the streaming kernels
 inline uint32_t shared_chunks(const ArenaGeom &g) { return (g.gf + kSharedChunkGroups - 1) / kSharedChunkGroups; }

@@ -414,20 +414,76 @@ struct SharedGateUp {
     uint32_t x_stride;
     uint16_t *acts;
     uint32_t blocks;
+    // an 8-bit shared expert (not null): its gate and up projections as one gated matrix of nibble planes, tiles
+    // 2 p and 2 p + 1 = rows 16 p ... 16 p + 15 of the gate and of the up projection (matrix.hip); arena_layer is unused
+    const uint8_t *tiles8, *scales8;
 };
 
 // What a kernel instantiated without the shared expert's role takes in its place: nothing to pass, nothing to load.
 struct NoSharedExpert {};
-template <bool SHARED, typename T>
-using SharedArg = std::conditional_t<SHARED, T, NoSharedExpert>;
-template <bool SHARED, typename T>
+// SHARED: 0 = no shared expert in the launch, 1 = a 4-bit one (arena tiles), 2 = an 8-bit one (nibble planes; the
+// gate/up kernels only - an instantiation of its own, so the 4-bit role's registers stay as they are)
+template <int SHARED, typename T>
+using SharedArg = std::conditional_t<SHARED != 0, T, NoSharedExpert>;
+template <int SHARED, typename T>
 SharedArg<SHARED, T> shared_arg(const T &v) {
-    if constexpr (SHARED) return v;
+    if constexpr (SHARED != 0) return v;
     else return NoSharedExpert{};
 }
 
-// A block in that role: block `bid` of sh.blocks walks its share of the dense expert's row blocks for all `rows` rows.
+// The 8-bit shared expert's gate/up rows: block `bid` of sh.blocks walks its share of the tile pairs. A pair's first tile
+// gives 16 gate rows (the sum of its two nibble-plane streams), its second the up rows; both are rounded to 16 bits in
+// front of the activation, as the resident-matrix GEMV does on the same tiles (matrix_gemv_kernel, gated form) and as the
+// reference's shared_int8_gate_up_act_simd does (Metal/Quant/dequant_int8.metal:131-136).
 template <bool F16>
+__device__ __forceinline__ void shared_gate_up8_rows(GateUpMerge &s_red, const SharedGateUp &sh, uint32_t rows, uint32_t bid,
+                                                     const KSlice &k, uint4 (&x0)[kRing], uint4 (&x1)[kRing], f32x4 (&sx)[kRing]) {
+    const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, jq = lane >> 4;
+    const uint32_t pairs = sh.g.gu_rb, gd = sh.g.gd;
+    uint32_t rb0, rb1;
+    split_range(pairs, sh.blocks, bid, rb0, rb1);
+    rb0 *= 2;
+    rb1 *= 2;
+    if (rb0 >= rb1) return;
+    const TileSource src = make_tile_source(sh.tiles8, (size_t)2 * pairs * gd * kTileBytes, sh.scales8,
+                                            (size_t)2 * pairs * gd * kTileScaleBytes);
+    WeightRing ring;
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) ring_fill(ring, u, src, rb0 * gd + min(k.g0 + u, k.g_last), lane);
+    prepare_token_rows<F16>(lane, x0, x1, sx);
+    const uint32_t col = 4 * jq + ks;       // the input row this lane finishes
+    uint16_t *out_col = sh.acts + (size_t)col * sh.g.f + j;
+    float gate_kept = 0.0f;
+    for (uint32_t rb = rb0; rb < rb1; ++rb) {
+        const uint32_t next_row = min(rb + 1, rb1 - 1) * gd;
+        TwoStreamAcc tot;
+        tot.a = f32x4{0.f, 0.f, 0.f, 0.f};
+        tot.b = tot.a;
+#pragma unroll
+        for (int u = 0; u < kRing; ++u)
+            ring_step<F16>(ring, u, (uint32_t)u < k.ng, x0[u], x1[u], sx[u], tot, src, next_row + min(k.g0 + u, k.g_last), lane);
+        const int buf = (rb - rb0) & 1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            s_red[buf][ks][r][lane] = tot.a[r];
+            s_red[buf][ks][4 + r][lane] = tot.b[r];
+        }
+        lds_barrier();
+        float va = s_red[buf][0][ks][lane], vb = s_red[buf][0][4 + ks][lane];
+#pragma unroll
+        for (int o = 1; o < kKSplit; ++o) {
+            va += s_red[buf][o][ks][lane];
+            vb += s_red[buf][o][4 + ks][lane];
+        }
+        const float v = Act<F16>::widen(Act<F16>::round(va + vb));
+        if (!(rb & 1u)) gate_kept = v;
+        else if (col < rows) out_col[(rb >> 1) * kTileRows] = Act<F16>::round(gelu_tanh_fast(gate_kept) * v);
+    }
+}
+
+// A block in that role: block `bid` of sh.blocks walks its share of the dense expert's row blocks for all `rows` rows.
+template <bool F16, bool PLANES8>
 __device__ __forceinline__ void shared_gate_up_role(GateUpMerge &s_red, PlanScratch &ps, const SharedGateUp &sh, uint32_t rows,
                                                     uint32_t bid) {
     const uint32_t lane = threadIdx.x & 63, ks = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -435,11 +491,15 @@ __device__ __forceinline__ void shared_gate_up_role(GateUpMerge &s_red, PlanScra
     uint4 x0[kRing], x1[kRing];
     f32x4 sx[kRing];
     load_token_rows(sh.x, sh.x_stride, rows, lane, k, x0, x1);
+    if constexpr (PLANES8) {
+        shared_gate_up8_rows<F16>(s_red, sh, rows, bid, k, x0, x1, sx);
+        return;
+    }
     gate_up_rows<F16, true>(s_red, ps, sh.arena_layer, sh.g, 1u, 1u, 0u, (uint16_t)0, rows, nullptr, k, x0, x1, sx, false, sh.acts,
                             bid, sh.blocks);
 }
 
-template <bool F16, bool DENSE = false, bool SHARED = false>
+template <bool F16, bool DENSE = false, int SHARED = 0>
 __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_t *__restrict__ arena_layer, ArenaGeom g,
                                                                     uint32_t top_k, uint32_t n_experts,
                                                                     const uint32_t *__restrict__ idx,
@@ -451,10 +511,10 @@ __global__ __launch_bounds__(256, 2) void skinny_gate_up_persistent(const uint8_
     __shared__ GateUpMerge s_red;
     __shared__ PlanScratch ps;
     uint32_t routed_blocks = gridDim.x;
-    if constexpr (SHARED) {
+    if constexpr (SHARED != 0) {
         routed_blocks -= sh.blocks;
         if (blockIdx.x >= routed_blocks) {
-            shared_gate_up_role<F16>(s_red, ps, sh, n_routes / top_k, blockIdx.x - routed_blocks);
+            shared_gate_up_role<F16, SHARED == 2>(s_red, ps, sh, n_routes / top_k, blockIdx.x - routed_blocks);
             return;
         }
     }
@@ -549,7 +609,7 @@ __device__ __forceinline__ void lone_wave_keys(const void *__restrict__ router_w
     }
 }
 
-template <bool W_F32, bool F16, bool SHARED>
+template <bool W_F32, bool F16, int SHARED>
 __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
     const uint8_t *__restrict__ arena_layer, ArenaGeom g, uint32_t top_k, uint32_t n_experts, const void *__restrict__ router_w,
     const uint16_t *__restrict__ effective_scale, const uint16_t *__restrict__ per_expert_scale,
@@ -590,8 +650,8 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
     }
     // the blocks that serve the shared expert need no routes: they start on its rows now
     uint32_t routed_blocks = gridDim.x;
-    if constexpr (!SHARED) routed_blocks -= prefetch_blocks;        // (the launch with the shared expert has no blocks to spare)
-    if (!SHARED && blockIdx.x >= routed_blocks) {
+    if constexpr (SHARED == 0) routed_blocks -= prefetch_blocks;        // (the launch with the shared expert has no blocks to spare)
+    if (SHARED == 0 && blockIdx.x >= routed_blocks) {
         // A decode step's spare blocks: once the row's routes are out they read the down tiles of its experts - the rows
         // the next launch's block on THIS XCD will want (blocks go to XCDs round robin) - so that launch finds them in
         // the XCD's L2. Nothing is kept; a block that never sees the routes just leaves.
@@ -629,11 +689,11 @@ __global__ __launch_bounds__(256, 2) void route_gate_up_persistent(
                 asm volatile("" ::"v"(tv[h][u].x), "v"(tv[h][u].y), "v"(tv[h][u].z), "v"(tv[h][u].w), "v"(sv[h][u].x), "v"(sv[h][u].y));
         return;
     }
-    if constexpr (SHARED) {
+    if constexpr (SHARED != 0) {
         routed_blocks -= sh.blocks;
         if (blockIdx.x >= routed_blocks) {
             __syncthreads();      // the logits' partial sums (in s_red) have been read
-            shared_gate_up_role<F16>(s_red, ps, sh, rows, blockIdx.x - routed_blocks);
+            shared_gate_up_role<F16, SHARED == 2>(s_red, ps, sh, rows, blockIdx.x - routed_blocks);
             return;
         }
     }
@@ -765,6 +825,9 @@ struct SharedDown {
     const uint16_t *acts;       // [rows][g.f]
     float *partials;            // [chunks][rows][g.d]
     uint32_t first_slot, rows;
+    // an 8-bit shared expert (not null): its down projection as nibble planes, 16 weight rows per tile row (matrix.hip) -
+    // twice the tile rows, so a chunk of its K takes two slots: first_slot + 2 c + h walks half h of chunk c's tile rows
+    const uint8_t *tiles8, *scales8;
 };
 
 template <bool OUT_BF16, bool F16, bool SHARED>
@@ -774,7 +837,7 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
                                                           float *__restrict__ partials_f32,
                                                           uint16_t *__restrict__ partials_bf16, uint32_t parts, RouteMail *mail,
                                                           SharedArg<SHARED, SharedDown> sh_arg) {
-    SharedDown sh{nullptr, g, nullptr, nullptr, 0xFFFFFFFFu, 0u};
+    SharedDown sh{nullptr, g, nullptr, nullptr, 0xFFFFFFFFu, 0u, nullptr, nullptr};
     if constexpr (SHARED) sh = sh_arg;
     __shared__ __align__(16) uint8_t s_act[kMaxRows * kDownLdsRow];
     __shared__ uint32_t s_route[kMaxRows];
@@ -782,7 +845,9 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
     if (mail && blockIdx.x == 0 && threadIdx.x == 0) advance_epoch(mail);
     const uint32_t slot_id = blockIdx.x / parts, part = blockIdx.x % parts;
     const bool shared = SHARED && slot_id >= sh.first_slot;
-    const uint32_t chunk = shared ? slot_id - sh.first_slot : 0u;
+    const bool planes8 = SHARED && shared && sh.tiles8 != nullptr;
+    const uint32_t shared_slot = shared ? slot_id - sh.first_slot : 0u;
+    const uint32_t chunk = planes8 ? shared_slot >> 1 : shared_slot;
     const PlanSlot &slot = plan->slots[shared ? 0u : slot_id];
     const uint32_t n = shared ? sh.rows : __builtin_amdgcn_readfirstlane(slot.n);
     const uint32_t expert = shared ? 0u : __builtin_amdgcn_readfirstlane(slot.expert);
@@ -805,12 +870,15 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
         // rows past the count re-read the last one (never stored): no load sits behind a branch
         early[k] = *reinterpret_cast<const uint4 *>(act_rows + (size_t)route_of(min(r, n - 1)) * act_stride + c * 8);
     }
-    const uint32_t rb = part * 4 + wave;
-    const bool has_row = rb < g.dn_rbp;
+    const uint32_t rb = planes8 ? ((shared_slot & 1u) * parts + part) * 4 + wave : part * 4 + wave;
+    const bool has_row = rb < (planes8 ? 2 * g.dn_rbp : g.dn_rbp);        // d is a multiple of 32: twice as many 16-row tile rows
     const ArenaGeom &eg = shared ? sh.g : g;
     const uint8_t *expert_base = shared ? sh.arena_layer : arena_layer + (size_t)expert * g.expert_bytes;
-    const TileSource src = make_tile_source(expert_base + eg.dn_tiles_off, (size_t)eg.dn_rbp * eg.gf * kTileBytes,
-                                            expert_base + eg.dn_scales_off, (size_t)eg.dn_rbp * eg.gf * kTileScaleBytes);
+    const TileSource src =
+        planes8 ? make_tile_source(sh.tiles8, (size_t)2 * g.dn_rbp * eg.gf * kTileBytes, sh.scales8,
+                                   (size_t)2 * g.dn_rbp * eg.gf * kTileScaleBytes)
+                : make_tile_source(expert_base + eg.dn_tiles_off, (size_t)eg.dn_rbp * eg.gf * kTileBytes,
+                                   expert_base + eg.dn_scales_off, (size_t)eg.dn_rbp * eg.gf * kTileScaleBytes);
     const uint32_t tile0 = rb * row_groups + g_first;      // the wave's first tile
     WeightRing ring;
     if (has_row) {
@@ -864,7 +932,9 @@ __global__ __launch_bounds__(256, 5) void skinny_down_lds(const uint8_t *__restr
         const uint32_t ts = 4 * jq + r;
         if (ts < n) {
             const size_t base = (size_t)s_route[ts] * g.d;
-            if (OUT_BF16 && !shared) {
+            if (planes8) {
+                rows_f32[base + rb * kTileRows + j] = tot.a[r] + tot.b[r];       // the two planes of one weight row
+            } else if (OUT_BF16 && !shared) {
                 partials_bf16[base + row_a] = Act<F16>::round(tot.a[r]);
                 partials_bf16[base + row_b] = Act<F16>::round(tot.b[r]);
             } else {
@@ -1152,8 +1222,11 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     // The shared expert rides along in the persistent gate/up launch and the LDS form of the down launch.
     if (shared && !(gu_persistent && dn_whole && rows_only && shared->g.d == g.d && shared->g.gd == g.gd))
         return hipErrorInvalidValue;
-    SharedGateUp sh_gu{nullptr, g, nullptr, 0u, nullptr, 0u};
-    SharedDown sh_dn{nullptr, g, nullptr, nullptr, 0xFFFFFFFFu, 0u};
+    const bool shared8 = shared && shared->gu_tiles8;
+    if (shared8 && (!shared->gu_scales8 || !shared->dn_tiles8 || !shared->dn_scales8 || shared->g.f % 16 || g.d % 32))
+        return hipErrorInvalidValue;
+    SharedGateUp sh_gu{nullptr, g, nullptr, 0u, nullptr, 0u, nullptr, nullptr};
+    SharedDown sh_dn{nullptr, g, nullptr, nullptr, 0xFFFFFFFFu, 0u, nullptr, nullptr};
     auto shared_blocks = [&](uint32_t cap, uint32_t routed_wanted) -> uint32_t {
         // Blocks for the shared expert's row blocks: one each when the grid has room (a decode step); else its share of
         // the resident blocks by row blocks, the routed experts counted at the number of live ones a block of t rows
@@ -1161,10 +1234,10 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
         // theirs may walk a row block or two more than a routed one: a fifth fewer than the fair share. Measured per
         // layer block of 16 / 8 / 4 rows with 12 ... 132 such blocks: flat within 0.5 us from 19 / 27 / 33 blocks up
         // (70.0 / 55.8 / 44.4 us; this rule picks 23 / 42 / 72), 6 to 12 us worse at 12 blocks.
-        const uint32_t rb = shared->g.gu_rb;
+        const uint32_t rb = shared->g.gu_rb, work = shared8 ? 2 * rb : rb;      // 8-bit: a row block is a pair of tiles
         if (routed_wanted + rb <= cap) return rb;
         const uint32_t live = min(slots, 3 * t + 2);
-        const uint32_t fair = (uint32_t)(((uint64_t)cap * rb) / ((uint64_t)live * g.gu_rb + rb));
+        const uint32_t fair = (uint32_t)(((uint64_t)cap * work) / ((uint64_t)live * g.gu_rb + work));
         return max(1u, min(rb, min(cap / 2, fair - fair / 5)));
     };
     if (fuse) {
@@ -1172,7 +1245,7 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
         uint32_t blocks = min(route->resident_blocks, max(max(slots, t), min(route->resident_blocks, slots * g.gu_rb)));
         if (shared) {
             const uint32_t sb = shared_blocks(route->resident_blocks, blocks);
-            sh_gu = SharedGateUp{shared->arena_layer, shared->g, shared->x, shared->x_stride, shared->acts, sb};
+            sh_gu = SharedGateUp{shared->arena_layer, shared->g, shared->x, shared->x_stride, shared->acts, sb, shared->gu_tiles8, shared->gu_scales8};
             blocks = max(t, min(blocks, route->resident_blocks - sb)) + sb;
         }
         // A decode step leaves blocks to spare: one per tile row of the down projection reads that row's tiles of the
@@ -1190,22 +1263,26 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
                        route->router_x_stride, t, route->mail, route->poll_ticks, const_cast<uint32_t *>(idx),                \
                        const_cast<uint16_t *>(w), plan,                                                                     \
                        x, x_stride, acts, shared_arg<SH>(sh_gu), prefetch_blocks)
-        if (shared) { if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true, true); else FFMOE_ROUTE_GU(false, true); }
-        else { if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true, false); else FFMOE_ROUTE_GU(false, false); }
+        if (shared8) { if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true, 2); else FFMOE_ROUTE_GU(false, 2); }
+        else if (shared) { if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true, 1); else FFMOE_ROUTE_GU(false, 1); }
+        else { if (route->rw.w_is_f32) FFMOE_ROUTE_GU(true, 0); else FFMOE_ROUTE_GU(false, 0); }
 #undef FFMOE_ROUTE_GU
     } else if (gu_persistent) {
         // plan slot of the profile stays empty: the gate/up kernel builds the plan itself
         uint32_t blocks = max(slots, min(resident, slots * g.gu_rb));
         if (shared) {
             const uint32_t sb = shared_blocks(max(resident, blocks), blocks);
-            sh_gu = SharedGateUp{shared->arena_layer, shared->g, shared->x, shared->x_stride, shared->acts, sb};
+            sh_gu = SharedGateUp{shared->arena_layer, shared->g, shared->x, shared->x_stride, shared->acts, sb, shared->gu_tiles8, shared->gu_scales8};
             blocks = max(1u, min(blocks, max(resident, blocks) - sb)) + sb;
         }
         if (dense)
             hipLaunchKernelGGL((skinny_gate_up_persistent<F16, true>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k,
                                n_experts, idx, w, t * top_k, plan, x, x_stride, acts, NoSharedExpert{});
+        else if (shared8)
+            hipLaunchKernelGGL((skinny_gate_up_persistent<F16, false, 2>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k,
+                               n_experts, idx, w, t * top_k, plan, x, x_stride, acts, sh_gu);
         else if (shared)
-            hipLaunchKernelGGL((skinny_gate_up_persistent<F16, false, true>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k,
+            hipLaunchKernelGGL((skinny_gate_up_persistent<F16, false, 1>), dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k,
                                n_experts, idx, w, t * top_k, plan, x, x_stride, acts, sh_gu);
         else
             hipLaunchKernelGGL(skinny_gate_up_persistent<F16>, dim3(blocks), dim3(256), 0, s, arena_layer, g, top_k, n_experts, idx,
@@ -1240,8 +1317,8 @@ hipError_t launch_verify_as(hipStream_t s, const uint8_t *arena_layer, ArenaGeom
     }
     const uint32_t dn_parts = (g.dn_rbp + 3) / 4;          // blocks per expert of the LDS form: four tile rows each
     const bool dense_ksplit = dense && gu_persistent;      // the plan-free forms go together
-    if (shared) sh_dn = SharedDown{shared->arena_layer, shared->g, shared->acts, shared->partials, slots, t};
-    const dim3 dn_grid = dn_whole    ? dim3((slots + (shared ? shared_chunks(shared->g) : 0u)) * dn_parts)
+    if (shared) sh_dn = SharedDown{shared->arena_layer, shared->g, shared->acts, shared->partials, slots, t, shared->dn_tiles8, shared->dn_scales8};
+    const dim3 dn_grid = dn_whole    ? dim3((slots + (shared ? shared_chunks(shared->g) * (shared8 ? 2u : 1u) : 0u)) * dn_parts)
                          : dn_ksplit ? dim3(max(slots, min(resident, slots * g.dn_rbp)))
                                      : dim3((g.dn_rbp + 3) / 4, slots);
 #define FFMOE_DOWN(BF)                                                                                                \
@@ -1378,14 +1455,18 @@ uint32_t route_launch_resident_blocks(uint32_t n_cus) {
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess) n = 0;
         least = n < least ? n : least;
     };
-    ask(route_gate_up_persistent<false, false, false>);
-    ask(route_gate_up_persistent<true, false, false>);
-    ask(route_gate_up_persistent<false, true, false>);
-    ask(route_gate_up_persistent<true, true, false>);
-    ask(route_gate_up_persistent<false, false, true>);
-    ask(route_gate_up_persistent<true, false, true>);
-    ask(route_gate_up_persistent<false, true, true>);
-    ask(route_gate_up_persistent<true, true, true>);
+    ask(route_gate_up_persistent<false, false, 0>);
+    ask(route_gate_up_persistent<true, false, 0>);
+    ask(route_gate_up_persistent<false, true, 0>);
+    ask(route_gate_up_persistent<true, true, 0>);
+    ask(route_gate_up_persistent<false, false, 1>);
+    ask(route_gate_up_persistent<true, false, 1>);
+    ask(route_gate_up_persistent<false, true, 1>);
+    ask(route_gate_up_persistent<true, true, 1>);
+    ask(route_gate_up_persistent<false, false, 2>);
+    ask(route_gate_up_persistent<true, false, 2>);
+    ask(route_gate_up_persistent<false, true, 2>);
+    ask(route_gate_up_persistent<true, true, 2>);
     (void)hipGetLastError();
     return least > 0 ? (uint32_t)least * n_cus : 0u;
 }

@@ -50,7 +50,7 @@ EXPORTS = [
     "ffmoe_layer_tail", "ffmoe_layer_tail_routed", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
     "ffmoe_verify_static", "ffmoe_route_verify_shared", "ffmoe_layer_tail_routed_shared", "ffmoe_sample_rows",
-    "ffmoe_matrix_create_int8", "ffmoe_matrix_create_int8_glu", "ffmoe_gelu_mul",
+    "ffmoe_matrix_create_int8", "ffmoe_matrix_create_int8_glu", "ffmoe_gelu_mul", "ffmoe_upload_expert_parts_int8",
 ]
 
 PROFILE_SLOTS = 16
@@ -249,6 +249,7 @@ def lib() -> C.CDLL:
     L.ffmoe_argmax_rows.argtypes = [vp, vp, vp, u32, u32, u32, C.c_float, vp, vp, errp]
     L.ffmoe_upload_expert_parts.argtypes = [vp, u32, u32, C.POINTER(Projection), C.POINTER(Projection),
                                             C.POINTER(Projection), i32, errp]
+    L.ffmoe_upload_expert_parts_int8.argtypes = [vp, u32, C.POINTER(Projection), C.POINTER(Projection), C.POINTER(Projection), errp]
     L.ffmoe_dense_ffn.argtypes = [vp, vp, u32, vp, u32, u32, vp, errp]
     L.ffmoe_post_attn_setup.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, vp, u32, vp, u32, vp, vp, vp, u32, u32,
                                         C.c_float, errp]
@@ -351,8 +352,9 @@ class Context:
             p, on_dev = C.c_void_p(blobs.data_ptr()), int(blobs.is_cuda)
         _check(self.L.ffmoe_upload_layer(self._h, layer, p, stride, C.byref(offsets), on_dev, C.byref(err)), err)
 
-    def upload_expert_parts(self, layer: int, expert: int, gate, up, down):
-        """One expert from three (W uint8, S bf16 bits, B bf16 bits) triples: all numpy arrays or all CUDA tensors."""
+    def upload_expert_parts(self, layer: int, expert: int, gate, up, down, int8: bool = False):
+        """One expert from three (W uint8, S bf16 bits, B bf16 bits) triples: all numpy arrays or all CUDA tensors.
+        int8: the triples hold 8-bit weights (W uint8 [rows, cols]); dense contexts only, expert 0."""
         import numpy as np
         keep, kinds = [], set()
 
@@ -373,6 +375,10 @@ class Context:
         g, u, dn = proj(gate), proj(up), proj(down)
         assert len(kinds) == 1, "all nine arrays must live on the same side"
         err = C.c_char_p()
+        if int8:
+            assert expert == 0
+            _check(self.L.ffmoe_upload_expert_parts_int8(self._h, layer, C.byref(g), C.byref(u), C.byref(dn), C.byref(err)), err)
+            return
         _check(self.L.ffmoe_upload_expert_parts(self._h, layer, expert, C.byref(g), C.byref(u), C.byref(dn),
                                                 kinds.pop(), C.byref(err)), err)
 

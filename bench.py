@@ -648,9 +648,10 @@ def main():
         t1 = timed(lambda: dense_step(x1s, y1s), 200, warm=10)
         shared["rows1"] = {"us": round(t1 * 1e6, 2), "GBs": round(s_payload / t1 / 1e9, 1)}
         # the same FFN in the 8-bit form the reference's packs hold by default (SharedExpertInt8.swift:56-135): two nibble
-        # planes per weight on the 4-bit streaming kernel; gate and up as one gated matrix (the activation is that pass's
-        # epilogue), then the down projection: two launches
-        m8, bytes8 = [], 0
+        # planes per weight on the 4-bit streaming kernels, as layers of a second dense context; gate and up are one gated
+        # matrix (the activation is that pass's epilogue), then the down projection: two launches per call
+        dense8 = ff.Context(D, FS, 1, 1, n_layers=LS, max_tokens=16)
+        bytes8 = 0
         for layer in range(LS):
             parts8 = []
             for rows, cols in ((FS, D), (FS, D), (D, FS)):
@@ -658,17 +659,13 @@ def main():
                 w8 = torch.randint(0, 256, (rows, cols), dtype=torch.uint8, device="cuda", generator=gen)
                 sc = (torch.randn((rows, g_), device="cuda", generator=gen) * 0.001).abs().to(torch.bfloat16)
                 bi = (-128.0 * sc.float() + torch.randn((rows, g_), device="cuda", generator=gen) * 1e-3).to(torch.bfloat16)
-                parts8.append((w8, sc, bi))
+                parts8.append((w8, sc.contiguous(), bi.contiguous()))
                 bytes8 += (rows * cols + 4 * rows * g_) if layer == 0 else 0
-            m8.append((ctx.matrix_int8_glu(parts8[0], parts8[1]), ctx.matrix_int8(*parts8[2])))
+            dense8.upload_expert_parts(layer, 0, *parts8, int8=True)
             del parts8
-        act8 = torch.empty((T, FS), dtype=torch.bfloat16, device="cuda")
 
         def int8_step(xin, yout):
-            gate_up8, down8 = m8[state["i"] % LS]
-            a8 = act8[:xin.shape[0]]
-            gate_up8.gemv(xin, out=a8)
-            down8.gemv(a8, out=yout)
+            dense8.dense_ffn(state["i"] % LS, xin, out=yout)
             state["i"] += 1
         t8_16 = timed(lambda: int8_step(x, y16), 200, warm=10)
         t8_1 = timed(lambda: int8_step(x1s, y1s), 200, warm=10)
@@ -746,15 +743,38 @@ def main():
         def run_inside():
             layer_block_inside(counter["i"])
             counter["i"] += 1
+        def layer_block_int8(i, inside):
+            # the block with the shared expert in the packs' default 8-bit form: separate calls with the combine in the
+            # tail (six launches), or inside the routed experts' launches like the 4-bit one (four)
+            ctx.post_attn_setup(hid_b, att_b, wn_b[0], wn_b[1], wn_b[2], out=outs_b)
+            if inside:
+                rc = Lib.ffmoe_route_verify_shared(h, dense8._h, stream, i % L, i % LS, pouts[2], D, pouts[1], D, pouts[0], D, T,
+                                                   pidx, pw, C.byref(err))
+                if rc:
+                    raise RuntimeError(err.value)
+                ctx.layer_tail_routed_shared(dense8, w, hid_b, wn_b[3], wn_b[4], 1.0)
+                return
+            dense8.dense_ffn(i % LS, outs_b[0], out=h1_b)
+            rc = Lib.ffmoe_route_verify(h, stream, i % L, pouts[2], D, pouts[1], D, T, None, None, pidx, pw, C.byref(err))
+            if rc:
+                raise RuntimeError(err.value)
+            ctx.layer_tail_routed(w, h1_b, hid_b, wn_b[3], wn_b[4], 1.0)
+
+        def run_int8(inside):
+            layer_block_int8(counter["i"], inside)
+            counter["i"] += 1
         t_seq = timed(lambda: run_block(False), 120, warm=30)
         t_con = timed(lambda: run_block(True), 120, warm=30)
+        t_i8 = timed(lambda: run_int8(False), 120, warm=30)
+        t_i8c = timed(lambda: run_int8(True), 120, warm=30)
         t_fus = timed(run_fused, 120, warm=30)
         t_ins = timed(run_inside, 120, warm=30)
         # the same chain of L layers as a HIP graph: nine launches per layer from Python are host-bound,
         # a replay shows the device time (the library only enqueues kernels, so the chain captures as it is)
         graph_us = {}
         for label, conc in (("one_stream", False), ("shared_expert_on_second_stream", True), ("combine_in_layer_tail", None),
-                            ("shared_expert_inside_routed_launches", "inside")):
+                            ("shared_expert_inside_routed_launches", "inside"), ("shared_expert_int8", "int8"),
+                            ("shared_expert_int8_inside_routed_launches", "int8i")):
             gph = torch.cuda.CUDAGraph()
             cap = torch.cuda.Stream()
             cap.wait_stream(main_s)
@@ -764,6 +784,8 @@ def main():
                 for i in range(L):
                     if conc == "inside":
                         layer_block_inside(i)
+                    elif conc in ("int8", "int8i"):
+                        layer_block_int8(i, conc == "int8i")
                     elif conc is None:
                         layer_block_fused(i)
                     else:
@@ -776,7 +798,10 @@ def main():
                                        "combine_in_layer_tail_us": round(t_fus * 1e6, 2),
                                        "shared_expert_inside_routed_launches_us": round(t_ins * 1e6, 2),
                                        "best_one_stream_us": round(min(t_seq, t_fus, t_ins) * 1e6, 2),
-                                       "launches": {"one_stream": 7, "combine_in_layer_tail": 6, "shared_expert_inside_routed_launches": 4},
+                                       "shared_expert_int8_us": round(t_i8 * 1e6, 2),
+                                       "shared_expert_int8_inside_routed_launches_us": round(t_i8c * 1e6, 2),
+                                       "launches": {"one_stream": 7, "combine_in_layer_tail": 6, "shared_expert_inside_routed_launches": 4,
+                                                    "shared_expert_int8": 6, "shared_expert_int8_inside_routed_launches": 4},
                                        "hip_graph_replay_us": graph_us,
                                        "steps": "post-attention setup, shared expert, router, routed experts, layer tail"}
         # the same block for a decode step (one row), separate calls against the shared expert inside the routed launches
@@ -798,14 +823,31 @@ def main():
             ctx.post_attn_setup(hid1, att1, wn_b[0], wn_b[1], wn_b[2], out=outs1)
             _, w1 = ctx.route_verify_shared(dense, i % L, i % LS, outs1[2], outs1[1], outs1[0])
             ctx.layer_tail_routed_shared(dense, w1, hid1, wn_b[3], wn_b[4], 1.0)
+        def block1_int8(inside):
+            i = counter["i"]
+            counter["i"] += 1
+            ctx.post_attn_setup(hid1, att1, wn_b[0], wn_b[1], wn_b[2], out=outs1)
+            if inside:
+                _, w1 = ctx.route_verify_shared(dense8, i % L, i % LS, outs1[2], outs1[1], outs1[0])
+                ctx.layer_tail_routed_shared(dense8, w1, hid1, wn_b[3], wn_b[4], 1.0)
+                return
+            dense8.dense_ffn(i % LS, outs1[0], out=h11)
+            _, _, w1 = ctx.route_verify(i % L, outs1[2], outs1[1], combine=False)
+            ctx.layer_tail_routed(w1, h11, hid1, wn_b[3], wn_b[4], 1.0)
         t1_sep = timed(block1_separate, 120, warm=30)
         t1_ins = timed(block1_inside, 120, warm=30)
+        t1_i8 = timed(lambda: block1_int8(False), 120, warm=30)
+        t1_i8c = timed(lambda: block1_int8(True), 120, warm=30)
         extra["layer_block_rows1"] = {"separate_calls_us": round(t1_sep * 1e6, 2),
                                       "shared_expert_inside_routed_launches_us": round(t1_ins * 1e6, 2),
-                                      "launches": {"separate_calls": 6, "shared_expert_inside_routed_launches": 4},
+                                      "shared_expert_int8_us": round(t1_i8 * 1e6, 2),
+                                      "shared_expert_int8_inside_routed_launches_us": round(t1_i8c * 1e6, 2),
+                                      "launches": {"separate_calls": 6, "shared_expert_inside_routed_launches": 4, "shared_expert_int8": 6,
+                                                   "shared_expert_int8_inside_routed_launches": 4},
                                       "moe_blocks_of_30_layers_ms": round(30 * t1_ins * 1e3, 3),
                                       "steps": "post-attention setup, shared expert, router, routed experts, layer tail (combine in the tail)"}
         dense.close()
+        dense8.close()
 
     # The row-wise steps either side of the MoE stage at the prefill chunk and at a verify block:
     # 2 row reads + 4 row writes (setup), 3 reads + 1 write (tail); weights stay in cache

@@ -467,6 +467,18 @@ int ffmoe_layer_tail_routed(ffmoe_ctx *ctx, void *stream, const uint16_t *route_
                             uint16_t *hidden, uint32_t hidden_stride, const uint16_t *w_postffn2, const uint16_t *w_postffn,
                             uint32_t t, float eps, float layer_scalar, char **err);
 
+/* The same for an 8-bit shared expert (each W uint8 [rows][cols], one value per byte; S/B as above; host or device
+ * memory), the form in which the reference's packs hold it by default (SharedExpertInt8.encode,
+ * Kernels/MoE/SharedExpertInt8.swift:56-135; Model.sharedExpertWeightBits, Runtime/Inference/Model.swift:13). Only on a
+ * context with n_experts = 1 and top_k = 1, d and f multiples of 64 up to FFMOE_MATRIX_MAX_N. The layer is then kept as
+ * a gated gate/up matrix and a down matrix of nibble planes (ffmoe_matrix_create_int8_glu / _int8) owned by the
+ * context, and ffmoe_dense_ffn, ffmoe_route_verify_shared and ffmoe_layer_tail_routed_shared serve it like a 4-bit
+ * layer: ffmoe_dense_ffn runs the two GEMV passes per 16 rows (gate and up are rounded to 16 bits in front of the
+ * activation, as the reference's fused kernel does, dequant_int8.metal:131-136). An upload in either width replaces
+ * the layer's 8-bit form or leaves it in place: the 8-bit form, once uploaded, is the one that is served. Blocking. */
+int ffmoe_upload_expert_parts_int8(ffmoe_ctx *ctx, uint32_t layer, const ffmoe_projection *gate,
+                                   const ffmoe_projection *up, const ffmoe_projection *down, char **err);
+
 /* The expert work of one MoE block for a decode step / verify block (t <= 16) with the shared expert inside the
  * routed experts' two launches: ffmoe_route_verify(ctx, ..., y = NULL) on (router_x, x) and ffmoe_dense_ffn(shared, ...)
  * on shared_x in one call. `shared` is a context with n_experts = 1 and top_k = 1 (ffmoe_upload_expert_parts /

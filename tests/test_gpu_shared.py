@@ -248,3 +248,129 @@ def test_route_verify_shared_argument_errors(ff, oracle, torch):
         ctx.route_verify_shared(wide, 0, 0, x, x, x)
     for c in (ctx, other, wide):
         c.close()
+
+
+def _int8_parts(oracle, g, d, fs, scale):
+    return tuple(oracle.quantize_int8(g.uniform(-scale, scale, r * c).reshape(r, c)) for r, c in ((fs, d), (fs, d), (d, fs)))
+
+
+def _int8_reference_rows(oracle, parts, x_bits):
+    """SharedExpertInt8Tests.swift:33-41 per row: DequantInt8GemvRef for gate and up, the activation rounded to 16 bits
+    once, DequantInt8GemvRef for down (float64 tanh: the single-precision form cancels below about -4)."""
+    (gW, gS, gB), (uW, uS, uB), (dW, dS, dB) = parts
+    out = []
+    for row in x_bits:
+        x = oracle.bf16_to_float(row)
+        g64 = oracle.gemv_int8_ref(gW, gS, gB, x).astype(np.float64)
+        u = oracle.gemv_int8_ref(uW, uS, uB, x)
+        act = (0.5 * g64 * (1.0 + np.tanh(0.7978845608028654 * (g64 + 0.044715 * g64 ** 3)))).astype(np.float32) * u
+        out.append(oracle.gemv_int8_ref(dW, dS, dB, oracle.bf16_to_float(oracle.bf16_bits(act))))
+    return np.stack(out)
+
+
+@pytest.mark.parametrize("d,fs,t", [(128, 64, 1), (128, 192, 16), (192, 1472, 5), (2816, 2112, 16), (128, 64, 40)])
+def test_dense_ffn_on_an_int8_layer(ff, oracle, torch, d, fs, t):
+    # the 8-bit shared expert as a layer of the dense context: ffmoe_dense_ffn equals the gated matrix + down matrix calls
+    # bit for bit (it runs the same two kernels, 16 rows at a time) and follows the reference's rows
+    g = oracle.seed_tree_key(0x1A8, f"dense-int8-d{d}-fs{fs}-t{t}")
+    parts = _int8_parts(oracle, g, d, fs, 0.4 if d < 1024 else 0.08)
+    dense = ff.Context(d, fs, 1, 1, n_layers=2, max_tokens=max(t, 16))
+    x = torch.zeros((1, d), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ff.FieldfareError, match="not uploaded"):
+        dense.dense_ffn(1, x)
+    dense.upload_expert_parts(1, 0, *parts, int8=True)
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    xt = bf16_tensor(torch, xb)
+    y = dense.dense_ffn(1, xt)
+    gate_up, down = dense.matrix_int8_glu(parts[0], parts[1]), dense.matrix_int8(*parts[2])
+    want = torch.cat([down.gemv(gate_up.gemv(xt[r0:r0 + 16])) for r0 in range(0, t, 16)])
+    assert torch.equal(y.view(torch.int16), want.view(torch.int16))
+    if d * fs <= 192 * 1472 or t <= 16:
+        rows = slice(0, min(t, 4) if d > 1024 else t)
+        ref = _int8_reference_rows(oracle, parts, xb[rows])
+        got = oracle.bf16_to_float(bits_of(y))[rows]
+        assert rel_err(got, ref) < 1e-2 and cosine(got, ref) > 0.9999, (rel_err(got, ref), cosine(got, ref))
+    with pytest.raises(ff.FieldfareError, match="outside"):
+        dense.dense_ffn(1, torch.zeros((max(t, 16) + 1, d), dtype=torch.bfloat16, device="cuda"))
+    routed = ff.Context(128, 64, 4, 2, n_layers=1, max_tokens=16)
+    with pytest.raises(ff.FieldfareError, match="n_experts = 1"):
+        routed.upload_expert_parts(0, 0, *_int8_parts(oracle, g, 128, 64, 0.4), int8=True)
+    for c in (gate_up, down, dense, routed):
+        c.close()
+
+
+@pytest.mark.parametrize("d,f,e,fs,t,mode", [
+    (128, 64, 16, 192, 5, "one_launch"),
+    (128, 64, 16, 1472, 16, "one_launch"),        # 23 groups: chunks of 11, 11 and 1, two down slots each
+    (128, 64, 16, 1472, 3, "router_launches"),
+    (128, 64, 16, 1472, 7, "no_hand_over"),
+    (2816, 704, 128, 2112, 1, "one_launch"),      # the model's shapes: decode step
+    (2816, 704, 128, 2112, 16, "one_launch"),     # verify block
+    (2816, 704, 128, 2112, 6, "router_launches"),
+])
+def test_int8_shared_expert_inside_the_routed_launches(ff, oracle, torch, d, f, e, fs, t, mode):
+    """ffmoe_route_verify_shared + ffmoe_layer_tail_routed_shared with the shared expert held 8-bit, against the separate
+    calls (ffmoe_route_verify, ffmoe_dense_ffn on the 8-bit layer, ffmoe_layer_tail): same routes bit for bit; the new
+    hidden rows agree to the rounding of the shared expert's row (its K is summed in chunks there), bit for bit with a
+    shared expert of zero weights; the shared expert's own row follows the reference. A 4-bit layer of the same dense
+    context is served side by side."""
+    from helpers import make_layer, to_ff_offsets
+    rng, pool, router = make_layer(oracle, 5, d, f, e, align=16)
+    ctx = ff.Context(d, f, e, 8, n_layers=1, max_tokens=16)
+    ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
+    ctx.upload_router_bf16(0, router)
+    g = oracle.seed_tree_key(0x5A4F, f"shared8-inside-d{d}-fs{fs}-t{t}-{mode}")
+    parts = _int8_parts(oracle, g, d, fs, 0.4 if d < 1024 else 0.08)
+    zero_parts = tuple(oracle.quantize_int8(np.zeros((r, c), np.float32)) for r, c in ((fs, d), (fs, d), (d, fs)))
+    parts4 = tuple(oracle.quantize_int4(g.uniform(-0.1, 0.1, r * c).reshape(r, c)) for r, c in ((fs, d), (fs, d), (d, fs)))
+    shared = ff.Context(d, fs, 1, 1, n_layers=3, max_tokens=16)
+    shared.upload_expert_parts(0, 0, *zero_parts, int8=True)
+    shared.upload_expert_parts(1, 0, *parts, int8=True)
+    shared.upload_expert_parts(2, 0, *parts4)
+    pad = 8
+    xb, rxb, sxb = (oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d) for _ in range(3))
+    x, rx, sx = bf16_tensor(torch, xb), bf16_tensor(torch, rxb), bf16_tensor(torch, sxb)
+    hid = np.full((t, d + pad), oracle.bf16_bits(np.float32(-25.0)), np.uint16)
+    hid[:, :d] = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    tw2, tw1 = (bf16_tensor(torch, oracle.bf16_bits(g.uniform(0.5, 1.5, d))) for _ in range(2))
+    if mode == "router_launches":
+        ctx.set_one_launch_routing(False)
+    if mode == "no_hand_over":
+        ctx.set_handover_timeout(0)
+    for layer_s in (0, 1, 2):
+        y, idx_a, w_a = ctx.route_verify(0, rx, x)
+        h1 = shared.dense_ffn(layer_s, sx)
+        hid_a = bf16_tensor(torch, hid)
+        ctx.layer_tail(y, h1, hid_a, tw2, tw1, 0.875, 1e-6, d=d)
+        idx_b, w_b = ctx.route_verify_shared(shared, 0, layer_s, rx, x, sx)
+        hid_b = bf16_tensor(torch, hid)
+        ctx.layer_tail_routed_shared(shared, w_b, hid_b, tw2, tw1, 0.875, 1e-6)
+        assert np.array_equal(idx_a.cpu().numpy(), idx_b.cpu().numpy()) and np.array_equal(bits_of(w_a), bits_of(w_b))
+        got, want = bits_of(hid_b), bits_of(hid_a)[:, :d]
+        assert np.array_equal(got[:, d:], hid[:, d:])
+        if layer_s == 0:
+            assert float(h1.abs().max()) == 0.0
+            assert np.array_equal(got[:, :d], want)
+        else:
+            gf, wf = oracle.bf16_to_float(got[:, :d]), oracle.bf16_to_float(want)
+            assert rel_err(gf, wf) < 1e-2 and cosine(gf, wf) > 0.9999, (layer_s, rel_err(gf, wf), cosine(gf, wf))
+            assert np.mean(got[:, :d] == want) > 0.8
+    # the shared expert's row itself: with the routed rows' norm weight at zero the tail is hidden + norm(h1) scaled
+    zero = torch.zeros_like(tw2)
+    one = torch.ones_like(tw1)
+    hid0 = torch.zeros((t, d), dtype=torch.bfloat16, device="cuda")
+    _, w_c = ctx.route_verify_shared(shared, 0, 1, rx, x, sx)
+    ctx.layer_tail_routed_shared(shared, w_c, hid0, zero, one, 1.0, 1e-6)
+    rows = slice(0, min(t, 3) if d > 1024 else t)
+    ref_bits = oracle.bf16_bits(_int8_reference_rows(oracle, parts, sxb[rows]).astype(np.float32))
+    n_ref = ref_bits.shape[0]
+    want0 = oracle.layer_tail(np.zeros((n_ref, d), np.uint16), ref_bits, np.zeros((n_ref, d), np.uint16), bits_of(zero), bits_of(one),
+                              1.0, 1e-6)
+    g0, w0 = oracle.bf16_to_float(bits_of(hid0))[rows], oracle.bf16_to_float(want0)
+    assert rel_err(g0, w0) < 1e-2 and cosine(g0, w0) > 0.9999, (rel_err(g0, w0), cosine(g0, w0))
+    if mode == "no_hand_over":
+        assert ctx.handover_giveups() > 0
+    elif mode == "one_launch":
+        assert ctx.handover_giveups() == 0
+    ctx.close()
+    shared.close()
