@@ -697,19 +697,19 @@ private:
 };
 
 // SharedExpertInt8 (Kernels/MoE/SharedExpertInt8.swift:40-135): y = down(gelu_tanh(gate(x)) * up(x)) with the three
-// projections 8-bit affine, the form in which the packs hold the shared expert by default. The Swift class binds
-// the projections on every call; here load() re-tiles one layer's three once (gate and up into one gated matrix, as
-// the Swift class's fused kernel reads them) and the object keeps them. The caller's activation scratch holds
-// F values per row, as there, and may be reused across layers.
+// projections 8-bit affine, the form in which the packs hold the shared expert by default. Same shape as
+// SharedExpertInt4 above: a dense context of one expert, load() once per layer (the layer is kept as a gated gate/up
+// matrix and a down matrix of nibble planes), calls name the layer, and the activation scratch the Swift caller
+// passes is the context's.
 class SharedExpertInt8 {
 public:
-    static constexpr int maxBatchRows = DequantInt8GEMV::maxBatchRows;
-    explicit SharedExpertInt8(Context &c) : c_(c) {}
-    ~SharedExpertInt8() { ffmoe_matrix_destroy(gateUp_); }
-    SharedExpertInt8(const SharedExpertInt8 &) = delete;
-    SharedExpertInt8 &operator=(const SharedExpertInt8 &) = delete;
-    // the guards of SharedExpertInt8.encode (SharedExpertInt8.swift:63-70), then the uploads
-    void load(const SharedExpertProjection &gate, const SharedExpertProjection &up, const SharedExpertProjection &down) {
+    explicit SharedExpertInt8(Context &dense) : c_(dense) {
+        if (dense.shape().n_experts != 1 || dense.shape().top_k != 1)
+            throw std::invalid_argument("the shared expert needs a context with n_experts = 1 and top_k = 1");
+    }
+    // the guards of SharedExpertInt8.encode (SharedExpertInt8.swift:63-70), then the upload; host or device pointers
+    void load(uint32_t layer, const SharedExpertProjection &gate, const SharedExpertProjection &up,
+              const SharedExpertProjection &down) {
         if (gate.rows != up.rows || gate.cols != up.cols)
             throw SharedExpertError(SharedExpertError::dimensionMismatch,
                                     "gate/up shapes differ: gate=(" + std::to_string(gate.rows) + "," + std::to_string(gate.cols) +
@@ -718,59 +718,32 @@ public:
             throw SharedExpertError(SharedExpertError::dimensionMismatch,
                                     "down expected (" + std::to_string(gate.cols) + "," + std::to_string(gate.rows) + "), got (" +
                                         std::to_string(down.rows) + "," + std::to_string(down.cols) + ")");
-        if (gate.cols % FFMOE_GROUP || gate.rows % FFMOE_GROUP) throw std::invalid_argument("N must be a multiple of 64");
-        ffmoe_matrix *gu = nullptr;
+        if (gate.rows != c_.shape().f || gate.cols != c_.shape().d)
+            throw SharedExpertError(SharedExpertError::dimensionMismatch,
+                                    "SharedExpert dimension mismatch: expected gate/up=(" + std::to_string(c_.shape().f) + "," +
+                                        std::to_string(c_.shape().d) + ")");
+        const ffmoe_projection g{gate.weights, gate.scales, gate.biases}, u{up.weights, up.scales, up.biases},
+            dn{down.weights, down.scales, down.biases};
         char *err = nullptr;
-        check(ffmoe_matrix_create_int8_glu(c_.raw(), gate.weights, gate.scales, gate.biases, up.weights, up.scales, up.biases,
-                                           gate.rows, gate.cols, &gu, &err), err);
-        ffmoe_matrix_destroy(gateUp_);
-        gateUp_ = gu;
-        f_ = gate.rows;
-        d_ = gate.cols;
-        down_.reset(new DequantInt8GEMV(c_, down.weights, down.scales, down.biases, down.rows, down.cols));
+        check(ffmoe_upload_expert_parts_int8(c_.raw(), layer, &g, &u, &dn, &err), err);
     }
-    // encode (SharedExpertInt8.swift:56-97): one row; scratchActElements is the room behind scratchAct in 16-bit values
-    void encode(void *stream, const uint16_t *x, uint16_t *y, uint16_t *scratchAct, size_t scratchActElements) {
-        encodeBlock(stream, x, y, 1, (int)d_, (int)d_, scratchAct, scratchActElements);
+    // encode (SharedExpertInt8.swift:56-97): one row
+    void encode(void *stream, uint32_t layer, const uint16_t *x, uint16_t *y) {
+        char *err = nullptr;
+        check(ffmoe_dense_ffn(c_.raw(), stream, layer, x, c_.shape().d, 1, y, &err), err);
     }
-    // a block of rows, each as encode does it; more than 16 rows go through in parts of 16 that reuse the scratch
-    void encodeBlock(void *stream, const uint16_t *x, uint16_t *y, int queryCount, int xStrideElements, int yStrideElements,
-                     uint16_t *scratchAct, size_t scratchActElements) {
-        if (!gateUp_) throw std::logic_error("SharedExpertInt8: load() first");
-        if (queryCount < 0) throw std::invalid_argument("queryCount must be non-negative");
-        if (xStrideElements < (int)d_) throw std::invalid_argument("x stride is too small");
-        if (yStrideElements < (int)d_) throw std::invalid_argument("y stride is too small");
-        const int part = queryCount < maxBatchRows ? queryCount : maxBatchRows;
-        if (scratchActElements < (size_t)part * f_)
-            throw SharedExpertError(SharedExpertError::scratchTooSmall,
-                                    "scratchAct needs " + std::to_string((size_t)part * f_) + " values, has " +
-                                        std::to_string(scratchActElements));
-        for (int r0 = 0; r0 < queryCount; r0 += maxBatchRows) {
-            const int rows = queryCount - r0 < maxBatchRows ? queryCount - r0 : maxBatchRows;
-            char *err = nullptr;
-            check(ffmoe_matrix_gemv(gateUp_, stream, x + (size_t)r0 * xStrideElements, (uint32_t)xStrideElements, (uint32_t)rows,
-                                    scratchAct, f_, 0, &err), err);
-            down_->encodeRows(stream, scratchAct, y + (size_t)r0 * yStrideElements, rows, f_, (uint32_t)yStrideElements);
-        }
-    }
-    uint32_t d() const { return d_; }
-    uint32_t intermediate() const { return f_; }
 
-private:
+protected:
     Context &c_;
-    ffmoe_matrix *gateUp_ = nullptr;
-    std::unique_ptr<DequantInt8GEMV> down_;
-    uint32_t f_ = 0, d_ = 0;
 };
 
-// SharedExpertRuntime (SharedExpertInt4.swift:92-130): picks the implementation by weight width. For 4 bits `c` is the
-// one-expert context SharedExpertInt4 takes and the calls name the layer; for 8 bits `c` is any context, one object
-// serves one layer (the `layer` arguments are ignored) and encode needs the activation scratch.
+// SharedExpertRuntime (SharedExpertInt4.swift:92-130): picks the implementation by weight width. `dense` is the
+// one-expert context both take.
 class SharedExpertRuntime {
 public:
-    SharedExpertRuntime(Context &c, int weightBits) {
-        if (weightBits == 4) int4_.reset(new SharedExpertInt4(c));
-        else if (weightBits == 8) int8_.reset(new SharedExpertInt8(c));
+    SharedExpertRuntime(Context &dense, int weightBits) : c_(dense) {
+        if (weightBits == 4) int4_.reset(new SharedExpertInt4(dense));
+        else if (weightBits == 8) int8_.reset(new SharedExpertInt8(dense));
         else
             throw SharedExpertError(SharedExpertError::unsupportedWeightBits,
                                     "SharedExpert unsupported weight bits: " + std::to_string(weightBits));
@@ -779,26 +752,29 @@ public:
     void load(uint32_t layer, const SharedExpertProjection &gate, const SharedExpertProjection &up,
               const SharedExpertProjection &down) {
         if (int4_) int4_->load(layer, gate, up, down);
-        else int8_->load(gate, up, down);
+        else int8_->load(layer, gate, up, down);
     }
-    void encode(void *stream, uint32_t layer, const uint16_t *x, uint16_t *y, uint16_t *scratchAct = nullptr,
-                size_t scratchActElements = 0) {
+    void encode(void *stream, uint32_t layer, const uint16_t *x, uint16_t *y) {
         if (int4_) int4_->encode(stream, layer, x, y);
-        else int8_->encode(stream, x, y, scratchAct, scratchActElements);
+        else int8_->encode(stream, layer, x, y);
     }
+
+protected:
+    Context &c_;
 
 private:
     std::unique_ptr<SharedExpertInt4> int4_;
     std::unique_ptr<SharedExpertInt8> int8_;
 };
 
-// PrefillSharedExpert.encodeBlock (PrefillSharedExpert.swift:94-137): a block of rows. The Swift class loops
-// its single-row operator below 32 tokens and batches above; here rows <= 16 stream the weights once for
-// all rows and more rows run the grouped GEMMs.
-class PrefillSharedExpert : public SharedExpertInt4 {
+// PrefillSharedExpert (PrefillSharedExpert.swift:19-33,94-137): a block of rows in either weight width (the Swift
+// class defaults to 8 bits). The Swift class loops its single-row operator below 32 tokens and batches the 4-bit
+// form above; here rows <= 16 stream the weights once for all rows; more rows run the grouped GEMMs (4 bits) or go
+// through 16 at a time (8 bits).
+class PrefillSharedExpert : public SharedExpertRuntime {
 public:
     static constexpr int batchedMinimumTokens = 17;
-    using SharedExpertInt4::SharedExpertInt4;
+    explicit PrefillSharedExpert(Context &dense, int weightBits = 4) : SharedExpertRuntime(dense, weightBits) {}
     void encodeBlock(void *stream, uint32_t layer, const uint16_t *x, uint16_t *y, int queryCount, int d, int intermediate,
                      int xStrideElements, int yStrideElements) {
         if (queryCount < 0) throw std::invalid_argument("queryCount must be non-negative");

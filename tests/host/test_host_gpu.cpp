@@ -411,37 +411,46 @@ int main() {
                 ref8[(size_t)r * d + i] = (float)ya;
             }
         }
-        SharedExpertInt8 shared8(ctx);
-        bool threwDims = false, threwScratch = false, threwUnloaded = false;
-        try { shared8.encode(stream, dx, dH2, nullptr, 0); } catch (const std::logic_error &) { threwUnloaded = true; }
+        ffmoe_shape dense8Shape{(uint32_t)d, (uint32_t)f, 1, 1, 2, 64};
+        Context dense8(0, dense8Shape);
+        PrefillSharedExpert shared8(dense8, 8);
+        EXPECT(shared8.weightBits() == 8);
+        bool threwDims = false, threwUnloaded = false, threwRouted = false;
+        try { shared8.encode(stream, 1, dx, dH2); } catch (const FieldfareError &e) { threwUnloaded = e.code == FFMOE_ERR_NO_LAYER; }
         EXPECT(threwUnloaded);
-        try { shared8.load(gate, up, up); } catch (const SharedExpertError &e) { threwDims = e.kind == SharedExpertError::dimensionMismatch; }
+        try { shared8.load(1, gate, up, up); } catch (const SharedExpertError &e) { threwDims = e.kind == SharedExpertError::dimensionMismatch; }
         EXPECT(threwDims);
-        shared8.load(gate, up, down);
-        EXPECT(shared8.d() == (uint32_t)d && shared8.intermediate() == (uint32_t)f);
-        const size_t scratchValues = (size_t)16 * f;
-        uint16_t *dScratch = nullptr;
-        HIP(hipMalloc(&dScratch, scratchValues * 2));
-        try { shared8.encodeBlock(stream, dx, dH2b, T, d, d, dScratch, scratchValues - 1); }
-        catch (const SharedExpertError &e) { threwScratch = e.kind == SharedExpertError::scratchTooSmall; }
-        EXPECT(threwScratch);
-        shared8.encode(stream, dx, dH2, dScratch, scratchValues);
-        shared8.encodeBlock(stream, dx, dH2b, T, d, d, dScratch, scratchValues);
+        try { SharedExpertInt8 onRouted(ctx); } catch (const std::invalid_argument &) { threwRouted = true; }
+        EXPECT(threwRouted);
+        shared8.load(1, gate, up, down);
+        shared8.encode(stream, 1, dx, dH2);
+        shared8.encodeBlock(stream, 1, dx, dH2b, T, d, f, d, d);
         HIP(hipStreamSynchronize(stream));
         double rel8 = 0, cos8 = 0;
-        errorStats(toHost(dH2, (size_t)d), std::vector<float>(ref8.begin(), ref8.begin() + d), rel8, cos8);
-        EXPECT(rel8 <= 1e-2 && cos8 >= 0.9999);
-        errorStats(toHost(dH2b, (size_t)T * d), ref8, rel8, cos8);
-        EXPECT(rel8 <= 1e-2 && cos8 >= 0.9999);
-        // the runtime that picks by weight width, on the same weights: the same row, bit for bit
         const std::vector<uint16_t> row0 = toHost(dH2, (size_t)d);
-        SharedExpertRuntime runtime8(ctx, 8);
-        EXPECT(runtime8.weightBits() == 8);
-        runtime8.load(0, gate, up, down);
-        runtime8.encode(stream, 0, dx, dH2, dScratch, scratchValues);
+        errorStats(row0, std::vector<float>(ref8.begin(), ref8.begin() + d), rel8, cos8);
+        EXPECT(rel8 <= 1e-2 && cos8 >= 0.9999);
+        const std::vector<uint16_t> block = toHost(dH2b, (size_t)T * d);
+        errorStats(block, ref8, rel8, cos8);
+        EXPECT(rel8 <= 1e-2 && cos8 >= 0.9999);
+        EXPECT(std::equal(row0.begin(), row0.end(), block.begin()));       // row 0 of the block is the single-row call's
+        // DequantInt8GEMV on the down projection: rows of the activation scratch are not exposed, so feed it x's first f values
+        DequantInt8GEMV down8(ctx, d8.w.data(), d8.s.data(), d8.b.data(), (uint32_t)d, (uint32_t)f);
+        EXPECT(down8.m() == (uint32_t)d && down8.n() == (uint32_t)f);
+        down8.encodeRows(stream, dx, dH2b, 3, (uint32_t)d, (uint32_t)d);
         HIP(hipStreamSynchronize(stream));
-        EXPECT(toHost(dH2, (size_t)d) == row0);
-        HIP(hipFree(dScratch));
+        std::vector<float> refDown((size_t)3 * d);
+        for (int r = 0; r < 3; ++r)
+            for (int i = 0; i < d; ++i) {
+                double acc = 0;
+                for (int j2 = 0; j2 < f; ++j2) acc += (double)d8.deq[(size_t)i * f + j2] * ffo_bf16_to_float(x[(size_t)r * d + j2]);
+                refDown[(size_t)r * d + i] = (float)acc;
+            }
+        errorStats(toHost(dH2b, (size_t)3 * d), refDown, rel8, cos8);
+        EXPECT(rel8 <= 1e-2 && cos8 >= 0.9999);
+        bool threwRows8 = false;
+        try { down8.encodeRows(stream, dx, dH2b, 17, (uint32_t)d, (uint32_t)d); } catch (const std::invalid_argument &) { threwRows8 = true; }
+        EXPECT(threwRows8);
     }
 
     // --- post-attention setup and layer tail through the mirrored classes: a 5-row block against the oracle's
