@@ -340,20 +340,22 @@ def test_prefill_router_fp16_fast_form_equals_pinned_form(oracle, ff, torch):
     ctx.close()
 
 
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("d,f,e,fs,t", [(128, 64, 16, 1472, 5), (2816, 704, 128, 2112, 16), (2816, 704, 128, 2112, 1)])
-def test_shared_expert_inside_the_routed_launches_fp16(oracle, ff, torch, d, f, e, fs, t):
+def test_shared_expert_inside_the_routed_launches_fp16(oracle, ff, torch, d, f, e, fs, t, bits):
     """FP16 rows through ffmoe_route_verify_shared + ffmoe_layer_tail_routed_shared against the separate FP16 calls
     (ffmoe_route_verify, ffmoe_dense_ffn, ffmoe_layer_tail): the same routes bit for bit, the new hidden rows to the
-    rounding of the shared expert's row (its K is summed in chunks)."""
+    rounding of the shared expert's row (its K is summed in chunks). The shared expert 4-bit and 8-bit."""
     _, pool, router = make_layer(oracle, 5, d, f, e, align=16)
     ctx = ff.Context(d, f, e, 8, n_layers=1, max_tokens=16, act_dtype="fp16")
     ctx.upload_layer(0, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
     ctx.upload_router_bf16(0, router)
     g = np.random.default_rng(d + fs + t)
     scale = 0.4 if d < 1024 else 0.08
-    parts = tuple(oracle.quantize_int4(g.uniform(-scale, scale, (r, c)).astype(np.float32)) for r, c in ((fs, d), (fs, d), (d, fs)))
+    quantize = oracle.quantize_int4 if bits == 4 else oracle.quantize_int8
+    parts = tuple(quantize(g.uniform(-scale, scale, (r, c)).astype(np.float32)) for r, c in ((fs, d), (fs, d), (d, fs)))
     shared = ff.Context(d, fs, 1, 1, n_layers=1, max_tokens=16, act_dtype="fp16")
-    shared.upload_expert_parts(0, 0, *parts)
+    shared.upload_expert_parts(0, 0, *parts, int8=bits == 8)
     x, rx, sx = (f16_tensor(torch, f16_bits(g.uniform(-1.0, 1.0, (t, d)))) for _ in range(3))
     hid = f16_bits(g.uniform(-1.0, 1.0, (t, d)))
     tw2, tw1 = (bf16_tensor(torch, oracle.bf16_bits(g.uniform(0.5, 1.5, d).astype(np.float32))) for _ in range(2))
