@@ -10,7 +10,8 @@ from helpers import bf16_tensor, bits_of, make_layer, to_ff_offsets
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("one_call", [False, True, "shared_inside"], ids=["router_then_verify", "route_verify", "shared_expert_inside"])
+@pytest.mark.parametrize("one_call", [False, True, "shared_inside", "shared8_inside"],
+                         ids=["router_then_verify", "route_verify", "shared_expert_inside", "shared_expert_int8_inside"])
 def test_router_verify_and_dense_chain_in_a_graph(oracle, one_call):
     """`route_verify`: the router, the select and gate/up share one launch whose blocks hand the logits and routes
     to each other through words stamped with an epoch that lives in device memory and is advanced by the call's
@@ -27,6 +28,12 @@ def test_router_verify_and_dense_chain_in_a_graph(oracle, one_call):
         _, pool, router = make_layer(oracle, 40 + layer, d, f, e)
         ctx.upload_layer(layer, pool.bytes, pool.stride, to_ff_offsets(ff, pool.offsets))
         ctx.upload_router_bf16(layer, router)
+        if one_call == "shared8_inside":
+            # the shared expert held 8-bit: the same calls serve it
+            parts8 = tuple(oracle.quantize_int8(rng.uniform(-0.2, 0.2, (r, c)).astype(np.float32))
+                           for r, c in ((2 * f, d), (2 * f, d), (d, 2 * f)))
+            dense.upload_expert_parts(layer, 0, *parts8, int8=True)
+            continue
         _, dpool, _ = make_layer(oracle, 70 + layer, d, 2 * f, 1)
         dense.upload_layer(layer, dpool.bytes, dpool.stride, to_ff_offsets(ff, dpool.offsets))
     x = bf16_tensor(torch, oracle.bf16_bits(rng.normal(0, 1, (t, d)).astype(np.float32)))
@@ -43,7 +50,7 @@ def test_router_verify_and_dense_chain_in_a_graph(oracle, one_call):
         # one decoder-layer MoE block per layer: setup -> (shared expert, router -> routed experts) -> tail
         for layer in range(layers):
             ctx.post_attn_setup(hidden, x, ws[0], ws[1], ws[2], out=outs)
-            if one_call == "shared_inside":
+            if one_call in ("shared_inside", "shared8_inside"):
                 # the shared expert inside the routed experts' launches, both combined in the tail: the call's last launch
                 # (the down projection) moves the epoch on
                 i_, w_ = ctx.route_verify_shared(dense, layer, layer, outs[2], outs[1], outs[0])
