@@ -187,6 +187,13 @@ int check_layer(ffmoe_ctx *ctx, uint32_t layer, bool need_experts, bool need_rou
     return FFMOE_OK;
 }
 
+// A layer that was uploaded 8-bit and is now uploaded 4-bit loses its 8-bit matrices.
+void drop_int8_form(ffmoe_layer &l) {
+    ffmoe_matrix_destroy(l.gate_up8);
+    ffmoe_matrix_destroy(l.down8);
+    l.gate_up8 = l.down8 = nullptr;
+}
+
 template <typename T>
 int upload_vec(T **dst, const T *src, size_t count, char **err) {
     if (*dst) { (void)hipFree(*dst); *dst = nullptr; }
@@ -375,6 +382,7 @@ int ffmoe_upload_layer(ffmoe_ctx *ctx, uint32_t layer, const void *blobs, size_t
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (staging) (void)hipFree(staging);
     if (e != hipSuccess) return fail(err, FFMOE_ERR_RUNTIME, "re-tiling layer %u failed: %s", layer, hipGetErrorString(e));
+    drop_int8_form(ctx->layers[layer]);
     ctx->layers[layer].experts_loaded = true;
     return FFMOE_OK;
 }
@@ -433,6 +441,7 @@ int ffmoe_upload_expert_parts(ffmoe_ctx *ctx, uint32_t layer, uint32_t expert, c
     if (e != hipSuccess)
         return fail(err, FFMOE_ERR_RUNTIME, "upload of expert %u of layer %u failed: %s", expert, layer, hipGetErrorString(e));
     ffmoe_layer &l = ctx->layers[layer];
+    drop_int8_form(l);      // the layer is 4-bit from here on
     if (l.part_loaded.size() != sh.n_experts) l.part_loaded.assign(sh.n_experts, false);
     l.part_loaded[expert] = true;
     bool all = true;

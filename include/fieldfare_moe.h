@@ -474,8 +474,8 @@ int ffmoe_layer_tail_routed(ffmoe_ctx *ctx, void *stream, const uint16_t *route_
  * a gated gate/up matrix and a down matrix of nibble planes (ffmoe_matrix_create_int8_glu / _int8) owned by the
  * context, and ffmoe_dense_ffn, ffmoe_route_verify_shared and ffmoe_layer_tail_routed_shared serve it like a 4-bit
  * layer: ffmoe_dense_ffn runs the two GEMV passes per 16 rows (gate and up are rounded to 16 bits in front of the
- * activation, as the reference's fused kernel does, dequant_int8.metal:131-136). An upload in either width replaces
- * the layer's 8-bit form or leaves it in place: the 8-bit form, once uploaded, is the one that is served. Blocking. */
+ * activation, as the reference's fused kernel does, dequant_int8.metal:131-136). A layer is served in the width of
+ * its latest upload: a later ffmoe_upload_layer / ffmoe_upload_expert_parts of the layer drops the 8-bit form. Blocking. */
 int ffmoe_upload_expert_parts_int8(ffmoe_ctx *ctx, uint32_t layer, const ffmoe_projection *gate,
                                    const ffmoe_projection *up, const ffmoe_projection *down, char **err);
 

@@ -292,6 +292,12 @@ def test_dense_ffn_on_an_int8_layer(ff, oracle, torch, d, fs, t):
         assert rel_err(got, ref) < 1e-2 and cosine(got, ref) > 0.9999, (rel_err(got, ref), cosine(got, ref))
     with pytest.raises(ff.FieldfareError, match="outside"):
         dense.dense_ffn(1, torch.zeros((max(t, 16) + 1, d), dtype=torch.bfloat16, device="cuda"))
+    # the layer is served in the width of its latest upload
+    parts4 = tuple(oracle.quantize_int4(np.zeros((r, c), np.float32)) for r, c in ((fs, d), (fs, d), (d, fs)))
+    dense.upload_expert_parts(1, 0, *parts4)
+    assert float(dense.dense_ffn(1, xt).abs().max()) == 0.0
+    dense.upload_expert_parts(1, 0, *parts, int8=True)
+    assert torch.equal(dense.dense_ffn(1, xt).view(torch.int16), want.view(torch.int16))
     routed = ff.Context(128, 64, 4, 2, n_layers=1, max_tokens=16)
     with pytest.raises(ff.FieldfareError, match="n_experts = 1"):
         routed.upload_expert_parts(0, 0, *_int8_parts(oracle, g, 128, 64, 0.4), int8=True)
