@@ -775,7 +775,7 @@ int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t
     if (reinterpret_cast<uintptr_t>(y) % 16) return fail(err, FFMOE_ERR_INVALID, "y must be 16-byte aligned");
     if (int rc = check_layer(ctx, layer, false, false, err)) return rc;
     if (ctx->layers[layer].gate_up8) {
-        // an 8-bit layer: the gated gate/up pass into the activation scratch, then the down pass, 16 rows at a time
+        // an 8-bit layer: the gated gate/up pass into the activation scratch, then the down pass
         const ffmoe_layer &l = ctx->layers[layer];
         const uint32_t cap = std::max<uint32_t>(ctx->shape.max_tokens, FFMOE_MAX_VERIFY_ROWS);
         if (!x || t == 0 || t > cap) return fail(err, FFMOE_ERR_INVALID, "rows = %u outside 1...%u", t, cap);
@@ -783,16 +783,16 @@ int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t
             return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
         hipStream_t s = static_cast<hipStream_t>(stream);
         claim_scratch(ctx, stream);
+        // two launches whatever the row count: a grid row per 16 input rows, each a pass of its own over the weights
+        // (from the caches after the first); the activation rows of a block of more than 16 go to the prefill scratch
+        uint16_t *acts = t <= FFMOE_MAX_VERIFY_ROWS ? ctx->acts : ctx->pf.acts;
         ctx->timer.begin(s);
-        for (uint32_t r0 = 0; r0 < t; r0 += FFMOE_MAX_VERIFY_ROWS) {
-            const uint32_t rows = std::min<uint32_t>(FFMOE_MAX_VERIFY_ROWS, t - r0);
-            FF_HIP(launch_matrix_gemv(s, l.gate_up8->tiles, l.gate_up8->scales, ctx->shape.f, ctx->shape.d, x + (size_t)r0 * x_stride,
-                                      x_stride, rows, ctx->acts, ctx->shape.f, false, ctx->n_cus, ctx->f16, true, true));
-            ctx->timer.mark(s, FFMOE_K_GATE_UP);
-            FF_HIP(launch_matrix_gemv(s, l.down8->tiles, l.down8->scales, ctx->shape.d, ctx->shape.f, ctx->acts, ctx->shape.f, rows,
-                                      y + (size_t)r0 * ctx->shape.d, ctx->shape.d, false, ctx->n_cus, ctx->f16, true, false));
-            ctx->timer.mark(s, FFMOE_K_DOWN);
-        }
+        FF_HIP(launch_matrix_gemv(s, l.gate_up8->tiles, l.gate_up8->scales, ctx->shape.f, ctx->shape.d, x, x_stride, t, acts,
+                                  ctx->shape.f, false, ctx->n_cus, ctx->f16, true, true));
+        ctx->timer.mark(s, FFMOE_K_GATE_UP);
+        FF_HIP(launch_matrix_gemv(s, l.down8->tiles, l.down8->scales, ctx->shape.d, ctx->shape.f, acts, ctx->shape.f, t, y,
+                                  ctx->shape.d, false, ctx->n_cus, ctx->f16, true, false));
+        ctx->timer.mark(s, FFMOE_K_DOWN);
         ctx->timer.finish();
         return FFMOE_OK;
     }

@@ -198,6 +198,14 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
     const uint32_t g_last = g1 > g0 ? g1 - 1 : n_groups - 1;
     const TileSource src = make_tile_source(tiles, (size_t)n_tiles * n_groups * kTileBytes, scales,
                                             (size_t)n_tiles * n_groups * kTileScaleBytes);
+    // more than 16 input rows (the plain forms only): grid row y takes rows 16 y ... 16 y + 15 - the same pass over the
+    // weights again, which then come from the caches
+    if (!GREEDY && blockIdx.y != 0) {
+        x += (size_t)blockIdx.y * FFMOE_MAX_VERIFY_ROWS * x_stride;
+        y_ = Y_F32 ? static_cast<void *>(reinterpret_cast<float *>(y_) + (size_t)blockIdx.y * FFMOE_MAX_VERIFY_ROWS * y_stride)
+                   : static_cast<void *>(reinterpret_cast<uint16_t *>(y_) + (size_t)blockIdx.y * FFMOE_MAX_VERIFY_ROWS * y_stride);
+    }
+    if (!GREEDY) rows = min((uint32_t)FFMOE_MAX_VERIFY_ROWS, rows - blockIdx.y * FFMOE_MAX_VERIFY_ROWS);
 
     WeightRing ring;
 #pragma unroll
@@ -403,7 +411,8 @@ hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t
                               const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
                               bool y_f32, uint32_t n_cus, bool f16, bool planes8, bool glu) {
     const uint32_t n_tiles = planes8 ? (m + 15) / 16 : (m + 31) / 32;      // gated: pairs of tiles
-    const dim3 grid(min(2 * n_cus, n_tiles));
+    if (rows == 0 || (rows + FFMOE_MAX_VERIFY_ROWS - 1) / FFMOE_MAX_VERIFY_ROWS > 65535u) return hipErrorInvalidValue;
+    const dim3 grid(min(2 * n_cus, n_tiles), (rows + FFMOE_MAX_VERIFY_ROWS - 1) / FFMOE_MAX_VERIFY_ROWS);
 #define FFMOE_MGEMV(Y, H, P, G)                                                                                             \
     hipLaunchKernelGGL((matrix_gemv_kernel<Y, H, false, false, P, G>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, \
                        rows, y, y_stride)

@@ -650,7 +650,7 @@ def main():
         # the same FFN in the 8-bit form the reference's packs hold by default (SharedExpertInt8.swift:56-135): two nibble
         # planes per weight on the 4-bit streaming kernels, as layers of a second dense context; gate and up are one gated
         # matrix (the activation is that pass's epilogue), then the down projection: two launches per call
-        dense8 = ff.Context(D, FS, 1, 1, n_layers=LS, max_tokens=16)
+        dense8 = ff.Context(D, FS, 1, 1, n_layers=LS, max_tokens=max(args.prefill_tokens, 16))
         bytes8 = 0
         for layer in range(LS):
             parts8 = []
@@ -680,6 +680,10 @@ def main():
             fl = 2.0 * 3 * D * FS * TPs
             shared[f"rows{TPs}"] = {"us": round(tp_ * 1e6, 1), "TFLOPs": round(fl / tp_ / 1e12, 1),
                                     "frac_mfma_peak": round(fl / tp_ / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+            # the 8-bit layer has no grouped-GEMM form (a 16-bit matrix tile cannot hold q * s + b of an 8-bit q): the
+            # rows go through the two streaming launches, a grid row and a pass over the (then cached) weights per 16 rows
+            tp8 = timed(lambda: int8_step(xps, yps), 4, warm=2)
+            shared["int8"][f"rows{TPs}"] = {"us": round(tp8 * 1e6, 1), "passes_over_the_weights": (TPs + 15) // 16}
             del xps, yps
         extra["shared_expert"] = shared
 
