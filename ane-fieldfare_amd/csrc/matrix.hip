@@ -412,7 +412,10 @@ hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t
                               bool y_f32, uint32_t n_cus, bool f16, bool planes8, bool glu) {
     const uint32_t n_tiles = planes8 ? (m + 15) / 16 : (m + 31) / 32;      // gated: pairs of tiles
     if (rows == 0 || (rows + FFMOE_MAX_VERIFY_ROWS - 1) / FFMOE_MAX_VERIFY_ROWS > 65535u) return hipErrorInvalidValue;
-    const dim3 grid(min(2 * n_cus, n_tiles), (rows + FFMOE_MAX_VERIFY_ROWS - 1) / FFMOE_MAX_VERIFY_ROWS);
+    dim3 grid(min(2 * n_cus, n_tiles), (rows + FFMOE_MAX_VERIFY_ROWS - 1) / FFMOE_MAX_VERIFY_ROWS);
+    // several grid rows: a multiple of 8 blocks per row keeps a tile on one XCD (blocks go to the XCDs round robin), whose L2
+    // then serves every pass after the first; the blocks past the tile count leave at once
+    if (grid.y > 1) grid.x = (grid.x + 7) / 8 * 8;
 #define FFMOE_MGEMV(Y, H, P, G)                                                                                             \
     hipLaunchKernelGGL((matrix_gemv_kernel<Y, H, false, false, P, G>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, \
                        rows, y, y_stride)
