@@ -1207,6 +1207,23 @@ int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_
     return FFMOE_OK;
 }
 
+int ffmoe_matrix_rows(ffmoe_matrix *mx, void *stream, const uint32_t *ids, uint32_t count, uint32_t token_id, float out_scale,
+                      uint16_t *out, uint32_t out_stride, char **err) {
+    if (!mx) return fail(err, FFMOE_ERR_INVALID, "null matrix");
+    if (!mx->ctx) return fail(err, FFMOE_ERR_INVALID, "the matrix's context was destroyed");
+    if (int rc = check_ctx(mx->ctx, err)) return rc;
+    if (mx->planes8) return fail(err, FFMOE_ERR_INVALID, "rows are looked up in a 4-bit matrix (the reference's embedding table is 4-bit)");
+    if (!out) return fail(err, FFMOE_ERR_INVALID, "null argument");
+    if (count == 0 || count > 65535u) return fail(err, FFMOE_ERR_INVALID, "count = %u outside 1...65535", count);
+    if (!ids && count != 1) return fail(err, FFMOE_ERR_INVALID, "without an id list the call looks up the one row token_id");
+    if (out_stride < mx->n || out_stride % 8 || reinterpret_cast<uintptr_t>(out) % 16)
+        return fail(err, FFMOE_ERR_INVALID, "out must be 16-byte aligned with a row stride that is a multiple of 8 and >= N");
+    if (!std::isfinite(out_scale)) return fail(err, FFMOE_ERR_INVALID, "out_scale must be finite");
+    FF_HIP(launch_matrix_rows(static_cast<hipStream_t>(stream), mx->tiles, mx->scales, mx->m, mx->n, ids, token_id, count, out_scale,
+                              out, out_stride, mx->ctx->f16));
+    return FFMOE_OK;
+}
+
 static int matrix_greedy_common(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
                                 float softcap, uint32_t *out_tokens, float *out_conf, char **err) {
     if (int rc = check_matrix_call(mx, x, x_stride, rows, err)) return rc;

@@ -455,6 +455,50 @@ hipError_t launch_gelu_mul(hipStream_t s, const uint16_t *gate, uint32_t gate_st
     return hipGetLastError();
 }
 
+// Rows of the resident 4-bit matrix dequantised: out[i][k] = round16((q s + b) * out_scale) for weight row ids[i] (or
+// the one row `token_id` when ids is null) - embed_lookup_int4 (Metal/Quant/dequant_int4.metal:53-73) on the re-tiled
+// copy, so that tied embeddings need no second table. One thread per 8 consecutive elements: one 32-bit word of a tile
+// (lane 16 (k / 8 % 4) + row % 16, word 2 (row / 16 % 2) + (k / 32 % 2)) and the row's scale pair. An id past the
+// table gives a row of zeros.
+template <bool F16>
+__global__ __launch_bounds__(256) void matrix_rows_kernel(const uint8_t *__restrict__ tiles, const uint8_t *__restrict__ scales,
+                                                          uint32_t m, uint32_t n_groups, const uint32_t *__restrict__ ids,
+                                                          uint32_t token_id, float out_scale, uint16_t *__restrict__ out,
+                                                          uint32_t out_stride) {
+    const uint32_t r = ids ? ids[blockIdx.y] : token_id;
+    for (uint32_t w = blockIdx.x * 256 + threadIdx.x; w < n_groups * 8; w += gridDim.x * 256) {
+        const uint32_t grp = w >> 3, piece = w & 7;
+        uint32_t packed[4] = {0, 0, 0, 0};
+        if (r < m) {
+            const size_t tile = (size_t)(r >> 5) * n_groups + grp;
+            const uint32_t i = r & 15, half = (r >> 4) & 1, jq = piece & 3, hi = piece >> 2;
+            const uint32_t word = reinterpret_cast<const uint32_t *>(tiles + tile * kTileBytes)[(jq * 16 + i) * 4 + half * 2 + hi];
+            const uint32_t sb = reinterpret_cast<const uint32_t *>(scales + tile * kTileScaleBytes)[i * 2 + half];
+            const float sc = bf16_to_f32((uint16_t)(sb & 0xFFFFu)), bi = bf16_to_f32((uint16_t)(sb >> 16));
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int pos = (t & 1) ? 4 + (t >> 1) : (t >> 1);          // arena order: position p = element 2p, p + 4 = element 2p + 1
+                const float q = (float)((word >> (4 * pos)) & 0xFu);
+                const float v = (q * sc + bi) * out_scale;                  // q * sc is exact in fp32: the reference's expression
+                packed[t >> 1] |= (uint32_t)Act<F16>::round(v) << (16 * (t & 1));
+            }
+        }
+        *reinterpret_cast<uint4 *>(out + (size_t)blockIdx.y * out_stride + grp * kGroup + 8 * piece) =
+            uint4{packed[0], packed[1], packed[2], packed[3]};
+    }
+}
+
+hipError_t launch_matrix_rows(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n, const uint32_t *ids,
+                              uint32_t token_id, uint32_t count, float out_scale, uint16_t *out, uint32_t out_stride, bool f16) {
+    if (count == 0 || count > 65535u) return hipErrorInvalidValue;
+    const dim3 grid(min(64u, (n / 8 + 255) / 256), count);
+    if (f16)
+        hipLaunchKernelGGL(matrix_rows_kernel<true>, grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, ids, token_id, out_scale, out, out_stride);
+    else
+        hipLaunchKernelGGL(matrix_rows_kernel<false>, grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, ids, token_id, out_scale, out, out_stride);
+    return hipGetLastError();
+}
+
 // keys per input row that launch_matrix_greedy leaves between its two kernels
 uint32_t greedy_segments(uint32_t m, uint32_t n_cus) { return min(2 * n_cus, (m + 31) / 32); }
 

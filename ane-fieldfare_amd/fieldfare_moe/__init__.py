@@ -50,7 +50,7 @@ EXPORTS = [
     "ffmoe_layer_tail", "ffmoe_layer_tail_routed", "ffmoe_route_verify", "ffmoe_set_handover_timeout", "ffmoe_set_one_launch_routing", "ffmoe_gemv_int4_listed",
     "ffmoe_layer_tail_norms", "ffmoe_rmsnorm", "ffmoe_set_activation_dtype", "ffmoe_prefill_dump_tiles",
     "ffmoe_verify_static", "ffmoe_route_verify_shared", "ffmoe_layer_tail_routed_shared", "ffmoe_sample_rows",
-    "ffmoe_matrix_create_int8", "ffmoe_matrix_create_int8_glu", "ffmoe_gelu_mul", "ffmoe_upload_expert_parts_int8",
+    "ffmoe_matrix_create_int8", "ffmoe_matrix_create_int8_glu", "ffmoe_gelu_mul", "ffmoe_upload_expert_parts_int8", "ffmoe_matrix_rows",
 ]
 
 PROFILE_SLOTS = 16
@@ -113,6 +113,17 @@ class Matrix:
         err = C.c_char_p()
         _check(self.L.ffmoe_matrix_gemv(self._h, _stream(), _ptr(x), _row_stride(x), rows, _ptr(y), _row_stride(y),
                                         int(f32_out), C.byref(err)), err)
+        return y
+
+    def rows(self, ids, out_scale: float = 1.0, out=None):
+        """Dequantised rows `ids` (an int or an int32 / uint32 CUDA tensor) times out_scale: [count, N] of the activation type."""
+        import torch
+        single = isinstance(ids, int)
+        count = 1 if single else int(ids.shape[0])
+        y = torch.empty((count, self.n), dtype=self.ctx.act, device="cuda") if out is None else out
+        err = C.c_char_p()
+        _check(self.L.ffmoe_matrix_rows(self._h, _stream(), None if single else _ptr(ids), count, ids if single else 0,
+                                        out_scale, _ptr(y), _row_stride(y), C.byref(err)), err)
         return y
 
     def greedy(self, x):
@@ -239,6 +250,7 @@ def lib() -> C.CDLL:
     L.ffmoe_prefill_plan_stats.argtypes = [vp, vp, C.POINTER(u32), C.POINTER(u32), vp, errp]
     L.ffmoe_matrix_create.argtypes = [vp, vp, vp, vp, u32, u32, i32, C.POINTER(vp), errp]
     L.ffmoe_matrix_create_int8.argtypes = [vp, vp, vp, vp, u32, u32, C.POINTER(vp), errp]
+    L.ffmoe_matrix_rows.argtypes = [vp, vp, vp, u32, u32, C.c_float, vp, u32, errp]
     L.ffmoe_matrix_create_int8_glu.argtypes = [vp, vp, vp, vp, vp, vp, vp, u32, u32, C.POINTER(vp), errp]
     L.ffmoe_gelu_mul.argtypes = [vp, vp, vp, u32, vp, u32, vp, u32, u32, u32, errp]
     L.ffmoe_matrix_destroy.argtypes = [vp]

@@ -575,6 +575,19 @@ public:
         check(ffmoe_sample_rows(c.raw(), stream, rowsLogits, logitsStrideElements, (uint32_t)rowCount, count, ids, &rule,
                                 sampling.keyOffset, outIndices, rowsConfidence, &err), err);
     }
+    // EmbedLookupInt4.encode (Kernels/Quant/EmbedLookupInt4.swift:14-44) on the chain's table - the model ties its
+    // embedding to the head, so the resident copy serves both: out[d] = round16((q s + b) * outScale) of row tokenId.
+    void encodeEmbedLookup(void *stream, uint32_t tokenId, float outScale, uint16_t *out) {
+        char *err = nullptr;
+        check(ffmoe_matrix_rows(mx_, stream, nullptr, 1, tokenId, outScale, out, d_, &err), err);
+    }
+    // the same for `count` token ids in device memory (the tokens a greedy call left): rows of outStrideElements values
+    void encodeEmbedLookupRows(void *stream, const uint32_t *tokenIds, int count, float outScale, uint16_t *out,
+                               uint32_t outStrideElements) {
+        if (count <= 0) throw std::invalid_argument("count must be positive");
+        char *err = nullptr;
+        check(ffmoe_matrix_rows(mx_, stream, tokenIds, (uint32_t)count, 0, outScale, out, outStrideElements, &err), err);
+    }
     uint32_t vocab() const { return vocab_; }
 
 private:

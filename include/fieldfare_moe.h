@@ -331,6 +331,16 @@ void ffmoe_matrix_destroy(ffmoe_matrix *mx);
 int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_t x_stride, uint32_t rows,
                       void *y, uint32_t y_stride, int y_f32, char **err);
 
+/* out[i][k] = round16((q s + b) * out_scale) for weight row ids[i] of a 4-bit matrix, i < count (ids: uint32 in device
+ * memory - e.g. the tokens ffmoe_matrix_greedy left - or NULL with count = 1 for the one row token_id): the embedding
+ * lookup of a model whose head and embedding share one table, served from the head's resident copy. Replaces
+ * EmbedLookupInt4.encode (Kernels/Quant/EmbedLookupInt4.swift:14-44, kernel embed_lookup_int4,
+ * Metal/Quant/dequant_int4.metal:53-73; out_scale = sqrt(hidden size) there). Bit for bit the reference's
+ * half((float(q) * s + b) * out_scale) in the context's activation type. An id >= M gives a row of zeros (the
+ * reference reads past its table). out 16-byte aligned, stride a multiple of 8 and >= N. */
+int ffmoe_matrix_rows(ffmoe_matrix *mx, void *stream, const uint32_t *ids, uint32_t count, uint32_t token_id,
+                      float out_scale, uint16_t *out, uint32_t out_stride, char **err);
+
 /* out[r][i] = round16(gelu_tanh(gate[r][i]) * up[r][i]) for `rows` rows of `count` values in the context's activation
  * type: gelu_mul_fp16 (Metal/Primitives/utility.metal:4-17, run by PrefillSharedExpert.encodeBatched,
  * Kernels/Prefill/MoE/PrefillSharedExpert.swift:78-91), and with two ffmoe_matrix_gemv calls in front and one behind

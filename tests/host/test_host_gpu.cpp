@@ -253,6 +253,25 @@ int main() {
         bool threwRows = false;
         try { head.encodeGreedyRows(stream, dx, d, 17, dTok); } catch (const std::invalid_argument &) { threwRows = true; }
         EXPECT(threwRows);
+        // the tied embedding: the rows of the three greedy tokens, and row 5 by value, from the same resident table
+        {
+            uint16_t *dEmb = nullptr;
+            HIP(hipMalloc(reinterpret_cast<void **>(&dEmb), (size_t)4 * d * 2));
+            const float outScale = std::sqrt((float)d);
+            head.encodeEmbedLookupRows(stream, dTok, 3, outScale, dEmb, d);
+            head.encodeEmbedLookup(stream, 5, outScale, dEmb + (size_t)3 * d);
+            HIP(hipStreamSynchronize(stream));
+            auto emb = toHost(dEmb, (size_t)4 * d);
+            std::vector<float> rowF(d);
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t id = r < 3 ? tok[r] : 5u;
+                ffo_dequantize_int4_affine(pool.data() + off.gate_w + (size_t)id * d / 2,
+                                           reinterpret_cast<uint16_t *>(pool.data() + off.gate_s) + (size_t)id * d / 64,
+                                           reinterpret_cast<uint16_t *>(pool.data() + off.gate_b) + (size_t)id * d / 64, d, rowF.data());
+                for (int i = 0; i < d; ++i) EXPECT(emb[(size_t)r * d + i] == ffo_bf16_bits(rowF[i] * outScale));
+            }
+            HIP(hipFree(dEmb));
+        }
         // the same choice with the winner's probability (softmax of the row's logits, no softcap): same tokens, and
         // the probability the fp64 softmax of the CPU logits gives
         float *dConf = nullptr, *dLogits = nullptr;

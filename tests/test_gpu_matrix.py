@@ -493,3 +493,51 @@ def test_final_row_head_matches_scalar_offset_path(ctx, oracle, torch):
     ref = oracle.gemv_int4_ref(W, S, B, oracle.bf16_to_float(ref_normed[0]))
     assert rel_err(a, ref) < 5e-3                                           # Tolerance.fp16Reduction
     head.close()
+
+
+@pytest.mark.parametrize("act", ["fp16", "bf16"])
+def test_embedding_rows_from_the_resident_table(ff, oracle, torch, act):
+    # embedLookupInt4_withSqrtDScale_matchesReference (EmbedLookupTests.swift:24-62): same seed, label, table (16 x 128),
+    # token 9 and scale sqrt(128); FP16 out as there (and bf16). The reference allows Tolerance.quantInt4; the kernel's
+    # expression half((q * s + b) * out_scale) is pinned bit for bit.
+    V, D = 16, 128
+    rng = oracle.seed_tree_key(0x131, "embed-lookup-int4-table")
+    W, S, B = oracle.quantize_int4(np.stack([rng.uniform(-1.0, 1.0, D) for _ in range(V)]))
+    c = ff.Context(128, 64, 16, 8, n_layers=1, max_tokens=16, act_dtype=act)
+    dtype = oracle.FP16 if act == "fp16" else oracle.BF16
+    table = c.matrix(W, S, B)
+    scale = np.float32(np.sqrt(np.float32(D)))
+    deq = oracle.dequantize_int4(W, S, B)
+    want = oracle.bits16(deq * scale, dtype)
+    got = bits_of(table.rows(9, float(scale)))
+    assert got.shape == (1, D) and np.array_equal(got[0], want[9])
+    # a list of ids in device memory: every row, a repeat, and one past the table (a row of zeros)
+    ids = torch.tensor(list(range(V)) + [3, V + 5], dtype=torch.int32, device="cuda")
+    rows = bits_of(table.rows(ids, float(scale)))
+    assert np.array_equal(rows[:V], want) and np.array_equal(rows[V], want[3]) and not rows[V + 1].any()
+    assert np.array_equal(bits_of(table.rows(ids, 1.0))[:V], oracle.bits16(deq, dtype))
+    table.close()
+    # a tall table with an odd row count and the model's width: rows either side of every tile boundary, into a padded output
+    g = np.random.default_rng(11)
+    m, n = 1000 + 7, 2816
+    W, S, B = oracle.quantize_int4(g.uniform(-1.0, 1.0, (m, n)).astype(np.float32))
+    table = c.matrix(W, S, B, greedy=True)
+    pick = np.array([0, 15, 16, 31, 32, 47, 48, 63, 64, 500, 991, 992, 1005, 1006], np.int32)
+    out = torch.full((len(pick), n + 8), -3.0, dtype=c.act, device="cuda")
+    table.rows(torch.from_numpy(pick).cuda(), 53.0, out=out)
+    want = oracle.bits16(oracle.dequantize_int4(W[pick], S[pick], B[pick]) * np.float32(53.0), dtype)
+    got = bits_of(out)
+    assert np.array_equal(got[:, :n], want) and (out[:, n:].float() == -3.0).all()
+    # the tokens of a greedy choice feed the lookup without leaving the device
+    x = torch.from_numpy(g.uniform(-1, 1, (4, n)).astype(np.float32)).cuda().to(c.act)
+    tok = table.greedy(x)
+    emb = bits_of(table.rows(tok, 1.0))
+    t_host = tok.cpu().numpy()
+    assert np.array_equal(emb, oracle.bits16(oracle.dequantize_int4(W[t_host], S[t_host], B[t_host]), dtype))
+    with pytest.raises(ff.FieldfareError, match="4-bit"):
+        m8 = c.matrix_int8(*oracle.quantize_int8(g.uniform(-1, 1, (16, 64)).astype(np.float32)))
+        m8.rows(0)
+    with pytest.raises(ff.FieldfareError, match="aligned"):
+        table.rows(0, out=torch.empty((1, n + 8), dtype=c.act, device="cuda")[:, 1:n + 1])
+    table.close()
+    c.close()
