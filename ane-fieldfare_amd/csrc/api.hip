@@ -2,6 +2,7 @@
 // argument validation and stream-ordered launches. No call here touches a CPU implementation of the
 // math: without a working HIP device every entry point fails with FFMOE_ERR_RUNTIME.
 #include <hip/hip_runtime.h>
+#include <rocblas/rocblas.h>
 
 #include <cstdarg>
 #include <cstdio>
@@ -27,7 +28,15 @@ struct ffmoe_layer {
     float router_norm_max = 0.0f;   // upper bound of the largest 2-norm of an expert's router row
     // a dense context's layer held 8-bit (ffmoe_upload_expert_parts_int8): the gated gate/up matrix and the down matrix
     struct ffmoe_matrix *gate_up8 = nullptr, *down8 = nullptr;
+    // the same weights as hi + lo rows of the activation type for the library GEMM that serves large row counts
+    // ([4 f][d] and [2 d][f]); null when the context's max_tokens stays below the row count from which it is used
+    uint16_t *gate_up8_hilo = nullptr, *down8_hilo = nullptr;
 };
+
+// From this many rows on an 8-bit dense layer goes through the library's dense GEMM on hi / lo rows instead of one
+// streaming pass per 16 rows (measured at 2816 -> 2112 -> 2816: streaming 19 us at 32 rows + 8.8 us per 32 more, 42 us at
+// 127; the GEMM form 50 us at 128, 58 at 192, 67 at 256, 100 at 1,024, 244 at 3,072).
+constexpr uint32_t kGemm8MinRows = 192;
 
 // A resident matrix: the re-tiled copy of one [m][n] INT4 weight plus the scratch of its greedy choice.
 struct ffmoe_matrix {
@@ -63,6 +72,9 @@ struct ffmoe_ctx {
     uint32_t *dense_idx = nullptr;   // [max(max_tokens,16)] zeros
     uint16_t *dense_w = nullptr;     // [max(max_tokens,16)] 1.0 in the activation type
     bool f16 = false;                // activations are FP16 (ffmoe_set_activation_dtype)
+    // the 8-bit dense layers' GEMM form: the library handle and the fp32 sums [max_tokens][max(4 f, 2 d)]
+    rocblas_handle blas = nullptr;
+    float *gemm8_sums = nullptr;
     KernelTimer timer;
     std::vector<ffmoe_matrix *> matrices;   // resident matrices created on this context and not yet destroyed
     // the stream the scratch was last used on, and the event a call on another stream waits for (claim_scratch)
@@ -192,6 +204,20 @@ void drop_int8_form(ffmoe_layer &l) {
     ffmoe_matrix_destroy(l.gate_up8);
     ffmoe_matrix_destroy(l.down8);
     l.gate_up8 = l.down8 = nullptr;
+    if (l.gate_up8_hilo) (void)hipFree(l.gate_up8_hilo);
+    if (l.down8_hilo) (void)hipFree(l.down8_hilo);
+    l.gate_up8_hilo = l.down8_hilo = nullptr;
+}
+
+// (Re)makes the hi / lo rows of an 8-bit layer in the context's activation type from its nibble planes. Blocking.
+hipError_t expand_int8_layer(ffmoe_ctx *ctx, ffmoe_layer &l) {
+    if (!l.gate_up8_hilo) return hipSuccess;
+    hipError_t e = launch_expand_planes8(nullptr, l.gate_up8->tiles, l.gate_up8->scales, ctx->shape.f, ctx->shape.d, true,
+                                         l.gate_up8_hilo, ctx->f16);
+    if (e == hipSuccess)
+        e = launch_expand_planes8(nullptr, l.down8->tiles, l.down8->scales, ctx->shape.d, ctx->shape.f, false, l.down8_hilo, ctx->f16);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    return e;
 }
 
 template <typename T>
@@ -304,11 +330,11 @@ void ffmoe_destroy(ffmoe_ctx *ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
     (void)hipDeviceSynchronize();
+    if (ctx->blas) (void)rocblas_destroy_handle(ctx->blas);
+    if (ctx->gemm8_sums) (void)hipFree(ctx->gemm8_sums);
     for (auto &l : ctx->layers) {
         // the layer's own 8-bit matrices: nobody else holds their handles
-        ffmoe_matrix_destroy(l.gate_up8);
-        ffmoe_matrix_destroy(l.down8);
-        l.gate_up8 = l.down8 = nullptr;
+        drop_int8_form(l);
         if (l.router_w) (void)hipFree(l.router_w);
         if (l.router_frag) (void)hipFree(l.router_frag);
         if (l.effective_scale) (void)hipFree(l.effective_scale);
@@ -783,6 +809,33 @@ int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t
             return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
         hipStream_t s = static_cast<hipStream_t>(stream);
         claim_scratch(ctx, stream);
+        if (t >= kGemm8MinRows && l.gate_up8_hilo) {
+            // many rows: two dense GEMMs of the library on the hi / lo rows (fp32 sums), each followed by the pass that adds
+            // a weight row's two columns and rounds as the streaming form does
+            const uint32_t f = ctx->shape.f, d = ctx->shape.d;
+            const rocblas_datatype dt = ctx->f16 ? rocblas_datatype_f16_r : rocblas_datatype_bf16_r;
+            const float one = 1.0f, zero = 0.0f;
+            auto gemm = [&](const uint16_t *w, uint32_t n_out, uint32_t k, const uint16_t *in, uint32_t in_stride) {
+                // row-major sums[t][n_out] = in[t][k] . w[n_out][k]^T, i.e. column-major w^T in
+                return rocblas_gemm_ex(ctx->blas, rocblas_operation_transpose, rocblas_operation_none, (rocblas_int)n_out, (rocblas_int)t,
+                                       (rocblas_int)k, &one, w, dt, (rocblas_int)k, in, dt, (rocblas_int)in_stride, &zero,
+                                       ctx->gemm8_sums, rocblas_datatype_f32_r, (rocblas_int)n_out, ctx->gemm8_sums,
+                                       rocblas_datatype_f32_r, (rocblas_int)n_out, rocblas_datatype_f32_r, rocblas_gemm_algo_standard,
+                                       0, 0);
+            };
+            if (rocblas_set_stream(ctx->blas, s) != rocblas_status_success) return fail(err, FFMOE_ERR_RUNTIME, "rocblas_set_stream failed");
+            ctx->timer.begin(s);
+            rocblas_status st = gemm(l.gate_up8_hilo, 4 * f, d, x, x_stride);
+            if (st != rocblas_status_success) return fail(err, FFMOE_ERR_RUNTIME, "rocblas_gemm_ex (gate/up): status %d", (int)st);
+            FF_HIP(launch_hilo_epilogue(s, ctx->gemm8_sums, t, f, true, ctx->pf.acts, f, ctx->f16));
+            ctx->timer.mark(s, FFMOE_K_GATE_UP);
+            st = gemm(l.down8_hilo, 2 * d, f, ctx->pf.acts, f);
+            if (st != rocblas_status_success) return fail(err, FFMOE_ERR_RUNTIME, "rocblas_gemm_ex (down): status %d", (int)st);
+            FF_HIP(launch_hilo_epilogue(s, ctx->gemm8_sums, t, d, false, y, d, ctx->f16));
+            ctx->timer.mark(s, FFMOE_K_DOWN);
+            ctx->timer.finish();
+            return FFMOE_OK;
+        }
         // two launches whatever the row count: a grid row per 16 input rows, each a pass of its own over the weights
         // (from the caches after the first); the activation rows of a block of more than 16 go to the prefill scratch
         uint16_t *acts = t <= FFMOE_MAX_VERIFY_ROWS ? ctx->acts : ctx->pf.acts;
@@ -926,7 +979,10 @@ int ffmoe_set_activation_dtype(ffmoe_ctx *ctx, int dtype, char **err) {
         FF_HIP(hipDeviceSynchronize());
         FF_HIP(hipMemsetD16(reinterpret_cast<hipDeviceptr_t>(ctx->dense_w), f16 ? 0x3C00 : 0x3F80, cap));
     }
+    const bool changed = ctx->f16 != f16;
     ctx->f16 = f16;
+    if (changed)
+        for (auto &l : ctx->layers) FF_HIP(expand_int8_layer(ctx, l));      // the GEMM form's rows are of the activation type
     return FFMOE_OK;
 }
 
@@ -1145,10 +1201,29 @@ int ffmoe_upload_expert_parts_int8(ffmoe_ctx *ctx, uint32_t layer, const ffmoe_p
         return rc;
     }
     ffmoe_layer &l = ctx->layers[layer];
-    ffmoe_matrix_destroy(l.gate_up8);
-    ffmoe_matrix_destroy(l.down8);
+    drop_int8_form(l);
     l.gate_up8 = gu;
     l.down8 = dn;
+    if (sh.max_tokens >= kGemm8MinRows) {
+        // large row counts go through the library's dense GEMM on hi / lo rows of the activation type
+        if (!ctx->blas && rocblas_create_handle(&ctx->blas) != rocblas_status_success) {
+            ctx->blas = nullptr;
+            drop_int8_form(l);
+            return fail(err, FFMOE_ERR_RUNTIME, "rocblas_create_handle failed");
+        }
+        hipError_t e = hipSuccess;
+        if (!ctx->gemm8_sums)
+            e = hipMalloc(reinterpret_cast<void **>(&ctx->gemm8_sums),
+                          (size_t)sh.max_tokens * std::max(4 * (size_t)sh.f, 2 * (size_t)sh.d) * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&l.gate_up8_hilo), (size_t)4 * sh.f * sh.d * sizeof(uint16_t));
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&l.down8_hilo), (size_t)2 * sh.d * sh.f * sizeof(uint16_t));
+        if (e == hipSuccess) e = expand_int8_layer(ctx, l);
+        if (e != hipSuccess) {
+            drop_int8_form(l);
+            return fail(err, e == hipErrorOutOfMemory ? FFMOE_ERR_ALLOC : FFMOE_ERR_RUNTIME, "the GEMM form of the 8-bit layer: %s",
+                        hipGetErrorString(e));
+        }
+    }
     return FFMOE_OK;
 }
 

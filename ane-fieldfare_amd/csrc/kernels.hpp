@@ -198,6 +198,10 @@ hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t
                               bool y_f32, uint32_t n_cus, bool f16 = false, bool planes8 = false, bool glu = false);
 hipError_t launch_matrix_rows(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n, const uint32_t *ids,
                               uint32_t token_id, uint32_t count, float out_scale, uint16_t *out, uint32_t out_stride, bool f16);
+hipError_t launch_expand_planes8(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n, bool glu,
+                                 uint16_t *out, bool f16);
+hipError_t launch_hilo_epilogue(hipStream_t s, const float *sums, uint32_t rows, uint32_t width, bool gated, uint16_t *out,
+                                uint32_t out_stride, bool f16);
 hipError_t launch_gelu_mul(hipStream_t s, const uint16_t *gate, uint32_t gate_stride, const uint16_t *up, uint32_t up_stride,
                            uint16_t *out, uint32_t out_stride, uint32_t rows, uint32_t count, bool f16);
 uint32_t greedy_segments(uint32_t m, uint32_t n_cus);

@@ -499,6 +499,82 @@ hipError_t launch_matrix_rows(hipStream_t s, const uint8_t *tiles, const uint8_t
     return hipGetLastError();
 }
 
+// An 8-bit matrix for the library's dense GEMM, used beyond the row counts the streaming passes are good for: a 16-bit
+// matrix element cannot hold w = q s + b of an 8-bit q, so w is written as two - hi = round16(w) and lo = round16(w - hi),
+// together 16 (bf16) or 22 (FP16) significant bits of w - and the GEMM multiplies by both: out[r] = hi rows, out[rows + r]
+// = lo rows ([2 m][n], row-major; the gated matrix: gate hi, gate lo, up hi, up lo, [4 f][n]). Read back from the nibble
+// planes, so it can be made again when the activation type changes. One thread per 8 consecutive elements.
+template <bool F16>
+__global__ __launch_bounds__(256) void expand_planes8_kernel(const uint8_t *__restrict__ tiles, const uint8_t *__restrict__ scales,
+                                                             uint32_t m, uint32_t n_groups, bool glu, uint16_t *__restrict__ out) {
+    const uint32_t n = n_groups * kGroup, tile_rows = (glu ? 2u : 1u) * ((m + 15) / 16);
+    const size_t total = (size_t)tile_rows * 16 * n_groups * 8;
+    for (size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x; gid < total; gid += (size_t)gridDim.x * 256) {
+        const uint32_t w = (uint32_t)(gid % (n_groups * 8)), stored_row = (uint32_t)(gid / (n_groups * 8));
+        const uint32_t grp = w >> 3, piece = w & 7, tr = stored_row >> 4, i = stored_row & 15;
+        // the weight row this stored row is, and where its hi / lo rows go
+        const uint32_t row = glu ? (tr >> 1) * 16 + i : stored_row;
+        if (row >= m) continue;
+        const size_t hi_row = glu ? ((tr & 1u) ? 2 * (size_t)m + row : row) : row, lo_row = hi_row + m;
+        const size_t tile = (size_t)tr * n_groups + grp;
+        const uint32_t jq = piece & 3, second = piece >> 2;
+        const uint32_t *lane_words = reinterpret_cast<const uint32_t *>(tiles + tile * kTileBytes) + (jq * 16 + i) * 4;
+        const uint32_t high = lane_words[second], low = lane_words[2 + second];
+        const uint2 sb = reinterpret_cast<const uint2 *>(scales + tile * kTileScaleBytes)[i];
+        const float sc = bf16_to_f32((uint16_t)(sb.y & 0xFFFFu)), bi = bf16_to_f32((uint16_t)(sb.x >> 16));
+        uint32_t hi_w[4] = {0, 0, 0, 0}, lo_w[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int pos = (t & 1) ? 4 + (t >> 1) : (t >> 1);
+            const float q = (float)(16u * ((high >> (4 * pos)) & 0xFu) + ((low >> (4 * pos)) & 0xFu));
+            const float v = q * sc + bi;                       // q * sc is exact in fp32 (8 + 8 bits): the reference's q s + b
+            const uint16_t h = Act<F16>::round(v);
+            hi_w[t >> 1] |= (uint32_t)h << (16 * (t & 1));
+            lo_w[t >> 1] |= (uint32_t)Act<F16>::round(v - Act<F16>::widen(h)) << (16 * (t & 1));
+        }
+        *reinterpret_cast<uint4 *>(out + hi_row * n + grp * kGroup + 8 * piece) = uint4{hi_w[0], hi_w[1], hi_w[2], hi_w[3]};
+        *reinterpret_cast<uint4 *>(out + lo_row * n + grp * kGroup + 8 * piece) = uint4{lo_w[0], lo_w[1], lo_w[2], lo_w[3]};
+    }
+}
+
+hipError_t launch_expand_planes8(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n, bool glu,
+                                 uint16_t *out, bool f16) {
+    const size_t total = (size_t)(glu ? 2 : 1) * ((m + 15) / 16) * 16 * (n / 8);
+    const dim3 grid((uint32_t)min((size_t)65535 * 16, (total + 255) / 256));
+    if (f16) hipLaunchKernelGGL(expand_planes8_kernel<true>, grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, glu, out);
+    else hipLaunchKernelGGL(expand_planes8_kernel<false>, grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, glu, out);
+    return hipGetLastError();
+}
+
+// Behind the GEMMs on the hi / lo rows: a weight row's result is the sum of its two columns.
+// gated: sums [rows][4 f] (gate hi, gate lo, up hi, up lo) -> act[r][j] = round16(gelu_tanh(round16(gate)) * round16(up)),
+// the same roundings as the streaming form's epilogue. plain: sums [rows][2 d] -> y[r][i] = round16(hi + lo).
+template <bool F16, bool GATED>
+__global__ __launch_bounds__(256) void hilo_epilogue_kernel(const float *__restrict__ sums, uint32_t width, uint16_t *__restrict__ out,
+                                                            uint32_t out_stride) {
+    const float *row = sums + (size_t)blockIdx.y * width * (GATED ? 4 : 2);
+    for (uint32_t j = blockIdx.x * 256 + threadIdx.x; j < width; j += gridDim.x * 256) {
+        float v = row[j] + row[width + j];
+        if (GATED) {
+            const float g = Act<F16>::widen(Act<F16>::round(v));
+            const float u = Act<F16>::widen(Act<F16>::round(row[2 * width + j] + row[3 * width + j]));
+            v = gelu_tanh_fast(g) * u;
+        }
+        out[(size_t)blockIdx.y * out_stride + j] = Act<F16>::round(v);
+    }
+}
+
+hipError_t launch_hilo_epilogue(hipStream_t s, const float *sums, uint32_t rows, uint32_t width, bool gated, uint16_t *out,
+                                uint32_t out_stride, bool f16) {
+    if (rows == 0 || rows > 65535u) return hipErrorInvalidValue;
+    const dim3 grid(min(16u, (width + 255) / 256), rows);
+#define FFMOE_HILO(H, G) hipLaunchKernelGGL((hilo_epilogue_kernel<H, G>), grid, dim3(256), 0, s, sums, width, out, out_stride)
+    if (f16) { if (gated) FFMOE_HILO(true, true); else FFMOE_HILO(true, false); }
+    else { if (gated) FFMOE_HILO(false, true); else FFMOE_HILO(false, false); }
+#undef FFMOE_HILO
+    return hipGetLastError();
+}
+
 // keys per input row that launch_matrix_greedy leaves between its two kernels
 uint32_t greedy_segments(uint32_t m, uint32_t n_cus) { return min(2 * n_cus, (m + 31) / 32); }
 

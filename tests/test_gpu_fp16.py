@@ -373,3 +373,32 @@ def test_shared_expert_inside_the_routed_launches_fp16(oracle, ff, torch, d, f, 
     assert ctx.handover_giveups() == 0
     ctx.close()
     shared.close()
+
+
+def test_int8_dense_layer_at_many_rows_follows_the_activation_type(oracle, ff, torch):
+    """The 8-bit dense layer's GEMM form (192 rows and more) keeps hi / lo rows of the weights in the activation type:
+    uploaded under bf16, the context is switched to FP16 and back - each time the rows are made again from the nibble
+    planes - and the 200-row call agrees with the streaming form of the same type (16 rows per matrix call)."""
+    d, fs, t = 192, 1472, 200
+    g = np.random.default_rng(21)
+    parts = tuple(oracle.quantize_int8(g.uniform(-0.4, 0.4, (r, c)).astype(np.float32)) for r, c in ((fs, d), (fs, d), (d, fs)))
+    dense = ff.Context(d, fs, 1, 1, n_layers=1, max_tokens=256)
+    dense.upload_expert_parts(0, 0, *parts, int8=True)
+    xv = g.uniform(-1.0, 1.0, (t, d)).astype(np.float32)
+    seen = {}
+    for act in ("bf16", "fp16", "bf16"):
+        dense.set_act_dtype(act)
+        x = f16_tensor(torch, f16_bits(xv)) if act == "fp16" else bf16_tensor(torch, oracle.bf16_bits(xv))
+        y = dense.dense_ffn(0, x)
+        assert y.dtype == (torch.float16 if act == "fp16" else torch.bfloat16)
+        gate_up, down = dense.matrix_int8_glu(parts[0], parts[1]), dense.matrix_int8(*parts[2])
+        want = torch.cat([down.gemv(gate_up.gemv(x[r0:r0 + 16])) for r0 in range(0, t, 16)])
+        yf, wf = y.float().cpu().numpy(), want.float().cpu().numpy()
+        assert rel_err(yf, wf) < 5e-3 and cosine(yf, wf) > 0.99999, (act, rel_err(yf, wf), cosine(yf, wf))
+        assert np.mean(bits_of(y) == bits_of(want)) > (0.5 if act == "fp16" else 0.9)       # FP16 rows show three more bits of the sum's order
+        if act in seen:
+            assert torch.equal(y.view(torch.int16), seen[act].view(torch.int16))        # back to bf16: the same rows again
+        seen[act] = y
+        gate_up.close()
+        down.close()
+    dense.close()

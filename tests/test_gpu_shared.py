@@ -268,10 +268,13 @@ def _int8_reference_rows(oracle, parts, x_bits):
     return np.stack(out)
 
 
-@pytest.mark.parametrize("d,fs,t", [(128, 64, 1), (128, 192, 16), (192, 1472, 5), (2816, 2112, 16), (128, 64, 40)])
+@pytest.mark.parametrize("d,fs,t", [(128, 64, 1), (128, 192, 16), (192, 1472, 5), (2816, 2112, 16), (128, 64, 40), (128, 64, 191),
+                                    (192, 1472, 200), (2816, 2112, 256), (64, 64, 192)])
 def test_dense_ffn_on_an_int8_layer(ff, oracle, torch, d, fs, t):
     # the 8-bit shared expert as a layer of the dense context: ffmoe_dense_ffn equals the gated matrix + down matrix calls
-    # bit for bit (it runs the same two kernels, 16 rows at a time) and follows the reference's rows
+    # bit for bit (it runs the same two kernels, a grid row per 16 rows) and follows the reference's rows; from 192 rows on
+    # it runs the library's dense GEMM on hi / lo rows of the weights instead, which sums in another order: the same rows
+    # to the rounding of a sum
     g = oracle.seed_tree_key(0x1A8, f"dense-int8-d{d}-fs{fs}-t{t}")
     parts = _int8_parts(oracle, g, d, fs, 0.4 if d < 1024 else 0.08)
     dense = ff.Context(d, fs, 1, 1, n_layers=2, max_tokens=max(t, 16))
@@ -284,9 +287,14 @@ def test_dense_ffn_on_an_int8_layer(ff, oracle, torch, d, fs, t):
     y = dense.dense_ffn(1, xt)
     gate_up, down = dense.matrix_int8_glu(parts[0], parts[1]), dense.matrix_int8(*parts[2])
     want = torch.cat([down.gemv(gate_up.gemv(xt[r0:r0 + 16])) for r0 in range(0, t, 16)])
-    assert torch.equal(y.view(torch.int16), want.view(torch.int16))
-    if d * fs <= 192 * 1472 or t <= 16:
-        rows = slice(0, min(t, 4) if d > 1024 else t)
+    if t < 192:
+        assert torch.equal(y.view(torch.int16), want.view(torch.int16))
+    else:
+        yf, wf = y.float().cpu().numpy(), want.float().cpu().numpy()
+        assert rel_err(yf, wf) < 5e-3 and cosine(yf, wf) > 0.99999 and np.mean(bits_of(y) == bits_of(want)) > 0.9, (
+            rel_err(yf, wf), cosine(yf, wf), np.mean(bits_of(y) == bits_of(want)))
+    if d * fs <= 192 * 1472 or t <= 16 or t >= 192:
+        rows = slice(0, min(t, 4) if d > 1024 or t > 40 else t)
         ref = _int8_reference_rows(oracle, parts, xb[rows])
         got = oracle.bf16_to_float(bits_of(y))[rows]
         assert rel_err(got, ref) < 1e-2 and cosine(got, ref) > 0.9999, (rel_err(got, ref), cosine(got, ref))
@@ -297,7 +305,7 @@ def test_dense_ffn_on_an_int8_layer(ff, oracle, torch, d, fs, t):
     dense.upload_expert_parts(1, 0, *parts4)
     assert float(dense.dense_ffn(1, xt).abs().max()) == 0.0
     dense.upload_expert_parts(1, 0, *parts, int8=True)
-    assert torch.equal(dense.dense_ffn(1, xt).view(torch.int16), want.view(torch.int16))
+    assert torch.equal(dense.dense_ffn(1, xt).view(torch.int16), y.view(torch.int16))
     routed = ff.Context(128, 64, 4, 2, n_layers=1, max_tokens=16)
     with pytest.raises(ff.FieldfareError, match="n_experts = 1"):
         routed.upload_expert_parts(0, 0, *_int8_parts(oracle, g, 128, 64, 0.4), int8=True)
