@@ -485,7 +485,8 @@ int ffmoe_layer_tail_routed(ffmoe_ctx *ctx, void *stream, const uint16_t *route_
  * context, and ffmoe_dense_ffn, ffmoe_route_verify_shared and ffmoe_layer_tail_routed_shared serve it like a 4-bit
  * layer: ffmoe_dense_ffn runs the two GEMV passes, a grid row per 16 rows, or from 192 rows on (when the context's
  * max_tokens reaches that) two dense GEMMs of rocBLAS on hi + lo rows of the weights, kept in the activation type for
- * that purpose (4 more bytes per weight), with the same roundings (gate and up are rounded to 16 bits in front of the
+ * that purpose (4 more bytes per weight; that form is not meant for stream capture: the library may allocate workspace
+ * on its first call), with the same roundings (gate and up are rounded to 16 bits in front of the
  * activation, as the reference's fused kernel does, dequant_int8.metal:131-136). A layer is served in the width of
  * its latest upload: a later ffmoe_upload_layer / ffmoe_upload_expert_parts of the layer drops the 8-bit form. Blocking. */
 int ffmoe_upload_expert_parts_int8(ffmoe_ctx *ctx, uint32_t layer, const ffmoe_projection *gate,
