@@ -852,6 +852,30 @@ def main():
                                                    "shared_expert_int8_inside_routed_launches": 4},
                                       "moe_blocks_of_30_layers_ms": round(30 * t1_ins * 1e3, 3),
                                       "steps": "post-attention setup, shared expert, router, routed experts, layer tail (combine in the tail)"}
+        # the same block at the prefill chunk: setup, shared expert (4-bit grouped GEMMs / 8-bit GEMM form), router + routed
+        # experts + combine, layer tail - one layer's MoE block for the chunk's tokens, shared expert in either width
+        if args.prefill_tokens:
+            TPb = args.prefill_tokens
+            hid_p = torch.randn((TPb, D), device="cuda", generator=gen).to(torch.bfloat16)
+            att_p = torch.randn((TPb, D), device="cuda", generator=gen).to(torch.bfloat16)
+            outs_p = tuple(torch.empty((TPb, D), dtype=torch.bfloat16, device="cuda") for _ in range(3))
+            h1_p = torch.empty((TPb, D), dtype=torch.bfloat16, device="cuda")
+            h2_p = torch.empty((TPb, D), dtype=torch.bfloat16, device="cuda")
+
+            def block_prefill(shared_ctx):
+                i = counter["i"]
+                counter["i"] += 1
+                ctx.post_attn_setup(hid_p, att_p, wn_b[0], wn_b[1], wn_b[2], out=outs_p)
+                shared_ctx.dense_ffn(i % LS, outs_p[0], out=h1_p)
+                idx_p, w_p = ctx.router(i % L, outs_p[2])
+                ctx.prefill(i % L, outs_p[1], idx_p, w_p, out=h2_p)
+                ctx.layer_tail(h2_p, h1_p, hid_p, wn_b[3], wn_b[4], 1.0)
+            tb4 = timed(lambda: block_prefill(dense), 2 * L, warm=2 * L)
+            tb8 = timed(lambda: block_prefill(dense8), 2 * L, warm=2 * L)
+            extra[f"layer_block_rows{TPb}"] = {"shared_expert_4bit_ms": round(tb4 * 1e3, 4), "shared_expert_8bit_ms": round(tb8 * 1e3, 4),
+                                               "tok_per_s_4bit": round(TPb / tb4, 1), "tok_per_s_8bit": round(TPb / tb8, 1),
+                                               "steps": "post-attention setup, shared expert, router, routed experts + combine, layer tail"}
+            del hid_p, att_p, outs_p, h1_p, h2_p
         dense.close()
         dense8.close()
 
