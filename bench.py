@@ -844,7 +844,20 @@ def main():
         t1_ins = timed(block1_inside, 120, warm=30)
         t1_i8 = timed(lambda: block1_int8(False), 120, warm=30)
         t1_i8c = timed(lambda: block1_int8(True), 120, warm=30)
+        # a serving loop replays the decode step as a HIP graph: L layers' blocks, shared expert inside, either width
+        graph1_us = {}
+        for label, fn in (("shared_expert_inside_routed_launches", block1_inside),
+                          ("shared_expert_int8_inside_routed_launches", lambda: block1_int8(True))):
+            gph = torch.cuda.CUDAGraph()
+            cap = torch.cuda.Stream()
+            cap.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.graph(gph, stream=cap):
+                for _ in range(L):
+                    fn()
+            graph1_us[label] = round(timed(gph.replay, 8, warm=2) / L * 1e6, 2)
+            del gph
         extra["layer_block_rows1"] = {"separate_calls_us": round(t1_sep * 1e6, 2),
+                                      "hip_graph_replay_us": graph1_us,
                                       "shared_expert_inside_routed_launches_us": round(t1_ins * 1e6, 2),
                                       "shared_expert_int8_us": round(t1_i8 * 1e6, 2),
                                       "shared_expert_int8_inside_routed_launches_us": round(t1_i8c * 1e6, 2),
