@@ -84,6 +84,25 @@ def test_shared_expert_rows(ff, oracle, torch, d, f, t):
     ctx.close()
 
 
+@pytest.mark.parametrize("d,f,t", [(128, 64, 17), (2816, 2112, 32), (256, 192, 23), (3072, 192, 20)])
+def test_shared_expert_17_to_32_rows_are_two_streaming_passes(ff, oracle, torch, d, f, t):
+    # a chunk's ragged end: rows 0-15 and the rest as two streaming passes - each row bit for bit the row run alone
+    g = oracle.seed_tree_key(0x5EED, f"shared-ffn-two-passes-d{d}-f{f}-t{t}")
+    scale = 0.4 if d < 1024 else 0.08
+    parts = tuple(oracle.quantize_int4(g.uniform(-scale, scale, r * c).reshape(r, c)) for r, c in ((f, d), (f, d), (d, f)))
+    xb = oracle.bf16_bits(g.uniform(-1.0, 1.0, t * d)).reshape(t, d)
+    ctx = _context(ff, parts, d, f, 64)
+    x = bf16_tensor(torch, xb)
+    y = bits_of(ctx.dense_ffn(0, x))
+    for r in (0, 15, 16, t - 1):
+        assert np.array_equal(bits_of(ctx.dense_ffn(0, x[r:r + 1]))[0], y[r]), f"row {r}"
+    sel = [0, 15, 16, t - 1]
+    ref = _reference_rows(oracle, parts, xb[sel])
+    yf = oracle.bf16_to_float(y[sel])
+    assert rel_err(yf, ref) < 1e-2 and cosine(yf, ref) > 0.9999
+    ctx.close()
+
+
 @pytest.mark.parametrize("d,f,t", [(128, 64, 40), (256, 192, 300), (2816, 2112, 64), (512, 640, 700)])
 def test_shared_expert_batched(ff, oracle, torch, d, f, t):
     # more than 16 rows: the grouped GEMMs ((512, 640, 700): three M-tiles against ten and four N-blocks, so that the
