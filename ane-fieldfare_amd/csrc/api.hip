@@ -37,6 +37,9 @@ struct ffmoe_layer {
 // streaming pass per 16 rows (measured at 2816 -> 2112 -> 2816: streaming 19 us at 32 rows + 8.8 us per 32 more, 42 us at
 // 127; the GEMM form 50 us at 128, 58 at 192, 67 at 256, 100 at 1,024, 244 at 3,072).
 constexpr uint32_t kGemm8MinRows = 192;
+// Up to this many rows a 4-bit dense layer streams its arena tiles through the resident-matrix GEMV (a grid row per 16
+// input rows) instead of running the grouped GEMMs.
+constexpr uint32_t kDenseStreamMaxRows = 384;
 
 // A resident matrix: the re-tiled copy of one [m][n] INT4 weight plus the scratch of its greedy choice.
 struct ffmoe_matrix {
@@ -841,10 +844,10 @@ int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t
         uint16_t *acts = t <= FFMOE_MAX_VERIFY_ROWS ? ctx->acts : ctx->pf.acts;
         ctx->timer.begin(s);
         FF_HIP(launch_matrix_gemv(s, l.gate_up8->tiles, l.gate_up8->scales, ctx->shape.f, ctx->shape.d, x, x_stride, t, acts,
-                                  ctx->shape.f, false, ctx->n_cus, ctx->f16, true, true));
+                                  ctx->shape.f, false, ctx->n_cus, ctx->f16, true, 1));
         ctx->timer.mark(s, FFMOE_K_GATE_UP);
         FF_HIP(launch_matrix_gemv(s, l.down8->tiles, l.down8->scales, ctx->shape.d, ctx->shape.f, acts, ctx->shape.f, t, y,
-                                  ctx->shape.d, false, ctx->n_cus, ctx->f16, true, false));
+                                  ctx->shape.d, false, ctx->n_cus, ctx->f16, true, 0));
         ctx->timer.mark(s, FFMOE_K_DOWN);
         ctx->timer.finish();
         return FFMOE_OK;
@@ -854,15 +857,29 @@ int ffmoe_dense_ffn(ffmoe_ctx *ctx, void *stream, uint32_t layer, const uint16_t
     if (t <= FFMOE_MAX_VERIFY_ROWS)
         return verify_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, nullptr, y, err, nullptr,
                              nullptr, true);
-    if (t <= 2 * FFMOE_MAX_VERIFY_ROWS) {
-        // 17 to 32 rows (a chunk's ragged end): two streaming passes beat the grouped GEMMs' fixed cost (measured at
-        // 2816 -> 2112 -> 2816: 27 us against 48 us; from 33 rows on the GEMMs win)
-        if (int rc = verify_common(ctx, stream, layer, x, x_stride, FFMOE_MAX_VERIFY_ROWS, ctx->dense_idx, ctx->dense_w, nullptr,
-                                   nullptr, y, err, nullptr, nullptr, true))
-            return rc;
-        return verify_common(ctx, stream, layer, x + (size_t)FFMOE_MAX_VERIFY_ROWS * x_stride, x_stride, t - FFMOE_MAX_VERIFY_ROWS,
-                             ctx->dense_idx, ctx->dense_w, nullptr, nullptr, y + (size_t)FFMOE_MAX_VERIFY_ROWS * ctx->shape.d, err,
-                             nullptr, nullptr, true);
+    if (t <= kDenseStreamMaxRows && matrix_shape_ok(ctx->shape.d) && matrix_shape_ok(ctx->shape.f) && ctx->shape.f % 16 == 0) {
+        // 17 rows to a few hundred (a short prompt, a chunk's ragged end): below the row count at which the grouped GEMMs'
+        // fixed cost (the weights' expansion per M-tile) is paid back, the resident-matrix GEMV streams the expert's arena
+        // tiles as they lie - a gate/up tile's two streams are a gate and an up row block, a down tile is a plain 4-bit
+        // matrix tile - with one grid row per 16 input rows: two launches.
+        if (int rc = check_layer(ctx, layer, true, false, err)) return rc;
+        const uint32_t cap = std::max<uint32_t>(ctx->shape.max_tokens, FFMOE_MAX_VERIFY_ROWS);
+        if (!x || t > cap) return fail(err, FFMOE_ERR_INVALID, "t = %u exceeds max_tokens = %u", t, cap);
+        if (x_stride < ctx->shape.d || x_stride % 8 || reinterpret_cast<uintptr_t>(x) % 16)
+            return fail(err, FFMOE_ERR_INVALID, "x must be 16-byte aligned with a stride that is a multiple of 8 and >= d");
+        const ArenaGeom &g = ctx->geom;
+        const uint8_t *expert = ctx->arena + (size_t)layer * ctx->layer_bytes;
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        claim_scratch(ctx, stream);
+        ctx->timer.begin(s);
+        FF_HIP(launch_matrix_gemv(s, expert + g.gu_tiles_off, expert + g.gu_scales_off, ctx->shape.f, ctx->shape.d, x, x_stride, t,
+                                  ctx->pf.acts, ctx->shape.f, false, ctx->n_cus, ctx->f16, false, 2));
+        ctx->timer.mark(s, FFMOE_K_GATE_UP);
+        FF_HIP(launch_matrix_gemv(s, expert + g.dn_tiles_off, expert + g.dn_scales_off, ctx->shape.d, ctx->shape.f, ctx->pf.acts,
+                                  ctx->shape.f, t, y, ctx->shape.d, false, ctx->n_cus, ctx->f16, false, 0));
+        ctx->timer.mark(s, FFMOE_K_DOWN);
+        ctx->timer.finish();
+        return FFMOE_OK;
     }
     return prefill_common(ctx, stream, layer, x, x_stride, t, ctx->dense_idx, ctx->dense_w, nullptr, 0, nullptr, y, err, true);
 }
@@ -1286,7 +1303,7 @@ int ffmoe_matrix_gemv(ffmoe_matrix *mx, void *stream, const uint16_t *x, uint32_
     ffmoe_ctx *ctx = mx->ctx;
     ctx->timer.begin(static_cast<hipStream_t>(stream));
     FF_HIP(launch_matrix_gemv(static_cast<hipStream_t>(stream), mx->tiles, mx->scales, mx->m, mx->n, x, x_stride, rows,
-                              y, y_stride, y_f32 != 0, ctx->n_cus, ctx->f16, mx->planes8, mx->glu));
+                              y, y_stride, y_f32 != 0, ctx->n_cus, ctx->f16, mx->planes8, mx->glu ? 1 : 0));
     ctx->timer.mark(static_cast<hipStream_t>(stream), FFMOE_K_GEMV);
     ctx->timer.finish();
     return FFMOE_OK;

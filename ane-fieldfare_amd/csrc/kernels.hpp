@@ -195,7 +195,7 @@ hipError_t launch_matrix_repack(hipStream_t s, const uint8_t *w, const uint16_t 
                                 uint32_t m, uint32_t n, uint8_t *tiles_out, uint8_t *scales_out, bool planes8 = false);
 hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                               const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
-                              bool y_f32, uint32_t n_cus, bool f16 = false, bool planes8 = false, bool glu = false);
+                              bool y_f32, uint32_t n_cus, bool f16 = false, bool planes8 = false, int glu = 0);
 hipError_t launch_matrix_rows(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n, const uint32_t *ids,
                               uint32_t token_id, uint32_t count, float out_scale, uint16_t *out, uint32_t out_stride, bool f16);
 hipError_t launch_expand_planes8(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n, bool glu,

@@ -167,7 +167,7 @@ __device__ __forceinline__ SoftmaxAcc softmax_shuffle(const SoftmaxAcc &a, int m
 // leaves the softmax pair of the sums it finished in conf_part[row * gridDim.x + block].
 // PLANES8: the matrix is an 8-bit one stored as two nibble planes (above): a tile is 16 rows, an output the sum of its
 // two streams.
-template <bool Y_F32, bool F16, bool GREEDY = false, bool CONF = false, bool PLANES8 = false, bool GLU = false>
+template <bool Y_F32, bool F16, bool GREEDY = false, bool CONF = false, bool PLANES8 = false, int GLU = 0>
 __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__restrict__ tiles,
                                                              const uint8_t *__restrict__ scales, uint32_t m,
                                                              uint32_t n_groups, const uint16_t *__restrict__ x,
@@ -176,13 +176,17 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
                                                              float softcap = 0.0f) {
     __shared__ float s_red[2][kKSplit][8][64];
     static_assert(!(PLANES8 && GREEDY), "the greedy choice is built for the 4-bit head only");
-    static_assert(PLANES8 || !GLU, "the gated form is built for the 8-bit planes only");
-    // GLU: tiles 2 p and 2 p + 1 hold rows 16 p ... 16 p + 15 of a gate and of an up projection; a block takes whole
+    static_assert((GLU == 1) ? PLANES8 : true, "tile pairs are the 8-bit planes' gated form");
+    static_assert((GLU == 2) ? !PLANES8 && !GREEDY : true, "gate and up as a tile's two streams is the 4-bit gated form");
+    // GLU == 2: a 4-bit tile's stream A holds 16 rows of a gate projection and its stream B the same rows of the up
+    // projection - the expert arena's gate/up tiles - and `m` counts the outputs gelu_tanh(gate . x) * (up . x), both sums
+    // fp32 in front of the activation as in the expert kernels (moe.metal:496).
+    // GLU == 1: tiles 2 p and 2 p + 1 hold rows 16 p ... 16 p + 15 of a gate and of an up projection; a block takes whole
     // pairs, and `m` counts the outputs gelu_tanh(gate . x) * (up . x)
-    const uint32_t n_tiles = GLU ? 2 * ((m + 15) / 16) : PLANES8 ? (m + 15) / 16 : (m + 31) / 32;
+    const uint32_t n_tiles = GLU == 1 ? 2 * ((m + 15) / 16) : (PLANES8 || GLU == 2) ? (m + 15) / 16 : (m + 31) / 32;
     uint32_t rb0, rb1;
-    split_range(GLU ? n_tiles / 2 : n_tiles, gridDim.x, blockIdx.x, rb0, rb1);
-    if (GLU) {
+    split_range(GLU == 1 ? n_tiles / 2 : n_tiles, gridDim.x, blockIdx.x, rb0, rb1);
+    if (GLU == 1) {
         rb0 *= 2;
         rb1 *= 2;
     }
@@ -247,7 +251,14 @@ __global__ __launch_bounds__(256, 2) void matrix_gemv_kernel(const uint8_t *__re
             va += s_red[buf][o][ks][lane];
             vb += s_red[buf][o][4 + ks][lane];
         }
-        if (GLU) {
+        if (GLU == 2) {
+            const uint32_t col = rb * kTileRows + j;
+            if (my_row < rows && col < m) {
+                const float act = gelu_tanh_fast(va) * vb;
+                if (Y_F32) y32[(size_t)my_row * y_stride + col] = act;
+                else y16[(size_t)my_row * y_stride + col] = Act<F16>::round(act);
+            }
+        } else if (GLU == 1) {
             // both projections are rounded to 16 bits in front of the activation, as shared_int8_gate_up_act_simd does
             // (Metal/Quant/dequant_int8.metal:131-136) and as two separate calls with the activation between them would
             const float v = Act<F16>::widen(Act<F16>::round(va + vb));
@@ -409,8 +420,10 @@ hipError_t launch_matrix_repack(hipStream_t s, const uint8_t *w, const uint16_t 
 
 hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t *scales, uint32_t m, uint32_t n,
                               const uint16_t *x, uint32_t x_stride, uint32_t rows, void *y, uint32_t y_stride,
-                              bool y_f32, uint32_t n_cus, bool f16, bool planes8, bool glu) {
-    const uint32_t n_tiles = planes8 ? (m + 15) / 16 : (m + 31) / 32;      // gated: pairs of tiles
+                              bool y_f32, uint32_t n_cus, bool f16, bool planes8, int glu) {
+    // glu: 0 plain, 1 the 8-bit planes' tile pairs, 2 a 4-bit tile's two streams as gate and up (m = the gated outputs)
+    if (glu == 2 && (planes8 || y_f32)) return hipErrorInvalidValue;
+    const uint32_t n_tiles = (planes8 || glu == 2) ? (m + 15) / 16 : (m + 31) / 32;      // glu == 1: pairs of tiles
     if (rows == 0 || (rows + FFMOE_MAX_VERIFY_ROWS - 1) / FFMOE_MAX_VERIFY_ROWS > 65535u) return hipErrorInvalidValue;
     dim3 grid(min(2 * n_cus, n_tiles), (rows + FFMOE_MAX_VERIFY_ROWS - 1) / FFMOE_MAX_VERIFY_ROWS);
     // several grid rows: a multiple of 8 blocks per row keeps a tile on one XCD (blocks go to the XCDs round robin), whose L2
@@ -419,15 +432,17 @@ hipError_t launch_matrix_gemv(hipStream_t s, const uint8_t *tiles, const uint8_t
 #define FFMOE_MGEMV(Y, H, P, G)                                                                                             \
     hipLaunchKernelGGL((matrix_gemv_kernel<Y, H, false, false, P, G>), grid, dim3(256), 0, s, tiles, scales, m, n / kGroup, x, x_stride, \
                        rows, y, y_stride)
-    if (glu) {
-        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, true, true); else FFMOE_MGEMV(false, true, true, true); }
-        else { if (y_f32) FFMOE_MGEMV(true, false, true, true); else FFMOE_MGEMV(false, false, true, true); }
+    if (glu == 2) {
+        if (f16) FFMOE_MGEMV(false, true, false, 2); else FFMOE_MGEMV(false, false, false, 2);
+    } else if (glu == 1) {
+        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, true, 1); else FFMOE_MGEMV(false, true, true, 1); }
+        else { if (y_f32) FFMOE_MGEMV(true, false, true, 1); else FFMOE_MGEMV(false, false, true, 1); }
     } else if (planes8) {
-        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, true, false); else FFMOE_MGEMV(false, true, true, false); }
-        else { if (y_f32) FFMOE_MGEMV(true, false, true, false); else FFMOE_MGEMV(false, false, true, false); }
+        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, true, 0); else FFMOE_MGEMV(false, true, true, 0); }
+        else { if (y_f32) FFMOE_MGEMV(true, false, true, 0); else FFMOE_MGEMV(false, false, true, 0); }
     } else {
-        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, false, false); else FFMOE_MGEMV(false, true, false, false); }
-        else { if (y_f32) FFMOE_MGEMV(true, false, false, false); else FFMOE_MGEMV(false, false, false, false); }
+        if (f16) { if (y_f32) FFMOE_MGEMV(true, true, false, 0); else FFMOE_MGEMV(false, true, false, 0); }
+        else { if (y_f32) FFMOE_MGEMV(true, false, false, 0); else FFMOE_MGEMV(false, false, false, 0); }
     }
 #undef FFMOE_MGEMV
     return hipGetLastError();

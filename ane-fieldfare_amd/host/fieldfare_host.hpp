@@ -782,8 +782,8 @@ private:
 
 // PrefillSharedExpert (PrefillSharedExpert.swift:19-33,94-137): a block of rows in either weight width (the Swift
 // class defaults to 8 bits). The Swift class loops its single-row operator below 32 tokens and batches the 4-bit
-// form above; here rows <= 16 stream the weights once for all rows and 17 to 32 rows twice; more rows run the grouped GEMMs
-// (4 bits), or a pass per 16 rows and from 192 rows on the library's dense GEMMs (8 bits).
+// form above; here rows <= 16 stream the weights once for all rows, a few hundred rows stream them once per 16 rows, and
+// more rows run the grouped GEMMs (4 bits, from 385 rows) or the library's dense GEMMs (8 bits, from 192 rows).
 class PrefillSharedExpert : public SharedExpertRuntime {
 public:
     static constexpr int batchedMinimumTokens = 17;

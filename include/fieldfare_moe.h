@@ -426,7 +426,8 @@ int ffmoe_upload_expert_parts(ffmoe_ctx *ctx, uint32_t layer, uint32_t expert, c
 
 /* y[t] = down( bf16( gelu_tanh(gate x[t]) * (up x[t]) ) ) for every row, weight 1, no routing: the
  * shared expert. Needs a context created with n_experts = 1 and top_k = 1 (f = the shared width).
- * Rows <= 16 run the streaming kernels of ffmoe_verify, 17 to 32 rows two such passes, more rows the grouped GEMMs
+ * Rows <= 16 run the streaming kernels of ffmoe_verify; 17 to 384 rows the resident-matrix GEMV on the expert's arena
+ * tiles, a grid row per 16 input rows (when d and f fit that kernel: <= FFMOE_MATRIX_MAX_N); more rows the grouped GEMMs
  * of ffmoe_prefill (the reference switches from its per-token GEMV loop to batched GEMMs at 32 tokens). Replaces
  * SharedExpertInt4.encode (Kernels/MoE/SharedExpertInt4.swift:32-89, kernel shared_gate_up_act_int4,
  * Metal/MoE/moe.metal:548-570) and PrefillSharedExpert.encodeBlock
