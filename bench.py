@@ -672,6 +672,16 @@ def main():
         shared["int8"] = {"bytes_per_layer": bytes8, "launches": 2,
                           "rows16": {"us": round(t8_16 * 1e6, 2), "GBs": round(bytes8 / t8_16 / 1e9, 1)},
                           "rows1": {"us": round(t8_1 * 1e6, 2), "GBs": round(bytes8 / t8_1 / 1e9, 1)}}
+        # a short prompt / a chunk's ragged end: 64 and 256 rows, both widths (a grid row of the streaming kernels per 16 rows)
+        if args.prefill_tokens >= 256:
+            for rows_m in (64, 256):
+                xm = torch.randn((rows_m, D), device="cuda", generator=gen).to(torch.bfloat16)
+                ym = torch.empty((rows_m, D), dtype=torch.bfloat16, device="cuda")
+                tm4 = timed(lambda: dense_step(xm, ym), 100, warm=20)
+                tm8 = timed(lambda: int8_step(xm, ym), 100, warm=20)
+                shared[f"rows{rows_m}"] = {"us": round(tm4 * 1e6, 2)}
+                shared["int8"][f"rows{rows_m}"] = {"us": round(tm8 * 1e6, 2)}
+                del xm, ym
         if args.prefill_tokens:
             TPs = args.prefill_tokens
             xps = torch.randn((TPs, D), device="cuda", generator=gen).to(torch.bfloat16)
